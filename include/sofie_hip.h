@@ -1,0 +1,277 @@
+/* sofie_hip.h -- C-ABI of the gfx950 (MI355X) runtime that SOFIE-emitted Session code calls.
+ *
+ * Every entry point is plain C: pointers, sizes, POD descriptors.  No C++ or torch types cross
+ * this boundary.  All functions return 0 on success and a non-zero status on failure; the text
+ * of the last failure on the calling thread is returned by sofie_hip_last_error().  The emitted
+ * C++ Session turns a non-zero status into std::runtime_error, which is the error convention of
+ * the reference's generated code (core/src/RModel.cxx:1839-1841, 1386-1389).
+ *
+ * Threading: a context is used by one thread at a time (the reference's rule is one Session per
+ * thread, core/inc/SOFIE/utils/SOFIEHelpers.hxx:31-51).  Different contexts are independent.
+ *
+ * Pointers in descriptors are DEVICE pointers unless the parameter says "host".  A Session
+ * normally forms them as arena base + planned offset (sofie_hip_arena_ptr).
+ */
+#ifndef SOFIE_HIP_H
+#define SOFIE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SOFIE_HIP_ABI_VERSION 1
+
+typedef struct sofie_hip_ctx sofie_hip_ctx;
+
+/* ---- status codes ------------------------------------------------------------------------- */
+enum {
+   SOFIE_HIP_OK = 0,
+   SOFIE_HIP_ERR_INVALID = 1,  /* bad argument / unsupported combination (nothing was launched) */
+   SOFIE_HIP_ERR_RUNTIME = 2,  /* a HIP call failed                                              */
+   SOFIE_HIP_ERR_NOMEM = 3     /* arena allocation failed or offset outside the arena            */
+};
+
+/* ---- context, stream, arena --------------------------------------------------------------- */
+
+/* Replaces the alpaka Session's devAcc/queue members and its unified pool allocation
+ * (core/src/RModel_ALPAKA.cxx:1090-1141, 443-540).  `external_stream` is a hipStream_t (or NULL
+ * for a stream owned by the context): the kExternalStream option of the reference
+ * (core/inc/SOFIE/RModel_Base.hxx:19-33). */
+int sofie_hip_ctx_create(sofie_hip_ctx **out, int device, void *external_stream);
+int sofie_hip_ctx_destroy(sofie_hip_ctx *ctx);
+const char *sofie_hip_last_error(void);
+int sofie_hip_abi_version(void);
+
+/* One hipMalloc for the whole Session: weights + planned intermediates (the reference allocates
+ * one `allocBuf<uint8_t>` of poolTotalBytes, core/src/RModel_ALPAKA.cxx:477-498).  `align` must
+ * be a power of two >= 256 (kPoolAlignBytes, core/src/RModel_ALPAKA.cxx:25). */
+int sofie_hip_arena_create(sofie_hip_ctx *ctx, size_t bytes, size_t align);
+/* kCustomMemory: adopt caller memory instead of allocating (MemoryProvider.assign,
+ * core/src/utils/SOFIE_common_helpers.cxx:741-804). */
+int sofie_hip_arena_adopt(sofie_hip_ctx *ctx, void *device_ptr, size_t bytes);
+void *sofie_hip_arena_ptr(sofie_hip_ctx *ctx, size_t offset); /* NULL if offset out of range */
+size_t sofie_hip_arena_bytes(sofie_hip_ctx *ctx);
+void *sofie_hip_stream(sofie_hip_ctx *ctx); /* the hipStream_t every launch below goes to */
+
+/* Host <-> arena copies (the user's alpaka::memcpy around infer, README.md:269-325; weight upload
+ * MoveInitializedTensorsToBuffers_ALPAKA, core/src/RModel_ALPAKA.cxx:1695-1707). Asynchronous on
+ * the context's stream; sofie_hip_sync waits. */
+int sofie_hip_upload(sofie_hip_ctx *ctx, void *dst_device, const void *src_host, size_t bytes);
+int sofie_hip_download(sofie_hip_ctx *ctx, void *dst_host, const void *src_device, size_t bytes);
+int sofie_hip_copy(sofie_hip_ctx *ctx, void *dst_device, const void *src_device, size_t bytes);
+int sofie_hip_fill_zero(sofie_hip_ctx *ctx, void *dst_device, size_t bytes); /* resetState, RModel_ALPAKA.cxx:1546-1568 */
+int sofie_hip_sync(sofie_hip_ctx *ctx);                                      /* alpaka::wait(queue) */
+
+/* ---- activation / epilogue vocabulary ------------------------------------------------------ */
+/* Scalar formulas follow the reference's CPU emitters:
+ *   RELU      x > 0 ? x : 0            core/src/utils/SOFIE_common_helpers.cxx:325-332
+ *   LEAKYRELU x >= 0 ? x : alpha*x     core/inc/SOFIE/operators/ROperator_Gemm.hxx:729-738
+ *   SIGMOID   1/(1+exp(-x))            core/inc/SOFIE/operators/ROperator_Sigmoid.hxx:43-59
+ *   GELU      0.5 x (1+erf(x/sqrt2))   core/inc/SOFIE/operators/ROperator_Gelu.hxx:42-71
+ *   GELU_TANH 0.5 x (1+tanh(0.7978845608028654 (x+0.044715 x^3)))   (same file)
+ *   TANH      std::tanh                core/inc/SOFIE/operators/ROperator_Tanh.hxx */
+enum {
+   SOFIE_ACT_NONE = 0,
+   SOFIE_ACT_RELU = 1,
+   SOFIE_ACT_LEAKYRELU = 2,
+   SOFIE_ACT_SIGMOID = 3,
+   SOFIE_ACT_GELU = 4,
+   SOFIE_ACT_GELU_TANH = 5,
+   SOFIE_ACT_TANH = 6
+};
+
+/* How a bias (the Gemm operand C) is broadcast onto Y[M,N]; the four cases the reference's Gemm
+ * emitter distinguishes (core/inc/SOFIE/operators/ROperator_Gemm.hxx:578-617). */
+enum {
+   SOFIE_BIAS_NONE = 0,
+   SOFIE_BIAS_ROW = 1,    /* C is [N] or [1,N]: Copy(Y + N*j, C, N) for every row j            */
+   SOFIE_BIAS_COL = 2,    /* C is [M,1]:        Fill(Y + N*j, C[j], N)                          */
+   SOFIE_BIAS_SCALAR = 3, /* C is [1,1]/[1]:    Fill(Y + N*j, C[0], N)                          */
+   SOFIE_BIAS_FULL = 4    /* C is [M,N]: passed to Gemm_Call as C, Y = alpha*A*B + beta*C       */
+};
+
+/* ---- fp32 Gemm / MatMul -------------------------------------------------------------------- */
+/* Replaces ROperator_Gemm<float>::Generate + Gemm_Call + BLAS::sgemm_ + Relu
+ * (core/inc/SOFIE/operators/ROperator_Gemm.hxx:419-741, core/src/utils/SOFIE_common_helpers.cxx:296-332)
+ * and, on the alpaka path, blas.gemm / blas.gemmrelu / blas.gemmStridedBatched + GemmBiasAddKernel
+ * (ROperator_Gemm.hxx:743-764, 931-1103).
+ *   Y[b] = act( alpha * op(A[b]) * op(B[b]) + beta_eff * broadcast(C) ),  b < batch
+ * Tensors are row-major as ONNX defines them: op(A) is [M,K], op(B) is [K,N], Y is [M,N].
+ * transA: A is stored [K,M]; transB: B is stored [N,K].  beta_eff is 1 for the broadcast cases and
+ * `beta` for SOFIE_BIAS_FULL, which is the reference's behaviour (ROperator_Gemm.hxx:580). */
+typedef struct sofie_gemm_f32_desc {
+   int32_t M, N, K;
+   int32_t transA, transB;
+   int32_t lda, ldb, ldy; /* row strides in elements of the STORED matrices; 0 = dense default */
+   float alpha, beta;
+   const float *A;
+   const float *B;
+   const float *C; /* bias or NULL */
+   int32_t bias_mode;
+   int32_t act;
+   float act_alpha; /* LeakyRelu slope */
+   float *Y;
+   int32_t batch; /* stacked MatMul count (>=1); strides in elements, 0 = operand shared */
+   int64_t strideA, strideB, strideC, strideY;
+} sofie_gemm_f32_desc;
+int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d);
+
+/* ---- int8 Gemm (MatMulInteger + fused requantisation) -------------------------------------- */
+/* No counterpart exists in the reference (ROperator_Gemm is float only,
+ * core/inc/SOFIE/operators/ROperator_Gemm.hxx:67; no quantised operator is registered,
+ * parsers/src/RModelParser_ONNX.cxx:279-367).  The semantics are the ONNX ones:
+ *   acc[m,n]  = sum_k int32(A[m,k]) * int32(B[k,n])              (exact)
+ *   acc      += bias_i32[n]                                      (if bias)
+ *   acc       = max(acc,0)                                       (if relu_acc)
+ * then by `out`:
+ *   SOFIE_I8OUT_I32    Y_i32 = acc
+ *   SOFIE_I8OUT_F32    Y_f32 = float(acc) * s              (DequantizeLinear; s = scale[n] or scale_scalar),
+ *                              then max(.,0) if relu_out
+ *   SOFIE_I8OUT_I8     Y_i8  = sat8(rne(float(acc) * s))   (requant), then max(.,0) if relu_out
+ *   SOFIE_I8OUT_I8_DQQ Y_i8  = sat8(rne((float(acc) * s) / q_scale))   (DequantizeLinear followed by the
+ *                              next layer's QuantizeLinear, same fp32 operations in the same order)
+ * One fp32 multiply (no fused multiply-add), round-half-to-even, saturation to [-128,127].
+ * A is [M,K] int8 row-major (lda), B is [K,N] row-major (ldb) or, with transB, stored [N,K].
+ * The MFMA kernel wants both operands K-contiguous; a B given as [K,N] is transposed into
+ * `workspace` (K*N bytes, 256-B aligned) on every call.  A constant B (a weight) is better re-laid
+ * out once at Session construction with sofie_hip_transpose_i8 and then passed with transB = 1. */
+enum { SOFIE_I8OUT_I32 = 0, SOFIE_I8OUT_F32 = 1, SOFIE_I8OUT_I8 = 2, SOFIE_I8OUT_I8_DQQ = 3 };
+typedef struct sofie_gemm_i8_desc {
+   int32_t M, N, K;
+   int32_t transA, transB;
+   int32_t lda, ldb, ldy; /* 0 = dense default */
+   const int8_t *A;
+   const int8_t *B;
+   const int32_t *bias; /* [N] or NULL */
+   const float *scale;  /* [N] per output channel, or NULL -> scale_scalar */
+   float scale_scalar;
+   float q_scale; /* SOFIE_I8OUT_I8_DQQ only */
+   int32_t relu_acc, relu_out;
+   int32_t out;
+   void *Y;
+   void *workspace; /* device scratch for operand re-layout, may be NULL if not needed */
+   size_t workspace_bytes;
+} sofie_gemm_i8_desc;
+int sofie_hip_gemm_i8(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d);
+/* Bytes of workspace sofie_hip_gemm_i8 needs for this descriptor (0 if none). */
+size_t sofie_hip_gemm_i8_workspace(const sofie_gemm_i8_desc *d);
+/* Re-layout of a [K,N] int8 matrix into [N,K] (weights, once, at Session construction; the
+ * analogue of the Conv weight re-layout into tensor_<Y>_f, ROperator_Conv.hxx:456-476). */
+int sofie_hip_transpose_i8(sofie_hip_ctx *ctx, int8_t *dst, const int8_t *src, int32_t rows, int32_t cols,
+                           int32_t ld_src, int32_t ld_dst);
+
+/* ---- FP8 (OCP e4m3fn) Gemm ------------------------------------------------------------------ */
+/* No counterpart in the reference (ETensorType ends at BFLOAT16, core/inc/SOFIE/utils/SOFIE_common.hxx:29-54).
+ *   acc[m,n] = sum_k f32(A[m,k]) * f32(B[k,n])   (fp32 accumulate, hardware summation order)
+ *   v        = acc * (scale_a*scale_b) + bias[n];   v = act(v);   Y = bf16_rne(v) or fp32
+ * A [M,K] e4m3fn bytes; B [K,N] or, with transB, [N,K]; same workspace rule as the int8 Gemm. */
+enum { SOFIE_F8OUT_BF16 = 0, SOFIE_F8OUT_F32 = 1 };
+typedef struct sofie_gemm_fp8_desc {
+   int32_t M, N, K;
+   int32_t transB;
+   int32_t lda, ldb, ldy;
+   const uint8_t *A;
+   const uint8_t *B;
+   const float *bias; /* [N] fp32 or NULL */
+   float scale;       /* scale_a * scale_b, formed in fp32 by the caller */
+   int32_t act;
+   int32_t out;
+   void *Y;
+   void *workspace;
+   size_t workspace_bytes;
+} sofie_gemm_fp8_desc;
+int sofie_hip_gemm_fp8(sofie_hip_ctx *ctx, const sofie_gemm_fp8_desc *d);
+/* fp32 -> e4m3fn: q = sat(rne_e4m3(x / scale)); saturating at +-448, NaN -> 0x7f. */
+int sofie_hip_quantize_fp8(sofie_hip_ctx *ctx, uint8_t *dst, const float *src, size_t n, float scale);
+
+/* ---- QuantizeLinear / DequantizeLinear (per tensor, symmetric, zero point 0) ---------------- */
+/* ONNX: q = sat8(rne(x / scale)) with fp32 division; y = float(q) * scale.  Not in the reference. */
+int sofie_hip_quantize_linear(sofie_hip_ctx *ctx, int8_t *dst, const float *src, size_t n, float scale);
+int sofie_hip_dequantize_linear_i8(sofie_hip_ctx *ctx, float *dst, const int8_t *src, size_t n, float scale);
+int sofie_hip_dequantize_linear_i32(sofie_hip_ctx *ctx, float *dst, const int32_t *src, size_t n, float scale);
+
+/* ---- stand-alone elementwise operators ------------------------------------------------------ */
+/* Replaces the CPU loops / alpaka kernels of ROperator_Relu, _Sigmoid, _Gelu, _LeakyRelu, _Tanh
+ * (core/inc/SOFIE/operators/ROperator_Relu.hxx:47-86 and siblings). dst may equal src. */
+int sofie_hip_unary_f32(sofie_hip_ctx *ctx, float *dst, const float *src, size_t n, int32_t act, float act_alpha);
+/* ROperator_BasicBinary<float,Add> with multidirectional broadcasting
+ * (core/inc/SOFIE/operators/ROperator_BasicBinary.hxx:380-510).  Shapes are right-aligned, rank<=6;
+ * a_shape/b_shape hold 1 where the operand is broadcast. */
+typedef struct sofie_add_desc {
+   int32_t rank;
+   int64_t y_shape[6];
+   int64_t a_shape[6];
+   int64_t b_shape[6];
+   const float *A;
+   const float *B;
+   float *Y;
+} sofie_add_desc;
+int sofie_hip_add_f32(sofie_hip_ctx *ctx, const sofie_add_desc *d);
+
+/* ---- Conv as GEMM --------------------------------------------------------------------------- */
+/* Replaces ROperator_Conv<float>::Generate: weight re-layout + per-image Im2col + Gemm_Call
+ * (core/inc/SOFIE/operators/ROperator_Conv.hxx:406-642; Im2col core/src/utils/SOFIE_common_helpers.cxx:47-83)
+ * and the alpaka Im2ColKernel/BiasBroadcastKernel/blas.matmul triple (ROperator_Conv.hxx:732-1103)
+ * with ONE implicit-GEMM launch over the whole batch (no materialised column matrix).
+ * X is NCHW [N,C,H,W], W is [Cout, C/group, kh, kw], Y is NCHW [N,Cout,OH,OW]; 1-D convs pass H=1,kh=1.
+ * pads follow the reference's order {h_begin, w_begin, h_end, w_end} (ROperator_Conv.hxx:517-530). */
+typedef struct sofie_conv_desc {
+   int32_t N, C, H, W;
+   int32_t Cout, kh, kw;
+   int32_t pad_h0, pad_w0, pad_h1, pad_w1;
+   int32_t stride_h, stride_w;
+   int32_t dil_h, dil_w;
+   int32_t group;
+   int32_t OH, OW; /* as computed by the caller's shape inference; checked */
+} sofie_conv_desc;
+int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float *X, const float *W,
+                       const float *bias /* [Cout] or NULL */, int32_t act, float act_alpha, float *Y);
+/* int8 form (no counterpart in the reference): acc = conv_i32(X_i8, W_i8) + bias_i32[co], then by `out`
+ *   SOFIE_I8OUT_I8   Y_i8  = sat8(rne(float(acc)*scale[co])), then max(.,0) if relu
+ *   SOFIE_I8OUT_F32  Y_f32 = float(acc)*scale[co], then max(.,0) if relu
+ *   SOFIE_I8OUT_I32  Y_i32 = relu ? max(acc,0) : acc
+ * Activations are NCHW (the ONNX layout) or NHWC (channels fastest), chosen per tensor: a chain of
+ * convolutions keeps NHWC between its layers.  W is the ONNX weight [Cout, C/group, kh, kw], or, with
+ * w_is_packed, the re-laid-out form sofie_hip_pack_conv_weight_i8 writes once at Session construction
+ * (the role of tensor_<Y>_f in the reference, ROperator_Conv.hxx:456-476).  The workspace holds the
+ * packed weights (unless w_is_packed) and the column matrix of as many images as fit (at least one). */
+enum { SOFIE_LAYOUT_NCHW = 0, SOFIE_LAYOUT_NHWC = 1 };
+typedef struct sofie_conv_i8_args {
+   const int8_t *X;
+   const int8_t *W;
+   const int32_t *bias; /* [Cout] or NULL */
+   const float *scale;  /* [Cout]; may be NULL for SOFIE_I8OUT_I32 */
+   int32_t relu;
+   int32_t out;
+   int32_t x_layout, y_layout;
+   int32_t w_is_packed;
+   void *Y;
+   void *workspace;
+   size_t workspace_bytes;
+} sofie_conv_i8_args;
+int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_conv_i8_args *a);
+size_t sofie_hip_conv_i8_workspace(const sofie_conv_desc *d, const sofie_conv_i8_args *a); /* minimum bytes */
+size_t sofie_hip_conv_weight_i8_packed_bytes(const sofie_conv_desc *d);
+int sofie_hip_pack_conv_weight_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, int8_t *dst, const int8_t *src);
+
+/* ---- pooling tail --------------------------------------------------------------------------- */
+/* GlobalAveragePool (ROperator_Pool, core/inc/SOFIE/operators/ROperator_Pool.hxx:225-237):
+ * Y[n,c] = (sum over the HW plane of X[n,c,:]) / float(HW); the fp32 sum is a tree reduction, so it
+ * agrees with the reference's sequential loop to rounding only. */
+int sofie_hip_global_avg_pool_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t NC, int32_t HW);
+/* int8 input, fp32 output: Y = (float(sum_i32) * scale) / float(HW), exact sum -- not in the reference. */
+int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y /* [N,C] */, const int8_t *X, int32_t N, int32_t C, int32_t HW,
+                                 int32_t x_layout /* SOFIE_LAYOUT_* */, float scale);
+
+/* ---- timing helper used by the benchmark ----------------------------------------------------- */
+/* hipEvent pair on the context's stream (torch's events only see torch's streams). */
+int sofie_hip_timer_start(sofie_hip_ctx *ctx);
+int sofie_hip_timer_stop(sofie_hip_ctx *ctx, float *elapsed_ms); /* records, synchronises, returns ms */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SOFIE_HIP_H */

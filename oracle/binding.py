@@ -1,0 +1,234 @@
+"""numpy/ctypes view of the CPU oracle (oracle/sofie_oracle.c).  TEST INFRASTRUCTURE.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg import this module; the
+product path (sofie_amd/) never does.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_libs = {}
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def load(omp=False):
+    name = "libsofie_oracle_omp.so" if omp else "libsofie_oracle.so"
+    if name not in _libs:
+        path = os.path.join(_HERE, name)
+        if not os.path.exists(path):
+            raise RuntimeError("%s is not built: run `make -C oracle`" % path)
+        lib = C.CDLL(path)
+        lib.oracle_e4m3_to_f32.restype = C.c_float
+        lib.oracle_e4m3_to_f32.argtypes = [C.c_uint8]
+        lib.oracle_f32_to_e4m3.restype = C.c_uint8
+        lib.oracle_f32_to_e4m3.argtypes = [C.c_float]
+        lib.oracle_f32_to_bf16.restype = C.c_uint16
+        lib.oracle_f32_to_bf16.argtypes = [C.c_float]
+        lib.oracle_num_threads.restype = C.c_int
+        _libs[name] = lib
+    return _libs[name]
+
+
+def load_ref_planner():
+    """The reference's own OrganizeMemory (oracle/_ref), or None where it was not built."""
+    path = os.path.join(_HERE, "_ref", "libref_planner.so")
+    if not os.path.exists(path):
+        return None
+    return C.CDLL(path)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def gemm_f32(A, B, C_=None, *, M, N, K, transA=0, transB=0, alpha=1.0, beta=1.0, bias_mode=0, act=0, act_alpha=0.0):
+    A, B = _f32(A), _f32(B)
+    Cc = None if C_ is None else _f32(C_)
+    Y = np.zeros((M, N), dtype=np.float32)
+    load().oracle_gemm_f32(C.c_int(M), C.c_int(N), C.c_int(K), C.c_int(transA), C.c_int(transB), C.c_float(alpha),
+                           C.c_float(beta), _ptr(A), _ptr(B), _ptr(Cc), C.c_int(bias_mode), C.c_int(act),
+                           C.c_float(act_alpha), _ptr(Y))
+    return Y
+
+
+def unary(x, act, alpha=0.0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    load().oracle_unary(_ptr(y), _ptr(x), C.c_size_t(x.size), C.c_int(act), C.c_float(alpha))
+    return y
+
+
+def add_broadcast(A, B):
+    A, B = _f32(A), _f32(B)
+    yshape = np.broadcast_shapes(A.shape, B.shape)
+    rank = len(yshape)
+    ash = (1,) * (rank - A.ndim) + A.shape
+    bsh = (1,) * (rank - B.ndim) + B.shape
+    Y = np.empty(yshape, dtype=np.float32)
+    arr = lambda s: (C.c_int64 * 6)(*(list(s) + [1] * (6 - len(s))))
+    load().oracle_add_broadcast(C.c_int(rank), arr(yshape), arr(ash), arr(bsh), _ptr(A), _ptr(B), _ptr(Y))
+    return Y
+
+
+def conv_out_hw(H, W, kh, kw, pads, strides, dils):
+    OH = (H + pads[0] + pads[2] - (dils[0] * (kh - 1) + 1)) // strides[0] + 1
+    OW = (W + pads[1] + pads[3] - (dils[1] * (kw - 1) + 1)) // strides[1] + 1
+    return OH, OW
+
+
+def conv_f32(X, W, bias=None, *, pads=(0, 0, 0, 0), strides=(1, 1), dils=(1, 1), group=1, act=0, act_alpha=0.0):
+    """X [N,C,H,W], W [Cout,C/group,kh,kw], pads (h0,w0,h1,w1)."""
+    X, W = _f32(X), _f32(W)
+    b = None if bias is None else _f32(bias)
+    N, Cc, H, Wd = X.shape
+    Cout, _, kh, kw = W.shape
+    OH, OW = conv_out_hw(H, Wd, kh, kw, pads, strides, dils)
+    Y = np.zeros((N, Cout, OH, OW), dtype=np.float32)
+    rc = load().oracle_conv_f32(N, Cc, H, Wd, Cout, kh, kw, pads[0], pads[1], pads[2], pads[3], strides[0], strides[1],
+                                dils[0], dils[1], group, _ptr(X), _ptr(W), _ptr(b), act, C.c_float(act_alpha), _ptr(Y))
+    if rc:
+        raise MemoryError("oracle_conv_f32")
+    return Y
+
+
+def im2col(x, kh, kw, pads, strides, dils):
+    """x [C,H,W] -> [C*kh*kw, OH*OW]; pads (h0,w0,h1,w1)."""
+    x = _f32(x)
+    Cc, H, W = x.shape
+    OH, OW = conv_out_hw(H, W, kh, kw, pads, strides, dils)
+    col = np.empty((Cc * kh * kw, OH * OW), dtype=np.float32)
+    load().oracle_im2col(_ptr(x), Cc, H, W, kh, kw, pads[0], pads[2], pads[1], pads[3], strides[0], strides[1], dils[0],
+                         dils[1], _ptr(col))
+    return col
+
+
+def global_avg_pool(X):
+    X = _f32(X)
+    N, Cc = X.shape[:2]
+    HW = int(np.prod(X.shape[2:]))
+    Y = np.empty((N, Cc) + (1,) * (X.ndim - 2), dtype=np.float32)
+    load().oracle_global_avg_pool(_ptr(Y), _ptr(X), N * Cc, HW)
+    return Y
+
+
+def global_avg_pool_i8(X, scale):
+    X = np.ascontiguousarray(X, dtype=np.int8)
+    N, Cc = X.shape[:2]
+    HW = int(np.prod(X.shape[2:]))
+    Y = np.empty((N, Cc), dtype=np.float32)
+    load().oracle_global_avg_pool_i8(_ptr(Y), _ptr(X), N * Cc, HW, C.c_float(scale))
+    return Y
+
+
+def organize_memory(begin, end, size, lib=None, fn="oracle_organize_memory"):
+    n = len(begin)
+    b = (C.c_int * n)(*begin)
+    e = (C.c_int * n)(*end)
+    s = (C.c_size_t * n)(*size)
+    off = (C.c_size_t * n)()
+    tot, tfree, lfree = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    lib = lib or load()
+    rc = getattr(lib, fn)(n, b, e, s, off, C.byref(tot), C.byref(tfree), C.byref(lfree))
+    if rc:
+        raise ValueError("organize_memory failed with %d" % rc)
+    return {"total_bytes": tot.value, "offsets": list(off), "total_free_bytes": tfree.value,
+            "largest_free_block": lfree.value}
+
+
+def quantize_linear(x, scale):
+    x = _f32(x)
+    q = np.empty(x.shape, dtype=np.int8)
+    load().oracle_quantize_linear(_ptr(q), _ptr(x), C.c_size_t(x.size), C.c_float(scale))
+    return q
+
+
+def dequantize_linear(q, scale):
+    q = np.ascontiguousarray(q)
+    y = np.empty(q.shape, dtype=np.float32)
+    if q.dtype == np.int8:
+        load().oracle_dequantize_linear_i8(_ptr(y), _ptr(q), C.c_size_t(q.size), C.c_float(scale))
+    elif q.dtype == np.int32:
+        load().oracle_dequantize_linear_i32(_ptr(y), _ptr(q), C.c_size_t(q.size), C.c_float(scale))
+    else:
+        raise TypeError(q.dtype)
+    return y
+
+
+_OUT_DTYPE = {0: np.int32, 1: np.float32, 2: np.int8, 3: np.int8}
+
+
+def matmul_integer(A, B, *, M, N, K, transA=0, transB=0, omp=False):
+    A = np.ascontiguousarray(A, dtype=np.int8)
+    B = np.ascontiguousarray(B, dtype=np.int8)
+    acc = np.empty((M, N), dtype=np.int32)
+    load(omp).oracle_matmul_integer(M, N, K, transA, transB, _ptr(A), _ptr(B), _ptr(acc))
+    return acc
+
+
+def gemm_i8_epilogue(acc, *, bias=None, scale=None, scale_scalar=1.0, q_scale=1.0, relu_acc=0, relu_out=0, out=0):
+    acc = np.ascontiguousarray(acc, dtype=np.int32)
+    M, N = acc.shape
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+    s = None if scale is None else _f32(scale)
+    Y = np.empty((M, N), dtype=_OUT_DTYPE[out])
+    load().oracle_gemm_i8_epilogue(M, N, _ptr(acc), _ptr(b), _ptr(s), C.c_float(scale_scalar), C.c_float(q_scale),
+                                   relu_acc, relu_out, out, _ptr(Y))
+    return Y
+
+
+def gemm_i8(A, B, *, M, N, K, transA=0, transB=0, omp=False, **epi):
+    return gemm_i8_epilogue(matmul_integer(A, B, M=M, N=N, K=K, transA=transA, transB=transB, omp=omp), **epi)
+
+
+def conv_i8(X, W, bias=None, scale=None, *, pads=(0, 0, 0, 0), strides=(1, 1), dils=(1, 1), group=1, relu=0, out=2,
+            omp=False):
+    X = np.ascontiguousarray(X, dtype=np.int8)
+    W = np.ascontiguousarray(W, dtype=np.int8)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+    s = None if scale is None else _f32(scale)
+    N, Cc, H, Wd = X.shape
+    Cout, _, kh, kw = W.shape
+    OH, OW = conv_out_hw(H, Wd, kh, kw, pads, strides, dils)
+    Y = np.empty((N, Cout, OH, OW), dtype=_OUT_DTYPE[out])
+    load(omp).oracle_conv_i8(N, Cc, H, Wd, Cout, kh, kw, pads[0], pads[1], pads[2], pads[3], strides[0], strides[1],
+                             dils[0], dils[1], group, _ptr(X), _ptr(W), _ptr(b), _ptr(s), relu, out, _ptr(Y))
+    return Y
+
+
+def e4m3_to_f32(codes):
+    lib = load()
+    codes = np.asarray(codes, dtype=np.uint8)
+    lut = np.array([lib.oracle_e4m3_to_f32(i) for i in range(256)], dtype=np.float32)
+    return lut[codes]
+
+
+def quantize_fp8(x, scale):
+    x = _f32(x)
+    q = np.empty(x.shape, dtype=np.uint8)
+    load().oracle_quantize_fp8(_ptr(q), _ptr(x), C.c_size_t(x.size), C.c_float(scale))
+    return q
+
+
+def f32_to_bf16_bits(x):
+    lib = load()
+    x = _f32(x)
+    return np.array([lib.oracle_f32_to_bf16(float(v)) for v in x.ravel()], dtype=np.uint16).reshape(x.shape)
+
+
+def bf16_bits_to_f32(b):
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def gemm_fp8(A, B, *, M, N, K, transB=0, bias=None, scale=1.0, act=0, out=1, want_abs_sum=False, omp=False):
+    A = np.ascontiguousarray(A, dtype=np.uint8)
+    B = np.ascontiguousarray(B, dtype=np.uint8)
+    b = None if bias is None else _f32(bias)
+    Y = np.empty((M, N), dtype=np.float32 if out == 1 else np.uint16)
+    sa = np.empty((M, N), dtype=np.float32) if want_abs_sum else None
+    load(omp).oracle_gemm_fp8(M, N, K, transB, _ptr(A), _ptr(B), _ptr(b), C.c_float(scale), act, out, _ptr(Y), _ptr(sa))
+    return (Y, sa) if want_abs_sum else Y

@@ -1,0 +1,699 @@
+/* sofie_oracle.c -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * A plain-C, CPU restatement of the reference's (ML4EP/SOFIE 1.0.1) generated inference code for
+ * the Gemm / Conv / epilogue / memory-plan path, plus the frozen definitions of the quantised
+ * operators the reference does not have.  Only the tests, the smoke check and the benchmark's
+ * cpu_baseline leg may load this library, and only as the checker.  The HIP runtime never calls it.
+ *
+ * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off: no fused multiply-add may be formed, so
+ * that every fp32 operation rounds exactly as written).
+ *
+ * What pins each function (tests/test_oracle_*.py):
+ *   gemm_f32 / gemm_call      golden outputs Linear_16/32/64, LinearWithSigmoid, LinearWithLeakyRelu
+ *                             of the reference's own tests; literal cases of its constant-folding
+ *                             tests; float64 brute force.
+ *   im2col / conv_f32         golden outputs of the reference's 18 Conv* fixtures; 7-loop direct
+ *                             convolution in float64.
+ *   relu/sigmoid/gelu/...     Gelu / GeluTanh golden outputs; closed forms.
+ *   global_avg_pool           GlobalAvgPool2d golden output.
+ *   organize_memory           the reference's MemoryPlanner.inc compiled as oracle/_ref and run on the
+ *                             same lifetimes; known totals of the Linear_16 plan.
+ *   quantize/dequantize, gemm_i8, conv_i8, e4m3 codec, gemm_fp8
+ *                             PARITY UNPINNED BY THE REFERENCE: it has no quantised operator
+ *                             (parsers/src/RModelParser_ONNX.cxx:279-367).  Pinned instead by what the
+ *                             ONNX definitions fix: exhaustive tables (all 256 e4m3 codes, all int8
+ *                             products), tie cases of round-half-even, int64 numpy matmul, identity /
+ *                             one-hot special cases.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORACLE_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------------------------------------
+ * fp32 path
+ * ---------------------------------------------------------------------------------------------- */
+
+/* Portable column-major SGEMM with the Fortran BLAS meaning of every argument; the reference leaves
+ * this to whatever BLAS is linked (core/src/utils/SOFIE_common_helpers.cxx:32-38).  The dot product
+ * runs over k in increasing order in fp32. */
+static void oracle_sgemm(char transa, char transb, int m, int n, int k, float alpha, const float *A, int lda,
+                         const float *B, int ldb, float beta, float *C, int ldc)
+{
+   const int ta = (transa == 't' || transa == 'T');
+   const int tb = (transb == 't' || transb == 'T');
+   for (int j = 0; j < n; ++j) {
+      for (int i = 0; i < m; ++i) {
+         float sum = 0.0f;
+         for (int p = 0; p < k; ++p) {
+            float a = ta ? A[(size_t)i * lda + p] : A[(size_t)p * lda + i];
+            float b = tb ? B[(size_t)p * ldb + j] : B[(size_t)j * ldb + p];
+            sum += a * b;
+         }
+         float *c = &C[(size_t)j * ldc + i];
+         *c = (beta == 0.0f) ? alpha * sum : alpha * sum + beta * *c;
+      }
+   }
+}
+
+/* Gemm_Call of the generated code (core/src/utils/SOFIE_common_helpers.cxx:296-310): optional copy of
+ * C into the output, then sgemm_ with lda = transa ? k : m, ldb = transb ? n : k, ldc = m. */
+ORACLE_API void oracle_gemm_call(float *output, int transa, int transb, int m, int n, int k, float alpha, const float *A,
+                                 const float *B, float beta, const float *C)
+{
+   int lda = transa ? k : m;
+   int ldb = transb ? n : k;
+   if (C != NULL)
+      memcpy(output, C, sizeof(float) * (size_t)m * (size_t)n);
+   oracle_sgemm(transa ? 't' : 'n', transb ? 't' : 'n', m, n, k, alpha, A, lda, B, ldb, beta, output, m);
+}
+
+/* Relu helper (SOFIE_common_helpers.cxx:325-332): NaN -> 0, -0 -> +0. */
+ORACLE_API void oracle_relu(float *out, const float *in, size_t n)
+{
+   for (size_t i = 0; i < n; ++i)
+      out[i] = (in[i] > 0.0f) ? in[i] : 0.0f;
+}
+/* LeakyRelu as fused by the Gemm emitter (ROperator_Gemm.hxx:729-738). */
+ORACLE_API void oracle_leaky_relu(float *out, const float *in, size_t n, float alpha)
+{
+   for (size_t i = 0; i < n; ++i)
+      out[i] = in[i] >= 0.0f ? in[i] : alpha * in[i];
+}
+/* ROperator_Sigmoid.hxx:43-59 */
+ORACLE_API void oracle_sigmoid(float *out, const float *in, size_t n)
+{
+   for (size_t i = 0; i < n; ++i)
+      out[i] = 1.0f / (1.0f + expf(-in[i]));
+}
+/* ROperator_Gelu.hxx:42-71, erf form */
+ORACLE_API void oracle_gelu(float *out, const float *in, size_t n)
+{
+   for (size_t i = 0; i < n; ++i)
+      out[i] = 0.5f * in[i] * (1.0f + erff(in[i] * 0.7071067811865475f));
+}
+/* ROperator_Gelu.hxx:42-71, tanh form */
+ORACLE_API void oracle_gelu_tanh(float *out, const float *in, size_t n)
+{
+   for (size_t i = 0; i < n; ++i) {
+      float x = in[i];
+      out[i] = 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+   }
+}
+ORACLE_API void oracle_tanh(float *out, const float *in, size_t n)
+{
+   for (size_t i = 0; i < n; ++i)
+      out[i] = tanhf(in[i]);
+}
+
+/* activation codes of include/sofie_hip.h */
+ORACLE_API void oracle_unary(float *out, const float *in, size_t n, int act, float alpha)
+{
+   switch (act) {
+   case 1: oracle_relu(out, in, n); break;
+   case 2: oracle_leaky_relu(out, in, n, alpha); break;
+   case 3: oracle_sigmoid(out, in, n); break;
+   case 4: oracle_gelu(out, in, n); break;
+   case 5: oracle_gelu_tanh(out, in, n); break;
+   case 6: oracle_tanh(out, in, n); break;
+   default:
+      if (out != in)
+         memmove(out, in, n * sizeof(float));
+   }
+}
+
+/* ROperator_Gemm<float>::Generate, CPU form (core/inc/SOFIE/operators/ROperator_Gemm.hxx:419-741):
+ * row-major A[M,K] (or [K,M] with transA), B[K,N] (or [N,K] with transB).
+ *   - a bias that is not Y-shaped is written into Y row by row (Copy for [N]/[1,N], Fill for [M,1] and
+ *     scalars) and beta becomes 1 (:578-617); a Y-shaped bias is passed to Gemm_Call as C with the
+ *     operator's beta; no bias forces beta = 0 (:491-499);
+ *   - the row-major product is obtained from the column-major BLAS by swapping the operands:
+ *     Gemm_Call(Y, transB, transA, n, m, k, alpha, B, A, beta, C) (:685-709);
+ *   - fused Relu / LeakyRelu run over Y afterwards (:724-738).
+ * bias_mode: 0 none, 1 row [N], 2 column [M,1], 3 scalar, 4 full [M,N]. act as in oracle_unary. */
+ORACLE_API void oracle_gemm_f32(int M, int N, int K, int transA, int transB, float alpha, float beta, const float *A,
+                                const float *B, const float *C, int bias_mode, int act, float act_alpha, float *Y)
+{
+   const float *c_arg = NULL;
+   if (bias_mode == 0) {
+      beta = 0.0f;
+   } else if (bias_mode == 4) {
+      c_arg = C;
+   } else {
+      beta = 1.0f;
+      for (int j = 0; j < M; ++j) {
+         float *row = Y + (size_t)N * j;
+         if (bias_mode == 1)
+            memcpy(row, C, sizeof(float) * (size_t)N);
+         else
+            for (int i = 0; i < N; ++i)
+               row[i] = (bias_mode == 2) ? C[j] : C[0];
+      }
+   }
+   oracle_gemm_call(Y, transB, transA, N, M, K, alpha, B, A, beta, c_arg);
+   oracle_unary(Y, Y, (size_t)M * (size_t)N, act, act_alpha);
+}
+
+/* ROperator_BasicBinary<float,Add>::Generate (core/inc/SOFIE/operators/ROperator_BasicBinary.hxx:380-510):
+ * nested loops over the output dims, a broadcast dim is read at index 0.  Shapes right-aligned, rank<=6. */
+ORACLE_API void oracle_add_broadcast(int rank, const int64_t *yshape, const int64_t *ashape, const int64_t *bshape,
+                                     const float *A, const float *B, float *Y)
+{
+   int64_t sa[6], sb[6], n = 1, ca = 1, cb = 1;
+   for (int d = rank - 1; d >= 0; --d) {
+      sa[d] = (ashape[d] == 1 && yshape[d] != 1) ? 0 : ca;
+      sb[d] = (bshape[d] == 1 && yshape[d] != 1) ? 0 : cb;
+      ca *= ashape[d];
+      cb *= bshape[d];
+      n *= yshape[d];
+   }
+   for (int64_t i = 0; i < n; ++i) {
+      int64_t rest = i, ia = 0, ib = 0;
+      for (int d = rank - 1; d >= 0; --d) {
+         int64_t idx = rest % yshape[d];
+         rest /= yshape[d];
+         ia += idx * sa[d];
+         ib += idx * sb[d];
+      }
+      Y[i] = A[ia] + B[ib];
+   }
+}
+
+/* UTILITY::Im2col (core/src/utils/SOFIE_common_helpers.cxx:47-83): rows (c,kh,kw), columns (oh,ow),
+ * zero outside the image; the unsigned-compare bounds test of :40-45. */
+static int in_range(int a, int b)
+{
+   return (unsigned)a < (unsigned)b;
+}
+ORACLE_API void oracle_im2col(const float *data_im, int channels, int height, int width, int kernel_h, int kernel_w,
+                              int pad_h_begin, int pad_h_end, int pad_w_begin, int pad_w_end, int stride_h, int stride_w,
+                              int dilation_h, int dilation_w, float *data_col)
+{
+   const int output_h = (height + pad_h_begin + pad_h_end - (dilation_h * (kernel_h - 1) + 1)) / stride_h + 1;
+   const int output_w = (width + pad_w_begin + pad_w_end - (dilation_w * (kernel_w - 1) + 1)) / stride_w + 1;
+   const int channel_size = height * width;
+   for (int channel = 0; channel < channels; ++channel, data_im += channel_size) {
+      for (int kr = 0; kr < kernel_h; ++kr) {
+         for (int kc = 0; kc < kernel_w; ++kc) {
+            int input_row = -pad_h_begin + kr * dilation_h;
+            for (int orow = 0; orow < output_h; ++orow, input_row += stride_h) {
+               if (!in_range(input_row, height)) {
+                  for (int oc = 0; oc < output_w; ++oc)
+                     *(data_col++) = 0.0f;
+               } else {
+                  int input_col = -pad_w_begin + kc * dilation_w;
+                  for (int oc = 0; oc < output_w; ++oc, input_col += stride_w)
+                     *(data_col++) = in_range(input_col, width) ? data_im[input_row * width + input_col] : 0.0f;
+               }
+            }
+         }
+      }
+   }
+}
+
+/* ROperator_Conv<float>::Generate for 1-D/2-D convolutions (core/inc/SOFIE/operators/ROperator_Conv.hxx:406-642):
+ *   1. the kernel is copied into the dilated layout tensor_<Y>_f, zero between the taps (:442-476);
+ *      from then on the convolution runs with kernel size k + (d-1)(k-1) and dilation 1 (:478);
+ *   2. for every image (and group): Im2col, then Gemm_Call(y, false,false, m=OH*OW, n=Cout/g,
+ *      k=Cin/g*KH*KW, 1, xcol, f, beta, bias) with the bias pre-broadcast to [Cout,OH,OW] and beta=1,
+ *      or beta=0 without a bias (:487-552, 560-616).
+ * X [N,C,H,W]; W [Cout, C/group, kh, kw]; pads {h_begin, w_begin, h_end, w_end}; Y [N,Cout,OH,OW].
+ * For a 1-D convolution pass H=1, kh=1, pads (0,p0,0,p1), stride_h=1, dil_h=1 (:517-523).
+ * `act`/`act_alpha`: an activation applied afterwards (a separate operator in the reference). */
+ORACLE_API int oracle_conv_f32(int N, int C, int H, int W, int Cout, int kh, int kw, int pad_h0, int pad_w0, int pad_h1,
+                               int pad_w1, int stride_h, int stride_w, int dil_h, int dil_w, int group, const float *X,
+                               const float *Wt, const float *bias, int act, float act_alpha, float *Y)
+{
+   const int Cg = C / group, Cout_g = Cout / group;
+   const int ekh = kh + (dil_h - 1) * (kh - 1), ekw = kw + (dil_w - 1) * (kw - 1);
+   const int OH = (H + pad_h0 + pad_h1 - ekh) / stride_h + 1;
+   const int OW = (W + pad_w0 + pad_w1 - ekw) / stride_w + 1;
+   const int m = OH * OW, k = Cg * ekh * ekw;
+   float *f = (float *)calloc((size_t)Cout * Cg * ekh * ekw, sizeof(float));
+   float *xcol = (float *)malloc(sizeof(float) * (size_t)k * (size_t)m);
+   float *bcast = bias ? (float *)malloc(sizeof(float) * (size_t)Cout * m) : NULL;
+   if (!f || !xcol || (bias && !bcast)) {
+      free(f);
+      free(xcol);
+      free(bcast);
+      return 1;
+   }
+   for (int oc = 0; oc < Cout; ++oc)
+      for (int ic = 0; ic < Cg; ++ic)
+         for (int y = 0; y < kh; ++y)
+            for (int x = 0; x < kw; ++x)
+               f[(size_t)oc * Cg * ekh * ekw + (size_t)ic * ekh * ekw + (size_t)y * dil_h * ekw + (size_t)x * dil_w] =
+                  Wt[(size_t)oc * Cg * kh * kw + (size_t)ic * kh * kw + (size_t)y * kw + x];
+   if (bias)
+      for (int oc = 0; oc < Cout; ++oc)
+         for (int i = 0; i < m; ++i)
+            bcast[(size_t)oc * m + i] = bias[oc];
+   const float beta = bias ? 1.0f : 0.0f;
+   for (int n = 0; n < N; ++n) {
+      for (int g = 0; g < group; ++g) {
+         size_t x_offset = (size_t)n * C * H * W + (size_t)g * Cg * H * W;
+         size_t g_offset = (size_t)g * Cout_g * m;
+         size_t out_offset = (size_t)n * Cout * m + g_offset;
+         oracle_im2col(X + x_offset, Cg, H, W, ekh, ekw, pad_h0, pad_h1, pad_w0, pad_w1, stride_h, stride_w, 1, 1, xcol);
+         oracle_gemm_call(Y + out_offset, 0, 0, m, Cout_g, k, 1.0f, xcol, f + (size_t)g * Cout_g * k, beta,
+                          bias ? bcast + g_offset : NULL);
+      }
+   }
+   oracle_unary(Y, Y, (size_t)N * Cout * m, act, act_alpha);
+   free(f);
+   free(xcol);
+   free(bcast);
+   return 0;
+}
+
+/* GlobalAveragePool = AveragePool with kernel == image (core/inc/SOFIE/operators/ROperator_Pool.hxx:225-237):
+ * sequential fp32 sum over the plane, then `value /= float(nsum)` (:362-368). */
+ORACLE_API void oracle_global_avg_pool(float *Y, const float *X, int NC, int HW)
+{
+   for (int p = 0; p < NC; ++p) {
+      float value = 0;
+      for (int i = 0; i < HW; ++i)
+         value += X[(size_t)p * HW + i];
+      value /= (float)HW;
+      Y[p] = value;
+   }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Memory planner: OrganizeMemory (core/inc/SOFIE/utils/shared/MemoryPlanner.inc:33-132).
+ * Tensor i lives in [begin[i], end[i]); events are swept in time order with frees (type 0) before
+ * allocations (type 1) at the same time; an allocation takes the smallest free block that fits
+ * (lowest offset among equals) from its start, else grows the pool; freed blocks merge with their
+ * neighbours.  Events with equal (time,type) are taken in tensor order here (the reference leaves
+ * that order to std::sort).  Returns 0, or 1 if some end <= begin, 2 if out of memory.
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct {
+   size_t off, size;
+} free_block;
+typedef struct {
+   int t, type, idx;
+} mem_event;
+static int cmp_event(const void *pa, const void *pb)
+{
+   const mem_event *a = (const mem_event *)pa, *b = (const mem_event *)pb;
+   if (a->t != b->t)
+      return a->t < b->t ? -1 : 1;
+   if (a->type != b->type)
+      return a->type < b->type ? -1 : 1;
+   return (a->idx > b->idx) - (a->idx < b->idx);
+}
+ORACLE_API int oracle_organize_memory(int n, const int *begin, const int *end, const size_t *size, size_t *offsets,
+                                      size_t *total_bytes, size_t *total_free_bytes, size_t *largest_free_block)
+{
+   for (int i = 0; i < n; ++i)
+      if (!(end[i] > begin[i]))
+         return 1;
+   mem_event *ev = (mem_event *)malloc(sizeof(mem_event) * (size_t)(2 * n + 1));
+   free_block *fl = (free_block *)malloc(sizeof(free_block) * (size_t)(n + 1)); /* sorted by offset */
+   char *live = (char *)calloc((size_t)n + 1, 1);
+   if (!ev || !fl || !live) {
+      free(ev);
+      free(fl);
+      free(live);
+      return 2;
+   }
+   for (int i = 0; i < n; ++i) {
+      ev[2 * i] = (mem_event){end[i], 0, i};
+      ev[2 * i + 1] = (mem_event){begin[i], 1, i};
+   }
+   qsort(ev, (size_t)(2 * n), sizeof(mem_event), cmp_event);
+   int nfree = 0;
+   size_t total = 0, tfree = 0, lfree = 0;
+   for (int e = 0; e < 2 * n; ++e) {
+      int idx = ev[e].idx;
+      if (ev[e].type == 0) {
+         if (!live[idx])
+            continue;
+         live[idx] = 0;
+         free_block fb = {offsets[idx], size[idx]};
+         int pos = 0;
+         while (pos < nfree && fl[pos].off < fb.off)
+            ++pos;
+         memmove(&fl[pos + 1], &fl[pos], sizeof(free_block) * (size_t)(nfree - pos));
+         fl[pos] = fb;
+         ++nfree;
+         if (pos > 0 && fl[pos - 1].off + fl[pos - 1].size == fl[pos].off) {
+            fl[pos - 1].size += fl[pos].size;
+            memmove(&fl[pos], &fl[pos + 1], sizeof(free_block) * (size_t)(nfree - pos - 1));
+            --nfree;
+            --pos;
+         }
+         if (pos + 1 < nfree && fl[pos].off + fl[pos].size == fl[pos + 1].off) {
+            fl[pos].size += fl[pos + 1].size;
+            memmove(&fl[pos + 1], &fl[pos + 2], sizeof(free_block) * (size_t)(nfree - pos - 2));
+            --nfree;
+         }
+      } else {
+         size_t need = size[idx];
+         int best = -1;
+         for (int i = 0; i < nfree; ++i)
+            if (fl[i].size >= need && (best < 0 || fl[i].size < fl[best].size))
+               best = i;
+         size_t before = total, off;
+         if (best >= 0) {
+            off = fl[best].off;
+            if (fl[best].size == need) {
+               memmove(&fl[best], &fl[best + 1], sizeof(free_block) * (size_t)(nfree - best - 1));
+               --nfree;
+            } else {
+               fl[best].off += need;
+               fl[best].size -= need;
+            }
+         } else {
+            off = total;
+            total += need;
+         }
+         offsets[idx] = off;
+         live[idx] = 1;
+         if (total > before) {
+            tfree = 0;
+            lfree = 0;
+            for (int i = 0; i < nfree; ++i) {
+               tfree += fl[i].size;
+               if (fl[i].size > lfree)
+                  lfree = fl[i].size;
+            }
+         }
+      }
+   }
+   *total_bytes = total;
+   *total_free_bytes = tfree;
+   *largest_free_block = lfree;
+   free(ev);
+   free(fl);
+   free(live);
+   return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Quantised operators (ONNX definitions; no counterpart in the reference -- see the header)
+ * ---------------------------------------------------------------------------------------------- */
+
+/* sat8(rne(v)): nearbyintf under the default rounding mode is round-half-to-even; NaN -> 0. */
+static inline int sat8_rne(float v)
+{
+   if (!(v == v))
+      return 0;
+   float r = nearbyintf(v);
+   if (r < -128.0f)
+      r = -128.0f;
+   if (r > 127.0f)
+      r = 127.0f;
+   return (int)r;
+}
+
+/* QuantizeLinear, per tensor, zero point 0: q = sat8(rne(x / scale)), fp32 division. */
+ORACLE_API void oracle_quantize_linear(int8_t *q, const float *x, size_t n, float scale)
+{
+   for (size_t i = 0; i < n; ++i)
+      q[i] = (int8_t)sat8_rne(x[i] / scale);
+}
+/* DequantizeLinear: y = float(q) * scale. */
+ORACLE_API void oracle_dequantize_linear_i8(float *y, const int8_t *q, size_t n, float scale)
+{
+   for (size_t i = 0; i < n; ++i)
+      y[i] = (float)q[i] * scale;
+}
+ORACLE_API void oracle_dequantize_linear_i32(float *y, const int32_t *q, size_t n, float scale)
+{
+   for (size_t i = 0; i < n; ++i)
+      y[i] = (float)q[i] * scale;
+}
+
+/* MatMulInteger: acc[m,n] = sum_k int32(A[m,k]) * int32(B[k,n]); A [M,K] row-major (or [K,M] with
+ * transA), B [K,N] row-major (or [N,K] with transB).  Threads split the rows. */
+ORACLE_API void oracle_matmul_integer(int M, int N, int K, int transA, int transB, const int8_t *A, const int8_t *B,
+                                      int32_t *acc)
+{
+   /* re-lay B as [N,K] so the inner loop is contiguous; the sum is exact in any order */
+   int8_t *bt = NULL, *at = NULL;
+   if (!transB) {
+      bt = (int8_t *)malloc((size_t)N * K + 1);
+      for (int k = 0; k < K; ++k)
+         for (int n = 0; n < N; ++n)
+            bt[(size_t)n * K + k] = B[(size_t)k * N + n];
+      B = bt;
+   }
+   if (transA) {
+      at = (int8_t *)malloc((size_t)M * K + 1);
+      for (int k = 0; k < K; ++k)
+         for (int m = 0; m < M; ++m)
+            at[(size_t)m * K + k] = A[(size_t)k * M + m];
+      A = at;
+   }
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+   for (int m = 0; m < M; ++m) {
+      const int8_t *a = A + (size_t)m * K;
+      for (int n = 0; n < N; ++n) {
+         const int8_t *b = B + (size_t)n * K;
+         int32_t s = 0;
+         for (int k = 0; k < K; ++k)
+            s += (int32_t)a[k] * (int32_t)b[k];
+         acc[(size_t)m * N + n] = s;
+      }
+   }
+   free(bt);
+   free(at);
+}
+
+/* The epilogue of the int8 Gemm, element by element (out kinds of include/sofie_hip.h):
+ *   acc += bias[n]; acc = max(acc,0) if relu_acc;
+ *   0: int32     1: float(acc)*s, then max(.,0) if relu_out     2: sat8(rne(float(acc)*s)), then max(.,0) if relu_out
+ *   3: sat8(rne((float(acc)*s)/q_scale))
+ * int32 -> fp32 conversion rounds to nearest even; one fp32 multiply, no fused multiply-add. */
+ORACLE_API void oracle_gemm_i8_epilogue(int M, int N, const int32_t *acc, const int32_t *bias, const float *scale,
+                                        float scale_scalar, float q_scale, int relu_acc, int relu_out, int out, void *Y)
+{
+   for (int m = 0; m < M; ++m) {
+      for (int n = 0; n < N; ++n) {
+         size_t i = (size_t)m * N + n;
+         int32_t a = acc[i] + (bias ? bias[n] : 0);
+         if (relu_acc && a < 0)
+            a = 0;
+         float s = scale ? scale[n] : scale_scalar;
+         switch (out) {
+         case 0: ((int32_t *)Y)[i] = a; break;
+         case 1: {
+            float v = (float)a * s;
+            if (relu_out && !(v > 0.0f))
+               v = 0.0f;
+            ((float *)Y)[i] = v;
+         } break;
+         case 2: {
+            int q = sat8_rne((float)a * s);
+            if (relu_out && q < 0)
+               q = 0;
+            ((int8_t *)Y)[i] = (int8_t)q;
+         } break;
+         default: {
+            float t = (float)a * s;
+            ((int8_t *)Y)[i] = (int8_t)sat8_rne(t / q_scale);
+         } break;
+         }
+      }
+   }
+}
+
+ORACLE_API int oracle_gemm_i8(int M, int N, int K, int transA, int transB, const int8_t *A, const int8_t *B,
+                              const int32_t *bias, const float *scale, float scale_scalar, float q_scale, int relu_acc,
+                              int relu_out, int out, void *Y)
+{
+   int32_t *acc = (int32_t *)malloc(sizeof(int32_t) * ((size_t)M * N + 1));
+   if (!acc)
+      return 1;
+   oracle_matmul_integer(M, N, K, transA, transB, A, B, acc);
+   oracle_gemm_i8_epilogue(M, N, acc, bias, scale, scale_scalar, q_scale, relu_acc, relu_out, out, Y);
+   free(acc);
+   return 0;
+}
+
+/* int8 convolution, direct 7-loop form: acc = sum X_i8 * W_i8 (+ bias_i32[co]); the output is NCHW.
+ * out: 0 int32, 1 float(acc)*scale[co] (then relu), 2 sat8(rne(float(acc)*scale[co])) then max(.,0) if relu. */
+ORACLE_API void oracle_conv_i8(int N, int C, int H, int W, int Cout, int kh, int kw, int pad_h0, int pad_w0, int pad_h1,
+                               int pad_w1, int stride_h, int stride_w, int dil_h, int dil_w, int group, const int8_t *X,
+                               const int8_t *Wt, const int32_t *bias, const float *scale, int relu, int out, void *Y)
+{
+   const int Cg = C / group, Cout_g = Cout / group;
+   const int OH = (H + pad_h0 + pad_h1 - (dil_h * (kh - 1) + 1)) / stride_h + 1;
+   const int OW = (W + pad_w0 + pad_w1 - (dil_w * (kw - 1) + 1)) / stride_w + 1;
+#ifdef _OPENMP
+#pragma omp parallel for collapse(2) schedule(static)
+#endif
+   for (int n = 0; n < N; ++n) {
+      for (int co = 0; co < Cout; ++co) {
+         int g = co / Cout_g;
+         for (int oh = 0; oh < OH; ++oh) {
+            for (int ow = 0; ow < OW; ++ow) {
+               int32_t a = bias ? bias[co] : 0;
+               for (int ci = 0; ci < Cg; ++ci) {
+                  for (int y = 0; y < kh; ++y) {
+                     int ih = oh * stride_h - pad_h0 + y * dil_h;
+                     if (!in_range(ih, H))
+                        continue;
+                     for (int x = 0; x < kw; ++x) {
+                        int iw = ow * stride_w - pad_w0 + x * dil_w;
+                        if (!in_range(iw, W))
+                           continue;
+                        a += (int32_t)X[(((size_t)n * C + g * Cg + ci) * H + ih) * W + iw] *
+                             (int32_t)Wt[(((size_t)co * Cg + ci) * kh + y) * kw + x];
+                     }
+                  }
+               }
+               size_t i = (((size_t)n * Cout + co) * OH + oh) * OW + ow;
+               if (out == 0) {
+                  ((int32_t *)Y)[i] = (relu && a < 0) ? 0 : a;
+               } else if (out == 1) {
+                  float v = (float)a * scale[co];
+                  ((float *)Y)[i] = relu ? ((v > 0.0f) ? v : 0.0f) : v;
+               } else {
+                  int q = sat8_rne((float)a * scale[co]);
+                  if (relu && q < 0)
+                     q = 0;
+                  ((int8_t *)Y)[i] = (int8_t)q;
+               }
+            }
+         }
+      }
+   }
+}
+
+/* Y = (float(sum_i32 over the plane) * scale) / float(HW) */
+ORACLE_API void oracle_global_avg_pool_i8(float *Y, const int8_t *X, int NC, int HW, float scale)
+{
+   for (int p = 0; p < NC; ++p) {
+      int32_t s = 0;
+      for (int i = 0; i < HW; ++i)
+         s += X[(size_t)p * HW + i];
+      Y[p] = ((float)s * scale) / (float)HW;
+   }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * FP8 (OCP e4m3fn: 1 sign, 4 exponent (bias 7), 3 mantissa; no infinity; 0x7f/0xff are NaN; max 448)
+ * ---------------------------------------------------------------------------------------------- */
+ORACLE_API float oracle_e4m3_to_f32(uint8_t v)
+{
+   int sign = v >> 7, e = (v >> 3) & 15, m = v & 7;
+   float r;
+   if (e == 15 && m == 7)
+      r = NAN;
+   else if (e == 0)
+      r = ldexpf((float)m, -9); /* subnormal: m/8 * 2^-6 */
+   else
+      r = ldexpf(1.0f + (float)m / 8.0f, e - 7);
+   return sign ? -r : r;
+}
+
+/* fp32 -> e4m3fn, round to nearest even, saturating to +-448 (also for +-inf); NaN -> 0x7f. */
+ORACLE_API uint8_t oracle_f32_to_e4m3(float x)
+{
+   if (x != x)
+      return 0x7f;
+   uint8_t sign = signbit(x) ? 0x80 : 0;
+   float a = fabsf(x);
+   if (a >= 448.0f)
+      return sign | 0x7e; /* 448 and above, including values that would round up past 448 */
+   int e;
+   (void)frexpf(a, &e); /* a = f * 2^e, f in [0.5,1) -> exponent of the leading bit is e-1 */
+   int exp = e - 1;
+   if (exp < -6)
+      exp = -6; /* subnormal range: fixed quantum 2^-9 */
+   float quantum = ldexpf(1.0f, exp - 3);
+   float q = nearbyintf(a / quantum); /* exact division by a power of two; ties to even */
+   float r = q * quantum;
+   if (r > 448.0f)
+      return sign | 0x7e;
+   /* encode r */
+   if (r < ldexpf(1.0f, -6))
+      return sign | (uint8_t)(r / ldexpf(1.0f, -9));
+   int e2;
+   float f2 = frexpf(r, &e2); /* r = f2 * 2^e2, f2 in [0.5,1) */
+   int be = e2 - 1 + 7;
+   int mant = (int)((f2 * 2.0f - 1.0f) * 8.0f);
+   return sign | (uint8_t)(be << 3) | (uint8_t)mant;
+}
+
+ORACLE_API void oracle_quantize_fp8(uint8_t *q, const float *x, size_t n, float scale)
+{
+   for (size_t i = 0; i < n; ++i)
+      q[i] = oracle_f32_to_e4m3(x[i] / scale);
+}
+
+/* fp32 -> bf16 bits, round to nearest even; NaN stays NaN. */
+ORACLE_API uint16_t oracle_f32_to_bf16(float x)
+{
+   uint32_t u;
+   memcpy(&u, &x, 4);
+   if ((u & 0x7fffffffu) > 0x7f800000u)
+      return (uint16_t)((u >> 16) | 0x40);
+   u += 0x7fffu + ((u >> 16) & 1u);
+   return (uint16_t)(u >> 16);
+}
+
+/* FP8 Gemm arbiter: products and sums in float64 (every e4m3 product is exact in fp32 and in fp64);
+ * v = float(acc) * scale + bias[n]; activation in fp32; output fp32 (out=1) or bf16 bits (out=0).
+ * Also returns sum_k |a*b| per element (fp32) when `abs_sum` is not NULL, for the error bound
+ * K * 2^-24 * sum|a*b| * scale on the hardware's fp32 accumulation. */
+ORACLE_API void oracle_gemm_fp8(int M, int N, int K, int transB, const uint8_t *A, const uint8_t *B, const float *bias,
+                                float scale, int act, int out, void *Y, float *abs_sum)
+{
+   float lut[256];
+   for (int i = 0; i < 256; ++i)
+      lut[i] = oracle_e4m3_to_f32((uint8_t)i);
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+   for (int m = 0; m < M; ++m) {
+      for (int n = 0; n < N; ++n) {
+         double s = 0.0, sa = 0.0;
+         for (int k = 0; k < K; ++k) {
+            double a = lut[A[(size_t)m * K + k]];
+            double b = transB ? lut[B[(size_t)n * K + k]] : lut[B[(size_t)k * N + n]];
+            s += a * b;
+            sa += fabs(a * b);
+         }
+         float v = (float)s * scale;
+         if (bias)
+            v = v + bias[n];
+         oracle_unary(&v, &v, 1, act, 0.0f);
+         size_t i = (size_t)m * N + n;
+         if (out == 1)
+            ((float *)Y)[i] = v;
+         else
+            ((uint16_t *)Y)[i] = oracle_f32_to_bf16(v);
+         if (abs_sum)
+            abs_sum[i] = (float)sa;
+      }
+   }
+}
+
+ORACLE_API int oracle_num_threads(void)
+{
+#ifdef _OPENMP
+   return omp_get_max_threads();
+#else
+   return 1;
+#endif
+}
+ORACLE_API void oracle_set_num_threads(int n)
+{
+#ifdef _OPENMP
+   omp_set_num_threads(n);
+#else
+   (void)n;
+#endif
+}

@@ -1,0 +1,80 @@
+// Shared declarations of the gfx950 runtime behind include/sofie_hip.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include "sofie_hip.h"
+
+struct sofie_hip_ctx {
+   int device = 0;
+   hipStream_t stream = nullptr;
+   bool owns_stream = false;
+   char *arena = nullptr;
+   size_t arena_bytes = 0;
+   bool owns_arena = false;
+   hipEvent_t ev0 = nullptr, ev1 = nullptr;
+};
+
+namespace sofie_hip {
+
+// Records the text returned by sofie_hip_last_error() for the calling thread and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define SOFIE_HIP_CHECK(expr)                                                                         \
+   do {                                                                                               \
+      hipError_t e_ = (expr);                                                                         \
+      if (e_ != hipSuccess)                                                                           \
+         return ::sofie_hip::fail(SOFIE_HIP_ERR_RUNTIME, "%s failed: %s (%s:%d)", #expr,              \
+                                  hipGetErrorString(e_), __FILE__, __LINE__);                         \
+   } while (0)
+
+#define SOFIE_HIP_REQUIRE(cond, ...)                                                                  \
+   do {                                                                                               \
+      if (!(cond))                                                                                    \
+         return ::sofie_hip::fail(SOFIE_HIP_ERR_INVALID, __VA_ARGS__);                                \
+   } while (0)
+
+inline int launch_status(const char *what)
+{
+   hipError_t e = hipGetLastError();
+   if (e != hipSuccess)
+      return fail(SOFIE_HIP_ERR_RUNTIME, "launch of %s failed: %s", what, hipGetErrorString(e));
+   return SOFIE_HIP_OK;
+}
+
+// ---- scalar formulas shared by every epilogue --------------------------------------------------
+
+// Activation on fp32, the reference's CPU formulas (see sofie_hip.h for the citations).
+__device__ __forceinline__ float apply_act(float v, int act, float alpha)
+{
+   switch (act) {
+   case SOFIE_ACT_RELU: return (v > 0.0f) ? v : 0.0f;
+   case SOFIE_ACT_LEAKYRELU: return (v >= 0.0f) ? v : alpha * v;
+   case SOFIE_ACT_SIGMOID: return 1.0f / (1.0f + expf(-v));
+   case SOFIE_ACT_GELU: return 0.5f * v * (1.0f + erff(v * 0.7071067811865475f));
+   case SOFIE_ACT_GELU_TANH: return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+   case SOFIE_ACT_TANH: return tanhf(v);
+   default: return v;
+   }
+}
+
+// sat8(rne(v)): round half to even, saturate to [-128,127]; NaN -> 0 (matches the CPU restatement,
+// which clamps before converting and maps NaN to 0).
+__device__ __forceinline__ int quantize_rne_sat8(float v)
+{
+   if (!(v == v))
+      return 0;
+   float r = __builtin_rintf(v); // v_rndne_f32
+   r = fminf(fmaxf(r, -128.0f), 127.0f);
+   return (int)r;
+}
+
+// fp32 multiply that the compiler may not fuse with a neighbouring add.
+__device__ __forceinline__ float mul_nofma(float a, float b)
+{
+   return __fmul_rn(a, b);
+}
+
+} // namespace sofie_hip

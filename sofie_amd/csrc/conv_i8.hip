@@ -1,0 +1,242 @@
+// int8 convolution as a GEMM over the whole batch: rows = output pixels (image, oh, ow), columns =
+// output channels, K = (kh, kw, ci) with ci fastest.  The weights are re-laid out once into
+// [Cout][Kp] (Kp = K rounded up to 16, zero filled); the column matrix of a group of images is built
+// in the workspace and multiplied on the matrix cores with the requantisation fused into the store.
+// Activations may be NCHW (the ONNX layout) or NHWC (channels fastest: what a chain of convolutions
+// keeps between layers, since it makes both the gather and the store contiguous).
+#include "i8_epilogue.hpp"
+
+namespace sofie_hip {
+
+struct ConvGeom {
+   int C, H, W, kh, kw, OH, OW, pad_h0, pad_w0, stride_h, stride_w, dil_h, dil_w;
+   int Cg, K, Kp; // channels per group, kh*kw*Cg, K rounded up to 16
+};
+
+// [Cout][Cg][kh][kw] -> [Cout][Kp] with k' = (ky*kw + kx)*Cg + ci
+__global__ __launch_bounds__(256) void pack_conv_weight_kernel(int8_t *__restrict__ dst, const int8_t *__restrict__ src, int Cout,
+                                                                ConvGeom g)
+{
+   const size_t total = (size_t)Cout * g.Kp;
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += stride) {
+      int co = (int)(i / g.Kp), k = (int)(i % g.Kp);
+      int8_t v = 0;
+      if (k < g.K) {
+         int ci = k % g.Cg, t = k / g.Cg;
+         int kx = t % g.kw, ky = t / g.kw;
+         v = src[(((size_t)co * g.Cg + ci) * g.kh + ky) * g.kw + kx];
+      }
+      dst[i] = v;
+   }
+}
+
+// One thread builds one 16-byte chunk of one row of the column matrix.
+template <bool NHWC_FAST>
+__global__ __launch_bounds__(256) void im2col_i8_kernel(int8_t *__restrict__ col, const int8_t *__restrict__ X, ConvGeom g,
+                                                         int c_first, int x_nhwc, long long m_first, long long rows)
+{
+   const int cpr = g.Kp / 16;
+   const size_t total = (size_t)rows * cpr;
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += stride) {
+      const long long m = m_first + (long long)(i / cpr);
+      const int chunk = (int)(i % cpr);
+      const int ow = (int)(m % g.OW);
+      const long long t = m / g.OW;
+      const int oh = (int)(t % g.OH);
+      const long long img = t / g.OH;
+      v4i out = v4i{0, 0, 0, 0};
+      if (NHWC_FAST) {
+         // Cg % 16 == 0: the chunk is 16 consecutive channels of one tap
+         const int k = chunk * 16;
+         const int ci = k % g.Cg, tap = k / g.Cg;
+         const int kx = tap % g.kw, ky = tap / g.kw;
+         const int ih = oh * g.stride_h - g.pad_h0 + ky * g.dil_h;
+         const int iw = ow * g.stride_w - g.pad_w0 + kx * g.dil_w;
+         if (k < g.K && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W)
+            out = *(const v4i *)(X + (((size_t)img * g.H + ih) * g.W + iw) * g.C + c_first + ci);
+      } else {
+         union {
+            v4i v;
+            int8_t b[16];
+         } u;
+         u.v = out;
+#pragma unroll
+         for (int j = 0; j < 16; ++j) {
+            const int k = chunk * 16 + j;
+            if (k < g.K) {
+               const int ci = k % g.Cg, tap = k / g.Cg;
+               const int kx = tap % g.kw, ky = tap / g.kw;
+               const int ih = oh * g.stride_h - g.pad_h0 + ky * g.dil_h;
+               const int iw = ow * g.stride_w - g.pad_w0 + kx * g.dil_w;
+               if ((unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W) {
+                  const size_t idx = x_nhwc ? (((size_t)img * g.H + ih) * g.W + iw) * g.C + c_first + ci
+                                            : (((size_t)img * g.C + c_first + ci) * g.H + ih) * g.W + iw;
+                  u.b[j] = X[idx];
+               }
+            }
+         }
+         out = u.v;
+      }
+      *(v4i *)(col + ((size_t)(m - m_first) * g.Kp) + chunk * 16) = out;
+   }
+}
+
+static inline size_t round256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+static int check_conv(const sofie_conv_desc *d, ConvGeom &g, const char *who)
+{
+   SOFIE_HIP_REQUIRE(d->N >= 0 && d->C > 0 && d->H > 0 && d->W > 0 && d->Cout > 0 && d->kh > 0 && d->kw > 0, "%s: bad shape", who);
+   SOFIE_HIP_REQUIRE(d->group > 0 && d->C % d->group == 0 && d->Cout % d->group == 0, "%s: group %d does not divide the channels", who, d->group);
+   SOFIE_HIP_REQUIRE(d->stride_h > 0 && d->stride_w > 0 && d->dil_h > 0 && d->dil_w > 0, "%s: bad stride or dilation", who);
+   SOFIE_HIP_REQUIRE(d->pad_h0 >= 0 && d->pad_w0 >= 0 && d->pad_h1 >= 0 && d->pad_w1 >= 0, "%s: negative padding", who);
+   const int eff_kh = d->dil_h * (d->kh - 1) + 1, eff_kw = d->dil_w * (d->kw - 1) + 1;
+   SOFIE_HIP_REQUIRE(d->H + d->pad_h0 + d->pad_h1 >= eff_kh && d->W + d->pad_w0 + d->pad_w1 >= eff_kw,
+                     "%s: kernel larger than the padded image", who);
+   const int OH = (d->H + d->pad_h0 + d->pad_h1 - eff_kh) / d->stride_h + 1;
+   const int OW = (d->W + d->pad_w0 + d->pad_w1 - eff_kw) / d->stride_w + 1;
+   SOFIE_HIP_REQUIRE(OH == d->OH && OW == d->OW, "%s: output shape %dx%d does not match the descriptor's %dx%d", who, OH, OW, d->OH, d->OW);
+   g.C = d->C; g.H = d->H; g.W = d->W; g.kh = d->kh; g.kw = d->kw; g.OH = OH; g.OW = OW;
+   g.pad_h0 = d->pad_h0; g.pad_w0 = d->pad_w0; g.stride_h = d->stride_h; g.stride_w = d->stride_w;
+   g.dil_h = d->dil_h; g.dil_w = d->dil_w;
+   g.Cg = d->C / d->group;
+   const long long K = (long long)g.Cg * d->kh * d->kw;
+   SOFIE_HIP_REQUIRE(K < (1 << 24), "%s: reduction too long", who);
+   g.K = (int)K;
+   g.Kp = (g.K + 15) & ~15;
+   return SOFIE_HIP_OK;
+}
+
+} // namespace sofie_hip
+
+using namespace sofie_hip;
+
+extern "C" {
+
+size_t sofie_hip_conv_weight_i8_packed_bytes(const sofie_conv_desc *d)
+{
+   if (!d || d->group <= 0)
+      return 0;
+   size_t K = (size_t)(d->C / d->group) * d->kh * d->kw;
+   return round256((size_t)d->Cout * ((K + 15) & ~(size_t)15));
+}
+
+int sofie_hip_pack_conv_weight_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, int8_t *dst, const int8_t *src)
+{
+   SOFIE_HIP_REQUIRE(ctx && d && dst && src, "sofie_hip_pack_conv_weight_i8: NULL argument");
+   ConvGeom g;
+   int st = check_conv(d, g, "sofie_hip_pack_conv_weight_i8");
+   if (st)
+      return st;
+   size_t total = (size_t)d->Cout * g.Kp;
+   size_t blocks = (total + 255) / 256;
+   if (blocks > 4096)
+      blocks = 4096;
+   hipLaunchKernelGGL(pack_conv_weight_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, dst, src, d->Cout, g);
+   return launch_status("pack_conv_weight_kernel");
+}
+
+size_t sofie_hip_conv_i8_workspace(const sofie_conv_desc *d, const sofie_conv_i8_args *a)
+{
+   if (!d || !a || d->group <= 0)
+      return 0;
+   size_t K = (size_t)(d->C / d->group) * d->kh * d->kw;
+   size_t Kp = (K + 15) & ~(size_t)15;
+   size_t need = round256((size_t)d->OH * d->OW * Kp); // the column matrix of one image
+   if (!a->w_is_packed)
+      need += sofie_hip_conv_weight_i8_packed_bytes(d);
+   return need;
+}
+
+int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_conv_i8_args *a)
+{
+   SOFIE_HIP_REQUIRE(ctx && d && a, "sofie_hip_conv_i8: NULL argument");
+   ConvGeom g;
+   int st = check_conv(d, g, "sofie_hip_conv_i8");
+   if (st)
+      return st;
+   SOFIE_HIP_REQUIRE(a->out == SOFIE_I8OUT_I32 || a->out == SOFIE_I8OUT_F32 || a->out == SOFIE_I8OUT_I8,
+                     "sofie_hip_conv_i8: unknown output kind %d", a->out);
+   SOFIE_HIP_REQUIRE((a->x_layout == SOFIE_LAYOUT_NCHW || a->x_layout == SOFIE_LAYOUT_NHWC) &&
+                        (a->y_layout == SOFIE_LAYOUT_NCHW || a->y_layout == SOFIE_LAYOUT_NHWC),
+                     "sofie_hip_conv_i8: unknown layout");
+   SOFIE_HIP_REQUIRE(a->out == SOFIE_I8OUT_I32 || a->scale != nullptr, "sofie_hip_conv_i8: per-channel scale is NULL");
+   if (d->N == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(a->X && a->W && a->Y, "sofie_hip_conv_i8: NULL tensor pointer");
+   const size_t need = sofie_hip_conv_i8_workspace(d, a);
+   SOFIE_HIP_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, "sofie_hip_conv_i8: a workspace of at least %zu bytes is needed", need);
+   SOFIE_HIP_REQUIRE(((uintptr_t)a->workspace & 255) == 0, "sofie_hip_conv_i8: workspace must be 256-byte aligned");
+
+   char *ws = (char *)a->workspace;
+   size_t ws_left = a->workspace_bytes;
+   const int8_t *Wp = a->W;
+   if (!a->w_is_packed) {
+      st = sofie_hip_pack_conv_weight_i8(ctx, d, (int8_t *)ws, a->W);
+      if (st)
+         return st;
+      Wp = (const int8_t *)ws;
+      size_t wb = sofie_hip_conv_weight_i8_packed_bytes(d);
+      ws += wb;
+      ws_left -= wb;
+   }
+   const int OHW = g.OH * g.OW;
+   const size_t per_image = (size_t)OHW * g.Kp;
+   long long imgs_per_chunk = (long long)(ws_left / per_image);
+   // keep one column matrix within reach of the 256 MB last-level cache
+   const long long cap = (long long)((192u << 20) / per_image);
+   if (imgs_per_chunk > cap)
+      imgs_per_chunk = cap > 0 ? cap : 1;
+   if (imgs_per_chunk > d->N)
+      imgs_per_chunk = d->N;
+   SOFIE_HIP_REQUIRE(imgs_per_chunk >= 1, "sofie_hip_conv_i8: workspace too small for one image");
+   SOFIE_HIP_REQUIRE(imgs_per_chunk * OHW < (1LL << 31), "sofie_hip_conv_i8: too many rows per chunk");
+   const int Cout_g = d->Cout / d->group;
+   const size_t esz = a->out == SOFIE_I8OUT_I8 ? 1 : 4;
+   const bool fast = a->x_layout == SOFIE_LAYOUT_NHWC && (g.Cg % 16 == 0) && (d->C % 16 == 0) && (((uintptr_t)a->X & 15) == 0);
+
+   for (long long img0 = 0; img0 < d->N; img0 += imgs_per_chunk) {
+      const long long imgs = (d->N - img0) < imgs_per_chunk ? (d->N - img0) : imgs_per_chunk;
+      const long long rows = imgs * OHW;
+      for (int grp = 0; grp < d->group; ++grp) {
+         size_t work = (size_t)rows * (g.Kp / 16);
+         size_t blocks = (work + 255) / 256;
+         if (blocks > 16384)
+            blocks = 16384;
+         if (fast)
+            hipLaunchKernelGGL(im2col_i8_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (int8_t *)ws, a->X, g,
+                               grp * g.Cg, 1, img0 * OHW, rows);
+         else
+            hipLaunchKernelGGL(im2col_i8_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (int8_t *)ws, a->X, g,
+                               grp * g.Cg, a->x_layout == SOFIE_LAYOUT_NHWC, img0 * OHW, rows);
+         st = launch_status("im2col_i8_kernel");
+         if (st)
+            return st;
+         I8Epilogue ep;
+         ep.bias = a->bias;
+         ep.scale = a->scale;
+         ep.scale_scalar = 1.0f;
+         ep.q_scale = 1.0f;
+         ep.relu_acc = (a->out == SOFIE_I8OUT_I32) ? a->relu : 0;
+         ep.relu_out = (a->out == SOFIE_I8OUT_I32) ? 0 : a->relu;
+         ep.out = a->out;
+         ep.ldy = d->Cout;
+         ep.n_offset = grp * Cout_g;
+         if (a->y_layout == SOFIE_LAYOUT_NHWC) {
+            ep.nchw_ohw = 0;
+            ep.Y = (char *)a->Y + (size_t)img0 * OHW * d->Cout * esz;
+         } else {
+            ep.nchw_ohw = OHW;
+            ep.Y = (char *)a->Y + (size_t)img0 * d->Cout * OHW * esz;
+         }
+         st = gemm_i8_nt(ctx->stream, (const int8_t *)ws, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.Kp, g.Kp, g.Kp, ep,
+                         forced_i8_tile());
+         if (st)
+            return st;
+      }
+   }
+   return SOFIE_HIP_OK;
+}
+
+} // extern "C"

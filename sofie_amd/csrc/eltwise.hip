@@ -1,0 +1,240 @@
+// HBM-bound elementwise operators: QuantizeLinear / DequantizeLinear, the stand-alone activations,
+// broadcast Add, GlobalAveragePool.  Each thread moves 16 bytes of the widest operand per step and
+// the grid strides over the tensor, so the launches stay coalesced for any length.
+#include "common.hpp"
+
+namespace sofie_hip {
+
+static inline unsigned grid_for(size_t work_items, unsigned block = 256, unsigned max_blocks = 256 * 32)
+{
+   size_t b = (work_items + block - 1) / block;
+   if (b < 1)
+      b = 1;
+   if (b > max_blocks)
+      b = max_blocks;
+   return (unsigned)b;
+}
+
+// q = sat8(rne(x / scale)), fp32 division (ONNX QuantizeLinear, zero point 0)
+__global__ __launch_bounds__(256) void quantize_linear_kernel(int8_t *__restrict__ dst, const float *__restrict__ src,
+                                                               size_t n, float scale, int vec)
+{
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+   if (vec) {
+      const size_t n4 = n / 4;
+      for (; i < n4; i += stride) {
+         float4 v = ((const float4 *)src)[i];
+         int q0 = quantize_rne_sat8(__fdiv_rn(v.x, scale));
+         int q1 = quantize_rne_sat8(__fdiv_rn(v.y, scale));
+         int q2 = quantize_rne_sat8(__fdiv_rn(v.z, scale));
+         int q3 = quantize_rne_sat8(__fdiv_rn(v.w, scale));
+         ((uint32_t *)dst)[i] = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) |
+                                ((uint32_t)(q3 & 0xff) << 24);
+      }
+      i = n4 * 4 + (blockIdx.x * (size_t)blockDim.x + threadIdx.x);
+      if (i < n)
+         dst[i] = (int8_t)quantize_rne_sat8(__fdiv_rn(src[i], scale));
+   } else {
+      for (; i < n; i += stride)
+         dst[i] = (int8_t)quantize_rne_sat8(__fdiv_rn(src[i], scale));
+   }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void dequantize_linear_kernel(float *__restrict__ dst, const T *__restrict__ src, size_t n,
+                                                                 float scale)
+{
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += stride)
+      dst[i] = mul_nofma((float)src[i], scale);
+}
+
+__global__ __launch_bounds__(256) void unary_f32_kernel(float *dst, const float *src, size_t n, int act, float alpha, int vec)
+{
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+   if (vec) {
+      const size_t n4 = n / 4;
+      for (; i < n4; i += stride) {
+         float4 v = ((const float4 *)src)[i];
+         v.x = apply_act(v.x, act, alpha);
+         v.y = apply_act(v.y, act, alpha);
+         v.z = apply_act(v.z, act, alpha);
+         v.w = apply_act(v.w, act, alpha);
+         ((float4 *)dst)[i] = v;
+      }
+      i = n4 * 4 + (blockIdx.x * (size_t)blockDim.x + threadIdx.x);
+      if (i < n)
+         dst[i] = apply_act(src[i], act, alpha);
+   } else {
+      for (; i < n; i += stride)
+         dst[i] = apply_act(src[i], act, alpha);
+   }
+}
+
+struct AddShape {
+   int rank;
+   long long y[6], sa[6], sb[6]; // output dims, element strides of A and B (0 where broadcast)
+};
+
+__global__ __launch_bounds__(256) void add_f32_kernel(float *__restrict__ Y, const float *__restrict__ A,
+                                                       const float *__restrict__ B, size_t n, AddShape sh)
+{
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+      size_t rest = i;
+      long long ia = 0, ib = 0;
+      for (int d = sh.rank - 1; d >= 0; --d) {
+         long long idx = (long long)(rest % (size_t)sh.y[d]);
+         rest /= (size_t)sh.y[d];
+         ia += idx * sh.sa[d];
+         ib += idx * sh.sb[d];
+      }
+      Y[i] = A[ia] + B[ib];
+   }
+}
+
+// One wave per (n,c) plane: lanes stride over the plane, then a wave reduction.
+template <typename T, typename ACC>
+__global__ __launch_bounds__(256) void gap_kernel(float *__restrict__ Y, const T *__restrict__ X, int NC, int HW, float mul)
+{
+   const int plane = blockIdx.x * 4 + (threadIdx.x >> 6);
+   const int lane = threadIdx.x & 63;
+   if (plane >= NC)
+      return;
+   const T *p = X + (size_t)plane * HW;
+   ACC s = 0;
+   for (int i = lane; i < HW; i += 64)
+      s += (ACC)p[i];
+#pragma unroll
+   for (int off = 32; off > 0; off >>= 1)
+      s += __shfl_xor(s, off, 64);
+   // fp32 input: sum / HW as the reference's pooling loop ends with `value /= float(nsum)`
+   // (core/inc/SOFIE/operators/ROperator_Pool.hxx:362-368); int8 input: (float(sum) * scale) / HW
+   if (lane == 0)
+      Y[plane] = __fdiv_rn(mul_nofma((float)s, mul), (float)HW);
+}
+
+// NHWC int8 input: one workgroup per image; thread c (strided) sums channel c over the pixels, so
+// consecutive lanes read consecutive bytes.
+__global__ __launch_bounds__(256) void gap_i8_nhwc_kernel(float *__restrict__ Y, const int8_t *__restrict__ X, int C, int HW,
+                                                           float scale)
+{
+   const int8_t *p = X + (size_t)blockIdx.x * HW * C;
+   for (int c = threadIdx.x; c < C; c += blockDim.x) {
+      int s = 0;
+      for (int i = 0; i < HW; ++i)
+         s += (int)p[(size_t)i * C + c];
+      Y[(size_t)blockIdx.x * C + c] = __fdiv_rn(mul_nofma((float)s, scale), (float)HW);
+   }
+}
+
+} // namespace sofie_hip
+
+using namespace sofie_hip;
+
+extern "C" {
+
+int sofie_hip_quantize_linear(sofie_hip_ctx *ctx, int8_t *dst, const float *src, size_t n, float scale)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_quantize_linear: ctx is NULL");
+   if (n == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(dst && src, "sofie_hip_quantize_linear: NULL pointer");
+   SOFIE_HIP_REQUIRE(scale > 0.0f, "sofie_hip_quantize_linear: scale must be positive");
+   const int vec = (((uintptr_t)src & 15) == 0) && (((uintptr_t)dst & 3) == 0);
+   hipLaunchKernelGGL(quantize_linear_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(256), 0, ctx->stream, dst, src, n, scale, vec);
+   return launch_status("quantize_linear_kernel");
+}
+
+int sofie_hip_dequantize_linear_i8(sofie_hip_ctx *ctx, float *dst, const int8_t *src, size_t n, float scale)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_dequantize_linear_i8: ctx is NULL");
+   if (n == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(dst && src, "sofie_hip_dequantize_linear_i8: NULL pointer");
+   hipLaunchKernelGGL(dequantize_linear_kernel<int8_t>, dim3(grid_for(n)), dim3(256), 0, ctx->stream, dst, src, n, scale);
+   return launch_status("dequantize_linear_kernel");
+}
+
+int sofie_hip_dequantize_linear_i32(sofie_hip_ctx *ctx, float *dst, const int32_t *src, size_t n, float scale)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_dequantize_linear_i32: ctx is NULL");
+   if (n == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(dst && src, "sofie_hip_dequantize_linear_i32: NULL pointer");
+   hipLaunchKernelGGL(dequantize_linear_kernel<int32_t>, dim3(grid_for(n)), dim3(256), 0, ctx->stream, dst, src, n, scale);
+   return launch_status("dequantize_linear_kernel");
+}
+
+int sofie_hip_unary_f32(sofie_hip_ctx *ctx, float *dst, const float *src, size_t n, int32_t act, float act_alpha)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_unary_f32: ctx is NULL");
+   SOFIE_HIP_REQUIRE(act >= SOFIE_ACT_NONE && act <= SOFIE_ACT_TANH, "sofie_hip_unary_f32: unknown activation %d", act);
+   if (n == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(dst && src, "sofie_hip_unary_f32: NULL pointer");
+   const int vec = (((uintptr_t)src & 15) == 0) && (((uintptr_t)dst & 15) == 0);
+   hipLaunchKernelGGL(unary_f32_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(256), 0, ctx->stream, dst, src, n, act, act_alpha, vec);
+   return launch_status("unary_f32_kernel");
+}
+
+int sofie_hip_add_f32(sofie_hip_ctx *ctx, const sofie_add_desc *d)
+{
+   SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_add_f32: NULL argument");
+   SOFIE_HIP_REQUIRE(d->rank >= 0 && d->rank <= 6, "sofie_hip_add_f32: rank %d not in [0,6]", d->rank);
+   AddShape sh;
+   sh.rank = d->rank;
+   size_t n = 1;
+   long long stride_a = 1, stride_b = 1;
+   for (int i = d->rank - 1; i >= 0; --i) {
+      SOFIE_HIP_REQUIRE(d->y_shape[i] >= 0, "sofie_hip_add_f32: negative dimension");
+      SOFIE_HIP_REQUIRE((d->a_shape[i] == d->y_shape[i] || d->a_shape[i] == 1) &&
+                           (d->b_shape[i] == d->y_shape[i] || d->b_shape[i] == 1),
+                        "sofie_hip_add_f32: operand dimension %d cannot be broadcast to the output", i);
+      sh.y[i] = d->y_shape[i];
+      sh.sa[i] = (d->a_shape[i] == 1 && d->y_shape[i] != 1) ? 0 : stride_a;
+      sh.sb[i] = (d->b_shape[i] == 1 && d->y_shape[i] != 1) ? 0 : stride_b;
+      stride_a *= d->a_shape[i];
+      stride_b *= d->b_shape[i];
+      n *= (size_t)d->y_shape[i];
+   }
+   if (n == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(d->A && d->B && d->Y, "sofie_hip_add_f32: NULL pointer");
+   hipLaunchKernelGGL(add_f32_kernel, dim3(grid_for(n)), dim3(256), 0, ctx->stream, d->Y, d->A, d->B, n, sh);
+   return launch_status("add_f32_kernel");
+}
+
+int sofie_hip_global_avg_pool_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t NC, int32_t HW)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_global_avg_pool_f32: ctx is NULL");
+   SOFIE_HIP_REQUIRE(NC >= 0 && HW > 0, "sofie_hip_global_avg_pool_f32: bad shape");
+   if (NC == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(Y && X, "sofie_hip_global_avg_pool_f32: NULL pointer");
+   hipLaunchKernelGGL((gap_kernel<float, float>), dim3((NC + 3) / 4), dim3(256), 0, ctx->stream, Y, X, NC, HW, 1.0f);
+   return launch_status("gap_kernel");
+}
+
+int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y, const int8_t *X, int32_t N, int32_t C, int32_t HW,
+                                 int32_t x_layout, float scale)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_global_avg_pool_i8: ctx is NULL");
+   SOFIE_HIP_REQUIRE(N >= 0 && C > 0 && HW > 0, "sofie_hip_global_avg_pool_i8: bad shape");
+   SOFIE_HIP_REQUIRE(x_layout == SOFIE_LAYOUT_NCHW || x_layout == SOFIE_LAYOUT_NHWC, "sofie_hip_global_avg_pool_i8: unknown layout");
+   SOFIE_HIP_REQUIRE((long long)N * C < (1LL << 31), "sofie_hip_global_avg_pool_i8: too many planes");
+   if (N == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(Y && X, "sofie_hip_global_avg_pool_i8: NULL pointer");
+   if (x_layout == SOFIE_LAYOUT_NHWC) {
+      hipLaunchKernelGGL(gap_i8_nhwc_kernel, dim3((unsigned)N), dim3(256), 0, ctx->stream, Y, X, C, HW, scale);
+      return launch_status("gap_i8_nhwc_kernel");
+   }
+   const int NC = N * C;
+   hipLaunchKernelGGL((gap_kernel<int8_t, int>), dim3((NC + 3) / 4), dim3(256), 0, ctx->stream, Y, X, NC, HW, scale);
+   return launch_status("gap_kernel");
+}
+
+} // extern "C"

@@ -1,0 +1,253 @@
+// fp32 Gemm / MatMul and fp32 convolution (implicit GEMM) with the bias + activation epilogue fused
+// into the store.  These are the small-batch, HBM/latency-bound operators of the fp32 path: tiles of
+// 64x64 outputs, K walked in slabs of 16 staged through LDS, 4x4 outputs per lane, fp32 FMA.
+// The operand fetch is a functor, so the same tile loop serves a strided/transposed Gemm and a
+// convolution whose column matrix is gathered on the fly (no materialised im2col).
+#include "common.hpp"
+
+namespace sofie_hip {
+
+constexpr int F32_BM = 64, F32_BN = 64, F32_BK = 16;
+
+struct GemmOperandA {
+   const float *p;
+   long long sm, sk; // element strides of op(A)[m,k]
+   __device__ __forceinline__ float operator()(int m, int k) const { return p[m * sm + k * sk]; }
+};
+struct GemmOperandB {
+   const float *p;
+   long long sk, sn; // element strides of op(B)[k,n]
+   __device__ __forceinline__ float operator()(int k, int n) const { return p[k * sk + n * sn]; }
+};
+
+struct F32Epilogue {
+   float alpha, beta;
+   const float *C;
+   int bias_mode;
+   long long ldc;
+   int act;
+   float act_alpha;
+};
+
+__device__ __forceinline__ float f32_epilogue(const F32Epilogue &ep, float acc, int m, int n)
+{
+   float v = ep.alpha * acc;
+   switch (ep.bias_mode) {
+   case SOFIE_BIAS_ROW: v += ep.C[n]; break;
+   case SOFIE_BIAS_COL: v += ep.C[m]; break;
+   case SOFIE_BIAS_SCALAR: v += ep.C[0]; break;
+   case SOFIE_BIAS_FULL: v += ep.beta * ep.C[m * ep.ldc + n]; break;
+   default: break;
+   }
+   return apply_act(v, ep.act, ep.act_alpha);
+}
+
+// The tile loop: acc[4][4] per lane over a 64x64 tile.  LA(m,k), LB(k,n) return 0-safe values only for
+// in-range indices; the loop bounds-checks before calling them.
+template <class LA, class LB>
+__device__ __forceinline__ void f32_tile_loop(const LA &la, const LB &lb, int M, int N, int K, int m0, int n0,
+                                              float (&acc)[4][4])
+{
+   __shared__ float sA[F32_BK][F32_BM + 4];
+   __shared__ float sB[F32_BK][F32_BN + 4];
+   const int t = threadIdx.x;
+   const int tx = t & 15, ty = t >> 4; // 16x16 lanes, each 4x4 outputs
+#pragma unroll
+   for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+         acc[i][j] = 0.0f;
+
+   for (int k0 = 0; k0 < K; k0 += F32_BK) {
+      // 64x16 elements of each operand, 256 threads -> 4 each
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+         int id = t + i * 256;
+         int kk = id & 15, mm = id >> 4; // k fastest for A: consecutive lanes walk k
+         int m = m0 + mm, k = k0 + kk;
+         sA[kk][mm] = (m < M && k < K) ? la(m, k) : 0.0f;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+         int id = t + i * 256;
+         int nn = id & 63, kk = id >> 6; // n fastest for B
+         int n = n0 + nn, k = k0 + kk;
+         sB[kk][nn] = (n < N && k < K) ? lb(k, n) : 0.0f;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < F32_BK; ++kk) {
+         float a[4], b[4];
+#pragma unroll
+         for (int i = 0; i < 4; ++i)
+            a[i] = sA[kk][ty * 4 + i];
+#pragma unroll
+         for (int j = 0; j < 4; ++j)
+            b[j] = sB[kk][tx * 4 + j];
+#pragma unroll
+         for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+               acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+      }
+      __syncthreads();
+   }
+}
+
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmOperandA la, GemmOperandB lb, int M, int N, int K, float *Y,
+                                                        long long ldy, F32Epilogue ep, long long strideA, long long strideB,
+                                                        long long strideC, long long strideY)
+{
+   const int b = blockIdx.z;
+   la.p += b * strideA;
+   lb.p += b * strideB;
+   if (ep.C)
+      ep.C += b * strideC;
+   Y += b * strideY;
+   const int m0 = blockIdx.x * F32_BM, n0 = blockIdx.y * F32_BN;
+   float acc[4][4];
+   f32_tile_loop(la, lb, M, N, K, m0, n0, acc);
+   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+#pragma unroll
+   for (int i = 0; i < 4; ++i) {
+      int m = m0 + ty * 4 + i;
+      if (m >= M)
+         continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+         int n = n0 + tx * 4 + j;
+         if (n < N)
+            Y[m * ldy + n] = f32_epilogue(ep, acc[i][j], m, n);
+      }
+   }
+}
+
+// Column-matrix element (row m = (image, oh, ow), column k = (ci, kh, kw)) gathered from NCHW input;
+// the same index arithmetic as the reference's Im2col, zero outside the image.
+struct ConvOperandA {
+   const float *X;
+   int C, H, W, kh, kw, OH, OW, pad_h0, pad_w0, stride_h, stride_w, dil_h, dil_w;
+   int c_first; // first input channel of this group
+   __device__ __forceinline__ float operator()(int m, int k) const
+   {
+      int ow = m % OW, t = m / OW;
+      int oh = t % OH, img = t / OH;
+      int kx = k % kw, t2 = k / kw;
+      int ky = t2 % kh, ci = t2 / kh;
+      int ih = oh * stride_h - pad_h0 + ky * dil_h;
+      int iw = ow * stride_w - pad_w0 + kx * dil_w;
+      if ((unsigned)ih >= (unsigned)H || (unsigned)iw >= (unsigned)W)
+         return 0.0f;
+      return X[(((size_t)img * C + c_first + ci) * H + ih) * W + iw];
+   }
+};
+struct ConvOperandB {
+   const float *Wt; // [Cout_g][Kg] rows of this group
+   int Kg;
+   __device__ __forceinline__ float operator()(int k, int n) const { return Wt[(size_t)n * Kg + k]; }
+};
+
+__global__ __launch_bounds__(256) void conv_f32_kernel(ConvOperandA la, const float *Wt, const float *bias, float *Y, int M,
+                                                        int Cout_g, int Kg, int Cg, int Cout, int OHW, int act, float act_alpha)
+{
+   const int g = blockIdx.z;
+   la.c_first = g * Cg;
+   ConvOperandB lb{Wt + (size_t)g * Cout_g * Kg, Kg};
+   const int m0 = blockIdx.x * F32_BM, n0 = blockIdx.y * F32_BN;
+   float acc[4][4];
+   f32_tile_loop(la, lb, M, Cout_g, Kg, m0, n0, acc);
+   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+#pragma unroll
+   for (int i = 0; i < 4; ++i) {
+      int m = m0 + ty * 4 + i;
+      if (m >= M)
+         continue;
+      int img = m / OHW, pix = m % OHW;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+         int n = n0 + tx * 4 + j;
+         if (n < Cout_g) {
+            int co = g * Cout_g + n;
+            float v = acc[i][j];
+            if (bias)
+               v += bias[co];
+            Y[((size_t)img * Cout + co) * OHW + pix] = apply_act(v, act, act_alpha);
+         }
+      }
+   }
+}
+
+} // namespace sofie_hip
+
+using namespace sofie_hip;
+
+extern "C" {
+
+int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d)
+{
+   SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_gemm_f32: NULL argument");
+   SOFIE_HIP_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "sofie_hip_gemm_f32: negative dimension");
+   SOFIE_HIP_REQUIRE(d->batch >= 1, "sofie_hip_gemm_f32: batch must be >= 1");
+   SOFIE_HIP_REQUIRE(d->bias_mode >= SOFIE_BIAS_NONE && d->bias_mode <= SOFIE_BIAS_FULL, "sofie_hip_gemm_f32: unknown bias mode %d", d->bias_mode);
+   SOFIE_HIP_REQUIRE(d->act >= SOFIE_ACT_NONE && d->act <= SOFIE_ACT_TANH, "sofie_hip_gemm_f32: unknown activation %d", d->act);
+   if (d->M == 0 || d->N == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(d->Y != nullptr, "sofie_hip_gemm_f32: Y is NULL");
+   SOFIE_HIP_REQUIRE(d->K == 0 || (d->A && d->B), "sofie_hip_gemm_f32: A or B is NULL");
+   SOFIE_HIP_REQUIRE(d->bias_mode == SOFIE_BIAS_NONE || d->C != nullptr, "sofie_hip_gemm_f32: bias mode set but C is NULL");
+   const int M = d->M, N = d->N, K = d->K;
+   const long long lda = d->lda ? d->lda : (d->transA ? M : K);
+   const long long ldb = d->ldb ? d->ldb : (d->transB ? K : N);
+   const long long ldy = d->ldy ? d->ldy : N;
+   SOFIE_HIP_REQUIRE(lda >= (d->transA ? M : K) && ldb >= (d->transB ? K : N) && ldy >= N,
+                     "sofie_hip_gemm_f32: leading dimension too small");
+   GemmOperandA la{d->A, d->transA ? 1 : lda, d->transA ? lda : 1};
+   GemmOperandB lb{d->B, d->transB ? 1 : ldb, d->transB ? ldb : 1};
+   F32Epilogue ep;
+   ep.alpha = d->alpha;
+   ep.beta = d->beta;
+   ep.C = d->bias_mode == SOFIE_BIAS_NONE ? nullptr : d->C;
+   ep.bias_mode = d->bias_mode;
+   ep.ldc = N;
+   ep.act = d->act;
+   ep.act_alpha = d->act_alpha;
+   const unsigned gy = (M + F32_BM - 1) / F32_BM, gx = (N + F32_BN - 1) / F32_BN;
+   SOFIE_HIP_REQUIRE(gx <= 65535 && d->batch <= 65535, "sofie_hip_gemm_f32: N or batch too large for one launch");
+   hipLaunchKernelGGL(gemm_f32_kernel, dim3(gy, gx, (unsigned)d->batch), dim3(256), 0, ctx->stream, la, lb, M, N, K, d->Y, ldy, ep,
+                      (long long)d->strideA, (long long)d->strideB, (long long)d->strideC, (long long)d->strideY);
+   return launch_status("gemm_f32_kernel");
+}
+
+int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float *X, const float *W, const float *bias,
+                       int32_t act, float act_alpha, float *Y)
+{
+   SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_conv_f32: NULL argument");
+   SOFIE_HIP_REQUIRE(d->N >= 0 && d->C > 0 && d->H > 0 && d->W > 0 && d->Cout > 0 && d->kh > 0 && d->kw > 0,
+                     "sofie_hip_conv_f32: bad shape");
+   SOFIE_HIP_REQUIRE(d->group > 0 && d->C % d->group == 0 && d->Cout % d->group == 0,
+                     "sofie_hip_conv_f32: group %d does not divide the channels", d->group);
+   SOFIE_HIP_REQUIRE(d->stride_h > 0 && d->stride_w > 0 && d->dil_h > 0 && d->dil_w > 0, "sofie_hip_conv_f32: bad stride or dilation");
+   SOFIE_HIP_REQUIRE(d->pad_h0 >= 0 && d->pad_w0 >= 0 && d->pad_h1 >= 0 && d->pad_w1 >= 0, "sofie_hip_conv_f32: negative padding");
+   const int eff_kh = d->dil_h * (d->kh - 1) + 1, eff_kw = d->dil_w * (d->kw - 1) + 1;
+   SOFIE_HIP_REQUIRE(d->H + d->pad_h0 + d->pad_h1 >= eff_kh && d->W + d->pad_w0 + d->pad_w1 >= eff_kw,
+                     "sofie_hip_conv_f32: kernel larger than the padded image");
+   const int OH = (d->H + d->pad_h0 + d->pad_h1 - eff_kh) / d->stride_h + 1;
+   const int OW = (d->W + d->pad_w0 + d->pad_w1 - eff_kw) / d->stride_w + 1;
+   SOFIE_HIP_REQUIRE(OH == d->OH && OW == d->OW, "sofie_hip_conv_f32: output shape %dx%d does not match the descriptor's %dx%d", OH, OW,
+                     d->OH, d->OW);
+   SOFIE_HIP_REQUIRE(act >= SOFIE_ACT_NONE && act <= SOFIE_ACT_TANH, "sofie_hip_conv_f32: unknown activation %d", act);
+   if (d->N == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(X && W && Y, "sofie_hip_conv_f32: NULL pointer");
+   const long long M = (long long)d->N * OH * OW;
+   SOFIE_HIP_REQUIRE(M < (1LL << 31), "sofie_hip_conv_f32: too many output pixels");
+   const int Cg = d->C / d->group, Cout_g = d->Cout / d->group, Kg = Cg * d->kh * d->kw;
+   ConvOperandA la{X, d->C, d->H, d->W, d->kh, d->kw, OH, OW, d->pad_h0, d->pad_w0, d->stride_h, d->stride_w, d->dil_h, d->dil_w, 0};
+   const unsigned gy = (unsigned)((M + F32_BM - 1) / F32_BM), gx = (Cout_g + F32_BN - 1) / F32_BN;
+   SOFIE_HIP_REQUIRE(gx <= 65535 && d->group <= 65535, "sofie_hip_conv_f32: too many channels or groups for one launch");
+   hipLaunchKernelGGL(conv_f32_kernel, dim3(gy, gx, (unsigned)d->group), dim3(256), 0, ctx->stream, la, W, bias, Y, (int)M, Cout_g, Kg,
+                      Cg, d->Cout, OH * OW, act, act_alpha);
+   return launch_status("conv_f32_kernel");
+}
+
+} // extern "C"

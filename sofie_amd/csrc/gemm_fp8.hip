@@ -1,0 +1,170 @@
+// FP8 (OCP e4m3fn) GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x64_f8f6f4, fp32 accumulate) with
+// scale + bias + activation + bf16 conversion fused into the store, and the fp32 -> e4m3fn quantiser.
+#include "mfma8_gemm.hpp"
+#include <cstdlib>
+
+namespace sofie_hip {
+
+// fp32 -> bf16 bits, round to nearest even; NaN stays NaN.
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float x)
+{
+   uint32_t u = __float_as_uint(x);
+   if ((u & 0x7fffffffu) > 0x7f800000u)
+      return (uint16_t)((u >> 16) | 0x40);
+   u += 0x7fffu + ((u >> 16) & 1u);
+   return (uint16_t)(u >> 16);
+}
+
+// fp32 -> e4m3fn code, round to nearest even, saturating at +-448 (also +-inf); NaN -> 0x7f.
+__device__ __forceinline__ uint8_t f32_to_e4m3_rne_sat(float x)
+{
+   uint32_t u = __float_as_uint(x);
+   uint8_t sign = (uint8_t)((u >> 24) & 0x80);
+   if ((u & 0x7fffffffu) > 0x7f800000u)
+      return 0x7f;
+   float a = fabsf(x);
+   if (a >= 448.0f)
+      return sign | 0x7e;
+   int e = (int)((u >> 23) & 0xff) - 127; // exponent of the leading bit (denormal fp32 -> far below range)
+   if (e < -6)
+      e = -6;
+   float q = __builtin_rintf(ldexpf(a, 3 - e)); // a / 2^(e-3), exact; ties to even
+   float r = ldexpf(q, e - 3);
+   if (r < 0.015625f) // 2^-6: subnormal codes, quantum 2^-9
+      return sign | (uint8_t)(int)ldexpf(r, 9);
+   uint32_t ur = __float_as_uint(r);
+   int er = (int)((ur >> 23) & 0xff) - 127;
+   return sign | (uint8_t)((er + 7) << 3) | (uint8_t)((ur >> 20) & 7);
+}
+
+__global__ __launch_bounds__(256) void quantize_fp8_kernel(uint8_t *__restrict__ dst, const float *__restrict__ src, size_t n,
+                                                            float scale)
+{
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += stride)
+      dst[i] = f32_to_e4m3_rne_sat(__fdiv_rn(src[i], scale));
+}
+
+struct F8Epilogue {
+   const float *bias;
+   float scale;
+   int act, out;
+   void *Y;
+   int ldy;
+   int vec_store;
+   int N;
+
+   __device__ __forceinline__ float value(float acc, int n) const
+   {
+      float v = mul_nofma(acc, scale);
+      if (bias)
+         v = v + bias[n];
+      return apply_act(v, act, 0.0f);
+   }
+   __device__ __forceinline__ void store4(int m, int n, float a0, float a1, float a2, float a3) const
+   {
+      float a[4] = {a0, a1, a2, a3}, v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+         v[i] = value(a[i], n + i < N ? n + i : N - 1);
+      const size_t row = (size_t)m * (size_t)ldy + n;
+      const bool full = (n + 3 < N) && vec_store;
+      if (out == SOFIE_F8OUT_F32) {
+         float *y = (float *)Y + row;
+         if (full) {
+            *(float4 *)y = make_float4(v[0], v[1], v[2], v[3]);
+         } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+               if (n + i < N)
+                  y[i] = v[i];
+         }
+      } else {
+         uint16_t *y = (uint16_t *)Y + row;
+         uint16_t h[4];
+#pragma unroll
+         for (int i = 0; i < 4; ++i)
+            h[i] = f32_to_bf16_rne(v[i]);
+         if (full) {
+            uint2 p;
+            p.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+            p.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+            *(uint2 *)y = p;
+         } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+               if (n + i < N)
+                  y[i] = h[i];
+         }
+      }
+   }
+};
+
+} // namespace sofie_hip
+
+using namespace sofie_hip;
+
+extern "C" {
+
+int sofie_hip_quantize_fp8(sofie_hip_ctx *ctx, uint8_t *dst, const float *src, size_t n, float scale)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_quantize_fp8: ctx is NULL");
+   if (n == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(dst && src, "sofie_hip_quantize_fp8: NULL pointer");
+   SOFIE_HIP_REQUIRE(scale > 0.0f, "sofie_hip_quantize_fp8: scale must be positive");
+   size_t blocks = (n + 255) / 256;
+   if (blocks > 8192)
+      blocks = 8192;
+   hipLaunchKernelGGL(quantize_fp8_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, dst, src, n, scale);
+   return launch_status("quantize_fp8_kernel");
+}
+
+int sofie_hip_gemm_fp8(sofie_hip_ctx *ctx, const sofie_gemm_fp8_desc *d)
+{
+   SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_gemm_fp8: NULL argument");
+   SOFIE_HIP_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "sofie_hip_gemm_fp8: negative dimension");
+   SOFIE_HIP_REQUIRE(d->out == SOFIE_F8OUT_BF16 || d->out == SOFIE_F8OUT_F32, "sofie_hip_gemm_fp8: unknown output kind %d", d->out);
+   SOFIE_HIP_REQUIRE(d->act >= SOFIE_ACT_NONE && d->act <= SOFIE_ACT_TANH && d->act != SOFIE_ACT_LEAKYRELU,
+                     "sofie_hip_gemm_fp8: unsupported activation %d", d->act);
+   if (d->M == 0 || d->N == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(d->Y != nullptr, "sofie_hip_gemm_fp8: Y is NULL");
+   SOFIE_HIP_REQUIRE(d->K == 0 || (d->A && d->B), "sofie_hip_gemm_fp8: A or B is NULL");
+   const int M = d->M, N = d->N, K = d->K;
+   int lda = d->lda ? d->lda : K;
+   int ldb = d->ldb ? d->ldb : (d->transB ? K : N);
+   int ldy = d->ldy ? d->ldy : N;
+   SOFIE_HIP_REQUIRE(lda >= K && ldb >= (d->transB ? K : N) && ldy >= N, "sofie_hip_gemm_fp8: leading dimension too small");
+   const int8_t *A = (const int8_t *)d->A, *Bt = (const int8_t *)d->B;
+   if (K > 0 && !d->transB) {
+      size_t need = (((size_t)K * (size_t)N) + 255) & ~(size_t)255;
+      SOFIE_HIP_REQUIRE(d->workspace != nullptr && d->workspace_bytes >= need,
+                        "sofie_hip_gemm_fp8: B is [K,N]; a workspace of %zu bytes is needed to re-lay it out", need);
+      SOFIE_HIP_REQUIRE(((uintptr_t)d->workspace & 255) == 0, "sofie_hip_gemm_fp8: workspace must be 256-byte aligned");
+      int st = transpose_i8(ctx->stream, (int8_t *)d->workspace, (const int8_t *)d->B, K, N, ldb, K);
+      if (st)
+         return st;
+      Bt = (const int8_t *)d->workspace;
+      ldb = K;
+   }
+   F8Epilogue ep;
+   ep.bias = d->bias;
+   ep.scale = d->scale;
+   ep.act = d->act;
+   ep.out = d->out;
+   ep.Y = d->Y;
+   ep.ldy = ldy;
+   ep.N = N;
+   const size_t esz = d->out == SOFIE_F8OUT_F32 ? 4 : 2;
+   ep.vec_store = (ldy % 4 == 0) && (((uintptr_t)d->Y & (4 * esz - 1)) == 0);
+   if (K == 0) {
+      A = (const int8_t *)d->Y;
+      Bt = (const int8_t *)d->Y;
+      lda = ldb = 16;
+   }
+   const char *s = getenv("SOFIE_HIP_F8_TILE");
+   return launch_mfma8_auto<MfmaF8, F8Epilogue>(ctx->stream, A, Bt, M, N, K, lda, ldb, ep, s ? atoi(s) : 0);
+}
+
+} // extern "C"

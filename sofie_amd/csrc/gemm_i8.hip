@@ -1,0 +1,154 @@
+// int8 x int8 -> int32 GEMM on the gfx950 matrix cores (v_mfma_i32_32x32x32_i8) with the
+// requantisation / dequantisation epilogue fused into the store, and the int8 re-layout kernel.
+#include "i8_epilogue.hpp"
+#include <cstdlib>
+
+namespace sofie_hip {
+
+// dst[c][r] = src[r][c] for an int8 matrix, through a 64x64 LDS tile.
+__global__ __launch_bounds__(256) void transpose_i8_kernel(int8_t *__restrict__ dst, const int8_t *__restrict__ src,
+                                                            int rows, int cols, int ld_src, int ld_dst)
+{
+   __shared__ int8_t tile[64][64 + 4];
+   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+   for (int i = ty; i < 64; i += 4) {
+      int r = r0 + i, c = c0 + tx;
+      tile[i][tx] = (r < rows && c < cols) ? src[(size_t)r * ld_src + c] : (int8_t)0;
+   }
+   __syncthreads();
+   for (int i = ty; i < 64; i += 4) {
+      int c = c0 + i, r = r0 + tx;
+      if (c < cols && r < rows)
+         dst[(size_t)c * ld_dst + r] = tile[tx][i];
+   }
+}
+
+
+int gemm_i8_nt(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep,
+               int force_tile)
+{
+   const size_t esz = ep.out == SOFIE_I8OUT_I32 || ep.out == SOFIE_I8OUT_F32 ? 4 : 1;
+   ep.vec_store = (ep.nchw_ohw == 0) && (ep.ldy % 4 == 0) && (ep.n_offset % 4 == 0) && (((uintptr_t)ep.Y & (4 * esz - 1)) == 0);
+   ep.N = N;
+   return launch_mfma8_auto<MfmaI8, I8Epilogue>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile);
+}
+
+// SOFIE_HIP_I8_TILE=256|128|64 forces a tile configuration (tuning and tests); unset = heuristic.
+int forced_i8_tile()
+{
+   const char *s = getenv("SOFIE_HIP_I8_TILE");
+   return s ? atoi(s) : 0;
+}
+
+int transpose_i8(hipStream_t stream, int8_t *dst, const int8_t *src, int rows, int cols, int ld_src, int ld_dst)
+{
+   dim3 grid((cols + 63) / 64, (rows + 63) / 64);
+   hipLaunchKernelGGL(transpose_i8_kernel, grid, dim3(256), 0, stream, dst, src, rows, cols, ld_src, ld_dst);
+   return launch_status("transpose_i8_kernel");
+}
+
+} // namespace sofie_hip
+
+using namespace sofie_hip;
+
+
+extern "C" {
+
+size_t sofie_hip_gemm_i8_workspace(const sofie_gemm_i8_desc *d)
+{
+   if (!d)
+      return 0;
+   size_t need = 0;
+   if (!d->transB)
+      need += (((size_t)d->K * (size_t)d->N) + 255) & ~(size_t)255;
+   if (d->transA)
+      need += (((size_t)d->K * (size_t)d->M) + 255) & ~(size_t)255;
+   return need;
+}
+
+int sofie_hip_transpose_i8(sofie_hip_ctx *ctx, int8_t *dst, const int8_t *src, int32_t rows, int32_t cols, int32_t ld_src,
+                           int32_t ld_dst)
+{
+   SOFIE_HIP_REQUIRE(ctx && dst && src, "sofie_hip_transpose_i8: NULL argument");
+   SOFIE_HIP_REQUIRE(rows >= 0 && cols >= 0, "sofie_hip_transpose_i8: negative shape");
+   if (rows == 0 || cols == 0)
+      return SOFIE_HIP_OK;
+   if (ld_src == 0)
+      ld_src = cols;
+   if (ld_dst == 0)
+      ld_dst = rows;
+   SOFIE_HIP_REQUIRE(ld_src >= cols && ld_dst >= rows, "sofie_hip_transpose_i8: leading dimension too small");
+   SOFIE_HIP_REQUIRE((rows + 63) / 64 <= 65535, "sofie_hip_transpose_i8: too many rows");
+   return transpose_i8(ctx->stream, dst, src, rows, cols, ld_src, ld_dst);
+}
+
+int sofie_hip_gemm_i8(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d)
+{
+   SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_gemm_i8: NULL argument");
+   SOFIE_HIP_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "sofie_hip_gemm_i8: negative dimension");
+   SOFIE_HIP_REQUIRE(d->out >= SOFIE_I8OUT_I32 && d->out <= SOFIE_I8OUT_I8_DQQ, "sofie_hip_gemm_i8: unknown output kind %d", d->out);
+   if (d->M == 0 || d->N == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(d->Y != nullptr, "sofie_hip_gemm_i8: Y is NULL");
+   SOFIE_HIP_REQUIRE(d->K == 0 || (d->A && d->B), "sofie_hip_gemm_i8: A or B is NULL");
+   SOFIE_HIP_REQUIRE(d->out != SOFIE_I8OUT_I8_DQQ || d->q_scale != 0.0f, "sofie_hip_gemm_i8: q_scale is 0");
+   const int M = d->M, N = d->N, K = d->K;
+   int lda = d->lda ? d->lda : (d->transA ? M : K);
+   int ldb = d->ldb ? d->ldb : (d->transB ? K : N);
+   int ldy = d->ldy ? d->ldy : N;
+   SOFIE_HIP_REQUIRE(lda >= (d->transA ? M : K) && ldb >= (d->transB ? K : N) && ldy >= N,
+                     "sofie_hip_gemm_i8: leading dimension too small");
+
+   const int8_t *A = d->A, *Bt = d->B;
+   char *ws = (char *)d->workspace;
+   size_t ws_left = d->workspace_bytes;
+   if (K > 0 && !d->transB) {
+      // B is [K,N]: the kernel wants [N,K]
+      size_t need = (((size_t)K * (size_t)N) + 255) & ~(size_t)255;
+      SOFIE_HIP_REQUIRE(ws != nullptr && ws_left >= need,
+                        "sofie_hip_gemm_i8: B is [K,N]; a workspace of %zu bytes is needed to re-lay it out", need);
+      SOFIE_HIP_REQUIRE(((uintptr_t)ws & 255) == 0, "sofie_hip_gemm_i8: workspace must be 256-byte aligned");
+      int st = transpose_i8(ctx->stream, (int8_t *)ws, d->B, K, N, ldb, K);
+      if (st)
+         return st;
+      Bt = (const int8_t *)ws;
+      ldb = K;
+      ws += need;
+      ws_left -= need;
+   }
+   if (K > 0 && d->transA) {
+      size_t need = (((size_t)K * (size_t)M) + 255) & ~(size_t)255;
+      SOFIE_HIP_REQUIRE(ws != nullptr && ws_left >= need,
+                        "sofie_hip_gemm_i8: A is stored [K,M]; a workspace of %zu more bytes is needed", need);
+      int st = transpose_i8(ctx->stream, (int8_t *)ws, d->A, K, M, lda, K);
+      if (st)
+         return st;
+      A = (const int8_t *)ws;
+      lda = K;
+   }
+
+   I8Epilogue ep;
+   ep.bias = d->bias;
+   ep.scale = d->scale;
+   ep.scale_scalar = d->scale_scalar;
+   ep.q_scale = d->q_scale;
+   ep.relu_acc = d->relu_acc;
+   ep.relu_out = d->relu_out;
+   ep.out = d->out;
+   ep.Y = d->Y;
+   ep.ldy = ldy;
+   ep.vec_store = 0;
+   ep.N = N;
+   ep.nchw_ohw = 0;
+   ep.n_offset = 0;
+   if (K == 0) {
+      // empty reduction: acc = 0 everywhere; run the kernel with K = 0 using any valid pointer
+      A = (const int8_t *)d->Y;
+      Bt = (const int8_t *)d->Y;
+      lda = ldb = 16;
+   }
+   return gemm_i8_nt(ctx->stream, A, Bt, M, N, K, lda, ldb, ep, forced_i8_tile());
+}
+
+} // extern "C"

@@ -1,0 +1,168 @@
+"""ctypes view of the C-ABI in include/sofie_hip.h (used by tests/ and bench.py).
+
+There is no fallback: if the library is not built, loading raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def lib_path():
+    return os.path.join(_HERE, "lib", "libsofie_hip.so")
+
+
+class SofieHipError(RuntimeError):
+    pass
+
+
+# activation / bias / output codes of include/sofie_hip.h
+ACT_NONE, ACT_RELU, ACT_LEAKYRELU, ACT_SIGMOID, ACT_GELU, ACT_GELU_TANH, ACT_TANH = range(7)
+BIAS_NONE, BIAS_ROW, BIAS_COL, BIAS_SCALAR, BIAS_FULL = range(5)
+I8OUT_I32, I8OUT_F32, I8OUT_I8, I8OUT_I8_DQQ = range(4)
+F8OUT_BF16, F8OUT_F32 = range(2)
+LAYOUT_NCHW, LAYOUT_NHWC = range(2)
+
+
+class GemmF32Desc(C.Structure):
+    _fields_ = [("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("transA", C.c_int32), ("transB", C.c_int32),
+                ("lda", C.c_int32), ("ldb", C.c_int32), ("ldy", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float),
+                ("A", C.c_void_p), ("B", C.c_void_p), ("C", C.c_void_p), ("bias_mode", C.c_int32), ("act", C.c_int32),
+                ("act_alpha", C.c_float), ("Y", C.c_void_p), ("batch", C.c_int32), ("strideA", C.c_int64),
+                ("strideB", C.c_int64), ("strideC", C.c_int64), ("strideY", C.c_int64)]
+
+
+class GemmI8Desc(C.Structure):
+    _fields_ = [("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("transA", C.c_int32), ("transB", C.c_int32),
+                ("lda", C.c_int32), ("ldb", C.c_int32), ("ldy", C.c_int32), ("A", C.c_void_p), ("B", C.c_void_p),
+                ("bias", C.c_void_p), ("scale", C.c_void_p), ("scale_scalar", C.c_float), ("q_scale", C.c_float),
+                ("relu_acc", C.c_int32), ("relu_out", C.c_int32), ("out", C.c_int32), ("Y", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
+class GemmFp8Desc(C.Structure):
+    _fields_ = [("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("transB", C.c_int32), ("lda", C.c_int32),
+                ("ldb", C.c_int32), ("ldy", C.c_int32), ("A", C.c_void_p), ("B", C.c_void_p), ("bias", C.c_void_p),
+                ("scale", C.c_float), ("act", C.c_int32), ("out", C.c_int32), ("Y", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
+class AddDesc(C.Structure):
+    _fields_ = [("rank", C.c_int32), ("y_shape", C.c_int64 * 6), ("a_shape", C.c_int64 * 6), ("b_shape", C.c_int64 * 6),
+                ("A", C.c_void_p), ("B", C.c_void_p), ("Y", C.c_void_p)]
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [("N", C.c_int32), ("C", C.c_int32), ("H", C.c_int32), ("W", C.c_int32), ("Cout", C.c_int32),
+                ("kh", C.c_int32), ("kw", C.c_int32), ("pad_h0", C.c_int32), ("pad_w0", C.c_int32),
+                ("pad_h1", C.c_int32), ("pad_w1", C.c_int32), ("stride_h", C.c_int32), ("stride_w", C.c_int32),
+                ("dil_h", C.c_int32), ("dil_w", C.c_int32), ("group", C.c_int32), ("OH", C.c_int32), ("OW", C.c_int32)]
+
+
+class ConvI8Args(C.Structure):
+    _fields_ = [("X", C.c_void_p), ("W", C.c_void_p), ("bias", C.c_void_p), ("scale", C.c_void_p),
+                ("relu", C.c_int32), ("out", C.c_int32), ("x_layout", C.c_int32), ("y_layout", C.c_int32),
+                ("w_is_packed", C.c_int32), ("Y", C.c_void_p), ("workspace", C.c_void_p),
+                ("workspace_bytes", C.c_size_t)]
+
+
+# every symbol include/sofie_hip.h declares: name -> (restype, argtypes)
+_P = C.c_void_p
+SYMBOLS = {
+    "sofie_hip_ctx_create": (C.c_int, [C.POINTER(_P), C.c_int, _P]),
+    "sofie_hip_ctx_destroy": (C.c_int, [_P]),
+    "sofie_hip_last_error": (C.c_char_p, []),
+    "sofie_hip_abi_version": (C.c_int, []),
+    "sofie_hip_arena_create": (C.c_int, [_P, C.c_size_t, C.c_size_t]),
+    "sofie_hip_arena_adopt": (C.c_int, [_P, _P, C.c_size_t]),
+    "sofie_hip_arena_ptr": (_P, [_P, C.c_size_t]),
+    "sofie_hip_arena_bytes": (C.c_size_t, [_P]),
+    "sofie_hip_stream": (_P, [_P]),
+    "sofie_hip_upload": (C.c_int, [_P, _P, _P, C.c_size_t]),
+    "sofie_hip_download": (C.c_int, [_P, _P, _P, C.c_size_t]),
+    "sofie_hip_copy": (C.c_int, [_P, _P, _P, C.c_size_t]),
+    "sofie_hip_fill_zero": (C.c_int, [_P, _P, C.c_size_t]),
+    "sofie_hip_sync": (C.c_int, [_P]),
+    "sofie_hip_gemm_f32": (C.c_int, [_P, C.POINTER(GemmF32Desc)]),
+    "sofie_hip_gemm_i8": (C.c_int, [_P, C.POINTER(GemmI8Desc)]),
+    "sofie_hip_gemm_i8_workspace": (C.c_size_t, [C.POINTER(GemmI8Desc)]),
+    "sofie_hip_transpose_i8": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
+    "sofie_hip_gemm_fp8": (C.c_int, [_P, C.POINTER(GemmFp8Desc)]),
+    "sofie_hip_quantize_fp8": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_float]),
+    "sofie_hip_quantize_linear": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_float]),
+    "sofie_hip_dequantize_linear_i8": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_float]),
+    "sofie_hip_dequantize_linear_i32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_float]),
+    "sofie_hip_unary_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_int32, C.c_float]),
+    "sofie_hip_add_f32": (C.c_int, [_P, C.POINTER(AddDesc)]),
+    "sofie_hip_conv_f32": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P, _P, C.c_int32, C.c_float, _P]),
+    "sofie_hip_conv_i8": (C.c_int, [_P, C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
+    "sofie_hip_conv_i8_workspace": (C.c_size_t, [C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
+    "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),
+    "sofie_hip_global_avg_pool_f32": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32]),
+    "sofie_hip_global_avg_pool_i8": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float]),
+    "sofie_hip_conv_weight_i8_packed_bytes": (C.c_size_t, [C.POINTER(ConvDesc)]),
+    "sofie_hip_timer_start": (C.c_int, [_P]),
+    "sofie_hip_timer_stop": (C.c_int, [_P, C.POINTER(C.c_float)]),
+}
+
+_lib = None
+
+
+def load_library(path=None):
+    """dlopen the runtime library and type every entry point; raises if it is missing."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or lib_path()
+    if not os.path.exists(p):
+        raise SofieHipError("%s is not built: run `python -c 'import __graft_entry__ as g; g.build()'`" % p)
+    lib = C.CDLL(p)
+    for name, (res, args) in SYMBOLS.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    if path is None:
+        _lib = lib
+    return lib
+
+
+class Runtime:
+    """One context (stream + optional arena) on one device; methods raise SofieHipError on failure."""
+
+    def __init__(self, device=0, external_stream=None):
+        self.lib = load_library()
+        h = C.c_void_p()
+        self._check(self.lib.sofie_hip_ctx_create(C.byref(h), device, external_stream))
+        self.ctx = h
+
+    def close(self):
+        if getattr(self, "ctx", None):
+            self.lib.sofie_hip_ctx_destroy(self.ctx)
+            self.ctx = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _check(self, status):
+        if status != 0:
+            raise SofieHipError("sofie_hip status %d: %s" % (status, (self.lib.sofie_hip_last_error() or b"").decode()))
+
+    def call(self, name, *args):
+        self._check(getattr(self.lib, name)(self.ctx, *args))
+
+    def sync(self):
+        self.call("sofie_hip_sync")
+
+    def stream(self):
+        return self.lib.sofie_hip_stream(self.ctx)
+
+    def timer_start(self):
+        self.call("sofie_hip_timer_start")
+
+    def timer_stop(self):
+        ms = C.c_float()
+        self.call("sofie_hip_timer_stop", C.byref(ms))
+        return ms.value

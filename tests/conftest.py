@@ -1,0 +1,23 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def rt():
+    """One runtime context on cuda:0 for the GPU tests; fails loudly if the HIP library is missing."""
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from sofie_amd import Runtime
+    r = Runtime(0)
+    yield r
+    r.close()

@@ -1,0 +1,97 @@
+"""int8 convolution (GEMM over the whole batch) through the C-ABI: bit-exact against the direct 7-loop oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from sofie_amd import runtime as R
+from tests import util
+from tests.test_gpu_f32 import conv_desc
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # N, C, H, W, Cout, kh, kw, pads, strides, dils, group
+    (1, 1, 5, 5, 1, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),
+    (2, 3, 9, 7, 5, 3, 3, (0, 0, 0, 0), (1, 1), (1, 1), 1),
+    (2, 4, 8, 8, 6, 3, 2, (1, 0, 2, 1), (2, 1), (1, 1), 2),
+    (1, 2, 10, 10, 4, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2), 1),
+    (3, 32, 6, 6, 8, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1), 2),
+    (4, 3, 16, 16, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),
+    (2, 64, 12, 12, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),
+    (2, 16, 9, 9, 32, 3, 3, (1, 1, 1, 1), (2, 2), (1, 1), 1),
+]
+
+
+def run_conv(rt, X, Wt, bias, scale, case, relu, out, x_layout, y_layout, packed, ws_images=None):
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    d = conv_desc(N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group)
+    Xd = X if x_layout == R.LAYOUT_NCHW else np.ascontiguousarray(X.transpose(0, 2, 3, 1))
+    dX, dW = util.to_dev(Xd), util.to_dev(Wt)
+    db = None if bias is None else util.to_dev(bias)
+    ds = None if scale is None else util.to_dev(scale)
+    odt = {0: np.int32, 1: np.float32, 2: np.int8}[out]
+    yshape = (N, Cout, d.OH, d.OW) if y_layout == R.LAYOUT_NCHW else (N, d.OH, d.OW, Cout)
+    dY = util.dev_empty(yshape, odt)
+    a = R.ConvI8Args()
+    a.X, a.W, a.bias, a.scale, a.Y = util.ptr(dX), util.ptr(dW), util.ptr(db), util.ptr(ds), util.ptr(dY)
+    a.relu, a.out, a.x_layout, a.y_layout = relu, out, x_layout, y_layout
+    keep = []
+    if packed:
+        nb = rt.lib.sofie_hip_conv_weight_i8_packed_bytes(C.byref(d))
+        dWp = util.dev_empty((nb,), np.int8)
+        rt.call("sofie_hip_pack_conv_weight_i8", C.byref(d), util.ptr(dWp), util.ptr(dW))
+        a.W, a.w_is_packed = util.ptr(dWp), 1
+        keep.append(dWp)
+    need = rt.lib.sofie_hip_conv_i8_workspace(C.byref(d), C.byref(a))
+    if ws_images:
+        need = need * ws_images
+    ws = util.dev_empty((need + 256,), np.int8)
+    a.workspace, a.workspace_bytes = util.ptr(ws), need
+    import torch
+    torch.cuda.synchronize()
+    print("conv_i8", case, relu, out, x_layout, y_layout, packed, flush=True)
+    rt.call("sofie_hip_conv_i8", C.byref(d), C.byref(a))
+    rt.sync()
+    y = util.to_host(dY)
+    return y if y_layout == R.LAYOUT_NCHW else np.ascontiguousarray(y.transpose(0, 3, 1, 2))
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("x_layout,y_layout,packed", [(0, 0, 0), (1, 1, 1), (0, 1, 0), (1, 0, 1)])
+def test_conv_i8_requant_bit_exact(rt, case, x_layout, y_layout, packed):
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    X = util.int8_sym(50, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.int8_sym(51, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
+    bias = util.int32_range(52, Cout, -2000, 2000)
+    K = (Cc // group) * kh * kw
+    scale = ((0.5 + util.uniform01(53, Cout)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    got = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, x_layout, y_layout, packed, ws_images=2)
+    want = ob.conv_i8(X, Wt, bias, scale, pads=pads, strides=strides, dils=dils, group=group, relu=1, out=2, omp=True)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("out,relu", [(R.I8OUT_I32, 0), (R.I8OUT_I32, 1), (R.I8OUT_F32, 0), (R.I8OUT_F32, 1), (R.I8OUT_I8, 0)])
+def test_conv_i8_output_kinds(rt, out, relu):
+    case = (3, 8, 7, 9, 12, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1)
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    X = util.int8_sym(60, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.int8_sym(61, Cout * Cc * kh * kw).reshape(Cout, Cc, kh, kw)
+    scale = ((0.5 + util.uniform01(63, Cout)) / np.float32(127.0 * 8.5)).astype(np.float32)
+    got = run_conv(rt, X, Wt, None, scale, case, relu, out, 0, 0, 0)
+    want = ob.conv_i8(X, Wt, None, scale, pads=pads, strides=strides, dils=dils, group=group, relu=relu, out=out)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
+def test_global_avg_pool_i8_both_layouts(rt):
+    N, Cc, H, W = 3, 20, 5, 7
+    X = util.int8_sym(70, N * Cc * H * W).reshape(N, Cc, H, W)
+    want = ob.global_avg_pool_i8(X, np.float32(0.031))
+    for layout in (0, 1):
+        Xd = X if layout == 0 else np.ascontiguousarray(X.transpose(0, 2, 3, 1))
+        dX = util.to_dev(Xd)
+        dY = util.dev_empty((N, Cc), np.float32)
+        rt.call("sofie_hip_global_avg_pool_i8", util.ptr(dY), util.ptr(dX), N, Cc, H * W, layout, C.c_float(0.031))
+        rt.sync()
+        assert np.array_equal(util.to_host(dY).view(np.uint32), want.view(np.uint32))

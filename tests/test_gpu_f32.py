@@ -1,0 +1,175 @@
+"""fp32 Gemm / Conv / elementwise operators through the C-ABI against the CPU restatement of SOFIE's
+generated code.  Tolerance: |got - want| <= 1e-5 * (|want| + sum_k |a_k b_k|) -- 1e-5 relative to the
+magnitude the dot product is formed from (the summation order of a GEMM is not part of its definition)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from sofie_amd import runtime as R
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+def gemm(rt, A, B, Cb, M, N, K, transA=0, transB=0, alpha=1.0, beta=1.0, bias_mode=0, act=0, act_alpha=0.0, batch=1,
+         strides=(0, 0, 0, 0)):
+    dA, dB = util.to_dev(A), util.to_dev(B)
+    dC = None if Cb is None else util.to_dev(Cb)
+    dY = util.dev_empty((batch, M, N), np.float32)
+    d = R.GemmF32Desc()
+    d.M, d.N, d.K, d.transA, d.transB = M, N, K, transA, transB
+    d.alpha, d.beta = alpha, beta
+    d.A, d.B, d.C, d.Y = util.ptr(dA), util.ptr(dB), util.ptr(dC), util.ptr(dY)
+    d.bias_mode, d.act, d.act_alpha = bias_mode, act, act_alpha
+    d.batch = batch
+    d.strideA, d.strideB, d.strideC, d.strideY = strides
+    import torch
+    torch.cuda.synchronize()
+    print("gemm_f32 M=%d N=%d K=%d tA=%d tB=%d bias=%d act=%d batch=%d" % (M, N, K, transA, transB, bias_mode, act, batch), flush=True)
+    rt.call("sofie_hip_gemm_f32", C.byref(d))
+    rt.sync()
+    y = util.to_host(dY)
+    return y[0] if batch == 1 else y
+
+
+def close(got, want, mag, rel=1e-5):
+    return np.all(np.abs(got.astype(np.float64) - want) <= rel * (np.abs(want) + mag) + 1e-30)
+
+
+@pytest.mark.parametrize("M,N,K,transA,transB", [(64, 128, 784, 0, 1), (64, 64, 128, 0, 1), (64, 10, 64, 0, 1), (16, 50, 100, 0, 0),
+                                                 (7, 5, 3, 1, 0), (65, 67, 33, 1, 1), (1, 1, 1, 0, 0), (130, 70, 257, 0, 0)])
+@pytest.mark.parametrize("bias_mode,act", [(0, 0), (1, 1), (2, 0), (3, 2), (4, 3), (1, 4)])
+def test_gemm_f32_matches_sofie_cpu_semantics(rt, M, N, K, transA, transB, bias_mode, act):
+    A = util.normal(1, M * K).reshape((K, M) if transA else (M, K))
+    B = util.normal(2, N * K, 0.05).reshape((N, K) if transB else (K, N))
+    Cshape = {0: None, 1: (N,), 2: (M, 1), 3: (1,), 4: (M, N)}[bias_mode]
+    Cb = None if Cshape is None else util.normal(3, int(np.prod(Cshape))).reshape(Cshape)
+    alpha, beta = 1.25, 0.5
+    got = gemm(rt, A, B, Cb, M, N, K, transA, transB, alpha, beta, bias_mode, act, 0.1)
+    want = ob.gemm_f32(A, B, Cb, M=M, N=N, K=K, transA=transA, transB=transB, alpha=alpha, beta=beta, bias_mode=bias_mode,
+                       act=act, act_alpha=0.1)
+    opA = A.T if transA else A
+    opB = B.T if transB else B
+    mag = np.abs(alpha) * (np.abs(opA).astype(np.float64) @ np.abs(opB).astype(np.float64)) + 1.0
+    assert close(got, want.astype(np.float64), mag)
+    # float64 textbook arbiter for the linear part
+    if act == 0:
+        ref = alpha * (opA.astype(np.float64) @ opB.astype(np.float64))
+        if bias_mode in (1, 2, 3):
+            ref = ref + Cb.astype(np.float64)
+        elif bias_mode == 4:
+            ref = ref + beta * Cb.astype(np.float64)
+        assert close(got, ref, mag)
+
+
+def test_relu_edge_cases_follow_the_cpu_helper(rt):
+    # Relu(NaN) = 0 and Relu(-0) = +0 on SOFIE's CPU path
+    x = np.array([np.nan, -0.0, 0.0, -1.0, 2.5, np.inf, -np.inf], dtype=np.float32)
+    dx = util.to_dev(x)
+    dy = util.dev_empty(x.shape, np.float32)
+    rt.call("sofie_hip_unary_f32", util.ptr(dy), util.ptr(dx), C.c_size_t(x.size), R.ACT_RELU, C.c_float(0))
+    rt.sync()
+    got = util.to_host(dy)
+    want = ob.unary(x, R.ACT_RELU)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_stacked_matmul(rt):
+    b, M, N, K = 5, 12, 9, 20
+    A = util.normal(5, b * M * K).reshape(b, M, K)
+    B = util.normal(6, b * K * N).reshape(b, K, N)
+    got = gemm(rt, A, B, None, M, N, K, batch=b, strides=(M * K, K * N, 0, M * N))
+    want = np.einsum("bmk,bkn->bmn", A.astype(np.float64), B.astype(np.float64))
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+    # shared B (stride 0)
+    got = gemm(rt, A, B[0], None, M, N, K, batch=b, strides=(M * K, 0, 0, M * N))
+    want = np.einsum("bmk,kn->bmn", A.astype(np.float64), B[0].astype(np.float64))
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("act", [R.ACT_RELU, R.ACT_LEAKYRELU, R.ACT_SIGMOID, R.ACT_GELU, R.ACT_GELU_TANH, R.ACT_TANH])
+@pytest.mark.parametrize("n", [1, 7, 4096 + 3])
+def test_unary(rt, act, n):
+    x = util.normal(10 + act, n, 2.0)
+    dx = util.to_dev(x)
+    dy = util.dev_empty((n,), np.float32)
+    rt.call("sofie_hip_unary_f32", util.ptr(dy), util.ptr(dx), C.c_size_t(n), act, C.c_float(0.2))
+    rt.sync()
+    want = ob.unary(x, act, 0.2)
+    assert np.allclose(util.to_host(dy), want, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("ash,bsh", [((4, 5), (4, 5)), ((4, 5), (5,)), ((4, 1), (1, 5)), ((2, 3, 4, 5), (3, 1, 5)), ((1,), (6, 7))])
+def test_add_broadcast(rt, ash, bsh):
+    A = util.normal(20, int(np.prod(ash))).reshape(ash)
+    B = util.normal(21, int(np.prod(bsh))).reshape(bsh)
+    ysh = np.broadcast_shapes(ash, bsh)
+    rank = len(ysh)
+    d = R.AddDesc()
+    d.rank = rank
+    for i, v in enumerate(ysh):
+        d.y_shape[i] = v
+    for i, v in enumerate((1,) * (rank - len(ash)) + tuple(ash)):
+        d.a_shape[i] = v
+    for i, v in enumerate((1,) * (rank - len(bsh)) + tuple(bsh)):
+        d.b_shape[i] = v
+    dA, dB = util.to_dev(A), util.to_dev(B)
+    dY = util.dev_empty(ysh, np.float32)
+    d.A, d.B, d.Y = util.ptr(dA), util.ptr(dB), util.ptr(dY)
+    rt.call("sofie_hip_add_f32", C.byref(d))
+    rt.sync()
+    got = util.to_host(dY)
+    assert np.array_equal(got, A + B)
+    assert np.array_equal(got, ob.add_broadcast(A, B))
+
+
+def conv_desc(N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group):
+    OH, OW = ob.conv_out_hw(H, W, kh, kw, pads, strides, dils)
+    d = R.ConvDesc()
+    (d.N, d.C, d.H, d.W, d.Cout, d.kh, d.kw) = (N, Cc, H, W, Cout, kh, kw)
+    (d.pad_h0, d.pad_w0, d.pad_h1, d.pad_w1) = pads
+    (d.stride_h, d.stride_w), (d.dil_h, d.dil_w) = strides, dils
+    d.group, d.OH, d.OW = group, OH, OW
+    return d
+
+
+CONV_CASES = [
+    # N, C, H, W, Cout, kh, kw, pads, strides, dils, group
+    (1, 1, 5, 5, 1, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),
+    (2, 3, 9, 7, 5, 3, 3, (0, 0, 0, 0), (1, 1), (1, 1), 1),
+    (2, 4, 8, 8, 6, 3, 2, (1, 0, 2, 1), (2, 1), (1, 1), 2),
+    (1, 2, 10, 10, 4, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2), 1),
+    (3, 8, 6, 6, 8, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1), 4),
+    (2, 3, 1, 20, 4, 1, 5, (0, 2, 0, 2), (1, 2), (1, 1), 1),
+    (4, 3, 16, 16, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("with_bias,act", [(False, 0), (True, 1)])
+def test_conv_f32(rt, case, with_bias, act):
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    X = util.uniform01(30, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.normal(31, Cout * (Cc // group) * kh * kw, 0.3).reshape(Cout, Cc // group, kh, kw)
+    b = util.normal(32, Cout) if with_bias else None
+    d = conv_desc(N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group)
+    dX, dW = util.to_dev(X), util.to_dev(Wt)
+    db = None if b is None else util.to_dev(b)
+    dY = util.dev_empty((N, Cout, d.OH, d.OW), np.float32)
+    print("conv_f32", case, flush=True)
+    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(dX), util.ptr(dW), util.ptr(db), act, C.c_float(0), util.ptr(dY))
+    rt.sync()
+    want = ob.conv_f32(X, Wt, b, pads=pads, strides=strides, dils=dils, group=group, act=act)
+    assert np.allclose(util.to_host(dY), want, rtol=1e-5, atol=1e-5)
+
+
+def test_global_avg_pool(rt):
+    X = util.normal(40, 3 * 7 * 33).reshape(3, 7, 33)
+    dX = util.to_dev(X)
+    dY = util.dev_empty((21,), np.float32)
+    rt.call("sofie_hip_global_avg_pool_f32", util.ptr(dY), util.ptr(dX), 21, 33)
+    rt.sync()
+    want = ob.global_avg_pool(X.reshape(3, 7, 33, 1)).reshape(21)
+    assert np.allclose(util.to_host(dY), want, rtol=1e-6, atol=1e-6)

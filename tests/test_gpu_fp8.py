@@ -1,0 +1,110 @@
+"""FP8 (e4m3fn) GEMM and quantiser through the C-ABI.
+
+Bound on the GEMM (fp32 accumulation in hardware order, products exact):
+   |acc - exact| <= K * 2^-24 * sum_k |a_k b_k|
+and then scale, bias, activation in fp32 and one bf16 rounding (relative 2^-9) for bf16 output."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from sofie_amd import runtime as R
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+def quantize_dev(rt, x, scale):
+    dx = util.to_dev(x)
+    dq = util.dev_empty(x.shape, np.uint8)
+    rt.call("sofie_hip_quantize_fp8", util.ptr(dq), util.ptr(dx), C.c_size_t(x.size), C.c_float(scale))
+    rt.sync()
+    return util.to_host(dq)
+
+
+def test_quantiser_bit_exact_incl_all_codes_ties_and_saturation(rt):
+    codes = np.arange(256, dtype=np.uint8)
+    vals = ob.e4m3_to_f32(codes)
+    finite = np.isfinite(vals)
+    # every representable value maps to its own code; midpoints between neighbours tie to even
+    pos = np.sort(vals[finite & (vals >= 0)])
+    mids = ((pos[:-1].astype(np.float64) + pos[1:].astype(np.float64)) / 2).astype(np.float32)
+    x = np.concatenate([vals[finite], mids, -mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9)),
+                        np.array([448, 449, 463.9, 464, 465, 1e9, np.inf, -np.inf, np.nan, 1e-10, -1e-10, 2 ** -10, 2 ** -9], dtype=np.float32),
+                        util.normal(77, 20000, 100.0)]).astype(np.float32)
+    got = quantize_dev(rt, x, 1.0)
+    want = ob.quantize_fp8(x, 1.0)
+    assert np.array_equal(got, want)
+    n = finite.sum()
+    assert np.array_equal(got[:n], codes[finite])
+    got = quantize_dev(rt, x, 0.37)
+    assert np.array_equal(got, ob.quantize_fp8(x, 0.37))
+
+
+def run_fp8(rt, A, B, M, N, K, transB=1, bias=None, scale=1.0, act=0, out=1):
+    dA, dB = util.to_dev(A), util.to_dev(B)
+    db = None if bias is None else util.to_dev(bias)
+    dY = util.dev_empty((M, N), np.float32 if out == 1 else np.uint16)
+    d = R.GemmFp8Desc()
+    d.M, d.N, d.K, d.transB = M, N, K, transB
+    d.A, d.B, d.bias, d.Y = util.ptr(dA), util.ptr(dB), util.ptr(db), util.ptr(dY)
+    d.scale, d.act, d.out = scale, act, out
+    ws = util.dev_empty((K * N + 256,), np.uint8)
+    d.workspace, d.workspace_bytes = util.ptr(ws), K * N + 256
+    import torch
+    torch.cuda.synchronize()
+    print("gemm_fp8 M=%d N=%d K=%d tB=%d act=%d out=%d" % (M, N, K, transB, act, out), flush=True)
+    rt.call("sofie_hip_gemm_fp8", C.byref(d))
+    rt.sync()
+    y = util.to_host(dY)
+    return y if out == 1 else y.view(np.uint16)
+
+
+def make_fp8(seed, rows, K):
+    x = util.normal(seed, rows * K).reshape(rows, K)
+    s = np.float32(np.abs(x).max() / 448.0)
+    return ob.quantize_fp8(x, s), s
+
+
+@pytest.mark.parametrize("M,N,K", [(32, 32, 64), (64, 64, 64), (33, 65, 47), (100, 200, 300), (256, 256, 256), (257, 129, 1040),
+                                   (1024, 1024, 1024)])
+@pytest.mark.parametrize("transB", [1, 0])
+def test_fp32_output_within_accumulation_bound(rt, M, N, K, transB):
+    A, sa = make_fp8(4001, M, K)
+    Bt, sb = make_fp8(4002, N, K)
+    B = Bt if transB else np.ascontiguousarray(Bt.T)
+    scale = np.float32(sa * sb)
+    got = run_fp8(rt, A, B, M, N, K, transB=transB, scale=scale, out=1)
+    want, abs_sum = ob.gemm_fp8(A, B, M=M, N=N, K=K, transB=transB, scale=scale, out=1, want_abs_sum=True, omp=True)
+    bound = (K * 2.0 ** -24) * abs_sum.astype(np.float64) * float(scale) + 2.0 ** -23 * np.abs(want) + 1e-30
+    assert np.all(np.abs(got.astype(np.float64) - want) <= bound)
+
+
+def test_exact_cases(rt):
+    # one-hot rows pick single products: no accumulation error at all
+    K, M, N = 128, 64, 64
+    Bt, sb = make_fp8(4002, N, K)
+    A = np.zeros((M, K), dtype=np.uint8)
+    one = ob.quantize_fp8(np.array([1.0], np.float32), 1.0)[0]
+    for m in range(M):
+        A[m, (m * 7) % K] = one
+    got = run_fp8(rt, A, Bt, M, N, K, scale=1.0, out=1)
+    want = ob.e4m3_to_f32(Bt)[:, [(m * 7) % K for m in range(M)]].T
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("act", [R.ACT_NONE, R.ACT_RELU, R.ACT_GELU])
+def test_bf16_output_with_bias_and_activation(rt, act):
+    M, N, K = 200, 136, 512
+    A, sa = make_fp8(4001, M, K)
+    Bt, sb = make_fp8(4002, N, K)
+    bias = util.normal(4003, N)
+    scale = np.float32(sa * sb)
+    got = ob.bf16_bits_to_f32(run_fp8(rt, A, Bt, M, N, K, bias=bias, scale=scale, act=act, out=0))
+    want, abs_sum = ob.gemm_fp8(A, Bt, M=M, N=N, K=K, transB=1, bias=bias, scale=scale, act=act, out=1, want_abs_sum=True)
+    # accumulation bound propagated through bias (exact add up to 1 ulp) and an activation with slope <= 1.13,
+    # plus half an ulp of bf16 (2^-9 relative) for the final rounding
+    acc_err = (K * 2.0 ** -24) * abs_sum.astype(np.float64) * float(scale)
+    bound = 1.2 * acc_err + 2.0 ** -8 * np.abs(want) + 1e-6
+    assert np.all(np.abs(got.astype(np.float64) - want) <= bound)
