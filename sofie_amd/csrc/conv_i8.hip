@@ -222,6 +222,9 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
          ep.relu_out = (a->out == SOFIE_I8OUT_I32) ? 0 : a->relu;
          ep.out = a->out;
          ep.ldy = d->Cout;
+         ep.stage_ok = 0;
+         ep.vec_param = 0;
+         ep.N = Cout_g;
          ep.n_offset = grp * Cout_g;
          if (a->y_layout == SOFIE_LAYOUT_NHWC) {
             ep.nchw_ohw = 0;

@@ -1,6 +1,6 @@
 // FP8 (OCP e4m3fn) GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x64_f8f6f4, fp32 accumulate) with
 // scale + bias + activation + bf16 conversion fused into the store, and the fp32 -> e4m3fn quantiser.
-#include "mfma8_gemm.hpp"
+#include "mfma8_gemm_dma.hpp"
 #include <cstdlib>
 
 namespace sofie_hip {
@@ -51,51 +51,56 @@ struct F8Epilogue {
    int act, out;
    void *Y;
    int ldy;
-   int vec_store;
+   int stage_ok;
    int N;
 
-   __device__ __forceinline__ float value(float acc, int n) const
+   template <class F>
+   __device__ __forceinline__ void dispatch(F f) const
    {
-      float v = mul_nofma(acc, scale);
-      if (bias)
-         v = v + bias[n];
-      return apply_act(v, act, 0.0f);
+      if (out == SOFIE_F8OUT_F32)
+         f(std::integral_constant<int, SOFIE_F8OUT_F32>{});
+      else
+         f(std::integral_constant<int, SOFIE_F8OUT_BF16>{});
    }
-   __device__ __forceinline__ void store4(int m, int n, float a0, float a1, float a2, float a3) const
+   template <int OUT>
+   static constexpr int out_bytes()
    {
-      float a[4] = {a0, a1, a2, a3}, v[4];
+      return OUT == SOFIE_F8OUT_F32 ? 4 : 2;
+   }
+   __device__ __forceinline__ bool rows_vectorizable() const { return stage_ok != 0; }
+   __device__ __forceinline__ char *out_base() const { return (char *)Y; }
+   __device__ __forceinline__ size_t out_index(int m, int n) const { return (size_t)m * (size_t)ldy + n; }
+   template <int C>
+   struct col_params {
+      float b[C];
+   };
+   template <int C>
+   __device__ __forceinline__ void load_params(int n, col_params<C> &p) const
+   {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-         v[i] = value(a[i], n + i < N ? n + i : N - 1);
-      const size_t row = (size_t)m * (size_t)ldy + n;
-      const bool full = (n + 3 < N) && vec_store;
-      if (out == SOFIE_F8OUT_F32) {
-         float *y = (float *)Y + row;
-         if (full) {
-            *(float4 *)y = make_float4(v[0], v[1], v[2], v[3]);
-         } else {
+      for (int i = 0; i < C; ++i)
+         p.b[i] = bias ? bias[n + i < N ? n + i : N - 1] : 0.0f;
+   }
+   // v = acc*scale + bias[n]; activation in fp32; then fp32 or bf16 (round to nearest even)
+   template <int OUT, int C>
+   __device__ __forceinline__ void pack4(const col_params<C> &p, int q, float a0, float a1, float a2, float a3, uint32_t *w) const
+   {
+      const float a[4] = {a0, a1, a2, a3};
+      float v[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-               if (n + i < N)
-                  y[i] = v[i];
-         }
-      } else {
-         uint16_t *y = (uint16_t *)Y + row;
-         uint16_t h[4];
+      for (int i = 0; i < 4; ++i) {
+         v[i] = mul_nofma(a[i], scale);
+         if (bias)
+            v[i] = v[i] + p.b[4 * q + i];
+         v[i] = apply_act(v[i], act, 0.0f);
+      }
+      if (OUT == SOFIE_F8OUT_F32) {
 #pragma unroll
          for (int i = 0; i < 4; ++i)
-            h[i] = f32_to_bf16_rne(v[i]);
-         if (full) {
-            uint2 p;
-            p.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
-            p.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
-            *(uint2 *)y = p;
-         } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-               if (n + i < N)
-                  y[i] = h[i];
-         }
+            w[i] = __float_as_uint(v[i]);
+      } else {
+         w[0] = (uint32_t)f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
+         w[1] = (uint32_t)f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
       }
    }
 };
@@ -157,14 +162,15 @@ int sofie_hip_gemm_fp8(sofie_hip_ctx *ctx, const sofie_gemm_fp8_desc *d)
    ep.ldy = ldy;
    ep.N = N;
    const size_t esz = d->out == SOFIE_F8OUT_F32 ? 4 : 2;
-   ep.vec_store = (ldy % 4 == 0) && (((uintptr_t)d->Y & (4 * esz - 1)) == 0);
+   ep.stage_ok = (((size_t)ldy * esz) % 16 == 0) && (((uintptr_t)d->Y & 15) == 0);
    if (K == 0) {
       A = (const int8_t *)d->Y;
       Bt = (const int8_t *)d->Y;
       lda = ldb = 16;
    }
    const char *s = getenv("SOFIE_HIP_F8_TILE");
-   return launch_mfma8_auto<MfmaF8, F8Epilogue>(ctx->stream, A, Bt, M, N, K, lda, ldb, ep, s ? atoi(s) : 0);
+   const char *v = getenv("SOFIE_HIP_GEMM_VARIANT");
+   return launch_mfma8_best<MfmaF8, F8Epilogue>(ctx->stream, A, Bt, M, N, K, lda, ldb, ep, s ? atoi(s) : 0, v ? atoi(v) : 0);
 }
 
 } // extern "C"

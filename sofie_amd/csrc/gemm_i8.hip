@@ -29,9 +29,14 @@ int gemm_i8_nt(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int
                int force_tile)
 {
    const size_t esz = ep.out == SOFIE_I8OUT_I32 || ep.out == SOFIE_I8OUT_F32 ? 4 : 1;
-   ep.vec_store = (ep.nchw_ohw == 0) && (ep.ldy % 4 == 0) && (ep.n_offset % 4 == 0) && (((uintptr_t)ep.Y & (4 * esz - 1)) == 0);
    ep.N = N;
-   return launch_mfma8_auto<MfmaI8, I8Epilogue>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile);
+   ep.stage_ok = (ep.nchw_ohw == 0) && (((size_t)ep.ldy * esz) % 16 == 0) && (((size_t)ep.n_offset * esz) % 16 == 0) &&
+                 (((uintptr_t)ep.Y & 15) == 0);
+   ep.vec_param = (ep.n_offset % 4 == 0) && (!ep.bias || ((uintptr_t)ep.bias & 15) == 0) &&
+                  (!ep.scale || ((uintptr_t)ep.scale & 15) == 0);
+   // SOFIE_HIP_GEMM_VARIANT: tuning alternative of the pipelined kernel; -1 = general kernel only
+   const char *v = getenv("SOFIE_HIP_GEMM_VARIANT");
+   return launch_mfma8_best<MfmaI8, I8Epilogue>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile, v ? atoi(v) : 0);
 }
 
 // SOFIE_HIP_I8_TILE=256|128|64 forces a tile configuration (tuning and tests); unset = heuristic.
@@ -138,7 +143,8 @@ int sofie_hip_gemm_i8(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d)
    ep.out = d->out;
    ep.Y = d->Y;
    ep.ldy = ldy;
-   ep.vec_store = 0;
+   ep.stage_ok = 0;
+   ep.vec_param = 0;
    ep.N = N;
    ep.nchw_ohw = 0;
    ep.n_offset = 0;

@@ -1,8 +1,8 @@
 // Store stage of the int8 GEMM and of the int8 convolution: bias, requantisation or dequantisation,
 // optional relu, and the output addressing (row-major [M,N], or NCHW when the GEMM rows are the
-// output pixels of a convolution).
+// output pixels of a convolution).  Plugs into tile_store_via_lds (mfma8_common.hpp).
 #pragma once
-#include "mfma8_gemm.hpp"
+#include "mfma8_gemm_dma.hpp"
 
 namespace sofie_hip {
 
@@ -14,93 +14,120 @@ struct I8Epilogue {
    int relu_acc, relu_out, out;
    void *Y;
    int ldy;
-   int vec_store; // Y/ldy alignment allows vector stores of 4 consecutive columns
+   int stage_ok;  // row-major Y whose rows allow 16-byte stores
+   int vec_param; // bias/scale may be read as 16-byte vectors
    int N;         // number of valid columns
    int nchw_ohw;  // 0: Y[m*ldy + n]; else m = (img, pix) and Y[(img*ldy + n)*nchw_ohw + pix], ldy = Cout
    int n_offset;  // added to n for bias/scale/Y addressing (grouped convolution)
 
-   __device__ __forceinline__ void store_one(size_t idx, int acc, float s) const
+   template <class F>
+   __device__ __forceinline__ void dispatch(F f) const
    {
       switch (out) {
-      case SOFIE_I8OUT_I32: ((int32_t *)Y)[idx] = acc; break;
-      case SOFIE_I8OUT_F32: {
-         float v = mul_nofma((float)acc, s);
-         if (relu_out)
-            v = v > 0.0f ? v : 0.0f;
-         ((float *)Y)[idx] = v;
-      } break;
-      case SOFIE_I8OUT_I8: {
+      case SOFIE_I8OUT_I32: f(std::integral_constant<int, SOFIE_I8OUT_I32>{}); break;
+      case SOFIE_I8OUT_F32: f(std::integral_constant<int, SOFIE_I8OUT_F32>{}); break;
+      case SOFIE_I8OUT_I8: f(std::integral_constant<int, SOFIE_I8OUT_I8>{}); break;
+      default: f(std::integral_constant<int, SOFIE_I8OUT_I8_DQQ>{}); break;
+      }
+   }
+   template <int OUT>
+   static constexpr int out_bytes()
+   {
+      return (OUT == SOFIE_I8OUT_I32 || OUT == SOFIE_I8OUT_F32) ? 4 : 1;
+   }
+   __device__ __forceinline__ bool rows_vectorizable() const { return stage_ok != 0; }
+   __device__ __forceinline__ char *out_base() const { return (char *)Y; }
+   __device__ __forceinline__ size_t out_index(int m, int n) const
+   {
+      if (nchw_ohw) {
+         const int img = m / nchw_ohw, pix = m - img * nchw_ohw;
+         return ((size_t)img * ldy + (n + n_offset)) * nchw_ohw + pix;
+      }
+      return (size_t)m * (size_t)ldy + n + n_offset;
+   }
+
+   // DequantizeLinear of one accumulator: one fp32 multiply, then max(.,0) if relu_out
+   __device__ __forceinline__ float to_f32(int acc, float s) const
+   {
+      float v = mul_nofma((float)acc, s);
+      if (relu_out)
+         v = v > 0.0f ? v : 0.0f;
+      return v;
+   }
+   // requantisation: sat8(rne(float(acc)*s)) then relu, or sat8(rne((float(acc)*s)/q_scale))
+   template <int OUT>
+   __device__ __forceinline__ int to_i8(int acc, float s) const
+   {
+      if (OUT == SOFIE_I8OUT_I8) {
          int q = quantize_rne_sat8(mul_nofma((float)acc, s));
          if (relu_out)
             q = q > 0 ? q : 0;
-         ((int8_t *)Y)[idx] = (int8_t)q;
-      } break;
-      default: ((int8_t *)Y)[idx] = (int8_t)quantize_rne_sat8(__fdiv_rn(mul_nofma((float)acc, s), q_scale)); break;
+         return q;
+      }
+      return quantize_rne_sat8(__fdiv_rn(mul_nofma((float)acc, s), q_scale));
+   }
+
+   // bias and scale of C consecutive columns
+   template <int C>
+   struct col_params {
+      int b[C];
+      float s[C];
+   };
+   template <int C>
+   __device__ __forceinline__ void load_params(int n, col_params<C> &p) const
+   {
+      if (vec_param && n + C <= N) {
+#pragma unroll
+         for (int q = 0; q < C / 4; ++q) {
+            v4i b = {0, 0, 0, 0};
+            if (bias)
+               b = *(const v4i *)(bias + n + n_offset + 4 * q);
+            float4 f = make_float4(scale_scalar, scale_scalar, scale_scalar, scale_scalar);
+            if (scale)
+               f = *(const float4 *)(scale + n + n_offset + 4 * q);
+            p.b[4 * q + 0] = b[0], p.b[4 * q + 1] = b[1], p.b[4 * q + 2] = b[2], p.b[4 * q + 3] = b[3];
+            p.s[4 * q + 0] = f.x, p.s[4 * q + 1] = f.y, p.s[4 * q + 2] = f.z, p.s[4 * q + 3] = f.w;
+         }
+      } else {
+#pragma unroll
+         for (int i = 0; i < C; ++i) {
+            const int nn = (n + i < N ? n + i : N - 1) + n_offset;
+            p.b[i] = bias ? bias[nn] : 0;
+            p.s[i] = scale ? scale[nn] : scale_scalar;
+         }
       }
    }
 
-   // 4 consecutive columns n..n+3 of row m; `a*` hold the exact int32 dot products.
-   __device__ __forceinline__ void store4(int m, int n, int a0, int a1, int a2, int a3) const
+   // converts columns 4q..4q+3 of the lane's columns (exact int32 dot products) into 4*out_bytes() bytes
+   template <int OUT, int C>
+   __device__ __forceinline__ void pack4(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, uint32_t *w) const
    {
       int acc[4] = {a0, a1, a2, a3};
       float s[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-         int nn = (n + i < N ? n + i : N - 1) + n_offset;
-         int b = bias ? bias[nn] : 0;
-         s[i] = scale ? scale[nn] : scale_scalar;
-         acc[i] += b;
+         acc[i] += p.b[4 * q + i];
+         s[i] = p.s[4 * q + i];
          if (relu_acc)
             acc[i] = acc[i] > 0 ? acc[i] : 0;
       }
-      if (nchw_ohw) {
-         const int img = m / nchw_ohw, pix = m - img * nchw_ohw;
+      if (OUT == SOFIE_I8OUT_I32) {
 #pragma unroll
          for (int i = 0; i < 4; ++i)
-            if (n + i < N)
-               store_one(((size_t)img * ldy + (n + i + n_offset)) * nchw_ohw + pix, acc[i], s[i]);
-         return;
-      }
-      const size_t row = (size_t)m * (size_t)ldy + n + n_offset;
-      if (!((n + 3 < N) && vec_store)) {
+            w[i] = (uint32_t)acc[i];
+      } else if (OUT == SOFIE_I8OUT_F32) {
 #pragma unroll
          for (int i = 0; i < 4; ++i)
-            if (n + i < N)
-               store_one(row + i, acc[i], s[i]);
-         return;
-      }
-      switch (out) {
-      case SOFIE_I8OUT_I32: *(v4i *)((int32_t *)Y + row) = v4i{acc[0], acc[1], acc[2], acc[3]}; break;
-      case SOFIE_I8OUT_F32: {
-         float v[4];
-#pragma unroll
-         for (int i = 0; i < 4; ++i) {
-            v[i] = mul_nofma((float)acc[i], s[i]);
-            if (relu_out)
-               v[i] = v[i] > 0.0f ? v[i] : 0.0f;
-         }
-         *(float4 *)((float *)Y + row) = make_float4(v[0], v[1], v[2], v[3]);
-      } break;
-      default: {
-         int q[4];
-#pragma unroll
-         for (int i = 0; i < 4; ++i) {
-            if (out == SOFIE_I8OUT_I8) {
-               q[i] = quantize_rne_sat8(mul_nofma((float)acc[i], s[i]));
-               if (relu_out)
-                  q[i] = q[i] > 0 ? q[i] : 0;
-            } else {
-               q[i] = quantize_rne_sat8(__fdiv_rn(mul_nofma((float)acc[i], s[i]), q_scale));
-            }
-         }
-         *(uint32_t *)((int8_t *)Y + row) = (uint32_t)(q[0] & 0xff) | ((uint32_t)(q[1] & 0xff) << 8) |
-                                            ((uint32_t)(q[2] & 0xff) << 16) | ((uint32_t)(q[3] & 0xff) << 24);
-      } break;
+            w[i] = __float_as_uint(to_f32(acc[i], s[i]));
+      } else {
+         const int q0 = to_i8<OUT>(acc[0], s[0]), q1 = to_i8<OUT>(acc[1], s[1]), q2 = to_i8<OUT>(acc[2], s[2]),
+                   q3 = to_i8<OUT>(acc[3], s[3]);
+         w[0] = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) | ((uint32_t)(q3 & 0xff) << 24);
       }
    }
 };
 
-// Y = epilogue(A[M,K] * Bt[N,K]^T); fills ep.vec_store and ep.N.  force_tile 0 = heuristic.
+// Y = epilogue(A[M,K] * Bt[N,K]^T); fills the derived fields of ep.  force_tile 0 = heuristic.
 int gemm_i8_nt(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep,
                int force_tile);
 int forced_i8_tile();

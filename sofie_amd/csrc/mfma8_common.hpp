@@ -1,0 +1,225 @@
+// Pieces shared by the int8 / FP8 matrix-core GEMM kernels: MFMA wrappers, the workgroup -> tile map,
+// the swizzled LDS slab layout and the tile store through LDS.
+#pragma once
+#include "common.hpp"
+#include <cstdlib>
+#include <type_traits>
+#include <utility>
+
+namespace sofie_hip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// Compile-time loop: f(std::integral_constant<int,0>{}), ..., f(std::integral_constant<int,N-1>{}).
+// Accumulator registers can only be named with compile-time indices; a run-time index would push the
+// whole accumulator array out of the register file.
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, Is...>)
+{
+   (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+   static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// int8: v_mfma_i32_32x32x32_i8, 16 bytes of K per lane and step.
+struct MfmaI8 {
+   typedef v16i acc_t;
+   typedef int elem_t;
+   static constexpr int KSTEP = 32; // K bytes per MFMA
+   static constexpr int CHUNKS = 1; // 16-byte chunks per lane and operand
+   struct frag_t {
+      v4i c[1];
+   };
+   static __device__ __forceinline__ acc_t mma(const frag_t &a, const frag_t &b, acc_t c)
+   {
+      return __builtin_amdgcn_mfma_i32_32x32x32_i8(a.c[0], b.c[0], c, 0, 0, 0);
+   }
+};
+
+// FP8 e4m3fn: v_mfma_f32_32x32x64_f8f6f4 (format code 0 = e4m3 for both operands, no block scaling),
+// 32 bytes of K per lane and step.
+struct MfmaF8 {
+   typedef v16f acc_t;
+   typedef float elem_t;
+   static constexpr int KSTEP = 64;
+   static constexpr int CHUNKS = 2;
+   struct frag_t {
+      v4i c[2];
+   };
+   static __device__ __forceinline__ acc_t mma(const frag_t &a, const frag_t &b, acc_t c)
+   {
+      v8i va = {a.c[0][0], a.c[0][1], a.c[0][2], a.c[0][3], a.c[1][0], a.c[1][1], a.c[1][2], a.c[1][3]};
+      v8i vb = {b.c[0][0], b.c[0][1], b.c[0][2], b.c[0][3], b.c[1][0], b.c[1][1], b.c[1][2], b.c[1][3]};
+      return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, vb, c, 0, 0, 0, 0, 0, 0);
+   }
+};
+
+// Maps the hardware workgroup id to an output tile.  Workgroups are dealt round-robin to the 8 XCDs,
+// each with its own L2: ids that land on one XCD are made consecutive, and consecutive ids walk the
+// tile grid in bands of `mode & 0xff` tile rows (0: plain row-major order), so the tiles resident on one
+// XCD at a time share A and Bt slabs through that XCD's L2.  mode & 0x100 skips the XCD regrouping.
+__device__ __forceinline__ void tile_of_block(int bid, int nwg, int tiles_m, int tiles_n, int mode, int &tm, int &tn)
+{
+   constexpr int NXCD = 8;
+   int id = bid;
+   if (!(mode & 0x100)) {
+      const int per = nwg / NXCD, rem = nwg % NXCD;
+      const int xcd = bid % NXCD, local = bid / NXCD;
+      id = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + local;
+   }
+   const int gm = mode & 0xff;
+   if (gm == 0) {
+      tm = id / tiles_n;
+      tn = id % tiles_n;
+      return;
+   }
+   const int width = gm * tiles_n;
+   const int group = id / width;
+   const int first_m = group * gm;
+   const int gsz = (tiles_m - first_m) < gm ? (tiles_m - first_m) : gm;
+   tm = first_m + (id % width) % gsz;
+   tn = (id % width) / gsz;
+}
+
+// SOFIE_HIP_SWIZZLE overrides the tile order (tuning); default: XCD regrouping, bands of 4 tile rows.
+inline int swizzle_mode()
+{
+   const char *s = getenv("SOFIE_HIP_SWIZZLE");
+   return s ? (int)strtol(s, nullptr, 0) : 4;
+}
+
+// Byte offset of 16-byte chunk c of row r in an LDS slab of BK-byte rows.  Chunk c is stored at chunk
+// position c ^ ((r / rows_per_256B) % chunks_per_row): the 16 lanes served together by one ds_read_b128
+// (16 consecutive rows, same logical chunk) then fall into 16 different 16-byte bank groups.
+template <int BK>
+__device__ __forceinline__ int lds_chunk_offset(int r, int c)
+{
+   constexpr int CPR = BK / 16;
+   constexpr int RPB = (256 / BK) > 0 ? (256 / BK) : 1;
+   return r * BK + (((c ^ ((r / RPB) % CPR))) << 4);
+}
+
+// Plain row-major operand: row r starts at base + r*ld.
+struct RowMajorRows {
+   const int8_t *base;
+   int ld;
+   __device__ __forceinline__ const int8_t *row(int r) const { return base + (size_t)r * (size_t)ld; }
+};
+
+// LDS bytes one wave needs for the tile store below (TN = columns of the wave tile).
+constexpr int tile_store_lds_bytes(int TN) { return 32 * (TN * 4 + 16); }
+
+// Tile store through LDS.  After the MFMAs a lane holds, per register group, 4 consecutive columns of
+// ONE row, and the 32 lanes of a half-wave hold 32 different rows; stored directly, a wave instruction
+// would touch 64 rows with 4..16 bytes each.  Instead, for each 32-row block of its tile, a wave parks the
+// raw 32-bit accumulators in its own LDS region (row stride TN*4+16 bytes: 16-byte aligned and spread
+// over the banks) and re-reads them row by row in a run-time loop, so that a lane converts and stores 16
+// consecutive output bytes and a wave instruction writes whole 128-byte lines.  Only the parking code is
+// unrolled over the accumulator registers; the conversion exists once per output mode, which keeps the
+// kernel small enough for the instruction cache.
+//
+// EPI provides
+//   template <class F> void dispatch(F f) const     f(std::integral_constant<int, MODE>{}) for the output mode
+//   template <int MODE> static constexpr int out_bytes()          bytes of one output element (1, 2, 4)
+//   struct col_params<C>; template <int C> void load_params(int n, col_params<C> &p) const
+//                                per-column constants (bias, scale) of columns n..n+C-1, clamped to N-1;
+//                                a lane's columns are the same for every row it stores, so they are fetched once
+//   template <int MODE, int C> void pack4(const col_params<C> &p, int q, T a0, T a1, T a2, T a3, uint32_t *w) const
+//                                converts columns 4q..4q+3 of the lane's C columns into 4*out_bytes bytes
+//   bool rows_vectorizable() const                row-major output whose rows allow 16-byte stores
+//   char *out_base() const;  size_t out_index(int m, int n) const     element index of (m,n)
+template <int MODE, int MT, int NT, class EPI, class ACC>
+__device__ __forceinline__ void tile_store_via_lds(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int M, int N,
+                                                   int lane, char *wsm)
+{
+   typedef typename std::remove_reference<decltype(acc[0][0][0])>::type elem_t;
+   constexpr int ESZ = EPI::template out_bytes<MODE>();
+   constexpr int TN = NT * 32;
+   constexpr int ROWB = TN * 4 + 16;
+   const int lr = lane & 31, lk = lane >> 5;
+   char *out = ep.out_base();
+   const bool vec = ep.rows_vectorizable();
+   static_for<MT>([&](auto ci) {
+      constexpr int i = decltype(ci)::value;
+      static_for<NT>([&](auto cj) {
+         constexpr int j = decltype(cj)::value;
+         static_for<4>([&](auto cg) {
+            constexpr int g = decltype(cg)::value;
+            typedef elem_t v4e __attribute__((ext_vector_type(4)));
+            *(v4e *)(wsm + lr * ROWB + (j * 32 + g * 8 + lk * 4) * 4) =
+               v4e{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+         });
+      });
+      __builtin_amdgcn_wave_barrier();
+      const int m_first = m_base + i * 32;
+      if (vec) {
+         constexpr int CPL = 16 / ESZ;     // columns per lane
+         constexpr int LPR = TN / CPL;     // lanes per row
+         constexpr int RPP = 64 / LPR;     // rows per pass
+         static_assert(TN % CPL == 0 && LPR <= 64 && 32 % RPP == 0, "wave tile width not supported by the tile store");
+         const int c0 = (lane % LPR) * CPL;
+         const int n = n_base + c0;
+         typename EPI::template col_params<CPL> prm;
+         ep.template load_params<CPL>(n < N ? n : N - 1, prm);
+#pragma unroll 1
+         for (int row0 = 0; row0 < 32; row0 += RPP) {
+            const int row = row0 + lane / LPR;
+            const int m = m_first + row;
+            if (m < M && n < N) {
+               uint32_t w[4];
+#pragma unroll
+               for (int q = 0; q < CPL / 4; ++q) {
+                  typedef elem_t v4e __attribute__((ext_vector_type(4)));
+                  const v4e a = *(const v4e *)(wsm + row * ROWB + (c0 + 4 * q) * 4);
+                  ep.template pack4<MODE, CPL>(prm, q, a[0], a[1], a[2], a[3], w + q * ESZ);
+               }
+               char *y = out + ep.out_index(m, n) * ESZ;
+               if (n + CPL <= N) {
+                  *(uint4 *)y = make_uint4(w[0], w[1], w[2], w[3]);
+               } else {
+                  const char *src = (const char *)w;
+                  for (int b = 0; b < (N - n) * ESZ; ++b)
+                     y[b] = src[b];
+               }
+            }
+         }
+      } else {
+         // any layout: a lane converts 4 columns and stores them one element at a time
+         constexpr int LPR = TN / 4;
+         constexpr int RPP = (64 / LPR) > 0 ? (64 / LPR) : 1;
+         static_assert(LPR <= 64, "wave tile too wide");
+         const int c0 = (lane % LPR) * 4;
+         const int n = n_base + c0;
+         typename EPI::template col_params<4> prm;
+         ep.template load_params<4>(n < N ? n : N - 1, prm);
+#pragma unroll 1
+         for (int row0 = 0; row0 < 32; row0 += RPP) {
+            const int row = row0 + lane / LPR;
+            const int m = m_first + row;
+            if (m < M && n < N) {
+               typedef elem_t v4e __attribute__((ext_vector_type(4)));
+               const v4e a = *(const v4e *)(wsm + row * ROWB + c0 * 4);
+               uint32_t w[4];
+               ep.template pack4<MODE, 4>(prm, 0, a[0], a[1], a[2], a[3], w);
+               const char *src = (const char *)w;
+               for (int e = 0; e < 4 && n + e < N; ++e) {
+                  char *y = out + ep.out_index(m, n + e) * ESZ;
+                  for (int b = 0; b < ESZ; ++b)
+                     y[b] = src[e * ESZ + b];
+               }
+            }
+         }
+      }
+      __builtin_amdgcn_wave_barrier();
+   });
+}
+
+int transpose_i8(hipStream_t stream, int8_t *dst, const int8_t *src, int rows, int cols, int ld_src, int ld_dst);
+
+} // namespace sofie_hip

@@ -1,83 +1,17 @@
-// Tile loop shared by the int8 and the FP8 GEMM: 1-byte operands, both K-contiguous in HBM ("NT"
-// form: A is [M,K] row-major, Bt is [N,K] row-major), 32x32 MFMA tiles, LDS double buffer.
+// General tile loop of the int8 and the FP8 GEMM: any K, any alignment.  1-byte operands, both
+// K-contiguous in HBM ("NT" form: A is [M,K] row-major, Bt is [N,K] row-major), 32x32 MFMA tiles,
+// slabs staged global -> registers -> LDS with one slab of prefetch.  Shapes that allow it run the
+// pipelined kernel of mfma8_gemm_dma.hpp instead; this one is the safety net (K tails, odd strides).
 //
-// A workgroup owns a BM x BN tile of Y and walks K in slabs of BK bytes.  A slab of A and of Bt is
-// staged in LDS as rows of BK bytes cut into 16-byte chunks; chunk c of row r is stored at chunk
-// position c ^ ((r / rows_per_256B) % chunks_per_row), so that the 16 lanes served together by one
-// ds_read_b128 (16 consecutive rows, same logical chunk) fall into 16 different 16-byte bank groups.
-// The MFMA is issued with the Bt rows as its first operand and the A rows as its second, so that a
-// lane ends up holding 4 consecutive output columns n of one output row m and can store them as one
-// vector.  Which K bytes a lane feeds to the MFMA only has to be the same for both operands, because
-// the dot product does not depend on the order of its terms (exactly for int8, to rounding for FP8).
+// A workgroup owns a BM x BN tile of Y and walks K in slabs of BK bytes kept in the swizzled LDS layout
+// of lds_chunk_offset.  The MFMA is issued with the Bt rows as its first operand and the A rows as its
+// second, so that a lane ends up holding 4 consecutive output columns n of one output row m.  Which K
+// bytes a lane feeds to the MFMA only has to be the same for both operands, because the dot product does
+// not depend on the order of its terms (exactly for int8, to rounding for FP8).
 #pragma once
-#include "common.hpp"
+#include "mfma8_common.hpp"
 
 namespace sofie_hip {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-
-// int8: v_mfma_i32_32x32x32_i8, 16 bytes of K per lane and step.
-struct MfmaI8 {
-   typedef v16i acc_t;
-   typedef int elem_t;
-   static constexpr int KSTEP = 32;  // K bytes per MFMA
-   static constexpr int CHUNKS = 1;  // 16-byte chunks per lane and operand
-   struct frag_t {
-      v4i c[1];
-   };
-   static __device__ __forceinline__ acc_t mma(const frag_t &a, const frag_t &b, acc_t c)
-   {
-      return __builtin_amdgcn_mfma_i32_32x32x32_i8(a.c[0], b.c[0], c, 0, 0, 0);
-   }
-};
-
-// FP8 e4m3fn: v_mfma_f32_32x32x64_f8f6f4 (format code 0 = e4m3 for both operands, no block scaling),
-// 32 bytes of K per lane and step.
-struct MfmaF8 {
-   typedef v16f acc_t;
-   typedef float elem_t;
-   static constexpr int KSTEP = 64;
-   static constexpr int CHUNKS = 2;
-   struct frag_t {
-      v4i c[2];
-   };
-   static __device__ __forceinline__ acc_t mma(const frag_t &a, const frag_t &b, acc_t c)
-   {
-      v8i va = {a.c[0][0], a.c[0][1], a.c[0][2], a.c[0][3], a.c[1][0], a.c[1][1], a.c[1][2], a.c[1][3]};
-      v8i vb = {b.c[0][0], b.c[0][1], b.c[0][2], b.c[0][3], b.c[1][0], b.c[1][1], b.c[1][2], b.c[1][3]};
-      return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, vb, c, 0, 0, 0, 0, 0, 0);
-   }
-};
-
-// Maps the hardware workgroup id to an output tile.  Workgroups are dealt round-robin to the 8 XCDs,
-// each with its own L2: ids that land on one XCD are made consecutive, and consecutive ids walk the
-// tile grid in bands of GROUP_M tile rows, so the tiles resident on one XCD at a time share A and Bt
-// slabs through that XCD's L2.
-__device__ __forceinline__ void tile_of_block(int bid, int nwg, int tiles_m, int tiles_n, int &tm, int &tn)
-{
-   constexpr int NXCD = 8;
-   constexpr int GROUP_M = 4;
-   const int per = nwg / NXCD, rem = nwg % NXCD;
-   const int xcd = bid % NXCD, local = bid / NXCD;
-   const int id = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + local;
-   const int width = GROUP_M * tiles_n;
-   const int group = id / width;
-   const int first_m = group * GROUP_M;
-   const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-   tm = first_m + (id % width) % gsz;
-   tn = (id % width) / gsz;
-}
-
-template <int BK>
-__device__ __forceinline__ int lds_chunk_offset(int r, int c)
-{
-   constexpr int CPR = BK / 16;                          // 16-byte chunks per row
-   constexpr int RPB = (256 / BK) > 0 ? (256 / BK) : 1;  // rows per 256 bytes of LDS
-   return r * BK + (((c ^ ((r / RPB) % CPR))) << 4);
-}
 
 // Loads one 16-byte chunk (bytes k..k+15 of the row at `row_ptr`); bytes at k >= K read as 0.
 template <bool ALIGNED>
@@ -102,18 +36,17 @@ __device__ __forceinline__ v4i load_chunk(const int8_t *row_ptr, int k, int K)
    }
 }
 
-// Plain row-major operand: row r starts at base + r*ld.
-struct RowMajorRows {
-   const int8_t *base;
-   int ld;
-   __device__ __forceinline__ const int8_t *row(int r) const { return base + (size_t)r * (size_t)ld; }
-};
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+constexpr size_t mfma8_general_lds_bytes()
+{
+   constexpr size_t ring = 2 * (size_t)(BM + BN) * BK;
+   constexpr size_t store = (size_t)WAVES_M * WAVES_N * tile_store_lds_bytes(BN / WAVES_N);
+   return ring > store ? ring : store;
+}
 
-// EPI must provide: void store4(int m, int n, elem_t a0, elem_t a1, elem_t a2, elem_t a3) const
-// for the 4 consecutive columns n..n+3 of row m (n < N guaranteed, n+3 may exceed N-1).
 template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool ALIGNED, class EPI>
-__device__ __forceinline__ void mfma8_gemm_tile(const RowMajorRows A, const RowMajorRows Bt, int M, int N, int K,
-                                                const EPI &ep, int tm, int tn, int8_t *smem)
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_kernel(RowMajorRows A, RowMajorRows Bt, int M, int N,
+                                                                            int K, EPI ep, int tiles_m, int tiles_n, int sw)
 {
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
    constexpr int CPR = BK / 16;
@@ -126,9 +59,12 @@ __device__ __forceinline__ void mfma8_gemm_tile(const RowMajorRows A, const RowM
    typedef typename MMA::acc_t acc_t;
    typedef typename MMA::frag_t frag_t;
 
+   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
    int8_t *sA = smem;               // [2][BM*BK]
    int8_t *sB = smem + 2 * BM * BK; // [2][BN*BK]
 
+   int tm, tn;
+   tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, sw, tm, tn);
    const int m0 = tm * BM, n0 = tn * BN;
    const int t = threadIdx.x;
    const int lane = t & 63, wave = t >> 6;
@@ -213,33 +149,25 @@ __device__ __forceinline__ void mfma8_gemm_tile(const RowMajorRows A, const RowM
       __syncthreads();
    }
 
-   // epilogue: lane holds row m = .. + lane%32 and, per group g of 4 registers, columns
-   // n = .. + 8*g + 4*(lane/32) + {0,1,2,3}
-#pragma unroll
-   for (int i = 0; i < MT; ++i) {
-      const int m = m0 + wm * TM + i * 32 + lr;
-      if (m >= M)
-         continue;
-#pragma unroll
-      for (int j = 0; j < NT; ++j) {
-#pragma unroll
-         for (int g = 0; g < 4; ++g) {
-            const int n = n0 + wn * TN + j * 32 + g * 8 + lk * 4;
-            if (n < N)
-               ep.store4(m, n, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-         }
-      }
-   }
+   // the slabs are dead (the loop ends with a barrier): the tile store reuses LDS, one region per wave
+   char *wsm = (char *)smem + wave * tile_store_lds_bytes(TN);
+   ep.dispatch([&](auto mode) {
+      tile_store_via_lds<decltype(mode)::value, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, M, N, lane, wsm);
+   });
 }
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool ALIGNED, class EPI>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_kernel(RowMajorRows A, RowMajorRows Bt, int M, int N,
-                                                                            int K, EPI ep, int tiles_m, int tiles_n)
+// One attribute call per kernel and device (it is far slower than a launch).
+template <class KERN>
+static int configure_lds_once(KERN kern, size_t smem, bool (&configured)[64])
 {
-   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
-   int tm, tn;
-   tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
-   mfma8_gemm_tile<MMA, BM, BN, BK, WAVES_M, WAVES_N, ALIGNED, EPI>(A, Bt, M, N, K, ep, tm, tn, smem);
+   int dev = 0;
+   SOFIE_HIP_CHECK(hipGetDevice(&dev));
+   if (dev < 0 || dev >= 64 || !configured[dev]) {
+      SOFIE_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+      if (dev >= 0 && dev < 64)
+         configured[dev] = true;
+   }
+   return SOFIE_HIP_OK;
 }
 
 template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, class EPI>
@@ -250,46 +178,52 @@ static int launch_mfma8(hipStream_t stream, const int8_t *A, const int8_t *Bt, i
    const long long nwg = (long long)tiles_m * tiles_n;
    if (nwg > 0x7fffffffLL)
       return fail(SOFIE_HIP_ERR_INVALID, "gemm: too many tiles");
-   constexpr size_t smem = 2 * (size_t)(BM + BN) * BK;
+   constexpr size_t smem = mfma8_general_lds_bytes<BM, BN, BK, WAVES_M, WAVES_N>();
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
    RowMajorRows a{A, lda}, b{Bt, ldb};
+   const int sw = swizzle_mode();
+   int st;
    if (aligned) {
       auto kern = mfma8_gemm_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, true, EPI>;
-      SOFIE_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n);
+      static bool configured[64] = {};
+      if ((st = configure_lds_once(kern, smem, configured)))
+         return st;
+      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n, sw);
    } else {
       auto kern = mfma8_gemm_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, false, EPI>;
-      SOFIE_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n);
+      static bool configured[64] = {};
+      if ((st = configure_lds_once(kern, smem, configured)))
+         return st;
+      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n, sw);
    }
    return launch_status("mfma8_gemm_kernel");
 }
 
-// Picks the tile: the largest one that still gives every one of the 256 CUs a workgroup.
+// Tile choice: the largest one that still gives every one of the 256 CUs a workgroup.
+inline int pick_tile(int M, int N, int force_tile)
+{
+   if (force_tile)
+      return force_tile;
+   auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+   if (tiles(256, 256) >= 256)
+      return 256;
+   if (tiles(128, 128) >= 192)
+      return 128;
+   return 64;
+}
+
 template <class MMA, class EPI>
 static int launch_mfma8_auto(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb,
                              const EPI &ep, int force_tile)
 {
    const bool aligned = (K % 16 == 0) && (lda % 16 == 0) && (ldb % 16 == 0) && (((uintptr_t)A & 15) == 0) &&
                         (((uintptr_t)Bt & 15) == 0);
-   auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-   int tile = force_tile;
-   if (tile == 0) {
-      if (tiles(256, 256) >= 256)
-         tile = 256;
-      else if (tiles(128, 128) >= 192)
-         tile = 128;
-      else
-         tile = 64;
-   }
-   switch (tile) {
+   switch (pick_tile(M, N, force_tile)) {
    case 256: return launch_mfma8<MMA, 256, 256, 64, 2, 2, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, aligned);
    case 128: return launch_mfma8<MMA, 128, 128, 64, 2, 2, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, aligned);
    case 64: return launch_mfma8<MMA, 64, 64, 64, 2, 2, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, aligned);
-   default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", tile);
+   default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", force_tile);
    }
 }
-
-int transpose_i8(hipStream_t stream, int8_t *dst, const int8_t *src, int rows, int cols, int ld_src, int ld_dst);
 
 } // namespace sofie_hip

@@ -114,6 +114,11 @@ def load_library(path=None):
     if _lib is not None and path is None:
         return _lib
     p = path or lib_path()
+    # torch wheels carry their own copy of the HIP runtime.  When torch shares the process (the tests use
+    # it to allocate device buffers) it has to initialise first, so that one runtime serves both.
+    import sys
+    if "torch" in sys.modules:
+        sys.modules["torch"].cuda.is_available()
     if not os.path.exists(p):
         raise SofieHipError("%s is not built: run `python -c 'import __graft_entry__ as g; g.build()'`" % p)
     lib = C.CDLL(p)
