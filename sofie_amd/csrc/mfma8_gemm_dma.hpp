@@ -40,7 +40,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(R
    constexpr int KS = BK / MMA::KSTEP;
    constexpr int STAGE_BYTES = (BM + BN) * BK;
    static_assert(BM % (RPI * NW) == 0 && BN % (RPI * NW) == 0, "tile rows must divide over the waves");
-   static_assert(STAGES >= 3 && (STAGES - 1) * LPT < 64, "ring needs >= 3 slots; vmcnt counts < 64 loads");
+   static_assert((STAGES - 1) * LPT < 64, "vmcnt counts fewer than 64 loads");
    typedef typename MMA::acc_t acc_t;
    typedef typename MMA::frag_t frag_t;
 
@@ -72,18 +72,24 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(R
       const int gr = n0 + row;
       gb[i] = Bt.row(gr < N ? gr : N - 1) + c * 16;
    }
-   auto issue_loads = [&](int kt, int stage) {
+   // One K-step's share of a slab's load instructions (A's first, then Bt's): part `part` of KS equal parts.
+   constexpr int KS_ = BK / MMA::KSTEP;
+   static_assert(LPT % KS_ == 0, "slab loads must divide over the K-steps");
+   auto issue_loads = [&](int kt, int stage, auto part_c) {
+      constexpr int part = decltype(part_c)::value; // 0..KS-1, or -1 for the whole slab
       if (DBG & 1)
          return;
       int8_t *sA = smem + stage * STAGE_BYTES;
       int8_t *sB = sA + BM * BK;
       const int koff = kt * BK;
-#pragma unroll
-      for (int i = 0; i < A_LD; ++i)
-         __builtin_amdgcn_global_load_lds((global_void_t *)(ga[i] + koff), (lds_void_t *)(sA + (i * NW + wave) * 1024), 16, 0, 0);
-#pragma unroll
-      for (int i = 0; i < B_LD; ++i)
-         __builtin_amdgcn_global_load_lds((global_void_t *)(gb[i] + koff), (lds_void_t *)(sB + (i * NW + wave) * 1024), 16, 0, 0);
+      constexpr int L0 = part < 0 ? 0 : part * (LPT / KS_), L1 = part < 0 ? LPT : (part + 1) * (LPT / KS_);
+      static_for<L1 - L0>([&](auto lc) {
+         constexpr int l = L0 + decltype(lc)::value;
+         if constexpr (l < A_LD)
+            __builtin_amdgcn_global_load_lds((global_void_t *)(ga[l] + koff), (lds_void_t *)(sA + (l * NW + wave) * 1024), 16, 0, 0);
+         else
+            __builtin_amdgcn_global_load_lds((global_void_t *)(gb[l - A_LD] + koff), (lds_void_t *)(sB + ((l - A_LD) * NW + wave) * 1024), 16, 0, 0);
+      });
    };
 
    acc_t acc[MT][NT];
@@ -95,11 +101,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(R
          for (int v = 0; v < 16; ++v)
             acc[i][j][v] = 0;
 
+   // prologue: slabs 0..STAGES-2 (a slab index past the end re-reads the last slab: harmless filler that
+   // keeps the number of loads per iteration, and with it the vmcnt bookkeeping, constant)
    const int KT = K / BK;
 #pragma unroll
    for (int s = 0; s < STAGES - 1; ++s)
-      if (s < KT)
-         issue_loads(s, s);
+      issue_loads(s < KT ? s : KT - 1, s, std::integral_constant<int, -1>{});
 
    auto read_frags = [&](const int8_t *cA, const int8_t *cB, int ks, frag_t(&fa)[MT], frag_t(&fb)[NT]) {
       if (DBG & 2)
@@ -116,60 +123,67 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(R
             fa[i].c[c] = *(const v4i *)(cA + lds_chunk_offset<BK>(wm * TM + i * 32 + lr, (ks * 2 + lk) * MMA::CHUNKS + c));
    };
 
-   // Software pipeline.  The fragments of K-step s+1 are read from LDS while the MFMAs of step s issue
-   // (one ds_read slotted after every second MFMA), across slab boundaries too: the wait for the next
-   // slab and the workgroup barrier sit inside the last K-step of the current slab, so the first
-   // fragments of slab kt+1 are on their way before the MFMAs of slab kt have drained.
-   //   barrier in the last step of slab kt  =>  every wave's loads of slab kt+1 have landed, and every
-   //   wave has issued all its reads of slab kt-1 (and kt), so the ring slot of slab kt-1 can be refilled.
+   // Software pipeline, one slab per iteration, everything interleaved at instruction granularity so
+   // that neither the LDS nor the vector-memory queue ever sees a burst (a burst of loads blocks the
+   // wave at issue and with it the MFMAs behind them):
+   //   K-step s:  MFMAs of step s  |  ds_reads of the fragments of step s+1  |  1/KS of the loads of slab kt+STAGES-1
+   // The loads of slab kt+STAGES-1 go to the ring slot of slab kt-1.  That slot was released by the barrier
+   // of iteration kt-1, which sits in the LAST K-step of a slab, after the wave has waited for its own
+   // LDS reads: passing it means every wave's loads of the NEXT slab have landed and every wave is done
+   // reading the CURRENT slab's LDS data (its last fragments are in registers).
+   static_assert(KS % 2 == 0, "the fragment double buffer is indexed by the parity of the K-step");
+   static_assert(STAGES >= 3, "the ring needs three slots: one computing, one landing, one being refilled");
    frag_t fa[2][MT], fb[2][NT];
    wait_vmcnt<(STAGES - 2) * LPT>();
-   if (KT < STAGES - 1)
-      wait_vmcnt<0>();
    __builtin_amdgcn_s_barrier();
    read_frags(smem, smem + BM * BK, 0, fa[0], fb[0]);
    int stage = 0;
-   int cur = 0;
+   int lstage = STAGES - 1; // slot refilled during this iteration
    for (int kt = 0; kt < KT; ++kt) {
       const int8_t *cA = smem + stage * STAGE_BYTES;
       const int8_t *cB = cA + BM * BK;
       const int nstage = (stage + 1 == STAGES) ? 0 : stage + 1;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
+      const int lslab = (kt + STAGES - 1 < KT) ? kt + STAGES - 1 : KT - 1;
+      static_for<KS>([&](auto ks_c) {
+         constexpr int ks = decltype(ks_c)::value;
          if (ks == KS - 1) {
-            // slab kt+1 must have landed before its first fragments are read below; slab kt+STAGES-1 is then
-            // requested into the slot slab kt-1 occupied
-            const int ahead = KT - 2 - kt; // slabs issued after kt+1
-            if (ahead >= STAGES - 3)
-               wait_vmcnt<(STAGES - 3) * LPT>();
-            else
-               wait_vmcnt<0>();
+            // issued so far, newest first: parts 0..KS-2 of slab kt+STAGES-1, then slabs kt+STAGES-2 ... kt+1.
+            // Slab kt+1 must have landed.
+            wait_vmcnt<(STAGES - 3) * LPT + (KS - 1) * (LPT / KS)>();
+            __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this wave's LDS reads of slab kt are complete
             __builtin_amdgcn_s_barrier();
-            if (kt + STAGES - 1 < KT)
-               issue_loads(kt + STAGES - 1, (stage + STAGES - 1) % STAGES);
-            // unconditional (after the last slab it reads a dead ring slot and the values are dropped):
-            // a branch here would split the block and undo the read/MFMA interleave
-            read_frags(smem + nstage * STAGE_BYTES, smem + nstage * STAGE_BYTES + BM * BK, 0, fa[cur ^ 1], fb[cur ^ 1]);
+            read_frags(smem + nstage * STAGE_BYTES, smem + nstage * STAGE_BYTES + BM * BK, 0, fa[0], fb[0]);
          } else {
-            read_frags(cA, cB, ks + 1, fa[cur ^ 1], fb[cur ^ 1]);
+            read_frags(cA, cB, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
          }
+         issue_loads(lslab, lstage, ks_c);
 #pragma unroll
          for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int j = 0; j < NT; ++j)
                if (!(DBG & 4))
-                  acc[i][j] = MMA::mma(fb[cur][j], fa[cur][i], acc[i][j]);
+                  acc[i][j] = MMA::mma(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
                else
-                  acc[i][j][0] += fb[cur][j].c[0][0] + fa[cur][i].c[0][0];
-         // interleave: one LDS read after every second MFMA
+                  acc[i][j][0] += fb[ks & 1][j].c[0][0] + fa[ks & 1][i].c[0][0];
+         // issue order within the step: MFMAs with the LDS reads and the loads slotted in between
+         constexpr int NMFMA = MT * NT;
+         constexpr int NREAD = (MT + NT) * MMA::CHUNKS;
+         constexpr int NLOAD = LPT / KS;
+         constexpr int GROUPS = NLOAD > 0 ? NLOAD : 1;
+         constexpr int MPG = NMFMA / GROUPS > 0 ? NMFMA / GROUPS : 1; // MFMAs per group
+         constexpr int RPG = (NREAD + GROUPS - 1) / GROUPS;            // LDS reads per group
 #pragma unroll
-         for (int g = 0; g < (MT + NT) * MMA::CHUNKS; ++g) {
-            __builtin_amdgcn_sched_group_barrier(0x008, (MT * NT) / ((MT + NT) * MMA::CHUNKS) > 0 ? (MT * NT) / ((MT + NT) * MMA::CHUNKS) : 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+         for (int g = 0; g < GROUPS; ++g) {
+            constexpr int HALF = MPG / 2 > 0 ? MPG / 2 : 1;
+            __builtin_amdgcn_sched_group_barrier(0x008, HALF, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, RPG - RPG / 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, MPG - HALF, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, RPG / 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
          }
-         cur ^= 1;
-      }
+      });
       stage = nstage;
+      lstage = (lstage + 1 == STAGES) ? 0 : lstage + 1;
    }
 
    // every wave is done with the ring (and nothing is in flight into it): the tile store reuses it
@@ -191,9 +205,10 @@ static int launch_mfma8_dma(hipStream_t stream, const int8_t *A, const int8_t *B
       return fail(SOFIE_HIP_ERR_INVALID, "gemm: too many tiles");
    if (K % BK != 0 || K < BK)
       return fail(SOFIE_HIP_ERR_INVALID, "gemm: the pipelined kernel needs K to be a multiple of %d", BK);
-   constexpr size_t smem = (size_t)STAGES * (BM + BN) * BK;
+   constexpr size_t ring = (size_t)STAGES * (BM + BN) * BK;
+   constexpr size_t store = (size_t)WAVES_M * WAVES_N * tile_store_lds_bytes(BN / WAVES_N);
+   constexpr size_t smem = ring > store ? ring : store;
    static_assert(smem <= 160 * 1024, "LDS ring larger than the CU's LDS");
-   static_assert(smem >= (size_t)WAVES_M * WAVES_N * tile_store_lds_bytes(BN / WAVES_N), "ring too small for the tile store");
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
    RowMajorRows a{A, lda}, b{Bt, ldb};
    auto kern = mfma8_gemm_dma_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG>;
@@ -218,28 +233,47 @@ static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *
    if (variant < 0 || !aligned || K < 64 || K % 64 != 0)
       return launch_mfma8_auto<MMA, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile);
    const int tile = pick_tile(M, N, force_tile);
-   switch (tile) {
-   case 256:
-      if (variant == 1)
-         return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      if (variant == 2)
-         return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 5, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+   const bool k128 = (K % 128 == 0);
+   if constexpr (MMA::KSTEP * 2 > 64) {
+      // two K-steps per slab are the minimum: a 64-byte K-step needs 128-byte slabs
+      if (!k128)
+         return launch_mfma8_auto<MMA, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile);
+      switch (tile) {
+      case 256: return launch_mfma8_dma<MMA, 256, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      case 128: return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      case 64: return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", tile);
+      }
+   } else {
+      switch (tile) {
+      case 256:
 #ifdef SOFIE_HIP_TUNING
-      if (variant == 11)
-         return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 1>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      if (variant == 12)
-         return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 2>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      if (variant == 13)
-         return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 3>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      if (variant == 14)
-         return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 4>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      if (variant == 16)
-         return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 6>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant >= 10 && variant < 18) {
+            switch (variant - 10) {
+            case 1: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 1>(stream, A, Bt, M, N, K, lda, ldb, ep);
+            case 2: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 2>(stream, A, Bt, M, N, K, lda, ldb, ep);
+            case 3: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 3>(stream, A, Bt, M, N, K, lda, ldb, ep);
+            case 4: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 4>(stream, A, Bt, M, N, K, lda, ldb, ep);
+            case 6: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 6>(stream, A, Bt, M, N, K, lda, ldb, ep);
+            default: break;
+            }
+         }
 #endif
-      return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-   case 128: return launch_mfma8_dma<MMA, 128, 128, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-   case 64: return launch_mfma8_dma<MMA, 64, 64, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-   default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", tile);
+         if (variant == 1)
+            return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 2)
+            return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 5, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      case 128:
+         if (variant == 1 || !k128)
+            return launch_mfma8_dma<MMA, 128, 128, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      case 64:
+         if (variant == 1 || !k128)
+            return launch_mfma8_dma<MMA, 64, 64, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", tile);
+      }
    }
 }
 

@@ -1,0 +1,90 @@
+#!/usr/bin/env python3
+"""Builds the committed golden fixtures from the data files of the reference's own tests.
+
+Reads (never imports or runs) files under /root/reference/tests:
+  models/onnx/<Model>.onnx                 binary model files  -> copied to tests/golden/models/
+  models/onnx/references/<Model>.ref.hxx   expected outputs    -> numbers extracted into fixtures.json
+  alpaka/TestAlpaka*.cxx                   literal input vectors of a few tests -> numbers extracted
+Run in the build container only:  python tests/golden/make_fixtures.py
+"""
+import json
+import os
+import re
+import shutil
+
+REF = "/root/reference/tests"
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+NUM = r"[-+]?(?:\d+\.?\d*|\.\d+)(?:[eE][-+]?\d+)?"
+
+
+def arrays_in(path):
+    """{name: [floats]} for every `float name[...] = {...};` in a C++ header."""
+    text = open(path).read()
+    out = {}
+    for m in re.finditer(r"float\s+(\w+)\s*\[[^\]]*\]\s*=\s*\{(.*?)\}\s*;", text, re.S):
+        body = re.sub(r"//[^\n]*", "", m.group(2))
+        out[m.group(1)] = [float(x) for x in re.findall(NUM, re.sub(r"(?<=[\d.])f\b", "", body))]
+    return out
+
+
+def vector_literal(path, test_name, var):
+    """The numbers of `std::vector<float> var({ ... })` inside TEST_F(..., test_name)."""
+    text = open(path).read()
+    start = text.index("TEST_F(SofieAlpakaTest, %s)" % test_name)
+    m = re.search(r"std::vector<float>\s+%s\s*\(\s*\{(.*?)\}\s*\)" % var, text[start:], re.S)
+    body = re.sub(r"(?<=[\d.])f\b", "", m.group(1))
+    return [float(x) for x in re.findall(NUM, body)]
+
+
+# model -> (expected-array name or None for "the only one", input spec)
+IOTA, ONES = {"kind": "iota"}, {"kind": "ones"}
+MODELS = {
+    "Linear_16": ("all_ones", [ONES]), "Linear_32": ("all_ones", [ONES]), "Linear_64": ("all_ones", [ONES]),
+    "LinearWithSigmoid": ("all_ones", [ONES]),
+    "ConvWithPadding": (None, [IOTA]), "ConvWithoutPadding": (None, [IOTA]), "ConvWithAutopadSameLower": (None, [IOTA]),
+    "ConvWithAutopadSameUpper": (None, [IOTA]), "ConvWithStridesPadding": (None, [IOTA]),
+    "ConvWithStridesNoPadding": (None, [IOTA]), "ConvWithAsymmetricPadding": (None, [IOTA]),
+    "ConvWithDilation": (None, [IOTA]), "ConvWithBias": (None, [IOTA]), "ConvBatch2": (None, [IOTA]),
+    "ConvBatch4": (None, [IOTA]), "ConvBatch8": (None, [IOTA]), "ConvGroup2": (None, [IOTA]), "ConvGroup4": (None, [IOTA]),
+    "ConvBatch4Group2": (None, [IOTA]), "Conv1d": (None, [IOTA]), "GlobalAvgPool2d": (None, [IOTA]),
+}
+
+
+def main():
+    fixtures = {}
+    os.makedirs(os.path.join(HERE, "models"), exist_ok=True)
+
+    def add(model, expected, inputs):
+        shutil.copyfile(os.path.join(REF, "models/onnx", model + ".onnx"), os.path.join(HERE, "models", model + ".onnx"))
+        os.chmod(os.path.join(HERE, "models", model + ".onnx"), 0o644)
+        fixtures[model] = {"inputs": inputs, "expected": expected,
+                           "source": "tests/models/onnx/%s.onnx + references/%s.ref.hxx" % (model, model)}
+
+    for model, (arr, inputs) in MODELS.items():
+        arrays = arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx"))
+        expected = arrays[arr] if arr else next(iter(arrays.values()))
+        add(model, expected, inputs)
+
+    # models whose inputs are literal vectors in the reference's test sources
+    add("ConvGroupBatch", arrays_in(os.path.join(REF, "models/onnx/references/ConvGroupBatch.ref.hxx"))["output"],
+        [{"kind": "values", "values": arrays_in(os.path.join(REF, "models/onnx/references/ConvGroupBatch_input.ref.hxx"))["data"]}])
+    un = os.path.join(REF, "alpaka/TestAlpakaElementwiseUnary.cxx")
+    for model in ("Gelu", "GeluTanh"):
+        add(model, arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx"))["outputs"],
+            [{"kind": "values", "values": vector_literal(un, model, "input")}])
+    lin = os.path.join(REF, "alpaka/TestAlpakaLinear.cxx")
+    add("LinearWithLeakyRelu", arrays_in(os.path.join(REF, "models/onnx/references/LinearWithLeakyRelu.ref.hxx"))["outputs"],
+        [{"kind": "values", "values": vector_literal(lin, "LinearWithLeakyRelu", "input")}])
+    bl = os.path.join(REF, "alpaka/TestAlpakaElementwiseBinaryLogic.cxx")
+    add("AddBroadcast1", arrays_in(os.path.join(REF, "models/onnx/references/AddBroadcast1.ref.hxx"))["output"],
+        [{"kind": "values", "values": vector_literal(bl, "AddBroadcast1", "A_vec")},
+         {"kind": "values", "values": vector_literal(bl, "AddBroadcast1", "B_vec")}])
+
+    with open(os.path.join(HERE, "fixtures.json"), "w") as f:
+        json.dump(fixtures, f, indent=0, sort_keys=True)
+    print("wrote %d fixtures" % len(fixtures))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,223 @@
+"""Runs the small ONNX graphs of the golden fixtures operator by operator, on the CPU oracle or through
+the HIP C-ABI.  The operator attribute conventions are the reference's (file:line cited at each)."""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+
+from tests import onnx_lite
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+ACT = {"Relu": 1, "LeakyRelu": 2, "Sigmoid": 3, "Gelu": 4, "Tanh": 6}
+
+
+def load_fixture(model):
+    fx = json.load(open(os.path.join(GOLDEN, "fixtures.json")))[model]
+    g = onnx_lite.load(os.path.join(GOLDEN, "models", model + ".onnx"))
+    inputs = []
+    for (name, shape), spec in zip(g["inputs"], fx["inputs"]):
+        n = int(np.prod(shape))
+        if spec["kind"] == "iota":
+            a = np.arange(n, dtype=np.float32)
+        elif spec["kind"] == "ones":
+            a = np.ones(n, dtype=np.float32)
+        else:
+            a = np.array(spec["values"], dtype=np.float32)
+        inputs.append(a.reshape(shape))
+    return g, inputs, np.array(fx["expected"], dtype=np.float32)
+
+
+def conv_geometry(attrs, xshape, wshape):
+    """pads / strides / dilations / group as ROperator_Conv::DoShapeInference resolves them
+    (core/inc/SOFIE/operators/ROperator_Conv.hxx:123-262): no `pads` attribute with auto_pad NOTSET means
+    pads of 1 (:172-175); SAME_UPPER/LOWER split (:176-197).  Returns 2-D geometry (1-D gets H=1)."""
+    dim = len(xshape) - 2
+    k = list(attrs.get("kernel_shape", wshape[2:]))
+    strides = list(attrs.get("strides", [1] * dim))
+    dils = list(attrs.get("dilations", [1] * dim))
+    group = attrs.get("group", 1)
+    auto = attrs.get("auto_pad", "NOTSET")
+    spatial = list(xshape[2:])
+    if auto == "NOTSET":
+        pads = list(attrs.get("pads", [1] * (2 * dim)))
+    elif auto in ("SAME_UPPER", "SAME_LOWER"):
+        pads = [0] * (2 * dim)
+        for d in range(dim):
+            ek = k[d] + (dils[d] - 1) * (k[d] - 1)
+            out = (spatial[d] + strides[d] - 1) // strides[d]
+            total = max(0, (out - 1) * strides[d] + ek - spatial[d])
+            lo, hi = (total // 2, total - total // 2) if auto == "SAME_UPPER" else (total - total // 2, total // 2)
+            pads[d], pads[d + dim] = lo, hi
+    elif auto == "VALID":
+        pads = [0] * (2 * dim)
+    else:
+        raise ValueError(auto)
+    if dim == 1:  # H = 1
+        return dict(k=(1, k[0]), pads=(0, pads[0], 0, pads[1]), strides=(1, strides[0]), dils=(1, dils[0]), group=group)
+    return dict(k=(k[0], k[1]), pads=(pads[0], pads[1], pads[2], pads[3]), strides=tuple(strides), dils=tuple(dils), group=group)
+
+
+def fuse(nodes):
+    """The parse-time fusions of the reference that matter here: Gemm followed by Relu on its only
+    consumer becomes one operator (parsers/src/RModelParser_ONNX.cxx:1208-1212)."""
+    out, i = [], 0
+    while i < len(nodes):
+        n = dict(nodes[i])
+        if n["op"] == "Gemm" and i + 1 < len(nodes) and nodes[i + 1]["op"] == "Relu" and nodes[i + 1]["inputs"] == n["outputs"]:
+            n["fused_act"] = 1
+            n["outputs"] = nodes[i + 1]["outputs"]
+            i += 1
+        out.append(n)
+        i += 1
+    return out
+
+
+class OracleBackend:
+    def __init__(self):
+        from oracle import binding
+        self.ob = binding
+
+    def gemm(self, A, B, Cb, transA, transB, alpha, beta, act):
+        M, K = (A.shape[1], A.shape[0]) if transA else A.shape
+        N = B.shape[0] if transB else B.shape[1]
+        mode = 0 if Cb is None else (4 if Cb.shape == (M, N) else 1 if Cb.size == N else 2 if Cb.size == M else 3)
+        return self.ob.gemm_f32(A, B, Cb, M=M, N=N, K=K, transA=transA, transB=transB, alpha=alpha, beta=beta, bias_mode=mode, act=act)
+
+    def unary(self, x, act, alpha):
+        return self.ob.unary(x, act, alpha)
+
+    def conv(self, X, W, b, geo):
+        return self.ob.conv_f32(X, W, b, pads=geo["pads"], strides=geo["strides"], dils=geo["dils"], group=geo["group"])
+
+    def gap(self, X):
+        return self.ob.global_avg_pool(X)
+
+    def add(self, A, B):
+        return self.ob.add_broadcast(A, B)
+
+
+class HipBackend:
+    """Every operator goes through the C-ABI on device buffers."""
+
+    def __init__(self, rt):
+        from sofie_amd import runtime as R
+        from tests import util
+        self.rt, self.R, self.u = rt, R, util
+
+    def gemm(self, A, B, Cb, transA, transB, alpha, beta, act):
+        R, u = self.R, self.u
+        M, K = (A.shape[1], A.shape[0]) if transA else A.shape
+        N = B.shape[0] if transB else B.shape[1]
+        mode = 0 if Cb is None else (4 if Cb.shape == (M, N) else 1 if Cb.size == N else 2 if Cb.size == M else 3)
+        dA, dB = u.to_dev(A), u.to_dev(B)
+        dC = None if Cb is None else u.to_dev(Cb)
+        dY = u.dev_empty((M, N), np.float32)
+        d = R.GemmF32Desc()
+        d.M, d.N, d.K, d.transA, d.transB, d.alpha, d.beta = M, N, K, transA, transB, alpha, beta
+        d.A, d.B, d.C, d.Y = u.ptr(dA), u.ptr(dB), u.ptr(dC), u.ptr(dY)
+        d.bias_mode, d.act, d.batch = mode, act, 1
+        import torch
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_gemm_f32", C.byref(d))
+        self.rt.sync()
+        return u.to_host(dY)
+
+    def unary(self, x, act, alpha):
+        u = self.u
+        dx = u.to_dev(np.ascontiguousarray(x, dtype=np.float32))
+        dy = u.dev_empty(x.shape, np.float32)
+        import torch
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_unary_f32", u.ptr(dy), u.ptr(dx), C.c_size_t(x.size), act, C.c_float(alpha))
+        self.rt.sync()
+        return u.to_host(dy)
+
+    def conv(self, X, W, b, geo):
+        from oracle.binding import conv_out_hw
+        R, u = self.R, self.u
+        N, Cc, H, Wd = X.shape
+        Cout, _, kh, kw = W.shape
+        OH, OW = conv_out_hw(H, Wd, kh, kw, geo["pads"], geo["strides"], geo["dils"])
+        d = R.ConvDesc()
+        (d.N, d.C, d.H, d.W, d.Cout, d.kh, d.kw) = (N, Cc, H, Wd, Cout, kh, kw)
+        (d.pad_h0, d.pad_w0, d.pad_h1, d.pad_w1) = geo["pads"]
+        (d.stride_h, d.stride_w), (d.dil_h, d.dil_w) = geo["strides"], geo["dils"]
+        d.group, d.OH, d.OW = geo["group"], OH, OW
+        dX, dW = u.to_dev(X), u.to_dev(W)
+        db = None if b is None else u.to_dev(b)
+        dY = u.dev_empty((N, Cout, OH, OW), np.float32)
+        import torch
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_conv_f32", C.byref(d), u.ptr(dX), u.ptr(dW), u.ptr(db), 0, C.c_float(0), u.ptr(dY))
+        self.rt.sync()
+        return u.to_host(dY)
+
+    def gap(self, X):
+        u = self.u
+        N, Cc = X.shape[:2]
+        HW = int(np.prod(X.shape[2:]))
+        dX = u.to_dev(X)
+        dY = u.dev_empty((N * Cc,), np.float32)
+        import torch
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_global_avg_pool_f32", u.ptr(dY), u.ptr(dX), N * Cc, HW)
+        self.rt.sync()
+        return u.to_host(dY).reshape((N, Cc) + (1,) * (X.ndim - 2))
+
+    def add(self, A, B):
+        R, u = self.R, self.u
+        ysh = np.broadcast_shapes(A.shape, B.shape)
+        rank = len(ysh)
+        d = R.AddDesc()
+        d.rank = rank
+        for i, v in enumerate(ysh):
+            d.y_shape[i] = v
+        for i, v in enumerate((1,) * (rank - A.ndim) + tuple(A.shape)):
+            d.a_shape[i] = v
+        for i, v in enumerate((1,) * (rank - B.ndim) + tuple(B.shape)):
+            d.b_shape[i] = v
+        dA, dB = u.to_dev(A), u.to_dev(B)
+        dY = u.dev_empty(ysh, np.float32)
+        d.A, d.B, d.Y = u.ptr(dA), u.ptr(dB), u.ptr(dY)
+        import torch
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_add_f32", C.byref(d))
+        self.rt.sync()
+        return u.to_host(dY)
+
+
+def run(g, inputs, be):
+    env = dict(g["initializers"])
+    for (name, _), a in zip(g["inputs"], inputs):
+        env[name] = a
+    for n in fuse(g["nodes"]):
+        op, a = n["op"], n["attrs"]
+        x = [env[i] if i else None for i in n["inputs"]]
+        if op == "Gemm":
+            y = be.gemm(x[0], x[1], x[2] if len(x) > 2 else None, a.get("transA", 0), a.get("transB", 0), a.get("alpha", 1.0),
+                        a.get("beta", 1.0), n.get("fused_act", 0))
+        elif op in ("Relu", "Sigmoid", "Tanh"):
+            y = be.unary(x[0], ACT[op], 0.0)
+        elif op == "LeakyRelu":
+            y = be.unary(x[0], 2, a.get("alpha", 0.01))
+        elif op == "Gelu":
+            y = be.unary(x[0], 5 if a.get("approximate", "none") == "tanh" else 4, 0.0)
+        elif op == "Conv":
+            X, W = x[0], x[1]
+            b = x[2] if len(x) > 2 else None
+            geo = conv_geometry(a, X.shape, W.shape)
+            one_d = X.ndim == 3
+            if one_d:
+                X, W = X[:, :, None, :], W[:, :, None, :]
+            y = be.conv(np.ascontiguousarray(X), np.ascontiguousarray(W), b, geo)
+            if one_d:
+                y = y[:, :, 0, :]
+        elif op == "GlobalAveragePool":
+            y = be.gap(x[0])
+        elif op == "Add":
+            y = be.add(x[0], x[1])
+        else:
+            raise NotImplementedError(op)
+        env[n["outputs"][0]] = y
+    return env[g["outputs"][0][0]]

@@ -1,0 +1,30 @@
+"""Pins the CPU oracle to the reference: every golden output the reference's own tests hold for the
+Gemm / Conv / epilogue path is reproduced within the reference's test tolerance (1e-3 absolute,
+tests/common/test_helpers.h:22; most agree to 1e-6)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from tests import graph_runner as gr
+
+FOUR_DECIMALS = ("Gelu", "GeluTanh", "LinearWithLeakyRelu")  # references printed with 4 decimals
+
+
+def golden_tolerance(model, expected):
+    """Half a unit of the last printed digit of the reference file, plus fp32 rounding of the result."""
+    if model in FOUR_DECIMALS:
+        return 0.6e-4
+    return 2e-5 + 2e-6 * float(np.abs(expected).max())
+
+
+MODELS = sorted(json.load(open(os.path.join(gr.GOLDEN, "fixtures.json"))).keys())
+
+
+@pytest.mark.parametrize("model", MODELS)
+def test_oracle_reproduces_reference_golden_output(model):
+    g, inputs, expected = gr.load_fixture(model)
+    got = gr.run(g, inputs, gr.OracleBackend()).ravel()
+    assert got.shape == expected.shape
+    assert np.abs(got - expected).max() <= golden_tolerance(model, expected), np.abs(got - expected).max()

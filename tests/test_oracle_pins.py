@@ -1,0 +1,290 @@
+"""Pins for the parts of the oracle the golden fixtures do not reach: closed forms, brute force in
+float64 / int64, exhaustive tables, the reference's literal test values, and the reference's own
+memory planner (oracle/_ref) where it is built."""
+import ctypes as C
+import itertools
+
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from tests import util
+
+
+# ---- fp32 Gemm: literals of the reference's constant-folding / MatMul tests --------------------------------
+
+def test_gemm_literals_of_the_reference_tests():
+    # Gemm_ConstantFolding: A=[[1,2,3],[4,5,6]] x B=[[7,8],[9,10],[11,12]] + C=[[1,1],[1,1]] -> {59,65,140,155}
+    # (tests/cpu/TestCustomModelsFromONNX.cxx:509-527)
+    A = np.arange(1, 7, dtype=np.float32).reshape(2, 3)
+    B = np.arange(7, 13, dtype=np.float32).reshape(3, 2)
+    Cb = np.ones((2, 2), dtype=np.float32)
+    y = ob.gemm_f32(A, B, Cb, M=2, N=2, K=3, bias_mode=4)
+    assert y.ravel().tolist() == [59, 65, 140, 155]
+    # ExternalStream model: Gemm+Relu of ones[1,3]... = 3.5 (tests/alpaka/TestAlpakaExternalStream.cxx:34-37):
+    # x = ones(3), W = 1, b = 0.5
+    y = ob.gemm_f32(np.ones((1, 3), np.float32), np.ones((3, 1), np.float32), np.array([0.5], np.float32), M=1, N=1, K=3,
+                    bias_mode=1, act=1)
+    assert y[0, 0] == 3.5
+
+
+@pytest.mark.parametrize("transA,transB,bias_mode,act", list(itertools.product([0, 1], [0, 1], [0, 1, 2, 3, 4], [0, 1, 2])))
+def test_gemm_f32_against_float64_brute_force(transA, transB, bias_mode, act):
+    M, N, K = 7, 5, 11
+    A = util.normal(1, M * K).reshape((K, M) if transA else (M, K))
+    B = util.normal(2, N * K).reshape((N, K) if transB else (K, N))
+    Cshape = {0: None, 1: (N,), 2: (M, 1), 3: (1,), 4: (M, N)}[bias_mode]
+    Cb = None if Cshape is None else util.normal(3, int(np.prod(Cshape))).reshape(Cshape)
+    alpha, beta = 0.75, 2.0
+    got = ob.gemm_f32(A, B, Cb, M=M, N=N, K=K, transA=transA, transB=transB, alpha=alpha, beta=beta, bias_mode=bias_mode,
+                      act=act, act_alpha=0.3)
+    opA = (A.T if transA else A).astype(np.float64)
+    opB = (B.T if transB else B).astype(np.float64)
+    ref = alpha * (opA @ opB)
+    if bias_mode in (1, 2, 3):
+        ref = ref + Cb.astype(np.float64)  # broadcast bias: beta is forced to 1 (ROperator_Gemm.hxx:580)
+    elif bias_mode == 4:
+        ref = ref + beta * Cb.astype(np.float64)
+    if act == 1:
+        ref = np.maximum(ref, 0)
+    elif act == 2:
+        ref = np.where(ref >= 0, ref, 0.3 * ref)
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-5)
+
+
+def test_relu_special_values():
+    x = np.array([np.nan, -0.0, 0.0, -1.0, 2.5, np.inf, -np.inf], dtype=np.float32)
+    y = ob.unary(x, 1)
+    assert y.tolist() == [0.0, 0.0, 0.0, 0.0, 2.5, np.inf, 0.0]
+    assert not np.signbit(y[1])  # -0 -> +0 as on the reference's CPU path
+
+
+def test_activations_closed_forms():
+    import math
+    x = np.linspace(-4, 4, 33, dtype=np.float32)
+    assert np.allclose(ob.unary(x, 3), 1 / (1 + np.exp(-x.astype(np.float64))), atol=1e-6)
+    assert np.allclose(ob.unary(x, 4), [0.5 * v * (1 + math.erf(v / math.sqrt(2))) for v in x.astype(np.float64)], atol=1e-6)
+    assert np.allclose(ob.unary(x, 5), [0.5 * v * (1 + math.tanh(0.7978845608028654 * (v + 0.044715 * v ** 3))) for v in x.astype(np.float64)], atol=1e-6)
+    assert np.allclose(ob.unary(x, 2, 0.1), np.where(x >= 0, x, 0.1 * x))
+    assert np.allclose(ob.unary(x, 6), np.tanh(x.astype(np.float64)), atol=1e-6)
+
+
+# ---- im2col / conv: direct 7-loop convolution in float64 -----------------------------------------------------
+
+def direct_conv(X, W, b, pads, strides, dils, group):
+    N, Cc, H, Wd = X.shape
+    Cout, Cg, kh, kw = W.shape
+    OH, OW = ob.conv_out_hw(H, Wd, kh, kw, pads, strides, dils)
+    Y = np.zeros((N, Cout, OH, OW))
+    for n, co, oh, ow in itertools.product(range(N), range(Cout), range(OH), range(OW)):
+        g = co // (Cout // group)
+        s = 0.0 if b is None else float(b[co])
+        for ci, y, x in itertools.product(range(Cg), range(kh), range(kw)):
+            ih, iw = oh * strides[0] - pads[0] + y * dils[0], ow * strides[1] - pads[1] + x * dils[1]
+            if 0 <= ih < H and 0 <= iw < Wd:
+                s += float(X[n, g * Cg + ci, ih, iw]) * float(W[co, ci, y, x])
+        Y[n, co, oh, ow] = s
+    return Y
+
+
+@pytest.mark.parametrize("case", [
+    (1, 1, 5, 5, 1, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1), (2, 4, 6, 7, 6, 3, 2, (1, 0, 2, 1), (2, 1), (1, 1), 2),
+    (1, 2, 9, 9, 4, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2), 1), (2, 3, 1, 12, 4, 1, 5, (0, 2, 0, 2), (1, 2), (1, 1), 1),
+    (1, 6, 5, 5, 6, 3, 3, (1, 1, 1, 1), (1, 1), (1, 2), 3)])
+def test_conv_f32_equals_direct_convolution(case):
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    X = util.normal(5, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.normal(6, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
+    b = util.normal(7, Cout)
+    for bias in (None, b):
+        got = ob.conv_f32(X, Wt, bias, pads=pads, strides=strides, dils=dils, group=group)
+        assert np.allclose(got, direct_conv(X, Wt, bias, pads, strides, dils, group), rtol=1e-5, atol=1e-5)
+
+
+def test_im2col_layout():
+    # rows (c,kh,kw), columns (oh,ow), zero outside the image
+    x = np.arange(2 * 3 * 3, dtype=np.float32).reshape(2, 3, 3)
+    col = ob.im2col(x, 2, 2, (1, 0, 0, 0), (1, 1), (1, 1))  # pad one row on top
+    assert col.shape == (8, 6)
+    assert col[0].tolist() == [0, 0, 3 * 0 + 0, 1, 3, 4]      # c=0,kh=0,kw=0: first output row reads the padding
+    assert col[3].tolist() == [1, 2, 4, 5, 7, 8]              # c=0,kh=1,kw=1
+    assert col[4].tolist() == [0, 0, 9, 10, 12, 13]           # c=1,kh=0,kw=0
+
+
+# ---- memory planner -----------------------------------------------------------------------------------------
+
+def check_plan(begin, end, size, plan):
+    off, total = plan["offsets"], plan["total_bytes"]
+    for i in range(len(begin)):
+        assert off[i] + size[i] <= total
+        for j in range(i):
+            if begin[i] < end[j] and begin[j] < end[i]:  # live together
+                assert off[i] + size[i] <= off[j] or off[j] + size[j] <= off[i], (i, j)
+
+
+def linear16_lifetimes(row_bytes):
+    # 10 chained Gemm(+Relu) operators, outputs [16,50] x9 then [16,10]; output i is produced by op i and last
+    # read by op i+1 -> lifetime [i, i+2).  The reference plans these into 2 x 3328 = 6656 bytes (256-byte aligned).
+    n = 10
+    begin = list(range(n))
+    end = [i + 2 for i in range(n)]
+    size = [row_bytes] * 9 + [768]
+    return begin, end, size
+
+
+def test_planner_linear16_known_total():
+    begin, end, size = linear16_lifetimes(3328)  # 16*50*4 = 3200 rounded up to 256
+    plan = ob.organize_memory(begin, end, size)
+    check_plan(begin, end, size, plan)
+    assert plan["total_bytes"] == 6656
+
+
+def test_planner_rejects_empty_lifetime():
+    with pytest.raises(ValueError):
+        ob.organize_memory([0, 3], [1, 3], [16, 16])
+
+
+def test_planner_equals_reference_planner():
+    ref = ob.load_ref_planner()
+    if ref is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    rng = np.random.default_rng(7)
+    cases = [linear16_lifetimes(3328)]
+    for _ in range(200):
+        n = int(rng.integers(1, 9))  # <= 16 events: std::sort is an insertion sort there, i.e. equal events keep tensor order
+        begin = [int(v) for v in rng.integers(0, 12, n)]
+        end = [b + int(v) for b, v in zip(begin, rng.integers(1, 6, n))]
+        size = [int(v) * 256 for v in rng.integers(1, 9, n)]
+        cases.append((begin, end, size))
+    for begin, end, size in cases:
+        mine = ob.organize_memory(begin, end, size)
+        theirs = ob.organize_memory(begin, end, size, lib=ref, fn="ref_organize_memory")
+        check_plan(begin, end, size, mine)
+        check_plan(begin, end, size, theirs)
+        if len(begin) <= 8:
+            assert mine == theirs
+    # larger plans: the reference leaves the order of equal events to std::sort, so only the invariants
+    # (no overlap of live tensors, everything inside the pool) are compared
+    for _ in range(50):
+        n = int(rng.integers(9, 40))
+        begin = [int(v) for v in rng.integers(0, 30, n)]
+        end = [b + int(v) for b, v in zip(begin, rng.integers(1, 8, n))]
+        size = [int(v) * 256 for v in rng.integers(1, 9, n)]
+        mine = ob.organize_memory(begin, end, size)
+        theirs = ob.organize_memory(begin, end, size, lib=ref, fn="ref_organize_memory")
+        check_plan(begin, end, size, mine)
+        check_plan(begin, end, size, theirs)
+        lower = max(sum(sz for b, e, sz in zip(begin, end, size) if b <= t < e) for t in range(40))
+        assert mine["total_bytes"] >= lower and theirs["total_bytes"] >= lower
+
+
+# ---- quantised operators (ONNX definitions) ------------------------------------------------------------------
+
+def test_quantize_linear_ties_saturation_nan():
+    s = np.float32(0.5)
+    x = np.array([0.25, 0.75, 1.25, -0.25, -0.75, 63.75, 100.0, -64.25, -100.0, np.nan, np.inf, -np.inf, 0.0], dtype=np.float32)
+    q = ob.quantize_linear(x, s)
+    #            0.5->0  1.5->2  2.5->2  -0.5->0  -1.5->-2  127.5->128->127  sat  -128.5->-128  sat  nan->0  +-inf sat
+    assert q.tolist() == [0, 2, 2, 0, -2, 127, 127, -128, -128, 0, 127, -128, 0]
+    xs = util.normal(3, 10000, 3.0)
+    sc = np.float32(0.0371)
+    want = np.clip(np.rint(xs / sc), -128, 127).astype(np.int8)  # numpy: fp32 divide, round half to even
+    assert np.array_equal(ob.quantize_linear(xs, sc), want)
+    assert np.array_equal(ob.dequantize_linear(want, sc), want.astype(np.float32) * sc)
+
+
+def test_all_int8_products_and_matmul_integer():
+    a = np.arange(-128, 128, dtype=np.int8)
+    A = np.repeat(a, 256).reshape(-1, 1)      # [65536,1]
+    B = np.tile(a, 256).reshape(-1, 1)        # B^T rows
+    # K = 1: acc[m, n] with m == n enumerates all 65536 products
+    acc = ob.matmul_integer(A[:512], B[:512], M=512, N=512, K=1, transB=1)
+    assert np.array_equal(acc, A[:512].astype(np.int32) @ B[:512].astype(np.int32).T)
+    prod = np.array([ob.matmul_integer(A[i:i + 1], B[i:i + 1], M=1, N=1, K=1, transB=1)[0, 0] for i in range(0, 65536, 257)])
+    assert np.array_equal(prod, (A[::257, 0].astype(np.int32) * B[::257, 0].astype(np.int32)))
+    for (M, N, K, tA, tB) in [(5, 7, 3, 0, 0), (9, 4, 33, 1, 0), (6, 6, 64, 0, 1), (3, 8, 17, 1, 1)]:
+        X = util.int8_sym(1, M * K).reshape((K, M) if tA else (M, K))
+        Y = util.int8_sym(2, N * K).reshape((N, K) if tB else (K, N))
+        ref = (X.T if tA else X).astype(np.int64) @ (Y.T if tB else Y).astype(np.int64)
+        assert np.array_equal(ob.matmul_integer(X, Y, M=M, N=N, K=K, transA=tA, transB=tB), ref)
+        assert np.array_equal(ob.matmul_integer(X, Y, M=M, N=N, K=K, transA=tA, transB=tB, omp=True), ref)
+    # identity and one-hot special cases
+    I = np.eye(16, dtype=np.int8)
+    X = util.int8_sym(3, 16 * 16).reshape(16, 16)
+    assert np.array_equal(ob.matmul_integer(X, I, M=16, N=16, K=16), X.astype(np.int32))
+
+
+def test_requant_epilogue_definition():
+    acc = np.array([[1, 3, 5, -1, -3, 255, -257, 1000, -1000, 0]], dtype=np.int32)
+    got = ob.gemm_i8_epilogue(acc, scale_scalar=np.float32(0.5), out=2)
+    assert got.tolist() == [[0, 2, 2, 0, -2, 127, -128, 127, -128, 0]]  # ties to even, saturation
+    got = ob.gemm_i8_epilogue(acc, scale_scalar=np.float32(0.5), out=2, relu_out=1)
+    assert got.tolist() == [[0, 2, 2, 0, 0, 127, 0, 127, 0, 0]]
+    bias = np.arange(10, dtype=np.int32)
+    got = ob.gemm_i8_epilogue(acc, bias=bias, out=0, relu_acc=1)
+    assert got.tolist() == [np.maximum(acc[0] + bias, 0).tolist()]  # bias added in int32 before anything else
+    # int32 -> fp32 is round-to-nearest-even above 2^24
+    big = np.array([[(1 << 24) + 1, (1 << 24) + 3, -(1 << 24) - 1]], dtype=np.int32)
+    got = ob.gemm_i8_epilogue(big, scale_scalar=np.float32(1.0), out=1)
+    assert got.tolist() == [[float(1 << 24), float((1 << 24) + 4), -float(1 << 24)]]
+    # DequantizeLinear followed by QuantizeLinear == the two separate operators
+    acc = util.int32_range(5, 4096, -200000, 200000).reshape(64, 64)
+    s, qs = np.float32(3.1e-4), np.float32(0.27)
+    fused = ob.gemm_i8_epilogue(acc, scale_scalar=s, q_scale=qs, out=3, relu_acc=1)
+    two = ob.quantize_linear(ob.dequantize_linear(np.maximum(acc, 0), s), qs)
+    assert np.array_equal(fused, two)
+
+
+def test_conv_i8_equals_float_conv_of_integers():
+    N, Cc, H, W, Cout, kh, kw = 2, 4, 6, 5, 6, 3, 3
+    X = util.int8_sym(8, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.int8_sym(9, Cout * 2 * kh * kw).reshape(Cout, 2, kh, kw)
+    bias = util.int32_range(10, Cout, -500, 500)
+    got = ob.conv_i8(X, Wt, bias, None, pads=(1, 1, 1, 1), strides=(1, 2), dils=(1, 1), group=2, out=0)
+    ref = direct_conv(X.astype(np.float64), Wt.astype(np.float64), bias.astype(np.float64), (1, 1, 1, 1), (1, 2), (1, 1), 2)
+    assert np.array_equal(got, ref.astype(np.int32))
+
+
+def test_e4m3_codec_exhaustive():
+    codes = np.arange(256, dtype=np.uint8)
+    vals = ob.e4m3_to_f32(codes)
+    # OCP e4m3fn: 0x7f/0xff NaN, max 448, smallest subnormal 2^-9, no infinities
+    assert np.isnan(vals[0x7F]) and np.isnan(vals[0xFF]) and np.isfinite(np.delete(vals, [0x7F, 0xFF])).all()
+    assert vals[0x7E] == 448 and vals[0x01] == 2.0 ** -9 and vals[0x08] == 2.0 ** -6 and vals[0x38] == 1.0 and vals[0xB8] == -1.0
+    for c in range(256):
+        s, e, m = c >> 7, (c >> 3) & 15, c & 7
+        if e == 15 and m == 7:
+            continue
+        want = (m / 8 * 2.0 ** -6) if e == 0 else (1 + m / 8) * 2.0 ** (e - 7)
+        assert vals[c] == (-want if s else want)
+    finite = np.isfinite(vals)
+    assert np.array_equal(ob.quantize_fp8(vals[finite], 1.0), codes[finite])  # every value encodes to itself
+    pos = np.sort(vals[finite & ~np.signbit(vals)])
+    mids = ((pos[:-1].astype(np.float64) + pos[1:].astype(np.float64)) / 2).astype(np.float32)
+    enc = ob.quantize_fp8(mids, 1.0)
+    assert (enc & 1 == 0).all()  # a midpoint goes to the neighbour with the even mantissa
+    lo, hi = ob.quantize_fp8(np.nextafter(mids, np.float32(0)), 1.0), ob.quantize_fp8(np.nextafter(mids, np.float32(1e9)), 1.0)
+    assert np.array_equal(ob.e4m3_to_f32(lo), pos[:-1]) and np.array_equal(ob.e4m3_to_f32(hi), pos[1:])
+    assert ob.quantize_fp8(np.array([448, 464, 465, 1e30, np.inf, -np.inf, np.nan], np.float32), 1.0).tolist() == [0x7E, 0x7E, 0x7E, 0x7E, 0x7E, 0xFE, 0x7F]
+
+
+def test_bf16_rounding():
+    x = np.array([1.0, 1.00390625, 1.01171875, -3.0, 3.3895314e38, np.inf], dtype=np.float32)
+    #             exact  tie->even(1.0)  tie->even(1.015625)
+    got = ob.bf16_bits_to_f32(ob.f32_to_bf16_bits(x))
+    assert got.tolist() == [1.0, 1.0, 1.015625, -3.0, np.inf, np.inf]
+
+
+def test_gemm_fp8_arbiter_is_exact_on_small_integers():
+    # small integers are exact in e4m3 and their dot products are exact in float
+    A = (util.int8_sym(11, 8 * 32).reshape(8, 32) % 5).astype(np.float32)
+    B = (util.int8_sym(12, 6 * 32).reshape(6, 32) % 4).astype(np.float32)
+    got = ob.gemm_fp8(ob.quantize_fp8(A, 1.0), ob.quantize_fp8(B, 1.0), M=8, N=6, K=32, transB=1, scale=1.0, out=1)
+    assert np.array_equal(got, A @ B.T)
+
+
+def test_global_avg_pool_i8():
+    X = util.int8_sym(13, 2 * 3 * 20).reshape(2, 3, 20)
+    got = ob.global_avg_pool_i8(X, np.float32(0.05))
+    want = (X.astype(np.int64).sum(-1).astype(np.float32) * np.float32(0.05)) / np.float32(20)
+    assert np.array_equal(got, want)
