@@ -266,7 +266,13 @@ int sofie_hip_global_avg_pool_f32(sofie_hip_ctx *ctx, float *Y, const float *X, 
 int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y /* [N,C] */, const int8_t *X, int32_t N, int32_t C, int32_t HW,
                                  int32_t x_layout /* SOFIE_LAYOUT_* */, float scale);
 
-/* ---- timing helper used by the benchmark ----------------------------------------------------- */
+/* ---- measurement helpers used by the benchmark ------------------------------------------------ */
+/* Register-only int8 MFMA loop on every CU (no counterpart in the reference): the rate the matrix
+ * cores of this board sustain with no memory traffic, with constant operands (random_operands = 0)
+ * or with operands that toggle every instruction (1: the board clocks down under its power limit).
+ * `scratch` receives one int per lane (CUs * 256 * 4 bytes). */
+int sofie_hip_mfma_i8_probe(sofie_hip_ctx *ctx, void *scratch, size_t scratch_bytes, int32_t iters, int32_t random_operands,
+                            double *ops_per_second);
 /* hipEvent pair on the context's stream (torch's events only see torch's streams). */
 int sofie_hip_timer_start(sofie_hip_ctx *ctx);
 int sofie_hip_timer_stop(sofie_hip_ctx *ctx, float *elapsed_ms); /* records, synchronises, returns ms */

@@ -9,7 +9,7 @@ CSRC = os.path.join(ROOT, "sofie_amd", "csrc")
 LIB_DIR = os.path.join(ROOT, "sofie_amd", "lib")
 LIB = os.path.join(LIB_DIR, "libsofie_hip.so")
 
-HIP_SOURCES = ["runtime.hip", "gemm_i8.hip", "gemm_f32.hip", "gemm_fp8.hip", "conv_i8.hip", "eltwise.hip"]
+HIP_SOURCES = ["runtime.hip", "gemm_i8.hip", "gemm_f32.hip", "gemm_fp8.hip", "conv_i8.hip", "eltwise.hip", "probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

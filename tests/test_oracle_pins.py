@@ -269,7 +269,7 @@ def test_e4m3_codec_exhaustive():
 
 
 def test_bf16_rounding():
-    x = np.array([1.0, 1.00390625, 1.01171875, -3.0, 3.3895314e38, np.inf], dtype=np.float32)
+    x = np.array([1.0, 1.00390625, 1.01171875, -3.0, 3.4e38, np.inf], dtype=np.float32)
     #             exact  tie->even(1.0)  tie->even(1.015625)
     got = ob.bf16_bits_to_f32(ob.f32_to_bf16_bits(x))
     assert got.tolist() == [1.0, 1.0, 1.015625, -3.0, np.inf, np.inf]
