@@ -59,15 +59,13 @@ def build_hip_library(jobs=8):
 
 def build_oracle():
     """Builds the CPU checker (and oracle/_ref when the reference checkout is present)."""
-    _run(["make", "-C", os.path.join(ROOT, "oracle"), "all"])
+    _run(["make", "-B", "-C", os.path.join(ROOT, "oracle"), "all"])
 
 
 def build_all():
     lib = build_hip_library()
     build_oracle()
-    emit_dir = os.path.join(ROOT, "sofie_amd", "emit")
-    if os.path.exists(os.path.join(emit_dir, "Makefile")):
-        _run(["make", "-C", emit_dir, "-j8", "all"])
+    _run(["make", "-C", os.path.join(ROOT, "sofie_amd", "emit"), "-B", "-j8", "all"])
     return lib
 
 

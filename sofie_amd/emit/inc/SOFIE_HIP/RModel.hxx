@@ -1,0 +1,100 @@
+// Model IR and Session generator of the gfx950 backend.  The model-building surface is the reference's
+// (core/inc/SOFIE/RModel.hxx:105-215): AddInputTensorInfo, AddInitializedTensor, AddOperator,
+// AddOutputTensorNameList, then GenerateGPU_HIP + OutputGenerated in place of Generate /
+// GenerateGPU_ALPAKA.  The emitted header keeps `SOFIE_<model>::Session(std::string filename)` and
+// `std::vector<float> infer(float const *...)` (core/src/RModel.cxx:1303-1334, 1529-1613).
+#ifndef SOFIE_HIP_RMODEL
+#define SOFIE_HIP_RMODEL
+
+#include "SOFIE_HIP/MemoryPlanner.hxx"
+#include "SOFIE_HIP/ROperator.hxx"
+
+#include <cstring>
+#include <map>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace SOFIE_HIP {
+
+constexpr std::size_t kPoolAlignBytes = 256; // as the reference's GPU pool (core/src/RModel_ALPAKA.cxx:25)
+
+class RModel {
+public:
+   RModel() = default;
+   explicit RModel(std::string name);
+   RModel(const RModel &) = delete;
+   RModel &operator=(const RModel &) = delete;
+
+   // ---- model building (the reference's names and meaning) ----
+   void AddInputTensorInfo(std::string input_name, ETensorType type, std::vector<std::size_t> shape);
+   void AddInputTensorName(std::string name);
+   void AddInitializedTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, std::shared_ptr<void> data);
+   // copies `data` (length = product of shape)
+   void AddInitializedTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, const void *data);
+   void AddConstantTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, const void *data);
+   void AddIntermediateTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape);
+   void AddOperator(std::unique_ptr<ROperator> op, int order_execution = -1);
+   void AddOutputTensorNameList(std::vector<std::string> output_tensor_names);
+
+   // ---- queries used by the operators ----
+   bool CheckIfTensorAlreadyExist(const std::string &tensor_name) const;
+   bool IsInitializedTensor(const std::string &name) const;
+   bool IsInputTensor(const std::string &name) const;
+   const std::vector<std::size_t> &GetTensorShape(const std::string &name) const;
+   ETensorType GetTensorType(const std::string &name) const;
+   std::shared_ptr<void> GetInitializedTensorData(const std::string &name) const;
+   void UpdateInitializedTensor(const std::string &name, ETensorType type, std::vector<std::size_t> shape, std::shared_ptr<void> data);
+   // a float scalar initializer (scales of the quantised operators); throws if it is not one
+   float GetScalarInitializer(const std::string &name) const;
+   const std::string &GetName() const { return fName; }
+   const std::vector<std::unique_ptr<ROperator>> &Operators() const { return fOperators; }
+
+   // ---- generation ----
+   void GenerateGPU_HIP(std::underlying_type_t<Options> options, int batchSize = -1, bool verbose = false);
+   void GenerateGPU_HIP(Options options = Options::kDefault, int batchSize = -1, bool verbose = false)
+   {
+      GenerateGPU_HIP(static_cast<std::underlying_type_t<Options>>(options), batchSize, verbose);
+   }
+   // writes <filename> (default <model>_GPU_HIP.hxx) and the weight file next to it (<stem>.dat)
+   void OutputGenerated(std::string filename = "");
+   const std::string &GetGeneratedCode() const { return fGC; }
+
+   // ---- memory plan of the last generation (bytes), for tests and tooling ----
+   struct PlannedTensor {
+      std::string name;
+      std::size_t offset, bytes;
+      int begin, end; // lifetime in operator indices, [begin, end); statics have begin = -1
+      bool pooled;
+   };
+   const std::vector<PlannedTensor> &GetMemoryPlan() const { return fPlan; }
+   std::size_t GetArenaBytes() const { return fArenaBytes; }
+   std::size_t GetIntermediateMemoryPoolSize() const { return fPoolBytes; }
+
+private:
+   void Initialize();
+   void FuseGemmActivations();
+   void PlanMemory();
+   void GenerateSessionCode(std::underlying_type_t<Options> options);
+   void WriteWeightFile(const std::string &filename) const;
+
+   std::string fName = "Model";
+   std::vector<std::string> fInputTensorNames;
+   std::vector<std::string> fOutputTensorNames;
+   std::unordered_map<std::string, TensorInfo> fInputTensorInfos;
+   std::map<std::string, InitializedTensor> fInitializedTensors; // ordered: header and weight file agree by construction
+   std::unordered_map<std::string, TensorInfo> fIntermediateTensorInfos;
+   std::vector<std::unique_ptr<ROperator>> fOperators;
+   std::vector<PlannedTensor> fPlan;
+   std::unordered_map<std::string, std::size_t> fOffsets;
+   std::size_t fArenaBytes = 0, fPoolBytes = 0;
+   bool fInitialized = false;
+   std::string fGC;
+   std::string fWeightFileName;
+
+   friend class FusionPlanner;
+};
+
+} // namespace SOFIE_HIP
+#endif

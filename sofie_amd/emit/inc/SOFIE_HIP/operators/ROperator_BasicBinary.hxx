@@ -1,0 +1,69 @@
+// Broadcast Add (core/inc/SOFIE/operators/ROperator_BasicBinary.hxx, the Add instance): one
+// sofie_hip_add_f32 call with the multidirectional broadcast resolved at generation time.
+#ifndef SOFIE_HIP_ROPERATOR_BASICBINARY
+#define SOFIE_HIP_ROPERATOR_BASICBINARY
+
+#include "SOFIE_HIP/operators/ROperator_Gemm.hxx"
+
+namespace SOFIE_HIP {
+
+enum EBasicBinaryOperator { Add };
+
+template <typename T, EBasicBinaryOperator Op>
+class ROperator_BasicBinary final : public ROperator {
+   static_assert(std::is_same<T, float>::value && Op == Add, "only the float Add is on this backend's path");
+
+public:
+   ROperator_BasicBinary(std::string nameA, std::string nameB, std::string nameY)
+      : fNA(UTILITY::Clean_name(nameA)), fNB(UTILITY::Clean_name(nameB)), fNY(UTILITY::Clean_name(nameY))
+   {
+      fInputTensorNames = {fNA, fNB};
+      fOutputTensorNames = {fNY};
+      fKind = OperatorKind::BINARY;
+   }
+   void Initialize(RModel &model) override
+   {
+      if (!model.CheckIfTensorAlreadyExist(fNA) || !model.CheckIfTensorAlreadyExist(fNB))
+         throw std::runtime_error("SOFIE Binary Op Input Tensor " + fNA + " or " + fNB + " is not found in model");
+      fShapeA = model.GetTensorShape(fNA);
+      fShapeB = model.GetTensorShape(fNB);
+      const std::size_t r = std::max(fShapeA.size(), fShapeB.size());
+      if (r > 6)
+         throw std::runtime_error("SOFIE Binary Op: rank above 6 is not supported");
+      fShapeA.insert(fShapeA.begin(), r - fShapeA.size(), 1);
+      fShapeB.insert(fShapeB.begin(), r - fShapeB.size(), 1);
+      fShapeY.resize(r);
+      for (std::size_t i = 0; i < r; ++i) {
+         if (fShapeA[i] != fShapeB[i] && fShapeA[i] != 1 && fShapeB[i] != 1)
+            throw std::runtime_error("SOFIE Binary Op: shapes " + ConvertShapeToString(fShapeA) + " and " + ConvertShapeToString(fShapeB) +
+                                     " cannot be broadcast");
+         fShapeY[i] = std::max(fShapeA[i], fShapeB[i]);
+      }
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShapeY);
+   }
+   std::string Generate_GPU_HIP(std::string opName) override
+   {
+      opName = "op_" + opName;
+      std::stringstream out;
+      auto list = [](const std::vector<std::size_t> &v) {
+         std::string s = "{";
+         for (std::size_t i = 0; i < 6; ++i)
+            s += std::to_string(i < v.size() ? v[i] : 1) + (i < 5 ? ", " : "");
+         return s + "}";
+      };
+      out << "\n" << SP << "//------ Add " << opName << " --> " << ConvertShapeToString(fShapeY) << "\n";
+      out << SP << "{\n";
+      out << SP << "   " << "sofie_add_desc d{" << fShapeY.size() << ", " << list(fShapeY) << ", " << list(fShapeA) << ", " << list(fShapeB)
+          << ", tensor_" << fNA << ", tensor_" << fNB << ", tensor_" << fNY << "};\n";
+      out << SP << "   " << "detail::Check(sofie_hip_add_f32(fCtx, &d), \"" << opName << " Add\");\n";
+      out << SP << "}\n";
+      return out.str();
+   }
+
+private:
+   std::string fNA, fNB, fNY;
+   std::vector<std::size_t> fShapeA, fShapeB, fShapeY;
+};
+
+} // namespace SOFIE_HIP
+#endif

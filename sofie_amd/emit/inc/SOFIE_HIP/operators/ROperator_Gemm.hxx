@@ -1,0 +1,204 @@
+// Gemm / MatMul emitter for the gfx950 backend: the operator of core/inc/SOFIE/operators/ROperator_Gemm.hxx
+// (same constructor arguments, same shape and bias rules), emitting one sofie_hip_gemm_f32 call with the
+// bias broadcast and the activation fused into the kernel's store instead of Copy/Fill + Gemm_Call + Relu.
+#ifndef SOFIE_HIP_ROPERATOR_GEMM
+#define SOFIE_HIP_ROPERATOR_GEMM
+
+#include "SOFIE_HIP/RModel.hxx"
+
+#include <iomanip>
+#include <limits>
+#include <sstream>
+
+namespace SOFIE_HIP {
+
+inline const char *ActivationEnumName(EActivationType a)
+{
+   switch (a) {
+   case EActivationType::RELU: return "SOFIE_ACT_RELU";
+   case EActivationType::LEAKYRELU: return "SOFIE_ACT_LEAKYRELU";
+   case EActivationType::SIGMOID: return "SOFIE_ACT_SIGMOID";
+   case EActivationType::GELU: return "SOFIE_ACT_GELU";
+   case EActivationType::GELU_TANH: return "SOFIE_ACT_GELU_TANH";
+   case EActivationType::TANH: return "SOFIE_ACT_TANH";
+   default: return "SOFIE_ACT_NONE";
+   }
+}
+
+inline std::string FloatLiteral(float v)
+{
+   std::ostringstream s;
+   s << std::setprecision(std::numeric_limits<float>::max_digits10) << v;
+   std::string t = s.str();
+   if (t.find_first_of(".eEn") == std::string::npos)
+      t += ".0";
+   return t + "f";
+}
+
+template <typename T>
+class ROperator_Gemm final : public ROperator {
+   static_assert(std::is_same<T, float>::value, "SOFIE - Unsupported type parsing a Gemm operator");
+
+public:
+   ROperator_Gemm(float alpha, float beta, int64_t transA, int64_t transB, std::string nameA, std::string nameB, std::string nameY,
+                  EActivationType activation = EActivationType::UNDEFINED)
+      : fAttrAlpha(alpha), fAttrBeta(beta), fAttrTransA(transA), fAttrTransB(transB), fNA(UTILITY::Clean_name(nameA)),
+        fNB(UTILITY::Clean_name(nameB)), fNY(UTILITY::Clean_name(nameY)), fActivation(activation)
+   {
+      fInputTensorNames = {fNA, fNB};
+      fOutputTensorNames = {fNY};
+      fKind = OperatorKind::GEMM;
+   }
+   ROperator_Gemm(float alpha, float beta, int64_t transA, int64_t transB, std::string nameA, std::string nameB, std::string nameC,
+                  std::string nameY, EActivationType activation = EActivationType::UNDEFINED)
+      : fAttrAlpha(alpha), fAttrBeta(beta), fAttrTransA(transA), fAttrTransB(transB), fNA(UTILITY::Clean_name(nameA)),
+        fNB(UTILITY::Clean_name(nameB)), fNC(UTILITY::Clean_name(nameC)), fNY(UTILITY::Clean_name(nameY)), fActivation(activation)
+   {
+      fInputTensorNames = {fNA, fNB, fNC};
+      fOutputTensorNames = {fNY};
+      fKind = OperatorKind::GEMM;
+   }
+
+   // used by the activation fusion of the generator (the reference's FuseGemmActivations,
+   // core/src/RModel_Fusion_ALPAKA.cxx:367-416)
+   bool HasActivation() const { return fActivation != EActivationType::UNDEFINED; }
+   void FuseActivation(EActivationType a, float alpha, const std::string &newOutput)
+   {
+      fActivation = a;
+      fActAlpha = alpha;
+      fNY = newOutput;
+      fOutputTensorNames = {fNY};
+   }
+
+   void Initialize(RModel &model) override
+   {
+      if (!model.CheckIfTensorAlreadyExist(fNA) || !model.CheckIfTensorAlreadyExist(fNB))
+         throw std::runtime_error("SOFIE Gemm Op Input Tensor " + fNA + " or " + fNB + " is not found in model");
+      if (!fNC.empty() && !model.CheckIfTensorAlreadyExist(fNC))
+         throw std::runtime_error("SOFIE Gemm Op Input Tensor " + fNC + " is not found in model");
+      if (model.GetTensorType(fNA) != ETensorType::FLOAT || model.GetTensorType(fNB) != ETensorType::FLOAT)
+         throw std::runtime_error("SOFIE Gemm Op: only float tensors; quantised products use ROperator_QGemm");
+      fShapeA = model.GetTensorShape(fNA);
+      fShapeB = model.GetTensorShape(fNB);
+      // MatMul conventions of the reference (ROperator_Gemm.hxx:183-215): a 1-D A gets a leading 1, a 1-D B a
+      // trailing 1, and the shorter shape is padded with leading 1s
+      bool prependOne = false, appendOne = false;
+      if (fShapeA.size() == 1) {
+         fShapeA.insert(fShapeA.begin(), 1);
+         prependOne = true;
+      }
+      if (fShapeB.size() == 1) {
+         fShapeB.push_back(1);
+         appendOne = true;
+      }
+      if (fShapeA.size() < 2 || fShapeB.size() < 2)
+         throw std::runtime_error("SOFIE Gemm Op Shape Inference only accept input tensor with >=2 dimensions");
+      while (fShapeA.size() < fShapeB.size())
+         fShapeA.insert(fShapeA.begin(), 1);
+      while (fShapeB.size() < fShapeA.size())
+         fShapeB.insert(fShapeB.begin(), 1);
+      const std::size_t r = fShapeA.size();
+      fM = fAttrTransA ? fShapeA[r - 1] : fShapeA[r - 2];
+      fK = fAttrTransA ? fShapeA[r - 2] : fShapeA[r - 1];
+      const std::size_t kB = fAttrTransB ? fShapeB[r - 1] : fShapeB[r - 2];
+      fN = fAttrTransB ? fShapeB[r - 2] : fShapeB[r - 1];
+      if (kB != fK)
+         throw std::runtime_error("SOFIE Gemm Op: the inner dimensions of " + fNA + " " + ConvertShapeToString(fShapeA) + " and " + fNB +
+                                  " " + ConvertShapeToString(fShapeB) + " do not agree");
+      // stacked MatMul: leading dims broadcast (1 or equal)
+      std::vector<std::size_t> shapeY;
+      fBatch = 1;
+      fStrideA = fStrideB = 0;
+      std::size_t leadA = 1, leadB = 1;
+      for (std::size_t i = 0; i + 2 < r; ++i) {
+         const std::size_t a = fShapeA[i], b = fShapeB[i];
+         if (a != b && a != 1 && b != 1)
+            throw std::runtime_error("SOFIE Gemm(MatMul) has invalid shape for inputs or output");
+         shapeY.push_back(std::max(a, b));
+         fBatch *= std::max(a, b);
+         leadA *= a;
+         leadB *= b;
+      }
+      if (fBatch > 1) {
+         if ((leadA != 1 && leadA != fBatch) || (leadB != 1 && leadB != fBatch))
+            throw std::runtime_error("SOFIE Gemm(MatMul): mixed broadcasting of the stacked dimensions is not supported");
+         fStrideA = leadA == 1 ? 0 : fM * fK;
+         fStrideB = leadB == 1 ? 0 : fK * fN;
+      }
+      shapeY.push_back(fM);
+      shapeY.push_back(fN);
+
+      // bias: the four broadcast cases of the reference (ROperator_Gemm.hxx:578-617) or a Y-shaped C
+      fBiasMode = "SOFIE_BIAS_NONE";
+      if (!fNC.empty()) {
+         if (model.GetTensorType(fNC) != ETensorType::FLOAT)
+            throw std::runtime_error("SOFIE Gemm Op: bias tensor " + fNC + " is not float");
+         auto shapeC = model.GetTensorShape(fNC);
+         std::vector<std::size_t> c2 = shapeC;
+         while (c2.size() > 2 && c2.front() == 1)
+            c2.erase(c2.begin());
+         if (c2.size() == 1)
+            c2.insert(c2.begin(), 1);
+         if (c2.empty())
+            c2 = {1, 1};
+         // a C with exactly Y's shape goes to the kernel as C with the operator's beta; anything else is a
+         // broadcast, for which the reference forces beta = 1 (ROperator_Gemm.hxx:580)
+         if (shapeC == shapeY)
+            fBiasMode = "SOFIE_BIAS_FULL";
+         else if (c2.size() == 2 && c2[0] == 1 && c2[1] == fN)
+            fBiasMode = "SOFIE_BIAS_ROW";
+         else if (c2.size() == 2 && c2[1] == 1 && c2[0] == fM)
+            fBiasMode = "SOFIE_BIAS_COL";
+         else if (c2.size() == 2 && c2[0] == 1 && c2[1] == 1)
+            fBiasMode = "SOFIE_BIAS_SCALAR";
+         else
+            throw std::runtime_error("SOFIE Gemm Op - bias tensor of shape " + ConvertShapeToString(shapeC) +
+                                     " cannot be uni-directional broadcasted to " + ConvertShapeToString(shapeY));
+         if (fBiasMode == std::string("SOFIE_BIAS_FULL") && fBatch > 1)
+            fStrideC = fM * fN;
+      } else if (fAttrBeta != 0) {
+         fAttrBeta = 0; // no bias: beta is forced to zero as in the reference (ROperator_Gemm.hxx:491-499)
+      }
+      if (prependOne)
+         shapeY.erase(shapeY.end() - 2);
+      if (appendOne)
+         shapeY.pop_back();
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, shapeY);
+   }
+
+   std::string Generate_GPU_HIP(std::string opName) override
+   {
+      opName = "op_" + opName;
+      if (fM == 0)
+         throw std::runtime_error("SOFIE Gemm Op called to Generate without being initialized first");
+      std::stringstream out;
+      out << "\n" << SP << "//--------- Gemm " << opName << " " << ConvertShapeToString(fShapeA) << " * " << ConvertShapeToString(fShapeB)
+          << " -> " << fNY << "\n";
+      out << SP << "{\n";
+      out << SP << "   " << "sofie_gemm_f32_desc d{};\n";
+      out << SP << "   " << "d.M = " << fM << "; d.N = " << fN << "; d.K = " << fK << "; d.transA = " << (fAttrTransA ? 1 : 0)
+          << "; d.transB = " << (fAttrTransB ? 1 : 0) << ";\n";
+      out << SP << "   " << "d.alpha = " << FloatLiteral(fAttrAlpha) << "; d.beta = " << FloatLiteral(fAttrBeta) << ";\n";
+      out << SP << "   " << "d.A = tensor_" << fNA << "; d.B = tensor_" << fNB << "; d.C = " << (fNC.empty() ? "nullptr" : "tensor_" + fNC)
+          << "; d.bias_mode = " << fBiasMode << ";\n";
+      out << SP << "   " << "d.act = " << ActivationEnumName(fActivation) << "; d.act_alpha = " << FloatLiteral(fActAlpha) << ";\n";
+      out << SP << "   " << "d.Y = tensor_" << fNY << "; d.batch = " << fBatch << "; d.strideA = " << fStrideA << "; d.strideB = " << fStrideB
+          << "; d.strideC = " << fStrideC << "; d.strideY = " << (fBatch > 1 ? fM * fN : 0) << ";\n";
+      out << SP << "   " << "detail::Check(sofie_hip_gemm_f32(fCtx, &d), \"" << opName << " Gemm\");\n";
+      out << SP << "}\n";
+      return out.str();
+   }
+
+private:
+   float fAttrAlpha = 1.0, fAttrBeta = 1.0;
+   int64_t fAttrTransA = 0, fAttrTransB = 0;
+   std::string fNA, fNB, fNC, fNY;
+   EActivationType fActivation = EActivationType::UNDEFINED;
+   float fActAlpha = 0.01f;
+   std::vector<std::size_t> fShapeA, fShapeB;
+   std::size_t fM = 0, fN = 0, fK = 0, fBatch = 1, fStrideA = 0, fStrideB = 0, fStrideC = 0;
+   std::string fBiasMode;
+};
+
+} // namespace SOFIE_HIP
+#endif

@@ -1,0 +1,573 @@
+// Model IR, fusion, memory plan and Session text of the gfx950 backend.
+#include "SOFIE_HIP/RModel.hxx"
+#include "SOFIE_HIP/operators/OperatorList.hxx"
+
+#include <cmath>
+#include <fstream>
+#include <iomanip>
+#include <iostream>
+#include <limits>
+#include <set>
+#include <sstream>
+
+namespace SOFIE_HIP {
+
+static std::size_t AlignUp(std::size_t v) { return (v + kPoolAlignBytes - 1) / kPoolAlignBytes * kPoolAlignBytes; }
+
+RModel::RModel(std::string name)
+{
+   // the model name is the file name without directory and extension, as the reference derives it
+   auto slash = name.find_last_of("/\\");
+   if (slash != std::string::npos)
+      name = name.substr(slash + 1);
+   auto dot = name.find_last_of('.');
+   if (dot != std::string::npos)
+      name = name.substr(0, dot);
+   fName = UTILITY::Clean_name(name);
+}
+
+void RModel::AddInputTensorInfo(std::string input_name, ETensorType type, std::vector<std::size_t> shape)
+{
+   input_name = UTILITY::Clean_name(input_name);
+   if (CheckIfTensorAlreadyExist(input_name))
+      throw std::runtime_error("SOFIE: input tensor with name " + input_name + " already exists \n");
+   fInputTensorInfos[input_name] = TensorInfo{type, shape};
+}
+
+void RModel::AddInputTensorName(std::string name) { fInputTensorNames.push_back(UTILITY::Clean_name(name)); }
+
+void RModel::AddInitializedTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, std::shared_ptr<void> data)
+{
+   tensor_name = UTILITY::Clean_name(tensor_name);
+   if (CheckIfTensorAlreadyExist(tensor_name))
+      throw std::runtime_error("SOFIE: initialized tensor with name " + tensor_name + " already exists \n");
+   if (GetTypeSize(type) == 0)
+      throw std::runtime_error("SOFIE: initialized tensor " + tensor_name + " has a type this backend cannot store");
+   fInitializedTensors[tensor_name] = InitializedTensor{type, shape, data, false};
+}
+
+void RModel::AddInitializedTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, const void *data)
+{
+   const std::size_t bytes = ConvertShapeToLength(shape) * GetTypeSize(type);
+   std::shared_ptr<void> copy(malloc(bytes ? bytes : 1), free);
+   if (bytes)
+      std::memcpy(copy.get(), data, bytes);
+   AddInitializedTensor(tensor_name, type, shape, copy);
+}
+
+void RModel::AddConstantTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, const void *data)
+{
+   AddInitializedTensor(tensor_name, type, shape, data);
+   fInitializedTensors[UTILITY::Clean_name(tensor_name)].constant = true;
+}
+
+void RModel::AddIntermediateTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape)
+{
+   tensor_name = UTILITY::Clean_name(tensor_name);
+   if (CheckIfTensorAlreadyExist(tensor_name))
+      throw std::runtime_error("SOFIE: intermediate tensor with name " + tensor_name + " already exists \n");
+   fIntermediateTensorInfos[tensor_name] = TensorInfo{type, shape};
+}
+
+void RModel::AddOperator(std::unique_ptr<ROperator> op, int order_execution)
+{
+   if (order_execution >= 0 && (std::size_t)order_execution <= fOperators.size())
+      fOperators.insert(fOperators.begin() + order_execution, std::move(op));
+   else
+      fOperators.push_back(std::move(op));
+}
+
+void RModel::AddOutputTensorNameList(std::vector<std::string> names)
+{
+   fOutputTensorNames.clear();
+   for (auto &n : names)
+      fOutputTensorNames.push_back(UTILITY::Clean_name(n));
+}
+
+bool RModel::CheckIfTensorAlreadyExist(const std::string &n) const
+{
+   return fInputTensorInfos.count(n) || fInitializedTensors.count(n) || fIntermediateTensorInfos.count(n);
+}
+bool RModel::IsInitializedTensor(const std::string &n) const { return fInitializedTensors.count(UTILITY::Clean_name(n)) != 0; }
+bool RModel::IsInputTensor(const std::string &n) const { return fInputTensorInfos.count(UTILITY::Clean_name(n)) != 0; }
+
+const std::vector<std::size_t> &RModel::GetTensorShape(const std::string &name) const
+{
+   auto a = fInputTensorInfos.find(name);
+   if (a != fInputTensorInfos.end())
+      return a->second.shape;
+   auto b = fInitializedTensors.find(name);
+   if (b != fInitializedTensors.end())
+      return b->second.shape;
+   auto c = fIntermediateTensorInfos.find(name);
+   if (c != fIntermediateTensorInfos.end())
+      return c->second.shape;
+   throw std::runtime_error("SOFIE tensor [" + name + "] for which the shape is requested is not found");
+}
+
+ETensorType RModel::GetTensorType(const std::string &name) const
+{
+   auto a = fInputTensorInfos.find(name);
+   if (a != fInputTensorInfos.end())
+      return a->second.type;
+   auto b = fInitializedTensors.find(name);
+   if (b != fInitializedTensors.end())
+      return b->second.type;
+   auto c = fIntermediateTensorInfos.find(name);
+   if (c != fIntermediateTensorInfos.end())
+      return c->second.type;
+   throw std::runtime_error("SOFIE tensor [" + name + "] for which the type is requested is not found");
+}
+
+std::shared_ptr<void> RModel::GetInitializedTensorData(const std::string &name) const
+{
+   auto f = fInitializedTensors.find(name);
+   if (f == fInitializedTensors.end())
+      throw std::runtime_error("SOFIE tensor [" + name + "] for which the data is requested is not found");
+   return f->second.data;
+}
+
+void RModel::UpdateInitializedTensor(const std::string &name, ETensorType type, std::vector<std::size_t> shape, std::shared_ptr<void> data)
+{
+   auto f = fInitializedTensors.find(name);
+   if (f == fInitializedTensors.end())
+      throw std::runtime_error("SOFIE tensor [" + name + "] for which update is requested is not found");
+   f->second = InitializedTensor{type, shape, data, f->second.constant};
+}
+
+float RModel::GetScalarInitializer(const std::string &name) const
+{
+   auto f = fInitializedTensors.find(UTILITY::Clean_name(name));
+   if (f == fInitializedTensors.end() || f->second.type != ETensorType::FLOAT || ConvertShapeToLength(f->second.shape) != 1)
+      throw std::runtime_error("SOFIE: " + name + " must be a float scalar initializer (per-tensor scale)");
+   return *static_cast<const float *>(f->second.data.get());
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Fusion.  (1) the reference's FuseGemmActivations (core/src/RModel_Fusion_ALPAKA.cxx:367-416): an
+// activation that is the only consumer of a Gemm / Conv output, which is not a graph output, moves into
+// that operator's store.  Unlike the reference's cuBLASLt epilogue it does not need a bias to be present.
+// (2) the quantised chain MatMulInteger -> Relu -> DequantizeLinear -> QuantizeLinear folds, link by link
+// under the same single-consumer rule, into the store of the int8 product.
+// ---------------------------------------------------------------------------------------------------------
+void RModel::FuseGemmActivations()
+{
+   auto consumers = [&](const std::string &t) {
+      std::vector<std::size_t> c;
+      for (std::size_t i = 0; i < fOperators.size(); ++i)
+         for (auto &in : fOperators[i]->GetInputTensorNames())
+            if (in == t)
+               c.push_back(i);
+      return c;
+   };
+   auto isOutput = [&](const std::string &t) { return std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), t) != fOutputTensorNames.end(); };
+   bool changed = true;
+   while (changed) {
+      changed = false;
+      for (std::size_t i = 0; i < fOperators.size() && !changed; ++i) {
+         ROperator *op = fOperators[i].get();
+         if (op->GetOutputTensorNames().size() != 1)
+            continue;
+         const std::string y = op->GetOutputTensorNames()[0];
+         if (isOutput(y))
+            continue;
+         auto cons = consumers(y);
+         if (cons.size() != 1)
+            continue;
+         ROperator *next = fOperators[cons[0]].get();
+         auto *act = dynamic_cast<ROperator_Activation *>(next);
+         if (auto *g = dynamic_cast<ROperator_Gemm<float> *>(op)) {
+            if (act && !g->HasActivation()) {
+               g->FuseActivation(act->Activation(), act->Alpha(), act->OutputName());
+               changed = true;
+            }
+         } else if (auto *c = dynamic_cast<ROperator_Conv<float> *>(op)) {
+            if (act && !c->HasActivation()) {
+               c->FuseActivation(act->Activation(), act->Alpha(), act->OutputName());
+               changed = true;
+            }
+         } else if (auto *q = dynamic_cast<ROperator_QGemm *>(op)) {
+            if (q->OutputKind() == ROperator_QGemm::Out::I32 && act && act->Activation() == EActivationType::RELU && !q->ReluOnAccumulator()) {
+               q->SetReluOnAccumulator();
+               q->SetOutputName(act->OutputName());
+               changed = true;
+            } else if (auto *dq = dynamic_cast<ROperator_DequantizeLinear *>(next)) {
+               if (q->OutputKind() == ROperator_QGemm::Out::I32) {
+                  q->SetDequantize(GetScalarInitializer(dq->ScaleName()));
+                  q->SetOutputName(dq->OutputName());
+                  changed = true;
+               }
+            } else if (auto *ql = dynamic_cast<ROperator_QuantizeLinear *>(next)) {
+               if (q->OutputKind() == ROperator_QGemm::Out::F32) {
+                  q->SetDequantizeQuantize(q->DequantScale(), GetScalarInitializer(ql->ScaleName()));
+                  q->SetOutputName(ql->OutputName());
+                  changed = true;
+               }
+            }
+         }
+         if (changed)
+            fOperators.erase(fOperators.begin() + cons[0]);
+      }
+   }
+}
+
+void RModel::Initialize()
+{
+   if (fInitialized)
+      return;
+   for (auto &n : fInputTensorNames)
+      if (!fInputTensorInfos.count(n))
+         throw std::runtime_error("SOFIE: input tensor " + n + " has no tensor info");
+   if (fInputTensorNames.empty())
+      for (auto &kv : fInputTensorInfos)
+         fInputTensorNames.push_back(kv.first);
+   FuseGemmActivations();
+   for (std::size_t i = 0; i < fOperators.size(); ++i) {
+      fOperators[i]->SetOpOrder(i);
+      fOperators[i]->Initialize(*this);
+   }
+   for (auto &o : fOutputTensorNames)
+      if (!CheckIfTensorAlreadyExist(o))
+         throw std::runtime_error("SOFIE: output tensor " + o + " is not produced by any operator");
+   fInitialized = true;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Memory plan: ONE arena.  Static regions first (weights, operator-owned buffers such as re-laid-out
+// weights, graph inputs, graph outputs), each 256-byte aligned; then the pool of intermediates and operator
+// workspaces, placed by OrganizeMemory from their lifetimes [producer, last consumer + 1), as the reference's
+// GPU generator does (core/src/RModel_ALPAKA.cxx:360-540).
+// ---------------------------------------------------------------------------------------------------------
+void RModel::PlanMemory()
+{
+   fPlan.clear();
+   fOffsets.clear();
+   std::size_t off = 0;
+   auto addStatic = [&](const std::string &name, std::size_t bytes) {
+      fPlan.push_back({name, off, bytes, -1, (int)fOperators.size() + 1, false});
+      fOffsets[name] = off;
+      off += AlignUp(bytes ? bytes : 1);
+   };
+   for (auto &kv : fInitializedTensors)
+      addStatic("tensor_" + kv.first, ConvertShapeToLength(kv.second.shape) * GetTypeSize(kv.second.type));
+   for (auto &op : fOperators)
+      for (auto &pb : op->GetPersistentBuffers())
+         addStatic(pb.first, pb.second);
+   for (auto &n : fInputTensorNames)
+      addStatic("tensor_" + n, ConvertShapeToLength(fInputTensorInfos[n].shape) * GetTypeSize(fInputTensorInfos[n].type));
+   for (auto &n : fOutputTensorNames)
+      if (fIntermediateTensorInfos.count(n))
+         addStatic("tensor_" + n, ConvertShapeToLength(fIntermediateTensorInfos[n].shape) * GetTypeSize(fIntermediateTensorInfos[n].type));
+   const std::size_t poolBase = off;
+
+   std::vector<TensorLifeInfo> life;
+   std::vector<std::string> names;
+   for (std::size_t i = 0; i < fOperators.size(); ++i) {
+      for (auto &y : fOperators[i]->GetOutputTensorNames()) {
+         if (!fIntermediateTensorInfos.count(y) || fOffsets.count("tensor_" + y))
+            continue; // graph outputs are static
+         int last = (int)i;
+         for (std::size_t j = i + 1; j < fOperators.size(); ++j)
+            for (auto &in : fOperators[j]->GetInputTensorNames())
+               if (in == y)
+                  last = (int)j;
+         const auto &ti = fIntermediateTensorInfos[y];
+         life.push_back({(int)i, last + 1, AlignUp(ConvertShapeToLength(ti.shape) * GetTypeSize(ti.type))});
+         names.push_back("tensor_" + y);
+      }
+      if (std::size_t ws = fOperators[i]->GetWorkspaceBytes()) {
+         life.push_back({(int)i, (int)i + 1, AlignUp(ws)});
+         names.push_back("workspace_op_" + std::to_string(i));
+      }
+   }
+   MemoryResult r = OrganizeMemory(life);
+   for (std::size_t t = 0; t < life.size(); ++t) {
+      fPlan.push_back({names[t], poolBase + r.offsets[t], life[t].size, life[t].begin, life[t].end, true});
+      fOffsets[names[t]] = poolBase + r.offsets[t];
+   }
+   fPoolBytes = r.total_bytes;
+   fArenaBytes = poolBase + r.total_bytes;
+   if (fArenaBytes == 0)
+      fArenaBytes = kPoolAlignBytes;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Session text
+// ---------------------------------------------------------------------------------------------------------
+static const char *kRuntimeHelpers = R"SOFIE(
+namespace detail {
+inline void Check(int status, const char *what)
+{
+   if (status != 0)
+      throw std::runtime_error(std::string("SOFIE HIP runtime error in ") + what + ": " + sofie_hip_last_error());
+}
+// Reads one tensor of the text weight file: a header line `tensor_<name> <length>` and the values
+// (the format of the reference's weight files, core/src/RModel.cxx:1929-1958).
+template <class T>
+inline void ReadTensorFromStream(std::istream &is, std::vector<T> &target, std::string const &expected_name, const std::size_t expected_length)
+{
+   std::string name;
+   std::size_t length;
+   is >> name >> length;
+   if (name != expected_name) {
+      std::string err_msg = "SOFIE failed to read the correct tensor name; expected name is " + expected_name + " , read " + name;
+      throw std::runtime_error(err_msg);
+   }
+   if (length != expected_length) {
+      std::string err_msg = "SOFIE failed to read the correct tensor size; expected size is " + std::to_string(expected_length) + " , read " + std::to_string(length);
+      throw std::runtime_error(err_msg);
+   }
+   target.resize(length);
+   for (std::size_t i = 0; i < length; ++i) {
+      if (sizeof(T) == 1) {
+         int v;
+         is >> v;
+         target[i] = static_cast<T>(v);
+      } else {
+         std::string tok;
+         is >> tok;
+         if (std::is_floating_point<T>::value)
+            target[i] = static_cast<T>(std::strtod(tok.c_str(), nullptr));
+         else
+            target[i] = static_cast<T>(std::strtoll(tok.c_str(), nullptr, 10));
+      }
+   }
+   if (is.fail())
+      throw std::runtime_error("SOFIE failed to read the values for tensor " + expected_name);
+}
+} // namespace detail
+)SOFIE";
+
+void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
+{
+   const bool externalStream = options & static_cast<std::underlying_type_t<Options>>(Options::kExternalStream);
+   const bool noWeightFile = options & static_cast<std::underlying_type_t<Options>>(Options::kNoWeightFile);
+   std::stringstream gc;
+   std::string guard = "SOFIE_" + fName;
+   std::transform(guard.begin(), guard.end(), guard.begin(), [](unsigned char c) { return std::toupper(c); });
+   gc << "//Code generated automatically by SOFIE (gfx950 HIP backend)\n";
+   gc << "#ifndef " << guard << "_GPU_HIP\n#define " << guard << "_GPU_HIP\n\n";
+   gc << "#include <array>\n#include <cstddef>\n#include <cstdint>\n#include <cstdlib>\n#include <fstream>\n#include <stdexcept>\n#include <string>\n"
+         "#include <tuple>\n#include <type_traits>\n#include <vector>\n#include \"sofie_hip.h\"\n\n";
+   gc << "namespace SOFIE_" << fName << " {\n" << kRuntimeHelpers << "\n";
+   gc << "struct Session {\n";
+   gc << "   // one arena: weights, operator-owned buffers, inputs, outputs, then the pool of intermediates\n";
+   gc << "   static constexpr std::size_t kArenaBytes = " << fArenaBytes << ";\n";
+   gc << "   static constexpr std::size_t kIntermediatePoolBytes = " << fPoolBytes << ";\n";
+   gc << "   sofie_hip_ctx *fCtx = nullptr;\n";
+   auto typeOf = [&](const std::string &planName) -> std::string {
+      if (planName.rfind("tensor_", 0) == 0)
+         return ConvertTypeToString(GetTensorType(planName.substr(7)));
+      return "int8_t";
+   };
+   for (auto &p : fPlan)
+      gc << "   " << typeOf(p.name) << " *" << p.name << " = nullptr; // arena offset " << p.offset << ", " << p.bytes << " bytes"
+         << (p.pooled ? ", live [" + std::to_string(p.begin) + "," + std::to_string(p.end) + ")" : "") << "\n";
+   gc << "\n";
+   // constructor
+   gc << "   Session(std::string filename = \"" << (noWeightFile ? "" : fName + "_GPU_HIP.dat") << "\"" << (externalStream ? ", void *stream = nullptr" : "")
+      << ", int device = 0)\n   {\n";
+   gc << "      detail::Check(sofie_hip_ctx_create(&fCtx, device, " << (externalStream ? "stream" : "nullptr") << "), \"Session\");\n";
+   gc << "      try {\n";
+   gc << "         detail::Check(sofie_hip_arena_create(fCtx, kArenaBytes, " << kPoolAlignBytes << "), \"arena allocation\");\n";
+   gc << "         char *base = static_cast<char *>(sofie_hip_arena_ptr(fCtx, 0));\n";
+   gc << "         if (!base)\n            throw std::runtime_error(\"SOFIE HIP runtime error: arena is null\");\n";
+   for (auto &p : fPlan)
+      gc << "         " << p.name << " = reinterpret_cast<" << typeOf(p.name) << " *>(base + " << p.offset << ");\n";
+   bool anyWeights = false, anyConstants = false;
+   for (auto &kv : fInitializedTensors)
+      (kv.second.constant ? anyConstants : anyWeights) = true;
+   if (anyWeights && !noWeightFile) {
+      gc << "         // read and upload the weights\n";
+      gc << "         std::ifstream f;\n         f.open(filename);\n";
+      gc << "         if (!f.is_open()) {\n            throw std::runtime_error(\"tmva-sofie failed to open file \" + filename + \" for input weights\");\n         }\n";
+      for (auto &kv : fInitializedTensors) {
+         if (kv.second.constant)
+            continue;
+         const std::size_t len = ConvertShapeToLength(kv.second.shape);
+         gc << "         {\n            std::vector<" << ConvertTypeToString(kv.second.type) << "> host;\n";
+         gc << "            detail::ReadTensorFromStream(f, host, \"tensor_" << kv.first << "\", " << len << ");\n";
+         gc << "            detail::Check(sofie_hip_upload(fCtx, tensor_" << kv.first << ", host.data(), " << len * GetTypeSize(kv.second.type)
+            << "), \"upload of tensor_" << kv.first << "\");\n";
+         gc << "            detail::Check(sofie_hip_sync(fCtx), \"upload of tensor_" << kv.first << "\");\n         }\n";
+      }
+      gc << "         f.close();\n";
+   }
+   if (anyConstants || noWeightFile) {
+      for (auto &kv : fInitializedTensors) {
+         if (!kv.second.constant && !noWeightFile)
+            continue;
+         const std::size_t len = ConvertShapeToLength(kv.second.shape);
+         gc << "         {\n            static const " << ConvertTypeToString(kv.second.type) << " host[" << (len ? len : 1) << "] = {";
+         for (std::size_t i = 0; i < len; ++i) {
+            if (kv.second.type == ETensorType::FLOAT)
+               gc << FloatLiteral(static_cast<const float *>(kv.second.data.get())[i]);
+            else if (kv.second.type == ETensorType::INT8)
+               gc << (int)static_cast<const int8_t *>(kv.second.data.get())[i];
+            else if (kv.second.type == ETensorType::INT32)
+               gc << static_cast<const int32_t *>(kv.second.data.get())[i];
+            else if (kv.second.type == ETensorType::INT64)
+               gc << static_cast<const int64_t *>(kv.second.data.get())[i];
+            else
+               gc << (unsigned)static_cast<const uint8_t *>(kv.second.data.get())[i];
+            gc << (i + 1 < len ? ", " : "");
+         }
+         gc << "};\n";
+         gc << "            detail::Check(sofie_hip_upload(fCtx, tensor_" << kv.first << ", host, " << len * GetTypeSize(kv.second.type)
+            << "), \"upload of tensor_" << kv.first << "\");\n";
+         gc << "            detail::Check(sofie_hip_sync(fCtx), \"upload of tensor_" << kv.first << "\");\n         }\n";
+      }
+   }
+   std::string init;
+   for (auto &op : fOperators)
+      init += op->GenerateInitCode_GPU_HIP();
+   if (!init.empty())
+      gc << "         // one-time operator set-up (weight re-layouts)\n" << init;
+   gc << "         detail::Check(sofie_hip_sync(fCtx), \"Session\");\n";
+   gc << "      } catch (...) {\n         sofie_hip_ctx_destroy(fCtx);\n         fCtx = nullptr;\n         throw;\n      }\n   }\n";
+   gc << "   ~Session() { sofie_hip_ctx_destroy(fCtx); }\n";
+   gc << "   Session(const Session &) = delete;\n   Session &operator=(const Session &) = delete;\n\n";
+   gc << "   std::size_t GetIntermediateMemoryPoolSize() const { return kIntermediatePoolBytes; }\n";
+   gc << "   void *stream() const { return sofie_hip_stream(fCtx); }\n\n";
+
+   // infer_nosync: the operators, inputs and outputs resident in the arena
+   gc << "   // enqueues one inference on the session's stream: inputs are read from the tensor_<input> regions of the arena,\n";
+   gc << "   // results land in the tensor_<output> regions (overwritten by the next call)\n";
+   gc << "   void infer_nosync()\n   {";
+   for (std::size_t i = 0; i < fOperators.size(); ++i)
+      gc << fOperators[i]->Generate_GPU_HIP(std::to_string(i));
+   gc << "   }\n\n";
+
+   // infer with host pointers: the CPU signature of the reference
+   std::string args;
+   for (std::size_t i = 0; i < fInputTensorNames.size(); ++i) {
+      const auto &ti = fInputTensorInfos[fInputTensorNames[i]];
+      args += ConvertTypeToString(ti.type) + " const* host_" + fInputTensorNames[i] + (i + 1 < fInputTensorNames.size() ? ", " : "");
+   }
+   bool sameType = true;
+   for (auto &o : fOutputTensorNames)
+      sameType = sameType && GetTensorType(o) == GetTensorType(fOutputTensorNames[0]);
+   std::string retType;
+   const std::string t0 = ConvertTypeToString(GetTensorType(fOutputTensorNames.at(0)));
+   if (fOutputTensorNames.size() == 1)
+      retType = "std::vector<" + t0 + ">";
+   else if (sameType)
+      retType = "std::vector<std::vector<" + t0 + ">>";
+   else {
+      retType = "std::tuple<";
+      for (std::size_t i = 0; i < fOutputTensorNames.size(); ++i)
+         retType += "std::vector<" + ConvertTypeToString(GetTensorType(fOutputTensorNames[i])) + ">" + (i + 1 < fOutputTensorNames.size() ? ", " : "");
+      retType += ">";
+   }
+   gc << "   " << retType << " infer(" << args << ")\n   {\n";
+   for (auto &n : fInputTensorNames) {
+      const auto &ti = fInputTensorInfos[n];
+      gc << "      detail::Check(sofie_hip_upload(fCtx, tensor_" << n << ", host_" << n << ", " << ConvertShapeToLength(ti.shape) * GetTypeSize(ti.type)
+         << "), \"upload of input " << n << "\");\n";
+   }
+   gc << "      infer_nosync();\n";
+   for (std::size_t i = 0; i < fOutputTensorNames.size(); ++i) {
+      const auto &o = fOutputTensorNames[i];
+      const std::size_t len = ConvertShapeToLength(GetTensorShape(o));
+      gc << "      std::vector<" << ConvertTypeToString(GetTensorType(o)) << "> out_" << i << "(" << len << ");\n";
+      gc << "      detail::Check(sofie_hip_download(fCtx, out_" << i << ".data(), tensor_" << o << ", " << len * GetTypeSize(GetTensorType(o))
+         << "), \"download of output " << o << "\");\n";
+   }
+   gc << "      detail::Check(sofie_hip_sync(fCtx), \"infer\");\n";
+   if (fOutputTensorNames.size() == 1)
+      gc << "      return out_0;\n";
+   else {
+      gc << "      return " << (sameType ? retType : std::string("std::make_tuple")) << (sameType ? "{" : "(");
+      for (std::size_t i = 0; i < fOutputTensorNames.size(); ++i)
+         gc << "std::move(out_" << i << ")" << (i + 1 < fOutputTensorNames.size() ? ", " : "");
+      gc << (sameType ? "};\n" : ");\n");
+   }
+   gc << "   }\n";
+   gc << "}; // end of Session\n\n";
+   auto dimsArray = [&](const std::string &what, const std::vector<std::string> &names) {
+      gc << "// " << what << " tensor shapes\n";
+      for (auto &n : names) {
+         const auto &s = GetTensorShape(n);
+         gc << "constexpr std::array<std::size_t, " << s.size() << "> dim_" << n << "{";
+         for (std::size_t i = 0; i < s.size(); ++i)
+            gc << s[i] << (i + 1 < s.size() ? ", " : "");
+         gc << "};\n";
+      }
+   };
+   dimsArray("input", fInputTensorNames);
+   dimsArray("output", fOutputTensorNames);
+   gc << "} //SOFIE_" << fName << "\n\n#endif  // " << guard << "_GPU_HIP\n";
+   fGC = gc.str();
+}
+
+void RModel::GenerateGPU_HIP(std::underlying_type_t<Options> options, int batchSize, bool verbose)
+{
+   (void)batchSize; // shapes are static in this backend; a model is built for its batch size
+   if (fOutputTensorNames.empty())
+      throw std::runtime_error("SOFIE: the model has no output tensor");
+   Initialize();
+   PlanMemory();
+   GenerateSessionCode(options);
+   if (verbose)
+      std::cout << "SOFIE HIP: " << fOperators.size() << " operators, arena " << fArenaBytes << " bytes, pool " << fPoolBytes << " bytes\n";
+}
+
+void RModel::WriteWeightFile(const std::string &filename) const
+{
+   std::ofstream f(filename);
+   if (!f.is_open())
+      throw std::runtime_error("tmva-sofie failed to open file " + filename + " for tensor weight data");
+   for (auto &kv : fInitializedTensors) {
+      if (kv.second.constant)
+         continue;
+      const std::size_t len = ConvertShapeToLength(kv.second.shape);
+      f << "tensor_" << kv.first << " " << len << "\n";
+      for (std::size_t i = 0; i < len; ++i) {
+         switch (kv.second.type) {
+         case ETensorType::FLOAT: {
+            float v = static_cast<const float *>(kv.second.data.get())[i];
+            if (v != 0. && std::abs(v) < std::numeric_limits<float>::min())
+               v = 0; // sub-normal values are rounded to zero, as the reference's writer does
+            if (std::isinf(v))
+               f << (v > 0 ? "inf" : "-inf");
+            else if (std::isnan(v))
+               f << "nan";
+            else
+               f << std::setprecision(std::numeric_limits<float>::max_digits10) << v;
+         } break;
+         case ETensorType::INT8: f << (int)static_cast<const int8_t *>(kv.second.data.get())[i]; break;
+         case ETensorType::UINT8: case ETensorType::BOOL: case ETensorType::FLOAT8E4M3FN:
+            f << (unsigned)static_cast<const uint8_t *>(kv.second.data.get())[i];
+            break;
+         case ETensorType::INT32: f << static_cast<const int32_t *>(kv.second.data.get())[i]; break;
+         case ETensorType::INT64: f << static_cast<const int64_t *>(kv.second.data.get())[i]; break;
+         default: throw std::runtime_error("sofie tensor tensor_" + kv.first + " with type " + ConvertTypeToString(kv.second.type) + " cannot be written to a file");
+         }
+         f << (i + 1 < len ? " " : "\n");
+      }
+      if (len == 0)
+         f << "\n";
+      if (f.fail())
+         throw std::runtime_error("sofie failed to write tensor data to file for  tensor_" + kv.first);
+   }
+}
+
+void RModel::OutputGenerated(std::string filename)
+{
+   if (fGC.empty())
+      throw std::runtime_error("SOFIE: OutputGenerated called before GenerateGPU_HIP");
+   if (filename.empty())
+      filename = fName + "_GPU_HIP.hxx";
+   std::ofstream f(filename);
+   if (!f.is_open())
+      throw std::runtime_error("tmva-sofie failed to open file " + filename + " for the generated code");
+   f << fGC;
+   f.close();
+   std::string dat = filename;
+   auto dot = dat.find_last_of('.');
+   if (dot != std::string::npos)
+      dat = dat.substr(0, dot);
+   WriteWeightFile(dat + ".dat");
+}
+
+} // namespace SOFIE_HIP

@@ -1,0 +1,411 @@
+#include "SOFIE_HIP/RModelParser_ONNX.hxx"
+#include "SOFIE_HIP/operators/OperatorList.hxx"
+
+#include <fstream>
+#include <iostream>
+#include <iterator>
+#include <map>
+
+namespace SOFIE_HIP {
+namespace {
+
+struct Slice {
+   const uint8_t *p = nullptr;
+   size_t n = 0;
+};
+
+struct Field {
+   uint32_t no;
+   uint32_t wt;
+   uint64_t v;   // varint or fixed value
+   Slice bytes;  // length-delimited payload
+};
+
+class Reader {
+public:
+   explicit Reader(Slice s) : fP(s.p), fEnd(s.p + s.n) {}
+   bool Next(Field &f)
+   {
+      if (fP >= fEnd)
+         return false;
+      uint64_t key = Varint();
+      f.no = (uint32_t)(key >> 3);
+      f.wt = (uint32_t)(key & 7);
+      f.v = 0;
+      f.bytes = Slice{};
+      switch (f.wt) {
+      case 0: f.v = Varint(); break;
+      case 1: f.v = Fixed(8); break;
+      case 5: f.v = Fixed(4); break;
+      case 2: {
+         uint64_t len = Varint();
+         if (len > (uint64_t)(fEnd - fP))
+            throw std::runtime_error("SOFIE ONNX parser: truncated file");
+         f.bytes = Slice{fP, (size_t)len};
+         fP += len;
+      } break;
+      default: throw std::runtime_error("SOFIE ONNX parser: unsupported wire type");
+      }
+      return true;
+   }
+
+private:
+   uint64_t Varint()
+   {
+      uint64_t r = 0;
+      int shift = 0;
+      while (true) {
+         if (fP >= fEnd)
+            throw std::runtime_error("SOFIE ONNX parser: truncated varint");
+         uint8_t b = *fP++;
+         r |= (uint64_t)(b & 0x7f) << shift;
+         if (!(b & 0x80))
+            return r;
+         shift += 7;
+      }
+   }
+   uint64_t Fixed(int n)
+   {
+      if (fEnd - fP < n)
+         throw std::runtime_error("SOFIE ONNX parser: truncated file");
+      uint64_t r = 0;
+      for (int i = 0; i < n; ++i)
+         r |= (uint64_t)fP[i] << (8 * i);
+      fP += n;
+      return r;
+   }
+   const uint8_t *fP, *fEnd;
+};
+
+std::string Str(Slice s) { return std::string((const char *)s.p, s.n); }
+
+std::vector<int64_t> PackedInts(const Field &f)
+{
+   std::vector<int64_t> out;
+   if (f.wt == 0) {
+      out.push_back((int64_t)f.v);
+      return out;
+   }
+   Reader r(f.bytes);
+   // a packed field is a sequence of bare varints: reuse the reader by faking keys is not possible, so decode here
+   const uint8_t *p = f.bytes.p, *e = f.bytes.p + f.bytes.n;
+   while (p < e) {
+      uint64_t v = 0;
+      int shift = 0;
+      while (p < e) {
+         uint8_t b = *p++;
+         v |= (uint64_t)(b & 0x7f) << shift;
+         if (!(b & 0x80))
+            break;
+         shift += 7;
+      }
+      out.push_back((int64_t)v);
+   }
+   return out;
+}
+
+float AsFloat(uint32_t bits)
+{
+   float f;
+   std::memcpy(&f, &bits, 4);
+   return f;
+}
+
+struct Tensor {
+   std::string name;
+   int dtype = 1;
+   std::vector<size_t> dims;
+   std::vector<uint8_t> raw;        // raw_data
+   std::vector<float> floats;       // float_data
+   std::vector<int64_t> ints;       // int32_data / int64_data
+};
+
+Tensor ParseTensor(Slice s)
+{
+   Tensor t;
+   Reader r(s);
+   Field f;
+   while (r.Next(f)) {
+      switch (f.no) {
+      case 1:
+         for (auto d : PackedInts(f))
+            t.dims.push_back((size_t)d);
+         break;
+      case 2: t.dtype = (int)f.v; break;
+      case 4:
+         if (f.wt == 2)
+            for (size_t i = 0; i + 4 <= f.bytes.n; i += 4) {
+               uint32_t b;
+               std::memcpy(&b, f.bytes.p + i, 4);
+               t.floats.push_back(AsFloat(b));
+            }
+         else
+            t.floats.push_back(AsFloat((uint32_t)f.v));
+         break;
+      case 5:
+      case 7:
+         for (auto v : PackedInts(f))
+            t.ints.push_back(v);
+         break;
+      case 8: t.name = Str(f.bytes); break;
+      case 9: t.raw.assign(f.bytes.p, f.bytes.p + f.bytes.n); break;
+      default: break;
+      }
+   }
+   return t;
+}
+
+struct Attr {
+   std::string s;
+   int64_t i = 0;
+   float f = 0;
+   std::vector<int64_t> ints;
+   bool has_i = false, has_f = false, has_s = false;
+};
+
+struct Node {
+   std::string op, name;
+   std::vector<std::string> in, out;
+   std::map<std::string, Attr> attrs;
+};
+
+Node ParseNode(Slice s)
+{
+   Node n;
+   Reader r(s);
+   Field f;
+   while (r.Next(f)) {
+      switch (f.no) {
+      case 1: n.in.push_back(Str(f.bytes)); break;
+      case 2: n.out.push_back(Str(f.bytes)); break;
+      case 3: n.name = Str(f.bytes); break;
+      case 4: n.op = Str(f.bytes); break;
+      case 5: {
+         Attr a;
+         std::string an;
+         Reader ra(f.bytes);
+         Field g;
+         while (ra.Next(g)) {
+            switch (g.no) {
+            case 1: an = Str(g.bytes); break;
+            case 2: a.f = AsFloat((uint32_t)g.v); a.has_f = true; break;
+            case 3: a.i = (int64_t)g.v; a.has_i = true; break;
+            case 4: a.s = Str(g.bytes); a.has_s = true; break;
+            case 8:
+               for (auto v : PackedInts(g))
+                  a.ints.push_back(v);
+               break;
+            default: break;
+            }
+         }
+         n.attrs[an] = a;
+      } break;
+      default: break;
+      }
+   }
+   return n;
+}
+
+struct ValueInfo {
+   std::string name;
+   int elem_type = 1;
+   std::vector<size_t> shape;
+   bool symbolic = false;
+};
+
+ValueInfo ParseValueInfo(Slice s)
+{
+   ValueInfo v;
+   Reader r(s);
+   Field f;
+   while (r.Next(f)) {
+      if (f.no == 1)
+         v.name = Str(f.bytes);
+      else if (f.no == 2) {
+         Reader rt(f.bytes);
+         Field t;
+         while (rt.Next(t))
+            if (t.no == 1) { // tensor_type
+               Reader rtt(t.bytes);
+               Field u;
+               while (rtt.Next(u)) {
+                  if (u.no == 1)
+                     v.elem_type = (int)u.v;
+                  else if (u.no == 2) { // shape
+                     Reader rs(u.bytes);
+                     Field d;
+                     while (rs.Next(d))
+                        if (d.no == 1) {
+                           Reader rd(d.bytes);
+                           Field x;
+                           bool value = false;
+                           while (rd.Next(x))
+                              if (x.no == 1) {
+                                 v.shape.push_back((size_t)x.v);
+                                 value = true;
+                              }
+                           if (!value) {
+                              v.shape.push_back(0);
+                              v.symbolic = true;
+                           }
+                        }
+                  }
+               }
+            }
+      }
+   }
+   return v;
+}
+
+std::vector<size_t> ToSizes(const std::vector<int64_t> &v) { return std::vector<size_t>(v.begin(), v.end()); }
+
+} // namespace
+
+std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verbose)
+{
+   std::ifstream in(filename, std::ios::binary);
+   if (!in.is_open())
+      throw std::runtime_error("SOFIE ONNX parser: failed to open " + filename);
+   std::vector<uint8_t> buf((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
+   Slice graph;
+   {
+      Reader r(Slice{buf.data(), buf.size()});
+      Field f;
+      while (r.Next(f))
+         if (f.no == 7)
+            graph = f.bytes;
+   }
+   if (!graph.p)
+      throw std::runtime_error("SOFIE ONNX parser: " + filename + " holds no graph");
+   std::vector<Node> nodes;
+   std::vector<Tensor> inits;
+   std::vector<ValueInfo> inputs, outputs;
+   {
+      Reader r(graph);
+      Field f;
+      while (r.Next(f)) {
+         if (f.no == 1)
+            nodes.push_back(ParseNode(f.bytes));
+         else if (f.no == 5)
+            inits.push_back(ParseTensor(f.bytes));
+         else if (f.no == 11)
+            inputs.push_back(ParseValueInfo(f.bytes));
+         else if (f.no == 12)
+            outputs.push_back(ParseValueInfo(f.bytes));
+      }
+   }
+   auto model = std::make_unique<RModel>(filename);
+   std::map<std::string, bool> isInit;
+   for (auto &t : inits) {
+      isInit[t.name] = true;
+      const ETensorType ty = static_cast<ETensorType>(t.dtype);
+      const size_t len = ConvertShapeToLength(t.dims);
+      const size_t esz = GetTypeSize(ty);
+      if (esz == 0)
+         throw std::runtime_error("SOFIE ONNX parser: initializer " + t.name + " has an unsupported data type " + std::to_string(t.dtype));
+      std::vector<uint8_t> data(len * esz);
+      if (!t.raw.empty()) {
+         if (t.raw.size() != data.size())
+            throw std::runtime_error("SOFIE ONNX parser: initializer " + t.name + " has raw data of the wrong size");
+         data = t.raw;
+      } else if (ty == ETensorType::FLOAT) {
+         if (t.floats.size() != len)
+            throw std::runtime_error("SOFIE ONNX parser: initializer " + t.name + " has the wrong number of values");
+         std::memcpy(data.data(), t.floats.data(), data.size());
+      } else {
+         if (t.ints.size() != len)
+            throw std::runtime_error("SOFIE ONNX parser: initializer " + t.name + " has the wrong number of values");
+         for (size_t i = 0; i < len; ++i) {
+            int64_t v = t.ints[i];
+            std::memcpy(data.data() + i * esz, &v, esz); // little endian: the low bytes
+         }
+      }
+      model->AddInitializedTensor(t.name, ty, t.dims, data.data());
+   }
+   for (auto &v : inputs) {
+      if (isInit.count(v.name))
+         continue;
+      if (v.symbolic)
+         throw std::runtime_error("SOFIE ONNX parser: input " + v.name + " has a symbolic dimension; this backend emits static shapes");
+      model->AddInputTensorInfo(v.name, static_cast<ETensorType>(v.elem_type), v.shape);
+      model->AddInputTensorName(v.name);
+   }
+   std::map<std::string, int> uses;
+   for (auto &n : nodes)
+      for (auto &i : n.in)
+         uses[i]++;
+   auto attrI = [](const Node &n, const char *k, int64_t def) { auto f = n.attrs.find(k); return f == n.attrs.end() || !f->second.has_i ? def : f->second.i; };
+   auto attrF = [](const Node &n, const char *k, float def) { auto f = n.attrs.find(k); return f == n.attrs.end() || !f->second.has_f ? def : f->second.f; };
+   auto attrS = [](const Node &n, const char *k, const char *def) { auto f = n.attrs.find(k); return f == n.attrs.end() || !f->second.has_s ? std::string(def) : f->second.s; };
+   auto attrV = [](const Node &n, const char *k) { auto f = n.attrs.find(k); return f == n.attrs.end() ? std::vector<size_t>{} : ToSizes(f->second.ints); };
+
+   std::vector<bool> consumed(nodes.size(), false);
+   for (size_t i = 0; i < nodes.size(); ++i) {
+      if (consumed[i])
+         continue;
+      const Node &n = nodes[i];
+      if (verbose)
+         std::cout << "SOFIE HIP parser: " << n.op << " " << n.name << "\n";
+      if (n.op == "Gemm") {
+         if (n.in.size() > 2 && !n.in[2].empty())
+            model->AddOperator(std::make_unique<ROperator_Gemm<float>>(attrF(n, "alpha", 1.f), attrF(n, "beta", 1.f), attrI(n, "transA", 0),
+                                                                       attrI(n, "transB", 0), n.in[0], n.in[1], n.in[2], n.out[0]));
+         else
+            model->AddOperator(std::make_unique<ROperator_Gemm<float>>(attrF(n, "alpha", 1.f), attrF(n, "beta", 1.f), attrI(n, "transA", 0),
+                                                                       attrI(n, "transB", 0), n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "MatMul") {
+         // MatMul whose only consumer is an Add of an initializer: one Gemm with bias
+         size_t addIdx = nodes.size();
+         if (uses[n.out[0]] == 1)
+            for (size_t j = i + 1; j < nodes.size(); ++j)
+               if (nodes[j].op == "Add" && nodes[j].in.size() == 2 && (nodes[j].in[0] == n.out[0] || nodes[j].in[1] == n.out[0])) {
+                  const std::string &other = nodes[j].in[0] == n.out[0] ? nodes[j].in[1] : nodes[j].in[0];
+                  if (isInit.count(other))
+                     addIdx = j;
+                  break;
+               }
+         if (addIdx < nodes.size()) {
+            const Node &a = nodes[addIdx];
+            const std::string &bias = a.in[0] == n.out[0] ? a.in[1] : a.in[0];
+            model->AddOperator(std::make_unique<ROperator_Gemm<float>>(1.f, 1.f, 0, 0, n.in[0], n.in[1], bias, a.out[0]));
+            consumed[addIdx] = true;
+         } else {
+            model->AddOperator(std::make_unique<ROperator_Gemm<float>>(1.f, 0.f, 0, 0, n.in[0], n.in[1], n.out[0]));
+         }
+      } else if (n.op == "Relu") {
+         model->AddOperator(std::make_unique<ROperator_Relu<float>>(n.in[0], n.out[0]));
+      } else if (n.op == "Sigmoid") {
+         model->AddOperator(std::make_unique<ROperator_Sigmoid<float>>(n.in[0], n.out[0]));
+      } else if (n.op == "Tanh") {
+         model->AddOperator(std::make_unique<ROperator_Tanh<float>>(n.in[0], n.out[0]));
+      } else if (n.op == "LeakyRelu") {
+         model->AddOperator(std::make_unique<ROperator_LeakyRelu<float>>(attrF(n, "alpha", 0.01f), n.in[0], n.out[0]));
+      } else if (n.op == "Gelu") {
+         model->AddOperator(std::make_unique<ROperator_Gelu<float>>(attrS(n, "approximate", "none"), n.in[0], n.out[0]));
+      } else if (n.op == "Add") {
+         model->AddOperator(std::make_unique<ROperator_BasicBinary<float, Add>>(n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "Conv") {
+         const std::string bias = n.in.size() > 2 ? n.in[2] : "";
+         model->AddOperator(std::make_unique<ROperator_Conv<float>>(attrS(n, "auto_pad", "NOTSET"), attrV(n, "dilations"), (size_t)attrI(n, "group", 1),
+                                                                    attrV(n, "kernel_shape"), attrV(n, "pads"), attrV(n, "strides"), n.in[0],
+                                                                    n.in[1], bias, n.out[0]));
+      } else if (n.op == "GlobalAveragePool") {
+         model->AddOperator(std::make_unique<ROperator_Pool<float>>(GlobalAveragePool, n.in[0], n.out[0]));
+      } else if (n.op == "QuantizeLinear") {
+         model->AddOperator(std::make_unique<ROperator_QuantizeLinear>(n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "DequantizeLinear") {
+         model->AddOperator(std::make_unique<ROperator_DequantizeLinear>(n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "MatMulInteger") {
+         model->AddOperator(MakeMatMulInteger(n.in[0], n.in[1], n.out[0]));
+      } else {
+         throw std::runtime_error("SOFIE Operator type " + n.op + " is not yet supported");
+      }
+   }
+   std::vector<std::string> outs;
+   for (auto &o : outputs)
+      outs.push_back(o.name);
+   model->AddOutputTensorNameList(outs);
+   return model;
+}
+
+} // namespace SOFIE_HIP

@@ -1,0 +1,163 @@
+"""The models that go through the C++ emitter: every golden fixture of the reference plus the BASELINE
+configurations this backend adds (built here as ONNX files from seeded data).  build_all() runs at build
+time on the CPU: it writes the ONNX files, runs sofie_hip_emit, and compiles each emitted header together
+with a tiny C harness into tests/emitted/lib<Model>.so.  The GPU tests only load those libraries."""
+import json
+import os
+import subprocess
+
+import numpy as np
+
+from tests import onnx_write as ow
+from tests import util
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+OUT = os.path.join(ROOT, "tests", "emitted")
+EMIT = os.path.join(ROOT, "sofie_amd", "emit", "bin", "sofie_hip_emit")
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+# ---- configuration models ------------------------------------------------------------------------------------
+
+def fp32_mlp(batch=64):
+    """BASELINE config 1: Gemm(transB=1)+Relu, Gemm+Relu, Gemm; 784 -> 128 -> 64 -> 10; W ~ N(0, 0.05), biases 0."""
+    dims = [784, 128, 64, 10]
+    init, nodes, x = {}, [], "X"
+    for l in range(3):
+        init["W%d" % l] = util.normal(1001 + l, dims[l + 1] * dims[l], 0.05).reshape(dims[l + 1], dims[l])
+        init["B%d" % l] = np.zeros(dims[l + 1], dtype=np.float32)
+        y = "G%d" % l
+        nodes.append(ow.node("Gemm", [x, "W%d" % l, "B%d" % l], [y], alpha=1.0, beta=1.0, transB=1))
+        if l < 2:
+            nodes.append(ow.node("Relu", [y], ["R%d" % l]))
+            y = "R%d" % l
+        x = y
+    X = util.uniform01(2001, batch * 784).reshape(batch, 784)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 784])], outputs=[(x, np.float32, [batch, 10])], init=init, feeds=[X])
+
+
+def int8_mlp(dims, batch, seed=1100):
+    """BASELINE config 2 as ONNX operators: per layer QuantizeLinear -> MatMulInteger -> Relu -> DequantizeLinear,
+    per-tensor symmetric scales (zero points 0).  Returns the model and the constants the CPU chain needs."""
+    from oracle import binding as ob
+    weights = [util.int8_sym(seed + 1 + l, dims[l] * dims[l + 1]).reshape(dims[l], dims[l + 1]) for l in range(len(dims) - 1)]
+    X = util.normal(seed + 1001, batch * dims[0]).reshape(batch, dims[0])
+    w_scales = [np.float32(1.0 / 127.0)] * len(weights)
+    in_scales = [np.float32(np.abs(X).max() / 127.0)]
+    h = X[:8]
+    for l, w in enumerate(weights[:-1]):
+        q = ob.quantize_linear(h, in_scales[l])
+        acc = np.maximum(ob.matmul_integer(q, w, M=h.shape[0], N=w.shape[1], K=w.shape[0], omp=True), 0)
+        h = ob.dequantize_linear(acc, np.float32(in_scales[l] * w_scales[l]))
+        in_scales.append(np.float32(max(h.max(), 1e-6) / 127.0))
+    init, nodes, x = {}, [], "X"
+    for l, w in enumerate(weights):
+        init["W%d" % l] = w
+        init["sx%d" % l] = np.array(in_scales[l], dtype=np.float32)
+        init["sy%d" % l] = np.array(np.float32(in_scales[l] * w_scales[l]), dtype=np.float32)
+        nodes.append(ow.node("QuantizeLinear", [x, "sx%d" % l], ["Q%d" % l]))
+        nodes.append(ow.node("MatMulInteger", ["Q%d" % l, "W%d" % l], ["A%d" % l]))
+        nodes.append(ow.node("Relu", ["A%d" % l], ["R%d" % l]))
+        nodes.append(ow.node("DequantizeLinear", ["R%d" % l, "sy%d" % l], ["D%d" % l]))
+        x = "D%d" % l
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, dims[0]])], outputs=[(x, np.float32, [batch, dims[-1]])], init=init,
+                feeds=[X], consts=dict(weights=weights, w_scales=w_scales, in_scales=in_scales))
+
+
+def fp32_cnn(batch=2):
+    """A small fp32 form of BASELINE config 5: 2 x [Conv3x3 s1 p1 + Relu], GlobalAveragePool, Gemm."""
+    init = {"W0": util.normal(5101, 8 * 3 * 9, 0.2).reshape(8, 3, 3, 3), "B0": util.normal(5102, 8, 0.1),
+            "W1": util.normal(5103, 16 * 8 * 9, 0.1).reshape(16, 8, 3, 3), "B1": util.normal(5104, 16, 0.1),
+            "WF": util.normal(5105, 16 * 10, 0.3).reshape(16, 10), "BF": util.normal(5106, 10, 0.1)}
+    nodes = [ow.node("Conv", ["X", "W0", "B0"], ["C0"], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1]),
+             ow.node("Relu", ["C0"], ["R0"]),
+             ow.node("Conv", ["R0", "W1", "B1"], ["C1"], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1]),
+             ow.node("Relu", ["C1"], ["R1"]),
+             ow.node("GlobalAveragePool", ["R1"], ["P"]),
+             ow.node("Gemm", ["P2", "WF", "BF"], ["Y"], alpha=1.0, beta=1.0)]
+    # GlobalAveragePool gives [N,16,1,1]; the Gemm reads it as [N,16]: same bytes, so the model feeds P straight in
+    nodes[-1] = ow.node("Gemm", ["P", "WF", "BF"], ["Y"], alpha=1.0, beta=1.0)
+    X = util.uniform01(5001, batch * 3 * 12 * 12).reshape(batch, 3, 12, 12)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 3, 12, 12])], outputs=[("Y", np.float32, [batch, 10])], init=init, feeds=[X])
+
+
+CONFIG_MODELS = {
+    "Config1_fp32_MLP": lambda: fp32_mlp(64),
+    "Config2_int8_MLP_small": lambda: int8_mlp([64, 128, 96, 32], 48),
+    "Config2_int8_MLP_mid": lambda: int8_mlp([256, 512, 512, 256], 256),
+}
+
+
+def golden_models():
+    return sorted(json.load(open(os.path.join(GOLDEN, "fixtures.json"))).keys())
+
+
+# ---- build ----------------------------------------------------------------------------------------------------
+
+HARNESS = r'''
+#include "%(model)s_GPU_HIP.hxx"
+#include <cstring>
+// C harness around the emitted Session for the Python tests: returns 0, or 1 with the exception text in err.
+extern "C" int run_model(const char *weights, const float *const *inputs, float *output, unsigned long output_len, char *err, int errlen)
+{
+   try {
+      SOFIE_%(model)s::Session s(weights);
+      auto y = s.infer(%(args)s);
+      if (y.size() != output_len)
+         throw std::runtime_error("output has " + std::to_string(y.size()) + " elements");
+      std::memcpy(output, y.data(), y.size() * sizeof(float));
+      // a second inference on the same session must give the same answer (the pool is reused)
+      auto y2 = s.infer(%(args)s);
+      if (std::memcmp(y.data(), y2.data(), y.size() * sizeof(float)) != 0)
+         throw std::runtime_error("second inference differs from the first");
+      return 0;
+   } catch (const std::exception &e) {
+      std::strncpy(err, e.what(), errlen - 1);
+      err[errlen - 1] = 0;
+      return 1;
+   }
+}
+extern "C" unsigned long arena_bytes() { return SOFIE_%(model)s::Session::kArenaBytes; }
+extern "C" unsigned long pool_bytes() { return SOFIE_%(model)s::Session::kIntermediatePoolBytes; }
+'''
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), r.stdout))
+    return r.stdout
+
+
+def emit_and_compile(model, onnx_path, n_inputs):
+    _run([EMIT, onnx_path, OUT])
+    src = os.path.join(OUT, model + "_harness.cxx")
+    with open(src, "w") as f:
+        f.write(HARNESS % dict(model=model, args=", ".join("inputs[%d]" % i for i in range(n_inputs))))
+    lib = os.path.join(OUT, "lib%s.so" % model)
+    _run(["g++", "-O1", "-std=c++20", "-fPIC", "-shared", "-I" + os.path.join(ROOT, "include"), "-I" + OUT, src, "-o", lib,
+          "-L" + os.path.join(ROOT, "sofie_amd", "lib"), "-lsofie_hip", "-Wl,-rpath," + os.path.join(ROOT, "sofie_amd", "lib"),
+          "-Wl,-rpath,$ORIGIN/../../sofie_amd/lib"])
+    return lib
+
+
+def build_all(jobs=8):
+    from concurrent.futures import ThreadPoolExecutor
+    from tests import onnx_lite
+    os.makedirs(OUT, exist_ok=True)
+    work = []
+    for m in golden_models():
+        p = os.path.join(GOLDEN, "models", m + ".onnx")
+        work.append((m, p, len(onnx_lite.load(p)["inputs"])))
+    for m, make in CONFIG_MODELS.items():
+        spec = make()
+        p = os.path.join(OUT, m + ".onnx")
+        ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)
+        work.append((m, p, len(spec["inputs"])))
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        list(ex.map(lambda w: emit_and_compile(*w), work))
+    return [w[0] for w in work]
+
+
+if __name__ == "__main__":
+    print("\n".join(build_all()))

@@ -1,0 +1,158 @@
+"""The C++ emitter (sofie_amd/emit): the text it generates and its memory plan, checked on the CPU.
+Reference behaviour mirrored: RModel::GenerateSessionCode (core/src/RModel.cxx:1167-1460), the planner
+OrganizeMemory (core/inc/SOFIE/MemoryPlanner.inc:67-170) and the Session/infer API of the generated code."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from tests import emitted_models as em
+from tests import onnx_write as ow
+
+
+@pytest.fixture(scope="module")
+def emitted():
+    if not os.path.exists(os.path.join(em.OUT, "libLinear_16.so")):
+        em.build_all()
+    return em.OUT
+
+
+def plan_of(onnx_path, tmp_path):
+    out = subprocess.run([em.EMIT, onnx_path, str(tmp_path), "--plan"], check=True, stdout=subprocess.PIPE, text=True).stdout.split("\n")
+    head = out[0].split()
+    rows = []
+    for line in out[1:]:
+        f = line.split()
+        if len(f) == 6:
+            rows.append(dict(name=f[0], offset=int(f[1]), bytes=int(f[2]), first=int(f[3]), last=int(f[4]), pooled=int(f[5])))
+    return int(head[1]), int(head[3]), rows
+
+
+def test_linear16_pool_matches_the_reference_planner(emitted, tmp_path):
+    # the reference's GPU planner gives 6656 bytes for this model (two 3200-byte activations alive at once,
+    # each rounded to 256): same figure from oracle/_ref's build of MemoryPlanner.inc in test_oracle_pins
+    arena, pool, rows = plan_of(os.path.join(em.GOLDEN, "models", "Linear_16.onnx"), tmp_path)
+    assert pool == 6656
+    assert arena == max(r["offset"] + r["bytes"] for r in rows)
+
+
+@pytest.mark.parametrize("model", ["Linear_16", "ConvWithPadding", "LinearWithSigmoid", "Config1_fp32_MLP", "Config2_int8_MLP_mid"])
+def test_plan_alignment_and_liveness(emitted, tmp_path, model):
+    path = os.path.join(em.GOLDEN, "models", model + ".onnx")
+    if not os.path.exists(path):
+        path = os.path.join(emitted, model + ".onnx")
+    arena, pool, rows = plan_of(path, tmp_path)
+    assert rows
+    for r in rows:
+        assert r["offset"] % 256 == 0 and r["offset"] + r["bytes"] <= arena
+    for i, a in enumerate(rows):
+        for b in rows[i + 1:]:
+            overlap_mem = a["offset"] < b["offset"] + b["bytes"] and b["offset"] < a["offset"] + a["bytes"]
+            if not overlap_mem:
+                continue
+            # sharing bytes is allowed only between pooled tensors whose lifetimes are disjoint
+            assert a["pooled"] and b["pooled"], (a, b)
+            assert a["last"] <= b["first"] or b["last"] <= a["first"], (a, b)
+    pooled = [r for r in rows if r["pooled"]]
+    if pooled:
+        lo = min(r["offset"] for r in pooled)
+        assert max(r["offset"] + r["bytes"] for r in pooled) - lo == pool
+        assert pool <= sum(r["bytes"] for r in pooled)
+
+
+def read(emitted, model):
+    return open(os.path.join(emitted, model + "_GPU_HIP.hxx")).read()
+
+
+def test_session_api_of_the_generated_header(emitted):
+    txt = read(emitted, "Linear_16")
+    assert "namespace SOFIE_Linear_16" in txt and "struct Session" in txt
+    assert re.search(r'Session\(std::string filename = "Linear_16_GPU_HIP\.dat"', txt)
+    assert re.search(r"std::vector<float> infer\(float const ?\*", txt)
+    assert "void infer_nosync()" in txt
+    assert "#include \"sofie_hip.h\"" in txt
+    # nothing in the generated code may allocate per inference
+    body = txt[txt.index("void infer_nosync()"):]
+    body = body[:body.index("std::vector<float> infer(")]
+    assert "arena_create" not in body and "hipMalloc" not in body and "new " not in body
+
+
+def test_gemm_relu_pairs_are_fused(emitted):
+    txt = read(emitted, "Linear_16")
+    body = txt[txt.index("void infer_nosync()"):]
+    assert body.count("sofie_hip_gemm_f32") == 10
+    assert "sofie_hip_unary_f32" not in body          # every Relu went into a Gemm epilogue
+    assert body.count("SOFIE_ACT_RELU") == 9
+    txt = read(emitted, "LinearWithSigmoid")
+    assert "SOFIE_ACT_SIGMOID" in txt
+
+
+def test_quantised_chain_collapses_to_one_kernel_per_layer(emitted):
+    txt = read(emitted, "Config2_int8_MLP_mid")
+    body = txt[txt.index("void infer_nosync()"):]
+    body = body[:body.index("infer(")]
+    assert body.count("sofie_hip_gemm_i8(") == 3
+    assert body.count("sofie_hip_quantize_linear(") == 1    # only the model input is quantised by its own kernel
+    assert "sofie_hip_dequantize_linear" not in body        # the last DequantizeLinear is the GEMM's fp32 store
+    assert body.count("SOFIE_I8OUT_I8_DQQ") == 2 and body.count("SOFIE_I8OUT_F32") == 1
+
+
+def test_conv_is_emitted_as_one_call_with_resolved_geometry(emitted):
+    txt = read(emitted, "ConvWithAsymmetricPadding")
+    assert txt.count("sofie_hip_conv_f32(") == 1
+    assert "im2col" not in txt.lower().replace("implicit im2col", "")
+
+
+def _emit(tmp_path, nodes, inputs, outputs, init, name="m"):
+    p = os.path.join(str(tmp_path), name + ".onnx")
+    ow.write(p, nodes, inputs, outputs, init, name=name)
+    return subprocess.run([em.EMIT, p, str(tmp_path)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+
+
+def test_unsupported_operator_is_refused_by_name(tmp_path):
+    r = _emit(tmp_path, [ow.node("LSTM", ["X"], ["Y"])], [("X", np.float32, [1, 4])], [("Y", np.float32, [1, 4])], {})
+    assert r.returncode != 0 and "LSTM" in r.stdout
+
+
+def test_shape_mismatch_is_refused(tmp_path):
+    init = {"W": np.zeros((5, 3), dtype=np.float32)}
+    r = _emit(tmp_path, [ow.node("Gemm", ["X", "W"], ["Y"])], [("X", np.float32, [2, 4])], [("Y", np.float32, [2, 3])], init)
+    assert r.returncode != 0 and "Gemm" in r.stdout
+
+
+def test_missing_input_tensor_is_refused(tmp_path):
+    r = _emit(tmp_path, [ow.node("Relu", ["nope"], ["Y"])], [("X", np.float32, [2, 4])], [("Y", np.float32, [2, 4])], {})
+    assert r.returncode != 0 and "nope" in r.stdout
+
+
+def test_session_fails_loudly_without_a_gpu(emitted):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("needs a machine without a GPU")
+    lib = ctypes.CDLL(os.path.join(emitted, "libLinear_16.so"))
+    err = ctypes.create_string_buffer(512)
+    x = np.ones(1600, dtype=np.float32)
+    y = np.zeros(160, dtype=np.float32)
+    inp = (ctypes.c_void_p * 1)(x.ctypes.data)
+    rc = lib.run_model(os.path.join(emitted, "Linear_16_GPU_HIP.dat").encode(), inp, y.ctypes.data_as(ctypes.c_void_p), ctypes.c_ulong(160), err, 512)
+    assert rc == 1 and b"SOFIE HIP runtime error" in err.value
+    assert not y.any()
+
+
+def test_weight_file_round_trip(emitted):
+    # the .dat file holds every initialised tensor as "name count" + values, fp32 printed so that it reads back exactly
+    from tests import onnx_lite
+    g = onnx_lite.load(os.path.join(em.GOLDEN, "models", "Linear_16.onnx"))
+    toks = open(os.path.join(emitted, "Linear_16_GPU_HIP.dat")).read().split()
+    i, seen = 0, {}
+    while i < len(toks):
+        name, n = toks[i], int(toks[i + 1])
+        seen[name] = np.array([float(t) for t in toks[i + 2:i + 2 + n]], dtype=np.float32)
+        i += 2 + n
+    assert len(seen) == len(g["initializers"])
+    for k, v in g["initializers"].items():
+        key = "tensor_" + re.sub(r"[^A-Za-z0-9_]", "_", k)
+        assert np.array_equal(seen[key], np.asarray(v, dtype=np.float32).ravel()), k

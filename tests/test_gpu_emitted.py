@@ -1,0 +1,63 @@
+"""Sessions written by the C++ emitter, compiled at build time, run on the GPU and compared with the reference's
+golden outputs and with the CPU oracle.  This is the user-visible path of the reference:
+parse -> Generate -> OutputGenerated -> #include the header -> Session s(weights); s.infer(x)
+(tests of the reference: core/test/TestCustomModelsFromONNX.cxx, the EmitFromONNX build step)."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+from tests import emitted_models as em
+from tests import graph_runner as gr
+from tests import onnx_lite
+from tests.test_oracle_golden import MODELS, golden_tolerance
+
+pytestmark = pytest.mark.gpu
+
+
+def run_emitted(model, inputs, out_len):
+    lib_path = os.path.join(em.OUT, "lib%s.so" % model)
+    assert os.path.exists(lib_path), "emitted models are built by __graft_entry__.build()"
+    lib = ctypes.CDLL(lib_path)
+    err = ctypes.create_string_buffer(1024)
+    arrs = [np.ascontiguousarray(a, dtype=np.float32) for a in inputs]
+    ptrs = (ctypes.c_void_p * len(arrs))(*[a.ctypes.data for a in arrs])
+    y = np.zeros(out_len, dtype=np.float32)
+    rc = lib.run_model(os.path.join(em.OUT, model + "_GPU_HIP.dat").encode(), ptrs, y.ctypes.data_as(ctypes.c_void_p),
+                       ctypes.c_ulong(out_len), err, 1024)
+    assert rc == 0, err.value.decode()
+    return y
+
+
+@pytest.mark.parametrize("model", MODELS)
+def test_emitted_session_reproduces_reference_golden_output(rt, model):
+    g, inputs, expected = gr.load_fixture(model)
+    print("emitted", model, flush=True)
+    got = run_emitted(model, inputs, expected.size)
+    assert np.abs(got - expected).max() <= golden_tolerance(model, expected)
+
+
+def test_emitted_fp32_mlp_matches_oracle(rt):
+    spec = em.fp32_mlp(64)
+    g = onnx_lite.load(os.path.join(em.OUT, "Config1_fp32_MLP.onnx"))
+    want = gr.run(g, spec["feeds"], gr.OracleBackend()).ravel()
+    print("emitted Config1_fp32_MLP", flush=True)
+    got = run_emitted("Config1_fp32_MLP", spec["feeds"], want.size)
+    assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+
+
+@pytest.mark.parametrize("model,dims,batch", [("Config2_int8_MLP_small", [64, 128, 96, 32], 48), ("Config2_int8_MLP_mid", [256, 512, 512, 256], 256)])
+def test_emitted_int8_mlp_is_bit_exact(rt, model, dims, batch):
+    from oracle import binding as ob
+    spec = em.int8_mlp(dims, batch)
+    c = spec["consts"]
+    h = spec["feeds"][0]
+    for l, w in enumerate(c["weights"]):   # the unfused ONNX chain, operator by operator
+        q = ob.quantize_linear(h, c["in_scales"][l])
+        acc = np.maximum(ob.matmul_integer(q, w, M=batch, N=w.shape[1], K=w.shape[0], omp=True), 0)
+        h = ob.dequantize_linear(acc, np.float32(c["in_scales"][l] * c["w_scales"][l]))
+    print("emitted", model, flush=True)
+    got = run_emitted(model, spec["feeds"], h.size)
+    assert np.array_equal(got.view(np.uint32), h.ravel().view(np.uint32))
+    assert np.abs(h).max() > 0
