@@ -1,6 +1,6 @@
 // FP8 (OCP e4m3fn) GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x64_f8f6f4, fp32 accumulate) with
 // scale + bias + activation + bf16 conversion fused into the store, and the fp32 -> e4m3fn quantiser.
-#include "mfma8_gemm_dma.hpp"
+#include "mfma8_gemm_pair.hpp"
 #include <cstdlib>
 
 namespace sofie_hip {
@@ -43,6 +43,26 @@ __global__ __launch_bounds__(256) void quantize_fp8_kernel(uint8_t *__restrict__
    const size_t stride = (size_t)gridDim.x * blockDim.x;
    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += stride)
       dst[i] = f32_to_e4m3_rne_sat(__fdiv_rn(src[i], scale));
+}
+
+// GELU (erf form) for the FP8 store: erf by the rational approximation 7.1.26 of Abramowitz & Stegun,
+//   erf(z) = 1 - (a1 t + ... + a5 t^5) exp(-z^2),  t = 1/(1 + p z),  z >= 0,   |error| <= 1.5e-7,
+// one exponential and one reciprocal per element instead of the library erff (the tile store of a
+// 256 x 256 tile evaluates it 256 times per lane, which with erff costs half as much as the whole K loop).
+// The absolute error of the result, <= 2e-7 |v|, is far inside the FP8 GEMM's stated bound.
+__device__ __forceinline__ float gelu_erf_fast(float v)
+{
+   const float z = __fmul_rn(v, 0.7071067811865475f);
+   const float az = fabsf(z);
+   const float t = __frcp_rn(__fmaf_rn(0.3275911f, az, 1.0f));
+   float poly = __fmaf_rn(t, 1.061405429f, -1.453152027f);
+   poly = __fmaf_rn(t, poly, 1.421413741f);
+   poly = __fmaf_rn(t, poly, -0.284496736f);
+   poly = __fmaf_rn(t, poly, 0.254829592f);
+   poly = __fmul_rn(poly, t);
+   const float q = __fmul_rn(poly, __expf(-__fmul_rn(az, az))); // erfc(|z|)
+   const float one_plus_erf = (z < 0.0f) ? q : (2.0f - q);
+   return __fmul_rn(__fmul_rn(0.5f, v), one_plus_erf);
 }
 
 struct F8Epilogue {
@@ -92,7 +112,7 @@ struct F8Epilogue {
          v[i] = mul_nofma(a[i], scale);
          if (bias)
             v[i] = v[i] + p.b[4 * q + i];
-         v[i] = apply_act(v[i], act, 0.0f);
+         v[i] = (act == SOFIE_ACT_GELU) ? gelu_erf_fast(v[i]) : apply_act(v[i], act, 0.0f);
       }
       if (OUT == SOFIE_F8OUT_F32) {
 #pragma unroll

@@ -50,27 +50,31 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(R
    tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, sw, tm, tn);
    const int m0 = tm * BM, n0 = tn * BN;
    const int t = threadIdx.x;
-   const int lane = t & 63, wave = t >> 6;
+   const int lane = t & 63;
+   const int wave = __builtin_amdgcn_readfirstlane(t >> 6); // uniform: keeps the LDS destinations of the loads in scalar registers
    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
    const int lr = lane & 31, lk = lane >> 5;
 
    // per-lane global source of every load instruction of a slab (k offset added per slab)
-   const int8_t *ga[A_LD], *gb[B_LD];
+   // Source of every load instruction of a slab: a uniform base (tile origin + k offset, scalar registers)
+   // plus a 32-bit per-lane offset, so that the address needs no vector arithmetic inside the loop.
+   const int8_t *const a_tile = A.row(m0), *const b_tile = Bt.row(n0);
+   uint32_t oa[A_LD], ob[B_LD];
 #pragma unroll
    for (int i = 0; i < A_LD; ++i) {
       const int row = (i * NW + wave) * RPI + lane / CPR; // row of the tile this lane fills
       constexpr int RPB = (256 / BK) > 0 ? (256 / BK) : 1;
       const int c = (lane % CPR) ^ ((row / RPB) % CPR);   // logical chunk stored at this lane's LDS position
-      const int gr = m0 + row;
-      ga[i] = A.row(gr < M ? gr : M - 1) + c * 16;
+      const int rc = (m0 + row < M) ? row : M - 1 - m0;   // rows past the edge re-read the last row
+      oa[i] = (uint32_t)rc * (uint32_t)A.ld + (uint32_t)(c * 16);
    }
 #pragma unroll
    for (int i = 0; i < B_LD; ++i) {
       const int row = (i * NW + wave) * RPI + lane / CPR;
       constexpr int RPB = (256 / BK) > 0 ? (256 / BK) : 1;
       const int c = (lane % CPR) ^ ((row / RPB) % CPR);
-      const int gr = n0 + row;
-      gb[i] = Bt.row(gr < N ? gr : N - 1) + c * 16;
+      const int rc = (n0 + row < N) ? row : N - 1 - n0;
+      ob[i] = (uint32_t)rc * (uint32_t)Bt.ld + (uint32_t)(c * 16);
    }
    // One K-step's share of a slab's load instructions (A's first, then Bt's): part `part` of KS equal parts.
    constexpr int KS_ = BK / MMA::KSTEP;
@@ -86,9 +90,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(R
       static_for<L1 - L0>([&](auto lc) {
          constexpr int l = L0 + decltype(lc)::value;
          if constexpr (l < A_LD)
-            __builtin_amdgcn_global_load_lds((global_void_t *)(ga[l] + koff), (lds_void_t *)(sA + (l * NW + wave) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_void_t *)((a_tile + koff) + oa[l]), (lds_void_t *)(sA + (l * NW + wave) * 1024), 16, 0, 0);
          else
-            __builtin_amdgcn_global_load_lds((global_void_t *)(gb[l - A_LD] + koff), (lds_void_t *)(sB + ((l - A_LD) * NW + wave) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_void_t *)((b_tile + koff) + ob[l - A_LD]), (lds_void_t *)(sB + ((l - A_LD) * NW + wave) * 1024), 16, 0, 0);
       });
    };
 
@@ -221,60 +225,3 @@ static int launch_mfma8_dma(hipStream_t stream, const int8_t *A, const int8_t *B
 
 } // namespace sofie_hip
 
-namespace sofie_hip {
-
-// Chooses between the pipelined kernel (aligned operands, K a multiple of 64) and the general one.
-// `variant` selects a tuning alternative of the pipelined kernel (0 = default); -1 forces the general kernel.
-template <class MMA, class EPI>
-static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb,
-                             const EPI &ep, int force_tile, int variant)
-{
-   const bool aligned = (lda % 16 == 0) && (ldb % 16 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)Bt & 15) == 0);
-   if (variant < 0 || !aligned || K < 64 || K % 64 != 0)
-      return launch_mfma8_auto<MMA, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile);
-   const int tile = pick_tile(M, N, force_tile);
-   const bool k128 = (K % 128 == 0);
-   if constexpr (MMA::KSTEP * 2 > 64) {
-      // two K-steps per slab are the minimum: a 64-byte K-step needs 128-byte slabs
-      if (!k128)
-         return launch_mfma8_auto<MMA, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile);
-      switch (tile) {
-      case 256: return launch_mfma8_dma<MMA, 256, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      case 128: return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      case 64: return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", tile);
-      }
-   } else {
-      switch (tile) {
-      case 256:
-#ifdef SOFIE_HIP_TUNING
-         if (variant >= 10 && variant < 18) {
-            switch (variant - 10) {
-            case 1: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 1>(stream, A, Bt, M, N, K, lda, ldb, ep);
-            case 2: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 2>(stream, A, Bt, M, N, K, lda, ldb, ep);
-            case 3: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 3>(stream, A, Bt, M, N, K, lda, ldb, ep);
-            case 4: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 4>(stream, A, Bt, M, N, K, lda, ldb, ep);
-            case 6: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 6>(stream, A, Bt, M, N, K, lda, ldb, ep);
-            default: break;
-            }
-         }
-#endif
-         if (variant == 1)
-            return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-         if (variant == 2)
-            return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 5, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-         return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      case 128:
-         if (variant == 1 || !k128)
-            return launch_mfma8_dma<MMA, 128, 128, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-         return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      case 64:
-         if (variant == 1 || !k128)
-            return launch_mfma8_dma<MMA, 64, 64, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-         return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
-      default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", tile);
-      }
-   }
-}
-
-} // namespace sofie_hip

@@ -1,0 +1,301 @@
+// Pipelined tile loop for the largest tile (256 x 256, 64-byte K slabs), where the LDS ring cannot hold
+// slabs of whole 128-byte cache lines: the slabs are loaded in PAIRS.  Slab 2p holds bytes [0,64) and slab
+// 2p+1 bytes [64,128) of the same cache line of every row; the two load instructions that fetch the two
+// halves of a line are issued back to back, so the vector L1 serves the second one and L2 is asked for
+// each line once (loading the halves a slab apart asks L2 twice: the measured L2 -> LDS rate is 13 TB/s
+// that way against 21 TB/s for whole lines).
+//
+// Ring of STAGES (odd) slab slots; slab s lives in slot s % STAGES.  Per pair p the loop runs slab 2p
+// (no loads issued) and slab 2p+1, during which the loads of pair p + (STAGES-1)/2 are issued, spread over
+// its K-steps, into the slots of slabs 2p-1 and 2p (both released by the barrier that ends slab 2p).
+// Everything else (operand roles, LDS layout, fragment double buffer, epilogue) is as in
+// mfma8_gemm_dma.hpp; the K-step index runs over the pair, so the fragment parity is a compile-time
+// constant for any number of K-steps per slab.
+#pragma once
+#include "mfma8_gemm_dma.hpp"
+
+namespace sofie_hip {
+
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(RowMajorRows A, RowMajorRows Bt, int M, int N,
+                                                                                 int K, EPI ep, int tiles_m, int tiles_n, int sw)
+{
+   constexpr int NW = WAVES_M * WAVES_N;
+   constexpr int CPR = BK / 16;
+   constexpr int RPI = 64 / CPR;
+   constexpr int A_LD = BM / RPI / NW, B_LD = BN / RPI / NW;
+   constexpr int LPT = A_LD + B_LD; // loads per lane and slab
+   constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
+   constexpr int MT = TM / 32, NT = TN / 32;
+   constexpr int KS = BK / MMA::KSTEP;
+   constexpr int STAGE_BYTES = (BM + BN) * BK;
+   constexpr int AHEAD = (STAGES - 1) / 2; // pairs between the one computing and the one being requested
+   static_assert(STAGES % 2 == 1 && STAGES >= 5, "an odd number of slots, at least five");
+   static_assert(BM % (RPI * NW) == 0 && BN % (RPI * NW) == 0, "tile rows must divide over the waves");
+   static_assert((STAGES - 1) * LPT < 64, "vmcnt counts fewer than 64 loads");
+   static_assert((2 * LPT) % KS == 0, "the loads of a pair must divide over the K-steps of a slab");
+   typedef typename MMA::acc_t acc_t;
+   typedef typename MMA::frag_t frag_t;
+
+   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+
+   int tm, tn;
+   tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, sw, tm, tn);
+   const int m0 = tm * BM, n0 = tn * BN;
+   const int t = threadIdx.x;
+   const int lane = t & 63;
+   const int wave = __builtin_amdgcn_readfirstlane(t >> 6); // uniform: keeps the LDS destinations of the loads in scalar registers
+   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+   const int lr = lane & 31, lk = lane >> 5;
+
+   // Source of every load instruction of a slab: a uniform base (tile origin + k offset, scalar registers)
+   // plus a 32-bit per-lane offset, so that the address needs no vector arithmetic inside the loop.
+   const int8_t *const a_tile = A.row(m0), *const b_tile = Bt.row(n0);
+   uint32_t oa[A_LD], ob[B_LD];
+#pragma unroll
+   for (int i = 0; i < A_LD; ++i) {
+      const int row = (i * NW + wave) * RPI + lane / CPR; // row of the tile this lane fills
+      constexpr int RPB = (256 / BK) > 0 ? (256 / BK) : 1;
+      const int c = (lane % CPR) ^ ((row / RPB) % CPR);   // logical chunk stored at this lane's LDS position
+      const int rc = (m0 + row < M) ? row : M - 1 - m0;   // rows past the edge re-read the last row
+      oa[i] = (uint32_t)rc * (uint32_t)A.ld + (uint32_t)(c * 16);
+   }
+#pragma unroll
+   for (int i = 0; i < B_LD; ++i) {
+      const int row = (i * NW + wave) * RPI + lane / CPR;
+      constexpr int RPB = (256 / BK) > 0 ? (256 / BK) : 1;
+      const int c = (lane % CPR) ^ ((row / RPB) % CPR);
+      const int rc = (n0 + row < N) ? row : N - 1 - n0;
+      ob[i] = (uint32_t)rc * (uint32_t)Bt.ld + (uint32_t)(c * 16);
+   }
+
+   // Loads [Q0, Q1) of the 2*LPT load instructions of pair `pair`: instruction q fetches row group q/2 of
+   // slab 2*pair + q%2, so the two halves of a cache line are requested by consecutive instructions.
+   auto issue_pair = [&](int pair, int slot0, int slot1, auto q0_c, auto q1_c) {
+      constexpr int Q0 = decltype(q0_c)::value, Q1 = decltype(q1_c)::value;
+      if (DBG & 1)
+         return;
+      const int koff = pair * 2 * BK;
+      static_for<Q1 - Q0>([&](auto qc) {
+         constexpr int q = Q0 + decltype(qc)::value;
+         constexpr int l = q / 2, half = q % 2;
+         int8_t *sA = smem + (half ? slot1 : slot0) * STAGE_BYTES;
+         int8_t *sB = sA + BM * BK;
+         if constexpr (l < A_LD)
+            __builtin_amdgcn_global_load_lds((global_void_t *)((a_tile + koff + half * BK) + oa[l]), (lds_void_t *)(sA + (l * NW + wave) * 1024), 16, 0, 0);
+         else
+            __builtin_amdgcn_global_load_lds((global_void_t *)((b_tile + koff + half * BK) + ob[l - A_LD]),
+                                             (lds_void_t *)(sB + ((l - A_LD) * NW + wave) * 1024), 16, 0, 0);
+      });
+   };
+
+   acc_t acc[MT][NT];
+#pragma unroll
+   for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+         for (int v = 0; v < 16; ++v)
+            acc[i][j][v] = 0;
+
+   // prologue: pairs 0 .. AHEAD-1 (a pair index past the end re-reads the last pair: filler that keeps the
+   // number of loads per iteration, and with it the vmcnt bookkeeping, constant)
+   const int KP = K / (2 * BK);
+#pragma unroll
+   for (int p = 0; p < AHEAD; ++p)
+      issue_pair(p < KP ? p : KP - 1, 2 * p, 2 * p + 1, std::integral_constant<int, 0>{}, std::integral_constant<int, 2 * LPT>{});
+
+   auto read_frags = [&](const int8_t *cA, const int8_t *cB, int ks, frag_t(&fa)[MT], frag_t(&fb)[NT]) {
+      if (DBG & 2)
+         return;
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+         for (int c = 0; c < MMA::CHUNKS; ++c)
+            fb[j].c[c] = *(const v4i *)(cB + lds_chunk_offset<BK>(wn * TN + j * 32 + lr, (ks * 2 + lk) * MMA::CHUNKS + c));
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+         for (int c = 0; c < MMA::CHUNKS; ++c)
+            fa[i].c[c] = *(const v4i *)(cA + lds_chunk_offset<BK>(wm * TM + i * 32 + lr, (ks * 2 + lk) * MMA::CHUNKS + c));
+   };
+
+   frag_t fa[2][MT], fb[2][NT];
+   wait_vmcnt<(AHEAD - 1) * 2 * LPT>(); // pair 0 has landed
+   __builtin_amdgcn_s_barrier();
+   read_frags(smem, smem + BM * BK, 0, fa[0], fb[0]);
+   int stage = 0;              // slot of the slab being computed
+   int lslot0 = STAGES - 1;    // slots the next requested pair goes to: those of slabs 2p-1 and 2p
+   int lslot1 = 0;
+   for (int kp = 0; kp < KP; ++kp) {
+      const int lpair = (kp + AHEAD < KP) ? kp + AHEAD : KP - 1;
+      static_for<2 * KS>([&](auto g_c) {
+         constexpr int g = decltype(g_c)::value; // K-step within the pair
+         constexpr int h = g / KS, ks = g % KS;
+         const int cur = (h == 0) ? stage : (stage + 1 == STAGES ? 0 : stage + 1);
+         const int8_t *cA = smem + cur * STAGE_BYTES;
+         const int8_t *cB = cA + BM * BK;
+         if (ks == KS - 1) {
+            const int nxt = (cur + 1 == STAGES) ? 0 : cur + 1;
+            if (h == 1) {
+               // issued so far, newest first: parts 0..KS-2 of pair kp+AHEAD, then pairs kp+AHEAD-1 ... kp+1.
+               // Pair kp+1 must have landed (its first slab is read next, its second one a slab later).
+               if (!(DBG & 8))
+                  wait_vmcnt<(AHEAD - 2) * 2 * LPT + (KS - 1) * (2 * LPT / KS)>();
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this wave's LDS reads of the current slab are complete
+            if (!(DBG & 16))
+               __builtin_amdgcn_s_barrier();
+            read_frags(smem + nxt * STAGE_BYTES, smem + nxt * STAGE_BYTES + BM * BK, 0, fa[(g + 1) & 1], fb[(g + 1) & 1]);
+         } else {
+            read_frags(cA, cB, ks + 1, fa[(g + 1) & 1], fb[(g + 1) & 1]);
+         }
+         constexpr int NLOAD = (h == 1) ? 2 * LPT / KS : 0;
+         if constexpr (h == 1)
+            issue_pair(lpair, lslot0, lslot1, std::integral_constant<int, ks * NLOAD>{}, std::integral_constant<int, (ks + 1) * NLOAD>{});
+#pragma unroll
+         for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+               if (!(DBG & 4))
+                  acc[i][j] = MMA::mma(fb[g & 1][j], fa[g & 1][i], acc[i][j]);
+               else
+                  acc[i][j][0] += fb[g & 1][j].c[0][0] + fa[g & 1][i].c[0][0];
+         // issue order within the step: MFMAs with the LDS reads and the loads slotted in between
+         constexpr int NMFMA = MT * NT;
+         constexpr int NREAD = (MT + NT) * MMA::CHUNKS;
+         constexpr int GROUPS = NLOAD > 0 ? NLOAD : 4;
+         constexpr int MPG = NMFMA / GROUPS > 0 ? NMFMA / GROUPS : 1;
+         constexpr int RPG = (NREAD + GROUPS - 1) / GROUPS;
+#pragma unroll
+         for (int gg = 0; gg < GROUPS; ++gg) {
+            constexpr int HALF = MPG / 2 > 0 ? MPG / 2 : 1;
+            __builtin_amdgcn_sched_group_barrier(0x008, HALF, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, RPG - RPG / 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, MPG - HALF, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, RPG / 2, 0);
+            if (NLOAD > 0)
+               __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+         }
+      });
+      stage = (stage + 2 >= STAGES) ? stage + 2 - STAGES : stage + 2;
+      lslot0 = (lslot0 + 2 >= STAGES) ? lslot0 + 2 - STAGES : lslot0 + 2;
+      lslot1 = (lslot1 + 2 >= STAGES) ? lslot1 + 2 - STAGES : lslot1 + 2;
+   }
+
+   wait_vmcnt<0>();
+   __syncthreads();
+   char *wsm = (char *)smem + wave * tile_store_lds_bytes(TN);
+   ep.dispatch([&](auto mode) {
+      tile_store_via_lds<decltype(mode)::value, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, M, N, lane, wsm);
+   });
+}
+
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0>
+static int launch_mfma8_pair(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb,
+                             const EPI &ep)
+{
+   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+   const long long nwg = (long long)tiles_m * tiles_n;
+   if (nwg > 0x7fffffffLL)
+      return fail(SOFIE_HIP_ERR_INVALID, "gemm: too many tiles");
+   if (K % (2 * BK) != 0 || K < 2 * BK)
+      return fail(SOFIE_HIP_ERR_INVALID, "gemm: the paired-slab kernel needs K to be a multiple of %d", 2 * BK);
+   constexpr size_t ring = (size_t)STAGES * (BM + BN) * BK;
+   constexpr size_t store = (size_t)WAVES_M * WAVES_N * tile_store_lds_bytes(BN / WAVES_N);
+   constexpr size_t smem = ring > store ? ring : store;
+   static_assert(smem <= 160 * 1024, "LDS ring larger than the CU's LDS");
+   constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
+   RowMajorRows a{A, lda}, b{Bt, ldb};
+   auto kern = mfma8_gemm_pair_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG>;
+   static bool configured[64] = {};
+   if (int st = configure_lds_once(kern, smem, configured))
+      return st;
+   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n, swizzle_mode());
+   return launch_status("mfma8_gemm_pair_kernel");
+}
+
+} // namespace sofie_hip
+
+namespace sofie_hip {
+
+// Chooses between the pipelined kernels (aligned operands, K a multiple of 64) and the general one.
+// `variant` selects a tuning alternative of the pipelined kernel (0 = default); -1 forces the general kernel.
+template <class MMA, class EPI>
+static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb,
+                             const EPI &ep, int force_tile, int variant)
+{
+   const bool aligned = (lda % 16 == 0) && (ldb % 16 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)Bt & 15) == 0);
+   if (variant < 0 || !aligned || K < 64 || K % 64 != 0)
+      return launch_mfma8_auto<MMA, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile);
+   const int tile = pick_tile(M, N, force_tile);
+   const bool k128 = (K % 128 == 0);
+   if constexpr (MMA::KSTEP * 2 > 64) {
+      // two K-steps per slab are the minimum: a 64-byte K-step needs 128-byte slabs
+      if (!k128)
+         return launch_mfma8_auto<MMA, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile);
+      switch (tile) {
+      case 256:
+         if (variant == 1)
+            return launch_mfma8_dma<MMA, 256, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      case 128: return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      case 64: return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", tile);
+      }
+   } else {
+      switch (tile) {
+      case 256:
+#ifdef SOFIE_HIP_TUNING
+         if (variant >= 10 && variant < 18) {
+            switch (variant - 10) {
+            case 1: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 1>(stream, A, Bt, M, N, K, lda, ldb, ep);
+            case 2: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 2>(stream, A, Bt, M, N, K, lda, ldb, ep);
+            case 3: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 3>(stream, A, Bt, M, N, K, lda, ldb, ep);
+            case 4: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 4>(stream, A, Bt, M, N, K, lda, ldb, ep);
+            case 6: return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI, 6>(stream, A, Bt, M, N, K, lda, ldb, ep);
+            default: break;
+            }
+         }
+         if (variant == 21)
+            return launch_mfma8_dma<MMA, 256, 128, 128, 2, 2, 3, EPI, 6>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 22)
+            return launch_mfma8_dma<MMA, 256, 128, 64, 2, 2, 4, EPI, 6>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 23)
+            return launch_mfma8_dma<MMA, 256, 128, 128, 2, 2, 3, EPI, 0>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 24)
+            return launch_mfma8_dma<MMA, 256, 128, 64, 2, 2, 4, EPI, 0>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 31)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 6>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 32)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 3>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 33)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 10>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 34)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 2>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 35)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 1>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 36)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 8>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 37)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 24>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 38)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 19>(stream, A, Bt, M, N, K, lda, ldb, ep);
+#endif
+         if (variant == 1 || !k128)
+            return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      case 128:
+         if (variant == 1 || !k128)
+            return launch_mfma8_dma<MMA, 128, 128, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      case 64:
+         if (variant == 1 || !k128)
+            return launch_mfma8_dma<MMA, 64, 64, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+      default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", tile);
+      }
+   }
+}
+
+} // namespace sofie_hip
