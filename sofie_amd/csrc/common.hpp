@@ -71,6 +71,19 @@ __device__ __forceinline__ int quantize_rne_sat8(float v)
    return (int)r;
 }
 
+// The same function for the GEMM store, where it runs once per output element: v_rndne_f32, then
+// v_cvt_i32_f32, which by itself saturates to the int32 range and turns NaN into 0, then an integer clamp
+// to [lo, 127] (lo = -128, or 0 when a relu follows: max(sat8(x), 0) == clamp(x, 0, 127)).
+__device__ __forceinline__ int quantize_rne_clamp(float v, int lo)
+{
+   const float r = __builtin_rintf(v);
+   int q;
+   asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(r));
+   int c;
+   asm("v_med3_i32 %0, %1, %2, %3" : "=v"(c) : "v"(q), "s"(lo), "v"(127)); // lo <= 127: the median is the clamp
+   return c;
+}
+
 // fp32 multiply that the compiler may not fuse with a neighbouring add.
 __device__ __forceinline__ float mul_nofma(float a, float b)
 {

@@ -182,6 +182,56 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
       ws_left -= wb;
    }
    const int OHW = g.OH * g.OW;
+   const int Cout_g = d->Cout / d->group;
+   const size_t esz = a->out == SOFIE_I8OUT_I8 ? 1 : 4;
+
+   // Implicit GEMM: the kernel reads the NHWC activations directly, one launch per group over the whole batch.
+   // Needs K slabs that lie inside one input pixel (channels per group a power of two >= 64) and 32-bit offsets.
+   {
+      const int ntaps = d->kh * d->kw;
+      const bool pow2 = (g.Cg & (g.Cg - 1)) == 0;
+      const long long xbytes = (long long)d->N * d->H * d->W * d->C;
+      const long long reach = xbytes + (long long)(d->pad_h0 + d->kh * d->dil_h + 1) * d->W * d->C + (long long)(d->pad_w0 + d->kw * d->dil_w + 1) * d->C;
+      const long long rows = (long long)d->N * OHW;
+      const int kw_recip = (65536 + d->kw - 1) / d->kw;
+      bool recip_ok = true;
+      for (int t = 0; t < ntaps; ++t)
+         recip_ok = recip_ok && (((t * kw_recip) >> 16) == t / d->kw);
+      const char *force = getenv("SOFIE_HIP_CONV_EXPLICIT");
+      const bool implicit = !(force && atoi(force)) && a->x_layout == SOFIE_LAYOUT_NHWC && pow2 && g.Cg >= 64 && ntaps <= 32 &&
+                            recip_ok && (d->C % 16 == 0) && (((uintptr_t)a->X & 15) == 0) && (((uintptr_t)Wp & 15) == 0) &&
+                            reach < (1LL << 31) && rows < (1LL << 31) && g.Kp == g.K;
+      if (implicit) {
+         int cg_shift = 0;
+         while ((1 << cg_shift) < g.Cg)
+            ++cg_shift;
+         for (int grp = 0; grp < d->group; ++grp) {
+            ConvRows src;
+            src.X = a->X + (size_t)grp * g.Cg;
+            src.H = d->H; src.W = d->W; src.C = d->C; src.OH = g.OH; src.OW = g.OW;
+            src.stride_h = d->stride_h; src.stride_w = d->stride_w; src.pad_h0 = d->pad_h0; src.pad_w0 = d->pad_w0;
+            src.dil_h = d->dil_h; src.dil_w = d->dil_w; src.kw = d->kw; src.ntaps = ntaps;
+            src.cg_shift = cg_shift; src.kw_recip = kw_recip;
+            I8Epilogue ep;
+            ep.bias = a->bias;
+            ep.scale = a->scale;
+            ep.scale_scalar = 1.0f;
+            ep.q_scale = 1.0f;
+            ep.relu_acc = (a->out == SOFIE_I8OUT_I32) ? a->relu : 0;
+            ep.relu_out = (a->out == SOFIE_I8OUT_I32) ? 0 : a->relu;
+            ep.out = a->out;
+            ep.ldy = d->Cout;
+            ep.N = Cout_g;
+            ep.n_offset = grp * Cout_g;
+            ep.nchw_ohw = (a->y_layout == SOFIE_LAYOUT_NHWC) ? 0 : OHW;
+            ep.Y = a->Y;
+            st = conv_i8_implicit(ctx->stream, src, g.Cg, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.K, ep, forced_i8_tile());
+            if (st)
+               return st;
+         }
+         return SOFIE_HIP_OK;
+      }
+   }
    const size_t per_image = (size_t)OHW * g.Kp;
    long long imgs_per_chunk = (long long)(ws_left / per_image);
    // keep one column matrix within reach of the 256 MB last-level cache
@@ -192,8 +242,6 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
       imgs_per_chunk = d->N;
    SOFIE_HIP_REQUIRE(imgs_per_chunk >= 1, "sofie_hip_conv_i8: workspace too small for one image");
    SOFIE_HIP_REQUIRE(imgs_per_chunk * OHW < (1LL << 31), "sofie_hip_conv_i8: too many rows per chunk");
-   const int Cout_g = d->Cout / d->group;
-   const size_t esz = a->out == SOFIE_I8OUT_I8 ? 1 : 4;
    const bool fast = a->x_layout == SOFIE_LAYOUT_NHWC && (g.Cg % 16 == 0) && (d->C % 16 == 0) && (((uintptr_t)a->X & 15) == 0);
 
    for (long long img0 = 0; img0 < d->N; img0 += imgs_per_chunk) {

@@ -116,8 +116,8 @@ __global__ __launch_bounds__(256) void gap_kernel(float *__restrict__ Y, const T
       Y[plane] = __fdiv_rn(mul_nofma((float)s, mul), (float)HW);
 }
 
-// NHWC int8 input: one workgroup per image; thread c (strided) sums channel c over the pixels, so
-// consecutive lanes read consecutive bytes.
+// NHWC int8 input, any channel count: one workgroup per image; thread c (strided) sums channel c over the
+// pixels, so consecutive lanes read consecutive bytes.
 __global__ __launch_bounds__(256) void gap_i8_nhwc_kernel(float *__restrict__ Y, const int8_t *__restrict__ X, int C, int HW,
                                                            float scale)
 {
@@ -127,6 +127,50 @@ __global__ __launch_bounds__(256) void gap_i8_nhwc_kernel(float *__restrict__ Y,
       for (int i = 0; i < HW; ++i)
          s += (int)p[(size_t)i * C + c];
       Y[(size_t)blockIdx.x * C + c] = __fdiv_rn(mul_nofma((float)s, scale), (float)HW);
+   }
+}
+
+// NHWC int8 input with C a multiple of 16 (and 16-byte aligned): one workgroup per (image, block of 256 channels).
+// A thread owns 16 consecutive channels and every (256 / chunks)-th pixel, reads 16 bytes per pixel, and the
+// per-thread int32 sums are added up through LDS (integer sums: exact in any order).
+__global__ __launch_bounds__(256) void gap_i8_nhwc_vec_kernel(float *__restrict__ Y, const int8_t *__restrict__ X, int C, int HW,
+                                                               float scale)
+{
+   __shared__ int part[256][17];
+   const int cblocks = (C + 255) / 256;
+   const int img = blockIdx.x / cblocks, cb = blockIdx.x % cblocks;
+   const int c_first = cb * 256;
+   const int chunks = ((C - c_first) < 256 ? (C - c_first) : 256) / 16; // 16-channel chunks in this block: 1..16
+   // threads beyond groups*chunks idle: the pixel groups must not overlap
+   const int groups = 256 / chunks;
+   const int chunk = threadIdx.x % chunks, group = threadIdx.x / chunks;
+   int s[16];
+#pragma unroll
+   for (int k = 0; k < 16; ++k)
+      s[k] = 0;
+   if (group < groups) {
+      const int8_t *p = X + (size_t)img * HW * C + c_first + chunk * 16;
+      for (int i = group; i < HW; i += groups) {
+         typedef int int4v __attribute__((ext_vector_type(4)));
+         const int4v v = *(const int4v *)(p + (size_t)i * C);
+#pragma unroll
+         for (int d = 0; d < 4; ++d)
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+               s[4 * d + b] += (int)(int8_t)(v[d] >> (8 * b));
+      }
+   }
+#pragma unroll
+   for (int k = 0; k < 16; ++k)
+      part[threadIdx.x][k] = s[k];
+   __syncthreads();
+   // thread t < chunks*16 finishes channel c_first + t: add the `groups` partial sums of that channel
+   if ((int)threadIdx.x < chunks * 16) {
+      const int ch = threadIdx.x / 16, k = threadIdx.x % 16;
+      int tot = 0;
+      for (int g = 0; g < groups; ++g)
+         tot += part[g * chunks + ch][k];
+      Y[(size_t)img * C + c_first + threadIdx.x] = __fdiv_rn(mul_nofma((float)tot, scale), (float)HW);
    }
 }
 
@@ -229,6 +273,11 @@ int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y, const int8_t *X, 
       return SOFIE_HIP_OK;
    SOFIE_HIP_REQUIRE(Y && X, "sofie_hip_global_avg_pool_i8: NULL pointer");
    if (x_layout == SOFIE_LAYOUT_NHWC) {
+      if (C % 16 == 0 && (((uintptr_t)X & 15) == 0) && (long long)N * ((C + 255) / 256) < 0x7fffffffLL) {
+         hipLaunchKernelGGL(gap_i8_nhwc_vec_kernel, dim3((unsigned)(N * ((C + 255) / 256))), dim3(256), 0, ctx->stream, Y, X, C, HW,
+                            scale);
+         return launch_status("gap_i8_nhwc_vec_kernel");
+      }
       hipLaunchKernelGGL(gap_i8_nhwc_kernel, dim3((unsigned)N), dim3(256), 0, ctx->stream, Y, X, C, HW, scale);
       return launch_status("gap_i8_nhwc_kernel");
    }

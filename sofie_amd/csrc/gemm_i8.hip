@@ -39,6 +39,18 @@ int gemm_i8_nt(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int
    return launch_mfma8_best<MfmaI8, I8Epilogue>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile, v ? atoi(v) : 0);
 }
 
+int conv_i8_implicit(hipStream_t stream, const ConvRows &src, int Cg, const int8_t *Wp, int M, int N, int K, I8Epilogue ep,
+                     int force_tile)
+{
+   const size_t esz = ep.out == SOFIE_I8OUT_I32 || ep.out == SOFIE_I8OUT_F32 ? 4 : 1;
+   ep.N = N;
+   ep.stage_ok = (ep.nchw_ohw == 0) && (((size_t)ep.ldy * esz) % 16 == 0) && (((size_t)ep.n_offset * esz) % 16 == 0) &&
+                 (((uintptr_t)ep.Y & 15) == 0);
+   ep.vec_param = (ep.n_offset % 4 == 0) && (!ep.bias || ((uintptr_t)ep.bias & 15) == 0) &&
+                  (!ep.scale || ((uintptr_t)ep.scale & 15) == 0);
+   return launch_mfma8_conv<I8Epilogue>(stream, src, Cg, Wp, M, N, K, ep, force_tile);
+}
+
 // SOFIE_HIP_I8_TILE=256|128|64 forces a tile configuration (tuning and tests); unset = heuristic.
 int forced_i8_tile()
 {
@@ -158,3 +170,11 @@ int sofie_hip_gemm_i8(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d)
 }
 
 } // extern "C"
+
+#ifdef SOFIE_HIP_TUNING
+// tuning builds only: per-workgroup timestamps of the paired-slab kernel (start, first slab landed, loop done, stored)
+extern "C" int sofie_hip_dbg_read_ts(unsigned long long *host, size_t n)
+{
+   return hipMemcpyFromSymbol(host, HIP_SYMBOL(sofie_hip::dbg_ts), n * sizeof(unsigned long long)) == hipSuccess ? 0 : 1;
+}
+#endif

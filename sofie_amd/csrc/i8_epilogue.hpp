@@ -58,13 +58,9 @@ struct I8Epilogue {
    template <int OUT>
    __device__ __forceinline__ int to_i8(int acc, float s) const
    {
-      if (OUT == SOFIE_I8OUT_I8) {
-         int q = quantize_rne_sat8(mul_nofma((float)acc, s));
-         if (relu_out)
-            q = q > 0 ? q : 0;
-         return q;
-      }
-      return quantize_rne_sat8(__fdiv_rn(mul_nofma((float)acc, s), q_scale));
+      if (OUT == SOFIE_I8OUT_I8)
+         return quantize_rne_clamp(mul_nofma((float)acc, s), relu_out ? 0 : -128);
+      return quantize_rne_clamp(__fdiv_rn(mul_nofma((float)acc, s), q_scale), -128);
    }
 
    // bias and scale of C consecutive columns
@@ -104,12 +100,12 @@ struct I8Epilogue {
    {
       int acc[4] = {a0, a1, a2, a3};
       float s[4];
+      const int acc_floor = relu_acc ? 0 : (int)0x80000000; // relu on the accumulator as one max
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
          acc[i] += p.b[4 * q + i];
          s[i] = p.s[4 * q + i];
-         if (relu_acc)
-            acc[i] = acc[i] > 0 ? acc[i] : 0;
+         acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
       }
       if (OUT == SOFIE_I8OUT_I32) {
 #pragma unroll
@@ -122,7 +118,10 @@ struct I8Epilogue {
       } else {
          const int q0 = to_i8<OUT>(acc[0], s[0]), q1 = to_i8<OUT>(acc[1], s[1]), q2 = to_i8<OUT>(acc[2], s[2]),
                    q3 = to_i8<OUT>(acc[3], s[3]);
-         w[0] = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) | ((uint32_t)(q3 & 0xff) << 24);
+         // low bytes of q0..q3 into one dword: three byte permutes
+         const uint32_t lo = __builtin_amdgcn_perm((uint32_t)q1, (uint32_t)q0, 0x0c0c0400u);
+         const uint32_t hi = __builtin_amdgcn_perm((uint32_t)q3, (uint32_t)q2, 0x0c0c0400u);
+         w[0] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
       }
    }
 };
@@ -131,5 +130,8 @@ struct I8Epilogue {
 int gemm_i8_nt(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep,
                int force_tile);
 int forced_i8_tile();
+// Convolution as an implicit GEMM: rows of A come from `src`, Wp is [N][K] with K = taps * Cg.
+int conv_i8_implicit(hipStream_t stream, const ConvRows &src, int Cg, const int8_t *Wp, int M, int N, int K, I8Epilogue ep,
+                     int force_tile);
 
 } // namespace sofie_hip

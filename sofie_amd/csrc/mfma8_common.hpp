@@ -106,10 +106,88 @@ __device__ __forceinline__ int lds_chunk_offset(int r, int c)
 }
 
 // Plain row-major operand: row r starts at base + r*ld.
+// The pipelined kernels address an operand through three hooks, so that the A operand can also be a
+// convolution input that is never laid out as a matrix (ConvRows below):
+//   lane_state<LD>            what a lane keeps per load instruction of a slab
+//   init(st, i, m0, row, cbyte, M)   load i of this lane fills tile row `row` with the 16 bytes at slab offset cbyte
+//   load_ptr(st, i, koff)     global address of those bytes for the slab that starts at reduction offset koff
 struct RowMajorRows {
    const int8_t *base;
    int ld;
    __device__ __forceinline__ const int8_t *row(int r) const { return base + (size_t)r * (size_t)ld; }
+
+   template <int LD>
+   struct lane_state {
+      const int8_t *tile; // uniform: first row of the tile
+      uint32_t off[LD];
+   };
+   template <int LD>
+   __device__ __forceinline__ void init(lane_state<LD> &st, int i, int m0, int row, int cbyte, int M) const
+   {
+      st.tile = this->row(m0);
+      const int rc = (m0 + row < M) ? row : M - 1 - m0; // rows past the edge re-read the last row
+      st.off[i] = (uint32_t)rc * (uint32_t)ld + (uint32_t)cbyte;
+   }
+   template <int LD>
+   __device__ __forceinline__ const int8_t *load_ptr(const lane_state<LD> &st, int i, int koff) const
+   {
+      return (st.tile + koff) + st.off[i];
+   }
+};
+
+// 256 zero bytes: what a load of a padded (out-of-image) position reads.
+static __device__ __attribute__((aligned(256))) int8_t conv_zero_page[256] = {};
+
+// A operand of a convolution computed as one GEMM over the whole batch, read straight from the NHWC
+// activation tensor: GEMM row m is the output pixel (n, oh, ow), the reduction index is
+// k = (tap kh_i*kw + kw_i) * Cg + channel, so a K slab of BK <= Cg bytes is BK consecutive channels of ONE input pixel.
+// Positions outside the image read zeros.  Needs Cg (channels per group) to be a power of two >= BK.
+struct ConvRows {
+   const int8_t *X;       // NHWC, first channel of the group
+   int H, W, C;           // C = channel stride of a pixel (all groups)
+   int OH, OW;
+   int stride_h, stride_w, pad_h0, pad_w0, dil_h, dil_w;
+   int kw, ntaps;
+   int cg_shift;          // log2(Cg)
+   int kw_recip;          // ceil(65536 / kw): tap / kw == (tap * kw_recip) >> 16 for every tap < ntaps (checked on the host)
+
+   template <int LD>
+   struct lane_state {
+      int32_t off[LD];   // byte offset of (n, oh*stride - pad, ow*stride - pad, cbyte) from X; may be negative
+      uint32_t mask[LD]; // bit t: tap t of this output pixel lies inside the image
+   };
+   template <int LD>
+   __device__ __forceinline__ void init(lane_state<LD> &st, int i, int m0, int row, int cbyte, int M) const
+   {
+      const int m = m0 + row;
+      uint32_t mask = 0;
+      int32_t off = 0;
+      if (m < M) {
+         const int ohw = OH * OW;
+         const int n = m / ohw, r = m - n * ohw;
+         const int oh = r / OW, ow = r - oh * OW;
+         const int ih0 = oh * stride_h - pad_h0, iw0 = ow * stride_w - pad_w0;
+         off = ((n * H + ih0) * W + iw0) * C + cbyte;
+         for (int t = 0; t < ntaps; ++t) {
+            const int khi = t / kw, kwi = t - khi * kw;
+            const int ih = ih0 + khi * dil_h, iw = iw0 + kwi * dil_w;
+            if (ih >= 0 && ih < H && iw >= 0 && iw < W)
+               mask |= 1u << t;
+         }
+      }
+      st.off[i] = off;
+      st.mask[i] = mask;
+   }
+   template <int LD>
+   __device__ __forceinline__ const int8_t *load_ptr(const lane_state<LD> &st, int i, int koff) const
+   {
+      const int tap = koff >> cg_shift;            // uniform
+      const int cbyte = koff & ((1 << cg_shift) - 1);
+      const int khi = (tap * kw_recip) >> 16, kwi = tap - khi * kw;
+      const int toff = (khi * dil_h * W + kwi * dil_w) * C + cbyte;
+      const int8_t *p = X + (ptrdiff_t)(st.off[i] + toff);
+      return ((st.mask[i] >> tap) & 1u) ? p : (const int8_t *)conv_zero_page;
+   }
 };
 
 // LDS bytes one wave needs for the tile store below (TN = columns of the wave tile).
@@ -117,101 +195,111 @@ constexpr int tile_store_lds_bytes(int TN) { return 32 * (TN * 4 + 16); }
 
 // Tile store through LDS.  After the MFMAs a lane holds, per register group, 4 consecutive columns of
 // ONE row, and the 32 lanes of a half-wave hold 32 different rows; stored directly, a wave instruction
-// would touch 64 rows with 4..16 bytes each.  Instead, for each 32-row block of its tile, a wave parks the
-// raw 32-bit accumulators in its own LDS region (row stride TN*4+16 bytes: 16-byte aligned and spread
-// over the banks) and re-reads them row by row in a run-time loop, so that a lane converts and stores 16
-// consecutive output bytes and a wave instruction writes whole 128-byte lines.  Only the parking code is
-// unrolled over the accumulator registers; the conversion exists once per output mode, which keeps the
-// kernel small enough for the instruction cache.
+// would touch 64 rows with 4..16 bytes each.  Instead, for each 32-row block of its tile, a wave
+//   1. converts its accumulators in registers (straight-line code, one pack4 per register group: bias,
+//      scale, rounding, activation, narrowing), which leaves 4 output elements = 4, 8 or 16 bytes,
+//   2. parks those bytes in its own LDS region, laid out as the output rows (row stride TN*ESZ+16 bytes),
+//   3. re-reads the region 16 bytes per lane, a row being covered by consecutive lanes, and stores: a wave
+//      instruction then writes whole 128-byte lines.
+// Converting before the transposition keeps the LDS traffic at the size of the OUTPUT (a quarter of the
+// accumulators for 1-byte outputs) and leaves nothing but a copy in the run-time loop of step 3.
 //
 // EPI provides
 //   template <class F> void dispatch(F f) const     f(std::integral_constant<int, MODE>{}) for the output mode
 //   template <int MODE> static constexpr int out_bytes()          bytes of one output element (1, 2, 4)
 //   struct col_params<C>; template <int C> void load_params(int n, col_params<C> &p) const
-//                                per-column constants (bias, scale) of columns n..n+C-1, clamped to N-1;
-//                                a lane's columns are the same for every row it stores, so they are fetched once
+//                                per-column constants (bias, scale) of columns n..n+C-1, clamped to N-1
 //   template <int MODE, int C> void pack4(const col_params<C> &p, int q, T a0, T a1, T a2, T a3, uint32_t *w) const
-//                                converts columns 4q..4q+3 of the lane's C columns into 4*out_bytes bytes
+//                                converts columns 4q..4q+3 of the C columns into 4*out_bytes bytes
 //   bool rows_vectorizable() const                row-major output whose rows allow 16-byte stores
 //   char *out_base() const;  size_t out_index(int m, int n) const     element index of (m,n)
 template <int MODE, int MT, int NT, class EPI, class ACC>
 __device__ __forceinline__ void tile_store_via_lds(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int M, int N,
                                                    int lane, char *wsm)
 {
-   typedef typename std::remove_reference<decltype(acc[0][0][0])>::type elem_t;
    constexpr int ESZ = EPI::template out_bytes<MODE>();
    constexpr int TN = NT * 32;
-   constexpr int ROWB = TN * 4 + 16;
+   constexpr int ROWB = TN * ESZ + 16; // 16-byte aligned rows, consecutive rows shifted over the banks
+   constexpr int QW = ESZ;             // dwords produced per group of 4 columns
    const int lr = lane & 31, lk = lane >> 5;
    char *out = ep.out_base();
    const bool vec = ep.rows_vectorizable();
+
+   // the lane's columns are the same in every 32-row block: their constants are fetched once
+   typename EPI::template col_params<4> prm[NT][4];
+   static_for<NT>([&](auto cj) {
+      constexpr int j = decltype(cj)::value;
+      static_for<4>([&](auto cg) {
+         constexpr int g = decltype(cg)::value;
+         const int n = n_base + j * 32 + g * 8 + lk * 4;
+         ep.template load_params<4>(n < N ? n : N - 1, prm[j][g]);
+      });
+   });
+
    static_for<MT>([&](auto ci) {
       constexpr int i = decltype(ci)::value;
       static_for<NT>([&](auto cj) {
          constexpr int j = decltype(cj)::value;
          static_for<4>([&](auto cg) {
             constexpr int g = decltype(cg)::value;
-            typedef elem_t v4e __attribute__((ext_vector_type(4)));
-            *(v4e *)(wsm + lr * ROWB + (j * 32 + g * 8 + lk * 4) * 4) =
-               v4e{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+            uint32_t w[QW];
+            ep.template pack4<MODE, 4>(prm[j][g], 0, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                                       acc[i][j][4 * g + 3], w);
+            char *dst = wsm + lr * ROWB + (j * 32 + g * 8 + lk * 4) * ESZ;
+            if constexpr (QW == 1)
+               *(uint32_t *)dst = w[0];
+            else if constexpr (QW == 2)
+               *(uint2 *)dst = make_uint2(w[0], w[1]);
+            else
+               *(uint4 *)dst = make_uint4(w[0], w[1], w[2], w[3]);
          });
       });
       __builtin_amdgcn_wave_barrier();
       const int m_first = m_base + i * 32;
       if (vec) {
-         constexpr int CPL = 16 / ESZ;     // columns per lane
-         constexpr int LPR = TN / CPL;     // lanes per row
-         constexpr int RPP = 64 / LPR;     // rows per pass
+         constexpr int CPL = 16 / ESZ;          // columns per lane
+         constexpr int LPR = TN / CPL;          // lanes per row
+         constexpr int RPP = 64 / LPR;          // rows per pass
          static_assert(TN % CPL == 0 && LPR <= 64 && 32 % RPP == 0, "wave tile width not supported by the tile store");
          const int c0 = (lane % LPR) * CPL;
          const int n = n_base + c0;
-         typename EPI::template col_params<CPL> prm;
-         ep.template load_params<CPL>(n < N ? n : N - 1, prm);
-#pragma unroll 1
+#pragma unroll 2
          for (int row0 = 0; row0 < 32; row0 += RPP) {
             const int row = row0 + lane / LPR;
             const int m = m_first + row;
+            const uint4 v = *(const uint4 *)(wsm + row * ROWB + c0 * ESZ);
             if (m < M && n < N) {
-               uint32_t w[4];
-#pragma unroll
-               for (int q = 0; q < CPL / 4; ++q) {
-                  typedef elem_t v4e __attribute__((ext_vector_type(4)));
-                  const v4e a = *(const v4e *)(wsm + row * ROWB + (c0 + 4 * q) * 4);
-                  ep.template pack4<MODE, CPL>(prm, q, a[0], a[1], a[2], a[3], w + q * ESZ);
-               }
                char *y = out + ep.out_index(m, n) * ESZ;
                if (n + CPL <= N) {
-                  *(uint4 *)y = make_uint4(w[0], w[1], w[2], w[3]);
+                  *(uint4 *)y = v;
                } else {
-                  const char *src = (const char *)w;
+                  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
                   for (int b = 0; b < (N - n) * ESZ; ++b)
-                     y[b] = src[b];
+                     y[b] = (char)(w[b >> 2] >> ((b & 3) * 8));
                }
             }
          }
       } else {
-         // any layout: a lane converts 4 columns and stores them one element at a time
+         // any layout: a lane takes 4 columns of a row and stores them one element at a time
          constexpr int LPR = TN / 4;
          constexpr int RPP = (64 / LPR) > 0 ? (64 / LPR) : 1;
          static_assert(LPR <= 64, "wave tile too wide");
          const int c0 = (lane % LPR) * 4;
          const int n = n_base + c0;
-         typename EPI::template col_params<4> prm;
-         ep.template load_params<4>(n < N ? n : N - 1, prm);
 #pragma unroll 1
          for (int row0 = 0; row0 < 32; row0 += RPP) {
             const int row = row0 + lane / LPR;
             const int m = m_first + row;
             if (m < M && n < N) {
-               typedef elem_t v4e __attribute__((ext_vector_type(4)));
-               const v4e a = *(const v4e *)(wsm + row * ROWB + c0 * 4);
-               uint32_t w[4];
-               ep.template pack4<MODE, 4>(prm, 0, a[0], a[1], a[2], a[3], w);
-               const char *src = (const char *)w;
+               const char *src = wsm + row * ROWB + c0 * ESZ;
                for (int e = 0; e < 4 && n + e < N; ++e) {
                   char *y = out + ep.out_index(m, n + e) * ESZ;
-                  for (int b = 0; b < ESZ; ++b)
-                     y[b] = src[e * ESZ + b];
+                  if constexpr (ESZ == 1)
+                     y[0] = src[e];
+                  else if constexpr (ESZ == 2)
+                     *(uint16_t *)y = *(const uint16_t *)(src + 2 * e);
+                  else
+                     *(uint32_t *)y = *(const uint32_t *)(src + 4 * e);
                }
             }
          }

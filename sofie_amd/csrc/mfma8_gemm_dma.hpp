@@ -26,8 +26,8 @@ __device__ __forceinline__ void wait_vmcnt()
    __builtin_amdgcn_s_waitcnt((N & 0xf) | ((N >> 4) << 14) | (0x7 << 4) | (0xf << 8));
 }
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(RowMajorRows A, RowMajorRows Bt, int M, int N,
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(ASRC A, RowMajorRows Bt, int M, int N,
                                                                                 int K, EPI ep, int tiles_m, int tiles_n, int sw)
 {
    constexpr int NW = WAVES_M * WAVES_N;
@@ -56,25 +56,23 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(R
    const int lr = lane & 31, lk = lane >> 5;
 
    // per-lane global source of every load instruction of a slab (k offset added per slab)
-   // Source of every load instruction of a slab: a uniform base (tile origin + k offset, scalar registers)
-   // plus a 32-bit per-lane offset, so that the address needs no vector arithmetic inside the loop.
-   const int8_t *const a_tile = A.row(m0), *const b_tile = Bt.row(n0);
-   uint32_t oa[A_LD], ob[B_LD];
+   // Source of every load instruction of a slab: a uniform part (tile origin + k offset, scalar registers)
+   // plus a 32-bit per-lane offset, so that the address needs (almost) no vector arithmetic inside the loop.
+   typename ASRC::template lane_state<A_LD> as;
+   typename RowMajorRows::template lane_state<B_LD> bs;
 #pragma unroll
    for (int i = 0; i < A_LD; ++i) {
       const int row = (i * NW + wave) * RPI + lane / CPR; // row of the tile this lane fills
       constexpr int RPB = (256 / BK) > 0 ? (256 / BK) : 1;
       const int c = (lane % CPR) ^ ((row / RPB) % CPR);   // logical chunk stored at this lane's LDS position
-      const int rc = (m0 + row < M) ? row : M - 1 - m0;   // rows past the edge re-read the last row
-      oa[i] = (uint32_t)rc * (uint32_t)A.ld + (uint32_t)(c * 16);
+      A.template init<A_LD>(as, i, m0, row, c * 16, M);
    }
 #pragma unroll
    for (int i = 0; i < B_LD; ++i) {
       const int row = (i * NW + wave) * RPI + lane / CPR;
       constexpr int RPB = (256 / BK) > 0 ? (256 / BK) : 1;
       const int c = (lane % CPR) ^ ((row / RPB) % CPR);
-      const int rc = (n0 + row < N) ? row : N - 1 - n0;
-      ob[i] = (uint32_t)rc * (uint32_t)Bt.ld + (uint32_t)(c * 16);
+      Bt.template init<B_LD>(bs, i, n0, row, c * 16, N);
    }
    // One K-step's share of a slab's load instructions (A's first, then Bt's): part `part` of KS equal parts.
    constexpr int KS_ = BK / MMA::KSTEP;
@@ -90,9 +88,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(R
       static_for<L1 - L0>([&](auto lc) {
          constexpr int l = L0 + decltype(lc)::value;
          if constexpr (l < A_LD)
-            __builtin_amdgcn_global_load_lds((global_void_t *)((a_tile + koff) + oa[l]), (lds_void_t *)(sA + (l * NW + wave) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_void_t *)A.template load_ptr<A_LD>(as, l, koff), (lds_void_t *)(sA + (l * NW + wave) * 1024), 16, 0, 0);
          else
-            __builtin_amdgcn_global_load_lds((global_void_t *)((b_tile + koff) + ob[l - A_LD]), (lds_void_t *)(sB + ((l - A_LD) * NW + wave) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_void_t *)Bt.template load_ptr<B_LD>(bs, l - A_LD, koff), (lds_void_t *)(sB + ((l - A_LD) * NW + wave) * 1024), 16, 0, 0);
       });
    };
 
@@ -199,8 +197,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(R
    });
 }
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0>
-static int launch_mfma8_dma(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb,
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows>
+static int launch_mfma8_dma_src(hipStream_t stream, const ASRC &a, const int8_t *Bt, int M, int N, int K, int ldb,
                             const EPI &ep)
 {
    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -214,13 +212,20 @@ static int launch_mfma8_dma(hipStream_t stream, const int8_t *A, const int8_t *B
    constexpr size_t smem = ring > store ? ring : store;
    static_assert(smem <= 160 * 1024, "LDS ring larger than the CU's LDS");
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
-   RowMajorRows a{A, lda}, b{Bt, ldb};
-   auto kern = mfma8_gemm_dma_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG>;
+   RowMajorRows b{Bt, ldb};
+   auto kern = mfma8_gemm_dma_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG, ASRC>;
    static bool configured[64] = {};
    if (int st = configure_lds_once(kern, smem, configured))
       return st;
    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n, swizzle_mode());
    return launch_status("mfma8_gemm_dma_kernel");
+}
+
+
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0>
+static int launch_mfma8_dma(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
+{
+   return launch_mfma8_dma_src<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG, RowMajorRows>(stream, RowMajorRows{A, lda}, Bt, M, N, K, ldb, ep);
 }
 
 } // namespace sofie_hip

@@ -16,8 +16,19 @@
 
 namespace sofie_hip {
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(RowMajorRows A, RowMajorRows Bt, int M, int N,
+#ifdef SOFIE_HIP_TUNING
+static __device__ unsigned long long dbg_ts[8192 * 4];
+#define SOFIE_TS(slot)                                                                              \
+   do {                                                                                             \
+      if (threadIdx.x == 0 && blockIdx.x < 8192)                                                    \
+         dbg_ts[blockIdx.x * 4 + (slot)] = wall_clock64();                                          \
+   } while (0)
+#else
+#define SOFIE_TS(slot) ((void)0)
+#endif
+
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(ASRC A, RowMajorRows Bt, int M, int N,
                                                                                  int K, EPI ep, int tiles_m, int tiles_n, int sw)
 {
    constexpr int NW = WAVES_M * WAVES_N;
@@ -39,6 +50,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
 
    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
 
+   SOFIE_TS(0);
    int tm, tn;
    tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, sw, tm, tn);
    const int m0 = tm * BM, n0 = tn * BN;
@@ -48,25 +60,23 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
    const int lr = lane & 31, lk = lane >> 5;
 
-   // Source of every load instruction of a slab: a uniform base (tile origin + k offset, scalar registers)
-   // plus a 32-bit per-lane offset, so that the address needs no vector arithmetic inside the loop.
-   const int8_t *const a_tile = A.row(m0), *const b_tile = Bt.row(n0);
-   uint32_t oa[A_LD], ob[B_LD];
+   // Source of every load instruction of a slab: a uniform part (tile origin + k offset, scalar registers)
+   // plus a 32-bit per-lane offset, so that the address needs (almost) no vector arithmetic inside the loop.
+   typename ASRC::template lane_state<A_LD> as;
+   typename RowMajorRows::template lane_state<B_LD> bs;
 #pragma unroll
    for (int i = 0; i < A_LD; ++i) {
       const int row = (i * NW + wave) * RPI + lane / CPR; // row of the tile this lane fills
       constexpr int RPB = (256 / BK) > 0 ? (256 / BK) : 1;
       const int c = (lane % CPR) ^ ((row / RPB) % CPR);   // logical chunk stored at this lane's LDS position
-      const int rc = (m0 + row < M) ? row : M - 1 - m0;   // rows past the edge re-read the last row
-      oa[i] = (uint32_t)rc * (uint32_t)A.ld + (uint32_t)(c * 16);
+      A.template init<A_LD>(as, i, m0, row, c * 16, M);
    }
 #pragma unroll
    for (int i = 0; i < B_LD; ++i) {
       const int row = (i * NW + wave) * RPI + lane / CPR;
       constexpr int RPB = (256 / BK) > 0 ? (256 / BK) : 1;
       const int c = (lane % CPR) ^ ((row / RPB) % CPR);
-      const int rc = (n0 + row < N) ? row : N - 1 - n0;
-      ob[i] = (uint32_t)rc * (uint32_t)Bt.ld + (uint32_t)(c * 16);
+      Bt.template init<B_LD>(bs, i, n0, row, c * 16, N);
    }
 
    // Loads [Q0, Q1) of the 2*LPT load instructions of pair `pair`: instruction q fetches row group q/2 of
@@ -82,9 +92,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
          int8_t *sA = smem + (half ? slot1 : slot0) * STAGE_BYTES;
          int8_t *sB = sA + BM * BK;
          if constexpr (l < A_LD)
-            __builtin_amdgcn_global_load_lds((global_void_t *)((a_tile + koff + half * BK) + oa[l]), (lds_void_t *)(sA + (l * NW + wave) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_void_t *)A.template load_ptr<A_LD>(as, l, koff + half * BK), (lds_void_t *)(sA + (l * NW + wave) * 1024), 16, 0, 0);
          else
-            __builtin_amdgcn_global_load_lds((global_void_t *)((b_tile + koff + half * BK) + ob[l - A_LD]),
+            __builtin_amdgcn_global_load_lds((global_void_t *)Bt.template load_ptr<B_LD>(bs, l - A_LD, koff + half * BK),
                                              (lds_void_t *)(sB + ((l - A_LD) * NW + wave) * 1024), 16, 0, 0);
       });
    };
@@ -123,6 +133,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
    frag_t fa[2][MT], fb[2][NT];
    wait_vmcnt<(AHEAD - 1) * 2 * LPT>(); // pair 0 has landed
    __builtin_amdgcn_s_barrier();
+   SOFIE_TS(1);
    read_frags(smem, smem + BM * BK, 0, fa[0], fb[0]);
    int stage = 0;              // slot of the slab being computed
    int lslot0 = STAGES - 1;    // slots the next requested pair goes to: those of slabs 2p-1 and 2p
@@ -185,14 +196,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
 
    wait_vmcnt<0>();
    __syncthreads();
+   SOFIE_TS(2);
    char *wsm = (char *)smem + wave * tile_store_lds_bytes(TN);
    ep.dispatch([&](auto mode) {
       tile_store_via_lds<decltype(mode)::value, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, M, N, lane, wsm);
    });
+   SOFIE_TS(3);
 }
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0>
-static int launch_mfma8_pair(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb,
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows>
+static int launch_mfma8_pair_src(hipStream_t stream, const ASRC &a, const int8_t *Bt, int M, int N, int K, int ldb,
                              const EPI &ep)
 {
    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -206,13 +219,20 @@ static int launch_mfma8_pair(hipStream_t stream, const int8_t *A, const int8_t *
    constexpr size_t smem = ring > store ? ring : store;
    static_assert(smem <= 160 * 1024, "LDS ring larger than the CU's LDS");
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
-   RowMajorRows a{A, lda}, b{Bt, ldb};
-   auto kern = mfma8_gemm_pair_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG>;
+   RowMajorRows b{Bt, ldb};
+   auto kern = mfma8_gemm_pair_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG, ASRC>;
    static bool configured[64] = {};
    if (int st = configure_lds_once(kern, smem, configured))
       return st;
    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n, swizzle_mode());
    return launch_status("mfma8_gemm_pair_kernel");
+}
+
+
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0>
+static int launch_mfma8_pair(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
+{
+   return launch_mfma8_pair_src<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG, RowMajorRows>(stream, RowMajorRows{A, lda}, Bt, M, N, K, ldb, ep);
 }
 
 } // namespace sofie_hip
@@ -295,6 +315,37 @@ static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *
          return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
       default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", tile);
       }
+   }
+}
+
+} // namespace sofie_hip
+
+namespace sofie_hip {
+
+// Convolution as one implicit GEMM: A is read through ConvRows (BK = 64 must divide the channels per group),
+// Wp is the packed weight [N][K] with K = taps * Cg.  Tile choice as for the GEMM, plus a 256 x 128 tile for
+// layers with at most 128 output channels.
+template <class EPI>
+static int launch_mfma8_conv(hipStream_t stream, const ConvRows &a, int Cg, const int8_t *Wp, int M, int N, int K, const EPI &ep,
+                             int force_tile)
+{
+   auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+   const bool pairs = (Cg % 128 == 0);
+   int tile = force_tile;
+   if (!tile)
+      tile = (N > 128 && tiles(256, 256) >= 256) ? 256 : (N > 64 && tiles(256, 128) >= 256) ? 257 : (tiles(128, 128) >= 192) ? 128 : 64;
+   switch (tile) {
+   case 256:
+      if (pairs)
+         return launch_mfma8_pair_src<MfmaI8, 256, 256, 64, 2, 2, 5, EPI, 0, ConvRows>(stream, a, Wp, M, N, K, K, ep);
+      return launch_mfma8_dma_src<MfmaI8, 256, 256, 64, 2, 2, 4, EPI, 0, ConvRows>(stream, a, Wp, M, N, K, K, ep);
+   case 257:
+      if (pairs)
+         return launch_mfma8_pair_src<MfmaI8, 256, 128, 64, 2, 2, 5, EPI, 0, ConvRows>(stream, a, Wp, M, N, K, K, ep);
+      return launch_mfma8_dma_src<MfmaI8, 256, 128, 64, 2, 2, 4, EPI, 0, ConvRows>(stream, a, Wp, M, N, K, K, ep);
+   case 128: return launch_mfma8_dma_src<MfmaI8, 128, 128, 64, 2, 2, 4, EPI, 0, ConvRows>(stream, a, Wp, M, N, K, K, ep);
+   case 64: return launch_mfma8_dma_src<MfmaI8, 64, 64, 64, 2, 2, 4, EPI, 0, ConvRows>(stream, a, Wp, M, N, K, K, ep);
+   default: return fail(SOFIE_HIP_ERR_INVALID, "conv: unknown tile %d", force_tile);
    }
 }
 

@@ -84,8 +84,8 @@ def test_conv_i8_output_kinds(rt, out, relu):
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
 
 
-def test_global_avg_pool_i8_both_layouts(rt):
-    N, Cc, H, W = 3, 20, 5, 7
+@pytest.mark.parametrize("N,Cc,H,W", [(3, 20, 5, 7), (3, 48, 5, 7), (2, 272, 4, 4), (4, 256, 9, 9), (1, 80, 33, 3)])
+def test_global_avg_pool_i8_both_layouts(rt, N, Cc, H, W):
     X = util.int8_sym(70, N * Cc * H * W).reshape(N, Cc, H, W)
     want = ob.global_avg_pool_i8(X, np.float32(0.031))
     for layout in (0, 1):
@@ -95,3 +95,29 @@ def test_global_avg_pool_i8_both_layouts(rt):
         rt.call("sofie_hip_global_avg_pool_i8", util.ptr(dY), util.ptr(dX), N, Cc, H * W, layout, C.c_float(0.031))
         rt.sync()
         assert np.array_equal(util.to_host(dY).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("tile", [256, 257, 128, 64])
+@pytest.mark.parametrize("case", [
+    (2, 128, 12, 12, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),      # paired-slab kernels (channels % 128 == 0)
+    (3, 64, 11, 9, 96, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),         # 64-byte slabs, ragged Cout
+    (2, 128, 10, 10, 64, 3, 2, (2, 0, 1, 1), (2, 1), (1, 2), 2),       # groups, stride, dilation, asymmetric pads
+    (1, 64, 7, 7, 32, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1), 1),          # 1x1
+])
+def test_conv_i8_implicit_gemm_every_tile(rt, case, tile, monkeypatch):
+    """NHWC input with a power-of-two channel count >= 64 takes the implicit-GEMM kernels (no column matrix)."""
+    monkeypatch.setenv("SOFIE_HIP_I8_TILE", str(tile))
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    X = util.int8_sym(80, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.int8_sym(81, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
+    bias = util.int32_range(82, Cout, -2000, 2000)
+    K = (Cc // group) * kh * kw
+    scale = ((0.5 + util.uniform01(83, Cout)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    want = ob.conv_i8(X, Wt, bias, scale, pads=pads, strides=strides, dils=dils, group=group, relu=1, out=2, omp=True)
+    got = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, R.LAYOUT_NHWC, R.LAYOUT_NHWC, 1)
+    assert np.array_equal(got, want)
+    # and the explicit column-matrix path gives the same bits
+    monkeypatch.setenv("SOFIE_HIP_CONV_EXPLICIT", "1")
+    monkeypatch.delenv("SOFIE_HIP_I8_TILE")
+    got2 = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, R.LAYOUT_NHWC, R.LAYOUT_NCHW, 1)
+    assert np.array_equal(got2, want)
