@@ -150,15 +150,27 @@ __global__ __launch_bounds__(256) void gap_i8_nhwc_vec_kernel(float *__restrict_
       s[k] = 0;
    if (group < groups) {
       const int8_t *p = X + (size_t)img * HW * C + c_first + chunk * 16;
-      for (int i = group; i < HW; i += groups) {
-         typedef int int4v __attribute__((ext_vector_type(4)));
-         const int4v v = *(const int4v *)(p + (size_t)i * C);
+      typedef int int4v __attribute__((ext_vector_type(4)));
+      auto add16 = [&](const int4v &v) {
 #pragma unroll
          for (int d = 0; d < 4; ++d)
 #pragma unroll
             for (int b = 0; b < 4; ++b)
                s[4 * d + b] += (int)(int8_t)(v[d] >> (8 * b));
+      };
+      int i = group;
+      // eight pixels per round: eight independent 16-byte loads in flight per lane
+      for (; i + 7 * groups < HW; i += 8 * groups) {
+         int4v v[8];
+#pragma unroll
+         for (int u = 0; u < 8; ++u)
+            v[u] = *(const int4v *)(p + (size_t)(i + u * groups) * C);
+#pragma unroll
+         for (int u = 0; u < 8; ++u)
+            add16(v[u]);
       }
+      for (; i < HW; i += groups)
+         add16(*(const int4v *)(p + (size_t)i * C));
    }
 #pragma unroll
    for (int k = 0; k < 16; ++k)

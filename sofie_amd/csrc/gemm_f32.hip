@@ -4,6 +4,7 @@
 // The operand fetch is a functor, so the same tile loop serves a strided/transposed Gemm and a
 // convolution whose column matrix is gathered on the fly (no materialised im2col).
 #include "common.hpp"
+#include <cstdlib>
 
 namespace sofie_hip {
 
@@ -122,6 +123,117 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmOperandA la, GemmOper
    }
 }
 
+// Small products (the fp32 MLP at batch 64 has 64x128, 64x64 and 64x10 outputs): the 64x64 tiles above would
+// occupy a handful of CUs and spend their time waiting for one 16-wide K slab after another.  Here a
+// workgroup is ONE wave that owns an 8x8 tile, one output per lane, so even these products spread over
+// more than a hundred CUs.  K is walked in chunks of 256: the 8 rows of op(A) and the 8 columns of op(B)
+// are staged in LDS with K contiguous (row pitch 260 floats: the 8 rows a wave reads at once fall into
+// different banks), the next chunk's loads are issued before the current chunk is consumed, and a lane
+// reads 4 K values of its row and its column per step into four partial sums (k mod 4), added at the end.
+constexpr int SK_T = 8, SK_KC = 256, SK_PITCH = SK_KC + 4;
+
+template <bool VEC_A, bool VEC_B>
+__global__ __launch_bounds__(64) void gemm_f32_skinny_kernel(GemmOperandA la, GemmOperandB lb, int M, int N, int K, float *Y,
+                                                              long long ldy, F32Epilogue ep, long long strideA, long long strideB,
+                                                              long long strideC, long long strideY)
+{
+   __shared__ __attribute__((aligned(16))) float sA[2][SK_T][SK_PITCH];
+   __shared__ __attribute__((aligned(16))) float sB[2][SK_T][SK_PITCH];
+   const int b = blockIdx.z;
+   la.p += b * strideA;
+   lb.p += b * strideB;
+   if (ep.C)
+      ep.C += b * strideC;
+   Y += b * strideY;
+   const int lane = threadIdx.x;
+   const int tm = lane >> 3, tn = lane & 7;
+   const int m0 = blockIdx.x * SK_T, n0 = blockIdx.y * SK_T;
+
+   // staging registers of one chunk: row i of the tile, K values 4*lane..4*lane+3 (vector form), or
+   // element lane + 64*j of the 8x256 block (scalar form, any strides)
+   float4 ra[SK_T], rb[SK_T];
+   float qa[VEC_A ? 1 : 32], qb[VEC_B ? 1 : 32];
+   auto fetch = [&](int k0) {
+      if (VEC_A) {
+#pragma unroll
+         for (int i = 0; i < SK_T; ++i) {
+            const int m = m0 + i, k = k0 + lane * 4;
+            ra[i] = (m < M && k < K) ? *(const float4 *)(la.p + m * la.sm + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+         }
+      } else {
+#pragma unroll
+         for (int j = 0; j < 32; ++j) {
+            const int id = lane + 64 * j, row = id & 7, kk = id >> 3; // rows fastest: a transposed operand is contiguous there
+            const int m = m0 + row, k = k0 + kk;
+            qa[j] = (m < M && k < K) ? la(m, k) : 0.0f;
+         }
+      }
+      if (VEC_B) {
+#pragma unroll
+         for (int i = 0; i < SK_T; ++i) {
+            const int n = n0 + i, k = k0 + lane * 4;
+            rb[i] = (n < N && k < K) ? *(const float4 *)(lb.p + n * lb.sn + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+         }
+      } else {
+#pragma unroll
+         for (int j = 0; j < 32; ++j) {
+            const int id = lane + 64 * j, row = id & 7, kk = id >> 3;
+            const int n = n0 + row, k = k0 + kk;
+            qb[j] = (n < N && k < K) ? lb(k, n) : 0.0f;
+         }
+      }
+   };
+   auto stage = [&](int buf) {
+      if (VEC_A) {
+#pragma unroll
+         for (int i = 0; i < SK_T; ++i)
+            *(float4 *)&sA[buf][i][lane * 4] = ra[i];
+      } else {
+#pragma unroll
+         for (int j = 0; j < 32; ++j) {
+            const int id = lane + 64 * j;
+            sA[buf][id & 7][id >> 3] = qa[j];
+         }
+      }
+      if (VEC_B) {
+#pragma unroll
+         for (int i = 0; i < SK_T; ++i)
+            *(float4 *)&sB[buf][i][lane * 4] = rb[i];
+      } else {
+#pragma unroll
+         for (int j = 0; j < 32; ++j) {
+            const int id = lane + 64 * j;
+            sB[buf][id & 7][id >> 3] = qb[j];
+         }
+      }
+   };
+
+   float acc4[4] = {0.0f, 0.0f, 0.0f, 0.0f}; // k = 0,1,2,3 (mod 4): four independent FMA chains, added at the end
+   fetch(0);
+   int buf = 0;
+   for (int k0 = 0; k0 < K; k0 += SK_KC) {
+      stage(buf);
+      if (k0 + SK_KC < K)
+         fetch(k0 + SK_KC); // in flight while this chunk is consumed
+      __builtin_amdgcn_wave_barrier();
+      const int kc = (K - k0) < SK_KC ? (K - k0) : SK_KC;
+#pragma unroll 4
+      for (int kk = 0; kk < kc; kk += 4) {
+         const float4 a = *(const float4 *)&sA[buf][tm][kk];
+         const float4 c = *(const float4 *)&sB[buf][tn][kk];
+         acc4[0] = fmaf(a.x, c.x, acc4[0]);
+         acc4[1] = fmaf(a.y, c.y, acc4[1]);
+         acc4[2] = fmaf(a.z, c.z, acc4[2]);
+         acc4[3] = fmaf(a.w, c.w, acc4[3]);
+      }
+      buf ^= 1;
+   }
+   const float acc = (acc4[0] + acc4[1]) + (acc4[2] + acc4[3]);
+   const int m = m0 + tm, n = n0 + tn;
+   if (m < M && n < N)
+      Y[m * ldy + n] = f32_epilogue(ep, acc, m, n);
+}
+
 // Column-matrix element (row m = (image, oh, ow), column k = (ci, kh, kw)) gathered from NCHW input;
 // the same index arithmetic as the reference's Im2col, zero outside the image.
 struct ConvOperandA {
@@ -213,6 +325,28 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d)
    ep.act_alpha = d->act_alpha;
    const unsigned gy = (M + F32_BM - 1) / F32_BM, gx = (N + F32_BN - 1) / F32_BN;
    SOFIE_HIP_REQUIRE(gx <= 65535 && d->batch <= 65535, "sofie_hip_gemm_f32: N or batch too large for one launch");
+   // few 64x64 tiles: one-wave workgroups with 8x8 tiles reach every CU (SOFIE_HIP_F32_SKINNY=0/1 overrides)
+   const char *force = getenv("SOFIE_HIP_F32_SKINNY");
+   const bool skinny = force ? atoi(force) != 0 : ((long long)gy * gx * d->batch < 192);
+   if (skinny && K > 0 && (N + SK_T - 1) / SK_T <= 65535) {
+      auto aligned16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
+      const bool va = !d->transA && K % 4 == 0 && lda % 4 == 0 && aligned16(d->A) && d->strideA % 4 == 0;
+      const bool vb = d->transB && K % 4 == 0 && ldb % 4 == 0 && aligned16(d->B) && d->strideB % 4 == 0;
+      const dim3 grid((M + SK_T - 1) / SK_T, (N + SK_T - 1) / SK_T, (unsigned)d->batch);
+#define SOFIE_SKINNY(VA, VB)                                                                                              \
+   hipLaunchKernelGGL((gemm_f32_skinny_kernel<VA, VB>), grid, dim3(64), 0, ctx->stream, la, lb, M, N, K, d->Y, ldy, ep,   \
+                      (long long)d->strideA, (long long)d->strideB, (long long)d->strideC, (long long)d->strideY)
+      if (va && vb)
+         SOFIE_SKINNY(true, true);
+      else if (va)
+         SOFIE_SKINNY(true, false);
+      else if (vb)
+         SOFIE_SKINNY(false, true);
+      else
+         SOFIE_SKINNY(false, false);
+#undef SOFIE_SKINNY
+      return launch_status("gemm_f32_skinny_kernel");
+   }
    hipLaunchKernelGGL(gemm_f32_kernel, dim3(gy, gx, (unsigned)d->batch), dim3(256), 0, ctx->stream, la, lb, M, N, K, d->Y, ldy, ep,
                       (long long)d->strideA, (long long)d->strideB, (long long)d->strideC, (long long)d->strideY);
    return launch_status("gemm_f32_kernel");

@@ -205,9 +205,10 @@ inline int pick_tile(int M, int N, int force_tile)
    if (force_tile)
       return force_tile;
    auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-   if (tiles(256, 256) >= 256)
+   // a tile wider than the matrix would spend its matrix-core time on columns that do not exist
+   if (N > 128 && tiles(256, 256) >= 256)
       return 256;
-   if (tiles(128, 128) >= 192)
+   if (N > 64 && tiles(128, 128) >= 192)
       return 128;
    return 64;
 }

@@ -323,8 +323,7 @@ static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *
 namespace sofie_hip {
 
 // Convolution as one implicit GEMM: A is read through ConvRows (BK = 64 must divide the channels per group),
-// Wp is the packed weight [N][K] with K = taps * Cg.  Tile choice as for the GEMM, plus a 256 x 128 tile for
-// layers with at most 128 output channels.
+// Wp is the packed weight [N][K] with K = taps * Cg.
 template <class EPI>
 static int launch_mfma8_conv(hipStream_t stream, const ConvRows &a, int Cg, const int8_t *Wp, int M, int N, int K, const EPI &ep,
                              int force_tile)
@@ -333,7 +332,10 @@ static int launch_mfma8_conv(hipStream_t stream, const ConvRows &a, int Cg, cons
    const bool pairs = (Cg % 128 == 0);
    int tile = force_tile;
    if (!tile)
-      tile = (N > 128 && tiles(256, 256) >= 256) ? 256 : (N > 64 && tiles(256, 128) >= 256) ? 257 : (tiles(128, 128) >= 192) ? 128 : 64;
+      // Short reductions (a 3x3 convolution over 64 or 128 channels) spend as long in the tile store as in the K loop:
+      // 128 x 128 tiles leave room for two workgroups per CU, so one's store overlaps the other's MFMAs.
+      // 257 = the 256 x 128 tile, by request only.
+      tile = (N > 128 && K > 1536 && tiles(256, 256) >= 256) ? 256 : (N > 64 && tiles(128, 128) >= 192) ? 128 : 64;
    switch (tile) {
    case 256:
       if (pairs)

@@ -39,9 +39,12 @@ def close(got, want, mag, rel=1e-5):
 
 
 @pytest.mark.parametrize("M,N,K,transA,transB", [(64, 128, 784, 0, 1), (64, 64, 128, 0, 1), (64, 10, 64, 0, 1), (16, 50, 100, 0, 0),
-                                                 (7, 5, 3, 1, 0), (65, 67, 33, 1, 1), (1, 1, 1, 0, 0), (130, 70, 257, 0, 0)])
+                                                 (7, 5, 3, 1, 0), (65, 67, 33, 1, 1), (1, 1, 1, 0, 0), (130, 70, 257, 0, 0), (9, 17, 520, 0, 1), (12, 20, 600, 1, 0)])
 @pytest.mark.parametrize("bias_mode,act", [(0, 0), (1, 1), (2, 0), (3, 2), (4, 3), (1, 4)])
-def test_gemm_f32_matches_sofie_cpu_semantics(rt, M, N, K, transA, transB, bias_mode, act):
+@pytest.mark.parametrize("kernel", ["tiles64", "wave8x8"])
+def test_gemm_f32_matches_sofie_cpu_semantics(rt, M, N, K, transA, transB, bias_mode, act, kernel, monkeypatch):
+    # both fp32 kernels on every shape: the 64x64-tile one and the one-wave 8x8-tile one for small products
+    monkeypatch.setenv("SOFIE_HIP_F32_SKINNY", "1" if kernel == "wave8x8" else "0")
     A = util.normal(1, M * K).reshape((K, M) if transA else (M, K))
     B = util.normal(2, N * K, 0.05).reshape((N, K) if transB else (K, N))
     Cshape = {0: None, 1: (N,), 2: (M, 1), 3: (1,), 4: (M, N)}[bias_mode]
