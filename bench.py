@@ -22,6 +22,10 @@ import numpy as np
 
 INT8_PEAK = 5.0e15  # MI355X dense int8 MFMA peak, op/s
 HBM_PEAK = 8.0e12
+# HBM bytes per launch of the dominant kernel (average of the layer-1 and layer-2 launches), from the FETCH_SIZE and
+# WRITE_SIZE counters of this same workload, each scaled by what the counter reads for a 256 MiB copy
+# (profiles/mfma8_gemm_dma_128x128_int8_mlp_batch1024.md): (15542 KiB * 2.000 + 4096 KiB * 1.000) * 1024
+DOMINANT_KERNEL_TRAFFIC_BYTES = 36024320
 
 
 def build_mlp():
@@ -87,6 +91,140 @@ def gemm_sweep(rt, sizes, reps=20, warmup=3):
     return out
 
 
+def fp8_sweep(rt, sizes, reps=20, warmup=3):
+    """Stand-alone FP8 e4m3 GEMM, fp32 accumulate, per-tensor scale, bias + GELU, bf16 output (BASELINE config 4)."""
+    from sofie_amd import runtime as R
+    from tests import util
+    import torch
+    out = []
+    for n in sizes:
+        M = N = K = n
+        g = torch.Generator(device="cuda")
+        g.manual_seed(4000 + n)
+        Af = torch.randn((M, K), generator=g, device="cuda", dtype=torch.float32)
+        Bf = torch.randn((N, K), generator=g, device="cuda", dtype=torch.float32)
+        A, Bt = util.dev_empty((M, K), np.uint8), util.dev_empty((N, K), np.uint8)
+        bias = util.to_dev(util.normal(4003, N))
+        Y = util.dev_empty((M, N), np.uint16)
+        torch.cuda.synchronize()
+        s = 4.0 / 448.0  # N(0,1) scaled into the e4m3 range: 4 sigma -> 448
+        rt.call("sofie_hip_quantize_fp8", util.ptr(A), util.ptr(Af), C.c_size_t(M * K), C.c_float(s))
+        rt.call("sofie_hip_quantize_fp8", util.ptr(Bt), util.ptr(Bf), C.c_size_t(N * K), C.c_float(s))
+        rt.sync()
+        del Af, Bf
+        d = R.GemmFp8Desc()
+        d.M, d.N, d.K, d.transB = M, N, K, 1
+        d.A, d.B, d.bias, d.Y = util.ptr(A), util.ptr(Bt), util.ptr(bias), util.ptr(Y)
+        d.scale, d.act, d.out = s * s, R.ACT_GELU, 0
+        fn = lambda: rt.call("sofie_hip_gemm_fp8", C.byref(d))
+        for _ in range(warmup):
+            fn()
+        best = None
+        for _ in range(3):
+            ms, _ = time_region(rt, fn, reps)
+            best = ms if best is None else min(best, ms)
+        t = best / reps * 1e-3
+        ops = 2.0 * M * N * K
+        out.append({"M": M, "N": N, "K": K, "ms": round(t * 1e3, 5), "tflops": round(ops / t / 1e12, 2),
+                    "frac_of_fp8_peak": round(ops / t / INT8_PEAK, 4)})
+        del A, Bt, Y
+        torch.cuda.empty_cache()
+    return out
+
+
+def fp32_mlp_leg(steps=200):
+    """BASELINE config 1: fp32 Gemm+Relu chain 784 -> 128 -> 64 -> 10 at batch 64, three fused launches; next to the CPU
+    restatement of the reference's generated code on the same batch."""
+    from sofie_amd import Runtime, runtime as R
+    from oracle import binding as ob
+    from tests import util
+    dims, batch = [784, 128, 64, 10], 64
+    rt = Runtime(0)
+    x = util.uniform01(2001, batch * 784).reshape(batch, 784)
+    ws = [util.normal(1001 + l, dims[l + 1] * dims[l], 0.05).reshape(dims[l + 1], dims[l]) for l in range(3)]
+    bs = [np.zeros(dims[l + 1], np.float32) for l in range(3)]
+    X = util.to_dev(x)
+    W, B = [util.to_dev(w) for w in ws], [util.to_dev(b) for b in bs]
+    H = [util.dev_empty((batch, dims[l + 1]), np.float32) for l in range(3)]
+    import torch
+    torch.cuda.synchronize()
+    descs, src = [], X
+    for l in range(3):
+        d = R.GemmF32Desc()
+        d.M, d.N, d.K, d.transB, d.alpha, d.beta = batch, dims[l + 1], dims[l], 1, 1.0, 1.0
+        d.A, d.B, d.C, d.Y = util.ptr(src), util.ptr(W[l]), util.ptr(B[l]), util.ptr(H[l])
+        d.bias_mode, d.act, d.batch = R.BIAS_ROW, (R.ACT_RELU if l < 2 else R.ACT_NONE), 1
+        descs.append(d)
+        src = H[l]
+
+    def step():
+        for d in descs:
+            rt.call("sofie_hip_gemm_f32", C.byref(d))
+    for _ in range(10):
+        step()
+    ms, _ = time_region(rt, step, steps)
+    got = util.to_host(H[2])
+    rt.close()
+    t0 = time.perf_counter()
+    reps = 20
+    for _ in range(reps):
+        h = x
+        for l in range(3):
+            h = ob.gemm_f32(h, ws[l], bs[l], M=batch, N=dims[l + 1], K=dims[l], transB=1, bias_mode=1, act=(1 if l < 2 else 0))
+    cpu_s = (time.perf_counter() - t0) / reps
+    err = float(np.abs(got - h).max() / max(1.0, np.abs(h).max()))
+    return {"us_per_batch": round(ms / steps * 1e3, 2), "inferences_per_s": round(batch / (ms / steps * 1e-3), 0),
+            "algorithmic_bytes": 641000, "hbm_gbps_algorithmic": round(641000 / (ms / steps * 1e-3) / 1e9, 1),
+            "max_rel_err_vs_oracle": err, "cpu_oracle_us_per_batch_1_core": round(cpu_s * 1e6, 1)}
+
+
+def int8_cnn_leg(steps=10):
+    """BASELINE config 5: 4 x [Conv3x3 s1 p1 + folded BatchNorm + Relu] 3->64->128->256->256 on 64x64 images, batch 256,
+    global average pool, Gemm 256->10; int8 weights, per-channel scales."""
+    from sofie_amd import Runtime
+    from sofie_amd.session import Int8CNNSession
+    from tests.refmodels import make_int8_cnn
+    batch = 256
+    m = make_int8_cnn(batch, 64)
+    rt = Runtime(0)
+    s = Int8CNNSession(rt, m["batch"], m["in_shape"], m["in_scale"], m["convs"], m["last_scale"], m["fc_w"], m["fc_b"])
+    s.upload_input(m["x"])
+    rt.sync()
+    for _ in range(3):
+        s.infer_nosync()
+    ms, _ = time_region(rt, s.infer_nosync, steps)
+    rt.close()
+    ops = 2.0 * batch * 64 * 64 * sum(cv["W"].size for cv in m["convs"])
+    t = ms / steps * 1e-3
+    return {"ms_per_batch": round(t * 1e3, 4), "images_per_s": round(batch / t, 0), "tops": round(ops / t / 1e12, 1),
+            "frac_of_int8_peak": round(ops / t / INT8_PEAK, 4)}
+
+
+def two_stream_leg(weights, w_scales, in_scales, batch, x, steps=200):
+    """The same MLP as two independent Sessions on two streams, batches enqueued alternately: the gaps between the
+    dependent launches of one inference are filled by the other's kernels."""
+    from sofie_amd import Runtime
+    from sofie_amd.session import Int8MLPSession
+    rts = [Runtime(0), Runtime(0)]
+    sess = [Int8MLPSession(rt, weights, w_scales, in_scales, batch) for rt in rts]
+    for s in sess:
+        s.upload_input(x)
+    for _ in range(10):
+        for s in sess:
+            s.infer_nosync()
+    for rt in rts:
+        rt.sync()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        sess[i & 1].infer_nosync()
+    for rt in rts:
+        rt.sync()
+    dt = time.perf_counter() - t0
+    for rt in rts:
+        rt.close()
+    return {"us_per_batch": round(dt / steps * 1e6, 2), "inferences_per_s": round(batch * steps / dt, 0)}
+
+
 def cpu_baseline(x, weights, w_scales, in_scales, rows):
     from oracle import binding as ob
     from tests.refmodels import int8_mlp_oracle
@@ -108,6 +246,9 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=64)
     ap.add_argument("--no-sweep", action="store_true", help="skip the stand-alone GEMM sweep (profiling runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three 256 MiB device-to-device copies: a kernel of known traffic that scales the FETCH_SIZE / "
+                         "WRITE_SIZE counters of a profiling run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (the path is data-parallel over the batch; "
@@ -168,7 +309,22 @@ def main():
         parity = bool(np.array_equal(y[:args.cpu_rows].view(np.uint32), ref.view(np.uint32)))
 
     sweep = [] if args.no_sweep else gemm_sweep(rt, [1024, 4096, 8192])
+    f8 = [] if args.no_sweep else fp8_sweep(rt, [1024, 4096, 8192])
+    if args.calibrate_copy:
+        nbytes = 256 << 20
+        src = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        dst = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        for _ in range(3):
+            rt.call("sofie_hip_copy", C.c_void_p(dst.data_ptr()), C.c_void_p(src.data_ptr()), C.c_size_t(nbytes))
+        rt.sync()
+        del src, dst
     rt.close()
+    extra = {}
+    if not args.no_sweep:
+        extra["fp32_mlp_batch64"] = fp32_mlp_leg()
+        extra["int8_cnn_batch256"] = int8_cnn_leg()
+        extra["int8_mlp_two_sessions_two_streams"] = two_stream_leg(weights, w_scales, in_scales, batch, x)
 
     algo_bytes = sum(w.size for w in weights) + 4 * batch * dims[0] + 4 * batch * dims[-1]
     line = {
@@ -183,11 +339,12 @@ def main():
                    "mlp_tops": round(ops_per_inference_batch / (ms_per_step * 1e-3) / 1e12, 2),
                    "mlp_algorithmic_bytes": algo_bytes,
                    "int8_mfma_register_only_tops": probe,
-                   "gemm_sweep_int8_requant_bias_relu": sweep},
+                   "gemm_sweep_int8_requant_bias_relu": sweep,
+                   "gemm_sweep_fp8_bias_gelu_bf16": f8, **extra},
         "roofline": {"bound": "mfma", "achieved": round(achieved / 1e12, 2), "peak": INT8_PEAK / 1e12, "unit": "TFLOP/s",
-                     "frac": round(achieved / INT8_PEAK, 4), "traffic": None,
+                     "frac": round(achieved / INT8_PEAK, 4), "traffic": DOMINANT_KERNEL_TRAFFIC_BYTES,
                      "frac_of_sustained_random_operand_rate": round(achieved / 1e12 / probe["random_operands"], 4),
-                     "kernel": "mfma8_gemm_dma_kernel<MfmaI8, 128, 128, ...> (layers 1 and 2 of the MLP: 2 launches per inference, "
+                     "kernel": "mfma8_gemm_dma_kernel<MfmaI8, 128, 128, 128, 2, 2, 3, ...> (layers 1 and 2 of the MLP: 2 launches per inference, "
                                "avg %.2f us, %.3e int8 op per launch on average)" % (avg_launch_s * 1e6, ops_per_launch)},
         "cpu_baseline": cpu,
     }
