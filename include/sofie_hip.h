@@ -236,8 +236,11 @@ int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float
  * Activations are NCHW (the ONNX layout) or NHWC (channels fastest), chosen per tensor: a chain of
  * convolutions keeps NHWC between its layers.  W is the ONNX weight [Cout, C/group, kh, kw], or, with
  * w_is_packed, the re-laid-out form sofie_hip_pack_conv_weight_i8 writes once at Session construction
- * (the role of tensor_<Y>_f in the reference, ROperator_Conv.hxx:456-476).  The workspace holds the
- * packed weights (unless w_is_packed) and the column matrix of as many images as fit (at least one). */
+ * (the role of tensor_<Y>_f in the reference, ROperator_Conv.hxx:456-476).  NHWC input whose channels
+ * per group are a power of two >= 64 (and at most 32 filter taps) is read directly by the GEMM kernel
+ * (implicit GEMM, no column matrix); any other case gathers a column matrix first.  The workspace holds
+ * the packed weights (unless w_is_packed) and, when a column matrix is needed, that of as many images as
+ * fit (at least one); sofie_hip_conv_i8_workspace returns the minimum, which may be 0. */
 enum { SOFIE_LAYOUT_NCHW = 0, SOFIE_LAYOUT_NHWC = 1 };
 typedef struct sofie_conv_i8_args {
    const int8_t *X;

@@ -137,13 +137,34 @@ int sofie_hip_pack_conv_weight_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, 
    return launch_status("pack_conv_weight_kernel");
 }
 
+// Shapes the implicit-GEMM kernels take (pointer alignment is checked at the call): NHWC input, channels per
+// group a power of two >= 64 (a 64-byte K slab then lies inside one input pixel), at most 32 filter taps,
+// 32-bit byte offsets.
+static bool conv_i8_implicit_shape(const sofie_conv_desc *d, int x_layout)
+{
+   if (d->group <= 0 || d->C % d->group != 0)
+      return false;
+   const int Cg = d->C / d->group, ntaps = d->kh * d->kw;
+   const long long xbytes = (long long)d->N * d->H * d->W * d->C;
+   const long long reach = xbytes + (long long)(d->pad_h0 + d->kh * d->dil_h + 1) * d->W * d->C + (long long)(d->pad_w0 + d->kw * d->dil_w + 1) * d->C;
+   const long long rows = (long long)d->N * d->OH * d->OW;
+   const int kw_recip = (65536 + d->kw - 1) / d->kw;
+   for (int t = 0; t < ntaps && t < 32; ++t)
+      if (((t * kw_recip) >> 16) != t / d->kw)
+         return false;
+   const char *force = getenv("SOFIE_HIP_CONV_EXPLICIT");
+   return !(force && atoi(force)) && x_layout == SOFIE_LAYOUT_NHWC && (Cg & (Cg - 1)) == 0 && Cg >= 64 && ntaps <= 32 &&
+          d->C % 16 == 0 && reach < (1LL << 31) && rows < (1LL << 31);
+}
+
 size_t sofie_hip_conv_i8_workspace(const sofie_conv_desc *d, const sofie_conv_i8_args *a)
 {
    if (!d || !a || d->group <= 0)
       return 0;
    size_t K = (size_t)(d->C / d->group) * d->kh * d->kw;
    size_t Kp = (K + 15) & ~(size_t)15;
-   size_t need = round256((size_t)d->OH * d->OW * Kp); // the column matrix of one image
+   // the column matrix of one image, unless the kernel reads the activations directly
+   size_t need = conv_i8_implicit_shape(d, a->x_layout) ? 0 : round256((size_t)d->OH * d->OW * Kp);
    if (!a->w_is_packed)
       need += sofie_hip_conv_weight_i8_packed_bytes(d);
    return need;
@@ -166,7 +187,8 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
       return SOFIE_HIP_OK;
    SOFIE_HIP_REQUIRE(a->X && a->W && a->Y, "sofie_hip_conv_i8: NULL tensor pointer");
    const size_t need = sofie_hip_conv_i8_workspace(d, a);
-   SOFIE_HIP_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, "sofie_hip_conv_i8: a workspace of at least %zu bytes is needed", need);
+   SOFIE_HIP_REQUIRE(need == 0 || (a->workspace != nullptr && a->workspace_bytes >= need),
+                     "sofie_hip_conv_i8: a workspace of at least %zu bytes is needed", need);
    SOFIE_HIP_REQUIRE(((uintptr_t)a->workspace & 255) == 0, "sofie_hip_conv_i8: workspace must be 256-byte aligned");
 
    char *ws = (char *)a->workspace;
@@ -189,18 +211,10 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
    // Needs K slabs that lie inside one input pixel (channels per group a power of two >= 64) and 32-bit offsets.
    {
       const int ntaps = d->kh * d->kw;
-      const bool pow2 = (g.Cg & (g.Cg - 1)) == 0;
-      const long long xbytes = (long long)d->N * d->H * d->W * d->C;
-      const long long reach = xbytes + (long long)(d->pad_h0 + d->kh * d->dil_h + 1) * d->W * d->C + (long long)(d->pad_w0 + d->kw * d->dil_w + 1) * d->C;
-      const long long rows = (long long)d->N * OHW;
       const int kw_recip = (65536 + d->kw - 1) / d->kw;
-      bool recip_ok = true;
-      for (int t = 0; t < ntaps; ++t)
-         recip_ok = recip_ok && (((t * kw_recip) >> 16) == t / d->kw);
-      const char *force = getenv("SOFIE_HIP_CONV_EXPLICIT");
-      const bool implicit = !(force && atoi(force)) && a->x_layout == SOFIE_LAYOUT_NHWC && pow2 && g.Cg >= 64 && ntaps <= 32 &&
-                            recip_ok && (d->C % 16 == 0) && (((uintptr_t)a->X & 15) == 0) && (((uintptr_t)Wp & 15) == 0) &&
-                            reach < (1LL << 31) && rows < (1LL << 31) && g.Kp == g.K;
+      const long long rows = (long long)d->N * OHW;
+      const bool implicit = conv_i8_implicit_shape(d, a->x_layout) && (((uintptr_t)a->X & 15) == 0) && (((uintptr_t)Wp & 15) == 0) &&
+                            g.Kp == g.K;
       if (implicit) {
          int cg_shift = 0;
          while ((1 << cg_shift) < g.Cg)
@@ -233,6 +247,9 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
       }
    }
    const size_t per_image = (size_t)OHW * g.Kp;
+   SOFIE_HIP_REQUIRE(ws != nullptr && ws_left >= per_image,
+                     "sofie_hip_conv_i8: the activations are not 16-byte aligned; a workspace of %zu bytes is needed for the column matrix",
+                     per_image);
    long long imgs_per_chunk = (long long)(ws_left / per_image);
    // keep one column matrix within reach of the 256 MB last-level cache
    const long long cap = (long long)((192u << 20) / per_image);

@@ -181,11 +181,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
 #pragma unroll
          for (int gg = 0; gg < GROUPS; ++gg) {
             constexpr int HALF = MPG / 2 > 0 ? MPG / 2 : 1;
+            if (NLOAD > 0 && !(DBG & (64 | 128)))
+               __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, HALF, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, RPG - RPG / 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, MPG - HALF, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, RPG / 2, 0);
-            if (NLOAD > 0)
+            if (NLOAD > 0 && (DBG & 64))
                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
          }
       });
@@ -299,6 +301,10 @@ static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *
             return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 8>(stream, A, Bt, M, N, K, lda, ldb, ep);
          if (variant == 37)
             return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 24>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 41)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 64>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 42)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 128>(stream, A, Bt, M, N, K, lda, ldb, ep);
          if (variant == 38)
             return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 19>(stream, A, Bt, M, N, K, lda, ldb, ep);
 #endif

@@ -48,6 +48,17 @@ public:
    void UpdateInitializedTensor(const std::string &name, ETensorType type, std::vector<std::size_t> shape, std::shared_ptr<void> data);
    // a float scalar initializer (scales of the quantised operators); throws if it is not one
    float GetScalarInitializer(const std::string &name) const;
+   // storage order of a 4-D activation: kLayoutNCHW (what ONNX defines, the default) or kLayoutNHWC (kept
+   // between quantised convolutions); set by the producing operator's Initialize
+   void SetTensorLayout(const std::string &name, int layout) { fTensorLayout[UTILITY::Clean_name(name)] = layout; }
+   int GetTensorLayout(const std::string &name) const
+   {
+      auto f = fTensorLayout.find(UTILITY::Clean_name(name));
+      return f == fTensorLayout.end() ? kLayoutNCHW : f->second;
+   }
+   bool IsOutputTensor(const std::string &name) const;
+   // kinds of the operators that read `name` (after fusion)
+   std::vector<OperatorKind> ConsumerKinds(const std::string &name) const;
    const std::string &GetName() const { return fName; }
    const std::vector<std::unique_ptr<ROperator>> &Operators() const { return fOperators; }
 
@@ -88,6 +99,7 @@ private:
    std::vector<std::unique_ptr<ROperator>> fOperators;
    std::vector<PlannedTensor> fPlan;
    std::unordered_map<std::string, std::size_t> fOffsets;
+   std::unordered_map<std::string, int> fTensorLayout;
    std::size_t fArenaBytes = 0, fPoolBytes = 0;
    bool fInitialized = false;
    std::string fGC;

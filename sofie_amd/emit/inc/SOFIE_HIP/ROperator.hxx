@@ -11,7 +11,8 @@ namespace SOFIE_HIP {
 
 class RModel;
 
-enum class OperatorKind { GEMM, CONV, UNARY, BINARY, POOL, QUANTIZE, DEQUANTIZE, QGEMM, QCONV, OTHER };
+enum class OperatorKind { GEMM, CONV, UNARY, BINARY, POOL, QUANTIZE, DEQUANTIZE, QGEMM, QCONV, QPOOL, OTHER };
+constexpr int kLayoutNCHW = 0, kLayoutNHWC = 1;
 
 class ROperator {
 public:

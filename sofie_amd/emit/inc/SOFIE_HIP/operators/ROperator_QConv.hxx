@@ -1,0 +1,255 @@
+// Quantised convolution chain of the gfx950 backend.  The reference has no quantised operator
+// (parsers/src/RModelParser_ONNX.cxx:279-367); these follow its operator contract
+// (core/inc/SOFIE/operators/ROperator.hxx:111-147), the geometry rules of its Conv
+// (core/inc/SOFIE/operators/ROperator_Conv.hxx:123-262) and the ONNX definitions:
+//   QLinearConv  acc = conv_i32(x_i8, w_i8) + B_i32[co];  y_i8 = sat8(rne(float(acc) * m[co])),
+//                m[co] = (x_scale * w_scale[co]) / y_scale formed once in fp32 by the generator; zero points 0.
+//                A Relu that follows is folded into the store.  Between two quantised convolutions the
+//                activation is kept NHWC (channels fastest), which is what the matrix-core kernel reads in place.
+//   DequantizeLinear + GlobalAveragePool on an int8 map  ->  one kernel: exact int32 sum, then * scale / HW.
+//   Flatten      a device copy (the tensors here are a few KB).
+#ifndef SOFIE_HIP_ROPERATOR_QCONV
+#define SOFIE_HIP_ROPERATOR_QCONV
+
+#include "SOFIE_HIP/operators/ROperator_Conv.hxx"
+
+#include <cmath>
+
+namespace SOFIE_HIP {
+
+class ROperator_QConv final : public ROperator {
+public:
+   // the nine inputs of ONNX QLinearConv (nameB may be empty)
+   ROperator_QConv(std::string autopad, std::vector<std::size_t> dilations, std::size_t group, std::vector<std::size_t> kernelShape,
+                   std::vector<std::size_t> pads, std::vector<std::size_t> strides, std::string nameX, std::string nameXScale,
+                   std::string nameXZero, std::string nameW, std::string nameWScale, std::string nameWZero, std::string nameYScale,
+                   std::string nameYZero, std::string nameB, std::string nameY)
+      : fAttrAutopad(autopad), fAttrDilations(dilations), fAttrGroup(group), fAttrKernelShape(kernelShape), fAttrPads(pads),
+        fAttrStrides(strides), fNX(UTILITY::Clean_name(nameX)), fNXS(UTILITY::Clean_name(nameXScale)), fNXZ(UTILITY::Clean_name(nameXZero)),
+        fNW(UTILITY::Clean_name(nameW)), fNWS(UTILITY::Clean_name(nameWScale)), fNWZ(UTILITY::Clean_name(nameWZero)),
+        fNYS(UTILITY::Clean_name(nameYScale)), fNYZ(UTILITY::Clean_name(nameYZero)), fNB(UTILITY::Clean_name(nameB)),
+        fNY(UTILITY::Clean_name(nameY))
+   {
+      fInputTensorNames = {fNX, fNW};
+      if (!fNB.empty())
+         fInputTensorNames.push_back(fNB);
+      fOutputTensorNames = {fNY};
+      fKind = OperatorKind::QCONV;
+   }
+   bool HasRelu() const { return fRelu; }
+   void FuseRelu(const std::string &newOutput)
+   {
+      fRelu = true;
+      fNY = newOutput;
+      fOutputTensorNames = {fNY};
+   }
+   const std::string &OutputName() const { return fNY; }
+
+   void Initialize(RModel &model) override
+   {
+      for (auto *n : {&fNX, &fNW})
+         if (!model.CheckIfTensorAlreadyExist(*n))
+            throw std::runtime_error("SOFIE QLinearConv Op Input Tensor " + *n + " is not found in model");
+      if (model.GetTensorType(fNX) != ETensorType::INT8)
+         throw std::runtime_error("SOFIE QLinearConv Op: input tensor " + fNX + " is not int8");
+      if (!model.IsInitializedTensor(fNW) || model.GetTensorType(fNW) != ETensorType::INT8)
+         throw std::runtime_error("SOFIE QLinearConv Op: weight tensor " + fNW + " must be an int8 initializer");
+      for (auto *z : {&fNXZ, &fNWZ, &fNYZ}) {
+         if (z->empty())
+            continue;
+         if (!model.IsInitializedTensor(*z) || model.GetTensorType(*z) != ETensorType::INT8)
+            throw std::runtime_error("SOFIE QLinearConv Op: zero point " + *z + " must be an int8 initializer");
+         const auto *p = static_cast<const int8_t *>(model.GetInitializedTensorData(*z).get());
+         for (std::size_t i = 0; i < ConvertShapeToLength(model.GetTensorShape(*z)); ++i)
+            if (p[i] != 0)
+               throw std::runtime_error("SOFIE QLinearConv Op: zero point " + *z + " is not 0; this backend emits symmetric quantisation only");
+      }
+      fGeo.Resolve(fAttrAutopad, fAttrDilations, fAttrGroup, fAttrKernelShape, fAttrPads, fAttrStrides, model.GetTensorShape(fNX),
+                   model.GetTensorShape(fNW));
+      const float xs = model.GetScalarInitializer(fNXS), ys = model.GetScalarInitializer(fNYS);
+      if (!(xs > 0) || !(ys > 0))
+         throw std::runtime_error("SOFIE QLinearConv Op: scales of " + fNX + " and " + fNY + " must be positive");
+      if (!model.IsInitializedTensor(fNWS) || model.GetTensorType(fNWS) != ETensorType::FLOAT)
+         throw std::runtime_error("SOFIE QLinearConv Op: weight scale " + fNWS + " must be a float initializer");
+      const std::size_t nws = ConvertShapeToLength(model.GetTensorShape(fNWS));
+      if (nws != 1 && nws != fGeo.Cout)
+         throw std::runtime_error("SOFIE QLinearConv Op: weight scale " + fNWS + " must have 1 or " + std::to_string(fGeo.Cout) + " elements");
+      const float *ws = static_cast<const float *>(model.GetInitializedTensorData(fNWS).get());
+      std::vector<float> m(fGeo.Cout);
+      for (std::size_t co = 0; co < fGeo.Cout; ++co) {
+         volatile float prod = xs * ws[nws == 1 ? 0 : co]; // two fp32 roundings, in this order
+         m[co] = prod / ys;
+      }
+      fNM = fNY + "_requant_scale";
+      model.AddInitializedTensor(fNM, ETensorType::FLOAT, {fGeo.Cout}, m.data());
+      if (!fNB.empty()) {
+         if (!model.IsInitializedTensor(fNB) || model.GetTensorType(fNB) != ETensorType::INT32 ||
+             ConvertShapeToLength(model.GetTensorShape(fNB)) != fGeo.Cout)
+            throw std::runtime_error("SOFIE QLinearConv Op: bias " + fNB + " must be an int32 initializer of " + std::to_string(fGeo.Cout) + " elements");
+      }
+      fXLayout = model.GetTensorLayout(fNX);
+      // channels-last output when every reader understands it
+      fYLayout = kLayoutNHWC;
+      if (model.IsOutputTensor(fNY))
+         fYLayout = kLayoutNCHW;
+      for (OperatorKind k : model.ConsumerKinds(fNY))
+         if (k != OperatorKind::QCONV && k != OperatorKind::QPOOL)
+            fYLayout = kLayoutNCHW;
+      model.AddIntermediateTensor(fNY, ETensorType::INT8, fGeo.OutputShape());
+      model.SetTensorLayout(fNY, fYLayout);
+   }
+   std::size_t PackedK() const { return ((fGeo.C / fGeo.group) * fGeo.kh * fGeo.kw + 15) / 16 * 16; }
+   std::vector<std::pair<std::string, std::size_t>> GetPersistentBuffers() override
+   {
+      return {{"packed_" + fNW, (fGeo.Cout * PackedK() + 255) / 256 * 256}};
+   }
+   std::string GenerateInitCode_GPU_HIP() override
+   {
+      std::stringstream out;
+      out << SP << "   " << "{\n";
+      out << SP << "      " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n";
+      out << SP << "      " << "detail::Check(sofie_hip_pack_conv_weight_i8(fCtx, &d, packed_" << fNW << ", tensor_" << fNW << "), \"re-layout of "
+          << fNW << "\");\n";
+      out << SP << "   " << "}\n";
+      return out.str();
+   }
+   // the runtime's rule for reading the activations in place (no column matrix): NHWC, channels per group a power
+   // of two >= 64, at most 32 taps, 32-bit offsets
+   bool ImplicitGemm() const
+   {
+      const std::size_t cg = fGeo.C / fGeo.group, taps = fGeo.kh * fGeo.kw;
+      const double xbytes = (double)fGeo.N * fGeo.H * fGeo.W * fGeo.C;
+      return fXLayout == kLayoutNHWC && (cg & (cg - 1)) == 0 && cg >= 64 && taps <= 32 && fGeo.C % 16 == 0 && xbytes < 2.0e9 &&
+             (double)fGeo.N * fGeo.OH * fGeo.OW < 2.0e9 && taps <= 32;
+   }
+   std::size_t GetWorkspaceBytes() override
+   {
+      if (ImplicitGemm())
+         return 0;
+      const std::size_t per_image = (fGeo.OH * fGeo.OW * PackedK() + 255) / 256 * 256;
+      std::size_t images = std::max<std::size_t>(1, (std::size_t(64) << 20) / per_image);
+      return per_image * std::min(images, fGeo.N);
+   }
+   std::string Generate_GPU_HIP(std::string opName) override
+   {
+      const std::string ws = "workspace_op_" + opName;
+      opName = "op_" + opName;
+      std::stringstream out;
+      out << "\n" << SP << "//----  operator QLinearConv " << opName << " --> " << ConvertShapeToString(fGeo.OutputShape())
+          << (fYLayout == kLayoutNHWC ? " (stored NHWC)" : "") << (ImplicitGemm() ? ", implicit GEMM" : ", column matrix") << "\n";
+      out << SP << "{\n";
+      out << SP << "   " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n";
+      out << SP << "   " << "sofie_conv_i8_args a{};\n";
+      out << SP << "   " << "a.X = tensor_" << fNX << "; a.W = packed_" << fNW << "; a.w_is_packed = 1; a.bias = "
+          << (fNB.empty() ? "nullptr" : "tensor_" + fNB) << "; a.scale = tensor_" << fNM << ";\n";
+      out << SP << "   " << "a.relu = " << (fRelu ? 1 : 0) << "; a.out = SOFIE_I8OUT_I8; a.x_layout = "
+          << (fXLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.y_layout = "
+          << (fYLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.Y = tensor_" << fNY << ";\n";
+      if (GetWorkspaceBytes())
+         out << SP << "   " << "a.workspace = " << ws << "; a.workspace_bytes = " << GetWorkspaceBytes() << ";\n";
+      out << SP << "   " << "detail::Check(sofie_hip_conv_i8(fCtx, &d, &a), \"" << opName << " QLinearConv\");\n";
+      out << SP << "}\n";
+      return out.str();
+   }
+
+private:
+   std::string fAttrAutopad;
+   std::vector<std::size_t> fAttrDilations;
+   std::size_t fAttrGroup;
+   std::vector<std::size_t> fAttrKernelShape, fAttrPads, fAttrStrides;
+   std::string fNX, fNXS, fNXZ, fNW, fNWS, fNWZ, fNYS, fNYZ, fNB, fNY, fNM;
+   bool fRelu = false;
+   int fXLayout = kLayoutNCHW, fYLayout = kLayoutNCHW;
+   ConvGeometry fGeo;
+};
+
+// DequantizeLinear(int8 feature map) followed by GlobalAveragePool, as one kernel over either layout
+class ROperator_QGlobalAveragePool final : public ROperator {
+public:
+   ROperator_QGlobalAveragePool(std::string nameX, std::string nameScale, std::string nameY)
+      : fNX(UTILITY::Clean_name(nameX)), fNS(UTILITY::Clean_name(nameScale)), fNY(UTILITY::Clean_name(nameY))
+   {
+      fInputTensorNames = {fNX};
+      fOutputTensorNames = {fNY};
+      fKind = OperatorKind::QPOOL;
+   }
+   void Initialize(RModel &model) override
+   {
+      if (!model.CheckIfTensorAlreadyExist(fNX))
+         throw std::runtime_error("SOFIE GlobalAveragePool op Input Tensor " + fNX + " is not found in model");
+      if (model.GetTensorType(fNX) != ETensorType::INT8)
+         throw std::runtime_error("SOFIE quantised GlobalAveragePool Op: input tensor " + fNX + " is not int8");
+      fShapeX = model.GetTensorShape(fNX);
+      if (fShapeX.size() < 3)
+         throw std::runtime_error("SOFIE Pool Op input data tensor" + fNX + " has fewer than 3 dimensions");
+      fScale = model.GetScalarInitializer(fNS);
+      fLayout = model.GetTensorLayout(fNX);
+      std::vector<std::size_t> shapeY(fShapeX.size(), 1);
+      shapeY[0] = fShapeX[0];
+      shapeY[1] = fShapeX[1];
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, shapeY);
+   }
+   std::string Generate_GPU_HIP(std::string opName) override
+   {
+      opName = "op_" + opName;
+      std::size_t hw = 1;
+      for (std::size_t i = 2; i < fShapeX.size(); ++i)
+         hw *= fShapeX[i];
+      std::stringstream out;
+      out << "\n" << SP << "//----  DequantizeLinear + GlobalAveragePool " << opName << "\n";
+      out << SP << "detail::Check(sofie_hip_global_avg_pool_i8(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << fShapeX[0] << ", " << fShapeX[1]
+          << ", " << hw << ", " << (fLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << ", " << FloatLiteral(fScale) << "), \""
+          << opName << " GlobalAveragePool\");\n";
+      return out.str();
+   }
+
+private:
+   std::string fNX, fNS, fNY;
+   std::vector<std::size_t> fShapeX;
+   float fScale = 1.0f;
+   int fLayout = kLayoutNCHW;
+};
+
+// Flatten(axis): [d0..dn) -> [prod(d0..axis), prod(axis..n)], same bytes; emitted as a copy
+class ROperator_Flatten final : public ROperator {
+public:
+   ROperator_Flatten(int axis, std::string nameX, std::string nameY) : fAxis(axis), fNX(UTILITY::Clean_name(nameX)), fNY(UTILITY::Clean_name(nameY))
+   {
+      fInputTensorNames = {fNX};
+      fOutputTensorNames = {fNY};
+   }
+   void Initialize(RModel &model) override
+   {
+      if (!model.CheckIfTensorAlreadyExist(fNX))
+         throw std::runtime_error("SOFIE Reshape Op Input Tensor " + fNX + "  is not found in model");
+      if (model.GetTensorLayout(fNX) != kLayoutNCHW)
+         throw std::runtime_error("SOFIE Flatten Op: input tensor " + fNX + " is stored channels-last");
+      const auto shape = model.GetTensorShape(fNX);
+      int axis = fAxis < 0 ? fAxis + (int)shape.size() : fAxis;
+      if (axis < 0 || axis > (int)shape.size())
+         throw std::runtime_error("SOFIE Flatten Op: axis out of range for " + fNX);
+      std::size_t a = 1, b = 1;
+      for (int i = 0; i < (int)shape.size(); ++i)
+         (i < axis ? a : b) *= shape[i];
+      fType = model.GetTensorType(fNX);
+      fBytes = a * b * GetTypeSize(fType);
+      model.AddIntermediateTensor(fNY, fType, {a, b});
+   }
+   std::string Generate_GPU_HIP(std::string opName) override
+   {
+      opName = "op_" + opName;
+      std::stringstream out;
+      out << "\n" << SP << "//----  Flatten " << opName << "\n";
+      out << SP << "detail::Check(sofie_hip_copy(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << fBytes << "), \"" << opName << " Flatten\");\n";
+      return out.str();
+   }
+
+private:
+   int fAxis;
+   std::string fNX, fNY;
+   ETensorType fType = ETensorType::FLOAT;
+   std::size_t fBytes = 0;
+};
+
+} // namespace SOFIE_HIP
+#endif

@@ -186,6 +186,18 @@ void RModel::FuseGemmActivations()
                c->FuseActivation(act->Activation(), act->Alpha(), act->OutputName());
                changed = true;
             }
+         } else if (auto *qc = dynamic_cast<ROperator_QConv *>(op)) {
+            if (act && act->Activation() == EActivationType::RELU && !qc->HasRelu()) {
+               qc->FuseRelu(act->OutputName());
+               changed = true;
+            }
+         } else if (auto *dqp = dynamic_cast<ROperator_DequantizeLinear *>(op)) {
+            // DequantizeLinear whose only reader is a GlobalAveragePool: one kernel on the int8 map
+            if (dynamic_cast<ROperator_Pool<float> *>(next)) {
+               fOperators[i] = std::make_unique<ROperator_QGlobalAveragePool>(dqp->GetInputTensorNames()[0], dqp->ScaleName(),
+                                                                              next->GetOutputTensorNames()[0]);
+               changed = true;
+            }
          } else if (auto *q = dynamic_cast<ROperator_QGemm *>(op)) {
             if (q->OutputKind() == ROperator_QGemm::Out::I32 && act && act->Activation() == EActivationType::RELU && !q->ReluOnAccumulator()) {
                q->SetReluOnAccumulator();
@@ -209,6 +221,22 @@ void RModel::FuseGemmActivations()
             fOperators.erase(fOperators.begin() + cons[0]);
       }
    }
+}
+
+bool RModel::IsOutputTensor(const std::string &name) const
+{
+   return std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), UTILITY::Clean_name(name)) != fOutputTensorNames.end();
+}
+
+std::vector<OperatorKind> RModel::ConsumerKinds(const std::string &name) const
+{
+   std::vector<OperatorKind> kinds;
+   const std::string n = UTILITY::Clean_name(name);
+   for (auto &op : fOperators)
+      for (auto &in : op->GetInputTensorNames())
+         if (in == n)
+            kinds.push_back(op->GetKind());
+   return kinds;
 }
 
 void RModel::Initialize()

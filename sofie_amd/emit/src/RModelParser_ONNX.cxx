@@ -395,6 +395,15 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          model->AddOperator(std::make_unique<ROperator_QuantizeLinear>(n.in[0], n.in[1], n.out[0]));
       } else if (n.op == "DequantizeLinear") {
          model->AddOperator(std::make_unique<ROperator_DequantizeLinear>(n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "QLinearConv") {
+         if (n.in.size() < 8)
+            throw std::runtime_error("SOFIE ONNX parser: QLinearConv " + n.name + " needs 8 or 9 inputs");
+         model->AddOperator(std::make_unique<ROperator_QConv>(attrS(n, "auto_pad", "NOTSET"), attrV(n, "dilations"), (size_t)attrI(n, "group", 1),
+                                                              attrV(n, "kernel_shape"), attrV(n, "pads"), attrV(n, "strides"), n.in[0], n.in[1],
+                                                              n.in[2], n.in[3], n.in[4], n.in[5], n.in[6], n.in[7],
+                                                              n.in.size() > 8 ? n.in[8] : "", n.out[0]));
+      } else if (n.op == "Flatten") {
+         model->AddOperator(std::make_unique<ROperator_Flatten>((int)attrI(n, "axis", 1), n.in[0], n.out[0]));
       } else if (n.op == "MatMulInteger") {
          model->AddOperator(MakeMatMulInteger(n.in[0], n.in[1], n.out[0]));
       } else {

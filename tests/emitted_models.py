@@ -81,7 +81,42 @@ def fp32_cnn(batch=2):
     return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 3, 12, 12])], outputs=[("Y", np.float32, [batch, 10])], init=init, feeds=[X])
 
 
+def int8_cnn(batch=2, hw=12, channels=(3, 64, 128, 256, 256), n_out=10):
+    """BASELINE config 5 as ONNX operators: QuantizeLinear, then per stage QLinearConv 3x3 s1 p1 (per-channel weight scales,
+    int32 bias: the folded BatchNorm) + Relu, then DequantizeLinear, GlobalAveragePool, Flatten, Gemm.  Returns the model and
+    the constants of the CPU chain (tests.refmodels.int8_cnn_oracle)."""
+    from tests.refmodels import make_int8_cnn
+    m = make_int8_cnn(batch, hw, channels, n_out)
+    init, nodes = {}, []
+    init["zp"] = np.zeros((), dtype=np.int8)
+    xs = np.float32(m["in_scale"])
+    init["sx"] = np.array(xs, dtype=np.float32)
+    nodes.append(ow.node("QuantizeLinear", ["X", "sx", "zp"], ["Q"]))
+    x = "Q"
+    for l, cv in enumerate(m["convs"]):
+        ys = np.float32(0.05 + 0.01 * l)                      # activation scale of this stage's output
+        wsc = (cv["scale"] * ys / xs).astype(np.float32)     # per-channel weight scales
+        cv["scale"] = ((xs * wsc).astype(np.float32) / ys).astype(np.float32)   # what the generator forms: two fp32 roundings
+        init["W%d" % l], init["B%d" % l] = cv["W"], cv["bias"]
+        init["xs%d" % l] = np.array(xs, dtype=np.float32)
+        init["ws%d" % l] = wsc
+        init["ys%d" % l] = np.array(ys, dtype=np.float32)
+        nodes.append(ow.node("QLinearConv", [x, "xs%d" % l, "zp", "W%d" % l, "ws%d" % l, "zp", "ys%d" % l, "zp", "B%d" % l], ["C%d" % l],
+                             kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1]))
+        nodes.append(ow.node("Relu", ["C%d" % l], ["R%d" % l]))
+        x, xs = "R%d" % l, ys
+    m["last_scale"] = xs
+    nodes.append(ow.node("DequantizeLinear", [x, "ys%d" % (len(m["convs"]) - 1), "zp"], ["D"]))
+    nodes.append(ow.node("GlobalAveragePool", ["D"], ["P"]))
+    nodes.append(ow.node("Flatten", ["P"], ["F"], axis=1))
+    init["WF"], init["BF"] = m["fc_w"], m["fc_b"]
+    nodes.append(ow.node("Gemm", ["F", "WF", "BF"], ["Y"], alpha=1.0, beta=1.0))
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch] + list(m["in_shape"]))], outputs=[("Y", np.float32, [batch, n_out])],
+                init=init, feeds=[m["x"]], consts=m)
+
+
 CONFIG_MODELS = {
+    "Config5_int8_CNN_small": lambda: int8_cnn(2, 12),
     "Config1_fp32_MLP": lambda: fp32_mlp(64),
     "Config2_int8_MLP_small": lambda: int8_mlp([64, 128, 96, 32], 48),
     "Config2_int8_MLP_mid": lambda: int8_mlp([256, 512, 512, 256], 256),

@@ -156,3 +156,28 @@ def test_weight_file_round_trip(emitted):
     for k, v in g["initializers"].items():
         key = "tensor_" + re.sub(r"[^A-Za-z0-9_]", "_", k)
         assert np.array_equal(seen[key], np.asarray(v, dtype=np.float32).ravel()), k
+
+
+def test_quantised_cnn_keeps_channels_last_and_reads_activations_in_place(emitted):
+    txt = read(emitted, "Config5_int8_CNN_small")
+    body = txt[txt.index("void infer_nosync()"):]
+    body = body[:body.index("infer(")]
+    assert body.count("sofie_hip_conv_i8(") == 4
+    assert "sofie_hip_unary_f32" not in body                      # the four Relu are in the convolutions' stores
+    assert body.count("a.relu = 1") == 4
+    assert body.count("implicit GEMM") == 3 and body.count("column matrix") == 1   # only the 3-channel input needs im2col
+    assert body.count("a.y_layout = SOFIE_LAYOUT_NHWC") == 4
+    assert body.count("a.x_layout = SOFIE_LAYOUT_NCHW") == 1     # the quantised model input
+    assert "sofie_hip_dequantize_linear" not in body and "sofie_hip_global_avg_pool_i8(" in body
+    # weights are re-laid out once, in the constructor
+    ctor = txt[txt.index("Session(std::string filename"):txt.index("void infer_nosync()")]
+    assert ctor.count("sofie_hip_pack_conv_weight_i8(") == 4
+
+
+def test_asymmetric_zero_point_is_refused(tmp_path):
+    init = {"W": np.ones((4, 3, 1, 1), dtype=np.int8), "s": np.array(0.5, dtype=np.float32), "z": np.zeros((), dtype=np.int8),
+            "z1": np.array(3, dtype=np.int8), "sx": np.array(0.1, dtype=np.float32)}
+    nodes = [ow.node("QuantizeLinear", ["X", "sx", "z"], ["Q"]),
+             ow.node("QLinearConv", ["Q", "s", "z1", "W", "s", "z", "s", "z"], ["Y"], kernel_shape=[1, 1], pads=[0, 0, 0, 0])]
+    r = _emit(tmp_path, nodes, [("X", np.float32, [1, 3, 4, 4])], [("Y", np.int8, [1, 4, 4, 4])], init)
+    assert r.returncode != 0 and "zero point" in r.stdout

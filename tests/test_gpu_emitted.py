@@ -61,3 +61,16 @@ def test_emitted_int8_mlp_is_bit_exact(rt, model, dims, batch):
     got = run_emitted(model, spec["feeds"], h.size)
     assert np.array_equal(got.view(np.uint32), h.ravel().view(np.uint32))
     assert np.abs(h).max() > 0
+
+
+def test_emitted_int8_cnn_matches_cpu_chain(rt):
+    """QuantizeLinear -> 4 x [QLinearConv + Relu] -> DequantizeLinear -> GlobalAveragePool -> Flatten -> Gemm, parsed from ONNX,
+    emitted, compiled: the int8 stages are bit-exact by construction of the kernels (checked operator by operator in
+    test_gpu_conv_i8), the fp32 tail is held to 1e-5."""
+    from tests.refmodels import int8_cnn_oracle
+    spec = em.int8_cnn(2, 12)
+    want = int8_cnn_oracle(spec["consts"], spec["feeds"][0]).ravel()
+    print("emitted Config5_int8_CNN_small", flush=True)
+    got = run_emitted("Config5_int8_CNN_small", spec["feeds"], want.size)
+    assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+    assert np.abs(want).max() > 1e-3
