@@ -215,6 +215,96 @@ inline std::unique_ptr<ROperator_QGemm> MakeMatMulInteger(std::string nameA, std
    return std::make_unique<ROperator_QGemm>(nameA, nameB, nameY);
 }
 
+// FP8 (OCP e4m3fn) Gemm: the fp32 activation is quantised per tensor at run time, the weight is an e4m3 initializer,
+// the matrix cores accumulate in fp32, and scale, bias, activation and the fp32 / bf16 conversion are fused into the store:
+//   Y = act( (e4m3(X / x_scale) x W_e4m3) * (x_scale * w_scale) + bias )
+// The reference has no 8-bit floating type (core/inc/SOFIE/SOFIE_common.hxx:29-54 stops at BFLOAT16).
+class ROperator_Fp8Gemm final : public ROperator {
+public:
+   ROperator_Fp8Gemm(float xScale, float wScale, int transB, std::string nameX, std::string nameW, std::string nameBias,
+                     EActivationType act, ETensorType outType, std::string nameY)
+      : fXScale(xScale), fWScale(wScale), fTransB(transB), fNX(UTILITY::Clean_name(nameX)), fNW(UTILITY::Clean_name(nameW)),
+        fNBias(UTILITY::Clean_name(nameBias)), fAct(act), fOutType(outType), fNY(UTILITY::Clean_name(nameY))
+   {
+      fInputTensorNames = {fNX, fNW};
+      if (!fNBias.empty())
+         fInputTensorNames.push_back(fNBias);
+      fOutputTensorNames = {fNY};
+      fKind = OperatorKind::QGEMM;
+   }
+   void Initialize(RModel &model) override
+   {
+      if (!model.CheckIfTensorAlreadyExist(fNX) || !model.CheckIfTensorAlreadyExist(fNW))
+         throw std::runtime_error("SOFIE Fp8Gemm Op Input Tensor " + fNX + " or " + fNW + " is not found in model");
+      if (model.GetTensorType(fNX) != ETensorType::FLOAT)
+         throw std::runtime_error("SOFIE Fp8Gemm Op: input tensor " + fNX + " is not float");
+      if (!model.IsInitializedTensor(fNW) || model.GetTensorType(fNW) != ETensorType::FLOAT8E4M3FN)
+         throw std::runtime_error("SOFIE Fp8Gemm Op: weight tensor " + fNW + " must be an e4m3 initializer");
+      if (!(fXScale > 0) || !(fWScale > 0))
+         throw std::runtime_error("SOFIE Fp8Gemm Op: scales must be positive");
+      if (fOutType != ETensorType::FLOAT && fOutType != ETensorType::BFLOAT16)
+         throw std::runtime_error("SOFIE Fp8Gemm Op: the output is float or bfloat16");
+      const auto sx = model.GetTensorShape(fNX), sw = model.GetTensorShape(fNW);
+      if (sx.size() != 2 || sw.size() != 2)
+         throw std::runtime_error("SOFIE Fp8Gemm Op: 2-D operands only");
+      fM = sx[0];
+      fK = sx[1];
+      fN = fTransB ? sw[0] : sw[1];
+      if ((fTransB ? sw[1] : sw[0]) != fK)
+         throw std::runtime_error("SOFIE Fp8Gemm Op: shapes " + ConvertShapeToString(sx) + " and " + ConvertShapeToString(sw) + " do not agree");
+      if (!fNBias.empty() && (!model.CheckIfTensorAlreadyExist(fNBias) || model.GetTensorType(fNBias) != ETensorType::FLOAT ||
+                              ConvertShapeToLength(model.GetTensorShape(fNBias)) != fN))
+         throw std::runtime_error("SOFIE Fp8Gemm Op: bias " + fNBias + " must be a float tensor of " + std::to_string(fN) + " elements");
+      model.AddIntermediateTensor(fNY, fOutType, {fM, fN});
+   }
+   std::vector<std::pair<std::string, std::size_t>> GetPersistentBuffers() override
+   {
+      if (fTransB)
+         return {};
+      return {{"packed_" + fNW, fK * fN}};
+   }
+   std::string GenerateInitCode_GPU_HIP() override
+   {
+      if (fTransB)
+         return "";
+      std::stringstream out;
+      out << SP << "   " << "detail::Check(sofie_hip_transpose_i8(fCtx, packed_" << fNW << ", reinterpret_cast<const int8_t *>(tensor_" << fNW << "), "
+          << fK << ", " << fN << ", 0, 0), \"re-layout of " << fNW << "\");\n";
+      return out.str();
+   }
+   std::size_t GetWorkspaceBytes() override { return ((fM * fK + 255) / 256) * 256; }
+   std::string Generate_GPU_HIP(std::string opName) override
+   {
+      const std::string ws = "workspace_op_" + opName;
+      opName = "op_" + opName;
+      volatile float prod = fXScale * fWScale;
+      std::stringstream out;
+      out << "\n" << SP << "//--------- Fp8Gemm " << opName << " e4m3 { " << fM << " , " << fK << " } * { " << fK << " , " << fN << " } -> " << fNY << "\n";
+      out << SP << "{\n";
+      out << SP << "   " << "detail::Check(sofie_hip_quantize_fp8(fCtx, reinterpret_cast<uint8_t *>(" << ws << "), tensor_" << fNX << ", " << fM * fK
+          << ", " << FloatLiteral(fXScale) << "), \"" << opName << " quantisation\");\n";
+      out << SP << "   " << "sofie_gemm_fp8_desc d{};\n";
+      out << SP << "   " << "d.M = " << fM << "; d.N = " << fN << "; d.K = " << fK << "; d.transB = 1;\n";
+      out << SP << "   " << "d.A = reinterpret_cast<const uint8_t *>(" << ws << "); d.B = "
+          << (fTransB ? "tensor_" + fNW : "reinterpret_cast<const uint8_t *>(packed_" + fNW + ")") << ";\n";
+      out << SP << "   " << "d.bias = " << (fNBias.empty() ? "nullptr" : "tensor_" + fNBias) << "; d.scale = " << FloatLiteral(prod)
+          << "; d.act = " << ActivationEnumName(fAct) << "; d.out = " << (fOutType == ETensorType::FLOAT ? "SOFIE_F8OUT_F32" : "SOFIE_F8OUT_BF16")
+          << "; d.Y = tensor_" << fNY << ";\n";
+      out << SP << "   " << "detail::Check(sofie_hip_gemm_fp8(fCtx, &d), \"" << opName << " Fp8Gemm\");\n";
+      out << SP << "}\n";
+      return out.str();
+   }
+
+private:
+   float fXScale, fWScale;
+   int fTransB;
+   std::string fNX, fNW, fNBias;
+   EActivationType fAct;
+   ETensorType fOutType;
+   std::string fNY;
+   std::size_t fM = 0, fN = 0, fK = 0;
+};
+
 // int8 Relu on an int32 accumulator tensor is only meaningful fused; as a stand-alone operator on int32 it
 // is not emitted (the fusion always removes it).
 

@@ -3,7 +3,9 @@
 // so that ones -> 3.5.  Usage: sofie_hip_emit_example <out_dir>
 #include "SOFIE_HIP/operators/OperatorList.hxx"
 
+#include <cstdint>
 #include <iostream>
+#include <vector>
 
 int main(int argc, char **argv)
 {
@@ -24,6 +26,26 @@ int main(int argc, char **argv)
       model.AddOutputTensorNameList({"Y"});
       model.GenerateGPU_HIP(Options::kExternalStream);
       model.OutputGenerated(std::string(argv[1]) + "/ApiGemmRelu_GPU_HIP.hxx");
+      // FP8 Gemm with bias and GELU: X[48,256] fp32, W e4m3 [96,256] (K contiguous), codes from a linear congruential
+      // sequence so that a test can rebuild them, bias[n] = 0.25 (n mod 7 - 3)
+      RModel f8("ApiFp8Gemm");
+      f8.AddInputTensorInfo("X", ETensorType::FLOAT, std::vector<std::size_t>{48, 256});
+      f8.AddInputTensorName("X");
+      std::vector<uint8_t> w8(96 * 256);
+      uint32_t s = 2024;
+      for (auto &v : w8) {
+         s = s * 1664525u + 1013904223u;
+         v = (uint8_t)((s >> 24) & 0xbe); // exponent at most 7 (|w| < 32), never the NaN code
+      }
+      std::vector<float> bias(96);
+      for (std::size_t n = 0; n < bias.size(); ++n)
+         bias[n] = 0.25f * ((int)(n % 7) - 3);
+      f8.AddInitializedTensor("W", ETensorType::FLOAT8E4M3FN, {96, 256}, w8.data());
+      f8.AddInitializedTensor("B", ETensorType::FLOAT, {96}, bias.data());
+      f8.AddOperator(std::make_unique<ROperator_Fp8Gemm>(0.03125f, 0.0078125f, 1, "X", "W", "B", EActivationType::GELU, ETensorType::FLOAT, "Y"));
+      f8.AddOutputTensorNameList({"Y"});
+      f8.GenerateGPU_HIP();
+      f8.OutputGenerated(std::string(argv[1]) + "/ApiFp8Gemm_GPU_HIP.hxx");
    } catch (const std::exception &e) {
       std::cerr << "error: " << e.what() << "\n";
       return 1;

@@ -164,8 +164,15 @@ def _run(cmd):
     return r.stdout
 
 
+API_MODELS = ("ApiGemmRelu", "ApiFp8Gemm")
+
+
 def emit_and_compile(model, onnx_path, n_inputs):
     _run([EMIT, onnx_path, OUT])
+    return compile_harness(model, n_inputs)
+
+
+def compile_harness(model, n_inputs):
     src = os.path.join(OUT, model + "_harness.cxx")
     with open(src, "w") as f:
         f.write(HARNESS % dict(model=model, args=", ".join("inputs[%d]" % i for i in range(n_inputs))))
@@ -191,7 +198,11 @@ def build_all(jobs=8):
         work.append((m, p, len(spec["inputs"])))
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(lambda w: emit_and_compile(*w), work))
-    return [w[0] for w in work]
+    # models built through the RModel API (no ONNX file): sofie_hip_emit_example writes their headers
+    _run([os.path.join(os.path.dirname(EMIT), "sofie_hip_emit_example"), OUT])
+    for m in API_MODELS:
+        compile_harness(m, 1)
+    return [w[0] for w in work] + list(API_MODELS)
 
 
 if __name__ == "__main__":

@@ -74,3 +74,32 @@ def test_emitted_int8_cnn_matches_cpu_chain(rt):
     got = run_emitted("Config5_int8_CNN_small", spec["feeds"], want.size)
     assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
     assert np.abs(want).max() > 1e-3
+
+
+def test_model_built_through_the_api_external_stream_option(rt):
+    # Y = Relu(X[1,3] * ones[3,1] + 0.5): ones -> 3.5 (the reference's tests/alpaka/TestAlpakaExternalStream.cxx:34-37)
+    got = run_emitted("ApiGemmRelu", [np.ones((1, 3), np.float32)], 1)
+    assert got.tolist() == [3.5]
+    got = run_emitted("ApiGemmRelu", [np.array([[-1.0, -2.0, 0.25]], np.float32)], 1)
+    assert got.tolist() == [0.0]
+
+
+def test_emitted_fp8_gemm_within_the_stated_bound(rt):
+    from oracle import binding as ob
+    from tests import util
+    M, K, N = 48, 256, 96
+    s, w8 = 2024, np.empty(N * K, dtype=np.uint8)
+    for i in range(N * K):                      # the code sequence of sofie_amd/emit/tools/emit_example_api.cxx
+        s = (s * 1664525 + 1013904223) & 0xFFFFFFFF
+        w8[i] = (s >> 24) & 0xBE
+    w8 = w8.reshape(N, K)
+    bias = (0.25 * ((np.arange(N) % 7) - 3)).astype(np.float32)
+    x = util.normal(77, M * K).reshape(M, K)
+    xs, wsc = np.float32(0.03125), np.float32(0.0078125)
+    a8 = ob.quantize_fp8(x, xs)
+    want, abs_sum = ob.gemm_fp8(a8, w8, M=M, N=N, K=K, transB=1, bias=bias, scale=np.float32(xs * wsc), act=4, out=1, want_abs_sum=True)
+    print("emitted ApiFp8Gemm", flush=True)
+    got = run_emitted("ApiFp8Gemm", [x], M * N).reshape(M, N)
+    bound = 1.2 * 2.0 ** -14 * abs_sum.astype(np.float64) * float(xs * wsc) + 1e-6
+    assert np.all(np.abs(got.astype(np.float64) - want) <= bound)
+    assert np.abs(want).max() > 0.5
