@@ -370,19 +370,32 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
 {
    const bool externalStream = options & static_cast<std::underlying_type_t<Options>>(Options::kExternalStream);
    const bool noWeightFile = options & static_cast<std::underlying_type_t<Options>>(Options::kNoWeightFile);
+   const bool customMemory = options & static_cast<std::underlying_type_t<Options>>(Options::kCustomMemory);
    std::stringstream gc;
    std::string guard = "SOFIE_" + fName;
    std::transform(guard.begin(), guard.end(), guard.begin(), [](unsigned char c) { return std::toupper(c); });
    gc << "//Code generated automatically by SOFIE (gfx950 HIP backend)\n";
    gc << "#ifndef " << guard << "_GPU_HIP\n#define " << guard << "_GPU_HIP\n\n";
    gc << "#include <array>\n#include <cstddef>\n#include <cstdint>\n#include <cstdlib>\n#include <fstream>\n#include <stdexcept>\n#include <string>\n"
-         "#include <tuple>\n#include <type_traits>\n#include <vector>\n#include \"sofie_hip.h\"\n\n";
+         "#include <tuple>\n#include <type_traits>\n#include <vector>\n#include \"sofie_hip.h\"\n";
+   if (customMemory)
+      gc << "#include <functional>\n";
+   gc << "\n";
    gc << "namespace SOFIE_" << fName << " {\n" << kRuntimeHelpers << "\n";
+   if (customMemory) {
+      // the reference's contract for caller-owned device memory (core/src/utils/SOFIE_common_helpers.cxx:741-804):
+      // alloc is called once for the whole block, assign (optional) maps an offset of the plan to an address, dealloc
+      // gets the block back when the Session ends
+      gc << "struct MemoryProvider {\n   std::function<void *(std::size_t)> alloc;\n   std::function<void *(std::size_t)> assign;\n"
+            "   std::function<void(void *)> dealloc;\n};\n\n";
+   }
    gc << "struct Session {\n";
    gc << "   // one arena: weights, operator-owned buffers, inputs, outputs, then the pool of intermediates\n";
    gc << "   static constexpr std::size_t kArenaBytes = " << fArenaBytes << ";\n";
    gc << "   static constexpr std::size_t kIntermediatePoolBytes = " << fPoolBytes << ";\n";
    gc << "   sofie_hip_ctx *fCtx = nullptr;\n";
+   if (customMemory)
+      gc << "   MemoryProvider fProvider;\n   void *fBlock = nullptr;\n";
    auto typeOf = [&](const std::string &planName) -> std::string {
       if (planName.rfind("tensor_", 0) == 0)
          return ConvertTypeToString(GetTensorType(planName.substr(7)));
@@ -393,15 +406,32 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
          << (p.pooled ? ", live [" + std::to_string(p.begin) + "," + std::to_string(p.end) + ")" : "") << "\n";
    gc << "\n";
    // constructor
-   gc << "   Session(std::string filename = \"" << (noWeightFile ? "" : fName + "_GPU_HIP.dat") << "\"" << (externalStream ? ", void *stream = nullptr" : "")
-      << ", int device = 0)\n   {\n";
+   gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "std::string filename = \""
+      << (noWeightFile ? "" : fName + "_GPU_HIP.dat") << "\"" << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
+   if (customMemory)
+      gc << "      : fProvider(std::move(provider))\n";
+   gc << "   {\n";
+   if (customMemory)
+      gc << "      if (!fProvider.alloc)\n         throw std::runtime_error(\"SOFIE HIP Session: the memory provider has no alloc function\");\n";
    gc << "      detail::Check(sofie_hip_ctx_create(&fCtx, device, " << (externalStream ? "stream" : "nullptr") << "), \"Session\");\n";
    gc << "      try {\n";
-   gc << "         detail::Check(sofie_hip_arena_create(fCtx, kArenaBytes, " << kPoolAlignBytes << "), \"arena allocation\");\n";
-   gc << "         char *base = static_cast<char *>(sofie_hip_arena_ptr(fCtx, 0));\n";
-   gc << "         if (!base)\n            throw std::runtime_error(\"SOFIE HIP runtime error: arena is null\");\n";
-   for (auto &p : fPlan)
-      gc << "         " << p.name << " = reinterpret_cast<" << typeOf(p.name) << " *>(base + " << p.offset << ");\n";
+   if (customMemory) {
+      gc << "         fBlock = fProvider.alloc(kArenaBytes);\n";
+      gc << "         if (!fBlock)\n            throw std::runtime_error(\"SOFIE HIP Session: the memory provider returned no block\");\n";
+      gc << "         detail::Check(sofie_hip_arena_adopt(fCtx, fBlock, kArenaBytes), \"adoption of the caller's block\");\n";
+      gc << "         auto place = [&](std::size_t offset) -> char * {\n"
+            "            void *p = fProvider.assign ? fProvider.assign(offset) : static_cast<char *>(fBlock) + offset;\n"
+            "            if (!p)\n               throw std::runtime_error(\"SOFIE HIP Session: the memory provider assigned no address\");\n"
+            "            return static_cast<char *>(p);\n         };\n";
+      for (auto &p : fPlan)
+         gc << "         " << p.name << " = reinterpret_cast<" << typeOf(p.name) << " *>(place(" << p.offset << "));\n";
+   } else {
+      gc << "         detail::Check(sofie_hip_arena_create(fCtx, kArenaBytes, " << kPoolAlignBytes << "), \"arena allocation\");\n";
+      gc << "         char *base = static_cast<char *>(sofie_hip_arena_ptr(fCtx, 0));\n";
+      gc << "         if (!base)\n            throw std::runtime_error(\"SOFIE HIP runtime error: arena is null\");\n";
+      for (auto &p : fPlan)
+         gc << "         " << p.name << " = reinterpret_cast<" << typeOf(p.name) << " *>(base + " << p.offset << ");\n";
+   }
    bool anyWeights = false, anyConstants = false;
    for (auto &kv : fInitializedTensors)
       (kv.second.constant ? anyConstants : anyWeights) = true;
@@ -452,10 +482,22 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    if (!init.empty())
       gc << "         // one-time operator set-up (weight re-layouts)\n" << init;
    gc << "         detail::Check(sofie_hip_sync(fCtx), \"Session\");\n";
-   gc << "      } catch (...) {\n         sofie_hip_ctx_destroy(fCtx);\n         fCtx = nullptr;\n         throw;\n      }\n   }\n";
-   gc << "   ~Session() { sofie_hip_ctx_destroy(fCtx); }\n";
+   if (customMemory) {
+      gc << "      } catch (...) {\n         sofie_hip_ctx_destroy(fCtx);\n         fCtx = nullptr;\n"
+            "         if (fBlock && fProvider.dealloc)\n            fProvider.dealloc(fBlock);\n         throw;\n      }\n   }\n";
+      gc << "   ~Session()\n   {\n      sofie_hip_ctx_destroy(fCtx); // waits for the stream; an adopted block is not freed by the runtime\n"
+            "      if (fBlock && fProvider.dealloc)\n         fProvider.dealloc(fBlock);\n   }\n";
+   } else {
+      gc << "      } catch (...) {\n         sofie_hip_ctx_destroy(fCtx);\n         fCtx = nullptr;\n         throw;\n      }\n   }\n";
+      gc << "   ~Session() { sofie_hip_ctx_destroy(fCtx); }\n";
+   }
    gc << "   Session(const Session &) = delete;\n   Session &operator=(const Session &) = delete;\n\n";
    gc << "   std::size_t GetIntermediateMemoryPoolSize() const { return kIntermediatePoolBytes; }\n";
+   // device-resident use: where to write the inputs and read the outputs around infer_nosync()
+   for (auto &n : fInputTensorNames)
+      gc << "   " << ConvertTypeToString(fInputTensorInfos[n].type) << " *device_input_" << n << "() const { return tensor_" << n << "; }\n";
+   for (auto &n : fOutputTensorNames)
+      gc << "   " << ConvertTypeToString(GetTensorType(n)) << " const *device_output_" << n << "() const { return tensor_" << n << "; }\n";
    gc << "   void *stream() const { return sofie_hip_stream(fCtx); }\n\n";
 
    // infer_nosync: the operators, inputs and outputs resident in the arena

@@ -26,6 +26,26 @@ int main(int argc, char **argv)
       model.AddOutputTensorNameList({"Y"});
       model.GenerateGPU_HIP(Options::kExternalStream);
       model.OutputGenerated(std::string(argv[1]) + "/ApiGemmRelu_GPU_HIP.hxx");
+      // the chain of the reference's tests/models/CustomMemoryModelGenerator.cxx, with caller-owned device memory:
+      // X[3,5] -> Gemm(W = 0.5, B = 1) -> Relu -> Sigmoid -> Tanh; ones -> tanh(sigmoid(3.5))
+      for (int withStream = 0; withStream < 2; ++withStream) {
+         RModel cm(withStream ? "CustomMemoryStreamChain" : "CustomMemoryChain");
+         cm.AddInputTensorInfo("X", ETensorType::FLOAT, std::vector<std::size_t>{3, 5});
+         cm.AddInputTensorName("X");
+         std::vector<float> W(5 * 4, 0.5f), B(4, 1.0f);
+         cm.AddInitializedTensor("W", ETensorType::FLOAT, {5, 4}, W.data());
+         cm.AddInitializedTensor("B", ETensorType::FLOAT, {4}, B.data());
+         cm.AddOperator(std::make_unique<ROperator_Gemm<float>>(1.0f, 1.0f, 0, 0, "X", "W", "B", "H1"));
+         cm.AddOperator(std::make_unique<ROperator_Relu<float>>("H1", "H2"));
+         cm.AddOperator(std::make_unique<ROperator_Sigmoid<float>>("H2", "H3"));
+         cm.AddOperator(std::make_unique<ROperator_Tanh<float>>("H3", "Y"));
+         cm.AddOutputTensorNameList({"Y"});
+         if (withStream)
+            cm.GenerateGPU_HIP(Options::kCustomMemory | Options::kExternalStream);
+         else
+            cm.GenerateGPU_HIP(Options::kCustomMemory);
+         cm.OutputGenerated(std::string(argv[1]) + "/" + cm.GetName() + "_GPU_HIP.hxx");
+      }
       // FP8 Gemm with bias and GELU: X[48,256] fp32, W e4m3 [96,256] (K contiguous), codes from a linear congruential
       // sequence so that a test can rebuild them, bias[n] = 0.25 (n mod 7 - 3)
       RModel f8("ApiFp8Gemm");

@@ -176,7 +176,10 @@ def compile_harness(model, n_inputs):
     src = os.path.join(OUT, model + "_harness.cxx")
     with open(src, "w") as f:
         f.write(HARNESS % dict(model=model, args=", ".join("inputs[%d]" % i for i in range(n_inputs))))
-    lib = os.path.join(OUT, "lib%s.so" % model)
+    return compile_shared(src, os.path.join(OUT, "lib%s.so" % model))
+
+
+def compile_shared(src, lib):
     _run(["g++", "-O1", "-std=c++20", "-fPIC", "-shared", "-I" + os.path.join(ROOT, "include"), "-I" + OUT, src, "-o", lib,
           "-L" + os.path.join(ROOT, "sofie_amd", "lib"), "-lsofie_hip", "-Wl,-rpath," + os.path.join(ROOT, "sofie_amd", "lib"),
           "-Wl,-rpath,$ORIGIN/../../sofie_amd/lib"])
@@ -202,6 +205,7 @@ def build_all(jobs=8):
     _run([os.path.join(os.path.dirname(EMIT), "sofie_hip_emit_example"), OUT])
     for m in API_MODELS:
         compile_harness(m, 1)
+    compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
     return [w[0] for w in work] + list(API_MODELS)
 
 

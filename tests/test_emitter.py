@@ -181,3 +181,12 @@ def test_asymmetric_zero_point_is_refused(tmp_path):
              ow.node("QLinearConv", ["Q", "s", "z1", "W", "s", "z", "s", "z"], ["Y"], kernel_shape=[1, 1], pads=[0, 0, 0, 0])]
     r = _emit(tmp_path, nodes, [("X", np.float32, [1, 3, 4, 4])], [("Y", np.int8, [1, 4, 4, 4])], init)
     assert r.returncode != 0 and "zero point" in r.stdout
+
+
+def test_custom_memory_header_allocates_nothing(emitted):
+    # the counterpart of the reference's GeneratedCodeHasNoAlpakaDeviceAllocation (tests/alpaka/TestAlpakaCustomMemory.cxx:103-111)
+    for model in ("CustomMemoryChain", "CustomMemoryStreamChain"):
+        txt = read(emitted, model)
+        assert "sofie_hip_arena_create" not in txt and "sofie_hip_arena_adopt(fCtx, fBlock, kArenaBytes)" in txt
+        assert "struct MemoryProvider" in txt and "Session(MemoryProvider provider, std::string filename" in txt
+    assert "void *stream = nullptr" in read(emitted, "CustomMemoryStreamChain")

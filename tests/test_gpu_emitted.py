@@ -103,3 +103,15 @@ def test_emitted_fp8_gemm_within_the_stated_bound(rt):
     bound = 1.2 * 2.0 ** -14 * abs_sum.astype(np.float64) * float(xs * wsc) + 1e-6
     assert np.all(np.abs(got.astype(np.float64) - want) <= bound)
     assert np.abs(want).max() > 0.5
+
+
+def test_custom_memory_sessions(rt):
+    """Options::kCustomMemory: the caller's MemoryProvider supplies the one block (tests/harness_custom_memory.cxx runs the
+    scenarios of the reference's TestAlpakaCustomMemory.cxx and reports them line by line)."""
+    lib = ctypes.CDLL(os.path.join(em.OUT, "libCustomMemory.so"))
+    report = ctypes.create_string_buffer(8192)
+    print("custom memory harness", flush=True)
+    failures = lib.run_custom_memory(em.OUT.encode(), report, 8192)
+    text = report.value.decode()
+    print(text)
+    assert failures == 0 and "FAIL" not in text and text.count("ok ") >= 14
