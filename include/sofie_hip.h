@@ -269,6 +269,13 @@ int sofie_hip_global_avg_pool_f32(sofie_hip_ctx *ctx, float *Y, const float *X, 
 int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y /* [N,C] */, const int8_t *X, int32_t N, int32_t C, int32_t HW,
                                  int32_t x_layout /* SOFIE_LAYOUT_* */, float scale);
 
+/* BatchNormalization at inference, for models whose normalisation was not folded into the weights
+ * (core/inc/SOFIE/operators/ROperator_BatchNormalization.hxx:139-158): X is [N, C, spatial...],
+ *   Y = (X - mean[c]) * fused_scale[c] + bias[c],   fused_scale[c] = scale[c] / sqrt(var[c] + eps) formed by the generator,
+ * then x > 0 ? x : 0 when `relu` is set (the reference's BN + Relu fusion).  Three separately rounded fp32 operations. */
+int sofie_hip_batchnorm_f32(sofie_hip_ctx *ctx, float *Y, const float *X, const float *fused_scale, const float *mean,
+                            const float *bias, int32_t N, int32_t C, int32_t spatial, int32_t relu);
+
 /* ---- measurement helpers used by the benchmark ------------------------------------------------ */
 /* Register-only int8 MFMA loop on every CU (no counterpart in the reference): the rate the matrix
  * cores of this board sustain with no memory traffic, with constant operands (random_operands = 0)

@@ -116,6 +116,17 @@ def global_avg_pool(X):
     return Y
 
 
+def batchnorm(X, scale, bias, mean, var, eps=1e-5, relu=0):
+    X = _f32(X)
+    Cc = X.shape[1]
+    scale, bias, mean, var = _f32(scale), _f32(bias), _f32(mean), _f32(var)
+    fused = np.empty(Cc, dtype=np.float32)
+    load().oracle_batchnorm_fused_scale(_ptr(fused), _ptr(scale), _ptr(var), Cc, C.c_float(eps))
+    Y = np.empty_like(X)
+    load().oracle_batchnorm(_ptr(Y), _ptr(X), _ptr(fused), _ptr(mean), _ptr(bias), X.shape[0], Cc, int(np.prod(X.shape[2:])), relu)
+    return Y, fused
+
+
 def global_avg_pool_i8(X, scale):
     X = np.ascontiguousarray(X, dtype=np.int8)
     N, Cc = X.shape[:2]

@@ -286,6 +286,29 @@ ORACLE_API void oracle_global_avg_pool(float *Y, const float *X, int NC, int HW)
    }
 }
 
+/* BatchNormalization at inference (core/inc/SOFIE/operators/ROperator_BatchNormalization.hxx:92-109, 139-148):
+ * Initialize forms fused_scale[c] = scale[c] / sqrt(var[c] + eps) once; the generated loop computes
+ * val = (x - mean[c]) * fused_scale[c] + bias[c], then `val > 0 ? val : 0` when a Relu was fused. */
+ORACLE_API void oracle_batchnorm_fused_scale(float *fused, const float *scale, const float *var, int C, float eps)
+{
+   for (int c = 0; c < C; ++c)
+      fused[c] = scale[c] / sqrtf(var[c] + eps);
+}
+ORACLE_API void oracle_batchnorm(float *Y, const float *X, const float *fused_scale, const float *mean, const float *bias, int N, int C,
+                                 int spatial, int relu)
+{
+   size_t i = 0;
+   for (int n = 0; n < N; ++n)
+      for (int c = 0; c < C; ++c) {
+         const float mean_val = mean[c], fused_scale_val = fused_scale[c], bias_val = bias[c];
+         for (int sp = 0; sp < spatial; ++sp) {
+            float val = (X[i] - mean_val) * fused_scale_val + bias_val;
+            Y[i] = relu ? ((val > 0.0f) ? val : 0.0f) : val;
+            i++;
+         }
+      }
+}
+
 /* ------------------------------------------------------------------------------------------------
  * Memory planner: OrganizeMemory (core/inc/SOFIE/utils/shared/MemoryPlanner.inc:33-132).
  * Tensor i lives in [begin[i], end[i]); events are swept in time order with frees (type 0) before

@@ -186,6 +186,21 @@ __global__ __launch_bounds__(256) void gap_i8_nhwc_vec_kernel(float *__restrict_
    }
 }
 
+// Y = (X - mean[c]) * fused_scale[c] + bias[c] (+ relu); element i belongs to channel (i / spatial) % C
+__global__ __launch_bounds__(256) void batchnorm_f32_kernel(float *__restrict__ Y, const float *__restrict__ X,
+                                                             const float *__restrict__ fused, const float *__restrict__ mean,
+                                                             const float *__restrict__ bias, size_t n, int C, int spatial, int relu)
+{
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+      const int c = (int)((i / (size_t)spatial) % (size_t)C);
+      float v = __fmul_rn(X[i] - mean[c], fused[c]) + bias[c];
+      if (relu)
+         v = v > 0.0f ? v : 0.0f;
+      Y[i] = v;
+   }
+}
+
 } // namespace sofie_hip
 
 using namespace sofie_hip;
@@ -261,6 +276,19 @@ int sofie_hip_add_f32(sofie_hip_ctx *ctx, const sofie_add_desc *d)
    SOFIE_HIP_REQUIRE(d->A && d->B && d->Y, "sofie_hip_add_f32: NULL pointer");
    hipLaunchKernelGGL(add_f32_kernel, dim3(grid_for(n)), dim3(256), 0, ctx->stream, d->Y, d->A, d->B, n, sh);
    return launch_status("add_f32_kernel");
+}
+
+int sofie_hip_batchnorm_f32(sofie_hip_ctx *ctx, float *Y, const float *X, const float *fused_scale, const float *mean,
+                            const float *bias, int32_t N, int32_t C, int32_t spatial, int32_t relu)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_batchnorm_f32: ctx is NULL");
+   SOFIE_HIP_REQUIRE(N >= 0 && C > 0 && spatial > 0, "sofie_hip_batchnorm_f32: bad shape");
+   if (N == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(Y && X && fused_scale && mean && bias, "sofie_hip_batchnorm_f32: NULL pointer");
+   const size_t n = (size_t)N * (size_t)C * (size_t)spatial;
+   hipLaunchKernelGGL(batchnorm_f32_kernel, dim3(grid_for(n)), dim3(256), 0, ctx->stream, Y, X, fused_scale, mean, bias, n, C, spatial, relu);
+   return launch_status("batchnorm_f32_kernel");
 }
 
 int sofie_hip_global_avg_pool_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t NC, int32_t HW)

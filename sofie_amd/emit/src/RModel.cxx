@@ -186,6 +186,11 @@ void RModel::FuseGemmActivations()
                c->FuseActivation(act->Activation(), act->Alpha(), act->OutputName());
                changed = true;
             }
+         } else if (auto *bn = dynamic_cast<ROperator_BatchNormalization<float> *>(op)) {
+            if (act && act->Activation() == EActivationType::RELU && !bn->HasActivation()) {
+               bn->FuseRelu(act->OutputName());
+               changed = true;
+            }
          } else if (auto *qc = dynamic_cast<ROperator_QConv *>(op)) {
             if (act && act->Activation() == EActivationType::RELU && !qc->HasRelu()) {
                qc->FuseRelu(act->OutputName());

@@ -395,6 +395,12 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          model->AddOperator(std::make_unique<ROperator_QuantizeLinear>(n.in[0], n.in[1], n.out[0]));
       } else if (n.op == "DequantizeLinear") {
          model->AddOperator(std::make_unique<ROperator_DequantizeLinear>(n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "BatchNormalization") {
+         if (n.in.size() != 5)
+            throw std::runtime_error("SOFIE ONNX parser: BatchNormalization " + n.name + " needs 5 inputs");
+         model->AddOperator(std::make_unique<ROperator_BatchNormalization<float>>(attrF(n, "epsilon", 1e-5f), attrF(n, "momentum", 0.9f),
+                                                                                   (size_t)attrI(n, "training_mode", 0), n.in[0], n.in[1], n.in[2],
+                                                                                   n.in[3], n.in[4], n.out[0]));
       } else if (n.op == "QLinearConv") {
          if (n.in.size() < 8)
             throw std::runtime_error("SOFIE ONNX parser: QLinearConv " + n.name + " needs 8 or 9 inputs");

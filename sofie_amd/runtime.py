@@ -99,6 +99,7 @@ SYMBOLS = {
     "sofie_hip_conv_i8_workspace": (C.c_size_t, [C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
     "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),
     "sofie_hip_global_avg_pool_f32": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32]),
+    "sofie_hip_batchnorm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "sofie_hip_global_avg_pool_i8": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float]),
     "sofie_hip_conv_weight_i8_packed_bytes": (C.c_size_t, [C.POINTER(ConvDesc)]),
     "sofie_hip_mfma_i8_probe": (C.c_int, [_P, _P, C.c_size_t, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),

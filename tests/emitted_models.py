@@ -115,7 +115,22 @@ def int8_cnn(batch=2, hw=12, channels=(3, 64, 128, 256, 256), n_out=10):
                 init=init, feeds=[m["x"]], consts=m)
 
 
+def conv_batchnorm_relu(batch=2):
+    """Conv 3x3 -> BatchNormalization (kept at run time) -> Relu -> GlobalAveragePool: a model whose normalisation
+    arrives un-folded."""
+    init = {"W": util.normal(6101, 8 * 3 * 9, 0.3).reshape(8, 3, 3, 3),
+            "gamma": (0.5 + util.uniform01(6102, 8)).astype(np.float32), "beta": util.normal(6103, 8, 0.2),
+            "mean": util.normal(6104, 8, 0.5), "var": (0.2 + util.uniform01(6105, 8)).astype(np.float32)}
+    nodes = [ow.node("Conv", ["X", "W"], ["C"], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1]),
+             ow.node("BatchNormalization", ["C", "gamma", "beta", "mean", "var"], ["N"], epsilon=1e-3),
+             ow.node("Relu", ["N"], ["R"]),
+             ow.node("GlobalAveragePool", ["R"], ["Y"])]
+    X = util.normal(6001, batch * 3 * 10 * 10).reshape(batch, 3, 10, 10)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 3, 10, 10])], outputs=[("Y", np.float32, [batch, 8, 1, 1])], init=init, feeds=[X])
+
+
 CONFIG_MODELS = {
+    "ConvBatchNormRelu": lambda: conv_batchnorm_relu(2),
     "Config5_int8_CNN_small": lambda: int8_cnn(2, 12),
     "Config1_fp32_MLP": lambda: fp32_mlp(64),
     "Config2_int8_MLP_small": lambda: int8_mlp([64, 128, 96, 32], 48),

@@ -215,6 +215,9 @@ def run(g, inputs, be):
                 y = y[:, :, 0, :]
         elif op == "GlobalAveragePool":
             y = be.gap(x[0])
+        elif op == "BatchNormalization":
+            from oracle import binding as ob
+            y, _ = ob.batchnorm(x[0], x[1], x[2], x[3], x[4], eps=a.get("epsilon", 1e-5))
         elif op == "Add":
             y = be.add(x[0], x[1])
         else:

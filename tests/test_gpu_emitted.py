@@ -115,3 +115,14 @@ def test_custom_memory_sessions(rt):
     text = report.value.decode()
     print(text)
     assert failures == 0 and "FAIL" not in text and text.count("ok ") >= 14
+
+
+def test_emitted_conv_batchnorm_relu(rt):
+    spec = em.conv_batchnorm_relu(2)
+    g = onnx_lite.load(os.path.join(em.OUT, "ConvBatchNormRelu.onnx"))
+    want = gr.run(g, spec["feeds"], gr.OracleBackend()).ravel()
+    print("emitted ConvBatchNormRelu", flush=True)
+    got = run_emitted("ConvBatchNormRelu", spec["feeds"], want.size)
+    assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+    txt = open(os.path.join(em.OUT, "ConvBatchNormRelu_GPU_HIP.hxx")).read()
+    assert "BatchNorm + ReLU" in txt and "sofie_hip_unary_f32" not in txt   # the Relu is folded into the normalisation

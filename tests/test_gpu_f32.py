@@ -176,3 +176,21 @@ def test_global_avg_pool(rt):
     rt.sync()
     want = ob.global_avg_pool(X.reshape(3, 7, 33, 1)).reshape(21)
     assert np.allclose(util.to_host(dY), want, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape", [(4, 6), (3, 5, 7), (2, 8, 5, 6), (1, 1, 1, 1)])
+@pytest.mark.parametrize("relu", [0, 1])
+def test_batchnorm_same_three_roundings_as_the_cpu_loop(rt, shape, relu):
+    Cc = shape[1]
+    X = util.normal(90, int(np.prod(shape))).reshape(shape)
+    gamma, beta = (0.5 + util.uniform01(91, Cc)).astype(np.float32), util.normal(92, Cc)
+    mean, var = util.normal(93, Cc, 0.3), (0.1 + util.uniform01(94, Cc)).astype(np.float32)
+    want, fused = ob.batchnorm(X, gamma, beta, mean, var, eps=1e-5, relu=relu)
+    dX, dF, dM, dB = util.to_dev(X), util.to_dev(fused), util.to_dev(mean), util.to_dev(beta)
+    dY = util.dev_empty(shape, np.float32)
+    import torch
+    torch.cuda.synchronize()
+    rt.call("sofie_hip_batchnorm_f32", util.ptr(dY), util.ptr(dX), util.ptr(dF), util.ptr(dM), util.ptr(dB), shape[0], Cc,
+            int(np.prod(shape[2:])), relu)
+    rt.sync()
+    assert np.array_equal(util.to_host(dY).view(np.uint32), want.view(np.uint32))

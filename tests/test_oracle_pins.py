@@ -288,3 +288,21 @@ def test_global_avg_pool_i8():
     got = ob.global_avg_pool_i8(X, np.float32(0.05))
     want = (X.astype(np.int64).sum(-1).astype(np.float32) * np.float32(0.05)) / np.float32(20)
     assert np.array_equal(got, want)
+
+
+def test_batchnorm_closed_forms():
+    # x == mean gives the bias; gamma == sqrt(var + eps) gives x - mean + bias; float64 arbiter for the general case
+    Cc = 5
+    mean, beta = util.normal(301, Cc), util.normal(302, Cc)
+    var = (0.2 + util.uniform01(303, Cc)).astype(np.float32)
+    X = np.broadcast_to(mean[None, :, None], (3, Cc, 4)).copy()
+    y, _ = ob.batchnorm(X, np.ones(Cc, np.float32), beta, mean, var)
+    assert np.array_equal(y, np.broadcast_to(beta[None, :, None], y.shape))
+    X = util.normal(304, 3 * Cc * 4).reshape(3, Cc, 4)
+    gamma = util.normal(305, Cc)
+    y, fused = ob.batchnorm(X, gamma, beta, mean, var, eps=1e-3)
+    ref = (X.astype(np.float64) - mean[None, :, None]) * (gamma.astype(np.float64) / np.sqrt(var.astype(np.float64) + 1e-3))[None, :, None] + beta[None, :, None]
+    assert np.abs(y - ref).max() <= 1e-6 * (1 + np.abs(ref).max())
+    assert np.allclose(fused, gamma / np.sqrt(var + np.float32(1e-3)), rtol=1e-6)
+    yr, _ = ob.batchnorm(X, gamma, beta, mean, var, eps=1e-3, relu=1)
+    assert np.array_equal(yr, np.where(y > 0, y, np.float32(0)))
