@@ -66,6 +66,7 @@ __device__ __forceinline__ float gelu_erf_fast(float v)
 }
 
 struct F8Epilogue {
+   static constexpr bool kConvertInRegisters = false; // activation (erf, tanh, exp) + bf16 rounding per element: keep the code once
    const float *bias;
    float scale;
    int act, out;

@@ -7,6 +7,7 @@
 namespace sofie_hip {
 
 struct I8Epilogue {
+   static constexpr bool kConvertInRegisters = true; // a handful of integer / fp32 instructions per element
    const int32_t *bias;
    const float *scale;
    float scale_scalar;

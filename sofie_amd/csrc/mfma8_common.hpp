@@ -214,8 +214,8 @@ constexpr int tile_store_lds_bytes(int TN) { return 32 * (TN * 4 + 16); }
 //   bool rows_vectorizable() const                row-major output whose rows allow 16-byte stores
 //   char *out_base() const;  size_t out_index(int m, int n) const     element index of (m,n)
 template <int MODE, int MT, int NT, class EPI, class ACC>
-__device__ __forceinline__ void tile_store_via_lds(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int M, int N,
-                                                   int lane, char *wsm)
+__device__ __forceinline__ void tile_store_convert_first(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int M, int N,
+                                                        int lane, char *wsm)
 {
    constexpr int ESZ = EPI::template out_bytes<MODE>();
    constexpr int TN = NT * 32;
@@ -306,6 +306,108 @@ __device__ __forceinline__ void tile_store_via_lds(const EPI &ep, ACC (&acc)[MT]
       }
       __builtin_amdgcn_wave_barrier();
    });
+}
+
+// The other order, for stores whose conversion is long (an erf per element): the raw 32-bit accumulators are parked and
+// the conversion runs in the run-time loop of the re-read, so its code exists once instead of once per accumulator
+// register.  (Unrolled over the 256 accumulators of a 256 x 256 tile, a GELU store is 80 KB of straight-line code that
+// is executed once per tile: every instruction is an instruction-cache miss.)
+template <int MODE, int MT, int NT, class EPI, class ACC>
+__device__ __forceinline__ void tile_store_convert_after(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int M, int N,
+                                                   int lane, char *wsm)
+{
+   typedef typename std::remove_reference<decltype(acc[0][0][0])>::type elem_t;
+   constexpr int ESZ = EPI::template out_bytes<MODE>();
+   constexpr int TN = NT * 32;
+   constexpr int ROWB = TN * 4 + 16;
+   const int lr = lane & 31, lk = lane >> 5;
+   char *out = ep.out_base();
+   const bool vec = ep.rows_vectorizable();
+   static_for<MT>([&](auto ci) {
+      constexpr int i = decltype(ci)::value;
+      static_for<NT>([&](auto cj) {
+         constexpr int j = decltype(cj)::value;
+         static_for<4>([&](auto cg) {
+            constexpr int g = decltype(cg)::value;
+            typedef elem_t v4e __attribute__((ext_vector_type(4)));
+            *(v4e *)(wsm + lr * ROWB + (j * 32 + g * 8 + lk * 4) * 4) =
+               v4e{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+         });
+      });
+      __builtin_amdgcn_wave_barrier();
+      const int m_first = m_base + i * 32;
+      if (vec) {
+         constexpr int CPL = 16 / ESZ;     // columns per lane
+         constexpr int LPR = TN / CPL;     // lanes per row
+         constexpr int RPP = 64 / LPR;     // rows per pass
+         static_assert(TN % CPL == 0 && LPR <= 64 && 32 % RPP == 0, "wave tile width not supported by the tile store");
+         const int c0 = (lane % LPR) * CPL;
+         const int n = n_base + c0;
+         typename EPI::template col_params<CPL> prm;
+         ep.template load_params<CPL>(n < N ? n : N - 1, prm);
+#pragma unroll 1
+         for (int row0 = 0; row0 < 32; row0 += RPP) {
+            const int row = row0 + lane / LPR;
+            const int m = m_first + row;
+            if (m < M && n < N) {
+               uint32_t w[4];
+#pragma unroll
+               for (int q = 0; q < CPL / 4; ++q) {
+                  typedef elem_t v4e __attribute__((ext_vector_type(4)));
+                  const v4e a = *(const v4e *)(wsm + row * ROWB + (c0 + 4 * q) * 4);
+                  ep.template pack4<MODE, CPL>(prm, q, a[0], a[1], a[2], a[3], w + q * ESZ);
+               }
+               char *y = out + ep.out_index(m, n) * ESZ;
+               if (n + CPL <= N) {
+                  *(uint4 *)y = make_uint4(w[0], w[1], w[2], w[3]);
+               } else {
+                  const char *src = (const char *)w;
+                  for (int b = 0; b < (N - n) * ESZ; ++b)
+                     y[b] = src[b];
+               }
+            }
+         }
+      } else {
+         // any layout: a lane converts 4 columns and stores them one element at a time
+         constexpr int LPR = TN / 4;
+         constexpr int RPP = (64 / LPR) > 0 ? (64 / LPR) : 1;
+         static_assert(LPR <= 64, "wave tile too wide");
+         const int c0 = (lane % LPR) * 4;
+         const int n = n_base + c0;
+         typename EPI::template col_params<4> prm;
+         ep.template load_params<4>(n < N ? n : N - 1, prm);
+#pragma unroll 1
+         for (int row0 = 0; row0 < 32; row0 += RPP) {
+            const int row = row0 + lane / LPR;
+            const int m = m_first + row;
+            if (m < M && n < N) {
+               typedef elem_t v4e __attribute__((ext_vector_type(4)));
+               const v4e a = *(const v4e *)(wsm + row * ROWB + c0 * 4);
+               uint32_t w[4];
+               ep.template pack4<MODE, 4>(prm, 0, a[0], a[1], a[2], a[3], w);
+               const char *src = (const char *)w;
+               for (int e = 0; e < 4 && n + e < N; ++e) {
+                  char *y = out + ep.out_index(m, n + e) * ESZ;
+                  for (int b = 0; b < ESZ; ++b)
+                     y[b] = src[e * ESZ + b];
+               }
+            }
+         }
+      }
+      __builtin_amdgcn_wave_barrier();
+   });
+}
+
+
+// EPI::kConvertInRegisters picks the order: true for the short integer conversions, false for long ones.
+template <int MODE, int MT, int NT, class EPI, class ACC>
+__device__ __forceinline__ void tile_store_via_lds(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int M, int N,
+                                                   int lane, char *wsm)
+{
+   if constexpr (EPI::kConvertInRegisters)
+      tile_store_convert_first<MODE, MT, NT>(ep, acc, m_base, n_base, M, N, lane, wsm);
+   else
+      tile_store_convert_after<MODE, MT, NT>(ep, acc, m_base, n_base, M, N, lane, wsm);
 }
 
 int transpose_i8(hipStream_t stream, int8_t *dst, const int8_t *src, int rows, int cols, int ld_src, int ld_dst);
