@@ -89,6 +89,7 @@ private:
    void PlanMemory();
    void GenerateSessionCode(std::underlying_type_t<Options> options);
    void WriteWeightFile(const std::string &filename) const;
+   void WriteSafetensorsFile(const std::string &filename) const;
 
    std::string fName = "Model";
    std::vector<std::string> fInputTensorNames;
@@ -102,6 +103,7 @@ private:
    std::unordered_map<std::string, int> fTensorLayout;
    std::size_t fArenaBytes = 0, fPoolBytes = 0;
    bool fInitialized = false;
+   bool fSafetensors = false;
    std::string fGC;
    std::string fWeightFileName;
 

@@ -14,7 +14,8 @@ namespace SOFIE_HIP {
 class RModelParser_ONNX {
 public:
    // throws std::runtime_error for an operator outside the path ("... is not yet supported")
-   std::unique_ptr<RModel> Parse(std::string filename, bool verbose = false);
+   // modelName: name of the generated namespace and files (default: the file's stem)
+   std::unique_ptr<RModel> Parse(std::string filename, bool verbose = false, std::string modelName = "");
 };
 
 } // namespace SOFIE_HIP

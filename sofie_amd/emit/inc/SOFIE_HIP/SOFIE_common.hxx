@@ -28,6 +28,7 @@ enum class EActivationType { UNDEFINED, RELU, LEAKYRELU, SIGMOID, GELU, GELU_TAN
 enum class Options {
    kDefault = 0x0,
    kNoWeightFile = 0x2,
+   kSafetensorsWeightFile = 0x100,
    kExternalStream = 0x400,
    kCustomMemory = 0x800,
 };

@@ -371,11 +371,272 @@ inline void ReadTensorFromStream(std::istream &is, std::vector<T> &target, std::
 } // namespace detail
 )SOFIE";
 
+
+// Weights in the safetensors container (the reference's Options::kSafetensorsWeightFile, core/src/RModel.cxx:1967-2010):
+// 8 bytes little-endian header length, a JSON header {"tensor_<name>": {"dtype": "F32", "shape": [..], "data_offsets": [b, e]}, ...},
+// then the raw little-endian tensor bytes.
+static const char *kSafetensorsHelpers = R"SOFIE(
+struct SafetensorsBlob {
+   const char *data = nullptr;
+   std::size_t size = 0;
+   SafetensorsBlob() = default;
+   SafetensorsBlob(const char *d, std::size_t n) : data(d), size(n) {}
+   SafetensorsBlob(const std::string &s) : data(s.data()), size(s.size()) {}
+};
+
+namespace detail {
+inline std::string LoadWeightsFromFile(const std::string &filename)
+{
+   std::ifstream f(filename, std::ios::binary);
+   if (!f.is_open())
+      throw std::runtime_error("tmva-sofie failed to open file " + filename + " for input weights");
+   std::string bytes((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+   if (f.bad())
+      throw std::runtime_error("tmva-sofie failed to read file " + filename);
+   return bytes;
+}
+
+// Reads the header of a safetensors payload once; Expect() checks a tensor against what the model needs,
+// Data() returns where its bytes start.  Every inconsistency is a std::runtime_error naming the tensor.
+class SafetensorsReader {
+public:
+   explicit SafetensorsReader(SafetensorsBlob blob)
+   {
+      if (!blob.data || blob.size < 8)
+         throw std::runtime_error("SOFIE safetensors: the payload is shorter than its 8-byte header length");
+      std::uint64_t n = 0;
+      for (int i = 0; i < 8; ++i)
+         n |= static_cast<std::uint64_t>(static_cast<unsigned char>(blob.data[i])) << (8 * i);
+      if (n > blob.size - 8)
+         throw std::runtime_error("SOFIE safetensors: the header length exceeds the payload");
+      fText = blob.data + 8;
+      fEnd = fText + n;
+      fPayload = blob.data + 8 + n;
+      fPayloadBytes = blob.size - 8 - n;
+      const char *p = fText;
+      Space(p);
+      Take(p, '{');
+      Space(p);
+      if (p < fEnd && *p == '}')
+         return;
+      for (;;) {
+         Space(p);
+         const std::string name = String(p);
+         Space(p);
+         Take(p, ':');
+         Space(p);
+         if (name == "__metadata__") {
+            SkipValue(p);
+         } else {
+            if (fEntries.count(name))
+               throw std::runtime_error("SOFIE safetensors: tensor " + name + " appears twice");
+            fEntries[name] = Entry(p, name);
+         }
+         Space(p);
+         if (p < fEnd && *p == ',') {
+            ++p;
+            continue;
+         }
+         Take(p, '}');
+         break;
+      }
+   }
+   void Expect(const std::string &name, const char *dtype, std::size_t elemBytes, std::size_t count) const
+   {
+      auto f = fEntries.find(name);
+      if (f == fEntries.end())
+         throw std::runtime_error("SOFIE safetensors: tensor " + name + " is missing");
+      const Info &e = f->second;
+      if (e.dtype != dtype)
+         throw std::runtime_error("SOFIE safetensors: tensor " + name + " has dtype " + e.dtype + ", the model needs " + dtype);
+      std::uint64_t len = 1;
+      for (auto d : e.shape)
+         len *= d;
+      if (len != count)
+         throw std::runtime_error("SOFIE safetensors: tensor " + name + " has " + std::to_string(len) + " elements, the model needs " +
+                                  std::to_string(count));
+      if (e.end < e.begin || e.end > fPayloadBytes || e.end - e.begin != count * elemBytes)
+         throw std::runtime_error("SOFIE safetensors: tensor " + name + " has data offsets that do not match its size");
+   }
+   const char *Data(const std::string &name) const { return fPayload + fEntries.at(name).begin; }
+
+private:
+   struct Info {
+      std::string dtype;
+      std::vector<std::uint64_t> shape;
+      std::uint64_t begin = 0, end = 0;
+   };
+   [[noreturn]] void Bad(const std::string &what) const { throw std::runtime_error("SOFIE safetensors: malformed header: " + what); }
+   void Space(const char *&p) const
+   {
+      while (p < fEnd && (*p == ' ' || *p == '\n' || *p == '\t' || *p == '\r'))
+         ++p;
+   }
+   void Take(const char *&p, char c) const
+   {
+      if (p >= fEnd || *p != c)
+         Bad(std::string("expected '") + c + "'");
+      ++p;
+   }
+   std::string String(const char *&p) const
+   {
+      Take(p, '"');
+      std::string s;
+      while (p < fEnd && *p != '"') {
+         if (*p == '\\') {
+            if (++p >= fEnd)
+               Bad("unterminated string");
+            if (*p == 'u') { // \uXXXX: tensor names of this backend are ASCII; keep the escape verbatim
+               s += "\\u";
+               ++p;
+               continue;
+            }
+            s.push_back(*p == 'n' ? '\n' : *p == 't' ? '\t' : *p);
+            ++p;
+            continue;
+         }
+         s.push_back(*p++);
+      }
+      Take(p, '"');
+      return s;
+   }
+   std::uint64_t Number(const char *&p) const
+   {
+      if (p >= fEnd || *p < '0' || *p > '9')
+         Bad("expected a non-negative integer");
+      std::uint64_t v = 0;
+      while (p < fEnd && *p >= '0' && *p <= '9') {
+         if (v > (~std::uint64_t(0) - 9) / 10)
+            Bad("number too large");
+         v = v * 10 + static_cast<std::uint64_t>(*p++ - '0');
+      }
+      return v;
+   }
+   std::vector<std::uint64_t> Numbers(const char *&p) const
+   {
+      std::vector<std::uint64_t> v;
+      Take(p, '[');
+      Space(p);
+      if (p < fEnd && *p == ']') {
+         ++p;
+         return v;
+      }
+      for (;;) {
+         Space(p);
+         v.push_back(Number(p));
+         Space(p);
+         if (p < fEnd && *p == ',') {
+            ++p;
+            continue;
+         }
+         Take(p, ']');
+         return v;
+      }
+   }
+   void SkipValue(const char *&p) const
+   {
+      Space(p);
+      if (p >= fEnd)
+         Bad("unexpected end");
+      if (*p == '"') {
+         String(p);
+      } else if (*p == '{' || *p == '[') {
+         const char close = *p == '{' ? '}' : ']';
+         ++p;
+         Space(p);
+         if (p < fEnd && *p == close) {
+            ++p;
+            return;
+         }
+         for (;;) {
+            Space(p);
+            if (close == '}') {
+               String(p);
+               Space(p);
+               Take(p, ':');
+            }
+            SkipValue(p);
+            Space(p);
+            if (p < fEnd && *p == ',') {
+               ++p;
+               continue;
+            }
+            Take(p, close);
+            return;
+         }
+      } else {
+         while (p < fEnd && *p != ',' && *p != '}' && *p != ']')
+            ++p;
+      }
+   }
+   Info Entry(const char *&p, const std::string &name) const
+   {
+      Info e;
+      bool haveType = false, haveShape = false, haveOffsets = false;
+      Take(p, '{');
+      for (;;) {
+         Space(p);
+         const std::string key = String(p);
+         Space(p);
+         Take(p, ':');
+         Space(p);
+         if (key == "dtype") {
+            e.dtype = String(p);
+            haveType = true;
+         } else if (key == "shape") {
+            e.shape = Numbers(p);
+            haveShape = true;
+         } else if (key == "data_offsets") {
+            auto o = Numbers(p);
+            if (o.size() != 2)
+               Bad("data_offsets of " + name + " must have two entries");
+            e.begin = o[0];
+            e.end = o[1];
+            haveOffsets = true;
+         } else {
+            SkipValue(p);
+         }
+         Space(p);
+         if (p < fEnd && *p == ',') {
+            ++p;
+            continue;
+         }
+         Take(p, '}');
+         break;
+      }
+      if (!haveType || !haveShape || !haveOffsets)
+         Bad("tensor " + name + " lacks dtype, shape or data_offsets");
+      return e;
+   }
+   const char *fText = nullptr, *fEnd = nullptr, *fPayload = nullptr;
+   std::size_t fPayloadBytes = 0;
+   std::map<std::string, Info> fEntries;
+};
+} // namespace detail
+)SOFIE";
+
+static std::string SafetensorsDType(ETensorType t)
+{
+   switch (t) {
+   case ETensorType::FLOAT: return "F32";
+   case ETensorType::DOUBLE: return "F64";
+   case ETensorType::INT64: return "I64";
+   case ETensorType::INT32: return "I32";
+   case ETensorType::INT8: return "I8";
+   case ETensorType::UINT8: return "U8";
+   case ETensorType::BOOL: return "BOOL";
+   case ETensorType::FLOAT8E4M3FN: return "F8_E4M3";
+   default: throw std::runtime_error("sofie tensor with type " + ConvertTypeToString(t) + " cannot be written to a safetensors file");
+   }
+}
+
 void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
 {
    const bool externalStream = options & static_cast<std::underlying_type_t<Options>>(Options::kExternalStream);
    const bool noWeightFile = options & static_cast<std::underlying_type_t<Options>>(Options::kNoWeightFile);
    const bool customMemory = options & static_cast<std::underlying_type_t<Options>>(Options::kCustomMemory);
+   const bool safetensors = !noWeightFile && (options & static_cast<std::underlying_type_t<Options>>(Options::kSafetensorsWeightFile));
+   fSafetensors = safetensors;
    std::stringstream gc;
    std::string guard = "SOFIE_" + fName;
    std::transform(guard.begin(), guard.end(), guard.begin(), [](unsigned char c) { return std::toupper(c); });
@@ -385,8 +646,12 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
          "#include <tuple>\n#include <type_traits>\n#include <vector>\n#include \"sofie_hip.h\"\n";
    if (customMemory)
       gc << "#include <functional>\n";
+   if (safetensors)
+      gc << "#include <iterator>\n#include <map>\n";
    gc << "\n";
    gc << "namespace SOFIE_" << fName << " {\n" << kRuntimeHelpers << "\n";
+   if (safetensors)
+      gc << kSafetensorsHelpers << "\n";
    if (customMemory) {
       // the reference's contract for caller-owned device memory (core/src/utils/SOFIE_common_helpers.cxx:741-804):
       // alloc is called once for the whole block, assign (optional) maps an offset of the plan to an address, dealloc
@@ -411,11 +676,29 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
          << (p.pooled ? ", live [" + std::to_string(p.begin) + "," + std::to_string(p.end) + ")" : "") << "\n";
    gc << "\n";
    // constructor
-   gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "std::string filename = \""
-      << (noWeightFile ? "" : fName + "_GPU_HIP.dat") << "\"" << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
+   if (safetensors) {
+      // the file is read whole and handed to the constructor that takes the payload
+      gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "std::string filename = \"" << fName << "_GPU_HIP.safetensors\""
+         << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
+      gc << "      : Session(" << (customMemory ? "std::move(provider), " : "") << "SafetensorsBlob(detail::LoadWeightsFromFile(filename))"
+         << (externalStream ? ", stream" : "") << ", device)\n   {\n   }\n";
+      gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "SafetensorsBlob weights_blob"
+         << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
+   } else {
+      gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "std::string filename = \""
+         << (noWeightFile ? "" : fName + "_GPU_HIP.dat") << "\"" << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
+   }
    if (customMemory)
       gc << "      : fProvider(std::move(provider))\n";
    gc << "   {\n";
+   if (safetensors) {
+      // the payload is checked against the model before any device work
+      gc << "      detail::SafetensorsReader sofie_weights_reader(weights_blob);\n";
+      for (auto &kv : fInitializedTensors)
+         if (!kv.second.constant)
+            gc << "      sofie_weights_reader.Expect(\"tensor_" << kv.first << "\", \"" << SafetensorsDType(kv.second.type) << "\", "
+               << GetTypeSize(kv.second.type) << ", " << ConvertShapeToLength(kv.second.shape) << ");\n";
+   }
    if (customMemory)
       gc << "      if (!fProvider.alloc)\n         throw std::runtime_error(\"SOFIE HIP Session: the memory provider has no alloc function\");\n";
    gc << "      detail::Check(sofie_hip_ctx_create(&fCtx, device, " << (externalStream ? "stream" : "nullptr") << "), \"Session\");\n";
@@ -440,7 +723,18 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    bool anyWeights = false, anyConstants = false;
    for (auto &kv : fInitializedTensors)
       (kv.second.constant ? anyConstants : anyWeights) = true;
-   if (anyWeights && !noWeightFile) {
+   if (anyWeights && safetensors) {
+      gc << "         // upload the weights straight from the payload\n";
+      for (auto &kv : fInitializedTensors) {
+         if (kv.second.constant)
+            continue;
+         const std::size_t bytes = ConvertShapeToLength(kv.second.shape) * GetTypeSize(kv.second.type);
+         if (bytes)
+            gc << "         detail::Check(sofie_hip_upload(fCtx, tensor_" << kv.first << ", sofie_weights_reader.Data(\"tensor_" << kv.first << "\"), "
+               << bytes << "), \"upload of tensor_" << kv.first << "\");\n";
+      }
+      gc << "         detail::Check(sofie_hip_sync(fCtx), \"upload of the weights\");\n";
+   } else if (anyWeights && !noWeightFile) {
       gc << "         // read and upload the weights\n";
       gc << "         std::ifstream f;\n         f.open(filename);\n";
       gc << "         if (!f.is_open()) {\n            throw std::runtime_error(\"tmva-sofie failed to open file \" + filename + \" for input weights\");\n         }\n";
@@ -642,7 +936,57 @@ void RModel::OutputGenerated(std::string filename)
    auto dot = dat.find_last_of('.');
    if (dot != std::string::npos)
       dat = dat.substr(0, dot);
-   WriteWeightFile(dat + ".dat");
+   if (fSafetensors)
+      WriteSafetensorsFile(dat + ".safetensors");
+   else
+      WriteWeightFile(dat + ".dat");
+}
+
+void RModel::WriteSafetensorsFile(const std::string &filename) const
+{
+   const std::uint16_t one = 1;
+   if (!*reinterpret_cast<const std::uint8_t *>(&one))
+      throw std::runtime_error("sofie: safetensors weights can only be written on a little-endian host");
+   auto escape = [](const std::string &in) {
+      std::string out;
+      for (char c : in) {
+         if (c == '"' || c == '\\')
+            out.push_back('\\');
+         out.push_back(c);
+      }
+      return out;
+   };
+   std::string header = "{";
+   std::uint64_t offset = 0;
+   bool first = true;
+   for (auto &kv : fInitializedTensors) { // std::map: sorted by name, as the reference's writer sorts them
+      if (kv.second.constant)
+         continue;
+      const std::uint64_t nbytes = ConvertShapeToLength(kv.second.shape) * GetTypeSize(kv.second.type);
+      header += std::string(first ? "" : ",") + "\"" + escape("tensor_" + kv.first) + "\":{\"dtype\":\"" + SafetensorsDType(kv.second.type) +
+                "\",\"shape\":[";
+      for (std::size_t i = 0; i < kv.second.shape.size(); ++i)
+         header += (i ? "," : "") + std::to_string(kv.second.shape[i]);
+      header += "],\"data_offsets\":[" + std::to_string(offset) + "," + std::to_string(offset + nbytes) + "]}";
+      offset += nbytes;
+      first = false;
+   }
+   header += "}";
+   std::ofstream f(filename, std::ios::binary);
+   if (!f.is_open())
+      throw std::runtime_error("tmva-sofie failed to open file " + filename + " for tensor weight data");
+   char size8[8];
+   for (int i = 0; i < 8; ++i)
+      size8[i] = static_cast<char>((static_cast<std::uint64_t>(header.size()) >> (8 * i)) & 0xff);
+   f.write(size8, 8);
+   f.write(header.data(), header.size());
+   for (auto &kv : fInitializedTensors) {
+      if (kv.second.constant)
+         continue;
+      f.write(static_cast<const char *>(kv.second.data.get()), ConvertShapeToLength(kv.second.shape) * GetTypeSize(kv.second.type));
+   }
+   if (f.fail())
+      throw std::runtime_error("sofie failed to write safetensors payload");
 }
 
 } // namespace SOFIE_HIP

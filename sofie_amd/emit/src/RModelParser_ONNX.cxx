@@ -261,7 +261,7 @@ std::vector<size_t> ToSizes(const std::vector<int64_t> &v) { return std::vector<
 
 } // namespace
 
-std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verbose)
+std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verbose, std::string modelName)
 {
    std::ifstream in(filename, std::ios::binary);
    if (!in.is_open())
@@ -294,7 +294,7 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
             outputs.push_back(ParseValueInfo(f.bytes));
       }
    }
-   auto model = std::make_unique<RModel>(filename);
+   auto model = std::make_unique<RModel>(modelName.empty() ? filename : modelName);
    std::map<std::string, bool> isInit;
    for (auto &t : inits) {
       isInit[t.name] = true;

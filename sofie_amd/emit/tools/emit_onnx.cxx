@@ -1,4 +1,4 @@
-// sofie_hip_emit <model.onnx> <out_dir>: parses a model and writes <out_dir>/<Model>_GPU_HIP.hxx + .dat
+// sofie_hip_emit <model.onnx> <out_dir> [--safetensors] [--name N]: parses a model and writes <out_dir>/<Model>_GPU_HIP.hxx + .dat (or .safetensors)
 // (the flow of the reference's emitter template, tests/templates/EmitFromONNX.cxx.in:21-31).
 #include "SOFIE_HIP/RModelParser_ONNX.hxx"
 
@@ -7,15 +7,28 @@
 int main(int argc, char **argv)
 {
    if (argc < 3) {
-      std::cerr << "usage: " << argv[0] << " <model.onnx> <out_dir> [--plan]\n";
+      std::cerr << "usage: " << argv[0] << " <model.onnx> <out_dir> [--plan] [--safetensors] [--name <ModelName>]\n";
       return 2;
    }
    try {
       SOFIE_HIP::RModelParser_ONNX parser;
-      auto model = parser.Parse(argv[1]);
-      model->GenerateGPU_HIP();
+      bool plan = false, safetensors = false;
+      std::string name;
+      for (int i = 3; i < argc; ++i) {
+         const std::string a = argv[i];
+         if (a == "--plan")
+            plan = true;
+         else if (a == "--safetensors")
+            safetensors = true;
+         else if (a == "--name" && i + 1 < argc)
+            name = argv[++i];
+         else
+            throw std::runtime_error("unknown argument " + a);
+      }
+      auto model = parser.Parse(argv[1], false, name);
+      model->GenerateGPU_HIP(safetensors ? SOFIE_HIP::Options::kSafetensorsWeightFile : SOFIE_HIP::Options::kDefault);
       model->OutputGenerated(std::string(argv[2]) + "/" + model->GetName() + "_GPU_HIP.hxx");
-      if (argc > 3 && std::string(argv[3]) == "--plan") {
+      if (plan) {
          std::cout << "arena " << model->GetArenaBytes() << " pool " << model->GetIntermediateMemoryPoolSize() << "\n";
          for (auto &p : model->GetMemoryPlan())
             std::cout << p.name << " " << p.offset << " " << p.bytes << " " << p.begin << " " << p.end << " " << (p.pooled ? 1 : 0) << "\n";

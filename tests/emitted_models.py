@@ -182,8 +182,8 @@ def _run(cmd):
 API_MODELS = ("ApiGemmRelu", "ApiFp8Gemm")
 
 
-def emit_and_compile(model, onnx_path, n_inputs):
-    _run([EMIT, onnx_path, OUT])
+def emit_and_compile(model, onnx_path, n_inputs, *flags):
+    _run([EMIT, onnx_path, OUT] + list(flags))
     return compile_harness(model, n_inputs)
 
 
@@ -214,6 +214,8 @@ def build_all(jobs=8):
         p = os.path.join(OUT, m + ".onnx")
         ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)
         work.append((m, p, len(spec["inputs"])))
+    # the same model with its weights in a safetensors file
+    work.append(("Linear_16_st", os.path.join(GOLDEN, "models", "Linear_16.onnx"), 1, "--safetensors", "--name", "Linear_16_st"))
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(lambda w: emit_and_compile(*w), work))
     # models built through the RModel API (no ONNX file): sofie_hip_emit_example writes their headers

@@ -190,3 +190,66 @@ def test_custom_memory_header_allocates_nothing(emitted):
         assert "sofie_hip_arena_create" not in txt and "sofie_hip_arena_adopt(fCtx, fBlock, kArenaBytes)" in txt
         assert "struct MemoryProvider" in txt and "Session(MemoryProvider provider, std::string filename" in txt
     assert "void *stream = nullptr" in read(emitted, "CustomMemoryStreamChain")
+
+
+# ---- safetensors weights (the reference's Options::kSafetensorsWeightFile; its tests: tests/cpu/TestSafetensorsWeights.cxx) ----
+
+def _run_session(emitted, model, weights_path):
+    lib = ctypes.CDLL(os.path.join(emitted, "lib%s.so" % model))
+    err = ctypes.create_string_buffer(1024)
+    x = np.ones(1600, dtype=np.float32)
+    y = np.zeros(160, dtype=np.float32)
+    inp = (ctypes.c_void_p * 1)(x.ctypes.data)
+    rc = lib.run_model(str(weights_path).encode(), inp, y.ctypes.data_as(ctypes.c_void_p), ctypes.c_ulong(160), err, 1024)
+    return rc, err.value.decode(), y
+
+
+def test_safetensors_file_is_read_by_the_safetensors_library(emitted):
+    from safetensors.numpy import load_file
+    from tests import onnx_lite
+    got = load_file(os.path.join(emitted, "Linear_16_st_GPU_HIP.safetensors"))
+    g = onnx_lite.load(os.path.join(em.GOLDEN, "models", "Linear_16.onnx"))
+    assert len(got) == len(g["initializers"])
+    for k, v in g["initializers"].items():
+        key = "tensor_" + re.sub(r"[^A-Za-z0-9_]", "_", k)
+        assert got[key].dtype == np.float32 and got[key].shape == np.asarray(v).shape
+        assert np.array_equal(got[key].view(np.uint32), np.asarray(v, dtype=np.float32).view(np.uint32)), k
+
+
+def test_safetensors_payload_is_validated_before_any_device_work(emitted, tmp_path):
+    """Every inconsistency of the payload is reported by name, and a payload that passes goes on to the device
+    (which this machine may not have: then the error is the runtime's, not the reader's)."""
+    import torch
+    from safetensors.numpy import load_file, save_file
+    good = load_file(os.path.join(emitted, "Linear_16_st_GPU_HIP.safetensors"))
+
+    def attempt(tensors, **kw):
+        path = tmp_path / "w.safetensors"
+        save_file(tensors, str(path), **kw)
+        return _run_session(emitted, "Linear_16_st", path)
+
+    rc, msg, _ = _run_session(emitted, "Linear_16_st", tmp_path / "missing.safetensors")
+    assert rc == 1 and "failed to open file" in msg
+    missing = dict(good)
+    del missing["tensor_18_bias"]
+    rc, msg, _ = attempt(missing)
+    assert rc == 1 and "tensor_18_bias is missing" in msg
+    wrong_type = dict(good)
+    wrong_type["tensor_0_bias"] = good["tensor_0_bias"].astype(np.float64)
+    rc, msg, _ = attempt(wrong_type)
+    assert rc == 1 and "tensor_0_bias has dtype F64" in msg
+    wrong_size = dict(good)
+    wrong_size["tensor_0_weight"] = good["tensor_0_weight"][:-1]
+    rc, msg, _ = attempt(wrong_size)
+    assert rc == 1 and "tensor_0_weight has" in msg and "elements" in msg
+    raw = open(os.path.join(emitted, "Linear_16_st_GPU_HIP.safetensors"), "rb").read()
+    for name, blob, text in (("short", raw[:5], "shorter than"), ("cut", raw[:8] + raw[8:40], "exceeds the payload"),
+                             ("payload", raw[:-100], "data offsets"), ("json", raw[:8] + b"[" + raw[9:], "malformed header")):
+        p = tmp_path / (name + ".safetensors")
+        p.write_bytes(blob)
+        rc, msg, _ = _run_session(emitted, "Linear_16_st", p)
+        assert rc == 1 and text in msg, (name, msg)
+    # a file written by the safetensors library itself (other key order, spaces, a __metadata__ entry) passes the reader
+    rc, msg, _ = attempt(dict(reversed(list(good.items()))), metadata={"producer": "test"})
+    if not torch.cuda.is_available():
+        assert rc == 1 and "SOFIE HIP runtime error in Session" in msg

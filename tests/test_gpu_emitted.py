@@ -126,3 +126,22 @@ def test_emitted_conv_batchnorm_relu(rt):
     assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
     txt = open(os.path.join(em.OUT, "ConvBatchNormRelu_GPU_HIP.hxx")).read()
     assert "BatchNorm + ReLU" in txt and "sofie_hip_unary_f32" not in txt   # the Relu is folded into the normalisation
+
+
+def test_safetensors_session_reproduces_the_golden_output(rt, tmp_path):
+    from safetensors.numpy import load_file, save_file
+    g, inputs, expected = gr.load_fixture("Linear_16")
+    lib = ctypes.CDLL(os.path.join(em.OUT, "libLinear_16_st.so"))
+    x = np.ascontiguousarray(inputs[0], dtype=np.float32)
+    ptrs = (ctypes.c_void_p * 1)(x.ctypes.data)
+    # the file the generator wrote, and the same tensors re-saved by the safetensors library (with metadata)
+    own = os.path.join(em.OUT, "Linear_16_st_GPU_HIP.safetensors")
+    resaved = str(tmp_path / "resaved.safetensors")
+    save_file(dict(reversed(list(load_file(own).items()))), resaved, metadata={"producer": "test"})
+    for path in (own, resaved):
+        y = np.zeros(expected.size, dtype=np.float32)
+        err = ctypes.create_string_buffer(1024)
+        print("safetensors", path, flush=True)
+        rc = lib.run_model(path.encode(), ptrs, y.ctypes.data_as(ctypes.c_void_p), ctypes.c_ulong(y.size), err, 1024)
+        assert rc == 0, err.value.decode()
+        assert np.abs(y - expected).max() <= golden_tolerance("Linear_16", expected)
