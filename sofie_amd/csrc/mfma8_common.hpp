@@ -168,11 +168,15 @@ struct ConvRows {
          const int oh = r / OW, ow = r - oh * OW;
          const int ih0 = oh * stride_h - pad_h0, iw0 = ow * stride_w - pad_w0;
          off = ((n * H + ih0) * W + iw0) * C + cbyte;
+         int khi = 0, kwi = 0; // tap t = khi * kw + kwi, stepped without dividing
          for (int t = 0; t < ntaps; ++t) {
-            const int khi = t / kw, kwi = t - khi * kw;
             const int ih = ih0 + khi * dil_h, iw = iw0 + kwi * dil_w;
-            if (ih >= 0 && ih < H && iw >= 0 && iw < W)
+            if ((unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W)
                mask |= 1u << t;
+            if (++kwi == kw) {
+               kwi = 0;
+               ++khi;
+            }
          }
       }
       st.off[i] = off;
