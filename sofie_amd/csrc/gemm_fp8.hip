@@ -1,6 +1,6 @@
 // FP8 (OCP e4m3fn) GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x64_f8f6f4, fp32 accumulate) with
 // scale + bias + activation + bf16 conversion fused into the store, and the fp32 -> e4m3fn quantiser.
-#include "mfma8_gemm_pair.hpp"
+#include "mfma8_dispatch.hpp"
 #include <cstdlib>
 
 namespace sofie_hip {

@@ -2,7 +2,7 @@
 // optional relu, and the output addressing (row-major [M,N], or NCHW when the GEMM rows are the
 // output pixels of a convolution).  Plugs into tile_store_via_lds (mfma8_common.hpp).
 #pragma once
-#include "mfma8_gemm_pair.hpp"
+#include "mfma8_dispatch.hpp"
 
 namespace sofie_hip {
 
