@@ -226,6 +226,10 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
             src.stride_h = d->stride_h; src.stride_w = d->stride_w; src.pad_h0 = d->pad_h0; src.pad_w0 = d->pad_w0;
             src.dil_h = d->dil_h; src.dil_w = d->dil_w; src.kw = d->kw; src.ntaps = ntaps;
             src.cg_shift = cg_shift; src.kw_recip = kw_recip;
+            // ceil(2^64 / d) for d >= 2; 0 stands for d == 1 (2^64 does not fit)
+            auto recip64 = [](unsigned d) -> unsigned long long { return d <= 1 ? 0ull : (~0ull / d) + 1; };
+            src.ohw_mul = recip64((unsigned)OHW);
+            src.ow_mul = recip64((unsigned)g.OW);
             I8Epilogue ep;
             ep.bias = a->bias;
             ep.scale = a->scale;

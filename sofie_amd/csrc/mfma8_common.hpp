@@ -150,6 +150,9 @@ struct ConvRows {
    int kw, ntaps;
    int cg_shift;          // log2(Cg)
    int kw_recip;          // ceil(65536 / kw): tap / kw == (tap * kw_recip) >> 16 for every tap < ntaps (checked on the host)
+   // m / (OH*OW) and r / OW by multiplication: floor(m / d) == (m * ceil(2^64 / d)) >> 64 for every 32-bit m
+   // (the error of the rounded-up reciprocal, < m / 2^64 * d... < 2^-32, cannot reach the next integer)
+   unsigned long long ohw_mul, ow_mul;
 
    template <int LD>
    struct lane_state {
@@ -164,8 +167,10 @@ struct ConvRows {
       int32_t off = 0;
       if (m < M) {
          const int ohw = OH * OW;
-         const int n = m / ohw, r = m - n * ohw;
-         const int oh = r / OW, ow = r - oh * OW;
+         const int n = ohw_mul ? (int)__umul64hi((unsigned long long)(unsigned)m, ohw_mul) : m; // 0 marks a divisor of 1
+         const int r = m - n * ohw;
+         const int oh = ow_mul ? (int)__umul64hi((unsigned long long)(unsigned)r, ow_mul) : r;
+         const int ow = r - oh * OW;
          const int ih0 = oh * stride_h - pad_h0, iw0 = ow * stride_w - pad_w0;
          off = ((n * H + ih0) * W + iw0) * C + cbyte;
          int khi = 0, kwi = 0; // tap t = khi * kw + kwi, stepped without dividing
