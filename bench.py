@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-Workload (BASELINE config 2): int8 quantised MLP 1024 -> 4096 -> 4096 -> 1024 at batch 1024,
+Workload (benchmark configuration 2): int8 quantised MLP 1024 -> 4096 -> 4096 -> 1024 at batch 1024,
 QuantizeLinear -> [int8 Gemm (int32 accumulate) -> Relu -> DequantizeLinear]x3, per-tensor scales,
 synthetic seeded data, fp32 input already resident in HBM.  One step = one inference over the batch.
 Prints ONE JSON line; `value` = inferences/s.  Also times the stand-alone int8 GEMM sweep
@@ -30,17 +30,16 @@ DOMINANT_KERNEL_TRAFFIC_BYTES = 36024320
 
 def build_mlp():
     from tests import util
-    from oracle import binding as ob
     dims, batch = [1024, 4096, 4096, 1024], 1024
     weights = [util.int8_sym(1101 + l, dims[l] * dims[l + 1]).reshape(dims[l], dims[l + 1]) for l in range(3)]
     x = util.normal(2101, batch * dims[0]).reshape(batch, dims[0])
     w_scales = [np.float32(1.0 / 127.0)] * 3
     in_scales = [np.float32(np.abs(x).max() / 127.0)]
     h = x[:8]
-    for l, w in enumerate(weights[:-1]):  # calibration of the frozen activation scales (model constants)
-        q = ob.quantize_linear(h, in_scales[l])
-        acc = np.maximum(ob.matmul_integer(q, w, M=8, N=w.shape[1], K=w.shape[0], omp=True), 0)
-        h = ob.dequantize_linear(acc, np.float32(in_scales[l] * w_scales[l]))
+    for l, w in enumerate(weights[:-1]):  # calibration of the frozen activation scales (model constants), plain numpy
+        q = np.clip(np.rint(h / in_scales[l]), -128, 127).astype(np.int32)
+        acc = np.maximum(q @ w.astype(np.int32), 0)
+        h = acc.astype(np.float32) * np.float32(in_scales[l] * w_scales[l])
         in_scales.append(np.float32(max(h.max(), 1e-6) / 127.0))
     return dims, batch, x, weights, w_scales, in_scales
 
@@ -57,7 +56,7 @@ def time_region(rt, fn, reps):
 
 
 def gemm_sweep(rt, sizes, reps=20, warmup=3):
-    """Stand-alone int8 GEMM with per-channel requant + bias + relu (BASELINE config 3)."""
+    """Stand-alone int8 GEMM with per-channel requant + bias + relu (benchmark configuration 3)."""
     from sofie_amd import runtime as R
     from tests import util
     import torch
@@ -92,7 +91,7 @@ def gemm_sweep(rt, sizes, reps=20, warmup=3):
 
 
 def fp8_sweep(rt, sizes, reps=20, warmup=3):
-    """Stand-alone FP8 e4m3 GEMM, fp32 accumulate, per-tensor scale, bias + GELU, bf16 output (BASELINE config 4)."""
+    """Stand-alone FP8 e4m3 GEMM, fp32 accumulate, per-tensor scale, bias + GELU, bf16 output (benchmark configuration 4)."""
     from sofie_amd import runtime as R
     from tests import util
     import torch
@@ -133,7 +132,7 @@ def fp8_sweep(rt, sizes, reps=20, warmup=3):
 
 
 def fp32_mlp_leg(steps=200):
-    """BASELINE config 1: fp32 Gemm+Relu chain 784 -> 128 -> 64 -> 10 at batch 64, three fused launches; next to the CPU
+    """benchmark configuration 1: fp32 Gemm+Relu chain 784 -> 128 -> 64 -> 10 at batch 64, three fused launches; next to the CPU
     restatement of the reference's generated code on the same batch."""
     from sofie_amd import Runtime, runtime as R
     from oracle import binding as ob
@@ -179,7 +178,7 @@ def fp32_mlp_leg(steps=200):
 
 
 def int8_cnn_leg(steps=10):
-    """BASELINE config 5: 4 x [Conv3x3 s1 p1 + folded BatchNorm + Relu] 3->64->128->256->256 on 64x64 images, batch 256,
+    """benchmark configuration 5: 4 x [Conv3x3 s1 p1 + folded BatchNorm + Relu] 3->64->128->256->256 on 64x64 images, batch 256,
     global average pool, Gemm 256->10; int8 weights, per-channel scales."""
     from sofie_amd import Runtime
     from sofie_amd.session import Int8CNNSession
@@ -336,7 +335,7 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": "int8 MLP 1024->4096->4096->1024, batch 1024, Q -> [i8 Gemm(i32) -> Relu -> DQ]x3, "
-                               "per-tensor symmetric scales, input resident in HBM (BASELINE configs[1])",
+                               "per-tensor symmetric scales, input resident in HBM (benchmark configuration 2)",
                    "global_batch": batch, "launches_per_step": 4, "wall_ms_per_step": round(wall / args.steps, 5),
                    "ms_per_step_of_5_regions": repeats, "median_ms_per_step": sorted(repeats)[2],
                    "parity_vs_oracle_rows": args.cpu_rows, "parity_bit_exact": parity,

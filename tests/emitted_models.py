@@ -1,4 +1,4 @@
-"""The models that go through the C++ emitter: every golden fixture of the reference plus the BASELINE
+"""The models that go through the C++ emitter: every golden fixture of the reference plus the benchmark
 configurations this backend adds (built here as ONNX files from seeded data).  build_all() runs at build
 time on the CPU: it writes the ONNX files, runs sofie_hip_emit, and compiles each emitted header together
 with a tiny C harness into tests/emitted/lib<Model>.so.  The GPU tests only load those libraries."""
@@ -20,7 +20,7 @@ GOLDEN = os.path.join(ROOT, "tests", "golden")
 # ---- configuration models ------------------------------------------------------------------------------------
 
 def fp32_mlp(batch=64):
-    """BASELINE config 1: Gemm(transB=1)+Relu, Gemm+Relu, Gemm; 784 -> 128 -> 64 -> 10; W ~ N(0, 0.05), biases 0."""
+    """benchmark configuration 1: Gemm(transB=1)+Relu, Gemm+Relu, Gemm; 784 -> 128 -> 64 -> 10; W ~ N(0, 0.05), biases 0."""
     dims = [784, 128, 64, 10]
     init, nodes, x = {}, [], "X"
     for l in range(3):
@@ -37,18 +37,17 @@ def fp32_mlp(batch=64):
 
 
 def int8_mlp(dims, batch, seed=1100):
-    """BASELINE config 2 as ONNX operators: per layer QuantizeLinear -> MatMulInteger -> Relu -> DequantizeLinear,
+    """benchmark configuration 2 as ONNX operators: per layer QuantizeLinear -> MatMulInteger -> Relu -> DequantizeLinear,
     per-tensor symmetric scales (zero points 0).  Returns the model and the constants the CPU chain needs."""
-    from oracle import binding as ob
     weights = [util.int8_sym(seed + 1 + l, dims[l] * dims[l + 1]).reshape(dims[l], dims[l + 1]) for l in range(len(dims) - 1)]
     X = util.normal(seed + 1001, batch * dims[0]).reshape(batch, dims[0])
     w_scales = [np.float32(1.0 / 127.0)] * len(weights)
     in_scales = [np.float32(np.abs(X).max() / 127.0)]
     h = X[:8]
     for l, w in enumerate(weights[:-1]):
-        q = ob.quantize_linear(h, in_scales[l])
-        acc = np.maximum(ob.matmul_integer(q, w, M=h.shape[0], N=w.shape[1], K=w.shape[0], omp=True), 0)
-        h = ob.dequantize_linear(acc, np.float32(in_scales[l] * w_scales[l]))
+        q = np.clip(np.rint(h / in_scales[l]), -128, 127).astype(np.int32)   # calibration only: plain numpy
+        acc = np.maximum(q @ w.astype(np.int32), 0)
+        h = acc.astype(np.float32) * np.float32(in_scales[l] * w_scales[l])
         in_scales.append(np.float32(max(h.max(), 1e-6) / 127.0))
     init, nodes, x = {}, [], "X"
     for l, w in enumerate(weights):
@@ -65,7 +64,7 @@ def int8_mlp(dims, batch, seed=1100):
 
 
 def fp32_cnn(batch=2):
-    """A small fp32 form of BASELINE config 5: 2 x [Conv3x3 s1 p1 + Relu], GlobalAveragePool, Gemm."""
+    """A small fp32 form of benchmark configuration 5: 2 x [Conv3x3 s1 p1 + Relu], GlobalAveragePool, Gemm."""
     init = {"W0": util.normal(5101, 8 * 3 * 9, 0.2).reshape(8, 3, 3, 3), "B0": util.normal(5102, 8, 0.1),
             "W1": util.normal(5103, 16 * 8 * 9, 0.1).reshape(16, 8, 3, 3), "B1": util.normal(5104, 16, 0.1),
             "WF": util.normal(5105, 16 * 10, 0.3).reshape(16, 10), "BF": util.normal(5106, 10, 0.1)}
@@ -82,7 +81,7 @@ def fp32_cnn(batch=2):
 
 
 def int8_cnn(batch=2, hw=12, channels=(3, 64, 128, 256, 256), n_out=10):
-    """BASELINE config 5 as ONNX operators: QuantizeLinear, then per stage QLinearConv 3x3 s1 p1 (per-channel weight scales,
+    """benchmark configuration 5 as ONNX operators: QuantizeLinear, then per stage QLinearConv 3x3 s1 p1 (per-channel weight scales,
     int32 bias: the folded BatchNorm) + Relu, then DequantizeLinear, GlobalAveragePool, Flatten, Gemm.  Returns the model and
     the constants of the CPU chain (tests.refmodels.int8_cnn_oracle)."""
     from tests.refmodels import make_int8_cnn

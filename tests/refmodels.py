@@ -17,7 +17,7 @@ def int8_mlp_oracle(x, weights, w_scales, in_scales, omp=False):
 
 
 def make_int8_cnn(batch, hw=64, channels=(3, 64, 128, 256, 256), n_out=10, seed=5200):
-    """BASELINE config 5 as model constants: Conv3x3 s1 p1 (+folded BatchNorm = per-channel scale and bias) + Relu
+    """benchmark configuration 5 as model constants: Conv3x3 s1 p1 (+folded BatchNorm = per-channel scale and bias) + Relu
     per stage, GlobalAveragePool, Gemm.  int8 weights U[-127,127], inputs U(0,1)."""
     from tests import util
     convs = []

@@ -145,7 +145,7 @@ def test_bad_arguments_are_refused(rt):
 
 
 def test_full_size_8192_sampled_rows_and_linearity(rt):
-    """BASELINE config 3 at M=N=K=8192: full rows checked bit-exactly against the oracle on a sample,
+    """benchmark configuration 3 at M=N=K=8192: full rows checked bit-exactly against the oracle on a sample,
     plus a size-independent property: G(A1) + G(A2) == G(A1 + A2) for int32 outputs."""
     import torch
     M = N = K = 8192

@@ -1,4 +1,4 @@
-"""End-to-end int8 MLP (BASELINE config 2) through the Session: bit-exact against the unfused CPU chain."""
+"""End-to-end int8 MLP (benchmark configuration 2) through the Session: bit-exact against the unfused CPU chain."""
 import numpy as np
 import pytest
 
