@@ -62,3 +62,45 @@ def test_config2_full_size_sampled_rows():
     want = int8_mlp_oracle(x[rows], weights, w_scales, in_scales, omp=True)
     assert np.array_equal(got[rows].view(np.uint32), want.view(np.uint32))
     assert (got > 0).mean() > 0.2  # the network is alive: relu does not kill every unit
+
+
+def test_inference_captured_in_a_hip_graph_replays_correctly():
+    """infer_nosync only enqueues kernels on the context's stream (no allocation, no memset): captured once into a HIP graph
+    on a caller-owned stream, every replay must reproduce the eager result, also with eager work and synchronisations in
+    between and after the input buffer has been overwritten with a new batch."""
+    import ctypes as C
+    import torch
+    from sofie_amd import Runtime
+    dims, batch = [256, 512, 384, 64], 96
+    x, weights, w_scales, in_scales = make_mlp(dims, batch)
+    x2 = np.ascontiguousarray(x[::-1] * np.float32(0.5))
+    stream = torch.cuda.Stream()
+    rt = Runtime(0, external_stream=C.c_void_p(stream.cuda_stream))
+    try:
+        sess = Int8MLPSession(rt, weights, w_scales, in_scales, batch)
+        eager, eager2 = sess.infer(x), sess.infer(x2)            # also the warm-up: kernel attributes are set outside the capture
+        want = int8_mlp_oracle(x, weights, w_scales, in_scales)
+        assert np.array_equal(eager.view(np.uint32), want.view(np.uint32))
+        sess.upload_input(x)
+        rt.sync()
+        graph = torch.cuda.CUDAGraph()
+        print("capturing the int8 MLP into a graph", flush=True)
+        with torch.cuda.graph(graph, stream=stream):
+            sess.infer_nosync()
+        y = np.empty((batch, dims[-1]), dtype=np.float32)
+
+        def fetch():
+            rt.call("sofie_hip_download", y.ctypes.data_as(C.c_void_p), sess.y_ptr, C.c_size_t(y.nbytes))
+            rt.sync()
+            return y.copy()
+        for replay, (inp, ref) in enumerate([(x, eager), (x2, eager2), (x, eager), (x, eager)]):
+            sess.upload_input(inp)
+            rt.call("sofie_hip_fill_zero", sess.y_ptr, C.c_size_t(y.nbytes))   # eager work between the replays
+            rt.sync()
+            graph.replay()
+            stream.synchronize()
+            got = fetch()
+            assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), "replay %d" % replay
+        del graph
+    finally:
+        rt.close()
