@@ -36,6 +36,17 @@ public:
       fOutputTensorNames = {fNY};
       fKind = OperatorKind::QCONV;
    }
+   // ONNX ConvInteger: the plain int32 accumulator is the output (no scales, no bias), NCHW
+   static std::unique_ptr<ROperator_QConv> MakeConvInteger(std::string autopad, std::vector<std::size_t> dilations, std::size_t group,
+                                                            std::vector<std::size_t> kernelShape, std::vector<std::size_t> pads,
+                                                            std::vector<std::size_t> strides, std::string nameX, std::string nameW,
+                                                            std::string nameXZero, std::string nameWZero, std::string nameY)
+   {
+      auto op = std::make_unique<ROperator_QConv>(autopad, dilations, group, kernelShape, pads, strides, nameX, "", nameXZero, nameW, "", nameWZero,
+                                                  "", "", "", nameY);
+      op->fInt32Out = true;
+      return op;
+   }
    bool HasRelu() const { return fRelu; }
    void FuseRelu(const std::string &newOutput)
    {
@@ -66,6 +77,12 @@ public:
       }
       fGeo.Resolve(fAttrAutopad, fAttrDilations, fAttrGroup, fAttrKernelShape, fAttrPads, fAttrStrides, model.GetTensorShape(fNX),
                    model.GetTensorShape(fNW));
+      fXLayout = model.GetTensorLayout(fNX);
+      if (fInt32Out) {
+         fYLayout = kLayoutNCHW;
+         model.AddIntermediateTensor(fNY, ETensorType::INT32, fGeo.OutputShape());
+         return;
+      }
       const float xs = model.GetScalarInitializer(fNXS), ys = model.GetScalarInitializer(fNYS);
       if (!(xs > 0) || !(ys > 0))
          throw std::runtime_error("SOFIE QLinearConv Op: scales of " + fNX + " and " + fNY + " must be positive");
@@ -87,7 +104,6 @@ public:
              ConvertShapeToLength(model.GetTensorShape(fNB)) != fGeo.Cout)
             throw std::runtime_error("SOFIE QLinearConv Op: bias " + fNB + " must be an int32 initializer of " + std::to_string(fGeo.Cout) + " elements");
       }
-      fXLayout = model.GetTensorLayout(fNX);
       // channels-last output when every reader understands it
       fYLayout = kLayoutNHWC;
       if (model.IsOutputTensor(fNY))
@@ -135,14 +151,14 @@ public:
       const std::string ws = "workspace_op_" + opName;
       opName = "op_" + opName;
       std::stringstream out;
-      out << "\n" << SP << "//----  operator QLinearConv " << opName << " --> " << ConvertShapeToString(fGeo.OutputShape())
+      out << "\n" << SP << "//----  operator " << (fInt32Out ? "ConvInteger " : "QLinearConv ") << opName << " --> " << ConvertShapeToString(fGeo.OutputShape())
           << (fYLayout == kLayoutNHWC ? " (stored NHWC)" : "") << (ImplicitGemm() ? ", implicit GEMM" : ", column matrix") << "\n";
       out << SP << "{\n";
       out << SP << "   " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n";
       out << SP << "   " << "sofie_conv_i8_args a{};\n";
       out << SP << "   " << "a.X = tensor_" << fNX << "; a.W = packed_" << fNW << "; a.w_is_packed = 1; a.bias = "
-          << (fNB.empty() ? "nullptr" : "tensor_" + fNB) << "; a.scale = tensor_" << fNM << ";\n";
-      out << SP << "   " << "a.relu = " << (fRelu ? 1 : 0) << "; a.out = SOFIE_I8OUT_I8; a.x_layout = "
+          << (fNB.empty() ? "nullptr" : "tensor_" + fNB) << "; a.scale = " << (fInt32Out ? std::string("nullptr") : "tensor_" + fNM) << ";\n";
+      out << SP << "   " << "a.relu = " << (fRelu ? 1 : 0) << "; a.out = " << (fInt32Out ? "SOFIE_I8OUT_I32" : "SOFIE_I8OUT_I8") << "; a.x_layout = "
           << (fXLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.y_layout = "
           << (fYLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.Y = tensor_" << fNY << ";\n";
       if (GetWorkspaceBytes())
@@ -158,7 +174,7 @@ private:
    std::size_t fAttrGroup;
    std::vector<std::size_t> fAttrKernelShape, fAttrPads, fAttrStrides;
    std::string fNX, fNXS, fNXZ, fNW, fNWS, fNWZ, fNYS, fNYZ, fNB, fNY, fNM;
-   bool fRelu = false;
+   bool fRelu = false, fInt32Out = false;
    int fXLayout = kLayoutNCHW, fYLayout = kLayoutNCHW;
    ConvGeometry fGeo;
 };

@@ -129,6 +129,8 @@ public:
       fNY = UTILITY::Clean_name(name);
       fOutputTensorNames = {fNY};
    }
+   void SetReluOnOutput() { fReluOut = true; }
+   bool ReluOnOutput() const { return fReluOut; }
    Out OutputKind() const { return fOut; }
    float DequantScale() const { return fScale; }
    bool ReluOnAccumulator() const { return fReluAcc; }

@@ -204,7 +204,11 @@ void RModel::FuseGemmActivations()
                changed = true;
             }
          } else if (auto *q = dynamic_cast<ROperator_QGemm *>(op)) {
-            if (q->OutputKind() == ROperator_QGemm::Out::I32 && act && act->Activation() == EActivationType::RELU && !q->ReluOnAccumulator()) {
+            if (q->OutputKind() == ROperator_QGemm::Out::I8_REQUANT && act && act->Activation() == EActivationType::RELU && !q->ReluOnOutput()) {
+               q->SetReluOnOutput(); // Relu on the requantised int8 value: max(sat8(x), 0)
+               q->SetOutputName(act->OutputName());
+               changed = true;
+            } else if (q->OutputKind() == ROperator_QGemm::Out::I32 && act && act->Activation() == EActivationType::RELU && !q->ReluOnAccumulator()) {
                q->SetReluOnAccumulator();
                q->SetOutputName(act->OutputName());
                changed = true;

@@ -408,6 +408,41 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
                                                               attrV(n, "kernel_shape"), attrV(n, "pads"), attrV(n, "strides"), n.in[0], n.in[1],
                                                               n.in[2], n.in[3], n.in[4], n.in[5], n.in[6], n.in[7],
                                                               n.in.size() > 8 ? n.in[8] : "", n.out[0]));
+      } else if (n.op == "ConvInteger") {
+         model->AddOperator(ROperator_QConv::MakeConvInteger(attrS(n, "auto_pad", "NOTSET"), attrV(n, "dilations"), (size_t)attrI(n, "group", 1),
+                                                             attrV(n, "kernel_shape"), attrV(n, "pads"), attrV(n, "strides"), n.in[0], n.in[1],
+                                                             n.in.size() > 2 ? n.in[2] : "", n.in.size() > 3 ? n.in[3] : "", n.out[0]));
+      } else if (n.op == "QLinearMatMul") {
+         // y = sat8(rne(acc * ((a_scale * b_scale[n]) / y_scale))): the multipliers are formed here, once, in fp32
+         if (n.in.size() != 8)
+            throw std::runtime_error("SOFIE ONNX parser: QLinearMatMul " + n.name + " needs 8 inputs");
+         for (int z : {2, 5, 7}) {
+            const std::string zn = UTILITY::Clean_name(n.in[z]);
+            if (!model->IsInitializedTensor(zn) || model->GetTensorType(zn) != ETensorType::INT8)
+               throw std::runtime_error("SOFIE ONNX parser: QLinearMatMul zero point " + n.in[z] + " must be an int8 initializer");
+            const auto *p = static_cast<const int8_t *>(model->GetInitializedTensorData(zn).get());
+            for (size_t k = 0; k < ConvertShapeToLength(model->GetTensorShape(zn)); ++k)
+               if (p[k] != 0)
+                  throw std::runtime_error("SOFIE ONNX parser: QLinearMatMul zero point " + n.in[z] + " is not 0; symmetric quantisation only");
+         }
+         const float as = model->GetScalarInitializer(n.in[1]), ys = model->GetScalarInitializer(n.in[6]);
+         const std::string bsn = UTILITY::Clean_name(n.in[4]), bn = UTILITY::Clean_name(n.in[3]);
+         if (!model->IsInitializedTensor(bsn) || model->GetTensorType(bsn) != ETensorType::FLOAT || !model->IsInitializedTensor(bn))
+            throw std::runtime_error("SOFIE ONNX parser: QLinearMatMul needs an initializer B with a float scale initializer");
+         const size_t ncols = model->GetTensorShape(bn).back(), nbs = ConvertShapeToLength(model->GetTensorShape(bsn));
+         if (nbs != 1 && nbs != ncols)
+            throw std::runtime_error("SOFIE ONNX parser: QLinearMatMul scale of B must have 1 or N elements");
+         const float *bs = static_cast<const float *>(model->GetInitializedTensorData(bsn).get());
+         std::vector<float> mult(ncols);
+         for (size_t c = 0; c < ncols; ++c) {
+            volatile float prod = as * bs[nbs == 1 ? 0 : c];
+            mult[c] = prod / ys;
+         }
+         const std::string mname = n.out[0] + "_requant_scale";
+         model->AddInitializedTensor(mname, ETensorType::FLOAT, {ncols}, mult.data());
+         auto op = std::make_unique<ROperator_QGemm>(n.in[0], n.in[3], n.out[0]);
+         op->SetRequantize(mname, false);
+         model->AddOperator(std::move(op));
       } else if (n.op == "Flatten") {
          model->AddOperator(std::make_unique<ROperator_Flatten>((int)attrI(n, "axis", 1), n.in[0], n.out[0]));
       } else if (n.op == "MatMulInteger") {

@@ -128,7 +128,40 @@ def conv_batchnorm_relu(batch=2):
     return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 3, 10, 10])], outputs=[("Y", np.float32, [batch, 8, 1, 1])], init=init, feeds=[X])
 
 
+def qlinear_matmul_relu(M=16, K=64, N=48):
+    """QuantizeLinear -> QLinearMatMul (per-column weight scales) -> Relu (int8) -> DequantizeLinear."""
+    W = util.int8_sym(7101, K * N).reshape(K, N)
+    sx, sy = np.float32(0.02), np.float32(0.05)
+    sw = ((0.5 + util.uniform01(7102, N)) * np.float32(sy / (sx * 73.0 * np.sqrt(K)))).astype(np.float32)
+    init = {"W": W, "sx": np.array(sx, np.float32), "sw": sw, "sy": np.array(sy, np.float32), "zp": np.zeros((), np.int8)}
+    nodes = [ow.node("QuantizeLinear", ["X", "sx", "zp"], ["Q"]),
+             ow.node("QLinearMatMul", ["Q", "sx", "zp", "W", "sw", "zp", "sy", "zp"], ["P"]),
+             ow.node("Relu", ["P"], ["R"]),
+             ow.node("DequantizeLinear", ["R", "sy", "zp"], ["Y"])]
+    X = util.normal(7001, M * K).reshape(M, K)
+    mult = ((sx * sw).astype(np.float32) / sy).astype(np.float32)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [M, K])], outputs=[("Y", np.float32, [M, N])], init=init, feeds=[X],
+                consts=dict(W=W, sx=sx, sy=sy, mult=mult))
+
+
+def conv_integer_dequantize(batch=2):
+    """QuantizeLinear -> ConvInteger (int32 accumulators out) -> Relu -> DequantizeLinear(int32)."""
+    W = util.int8_sym(7201, 6 * 4 * 9).reshape(6, 4, 3, 3)
+    sx = np.float32(0.03)
+    sacc = np.float32(sx * 0.01)
+    init = {"W": W, "sx": np.array(sx, np.float32), "sacc": np.array(sacc, np.float32), "zp": np.zeros((), np.int8)}
+    nodes = [ow.node("QuantizeLinear", ["X", "sx", "zp"], ["Q"]),
+             ow.node("ConvInteger", ["Q", "W", "zp", "zp"], ["A"], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1]),
+             ow.node("Relu", ["A"], ["R"]),
+             ow.node("DequantizeLinear", ["R", "sacc"], ["Y"])]
+    X = util.normal(7202, batch * 4 * 7 * 7).reshape(batch, 4, 7, 7)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 4, 7, 7])], outputs=[("Y", np.float32, [batch, 6, 7, 7])], init=init,
+                feeds=[X], consts=dict(W=W, sx=sx, sacc=sacc))
+
+
 CONFIG_MODELS = {
+    "QLinearMatMulRelu": lambda: qlinear_matmul_relu(),
+    "ConvIntegerDequantize": lambda: conv_integer_dequantize(),
     "ConvBatchNormRelu": lambda: conv_batchnorm_relu(2),
     "Config5_int8_CNN_small": lambda: int8_cnn(2, 12),
     "Config1_fp32_MLP": lambda: fp32_mlp(64),

@@ -174,6 +174,20 @@ def test_quantised_cnn_keeps_channels_last_and_reads_activations_in_place(emitte
     assert ctor.count("sofie_hip_pack_conv_weight_i8(") == 4
 
 
+def test_qlinear_matmul_and_conv_integer_become_one_launch_each(emitted):
+    txt = read(emitted, "QLinearMatMulRelu")
+    body = txt[txt.index("void infer_nosync()"):]
+    body = body[:body.index("infer(")]
+    # the Relu on the int8 output rides in the GEMM's store; multipliers a_scale*b_scale[n]/y_scale are a weight
+    assert body.count("sofie_hip_gemm_i8(") == 1 and "d.relu_out = 1" in body and "sofie_hip_unary_f32" not in body
+    assert "tensor_P_requant_scale" in txt
+    txt = read(emitted, "ConvIntegerDequantize")
+    body = txt[txt.index("void infer_nosync()"):]
+    body = body[:body.index("infer(")]
+    assert body.count("sofie_hip_conv_i8(") == 1 and "a.out = SOFIE_I8OUT_I32" in body and "a.relu = 1" in body
+    assert "sofie_hip_dequantize_linear_i32(" in body and "sofie_hip_unary_f32" not in body
+
+
 def test_asymmetric_zero_point_is_refused(tmp_path):
     init = {"W": np.ones((4, 3, 1, 1), dtype=np.int8), "s": np.array(0.5, dtype=np.float32), "z": np.zeros((), dtype=np.int8),
             "z1": np.array(3, dtype=np.int8), "sx": np.array(0.1, dtype=np.float32)}

@@ -145,3 +145,33 @@ def test_safetensors_session_reproduces_the_golden_output(rt, tmp_path):
         rc = lib.run_model(path.encode(), ptrs, y.ctypes.data_as(ctypes.c_void_p), ctypes.c_ulong(y.size), err, 1024)
         assert rc == 0, err.value.decode()
         assert np.abs(y - expected).max() <= golden_tolerance("Linear_16", expected)
+
+
+def test_emitted_qlinear_matmul_relu_is_bit_exact(rt):
+    from oracle import binding as ob
+    spec = em.qlinear_matmul_relu()
+    c, x = spec["consts"], spec["feeds"][0]
+    M, K = x.shape
+    N = c["W"].shape[1]
+    q = ob.quantize_linear(x, c["sx"])
+    y8 = ob.gemm_i8(q, c["W"], M=M, N=N, K=K, scale=c["mult"], relu_out=1, out=2)
+    want = ob.dequantize_linear(y8, c["sy"])
+    print("emitted QLinearMatMulRelu", flush=True)
+    got = run_emitted("QLinearMatMulRelu", [x], M * N).reshape(M, N)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert (y8 > 0).any() and (y8 == 0).any()
+    txt = open(os.path.join(em.OUT, "QLinearMatMulRelu_GPU_HIP.hxx")).read()
+    assert "d.relu_out = 1" in txt and "SOFIE_I8OUT_I8;" in txt and "sofie_hip_unary_f32" not in txt
+
+
+def test_emitted_conv_integer_chain_is_bit_exact(rt):
+    from oracle import binding as ob
+    spec = em.conv_integer_dequantize()
+    c, x = spec["consts"], spec["feeds"][0]
+    q = ob.quantize_linear(x, c["sx"])
+    acc = ob.conv_i8(q, c["W"], None, None, pads=(1, 1, 1, 1), relu=1, out=0)
+    want = ob.dequantize_linear(acc, c["sacc"])
+    print("emitted ConvIntegerDequantize", flush=True)
+    got = run_emitted("ConvIntegerDequantize", [x], want.size).reshape(want.shape)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert (acc > 0).any()
