@@ -29,12 +29,17 @@ public:
 
    // ---- model building (the reference's names and meaning) ----
    void AddInputTensorInfo(std::string input_name, ETensorType type, std::vector<std::size_t> shape);
+   // an input whose LEADING dimension may be a named parameter (the batch): the Session then takes its maximum in
+   // the constructor and its value in every infer call (core/src/RModel.cxx:1375-1395, 1537-1547); a positive
+   // batchSize given to GenerateGPU_HIP fixes it at generation time instead
+   void AddInputTensorInfo(std::string input_name, ETensorType type, std::vector<Dim> shape);
    void AddInputTensorName(std::string name);
    void AddInitializedTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, std::shared_ptr<void> data);
    // copies `data` (length = product of shape)
    void AddInitializedTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, const void *data);
    void AddConstantTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, const void *data);
-   void AddIntermediateTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape);
+   // `batched`: the leading dimension is the run-time batch (given as 1 in `shape`)
+   void AddIntermediateTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, bool batched = false);
    void AddOperator(std::unique_ptr<ROperator> op, int order_execution = -1);
    void AddOutputTensorNameList(std::vector<std::string> output_tensor_names);
 
@@ -57,6 +62,10 @@ public:
       return f == fTensorLayout.end() ? kLayoutNCHW : f->second;
    }
    bool IsOutputTensor(const std::string &name) const;
+   // true if the tensor's leading dimension is the run-time batch; its stored shape then has 1 there
+   bool IsDynamicTensor(const std::string &name) const { return fBatched.count(UTILITY::Clean_name(name)) != 0; }
+   bool HasDynamicBatch() const { return !fBatchParam.empty(); }
+   const std::string &GetBatchParamName() const { return fBatchParam; }
    // kinds of the operators that read `name` (after fusion)
    std::vector<OperatorKind> ConsumerKinds(const std::string &name) const;
    const std::string &GetName() const { return fName; }
@@ -78,13 +87,17 @@ public:
       std::size_t offset, bytes;
       int begin, end; // lifetime in operator indices, [begin, end); statics have begin = -1
       bool pooled;
+      bool perBatch = false; // offset and bytes are per batch entry, counted from the end of the static region
    };
    const std::vector<PlannedTensor> &GetMemoryPlan() const { return fPlan; }
    std::size_t GetArenaBytes() const { return fArenaBytes; }
    std::size_t GetIntermediateMemoryPoolSize() const { return fPoolBytes; }
+   // with a run-time batch the arena is GetStaticBytes() + capacity * GetBytesPerBatchEntry()
+   std::size_t GetStaticBytes() const { return fStaticBytes; }
+   std::size_t GetBytesPerBatchEntry() const { return fBatchEntryBytes; }
 
 private:
-   void Initialize();
+   void Initialize(int batchSize);
    void FuseGemmActivations();
    void PlanMemory();
    void GenerateSessionCode(std::underlying_type_t<Options> options);
@@ -101,7 +114,11 @@ private:
    std::vector<PlannedTensor> fPlan;
    std::unordered_map<std::string, std::size_t> fOffsets;
    std::unordered_map<std::string, int> fTensorLayout;
-   std::size_t fArenaBytes = 0, fPoolBytes = 0;
+   std::size_t fArenaBytes = 0, fPoolBytes = 0, fStaticBytes = 0, fBatchEntryBytes = 0;
+   std::unordered_map<std::string, std::vector<Dim>> fInputDimShapes;
+   std::unordered_map<std::string, bool> fBatched;
+   std::string fBatchParam;
+   std::size_t fBatchDefault = 1;
    bool fInitialized = false;
    bool fSafetensors = false;
    std::string fGC;

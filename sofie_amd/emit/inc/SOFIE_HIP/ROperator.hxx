@@ -28,6 +28,8 @@ public:
    virtual std::vector<std::pair<std::string, std::size_t>> GetPersistentBuffers() { return {}; }
    // bytes of scratch the operator needs while it runs (planned like an intermediate tensor that lives for this operator)
    virtual std::size_t GetWorkspaceBytes() { return 0; }
+   // in a model with a run-time batch: true if GetWorkspaceBytes() is the need of ONE batch entry
+   virtual bool WorkspacePerBatchEntry() const { return false; }
    virtual OperatorKind GetKind() const { return fKind; }
    const std::vector<std::string> &GetInputTensorNames() const { return fInputTensorNames; }
    const std::vector<std::string> &GetOutputTensorNames() const { return fOutputTensorNames; }

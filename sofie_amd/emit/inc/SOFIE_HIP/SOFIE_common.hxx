@@ -90,6 +90,38 @@ inline std::string Clean_name(std::string s)
 }
 } // namespace UTILITY
 
+// One dimension of an input shape: a number, or a named parameter that is fixed when the Session runs
+// (the reference's Dim, core/inc/SOFIE/utils/SOFIE_common.hxx:64-89).  `dim` of a parameter is its default value.
+struct Dim {
+   bool isParam = false;
+   std::size_t dim = 0;
+   std::string param;
+   Dim() = default;
+   Dim(std::size_t d) : dim(d) {}
+   Dim(const std::string &p, std::size_t d = 0) : isParam(true), dim(d), param(p)
+   {
+      if (!p.empty() && std::all_of(p.begin(), p.end(), [](unsigned char c) { return std::isdigit(c) != 0; })) {
+         isParam = false;
+         dim = std::stoull(p);
+      }
+   }
+   std::string GetVal() const { return isParam ? param : std::to_string(dim); }
+};
+
+// Text of a count in the emitted code.  In a model with a run-time batch, tensors that carry the batch as
+// their leading dimension are kept with that dimension = 1 and their counts are multiplied by the Session's
+// `sofie_batch` when the code runs.
+inline std::string BatchScaled(bool dynamic, std::size_t unit)
+{
+   return dynamic ? "sofie_batch * " + std::to_string(unit) : std::to_string(unit);
+}
+
+// the same for an argument or field of type int32_t
+inline std::string BatchScaledInt(bool dynamic, std::size_t unit)
+{
+   return dynamic ? "static_cast<std::int32_t>(sofie_batch * " + std::to_string(unit) + ")" : std::to_string(unit);
+}
+
 struct InitializedTensor {
    ETensorType type = ETensorType::UNDEFINED;
    std::vector<std::size_t> shape;

@@ -28,6 +28,13 @@ public:
       fShapeA = model.GetTensorShape(fNA);
       fShapeB = model.GetTensorShape(fNB);
       const std::size_t r = std::max(fShapeA.size(), fShapeB.size());
+      // a batched operand's leading dimension must be the result's leading dimension
+      fDynA = model.IsDynamicTensor(fNA);
+      fDynB = model.IsDynamicTensor(fNB);
+      if ((fDynA && fShapeA.size() != r) || (fDynB && fShapeB.size() != r))
+         throw std::runtime_error("SOFIE Binary Op: with a run-time batch the batched operand must have the rank of the result");
+      if ((fDynA && !fDynB && fShapeB.size() == r && fShapeB[0] != 1) || (fDynB && !fDynA && fShapeA.size() == r && fShapeA[0] != 1))
+         throw std::runtime_error("SOFIE Binary Op: an operand without the batch cannot have a leading dimension above 1");
       if (r > 6)
          throw std::runtime_error("SOFIE Binary Op: rank above 6 is not supported");
       fShapeA.insert(fShapeA.begin(), r - fShapeA.size(), 1);
@@ -39,21 +46,21 @@ public:
                                      " cannot be broadcast");
          fShapeY[i] = std::max(fShapeA[i], fShapeB[i]);
       }
-      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShapeY);
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShapeY, fDynA || fDynB);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
       opName = "op_" + opName;
       std::stringstream out;
-      auto list = [](const std::vector<std::size_t> &v) {
+      auto list = [](const std::vector<std::size_t> &v, bool batched) {
          std::string s = "{";
          for (std::size_t i = 0; i < 6; ++i)
-            s += std::to_string(i < v.size() ? v[i] : 1) + (i < 5 ? ", " : "");
+            s += BatchScaled(batched && i == 0, i < v.size() ? v[i] : 1) + (i < 5 ? ", " : "");
          return s + "}";
       };
       out << "\n" << SP << "//------ Add " << opName << " --> " << ConvertShapeToString(fShapeY) << "\n";
       out << SP << "{\n";
-      out << SP << "   " << "sofie_add_desc d{" << fShapeY.size() << ", " << list(fShapeY) << ", " << list(fShapeA) << ", " << list(fShapeB)
+      out << SP << "   " << "sofie_add_desc d{" << fShapeY.size() << ", " << list(fShapeY, fDynA || fDynB) << ", " << list(fShapeA, fDynA) << ", " << list(fShapeB, fDynB)
           << ", tensor_" << fNA << ", tensor_" << fNB << ", tensor_" << fNY << "};\n";
       out << SP << "   " << "detail::Check(sofie_hip_add_f32(fCtx, &d), \"" << opName << " Add\");\n";
       out << SP << "}\n";
@@ -63,6 +70,7 @@ public:
 private:
    std::string fNA, fNB, fNY;
    std::vector<std::size_t> fShapeA, fShapeB, fShapeY;
+   bool fDynA = false, fDynB = false;
 };
 
 } // namespace SOFIE_HIP

@@ -32,14 +32,15 @@ public:
          throw std::runtime_error("SOFIE Activation Op: input tensor " + fNX + " is not float (an integer Relu is only emitted fused "
                                   "into the MatMulInteger that produces its input)");
       fShape = model.GetTensorShape(fNX);
-      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShape);
+      fDynamic = model.IsDynamicTensor(fNX);
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShape, fDynamic);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
       opName = "op_" + opName;
       std::stringstream out;
       out << "\n" << SP << "//------ " << ActivationEnumName(fAct) << " " << opName << "\n";
-      out << SP << "detail::Check(sofie_hip_unary_f32(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << ConvertShapeToLength(fShape)
+      out << SP << "detail::Check(sofie_hip_unary_f32(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << BatchScaled(fDynamic, ConvertShapeToLength(fShape))
           << ", " << ActivationEnumName(fAct) << ", " << FloatLiteral(fAlpha) << "), \"" << opName << " activation\");\n";
       return out.str();
    }
@@ -50,6 +51,7 @@ protected:
    std::string fNX, fNY;
    std::vector<std::size_t> fShape;
    ETensorType fType = ETensorType::FLOAT;
+   bool fDynamic = false;
 };
 
 // the reference's class names

@@ -61,7 +61,8 @@ public:
          fused[i] = scale[i] / std::sqrt(shifted);
       }
       model.AddInitializedTensor(fNFusedScale, ETensorType::FLOAT, {channels}, fused.data());
-      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShapeX);
+      fDynamic = model.IsDynamicTensor(fNX);
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShapeX, fDynamic);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
@@ -74,7 +75,7 @@ public:
       std::stringstream out;
       out << "\n" << SP << "//---- BatchNorm" << (fActivation == EActivationType::RELU ? " + ReLU " : " ") << opName << "\n";
       out << SP << "detail::Check(sofie_hip_batchnorm_f32(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", tensor_" << fNFusedScale << ", tensor_"
-          << fNMean << ", tensor_" << fNB << ", " << fShapeX[0] << ", " << fShapeX[1] << ", " << spatial << ", "
+          << fNMean << ", tensor_" << fNB << ", " << BatchScaledInt(fDynamic, fShapeX[0]) << ", " << fShapeX[1] << ", " << spatial << ", "
           << (fActivation == EActivationType::RELU ? 1 : 0) << "), \"" << opName << " BatchNormalization\");\n";
       return out.str();
    }
@@ -85,6 +86,7 @@ private:
    std::string fNX, fNScale, fNB, fNMean, fNVar, fNY, fNFusedScale;
    std::vector<std::size_t> fShapeX;
    EActivationType fActivation;
+   bool fDynamic = false;
 };
 
 } // namespace SOFIE_HIP

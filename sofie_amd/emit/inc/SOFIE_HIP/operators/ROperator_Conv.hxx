@@ -87,6 +87,11 @@ struct ConvGeometry {
          return {N, Cout, OW};
       return {N, Cout, OH, OW};
    }
+   // statement that scales the descriptor's image count by the run-time batch
+   std::string BatchLine(bool dynamic, const std::string &indent) const
+   {
+      return dynamic ? indent + "d.N = static_cast<std::int32_t>(sofie_batch * " + std::to_string(N) + ");\n" : std::string();
+   }
    std::string DescInitializer() const
    {
       std::stringstream s;
@@ -145,7 +150,8 @@ public:
          if (shapeB.size() != 1 || shapeB[0] != fGeo.Cout)
             throw std::runtime_error("SOFIE Conv op " + fNY + " : invalid shape for Bias tensor " + fNB + " : " + ConvertShapeToString(shapeB));
       }
-      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fGeo.OutputShape());
+      fDynamic = model.IsDynamicTensor(fNX);
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fGeo.OutputShape(), fDynamic);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
@@ -155,7 +161,7 @@ public:
       std::stringstream out;
       out << "\n" << SP << "//----  operator Conv " << opName << " --> " << ConvertShapeToString(fGeo.OutputShape()) << "\n";
       out << SP << "{\n";
-      out << SP << "   " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n";
+      out << SP << "   " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n" << fGeo.BatchLine(fDynamic, SP + "   ");
       out << SP << "   " << "detail::Check(sofie_hip_conv_f32(fCtx, &d, tensor_" << fNX << ", tensor_" << fNW << ", "
           << (fNB.empty() ? "nullptr" : "tensor_" + fNB) << ", " << ActivationEnumName(fActivation) << ", " << FloatLiteral(fActAlpha)
           << ", tensor_" << fNY << "), \"" << opName << " Conv\");\n";
@@ -172,6 +178,7 @@ private:
    EActivationType fActivation = EActivationType::UNDEFINED;
    float fActAlpha = 0.01f;
    ConvGeometry fGeo;
+   bool fDynamic = false;
 };
 
 } // namespace SOFIE_HIP

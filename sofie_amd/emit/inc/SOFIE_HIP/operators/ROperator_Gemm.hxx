@@ -80,6 +80,12 @@ public:
          throw std::runtime_error("SOFIE Gemm Op: only float tensors; quantised products use ROperator_QGemm");
       fShapeA = model.GetTensorShape(fNA);
       fShapeB = model.GetTensorShape(fNB);
+      // a run-time batch is the leading dimension of the operand (kept as 1 in its shape)
+      const bool dynA = model.IsDynamicTensor(fNA), dynB = model.IsDynamicTensor(fNB);
+      fDynamic = dynA || dynB;
+      if (fDynamic && (fShapeA.size() < 2 || fShapeB.size() < 2 || (dynA && fShapeA.size() < fShapeB.size()) ||
+                       (dynB && fShapeB.size() < fShapeA.size())))
+         throw std::runtime_error("SOFIE Gemm Op: with a run-time batch the batched operand must have the full rank of the product");
       // MatMul conventions of the reference (ROperator_Gemm.hxx:183-215): a 1-D A gets a leading 1, a 1-D B a
       // trailing 1, and the shorter shape is padded with leading 1s
       bool prependOne = false, appendOne = false;
@@ -125,6 +131,21 @@ public:
          fStrideA = leadA == 1 ? 0 : fM * fK;
          fStrideB = leadB == 1 ? 0 : fK * fN;
       }
+      fDynamicRows = fDynamicStack = false;
+      if (fDynamic && r == 2) {
+         // Y[batch, N] = A[batch, K] * B: the rows of the product grow with the batch
+         if (dynB || fAttrTransA)
+            throw std::runtime_error("SOFIE Gemm Op: a run-time batch must be the row dimension of A");
+         fDynamicRows = true;
+      } else if (fDynamic) {
+         // stacked product: the number of stacked matrices grows with the batch; an operand without the batch
+         // must be one matrix shared by all
+         if ((!dynA && leadA != 1) || (!dynB && leadB != 1))
+            throw std::runtime_error("SOFIE Gemm(MatMul): with a run-time batch the other operand must be a single matrix");
+         fDynamicStack = true;
+         fStrideA = dynA ? fM * fK : 0;
+         fStrideB = dynB ? fK * fN : 0;
+      }
       shapeY.push_back(fM);
       shapeY.push_back(fN);
 
@@ -143,18 +164,21 @@ public:
             c2 = {1, 1};
          // a C with exactly Y's shape goes to the kernel as C with the operator's beta; anything else is a
          // broadcast, for which the reference forces beta = 1 (ROperator_Gemm.hxx:580)
-         if (shapeC == shapeY)
+         // (with a run-time batch only a C that carries the batch itself can have Y's shape)
+         if (shapeC == shapeY && (!fDynamic || model.IsDynamicTensor(fNC)))
             fBiasMode = "SOFIE_BIAS_FULL";
+         else if (fDynamic && model.IsDynamicTensor(fNC))
+            throw std::runtime_error("SOFIE Gemm Op - a batched bias tensor must have the shape of the product");
          else if (c2.size() == 2 && c2[0] == 1 && c2[1] == fN)
             fBiasMode = "SOFIE_BIAS_ROW";
-         else if (c2.size() == 2 && c2[1] == 1 && c2[0] == fM)
+         else if (c2.size() == 2 && c2[1] == 1 && c2[0] == fM && !fDynamicRows)
             fBiasMode = "SOFIE_BIAS_COL";
          else if (c2.size() == 2 && c2[0] == 1 && c2[1] == 1)
             fBiasMode = "SOFIE_BIAS_SCALAR";
          else
             throw std::runtime_error("SOFIE Gemm Op - bias tensor of shape " + ConvertShapeToString(shapeC) +
                                      " cannot be uni-directional broadcasted to " + ConvertShapeToString(shapeY));
-         if (fBiasMode == std::string("SOFIE_BIAS_FULL") && fBatch > 1)
+         if (fBiasMode == std::string("SOFIE_BIAS_FULL") && (fBatch > 1 || fDynamicStack))
             fStrideC = fM * fN;
       } else if (fAttrBeta != 0) {
          fAttrBeta = 0; // no bias: beta is forced to zero as in the reference (ROperator_Gemm.hxx:491-499)
@@ -163,7 +187,7 @@ public:
          shapeY.erase(shapeY.end() - 2);
       if (appendOne)
          shapeY.pop_back();
-      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, shapeY);
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, shapeY, fDynamic);
    }
 
    std::string Generate_GPU_HIP(std::string opName) override
@@ -176,14 +200,14 @@ public:
           << " -> " << fNY << "\n";
       out << SP << "{\n";
       out << SP << "   " << "sofie_gemm_f32_desc d{};\n";
-      out << SP << "   " << "d.M = " << fM << "; d.N = " << fN << "; d.K = " << fK << "; d.transA = " << (fAttrTransA ? 1 : 0)
+      out << SP << "   " << "d.M = " << BatchScaledInt(fDynamicRows, fM) << "; d.N = " << fN << "; d.K = " << fK << "; d.transA = " << (fAttrTransA ? 1 : 0)
           << "; d.transB = " << (fAttrTransB ? 1 : 0) << ";\n";
       out << SP << "   " << "d.alpha = " << FloatLiteral(fAttrAlpha) << "; d.beta = " << FloatLiteral(fAttrBeta) << ";\n";
       out << SP << "   " << "d.A = tensor_" << fNA << "; d.B = tensor_" << fNB << "; d.C = " << (fNC.empty() ? "nullptr" : "tensor_" + fNC)
           << "; d.bias_mode = " << fBiasMode << ";\n";
       out << SP << "   " << "d.act = " << ActivationEnumName(fActivation) << "; d.act_alpha = " << FloatLiteral(fActAlpha) << ";\n";
-      out << SP << "   " << "d.Y = tensor_" << fNY << "; d.batch = " << fBatch << "; d.strideA = " << fStrideA << "; d.strideB = " << fStrideB
-          << "; d.strideC = " << fStrideC << "; d.strideY = " << (fBatch > 1 ? fM * fN : 0) << ";\n";
+      out << SP << "   " << "d.Y = tensor_" << fNY << "; d.batch = " << BatchScaledInt(fDynamicStack, fBatch) << "; d.strideA = " << fStrideA << "; d.strideB = "
+          << fStrideB << "; d.strideC = " << fStrideC << "; d.strideY = " << (fBatch > 1 || fDynamicStack ? fM * fN : 0) << ";\n";
       out << SP << "   " << "detail::Check(sofie_hip_gemm_f32(fCtx, &d), \"" << opName << " Gemm\");\n";
       out << SP << "}\n";
       return out.str();
@@ -198,6 +222,7 @@ private:
    std::vector<std::size_t> fShapeA, fShapeB;
    std::size_t fM = 0, fN = 0, fK = 0, fBatch = 1, fStrideA = 0, fStrideB = 0, fStrideC = 0;
    std::string fBiasMode;
+   bool fDynamic = false, fDynamicRows = false, fDynamicStack = false;
 };
 
 } // namespace SOFIE_HIP

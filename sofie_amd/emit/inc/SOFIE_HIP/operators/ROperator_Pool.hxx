@@ -32,7 +32,8 @@ public:
       std::vector<std::size_t> shapeY(fShapeX.size(), 1);
       shapeY[0] = fShapeX[0];
       shapeY[1] = fShapeX[1];
-      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, shapeY);
+      fDynamic = model.IsDynamicTensor(fNX);
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, shapeY, fDynamic);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
@@ -42,7 +43,7 @@ public:
          hw *= fShapeX[i];
       std::stringstream out;
       out << "\n" << SP << "//----  operator GlobalAveragePool " << opName << "\n";
-      out << SP << "detail::Check(sofie_hip_global_avg_pool_f32(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << fShapeX[0] * fShapeX[1]
+      out << SP << "detail::Check(sofie_hip_global_avg_pool_f32(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << BatchScaledInt(fDynamic, fShapeX[0] * fShapeX[1])
           << ", " << hw << "), \"" << opName << " GlobalAveragePool\");\n";
       return out.str();
    }
@@ -52,6 +53,7 @@ private:
    std::string fNX, fNY;
    std::vector<std::size_t> fShapeX;
    ETensorType fType = ETensorType::FLOAT;
+   bool fDynamic = false;
 };
 
 } // namespace SOFIE_HIP

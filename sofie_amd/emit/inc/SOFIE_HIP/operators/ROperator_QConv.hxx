@@ -78,9 +78,10 @@ public:
       fGeo.Resolve(fAttrAutopad, fAttrDilations, fAttrGroup, fAttrKernelShape, fAttrPads, fAttrStrides, model.GetTensorShape(fNX),
                    model.GetTensorShape(fNW));
       fXLayout = model.GetTensorLayout(fNX);
+      fDynamic = model.IsDynamicTensor(fNX);
       if (fInt32Out) {
          fYLayout = kLayoutNCHW;
-         model.AddIntermediateTensor(fNY, ETensorType::INT32, fGeo.OutputShape());
+         model.AddIntermediateTensor(fNY, ETensorType::INT32, fGeo.OutputShape(), fDynamic);
          return;
       }
       const float xs = model.GetScalarInitializer(fNXS), ys = model.GetScalarInitializer(fNYS);
@@ -111,7 +112,7 @@ public:
       for (OperatorKind k : model.ConsumerKinds(fNY))
          if (k != OperatorKind::QCONV && k != OperatorKind::QPOOL)
             fYLayout = kLayoutNCHW;
-      model.AddIntermediateTensor(fNY, ETensorType::INT8, fGeo.OutputShape());
+      model.AddIntermediateTensor(fNY, ETensorType::INT8, fGeo.OutputShape(), fDynamic);
       model.SetTensorLayout(fNY, fYLayout);
    }
    std::size_t PackedK() const { return ((fGeo.C / fGeo.group) * fGeo.kh * fGeo.kw + 15) / 16 * 16; }
@@ -144,8 +145,9 @@ public:
          return 0;
       const std::size_t per_image = (fGeo.OH * fGeo.OW * PackedK() + 255) / 256 * 256;
       std::size_t images = std::max<std::size_t>(1, (std::size_t(64) << 20) / per_image);
-      return per_image * std::min(images, fGeo.N);
+      return per_image * std::min(images, fGeo.N); // with a run-time batch N is 1: the column matrix of one image per batch entry
    }
+   bool WorkspacePerBatchEntry() const override { return fDynamic; }
    std::string Generate_GPU_HIP(std::string opName) override
    {
       const std::string ws = "workspace_op_" + opName;
@@ -154,7 +156,7 @@ public:
       out << "\n" << SP << "//----  operator " << (fInt32Out ? "ConvInteger " : "QLinearConv ") << opName << " --> " << ConvertShapeToString(fGeo.OutputShape())
           << (fYLayout == kLayoutNHWC ? " (stored NHWC)" : "") << (ImplicitGemm() ? ", implicit GEMM" : ", column matrix") << "\n";
       out << SP << "{\n";
-      out << SP << "   " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n";
+      out << SP << "   " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n" << fGeo.BatchLine(fDynamic, SP + "   ");
       out << SP << "   " << "sofie_conv_i8_args a{};\n";
       out << SP << "   " << "a.X = tensor_" << fNX << "; a.W = packed_" << fNW << "; a.w_is_packed = 1; a.bias = "
           << (fNB.empty() ? "nullptr" : "tensor_" + fNB) << "; a.scale = " << (fInt32Out ? std::string("nullptr") : "tensor_" + fNM) << ";\n";
@@ -162,7 +164,7 @@ public:
           << (fXLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.y_layout = "
           << (fYLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.Y = tensor_" << fNY << ";\n";
       if (GetWorkspaceBytes())
-         out << SP << "   " << "a.workspace = " << ws << "; a.workspace_bytes = " << GetWorkspaceBytes() << ";\n";
+         out << SP << "   " << "a.workspace = " << ws << "; a.workspace_bytes = " << BatchScaled(fDynamic, GetWorkspaceBytes()) << ";\n";
       out << SP << "   " << "detail::Check(sofie_hip_conv_i8(fCtx, &d, &a), \"" << opName << " QLinearConv\");\n";
       out << SP << "}\n";
       return out.str();
@@ -174,7 +176,7 @@ private:
    std::size_t fAttrGroup;
    std::vector<std::size_t> fAttrKernelShape, fAttrPads, fAttrStrides;
    std::string fNX, fNXS, fNXZ, fNW, fNWS, fNWZ, fNYS, fNYZ, fNB, fNY, fNM;
-   bool fRelu = false, fInt32Out = false;
+   bool fRelu = false, fInt32Out = false, fDynamic = false;
    int fXLayout = kLayoutNCHW, fYLayout = kLayoutNCHW;
    ConvGeometry fGeo;
 };
@@ -203,7 +205,8 @@ public:
       std::vector<std::size_t> shapeY(fShapeX.size(), 1);
       shapeY[0] = fShapeX[0];
       shapeY[1] = fShapeX[1];
-      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, shapeY);
+      fDynamic = model.IsDynamicTensor(fNX);
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, shapeY, fDynamic);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
@@ -213,7 +216,7 @@ public:
          hw *= fShapeX[i];
       std::stringstream out;
       out << "\n" << SP << "//----  DequantizeLinear + GlobalAveragePool " << opName << "\n";
-      out << SP << "detail::Check(sofie_hip_global_avg_pool_i8(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << fShapeX[0] << ", " << fShapeX[1]
+      out << SP << "detail::Check(sofie_hip_global_avg_pool_i8(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << BatchScaledInt(fDynamic, fShapeX[0]) << ", " << fShapeX[1]
           << ", " << hw << ", " << (fLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << ", " << FloatLiteral(fScale) << "), \""
           << opName << " GlobalAveragePool\");\n";
       return out.str();
@@ -224,6 +227,7 @@ private:
    std::vector<std::size_t> fShapeX;
    float fScale = 1.0f;
    int fLayout = kLayoutNCHW;
+   bool fDynamic = false;
 };
 
 // Flatten(axis): [d0..dn) -> [prod(d0..axis), prod(axis..n)], same bytes; emitted as a copy
@@ -249,14 +253,17 @@ public:
          (i < axis ? a : b) *= shape[i];
       fType = model.GetTensorType(fNX);
       fBytes = a * b * GetTypeSize(fType);
-      model.AddIntermediateTensor(fNY, fType, {a, b});
+      fDynamic = model.IsDynamicTensor(fNX);
+      if (fDynamic && axis < 1)
+         throw std::runtime_error("SOFIE Flatten Op: axis 0 would fold the run-time batch of " + fNX + " into the second dimension");
+      model.AddIntermediateTensor(fNY, fType, {a, b}, fDynamic);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
       opName = "op_" + opName;
       std::stringstream out;
       out << "\n" << SP << "//----  Flatten " << opName << "\n";
-      out << SP << "detail::Check(sofie_hip_copy(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << fBytes << "), \"" << opName << " Flatten\");\n";
+      out << SP << "detail::Check(sofie_hip_copy(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << BatchScaled(fDynamic, fBytes) << "), \"" << opName << " Flatten\");\n";
       return out.str();
    }
 
@@ -265,6 +272,7 @@ private:
    std::string fNX, fNY;
    ETensorType fType = ETensorType::FLOAT;
    std::size_t fBytes = 0;
+   bool fDynamic = false;
 };
 
 } // namespace SOFIE_HIP

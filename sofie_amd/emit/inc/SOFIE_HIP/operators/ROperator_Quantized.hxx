@@ -35,14 +35,15 @@ public:
       if (!(fScale > 0))
          throw std::runtime_error("SOFIE QuantizeLinear Op: scale " + fNS + " must be positive");
       fShape = model.GetTensorShape(fNX);
-      model.AddIntermediateTensor(fNY, ETensorType::INT8, fShape);
+      fDynamic = model.IsDynamicTensor(fNX);
+      model.AddIntermediateTensor(fNY, ETensorType::INT8, fShape, fDynamic);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
       opName = "op_" + opName;
       std::stringstream out;
       out << "\n" << SP << "//------ QuantizeLinear " << opName << "\n";
-      out << SP << "detail::Check(sofie_hip_quantize_linear(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << ConvertShapeToLength(fShape)
+      out << SP << "detail::Check(sofie_hip_quantize_linear(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << BatchScaled(fDynamic, ConvertShapeToLength(fShape))
           << ", " << FloatLiteral(fScale) << "), \"" << opName << " QuantizeLinear\");\n";
       return out.str();
    }
@@ -51,6 +52,7 @@ private:
    std::string fNX, fNS, fNY;
    float fScale = 0;
    std::vector<std::size_t> fShape;
+   bool fDynamic = false;
 };
 
 class ROperator_DequantizeLinear final : public ROperator {
@@ -73,7 +75,8 @@ public:
          throw std::runtime_error("SOFIE DequantizeLinear Op: input tensor " + fNX + " is neither int8 nor int32");
       fScale = model.GetScalarInitializer(fNS);
       fShape = model.GetTensorShape(fNX);
-      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShape);
+      fDynamic = model.IsDynamicTensor(fNX);
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShape, fDynamic);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
@@ -81,7 +84,7 @@ public:
       std::stringstream out;
       out << "\n" << SP << "//------ DequantizeLinear " << opName << "\n";
       out << SP << "detail::Check(sofie_hip_dequantize_linear_" << (fType == ETensorType::INT8 ? "i8" : "i32") << "(fCtx, tensor_" << fNY
-          << ", tensor_" << fNX << ", " << ConvertShapeToLength(fShape) << ", " << FloatLiteral(fScale) << "), \"" << opName
+          << ", tensor_" << fNX << ", " << BatchScaled(fDynamic, ConvertShapeToLength(fShape)) << ", " << FloatLiteral(fScale) << "), \"" << opName
           << " DequantizeLinear\");\n";
       return out.str();
    }
@@ -91,6 +94,7 @@ private:
    float fScale = 0;
    ETensorType fType = ETensorType::INT8;
    std::vector<std::size_t> fShape;
+   bool fDynamic = false;
 };
 
 // int8 x int8 -> int32 product with everything that can ride on its store.  As a plain MatMulInteger the
@@ -148,6 +152,9 @@ public:
       fK = sA[1];
       fN = sB[1];
       fWeightIsInitializer = model.IsInitializedTensor(fNB);
+      fDynamic = model.IsDynamicTensor(fNA);
+      if (model.IsDynamicTensor(fNB))
+         throw std::runtime_error("SOFIE QGemm Op: a run-time batch must be the row dimension of A");
       if (!fNBias.empty()) {
          if (!model.CheckIfTensorAlreadyExist(fNBias) || model.GetTensorType(fNBias) != ETensorType::INT32 ||
              ConvertShapeToLength(model.GetTensorShape(fNBias)) != fN)
@@ -159,7 +166,7 @@ public:
             throw std::runtime_error("SOFIE QGemm Op: scale " + fNScale + " must be a float tensor of " + std::to_string(fN) + " elements");
       }
       const ETensorType ty = fOut == Out::I32 ? ETensorType::INT32 : fOut == Out::F32 ? ETensorType::FLOAT : ETensorType::INT8;
-      model.AddIntermediateTensor(fNY, ty, {fM, fN});
+      model.AddIntermediateTensor(fNY, ty, {fM, fN}, fDynamic);
    }
    // a constant B is re-laid out once into [N,K] (K contiguous, what the matrix-core kernel reads)
    std::vector<std::pair<std::string, std::size_t>> GetPersistentBuffers() override
@@ -186,7 +193,7 @@ public:
       out << "\n" << SP << "//--------- QGemm " << opName << " int8 { " << fM << " , " << fK << " } * { " << fK << " , " << fN << " } -> " << fNY << "\n";
       out << SP << "{\n";
       out << SP << "   " << "sofie_gemm_i8_desc d{};\n";
-      out << SP << "   " << "d.M = " << fM << "; d.N = " << fN << "; d.K = " << fK << ";\n";
+      out << SP << "   " << "d.M = " << BatchScaledInt(fDynamic, fM) << "; d.N = " << fN << "; d.K = " << fK << ";\n";
       if (fWeightIsInitializer)
          out << SP << "   " << "d.A = tensor_" << fNA << "; d.B = packed_" << fNB << "; d.transB = 1;\n";
       else
@@ -206,7 +213,7 @@ public:
 private:
    std::string fNA, fNB, fNY, fNBias, fNScale;
    std::size_t fM = 0, fN = 0, fK = 0;
-   bool fWeightIsInitializer = false, fReluAcc = false, fReluOut = false;
+   bool fWeightIsInitializer = false, fReluAcc = false, fReluOut = false, fDynamic = false;
    Out fOut = Out::I32;
    float fScale = 1.0f, fQScale = 1.0f;
 };
@@ -257,7 +264,8 @@ public:
       if (!fNBias.empty() && (!model.CheckIfTensorAlreadyExist(fNBias) || model.GetTensorType(fNBias) != ETensorType::FLOAT ||
                               ConvertShapeToLength(model.GetTensorShape(fNBias)) != fN))
          throw std::runtime_error("SOFIE Fp8Gemm Op: bias " + fNBias + " must be a float tensor of " + std::to_string(fN) + " elements");
-      model.AddIntermediateTensor(fNY, fOutType, {fM, fN});
+      fDynamic = model.IsDynamicTensor(fNX);
+      model.AddIntermediateTensor(fNY, fOutType, {fM, fN}, fDynamic);
    }
    std::vector<std::pair<std::string, std::size_t>> GetPersistentBuffers() override
    {
@@ -274,7 +282,9 @@ public:
           << fK << ", " << fN << ", 0, 0), \"re-layout of " << fNW << "\");\n";
       return out.str();
    }
-   std::size_t GetWorkspaceBytes() override { return ((fM * fK + 255) / 256) * 256; }
+   // the e4m3 copy of the activations: K bytes per row
+   std::size_t GetWorkspaceBytes() override { return fDynamic ? fM * fK : ((fM * fK + 255) / 256) * 256; }
+   bool WorkspacePerBatchEntry() const override { return fDynamic; }
    std::string Generate_GPU_HIP(std::string opName) override
    {
       const std::string ws = "workspace_op_" + opName;
@@ -283,10 +293,10 @@ public:
       std::stringstream out;
       out << "\n" << SP << "//--------- Fp8Gemm " << opName << " e4m3 { " << fM << " , " << fK << " } * { " << fK << " , " << fN << " } -> " << fNY << "\n";
       out << SP << "{\n";
-      out << SP << "   " << "detail::Check(sofie_hip_quantize_fp8(fCtx, reinterpret_cast<uint8_t *>(" << ws << "), tensor_" << fNX << ", " << fM * fK
+      out << SP << "   " << "detail::Check(sofie_hip_quantize_fp8(fCtx, reinterpret_cast<uint8_t *>(" << ws << "), tensor_" << fNX << ", " << BatchScaled(fDynamic, fM * fK)
           << ", " << FloatLiteral(fXScale) << "), \"" << opName << " quantisation\");\n";
       out << SP << "   " << "sofie_gemm_fp8_desc d{};\n";
-      out << SP << "   " << "d.M = " << fM << "; d.N = " << fN << "; d.K = " << fK << "; d.transB = 1;\n";
+      out << SP << "   " << "d.M = " << BatchScaledInt(fDynamic, fM) << "; d.N = " << fN << "; d.K = " << fK << "; d.transB = 1;\n";
       out << SP << "   " << "d.A = reinterpret_cast<const uint8_t *>(" << ws << "); d.B = "
           << (fTransB ? "tensor_" + fNW : "reinterpret_cast<const uint8_t *>(packed_" + fNW + ")") << ";\n";
       out << SP << "   " << "d.bias = " << (fNBias.empty() ? "nullptr" : "tensor_" + fNBias) << "; d.scale = " << FloatLiteral(prod)
@@ -305,6 +315,7 @@ private:
    ETensorType fOutType;
    std::string fNY;
    std::size_t fM = 0, fN = 0, fK = 0;
+   bool fDynamic = false;
 };
 
 // int8 Relu on an int32 accumulator tensor is only meaningful fused; as a stand-alone operator on int32 it

@@ -34,6 +34,24 @@ void RModel::AddInputTensorInfo(std::string input_name, ETensorType type, std::v
    fInputTensorInfos[input_name] = TensorInfo{type, shape};
 }
 
+void RModel::AddInputTensorInfo(std::string input_name, ETensorType type, std::vector<Dim> shape)
+{
+   std::vector<std::size_t> fixed;
+   bool anyParam = false;
+   for (std::size_t i = 0; i < shape.size(); ++i) {
+      if (shape[i].isParam) {
+         if (i != 0)
+            throw std::runtime_error("SOFIE: input tensor " + input_name + " has the parameter " + shape[i].param +
+                                     " in dimension " + std::to_string(i) + "; only the leading (batch) dimension may be a parameter");
+         anyParam = true;
+      }
+      fixed.push_back(shape[i].isParam ? 1 : shape[i].dim);
+   }
+   AddInputTensorInfo(input_name, type, fixed);
+   if (anyParam)
+      fInputDimShapes[UTILITY::Clean_name(input_name)] = std::move(shape);
+}
+
 void RModel::AddInputTensorName(std::string name) { fInputTensorNames.push_back(UTILITY::Clean_name(name)); }
 
 void RModel::AddInitializedTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, std::shared_ptr<void> data)
@@ -61,12 +79,16 @@ void RModel::AddConstantTensor(std::string tensor_name, ETensorType type, std::v
    fInitializedTensors[UTILITY::Clean_name(tensor_name)].constant = true;
 }
 
-void RModel::AddIntermediateTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape)
+void RModel::AddIntermediateTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape, bool batched)
 {
    tensor_name = UTILITY::Clean_name(tensor_name);
    if (CheckIfTensorAlreadyExist(tensor_name))
       throw std::runtime_error("SOFIE: intermediate tensor with name " + tensor_name + " already exists \n");
+   if (batched && (shape.empty() || shape[0] != 1))
+      throw std::runtime_error("SOFIE: tensor " + tensor_name + " does not carry the run-time batch as its leading dimension");
    fIntermediateTensorInfos[tensor_name] = TensorInfo{type, shape};
+   if (batched)
+      fBatched[tensor_name] = true;
 }
 
 void RModel::AddOperator(std::unique_ptr<ROperator> op, int order_execution)
@@ -248,10 +270,24 @@ std::vector<OperatorKind> RModel::ConsumerKinds(const std::string &name) const
    return kinds;
 }
 
-void RModel::Initialize()
+void RModel::Initialize(int batchSize)
 {
    if (fInitialized)
       return;
+   // the batch parameter: fixed now if a batch size is given, else left to the Session
+   for (auto &kv : fInputDimShapes) {
+      const Dim &d = kv.second[0];
+      if (batchSize > 0) {
+         fInputTensorInfos[kv.first].shape[0] = static_cast<std::size_t>(batchSize);
+         continue;
+      }
+      if (!fBatchParam.empty() && fBatchParam != d.param)
+         throw std::runtime_error("SOFIE: inputs use two shape parameters, " + fBatchParam + " and " + d.param +
+                                  "; this backend takes one (the batch)");
+      fBatchParam = d.param;
+      fBatchDefault = std::max<std::size_t>(fBatchDefault, d.dim ? d.dim : 1);
+      fBatched[kv.first] = true;
+   }
    for (auto &n : fInputTensorNames)
       if (!fInputTensorInfos.count(n))
          throw std::runtime_error("SOFIE: input tensor " + n + " has no tensor info");
@@ -262,6 +298,15 @@ void RModel::Initialize()
    for (std::size_t i = 0; i < fOperators.size(); ++i) {
       fOperators[i]->SetOpOrder(i);
       fOperators[i]->Initialize(*this);
+      // an operator that reads a batched tensor has to say what it makes of the batch
+      bool batchedIn = false, batchedOut = false;
+      for (auto &in : fOperators[i]->GetInputTensorNames())
+         batchedIn = batchedIn || IsDynamicTensor(in);
+      for (auto &y : fOperators[i]->GetOutputTensorNames())
+         batchedOut = batchedOut || IsDynamicTensor(y);
+      if (batchedIn && !batchedOut)
+         throw std::runtime_error("SOFIE: operator " + std::to_string(i) + " (output " + fOperators[i]->GetOutputTensorNames().at(0) +
+                                  ") does not support a run-time batch; generate with a fixed batch size");
    }
    for (auto &o : fOutputTensorNames)
       if (!CheckIfTensorAlreadyExist(o))
@@ -279,51 +324,81 @@ void RModel::PlanMemory()
 {
    fPlan.clear();
    fOffsets.clear();
-   std::size_t off = 0;
+   const bool dyn = HasDynamicBatch();
+   // With a run-time batch the arena has two parts.  The static part holds what does not depend on the batch.  Everything
+   // that carries the batch is planned for ONE batch entry, in units of 16 bytes; the Session multiplies those offsets by
+   // its capacity (the maximum batch rounded up to a multiple of 16), so regions that are disjoint per entry stay disjoint
+   // and every region starts on a 256-byte boundary.
+   const std::size_t entryAlign = 16;
+   auto alignEntry = [&](std::size_t b) { return (b + entryAlign - 1) / entryAlign * entryAlign; };
+   std::size_t off = 0, entryOff = 0;
    auto addStatic = [&](const std::string &name, std::size_t bytes) {
-      fPlan.push_back({name, off, bytes, -1, (int)fOperators.size() + 1, false});
+      fPlan.push_back({name, off, bytes, -1, (int)fOperators.size() + 1, false, false});
       fOffsets[name] = off;
       off += AlignUp(bytes ? bytes : 1);
    };
+   auto addPerEntry = [&](const std::string &name, std::size_t bytes) {
+      fPlan.push_back({name, entryOff, bytes, -1, (int)fOperators.size() + 1, false, true});
+      fOffsets[name] = entryOff;
+      entryOff += alignEntry(bytes ? bytes : 1);
+   };
+   auto tensorBytes = [&](const TensorInfo &ti) { return ConvertShapeToLength(ti.shape) * GetTypeSize(ti.type); };
    for (auto &kv : fInitializedTensors)
       addStatic("tensor_" + kv.first, ConvertShapeToLength(kv.second.shape) * GetTypeSize(kv.second.type));
    for (auto &op : fOperators)
       for (auto &pb : op->GetPersistentBuffers())
          addStatic(pb.first, pb.second);
+   auto addGraphTensor = [&](const std::string &n, const TensorInfo &ti) {
+      if (IsDynamicTensor(n))
+         addPerEntry("tensor_" + n, tensorBytes(ti));
+      else
+         addStatic("tensor_" + n, tensorBytes(ti));
+   };
    for (auto &n : fInputTensorNames)
-      addStatic("tensor_" + n, ConvertShapeToLength(fInputTensorInfos[n].shape) * GetTypeSize(fInputTensorInfos[n].type));
+      addGraphTensor(n, fInputTensorInfos[n]);
    for (auto &n : fOutputTensorNames)
       if (fIntermediateTensorInfos.count(n))
-         addStatic("tensor_" + n, ConvertShapeToLength(fIntermediateTensorInfos[n].shape) * GetTypeSize(fIntermediateTensorInfos[n].type));
-   const std::size_t poolBase = off;
+         addGraphTensor(n, fIntermediateTensorInfos[n]);
 
    std::vector<TensorLifeInfo> life;
    std::vector<std::string> names;
    for (std::size_t i = 0; i < fOperators.size(); ++i) {
       for (auto &y : fOperators[i]->GetOutputTensorNames()) {
          if (!fIntermediateTensorInfos.count(y) || fOffsets.count("tensor_" + y))
-            continue; // graph outputs are static
+            continue; // graph outputs are placed above
+         const auto &ti = fIntermediateTensorInfos[y];
+         if (dyn && !IsDynamicTensor(y)) { // rare: an intermediate that does not depend on the batch keeps a region of its own
+            addStatic("tensor_" + y, tensorBytes(ti));
+            continue;
+         }
          int last = (int)i;
          for (std::size_t j = i + 1; j < fOperators.size(); ++j)
             for (auto &in : fOperators[j]->GetInputTensorNames())
                if (in == y)
                   last = (int)j;
-         const auto &ti = fIntermediateTensorInfos[y];
-         life.push_back({(int)i, last + 1, AlignUp(ConvertShapeToLength(ti.shape) * GetTypeSize(ti.type))});
+         life.push_back({(int)i, last + 1, dyn ? alignEntry(tensorBytes(ti)) : AlignUp(tensorBytes(ti))});
          names.push_back("tensor_" + y);
       }
       if (std::size_t ws = fOperators[i]->GetWorkspaceBytes()) {
-         life.push_back({(int)i, (int)i + 1, AlignUp(ws)});
-         names.push_back("workspace_op_" + std::to_string(i));
+         const std::string wname = "workspace_op_" + std::to_string(i);
+         if (dyn && !fOperators[i]->WorkspacePerBatchEntry()) {
+            addStatic(wname, ws);
+            continue;
+         }
+         life.push_back({(int)i, (int)i + 1, dyn ? alignEntry(ws) : AlignUp(ws)});
+         names.push_back(wname);
       }
    }
+   const std::size_t poolBase = dyn ? entryOff : off;
    MemoryResult r = OrganizeMemory(life);
    for (std::size_t t = 0; t < life.size(); ++t) {
-      fPlan.push_back({names[t], poolBase + r.offsets[t], life[t].size, life[t].begin, life[t].end, true});
+      fPlan.push_back({names[t], poolBase + r.offsets[t], life[t].size, life[t].begin, life[t].end, true, dyn});
       fOffsets[names[t]] = poolBase + r.offsets[t];
    }
-   fPoolBytes = r.total_bytes;
-   fArenaBytes = poolBase + r.total_bytes;
+   fPoolBytes = r.total_bytes; // per batch entry when the batch is a run-time parameter
+   fStaticBytes = off;
+   fBatchEntryBytes = dyn ? entryOff + r.total_bytes : 0;
+   fArenaBytes = dyn ? off + entryAlign * fBatchEntryBytes : poolBase + r.total_bytes; // dynamic: the smallest Session (capacity 16)
    if (fArenaBytes == 0)
       fArenaBytes = kPoolAlignBytes;
 }
@@ -665,8 +740,26 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    }
    gc << "struct Session {\n";
    gc << "   // one arena: weights, operator-owned buffers, inputs, outputs, then the pool of intermediates\n";
-   gc << "   static constexpr std::size_t kArenaBytes = " << fArenaBytes << ";\n";
-   gc << "   static constexpr std::size_t kIntermediatePoolBytes = " << fPoolBytes << ";\n";
+   const bool dyn = HasDynamicBatch();
+   // name of the batch parameter in the emitted signatures (the reference uses the parameter's own name)
+   std::string bp = fBatchParam;
+   for (const char *reserved : {"filename", "stream", "device", "provider", "weights_blob", "base", "place", "f", "host", "init"})
+      if (bp == reserved)
+         bp += "_batch";
+   const std::string arenaBytes = dyn ? "ArenaBytes(fMaxBatch)" : "kArenaBytes";
+   if (dyn) {
+      gc << "   // the batch is a run-time parameter: what carries it is planned per batch entry and scaled by the capacity,\n";
+      gc << "   // the constructor's maximum rounded up to a multiple of 16 (every region stays 256-byte aligned)\n";
+      gc << "   static constexpr std::size_t kStaticBytes = " << fStaticBytes << ";\n";
+      gc << "   static constexpr std::size_t kBytesPerBatchEntry = " << fBatchEntryBytes << ";\n";
+      gc << "   static constexpr std::size_t kIntermediatePoolBytesPerBatchEntry = " << fPoolBytes << ";\n";
+      gc << "   static std::size_t Capacity(std::size_t maxBatch) { return ((maxBatch ? maxBatch : 1) + 15) / 16 * 16; }\n";
+      gc << "   static std::size_t ArenaBytes(std::size_t maxBatch) { return kStaticBytes + Capacity(maxBatch) * kBytesPerBatchEntry; }\n";
+      gc << "   std::size_t fMaxBatch = 0, fCapacity = 0;\n";
+   } else {
+      gc << "   static constexpr std::size_t kArenaBytes = " << fArenaBytes << ";\n";
+      gc << "   static constexpr std::size_t kIntermediatePoolBytes = " << fPoolBytes << ";\n";
+   }
    gc << "   sofie_hip_ctx *fCtx = nullptr;\n";
    if (customMemory)
       gc << "   MemoryProvider fProvider;\n   void *fBlock = nullptr;\n";
@@ -675,26 +768,32 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
          return ConvertTypeToString(GetTensorType(planName.substr(7)));
       return "int8_t";
    };
+   auto offsetText = [&](const PlannedTensor &p) {
+      return p.perBatch ? "kStaticBytes + fCapacity * " + std::to_string(p.offset) : std::to_string(p.offset);
+   };
    for (auto &p : fPlan)
-      gc << "   " << typeOf(p.name) << " *" << p.name << " = nullptr; // arena offset " << p.offset << ", " << p.bytes << " bytes"
-         << (p.pooled ? ", live [" + std::to_string(p.begin) + "," + std::to_string(p.end) + ")" : "") << "\n";
+      gc << "   " << typeOf(p.name) << " *" << p.name << " = nullptr; // " << (p.perBatch ? "per batch entry: offset " : "arena offset ") << p.offset
+         << ", " << p.bytes << " bytes" << (p.pooled ? ", live [" + std::to_string(p.begin) + "," + std::to_string(p.end) + ")" : "") << "\n";
    gc << "\n";
    // constructor
    if (safetensors) {
       // the file is read whole and handed to the constructor that takes the payload
       gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "std::string filename = \"" << fName << "_GPU_HIP.safetensors\""
-         << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
+         << (dyn ? ", std::size_t " + bp + " = " + std::to_string(fBatchDefault) : std::string()) << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
       gc << "      : Session(" << (customMemory ? "std::move(provider), " : "") << "SafetensorsBlob(detail::LoadWeightsFromFile(filename))"
-         << (externalStream ? ", stream" : "") << ", device)\n   {\n   }\n";
+         << (dyn ? ", " + bp : std::string()) << (externalStream ? ", stream" : "") << ", device)\n   {\n   }\n";
       gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "SafetensorsBlob weights_blob"
-         << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
+         << (dyn ? ", std::size_t " + bp + " = " + std::to_string(fBatchDefault) : std::string()) << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
    } else {
       gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "std::string filename = \""
-         << (noWeightFile ? "" : fName + "_GPU_HIP.dat") << "\"" << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
+         << (noWeightFile ? "" : fName + "_GPU_HIP.dat") << "\"" << (dyn ? ", std::size_t " + bp + " = " + std::to_string(fBatchDefault) : std::string()) << (externalStream ? ", void *stream = nullptr" : "")
+         << ", int device = 0)\n";
    }
    if (customMemory)
       gc << "      : fProvider(std::move(provider))\n";
    gc << "   {\n";
+   if (dyn)
+      gc << "      fMaxBatch = " << bp << ";\n      fCapacity = Capacity(" << bp << ");\n";
    if (safetensors) {
       // the payload is checked against the model before any device work
       gc << "      detail::SafetensorsReader sofie_weights_reader(weights_blob);\n";
@@ -708,21 +807,21 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    gc << "      detail::Check(sofie_hip_ctx_create(&fCtx, device, " << (externalStream ? "stream" : "nullptr") << "), \"Session\");\n";
    gc << "      try {\n";
    if (customMemory) {
-      gc << "         fBlock = fProvider.alloc(kArenaBytes);\n";
+      gc << "         fBlock = fProvider.alloc(" << arenaBytes << ");\n";
       gc << "         if (!fBlock)\n            throw std::runtime_error(\"SOFIE HIP Session: the memory provider returned no block\");\n";
-      gc << "         detail::Check(sofie_hip_arena_adopt(fCtx, fBlock, kArenaBytes), \"adoption of the caller's block\");\n";
+      gc << "         detail::Check(sofie_hip_arena_adopt(fCtx, fBlock, " << arenaBytes << "), \"adoption of the caller's block\");\n";
       gc << "         auto place = [&](std::size_t offset) -> char * {\n"
             "            void *p = fProvider.assign ? fProvider.assign(offset) : static_cast<char *>(fBlock) + offset;\n"
             "            if (!p)\n               throw std::runtime_error(\"SOFIE HIP Session: the memory provider assigned no address\");\n"
             "            return static_cast<char *>(p);\n         };\n";
       for (auto &p : fPlan)
-         gc << "         " << p.name << " = reinterpret_cast<" << typeOf(p.name) << " *>(place(" << p.offset << "));\n";
+         gc << "         " << p.name << " = reinterpret_cast<" << typeOf(p.name) << " *>(place(" << offsetText(p) << "));\n";
    } else {
-      gc << "         detail::Check(sofie_hip_arena_create(fCtx, kArenaBytes, " << kPoolAlignBytes << "), \"arena allocation\");\n";
+      gc << "         detail::Check(sofie_hip_arena_create(fCtx, " << arenaBytes << ", " << kPoolAlignBytes << "), \"arena allocation\");\n";
       gc << "         char *base = static_cast<char *>(sofie_hip_arena_ptr(fCtx, 0));\n";
       gc << "         if (!base)\n            throw std::runtime_error(\"SOFIE HIP runtime error: arena is null\");\n";
       for (auto &p : fPlan)
-         gc << "         " << p.name << " = reinterpret_cast<" << typeOf(p.name) << " *>(base + " << p.offset << ");\n";
+         gc << "         " << p.name << " = reinterpret_cast<" << typeOf(p.name) << " *>(base + " << offsetText(p) << ");\n";
    }
    bool anyWeights = false, anyConstants = false;
    for (auto &kv : fInitializedTensors)
@@ -795,7 +894,10 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
       gc << "   ~Session() { sofie_hip_ctx_destroy(fCtx); }\n";
    }
    gc << "   Session(const Session &) = delete;\n   Session &operator=(const Session &) = delete;\n\n";
-   gc << "   std::size_t GetIntermediateMemoryPoolSize() const { return kIntermediatePoolBytes; }\n";
+   gc << "   std::size_t GetIntermediateMemoryPoolSize() const { return "
+      << (dyn ? "fCapacity * kIntermediatePoolBytesPerBatchEntry" : "kIntermediatePoolBytes") << "; }\n";
+   if (dyn)
+      gc << "   std::size_t GetMaxBatch() const { return fMaxBatch; }\n";
    // device-resident use: where to write the inputs and read the outputs around infer_nosync()
    for (auto &n : fInputTensorNames)
       gc << "   " << ConvertTypeToString(fInputTensorInfos[n].type) << " *device_input_" << n << "() const { return tensor_" << n << "; }\n";
@@ -806,13 +908,21 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    // infer_nosync: the operators, inputs and outputs resident in the arena
    gc << "   // enqueues one inference on the session's stream: inputs are read from the tensor_<input> regions of the arena,\n";
    gc << "   // results land in the tensor_<output> regions (overwritten by the next call)\n";
-   gc << "   void infer_nosync()\n   {";
+   if (dyn) {
+      gc << "   // " << bp << ": the batch of this call, at most the constructor's maximum\n";
+      gc << "   void infer_nosync(std::size_t " << bp << ")\n   {\n";
+      gc << "      if (" << bp << " > fMaxBatch) {\n         throw std::runtime_error(\"sofie: dynamic input tensor shape parameter " << fBatchParam
+         << " exceeds the initialized maximum allowed shape.\");\n      }\n";
+      gc << "      if (" << bp << " == 0)\n         return;\n";
+      gc << "      const std::int64_t sofie_batch = static_cast<std::int64_t>(" << bp << ");\n      (void)sofie_batch;";
+   } else
+      gc << "   void infer_nosync()\n   {";
    for (std::size_t i = 0; i < fOperators.size(); ++i)
       gc << fOperators[i]->Generate_GPU_HIP(std::to_string(i));
    gc << "   }\n\n";
 
    // infer with host pointers: the CPU signature of the reference
-   std::string args;
+   std::string args = dyn ? "std::size_t " + bp + (fInputTensorNames.empty() ? "" : ", ") : "";
    for (std::size_t i = 0; i < fInputTensorNames.size(); ++i) {
       const auto &ti = fInputTensorInfos[fInputTensorNames[i]];
       args += ConvertTypeToString(ti.type) + " const* host_" + fInputTensorNames[i] + (i + 1 < fInputTensorNames.size() ? ", " : "");
@@ -833,17 +943,21 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
       retType += ">";
    }
    gc << "   " << retType << " infer(" << args << ")\n   {\n";
+   if (dyn)
+      gc << "      if (" << bp << " > fMaxBatch) {\n         throw std::runtime_error(\"sofie: dynamic input tensor shape parameter " << fBatchParam
+         << " exceeds the initialized maximum allowed shape.\");\n      }\n";
    for (auto &n : fInputTensorNames) {
       const auto &ti = fInputTensorInfos[n];
-      gc << "      detail::Check(sofie_hip_upload(fCtx, tensor_" << n << ", host_" << n << ", " << ConvertShapeToLength(ti.shape) * GetTypeSize(ti.type)
-         << "), \"upload of input " << n << "\");\n";
+      gc << "      detail::Check(sofie_hip_upload(fCtx, tensor_" << n << ", host_" << n << ", " << (IsDynamicTensor(n) ? bp + " * " : "")
+         << ConvertShapeToLength(ti.shape) * GetTypeSize(ti.type) << "), \"upload of input " << n << "\");\n";
    }
-   gc << "      infer_nosync();\n";
+   gc << "      infer_nosync(" << (dyn ? bp : "") << ");\n";
    for (std::size_t i = 0; i < fOutputTensorNames.size(); ++i) {
       const auto &o = fOutputTensorNames[i];
       const std::size_t len = ConvertShapeToLength(GetTensorShape(o));
-      gc << "      std::vector<" << ConvertTypeToString(GetTensorType(o)) << "> out_" << i << "(" << len << ");\n";
-      gc << "      detail::Check(sofie_hip_download(fCtx, out_" << i << ".data(), tensor_" << o << ", " << len * GetTypeSize(GetTensorType(o))
+      const std::string scale = IsDynamicTensor(o) ? bp + " * " : "";
+      gc << "      std::vector<" << ConvertTypeToString(GetTensorType(o)) << "> out_" << i << "(" << scale << len << ");\n";
+      gc << "      detail::Check(sofie_hip_download(fCtx, out_" << i << ".data(), tensor_" << o << ", " << scale << len * GetTypeSize(GetTensorType(o))
          << "), \"download of output " << o << "\");\n";
    }
    gc << "      detail::Check(sofie_hip_sync(fCtx), \"infer\");\n";
@@ -858,12 +972,12 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    gc << "   }\n";
    gc << "}; // end of Session\n\n";
    auto dimsArray = [&](const std::string &what, const std::vector<std::string> &names) {
-      gc << "// " << what << " tensor shapes\n";
+      gc << "// " << what << " tensor shapes" << (dyn ? " (0 stands for the run-time parameter " + fBatchParam + ")" : "") << "\n";
       for (auto &n : names) {
          const auto &s = GetTensorShape(n);
          gc << "constexpr std::array<std::size_t, " << s.size() << "> dim_" << n << "{";
          for (std::size_t i = 0; i < s.size(); ++i)
-            gc << s[i] << (i + 1 < s.size() ? ", " : "");
+            gc << (i == 0 && IsDynamicTensor(n) ? 0 : s[i]) << (i + 1 < s.size() ? ", " : "");
          gc << "};\n";
       }
    };
@@ -875,10 +989,9 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
 
 void RModel::GenerateGPU_HIP(std::underlying_type_t<Options> options, int batchSize, bool verbose)
 {
-   (void)batchSize; // shapes are static in this backend; a model is built for its batch size
    if (fOutputTensorNames.empty())
       throw std::runtime_error("SOFIE: the model has no output tensor");
-   Initialize();
+   Initialize(batchSize);
    PlanMemory();
    GenerateSessionCode(options);
    if (verbose)

@@ -210,6 +210,7 @@ struct ValueInfo {
    std::string name;
    int elem_type = 1;
    std::vector<size_t> shape;
+   std::vector<Dim> dims; // the same with named parameters kept
    bool symbolic = false;
 };
 
@@ -239,13 +240,18 @@ ValueInfo ParseValueInfo(Slice s)
                            Reader rd(d.bytes);
                            Field x;
                            bool value = false;
+                           std::string param;
                            while (rd.Next(x))
                               if (x.no == 1) {
                                  v.shape.push_back((size_t)x.v);
+                                 v.dims.push_back(Dim((size_t)x.v));
                                  value = true;
+                              } else if (x.no == 2) {
+                                 param = Str(x.bytes);
                               }
                            if (!value) {
                               v.shape.push_back(0);
+                              v.dims.push_back(Dim(param.empty() ? std::string("batch") : param, 1));
                               v.symbolic = true;
                            }
                         }
@@ -325,9 +331,10 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
    for (auto &v : inputs) {
       if (isInit.count(v.name))
          continue;
-      if (v.symbolic)
-         throw std::runtime_error("SOFIE ONNX parser: input " + v.name + " has a symbolic dimension; this backend emits static shapes");
-      model->AddInputTensorInfo(v.name, static_cast<ETensorType>(v.elem_type), v.shape);
+      if (v.symbolic) // a named leading dimension: the batch, fixed at generation (batchSize) or by the Session
+         model->AddInputTensorInfo(v.name, static_cast<ETensorType>(v.elem_type), v.dims);
+      else
+         model->AddInputTensorInfo(v.name, static_cast<ETensorType>(v.elem_type), v.shape);
       model->AddInputTensorName(v.name);
    }
    std::map<std::string, int> uses;

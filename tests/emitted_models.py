@@ -159,6 +159,39 @@ def conv_integer_dequantize(batch=2):
                 feeds=[X], consts=dict(W=W, sx=sx, sacc=sacc))
 
 
+def with_named_batch(spec, param="N"):
+    """The same graph with the leading dimension of every input and output left as a named parameter."""
+    spec = dict(spec)
+    spec["inputs"] = [(n, dt, [param] + list(sh[1:])) for n, dt, sh in spec["inputs"]]
+    spec["outputs"] = [(n, dt, [param] + list(sh[1:])) for n, dt, sh in spec["outputs"]]
+    return spec
+
+
+def dynamic_linear():
+    """Gemm + Relu with the batch as a run-time parameter: the weights of the reference's own test
+    (tests/alpaka/TestAlpakaLinear.cxx:121-159)."""
+    W = np.array([[0.5, -1.0, 0.25], [0.75, 0.5, -0.5], [-0.25, 1.0, 0.75], [1.5, -0.75, 0.5]], np.float32)
+    B = np.array([0.5, -0.5, 0.25], np.float32)
+    nodes = [ow.node("Gemm", ["X", "W", "B"], ["G"]), ow.node("Relu", ["G"], ["Y"])]
+    return dict(nodes=nodes, inputs=[("X", np.float32, ["N", 4])], outputs=[("Y", np.float32, ["N", 3])], init={"W": W, "B": B},
+                consts=dict(W=W, B=B))
+
+
+def dynamic_matmul_batched():
+    """A[N,4,8] x B[N,8,6], both operands carrying the run-time batch (tests/alpaka/TestAlpakaLinear.cxx:161-210)."""
+    nodes = [ow.node("MatMul", ["A", "B"], ["Y"])]
+    return dict(nodes=nodes, inputs=[("A", np.float32, ["N", 4, 8]), ("B", np.float32, ["N", 8, 6])],
+                outputs=[("Y", np.float32, ["N", 4, 6])], init={})
+
+
+DYNAMIC_MODELS = {
+    "DynamicLinear": dynamic_linear,
+    "DynamicMatMulBatched": dynamic_matmul_batched,
+    "Dynamic_int8_MLP": lambda: with_named_batch(int8_mlp([64, 128, 96, 32], 48), "batch_size"),
+    "Dynamic_int8_CNN": lambda: with_named_batch(int8_cnn(2, 12), "N"),
+    "Dynamic_ConvBatchNormRelu": lambda: with_named_batch(conv_batchnorm_relu(2), "bs"),
+}
+
 CONFIG_MODELS = {
     "QLinearMatMulRelu": lambda: qlinear_matmul_relu(),
     "ConvIntegerDequantize": lambda: conv_integer_dequantize(),
@@ -204,6 +237,45 @@ extern "C" unsigned long pool_bytes() { return SOFIE_%(model)s::Session::kInterm
 '''
 
 
+# Sessions with a run-time batch: kept open across calls so that a test can change the batch between inferences.
+DYNAMIC_HARNESS = r'''
+#include "%(model)s_GPU_HIP.hxx"
+#include <cstring>
+using Session = SOFIE_%(model)s::Session;
+static int fail(char *err, int errlen, const char *what)
+{
+   std::strncpy(err, what, errlen - 1);
+   err[errlen - 1] = 0;
+   return 1;
+}
+extern "C" void *dyn_open(const char *weights, unsigned long max_batch, char *err, int errlen)
+{
+   try {
+      return new Session(weights, max_batch);
+   } catch (const std::exception &e) {
+      fail(err, errlen, e.what());
+      return nullptr;
+   }
+}
+extern "C" void dyn_close(void *s) { delete static_cast<Session *>(s); }
+extern "C" long dyn_infer(void *s, unsigned long batch, const float *const *inputs, float *output, unsigned long capacity, char *err, int errlen)
+{
+   try {
+      auto y = static_cast<Session *>(s)->infer(batch, %(args)s);
+      if (y.size() > capacity)
+         throw std::runtime_error("output has " + std::to_string(y.size()) + " elements");
+      std::memcpy(output, y.data(), y.size() * sizeof(float));
+      return (long)y.size();
+   } catch (const std::exception &e) {
+      fail(err, errlen, e.what());
+      return -1;
+   }
+}
+extern "C" unsigned long arena_bytes(unsigned long max_batch) { return Session::ArenaBytes(max_batch); }
+extern "C" unsigned long pool_bytes(void *s) { return static_cast<Session *>(s)->GetIntermediateMemoryPoolSize(); }
+'''
+
+
 def _run(cmd):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
@@ -223,6 +295,14 @@ def compile_harness(model, n_inputs):
     src = os.path.join(OUT, model + "_harness.cxx")
     with open(src, "w") as f:
         f.write(HARNESS % dict(model=model, args=", ".join("inputs[%d]" % i for i in range(n_inputs))))
+    return compile_shared(src, os.path.join(OUT, "lib%s.so" % model))
+
+
+def emit_and_compile_dynamic(model, onnx_path, n_inputs):
+    _run([EMIT, onnx_path, OUT])
+    src = os.path.join(OUT, model + "_harness.cxx")
+    with open(src, "w") as f:
+        f.write(DYNAMIC_HARNESS % dict(model=model, args=", ".join("inputs[%d]" % i for i in range(n_inputs))))
     return compile_shared(src, os.path.join(OUT, "lib%s.so" % model))
 
 
@@ -248,8 +328,16 @@ def build_all(jobs=8):
         work.append((m, p, len(spec["inputs"])))
     # the same model with its weights in a safetensors file
     work.append(("Linear_16_st", os.path.join(GOLDEN, "models", "Linear_16.onnx"), 1, "--safetensors", "--name", "Linear_16_st"))
+    dynamic = []
+    for m, make in DYNAMIC_MODELS.items():
+        spec = make()
+        p = os.path.join(OUT, m + ".onnx")
+        ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)
+        dynamic.append((m, p, len(spec["inputs"])))
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(lambda w: emit_and_compile(*w), work))
+        list(ex.map(lambda w: emit_and_compile_dynamic(*w), dynamic))
+    work += dynamic
     # models built through the RModel API (no ONNX file): sofie_hip_emit_example writes their headers
     _run([os.path.join(os.path.dirname(EMIT), "sofie_hip_emit_example"), OUT])
     for m in API_MODELS:

@@ -60,7 +60,8 @@ def node(op, inputs, outputs, **attrs):
 
 
 def value_info(name, elem_type, shape):
-    dims = b"".join(_ld(1, _vi(1, d)) for d in shape)
+    # an int is a dim_value, a str a dim_param (a named, run-time dimension)
+    dims = b"".join(_ld(1, _ld(2, d.encode()) if isinstance(d, str) else _vi(1, d)) for d in shape)
     ttype = _vi(1, elem_type) + _ld(2, dims)
     return _ld(1, name.encode()) + _ld(2, _ld(1, ttype))
 

@@ -188,6 +188,66 @@ def test_qlinear_matmul_and_conv_integer_become_one_launch_each(emitted):
     assert "sofie_hip_dequantize_linear_i32(" in body and "sofie_hip_unary_f32" not in body
 
 
+def test_run_time_batch_signatures_follow_the_reference_convention(emitted):
+    txt = read(emitted, "DynamicLinear")
+    # the constructor takes the maximum after the weight file, infer takes the value first (core/src/RModel.cxx:1537-1547, 1375-1395)
+    assert re.search(r'Session\(std::string filename = "DynamicLinear_GPU_HIP.dat", std::size_t N = 1, int device = 0\)', txt)
+    assert re.search(r"std::vector<float> infer\(std::size_t N, float const ?\* ?host_X\)", txt)
+    assert "void infer_nosync(std::size_t N)" in txt
+    assert "sofie: dynamic input tensor shape parameter N exceeds the initialized maximum allowed shape." in txt
+    assert "d.M = static_cast<std::int32_t>(sofie_batch * 1); d.N = 3; d.K = 4;" in txt
+    assert "sofie_hip_upload(fCtx, tensor_X, host_X, N * 16)" in txt and "out_0(N * 3)" in txt
+    assert "kArenaBytes" not in txt and "ArenaBytes(fMaxBatch)" in txt
+    # the int8 chain: every row count scales, the re-laid-out weights do not
+    txt = read(emitted, "Dynamic_int8_MLP")
+    assert txt.count("d.M = static_cast<std::int32_t>(sofie_batch * 1)") == 3
+    assert "std::size_t batch_size = 1" in txt
+
+
+def test_a_batch_given_at_generation_makes_a_static_session(emitted, tmp_path):
+    r = subprocess.run([em.EMIT, os.path.join(emitted, "DynamicLinear.onnx"), str(tmp_path), "--batch", "4"], stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
+    txt = open(os.path.join(str(tmp_path), "DynamicLinear_GPU_HIP.hxx")).read()
+    assert "sofie_batch" not in txt and "kArenaBytes" in txt and "d.M = 4; d.N = 3; d.K = 4;" in txt
+    assert re.search(r"std::vector<float> infer\(float const ?\* ?host_X\)", txt)
+    assert "dim_X{4, 4}" in txt
+
+
+def test_per_batch_entry_plan_scales_without_overlap(emitted, tmp_path):
+    out = subprocess.run([em.EMIT, os.path.join(emitted, "Dynamic_int8_CNN.onnx"), str(tmp_path), "--plan"], check=True,
+                         stdout=subprocess.PIPE, text=True).stdout.split("\n")
+    head = out[1].split()
+    assert head[0] == "static" and head[2] == "per_batch_entry" and head[5] == "N"
+    static_bytes, entry_bytes = int(head[1]), int(head[3])
+    rows = [l.split() for l in out[2:] if len(l.split()) == 7]
+    per = [dict(name=f[0], offset=int(f[1]), bytes=int(f[2]), first=int(f[3]), last=int(f[4]), pooled=int(f[5])) for f in rows if f[6] == "per_batch_entry"]
+    fixed = [dict(name=f[0], offset=int(f[1]), bytes=int(f[2])) for f in rows if f[6] == "static"]
+    assert static_bytes % 256 == 0 and all(r["offset"] % 256 == 0 and r["offset"] + r["bytes"] <= static_bytes for r in fixed)
+    names = {r["name"] for r in per}
+    assert {"tensor_X", "tensor_Y", "tensor_Q", "tensor_R0", "workspace_op_1"} <= names and not any(n.startswith("packed_") for n in names)
+    # per-entry offsets are multiples of 16, so that capacity (a multiple of 16) times the offset is a multiple of 256
+    assert all(r["offset"] % 16 == 0 and r["offset"] + r["bytes"] <= entry_bytes for r in per)
+    for i, a in enumerate(per):
+        for b in per[i + 1:]:
+            if a["offset"] < b["offset"] + b["bytes"] and b["offset"] < a["offset"] + a["bytes"]:
+                assert a["pooled"] and b["pooled"] and (a["last"] <= b["first"] or b["last"] <= a["first"]), (a, b)
+
+
+def test_parameter_outside_the_leading_dimension_is_refused(tmp_path):
+    nodes = [ow.node("Relu", ["X"], ["Y"])]
+    r = _emit(tmp_path, nodes, [("X", np.float32, [4, "K"])], [("Y", np.float32, [4, "K"])], {})
+    assert r.returncode != 0 and "only the leading (batch) dimension may be a parameter" in r.stdout
+    # two different parameters cannot both be the batch
+    nodes = [ow.node("Add", ["A", "B"], ["Y"])]
+    r = _emit(tmp_path, nodes, [("A", np.float32, ["N", 4]), ("B", np.float32, ["M", 4])], [("Y", np.float32, ["N", 4])], {})
+    assert r.returncode != 0 and "two shape parameters" in r.stdout
+    # a transposed batched operand has no row dimension to grow
+    nodes = [ow.node("Gemm", ["X", "W"], ["Y"], transA=1)]
+    r = _emit(tmp_path, nodes, [("X", np.float32, ["N", 4])], [("Y", np.float32, [4, 3])], {"W": np.ones((1, 3), np.float32)})
+    assert r.returncode != 0 and "run-time batch" in r.stdout
+
+
 def test_asymmetric_zero_point_is_refused(tmp_path):
     init = {"W": np.ones((4, 3, 1, 1), dtype=np.int8), "s": np.array(0.5, dtype=np.float32), "z": np.zeros((), dtype=np.int8),
             "z1": np.array(3, dtype=np.int8), "sx": np.array(0.1, dtype=np.float32)}

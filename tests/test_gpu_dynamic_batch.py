@@ -1,0 +1,141 @@
+"""Sessions whose batch is a run-time parameter: the constructor takes the maximum, every infer call the batch
+(the reference's convention, core/src/RModel.cxx:1375-1395, 1537-1547; its tests: tests/alpaka/TestAlpakaLinear.cxx:121-210).
+One Session serves several batch sizes; each result is compared with the CPU oracle on the same rows."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+from tests import emitted_models as em
+from tests import graph_runner as gr
+from tests import onnx_lite
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+class DynamicSession:
+    def __init__(self, model, max_batch):
+        path = os.path.join(em.OUT, "lib%s.so" % model)
+        assert os.path.exists(path), "emitted models are built by __graft_entry__.build()"
+        self.lib = ctypes.CDLL(path)
+        self.lib.dyn_open.restype = ctypes.c_void_p
+        self.lib.dyn_open.argtypes = [ctypes.c_char_p, ctypes.c_ulong, ctypes.c_char_p, ctypes.c_int]
+        self.lib.dyn_close.argtypes = [ctypes.c_void_p]
+        self.lib.dyn_infer.restype = ctypes.c_long
+        self.lib.dyn_infer.argtypes = [ctypes.c_void_p, ctypes.c_ulong, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_ulong, ctypes.c_char_p, ctypes.c_int]
+        self.lib.arena_bytes.restype = ctypes.c_ulong
+        self.lib.arena_bytes.argtypes = [ctypes.c_ulong]
+        self.lib.pool_bytes.restype = ctypes.c_ulong
+        self.lib.pool_bytes.argtypes = [ctypes.c_void_p]
+        self.err = ctypes.create_string_buffer(1024)
+        print("dynamic session", model, "max batch", max_batch, flush=True)
+        self.h = self.lib.dyn_open(os.path.join(em.OUT, model + "_GPU_HIP.dat").encode(), max_batch, self.err, 1024)
+        assert self.h, self.err.value.decode()
+
+    def infer(self, batch, inputs, capacity):
+        arrs = [np.ascontiguousarray(a, dtype=np.float32) for a in inputs]
+        ptrs = (ctypes.c_void_p * len(arrs))(*[a.ctypes.data for a in arrs])
+        y = np.zeros(capacity, dtype=np.float32)
+        n = self.lib.dyn_infer(self.h, batch, ptrs, y.ctypes.data_as(ctypes.c_void_p), capacity, self.err, 1024)
+        if n < 0:
+            raise RuntimeError(self.err.value.decode())
+        return y[:n]
+
+    def close(self):
+        if self.h:
+            self.lib.dyn_close(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+
+def test_dynamic_linear_as_the_reference_tests_it(rt):
+    c = em.dynamic_linear()["consts"]
+    for n in (1, 8):
+        x = ((np.arange(n * 4) % 7).astype(np.float32) - 3.0).reshape(n, 4)
+        want = np.maximum(x.astype(np.float64) @ c["W"].astype(np.float64) + c["B"], 0)
+        with DynamicSession("DynamicLinear", n) as s:
+            got = s.infer(n, [x], n * 3)
+        assert got.size == n * 3 and np.abs(got.reshape(n, 3) - want).max() <= 1e-5
+
+
+def test_dynamic_matmul_with_both_operands_batched(rt):
+    M, K, Nc = 4, 8, 6
+    for n in (1, 5):
+        a = (((np.arange(n * M * K) % 11).astype(np.float32) - 5.0) * np.float32(0.3)).reshape(n, M, K)
+        b = (((np.arange(n * K * Nc) % 7).astype(np.float32) - 3.0) * np.float32(0.5)).reshape(n, K, Nc)
+        want = np.matmul(a.astype(np.float64), b.astype(np.float64))
+        with DynamicSession("DynamicMatMulBatched", n) as s:
+            got = s.infer(n, [a, b], n * M * Nc)
+        assert np.abs(got.reshape(n, M, Nc) - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
+
+
+def test_one_session_serves_several_batches_and_refuses_more_than_its_maximum(rt):
+    c = em.dynamic_linear()["consts"]
+    x = util.normal(8101, 8 * 4).reshape(8, 4)
+    want = np.maximum(x @ c["W"] + c["B"], 0).astype(np.float32)
+    with DynamicSession("DynamicLinear", 8) as s:
+        first = s.infer(8, [x], 24).copy()
+        assert np.abs(first.reshape(8, 3) - want).max() <= 1e-5
+        small = s.infer(3, [x[:3]], 24)
+        assert small.size == 9 and np.array_equal(small, first[:9])
+        assert s.infer(0, [x], 24).size == 0
+        again = s.infer(8, [x], 24)
+        assert np.array_equal(again, first)
+        with pytest.raises(RuntimeError, match="dynamic input tensor shape parameter N exceeds the initialized maximum allowed shape"):
+            s.infer(9, [np.zeros((9, 4), np.float32)], 27)
+        # the arena grows in steps of 16 batch entries and linearly beyond
+        a = [s.lib.arena_bytes(n) for n in (1, 16, 17, 32, 48)]
+        assert a[0] == a[1] < a[2] == a[3] < a[4] and a[4] - a[3] == a[3] - a[1]
+
+
+def test_dynamic_int8_mlp_is_bit_exact_for_every_batch(rt):
+    from oracle import binding as ob
+    spec = em.int8_mlp([64, 128, 96, 32], 48)
+    c, x = spec["consts"], spec["feeds"][0]
+    with DynamicSession("Dynamic_int8_MLP", 48) as s:
+        for n in (48, 1, 17, 48):
+            h = x[:n]
+            for l, w in enumerate(c["weights"]):
+                q = ob.quantize_linear(h, c["in_scales"][l])
+                acc = np.maximum(ob.matmul_integer(q, w, M=n, N=w.shape[1], K=w.shape[0], omp=True), 0)
+                h = ob.dequantize_linear(acc, np.float32(c["in_scales"][l] * c["w_scales"][l]))
+            print("Dynamic_int8_MLP batch", n, flush=True)
+            got = s.infer(n, [x[:n]], 48 * 32)
+            assert got.size == h.size and np.array_equal(got.view(np.uint32), h.ravel().view(np.uint32))
+            assert np.abs(h).max() > 0
+
+
+def test_dynamic_int8_cnn_matches_cpu_chain_for_every_batch(rt):
+    from tests.refmodels import int8_cnn_oracle
+    spec = em.int8_cnn(2, 12)
+    x = np.concatenate([spec["feeds"][0], util.normal(8201, 3 * 3 * 12 * 12).reshape(3, 3, 12, 12)])
+    with DynamicSession("Dynamic_int8_CNN", 5) as s:
+        assert s.lib.pool_bytes(s.h) > 0
+        for n in (5, 2, 1, 5):
+            want = int8_cnn_oracle(spec["consts"], x[:n]).ravel()
+            print("Dynamic_int8_CNN batch", n, flush=True)
+            got = s.infer(n, [x[:n]], 50)
+            assert got.size == want.size == n * 10
+            assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+            assert np.abs(want).max() > 1e-3
+
+
+def test_dynamic_conv_batchnorm_relu(rt):
+    spec = em.conv_batchnorm_relu(2)
+    g = onnx_lite.load(os.path.join(em.OUT, "ConvBatchNormRelu.onnx"))     # the same weights with a fixed batch of 2
+    x2 = spec["feeds"][0]
+    x = np.concatenate([x2, util.normal(8301, x2[:1].size).reshape(x2[:1].shape)])
+    want = gr.run(g, [x], gr.OracleBackend())
+    with DynamicSession("Dynamic_ConvBatchNormRelu", 3) as s:
+        for n in (3, 1):
+            print("Dynamic_ConvBatchNormRelu batch", n, flush=True)
+            got = s.infer(n, [x[:n]], want.size)
+            w = want[:n].ravel()
+            assert got.size == w.size and np.abs(got - w).max() <= 1e-5 * max(1.0, float(np.abs(w).max()))
