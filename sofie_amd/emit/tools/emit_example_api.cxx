@@ -46,6 +46,23 @@ int main(int argc, char **argv)
             cm.GenerateGPU_HIP(Options::kCustomMemory);
          cm.OutputGenerated(std::string(argv[1]) + "/" + cm.GetName() + "_GPU_HIP.hxx");
       }
+      // the same chain with every Session option at once: the batch a run-time parameter (default 2), caller-owned memory,
+      // caller-owned stream, weights in a safetensors file
+      {
+         RModel all("CustomMemoryDynamicChain");
+         all.AddInputTensorInfo("X", ETensorType::FLOAT, std::vector<Dim>{Dim(std::string("N"), 2), Dim(5)});
+         all.AddInputTensorName("X");
+         std::vector<float> W(5 * 4, 0.5f), B(4, 1.0f);
+         all.AddInitializedTensor("W", ETensorType::FLOAT, {5, 4}, W.data());
+         all.AddInitializedTensor("B", ETensorType::FLOAT, {4}, B.data());
+         all.AddOperator(std::make_unique<ROperator_Gemm<float>>(1.0f, 1.0f, 0, 0, "X", "W", "B", "H1"));
+         all.AddOperator(std::make_unique<ROperator_Relu<float>>("H1", "H2"));
+         all.AddOperator(std::make_unique<ROperator_Sigmoid<float>>("H2", "H3"));
+         all.AddOperator(std::make_unique<ROperator_Tanh<float>>("H3", "Y"));
+         all.AddOutputTensorNameList({"Y"});
+         all.GenerateGPU_HIP((Options::kCustomMemory | Options::kExternalStream) | static_cast<std::underlying_type_t<Options>>(Options::kSafetensorsWeightFile));
+         all.OutputGenerated(std::string(argv[1]) + "/" + all.GetName() + "_GPU_HIP.hxx");
+      }
       // FP8 Gemm with bias and GELU: X[48,256] fp32, W e4m3 [96,256] (K contiguous), codes from a linear congruential
       // sequence so that a test can rebuild them, bias[n] = 0.25 (n mod 7 - 3)
       RModel f8("ApiFp8Gemm");

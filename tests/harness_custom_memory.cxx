@@ -4,6 +4,7 @@
 // The device block comes from a second runtime context's arena, so this file needs no HIP header.
 #include "CustomMemoryChain_GPU_HIP.hxx"
 #include "CustomMemoryStreamChain_GPU_HIP.hxx"
+#include "CustomMemoryDynamicChain_GPU_HIP.hxx"
 
 #include <cmath>
 #include <cstdio>
@@ -116,6 +117,41 @@ extern "C" int run_custom_memory(const char *dir, char *report, int len)
             expect(ChainOk(s.infer(ones.data())), "chain result on the caller's stream");
          }
          expect(st.allocations == 1 && st.deallocations == 1, "external stream and custom memory: one block, returned");
+      }
+      {
+         // run-time batch + caller's memory + caller's stream + safetensors weights in one Session
+         using namespace SOFIE_CustomMemoryDynamicChain;
+         const std::string w3 = std::string(dir) + "/CustomMemoryDynamicChain_GPU_HIP.safetensors";
+         const float want = std::tanh(1.f / (1.f + std::exp(-3.5f)));
+         auto rowsOk = [&](const std::vector<float> &y, std::size_t rows) {
+            bool ok = y.size() == rows * 4;
+            for (float v : y)
+               ok = ok && std::fabs(v - want) <= 1e-5f;
+            return ok;
+         };
+         State st;
+         {
+            Session s(MakeProvider<MemoryProvider>(st, memory, true), w3, 7, sofie_hip_stream(helper));
+            expect(st.allocations == 1 && st.blockBytes == Session::ArenaBytes(7) && st.blockBytes == Session::ArenaBytes(16) &&
+                      Session::ArenaBytes(17) > st.blockBytes,
+                   "run-time batch: the block is the static part plus 16 batch entries");
+            bool aligned = !st.offsets.empty();
+            for (std::size_t o : st.offsets)
+               aligned = aligned && o % 256 == 0 && o < st.blockBytes;
+            expect(aligned, "run-time batch: every tensor assigned at a 256-byte offset inside the block");
+            std::vector<float> x(7 * 5, 1.f);
+            expect(rowsOk(s.infer(7, x.data()), 7), "run-time batch: 7 rows");
+            expect(rowsOk(s.infer(2, x.data()), 2), "run-time batch: 2 rows on the same session");
+            bool threw = false;
+            try {
+               s.infer(8, x.data());
+            } catch (const std::runtime_error &) {
+               threw = true;
+            }
+            expect(threw, "run-time batch: more than the maximum is refused");
+            expect(s.stream() == sofie_hip_stream(helper) && s.GetMaxBatch() == 7, "run-time batch: caller's stream, maximum kept");
+         }
+         expect(st.deallocations == 1, "run-time batch: block returned once");
       }
    } catch (const std::exception &e) {
       out << "FAIL exception: " << e.what() << "\n";
