@@ -722,7 +722,7 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    gc << "//Code generated automatically by SOFIE (gfx950 HIP backend)\n";
    gc << "#ifndef " << guard << "_GPU_HIP\n#define " << guard << "_GPU_HIP\n\n";
    gc << "#include <array>\n#include <cstddef>\n#include <cstdint>\n#include <cstdlib>\n#include <fstream>\n#include <stdexcept>\n#include <string>\n"
-         "#include <tuple>\n#include <type_traits>\n#include <vector>\n#include \"sofie_hip.h\"\n";
+         "#include <tuple>\n#include <type_traits>\n#include <vector>\n#if __cplusplus >= 202002L\n#include <span>\n#endif\n#include \"sofie_hip.h\"\n";
    if (customMemory)
       gc << "#include <functional>\n";
    if (safetensors)
@@ -738,6 +738,9 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
       gc << "struct MemoryProvider {\n   std::function<void *(std::size_t)> alloc;\n   std::function<void *(std::size_t)> assign;\n"
             "   std::function<void(void *)> dealloc;\n};\n\n";
    }
+   // views of device memory owned by the caller (the reference's ViewF1D / ViewConstF1D, README.md:283-297)
+   gc << "template <class T>\nstruct DeviceView {\n   T *data = nullptr;\n   std::size_t size = 0; // elements\n};\n"
+         "using ViewF1D = DeviceView<float>;\nusing ViewConstF1D = DeviceView<float const>;\n\n";
    gc << "struct Session {\n";
    gc << "   // one arena: weights, operator-owned buffers, inputs, outputs, then the pool of intermediates\n";
    const bool dyn = HasDynamicBatch();
@@ -905,21 +908,108 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
       gc << "   " << ConvertTypeToString(GetTensorType(n)) << " const *device_output_" << n << "() const { return tensor_" << n << "; }\n";
    gc << "   void *stream() const { return sofie_hip_stream(fCtx); }\n\n";
 
-   // infer_nosync: the operators, inputs and outputs resident in the arena
+   // doInfer: the operators.  The graph inputs and outputs are parameters named like the members they shadow, so that the
+   // same statements run on the arena's regions (infer_nosync) or on memory of the caller (the overload that takes views).
+   std::vector<std::string> boundOutputs; // graph outputs an operator writes (an output that is an input or a weight is not)
+   for (auto &o : fOutputTensorNames)
+      if (fIntermediateTensorInfos.count(o) && std::find(boundOutputs.begin(), boundOutputs.end(), o) == boundOutputs.end())
+         boundOutputs.push_back(o);
+   gc << "   // the operators of the model; the graph inputs and outputs are passed in (these parameters shadow the members)\n";
+   gc << "   void doInfer(" << (dyn ? "std::int64_t sofie_batch" : "");
+   {
+      bool first = !dyn;
+      for (auto &n : fInputTensorNames) {
+         gc << (first ? "" : ", ") << ConvertTypeToString(fInputTensorInfos[n].type) << " const *tensor_" << n;
+         first = false;
+      }
+      for (auto &o : boundOutputs) {
+         gc << (first ? "" : ", ") << ConvertTypeToString(GetTensorType(o)) << " *tensor_" << o;
+         first = false;
+      }
+   }
+   gc << ")\n   {";
+   if (dyn)
+      gc << "\n      (void)sofie_batch;";
+   for (std::size_t i = 0; i < fOperators.size(); ++i)
+      gc << fOperators[i]->Generate_GPU_HIP(std::to_string(i));
+   gc << "   }\n\n";
+   auto boundArgs = [&](const std::string &inPrefix, const std::string &outPrefix) {
+      std::string a = dyn ? "static_cast<std::int64_t>(" + bp + ")" : "";
+      for (auto &n : fInputTensorNames)
+         a += std::string(a.empty() ? "" : ", ") + inPrefix + n;
+      for (auto &o : boundOutputs)
+         a += std::string(a.empty() ? "" : ", ") + outPrefix + o;
+      return a;
+   };
+   const std::string batchCheck = !dyn ? std::string()
+                                       : "      if (" + bp + " > fMaxBatch) {\n         throw std::runtime_error(\"sofie: dynamic input tensor shape parameter " +
+                                            fBatchParam + " exceeds the initialized maximum allowed shape.\");\n      }\n";
+   // infer_nosync: inputs and outputs resident in the arena
    gc << "   // enqueues one inference on the session's stream: inputs are read from the tensor_<input> regions of the arena,\n";
    gc << "   // results land in the tensor_<output> regions (overwritten by the next call)\n";
    if (dyn) {
       gc << "   // " << bp << ": the batch of this call, at most the constructor's maximum\n";
-      gc << "   void infer_nosync(std::size_t " << bp << ")\n   {\n";
-      gc << "      if (" << bp << " > fMaxBatch) {\n         throw std::runtime_error(\"sofie: dynamic input tensor shape parameter " << fBatchParam
-         << " exceeds the initialized maximum allowed shape.\");\n      }\n";
+      gc << "   void infer_nosync(std::size_t " << bp << ")\n   {\n" << batchCheck;
       gc << "      if (" << bp << " == 0)\n         return;\n";
-      gc << "      const std::int64_t sofie_batch = static_cast<std::int64_t>(" << bp << ");\n      (void)sofie_batch;";
    } else
-      gc << "   void infer_nosync()\n   {";
-   for (std::size_t i = 0; i < fOperators.size(); ++i)
-      gc << fOperators[i]->Generate_GPU_HIP(std::to_string(i));
-   gc << "   }\n\n";
+      gc << "   void infer_nosync()\n   {\n";
+   gc << "      doInfer(" << boundArgs("tensor_", "tensor_") << ");\n   }\n\n";
+
+   // infer on views of device memory: the third signature of the reference's GPU sessions
+   // (infer(std::span<ViewConstF1D const> inputs, std::span<ViewF1D> outputs, params...))
+   bool allFloat = true;
+   for (auto &n : fInputTensorNames)
+      allFloat = allFloat && fInputTensorInfos[n].type == ETensorType::FLOAT;
+   for (auto &o : fOutputTensorNames)
+      allFloat = allFloat && GetTensorType(o) == ETensorType::FLOAT;
+   if (allFloat) {
+      gc << "#if __cplusplus >= 202002L\n";
+      gc << "   // Runs the model on device memory of the caller and waits.  inputs[i] / outputs[i] follow the order of the model's\n";
+      gc << "   // inputs / outputs.  Views that start on a 256-byte boundary are read and written in place (no copy); any other\n";
+      gc << "   // view goes through the session's own region with one device-to-device copy.\n";
+      gc << "   void infer(std::span<ViewConstF1D const> inputs, std::span<ViewF1D> outputs" << (dyn ? ", std::size_t " + bp : "") << ")\n   {\n";
+      gc << batchCheck;
+      gc << "      if (inputs.size() != " << fInputTensorNames.size() << " || outputs.size() != " << fOutputTensorNames.size()
+         << ")\n         throw std::runtime_error(\"SOFIE HIP Session: infer takes " << fInputTensorNames.size() << " input and "
+         << fOutputTensorNames.size() << " output views\");\n";
+      auto lenOf = [&](const std::string &n) {
+         return (IsDynamicTensor(n) ? bp + " * " : std::string()) + std::to_string(ConvertShapeToLength(GetTensorShape(n)));
+      };
+      for (std::size_t i = 0; i < fInputTensorNames.size(); ++i)
+         gc << "      if (inputs[" << i << "].size < " << lenOf(fInputTensorNames[i]) << " || !inputs[" << i << "].data)\n"
+            << "         throw std::runtime_error(\"SOFIE HIP Session: the view of input " << fInputTensorNames[i] << " is too small\");\n";
+      for (std::size_t i = 0; i < fOutputTensorNames.size(); ++i)
+         gc << "      if (outputs[" << i << "].size < " << lenOf(fOutputTensorNames[i]) << " || !outputs[" << i << "].data)\n"
+            << "         throw std::runtime_error(\"SOFIE HIP Session: the view of output " << fOutputTensorNames[i] << " is too small\");\n";
+      if (dyn)
+         gc << "      if (" << bp << " == 0)\n         return;\n";
+      gc << "      auto inPlace = [](const void *p) { return (reinterpret_cast<std::uintptr_t>(p) & 255) == 0; };\n";
+      for (std::size_t i = 0; i < fInputTensorNames.size(); ++i) {
+         const auto &n = fInputTensorNames[i];
+         gc << "      float const *in_" << n << " = inputs[" << i << "].data;\n";
+         gc << "      if (!inPlace(in_" << n << ")) {\n         detail::Check(sofie_hip_copy(fCtx, tensor_" << n << ", in_" << n << ", (" << lenOf(n)
+            << ") * sizeof(float)), \"copy of input " << n << "\");\n         in_" << n << " = tensor_" << n << ";\n      }\n";
+      }
+      for (std::size_t i = 0; i < fOutputTensorNames.size(); ++i) {
+         const auto &o = fOutputTensorNames[i];
+         if (std::find(boundOutputs.begin(), boundOutputs.end(), o) == boundOutputs.end())
+            continue;
+         // the first view of an output is the one the operators write
+         bool firstUse = std::find(fOutputTensorNames.begin(), fOutputTensorNames.begin() + i, o) == fOutputTensorNames.begin() + i;
+         if (firstUse)
+            gc << "      float *out_" << o << " = inPlace(outputs[" << i << "].data) ? outputs[" << i << "].data : tensor_" << o << ";\n";
+      }
+      gc << "      doInfer(" << boundArgs("in_", "out_") << ");\n";
+      for (std::size_t i = 0; i < fOutputTensorNames.size(); ++i) {
+         const auto &o = fOutputTensorNames[i];
+         const bool bound = std::find(boundOutputs.begin(), boundOutputs.end(), o) != boundOutputs.end();
+         const std::string src = bound ? "out_" + o : "tensor_" + o;
+         gc << "      if (outputs[" << i << "].data != " << src << ")\n         detail::Check(sofie_hip_copy(fCtx, outputs[" << i << "].data, " << src
+            << ", (" << lenOf(o) << ") * sizeof(float)), \"copy of output " << o << "\");\n";
+      }
+      gc << "      detail::Check(sofie_hip_sync(fCtx), \"infer\");\n   }\n";
+      gc << "#endif\n\n";
+   }
 
    // infer with host pointers: the CPU signature of the reference
    std::string args = dyn ? "std::size_t " + bp + (fInputTensorNames.empty() ? "" : ", ") : "";

@@ -232,6 +232,58 @@ extern "C" int run_model(const char *weights, const float *const *inputs, float 
       return 1;
    }
 }
+// The same inference on device memory of the caller, through infer(std::span<ViewConstF1D const>, std::span<ViewF1D>).
+// The caller's memory is the arena of a second context; `misalign` (in floats) moves every view off the 256-byte boundary,
+// which makes the Session copy through its own regions instead of working in place.
+extern "C" int run_model_views(const char *weights, const float *const *inputs, const unsigned long *input_lens, int n_inputs, float *output,
+                               unsigned long output_len, int misalign, char *err, int errlen)
+{
+   sofie_hip_ctx *helper = nullptr;
+   int rc = 0;
+   try {
+      using namespace SOFIE_%(model)s;
+      std::size_t total = 4096;
+      for (int i = 0; i < n_inputs; ++i)
+         total += (input_lens[i] * sizeof(float) + 511) / 256 * 256;
+      total += (output_len * sizeof(float) + 511) / 256 * 256;
+      if (sofie_hip_ctx_create(&helper, 0, nullptr) || sofie_hip_arena_create(helper, total, 256))
+         throw std::runtime_error(sofie_hip_last_error());
+      char *base = static_cast<char *>(sofie_hip_arena_ptr(helper, 0));
+      std::size_t off = 0;
+      std::vector<ViewConstF1D> in;
+      for (int i = 0; i < n_inputs; ++i) {
+         float *p = reinterpret_cast<float *>(base + off) + misalign;
+         detail::Check(sofie_hip_upload(helper, p, inputs[i], input_lens[i] * sizeof(float)), "upload");
+         in.push_back(ViewConstF1D{p, input_lens[i]});
+         off += (input_lens[i] * sizeof(float) + 511) / 256 * 256;
+      }
+      float *out = reinterpret_cast<float *>(base + off) + misalign;
+      detail::Check(sofie_hip_fill_zero(helper, out, output_len * sizeof(float)), "clear");
+      detail::Check(sofie_hip_sync(helper), "upload");
+      std::vector<ViewF1D> outs{ViewF1D{out, output_len}};
+      Session s(weights);
+      s.infer(std::span<ViewConstF1D const>(in), std::span<ViewF1D>(outs));
+      detail::Check(sofie_hip_download(helper, output, out, output_len * sizeof(float)), "download");
+      detail::Check(sofie_hip_sync(helper), "download");
+      // a view that is too small is refused before anything runs
+      outs[0].size = output_len - 1;
+      bool threw = false;
+      try {
+         s.infer(std::span<ViewConstF1D const>(in), std::span<ViewF1D>(outs));
+      } catch (const std::runtime_error &) {
+         threw = true;
+      }
+      if (!threw)
+         throw std::runtime_error("a short output view was accepted");
+   } catch (const std::exception &e) {
+      std::strncpy(err, e.what(), errlen - 1);
+      err[errlen - 1] = 0;
+      rc = 1;
+   }
+   if (helper)
+      sofie_hip_ctx_destroy(helper);
+   return rc;
+}
 extern "C" unsigned long arena_bytes() { return SOFIE_%(model)s::Session::kArenaBytes; }
 extern "C" unsigned long pool_bytes() { return SOFIE_%(model)s::Session::kIntermediatePoolBytes; }
 '''

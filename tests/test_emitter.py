@@ -20,6 +20,12 @@ def emitted():
     return em.OUT
 
 
+def ops_body(txt):
+    """The statements of the operators: the body of Session::doInfer."""
+    body = txt[txt.index("void doInfer("):]
+    return body[:body.index("void infer_nosync(")]
+
+
 def plan_of(onnx_path, tmp_path):
     out = subprocess.run([em.EMIT, onnx_path, str(tmp_path), "--plan"], check=True, stdout=subprocess.PIPE, text=True).stdout.split("\n")
     head = out[0].split()
@@ -75,14 +81,14 @@ def test_session_api_of_the_generated_header(emitted):
     assert "void infer_nosync()" in txt
     assert "#include \"sofie_hip.h\"" in txt
     # nothing in the generated code may allocate per inference
-    body = txt[txt.index("void infer_nosync()"):]
+    body = txt[txt.index("void doInfer("):]
     body = body[:body.index("std::vector<float> infer(")]
     assert "arena_create" not in body and "hipMalloc" not in body and "new " not in body
 
 
 def test_gemm_relu_pairs_are_fused(emitted):
     txt = read(emitted, "Linear_16")
-    body = txt[txt.index("void infer_nosync()"):]
+    body = ops_body(txt)
     assert body.count("sofie_hip_gemm_f32") == 10
     assert "sofie_hip_unary_f32" not in body          # every Relu went into a Gemm epilogue
     assert body.count("SOFIE_ACT_RELU") == 9
@@ -92,8 +98,7 @@ def test_gemm_relu_pairs_are_fused(emitted):
 
 def test_quantised_chain_collapses_to_one_kernel_per_layer(emitted):
     txt = read(emitted, "Config2_int8_MLP_mid")
-    body = txt[txt.index("void infer_nosync()"):]
-    body = body[:body.index("infer(")]
+    body = ops_body(txt)
     assert body.count("sofie_hip_gemm_i8(") == 3
     assert body.count("sofie_hip_quantize_linear(") == 1    # only the model input is quantised by its own kernel
     assert "sofie_hip_dequantize_linear" not in body        # the last DequantizeLinear is the GEMM's fp32 store
@@ -160,8 +165,7 @@ def test_weight_file_round_trip(emitted):
 
 def test_quantised_cnn_keeps_channels_last_and_reads_activations_in_place(emitted):
     txt = read(emitted, "Config5_int8_CNN_small")
-    body = txt[txt.index("void infer_nosync()"):]
-    body = body[:body.index("infer(")]
+    body = ops_body(txt)
     assert body.count("sofie_hip_conv_i8(") == 4
     assert "sofie_hip_unary_f32" not in body                      # the four Relu are in the convolutions' stores
     assert body.count("a.relu = 1") == 4
@@ -170,20 +174,18 @@ def test_quantised_cnn_keeps_channels_last_and_reads_activations_in_place(emitte
     assert body.count("a.x_layout = SOFIE_LAYOUT_NCHW") == 1     # the quantised model input
     assert "sofie_hip_dequantize_linear" not in body and "sofie_hip_global_avg_pool_i8(" in body
     # weights are re-laid out once, in the constructor
-    ctor = txt[txt.index("Session(std::string filename"):txt.index("void infer_nosync()")]
+    ctor = txt[txt.index("Session(std::string filename"):txt.index("void doInfer(")]
     assert ctor.count("sofie_hip_pack_conv_weight_i8(") == 4
 
 
 def test_qlinear_matmul_and_conv_integer_become_one_launch_each(emitted):
     txt = read(emitted, "QLinearMatMulRelu")
-    body = txt[txt.index("void infer_nosync()"):]
-    body = body[:body.index("infer(")]
+    body = ops_body(txt)
     # the Relu on the int8 output rides in the GEMM's store; multipliers a_scale*b_scale[n]/y_scale are a weight
     assert body.count("sofie_hip_gemm_i8(") == 1 and "d.relu_out = 1" in body and "sofie_hip_unary_f32" not in body
     assert "tensor_P_requant_scale" in txt
     txt = read(emitted, "ConvIntegerDequantize")
-    body = txt[txt.index("void infer_nosync()"):]
-    body = body[:body.index("infer(")]
+    body = ops_body(txt)
     assert body.count("sofie_hip_conv_i8(") == 1 and "a.out = SOFIE_I8OUT_I32" in body and "a.relu = 1" in body
     assert "sofie_hip_dequantize_linear_i32(" in body and "sofie_hip_unary_f32" not in body
 
@@ -246,6 +248,19 @@ def test_parameter_outside_the_leading_dimension_is_refused(tmp_path):
     nodes = [ow.node("Gemm", ["X", "W"], ["Y"], transA=1)]
     r = _emit(tmp_path, nodes, [("X", np.float32, ["N", 4])], [("Y", np.float32, [4, 3])], {"W": np.ones((1, 3), np.float32)})
     assert r.returncode != 0 and "run-time batch" in r.stdout
+
+
+def test_view_based_infer_binds_the_callers_memory(emitted):
+    txt = read(emitted, "Linear_16")
+    # the operators take the graph inputs and outputs as parameters; infer_nosync binds the arena's regions,
+    # the overload on views binds the caller's memory (README.md:291-297 of the reference lists the three signatures)
+    assert re.search(r"void doInfer\(float const \*tensor_\w+, float \*tensor_\w+\)", txt)
+    assert "void infer(std::span<ViewConstF1D const> inputs, std::span<ViewF1D> outputs)" in txt
+    assert "using ViewF1D = DeviceView<float>;" in txt and "#if __cplusplus >= 202002L" in txt
+    # a model whose input is not float has no such overload (the views are float views)
+    assert "std::span<ViewConstF1D const>" in read(emitted, "Config5_int8_CNN_small")
+    txt = read(emitted, "DynamicLinear")
+    assert "void infer(std::span<ViewConstF1D const> inputs, std::span<ViewF1D> outputs, std::size_t N)" in txt
 
 
 def test_asymmetric_zero_point_is_refused(tmp_path):

@@ -175,3 +175,33 @@ def test_emitted_conv_integer_chain_is_bit_exact(rt):
     got = run_emitted("ConvIntegerDequantize", [x], want.size).reshape(want.shape)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     assert (acc > 0).any()
+
+
+VIEW_MODELS = [("Linear_16", None), ("ConvWithPadding", None), ("LinearWithSigmoid", None), ("Config1_fp32_MLP", lambda: em.fp32_mlp(64)),
+               ("Config2_int8_MLP_small", lambda: em.int8_mlp([64, 128, 96, 32], 48)), ("Config5_int8_CNN_small", lambda: em.int8_cnn(2, 12)),
+               ("ConvBatchNormRelu", lambda: em.conv_batchnorm_relu(2))]
+
+
+@pytest.mark.parametrize("misalign", [0, 3])
+@pytest.mark.parametrize("model,make", VIEW_MODELS)
+def test_infer_on_views_of_device_memory_equals_infer_on_host_pointers(rt, model, make, misalign):
+    """infer(std::span<ViewConstF1D const>, std::span<ViewF1D>) (the reference's third infer signature): in place on
+    aligned views, through the session's regions otherwise; either way the bits of infer(host pointers)."""
+    if make:
+        spec = make()
+        inputs, out_len = spec["feeds"], int(np.prod(spec["outputs"][0][2]))
+    else:
+        _, inputs, expected = gr.load_fixture(model)
+        out_len = int(expected.size)
+    arrs = [np.ascontiguousarray(a, dtype=np.float32) for a in inputs]
+    lib = ctypes.CDLL(os.path.join(em.OUT, "lib%s.so" % model))
+    err = ctypes.create_string_buffer(1024)
+    weights = os.path.join(em.OUT, model + "_GPU_HIP.dat").encode()
+    ptrs = (ctypes.c_void_p * len(arrs))(*[a.ctypes.data for a in arrs])
+    lens = (ctypes.c_ulong * len(arrs))(*[a.size for a in arrs])
+    want = run_emitted(model, arrs, out_len)
+    got = np.zeros(out_len, dtype=np.float32)
+    print("views", model, "misalign", misalign, flush=True)
+    rc = lib.run_model_views(weights, ptrs, lens, len(arrs), got.ctypes.data_as(ctypes.c_void_p), ctypes.c_ulong(out_len), misalign, err, 1024)
+    assert rc == 0, err.value.decode()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)) and np.abs(want).max() > 0
