@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define SOFIE_HIP_ABI_VERSION 1
+#define SOFIE_HIP_ABI_VERSION 2
 
 typedef struct sofie_hip_ctx sofie_hip_ctx;
 
@@ -80,8 +80,38 @@ enum {
    SOFIE_ACT_SIGMOID = 3,
    SOFIE_ACT_GELU = 4,
    SOFIE_ACT_GELU_TANH = 5,
-   SOFIE_ACT_TANH = 6
+   SOFIE_ACT_TANH = 6,
+   /* The reference's other one-to-one float operators (formulas of core/inc/SOFIE/operators/ROperator_BasicUnary.hxx:17-103
+    * and ROperator_Clip.hxx:18), usable wherever an activation code is:                                              */
+   SOFIE_ACT_RECIPROCAL = 7, /* 1/x                                   */
+   SOFIE_ACT_SQRT = 8,
+   SOFIE_ACT_NEG = 9,
+   SOFIE_ACT_EXP = 10,
+   SOFIE_ACT_LOG = 11,
+   SOFIE_ACT_SIN = 12,
+   SOFIE_ACT_COS = 13,
+   SOFIE_ACT_ABS = 14,
+   SOFIE_ACT_SOFTPLUS = 15,  /* x >= 20 ? x : log1p(exp(x))           */
+   SOFIE_ACT_ATAN = 16,
+   SOFIE_ACT_FLOOR = 17,
+   SOFIE_ACT_ASINH = 18,
+   SOFIE_ACT_ACOSH = 19,
+   SOFIE_ACT_ATANH = 20,
+   SOFIE_ACT_CLIP = 21,      /* max(alpha, min(beta, x))              */
+   SOFIE_ACT_LAST = 21
 };
+
+/* A chain of one-to-one operators applied, in order, to every element an operator stores: what the reference's
+ * elementwise fusion builds from GetElementwiseExpr (core/inc/SOFIE/operators/ROperator_ALPAKA.hxx:57-76) when
+ * such operators follow a Gemm or a Conv.  op[i] is a SOFIE_ACT_* code, alpha[i] / beta[i] its parameters
+ * (LeakyRelu slope; Clip bounds). */
+#define SOFIE_MAX_POST_OPS 4
+typedef struct sofie_post_ops {
+   int32_t count; /* 0..SOFIE_MAX_POST_OPS */
+   int32_t op[SOFIE_MAX_POST_OPS];
+   float alpha[SOFIE_MAX_POST_OPS];
+   float beta[SOFIE_MAX_POST_OPS];
+} sofie_post_ops;
 
 /* How a bias (the Gemm operand C) is broadcast onto Y[M,N]; the four cases the reference's Gemm
  * emitter distinguishes (core/inc/SOFIE/operators/ROperator_Gemm.hxx:578-617). */
@@ -116,6 +146,7 @@ typedef struct sofie_gemm_f32_desc {
    float *Y;
    int32_t batch; /* stacked MatMul count (>=1); strides in elements, 0 = operand shared */
    int64_t strideA, strideB, strideC, strideY;
+   const sofie_post_ops *post; /* applied after `act`; NULL = none */
 } sofie_gemm_f32_desc;
 int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d);
 
@@ -197,6 +228,8 @@ int sofie_hip_dequantize_linear_i32(sofie_hip_ctx *ctx, float *dst, const int32_
 /* Replaces the CPU loops / alpaka kernels of ROperator_Relu, _Sigmoid, _Gelu, _LeakyRelu, _Tanh
  * (core/inc/SOFIE/operators/ROperator_Relu.hxx:47-86 and siblings). dst may equal src. */
 int sofie_hip_unary_f32(sofie_hip_ctx *ctx, float *dst, const float *src, size_t n, int32_t act, float act_alpha);
+/* several of them in one pass over the data: dst[i] = op[count-1](... op[0](src[i])) */
+int sofie_hip_unary_chain_f32(sofie_hip_ctx *ctx, float *dst, const float *src, size_t n, const sofie_post_ops *ops);
 /* ROperator_BasicBinary<float,Add> with multidirectional broadcasting
  * (core/inc/SOFIE/operators/ROperator_BasicBinary.hxx:380-510).  Shapes are right-aligned, rank<=6;
  * a_shape/b_shape hold 1 where the operand is broadcast. */
@@ -228,7 +261,8 @@ typedef struct sofie_conv_desc {
    int32_t OH, OW; /* as computed by the caller's shape inference; checked */
 } sofie_conv_desc;
 int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float *X, const float *W,
-                       const float *bias /* [Cout] or NULL */, int32_t act, float act_alpha, float *Y);
+                       const float *bias /* [Cout] or NULL */, int32_t act, float act_alpha, float *Y,
+                       const sofie_post_ops *post /* applied after `act`; NULL = none */);
 /* int8 form (no counterpart in the reference): acc = conv_i32(X_i8, W_i8) + bias_i32[co], then by `out`
  *   SOFIE_I8OUT_I8   Y_i8  = sat8(rne(float(acc)*scale[co])), then max(.,0) if relu
  *   SOFIE_I8OUT_F32  Y_f32 = float(acc)*scale[co], then max(.,0) if relu

@@ -63,6 +63,18 @@ def unary(x, act, alpha=0.0):
     return y
 
 
+def unary_chain(x, ops):
+    """ops: [(code, alpha, beta)], applied in order (the codes of include/sofie_hip.h)."""
+    x = _f32(x)
+    y = np.empty_like(x)
+    n = len(ops)
+    op = (C.c_int * max(n, 1))(*[int(o[0]) for o in ops])
+    al = (C.c_float * max(n, 1))(*[float(o[1]) for o in ops])
+    be = (C.c_float * max(n, 1))(*[float(o[2]) for o in ops])
+    load().oracle_unary_chain(_ptr(y), _ptr(x), C.c_size_t(x.size), C.c_int(n), op, al, be)
+    return y
+
+
 def add_broadcast(A, B):
     A, B = _f32(A), _f32(B)
     yshape = np.broadcast_shapes(A.shape, B.shape)

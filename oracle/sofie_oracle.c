@@ -113,6 +113,37 @@ ORACLE_API void oracle_tanh(float *out, const float *in, size_t n)
       out[i] = tanhf(in[i]);
 }
 
+/* The reference's remaining one-to-one float operators, codes 7..21 of include/sofie_hip.h:
+ * UnaryOpTraits<T, ...>::Op (core/inc/SOFIE/operators/ROperator_BasicUnary.hxx:17-103: 1/x, std::sqrt, -x, std::exp,
+ * std::log, std::sin, std::cos, std::abs, Softplus as x >= 20 ? x : log1p(exp(x)), std::atan, std::floor, std::asinh,
+ * std::acosh, std::atanh) and Clip, Y = max(min_val, min(max_val, X)) (ROperator_Clip.hxx:18). */
+ORACLE_API void oracle_basic_unary(float *out, const float *in, size_t n, int op, float alpha, float beta)
+{
+   for (size_t i = 0; i < n; ++i) {
+      const float x = in[i];
+      float y = x;
+      switch (op) {
+      case 7: y = 1.0f / x; break;
+      case 8: y = sqrtf(x); break;
+      case 9: y = -x; break;
+      case 10: y = expf(x); break;
+      case 11: y = logf(x); break;
+      case 12: y = sinf(x); break;
+      case 13: y = cosf(x); break;
+      case 14: y = fabsf(x); break;
+      case 15: y = (x >= 20.0f) ? x : log1pf(expf(x)); break;
+      case 16: y = atanf(x); break;
+      case 17: y = floorf(x); break;
+      case 18: y = asinhf(x); break;
+      case 19: y = acoshf(x); break;
+      case 20: y = atanhf(x); break;
+      case 21: y = fmaxf(alpha, fminf(beta, x)); break;
+      default: break;
+      }
+      out[i] = y;
+   }
+}
+
 /* activation codes of include/sofie_hip.h */
 ORACLE_API void oracle_unary(float *out, const float *in, size_t n, int act, float alpha)
 {
@@ -124,8 +155,23 @@ ORACLE_API void oracle_unary(float *out, const float *in, size_t n, int act, flo
    case 5: oracle_gelu_tanh(out, in, n); break;
    case 6: oracle_tanh(out, in, n); break;
    default:
-      if (out != in)
+      if (act >= 7 && act <= 21)
+         oracle_basic_unary(out, in, n, act, alpha, 0.0f);
+      else if (out != in)
          memmove(out, in, n * sizeof(float));
+   }
+}
+
+/* a chain of one-to-one operators, applied in order (codes, alpha, beta as in sofie_post_ops) */
+ORACLE_API void oracle_unary_chain(float *out, const float *in, size_t n, int count, const int *op, const float *alpha, const float *beta)
+{
+   if (out != in)
+      memmove(out, in, n * sizeof(float));
+   for (int i = 0; i < count; ++i) {
+      if (op[i] >= 7 && op[i] <= 21)
+         oracle_basic_unary(out, out, n, op[i], alpha[i], beta[i]);
+      else
+         oracle_unary(out, out, n, op[i], alpha[i]);
    }
 }
 

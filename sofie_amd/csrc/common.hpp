@@ -47,7 +47,7 @@ inline int launch_status(const char *what)
 // ---- scalar formulas shared by every epilogue --------------------------------------------------
 
 // Activation on fp32, the reference's CPU formulas (see sofie_hip.h for the citations).
-__device__ __forceinline__ float apply_act(float v, int act, float alpha)
+__device__ __forceinline__ float apply_act(float v, int act, float alpha, float beta = 0.0f)
 {
    switch (act) {
    case SOFIE_ACT_RELU: return (v > 0.0f) ? v : 0.0f;
@@ -56,8 +56,72 @@ __device__ __forceinline__ float apply_act(float v, int act, float alpha)
    case SOFIE_ACT_GELU: return 0.5f * v * (1.0f + erff(v * 0.7071067811865475f));
    case SOFIE_ACT_GELU_TANH: return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
    case SOFIE_ACT_TANH: return tanhf(v);
+   case SOFIE_ACT_RECIPROCAL: return 1.0f / v;
+   case SOFIE_ACT_SQRT: return sqrtf(v);
+   case SOFIE_ACT_NEG: return -v;
+   case SOFIE_ACT_EXP: return expf(v);
+   case SOFIE_ACT_LOG: return logf(v);
+   case SOFIE_ACT_SIN: return sinf(v);
+   case SOFIE_ACT_COS: return cosf(v);
+   case SOFIE_ACT_ABS: return fabsf(v);
+   case SOFIE_ACT_SOFTPLUS: return (v >= 20.0f) ? v : log1pf(expf(v));
+   case SOFIE_ACT_ATAN: return atanf(v);
+   case SOFIE_ACT_FLOOR: return floorf(v);
+   case SOFIE_ACT_ASINH: return asinhf(v);
+   case SOFIE_ACT_ACOSH: return acoshf(v);
+   case SOFIE_ACT_ATANH: return atanhf(v);
+   case SOFIE_ACT_CLIP: return fmaxf(alpha, fminf(beta, v));
    default: return v;
    }
+}
+
+// An operator's own activation followed by the caller's chain of one-to-one operators, by value in the kernel
+// arguments; `count` is the same for every lane, so the loop does not diverge.
+struct PostChain {
+   int count = 0;
+   int op[SOFIE_MAX_POST_OPS + 1];
+   float alpha[SOFIE_MAX_POST_OPS + 1];
+   float beta[SOFIE_MAX_POST_OPS + 1];
+};
+
+__device__ __forceinline__ float apply_chain(float v, const PostChain &c)
+{
+   for (int i = 0; i < c.count; ++i)
+      v = apply_act(v, c.op[i], c.alpha[i], c.beta[i]);
+   return v;
+}
+
+// Host side: checks the codes and builds the chain {act, post...}.  Returns false (with `bad` set to the offending
+// code, or -1 for a bad count) if anything is out of range.
+inline bool make_post_chain(PostChain &c, int act, float act_alpha, const sofie_post_ops *post, int &bad)
+{
+   c.count = 0;
+   bad = act;
+   if (act < SOFIE_ACT_NONE || act > SOFIE_ACT_LAST)
+      return false;
+   if (act != SOFIE_ACT_NONE) {
+      c.op[0] = act;
+      c.alpha[0] = act_alpha;
+      c.beta[0] = 0.0f;
+      c.count = 1;
+   }
+   if (!post)
+      return true;
+   bad = -1;
+   if (post->count < 0 || post->count > SOFIE_MAX_POST_OPS)
+      return false;
+   for (int i = 0; i < post->count; ++i) {
+      bad = post->op[i];
+      if (post->op[i] < SOFIE_ACT_NONE || post->op[i] > SOFIE_ACT_LAST)
+         return false;
+      if (post->op[i] == SOFIE_ACT_NONE)
+         continue;
+      c.op[c.count] = post->op[i];
+      c.alpha[c.count] = post->alpha[i];
+      c.beta[c.count] = post->beta[i];
+      ++c.count;
+   }
+   return true;
 }
 
 // sat8(rne(v)): round half to even, saturate to [-128,127]; NaN -> 0 (matches the CPU restatement,

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void dequantize_linear_kernel(float *__restric
       dst[i] = mul_nofma((float)src[i], scale);
 }
 
-__global__ __launch_bounds__(256) void unary_f32_kernel(float *dst, const float *src, size_t n, int act, float alpha, int vec)
+__global__ __launch_bounds__(256) void unary_f32_kernel(float *dst, const float *src, size_t n, PostChain chain, int vec)
 {
    const size_t stride = (size_t)gridDim.x * blockDim.x;
    size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
@@ -58,18 +58,18 @@ __global__ __launch_bounds__(256) void unary_f32_kernel(float *dst, const float 
       const size_t n4 = n / 4;
       for (; i < n4; i += stride) {
          float4 v = ((const float4 *)src)[i];
-         v.x = apply_act(v.x, act, alpha);
-         v.y = apply_act(v.y, act, alpha);
-         v.z = apply_act(v.z, act, alpha);
-         v.w = apply_act(v.w, act, alpha);
+         v.x = apply_chain(v.x, chain);
+         v.y = apply_chain(v.y, chain);
+         v.z = apply_chain(v.z, chain);
+         v.w = apply_chain(v.w, chain);
          ((float4 *)dst)[i] = v;
       }
       i = n4 * 4 + (blockIdx.x * (size_t)blockDim.x + threadIdx.x);
       if (i < n)
-         dst[i] = apply_act(src[i], act, alpha);
+         dst[i] = apply_chain(src[i], chain);
    } else {
       for (; i < n; i += stride)
-         dst[i] = apply_act(src[i], act, alpha);
+         dst[i] = apply_chain(src[i], chain);
    }
 }
 
@@ -239,16 +239,36 @@ int sofie_hip_dequantize_linear_i32(sofie_hip_ctx *ctx, float *dst, const int32_
    return launch_status("dequantize_linear_kernel");
 }
 
+static int launch_unary_chain(sofie_hip_ctx *ctx, float *dst, const float *src, size_t n, const PostChain &chain)
+{
+   const int vec = (((uintptr_t)src & 15) == 0) && (((uintptr_t)dst & 15) == 0);
+   hipLaunchKernelGGL(unary_f32_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(256), 0, ctx->stream, dst, src, n, chain, vec);
+   return launch_status("unary_f32_kernel");
+}
+
 int sofie_hip_unary_f32(sofie_hip_ctx *ctx, float *dst, const float *src, size_t n, int32_t act, float act_alpha)
 {
    SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_unary_f32: ctx is NULL");
-   SOFIE_HIP_REQUIRE(act >= SOFIE_ACT_NONE && act <= SOFIE_ACT_TANH, "sofie_hip_unary_f32: unknown activation %d", act);
+   PostChain chain;
+   int bad = 0;
+   SOFIE_HIP_REQUIRE(make_post_chain(chain, act, act_alpha, nullptr, bad), "sofie_hip_unary_f32: unknown activation %d", act);
    if (n == 0)
       return SOFIE_HIP_OK;
    SOFIE_HIP_REQUIRE(dst && src, "sofie_hip_unary_f32: NULL pointer");
-   const int vec = (((uintptr_t)src & 15) == 0) && (((uintptr_t)dst & 15) == 0);
-   hipLaunchKernelGGL(unary_f32_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(256), 0, ctx->stream, dst, src, n, act, act_alpha, vec);
-   return launch_status("unary_f32_kernel");
+   return launch_unary_chain(ctx, dst, src, n, chain);
+}
+
+int sofie_hip_unary_chain_f32(sofie_hip_ctx *ctx, float *dst, const float *src, size_t n, const sofie_post_ops *ops)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr && ops != nullptr, "sofie_hip_unary_chain_f32: NULL argument");
+   PostChain chain;
+   int bad = 0;
+   SOFIE_HIP_REQUIRE(make_post_chain(chain, SOFIE_ACT_NONE, 0.0f, ops, bad),
+                     "sofie_hip_unary_chain_f32: unknown operator %d (or more than %d operators)", bad, SOFIE_MAX_POST_OPS);
+   if (n == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(dst && src, "sofie_hip_unary_chain_f32: NULL pointer");
+   return launch_unary_chain(ctx, dst, src, n, chain);
 }
 
 int sofie_hip_add_f32(sofie_hip_ctx *ctx, const sofie_add_desc *d)

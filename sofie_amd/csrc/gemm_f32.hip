@@ -26,8 +26,7 @@ struct F32Epilogue {
    const float *C;
    int bias_mode;
    long long ldc;
-   int act;
-   float act_alpha;
+   PostChain chain; // the activation, then the caller's chain of one-to-one operators
 };
 
 __device__ __forceinline__ float f32_epilogue(const F32Epilogue &ep, float acc, int m, int n)
@@ -40,7 +39,7 @@ __device__ __forceinline__ float f32_epilogue(const F32Epilogue &ep, float acc, 
    case SOFIE_BIAS_FULL: v += ep.beta * ep.C[m * ep.ldc + n]; break;
    default: break;
    }
-   return apply_act(v, ep.act, ep.act_alpha);
+   return apply_chain(v, ep.chain);
 }
 
 // The tile loop: acc[4][4] per lane over a 64x64 tile.  LA(m,k), LB(k,n) return 0-safe values only for
@@ -260,7 +259,7 @@ struct ConvOperandB {
 };
 
 __global__ __launch_bounds__(256) void conv_f32_kernel(ConvOperandA la, const float *Wt, const float *bias, float *Y, int M,
-                                                        int Cout_g, int Kg, int Cg, int Cout, int OHW, int act, float act_alpha)
+                                                        int Cout_g, int Kg, int Cg, int Cout, int OHW, PostChain chain)
 {
    const int g = blockIdx.z;
    la.c_first = g * Cg;
@@ -283,7 +282,7 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(ConvOperandA la, const fl
             float v = acc[i][j];
             if (bias)
                v += bias[co];
-            Y[((size_t)img * Cout + co) * OHW + pix] = apply_act(v, act, act_alpha);
+            Y[((size_t)img * Cout + co) * OHW + pix] = apply_chain(v, chain);
          }
       }
    }
@@ -301,7 +300,10 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d)
    SOFIE_HIP_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "sofie_hip_gemm_f32: negative dimension");
    SOFIE_HIP_REQUIRE(d->batch >= 1, "sofie_hip_gemm_f32: batch must be >= 1");
    SOFIE_HIP_REQUIRE(d->bias_mode >= SOFIE_BIAS_NONE && d->bias_mode <= SOFIE_BIAS_FULL, "sofie_hip_gemm_f32: unknown bias mode %d", d->bias_mode);
-   SOFIE_HIP_REQUIRE(d->act >= SOFIE_ACT_NONE && d->act <= SOFIE_ACT_TANH, "sofie_hip_gemm_f32: unknown activation %d", d->act);
+   F32Epilogue ep;
+   int bad = 0;
+   SOFIE_HIP_REQUIRE(make_post_chain(ep.chain, d->act, d->act_alpha, d->post, bad),
+                     "sofie_hip_gemm_f32: unknown activation or post operator %d (or more than %d post operators)", bad, SOFIE_MAX_POST_OPS);
    if (d->M == 0 || d->N == 0)
       return SOFIE_HIP_OK;
    SOFIE_HIP_REQUIRE(d->Y != nullptr, "sofie_hip_gemm_f32: Y is NULL");
@@ -315,14 +317,11 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d)
                      "sofie_hip_gemm_f32: leading dimension too small");
    GemmOperandA la{d->A, d->transA ? 1 : lda, d->transA ? lda : 1};
    GemmOperandB lb{d->B, d->transB ? 1 : ldb, d->transB ? ldb : 1};
-   F32Epilogue ep;
    ep.alpha = d->alpha;
    ep.beta = d->beta;
    ep.C = d->bias_mode == SOFIE_BIAS_NONE ? nullptr : d->C;
    ep.bias_mode = d->bias_mode;
    ep.ldc = N;
-   ep.act = d->act;
-   ep.act_alpha = d->act_alpha;
    const unsigned gy = (M + F32_BM - 1) / F32_BM, gx = (N + F32_BN - 1) / F32_BN;
    SOFIE_HIP_REQUIRE(gx <= 65535 && d->batch <= 65535, "sofie_hip_gemm_f32: N or batch too large for one launch");
    // few 64x64 tiles: one-wave workgroups with 8x8 tiles reach every CU (SOFIE_HIP_F32_SKINNY=0/1 overrides)
@@ -353,7 +352,7 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d)
 }
 
 int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float *X, const float *W, const float *bias,
-                       int32_t act, float act_alpha, float *Y)
+                       int32_t act, float act_alpha, float *Y, const sofie_post_ops *post)
 {
    SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_conv_f32: NULL argument");
    SOFIE_HIP_REQUIRE(d->N >= 0 && d->C > 0 && d->H > 0 && d->W > 0 && d->Cout > 0 && d->kh > 0 && d->kw > 0,
@@ -369,7 +368,10 @@ int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float
    const int OW = (d->W + d->pad_w0 + d->pad_w1 - eff_kw) / d->stride_w + 1;
    SOFIE_HIP_REQUIRE(OH == d->OH && OW == d->OW, "sofie_hip_conv_f32: output shape %dx%d does not match the descriptor's %dx%d", OH, OW,
                      d->OH, d->OW);
-   SOFIE_HIP_REQUIRE(act >= SOFIE_ACT_NONE && act <= SOFIE_ACT_TANH, "sofie_hip_conv_f32: unknown activation %d", act);
+   PostChain chain;
+   int bad = 0;
+   SOFIE_HIP_REQUIRE(make_post_chain(chain, act, act_alpha, post, bad),
+                     "sofie_hip_conv_f32: unknown activation or post operator %d (or more than %d post operators)", bad, SOFIE_MAX_POST_OPS);
    if (d->N == 0)
       return SOFIE_HIP_OK;
    SOFIE_HIP_REQUIRE(X && W && Y, "sofie_hip_conv_f32: NULL pointer");
@@ -380,7 +382,7 @@ int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float
    const unsigned gy = (unsigned)((M + F32_BM - 1) / F32_BM), gx = (Cout_g + F32_BN - 1) / F32_BN;
    SOFIE_HIP_REQUIRE(gx <= 65535 && d->group <= 65535, "sofie_hip_conv_f32: too many channels or groups for one launch");
    hipLaunchKernelGGL(conv_f32_kernel, dim3(gy, gx, (unsigned)d->group), dim3(256), 0, ctx->stream, la, W, bias, Y, (int)M, Cout_g, Kg,
-                      Cg, d->Cout, OH * OW, act, act_alpha);
+                      Cg, d->Cout, OH * OW, chain);
    return launch_status("conv_f32_kernel");
 }
 

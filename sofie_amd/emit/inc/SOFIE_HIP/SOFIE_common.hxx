@@ -21,7 +21,20 @@ enum class ETensorType {
    FLOAT16 = 10, DOUBLE = 11, UINT32 = 12, UINT64 = 13, BFLOAT16 = 16, FLOAT8E4M3FN = 17
 };
 
-enum class EActivationType { UNDEFINED, RELU, LEAKYRELU, SIGMOID, GELU, GELU_TANH, TANH };
+// the six activations a producer can take as its own, then the reference's other one-to-one float operators
+// (EBasicUnaryOperator, core/inc/SOFIE/operators/ROperator_BasicUnary.hxx:11, and Clip)
+enum class EActivationType {
+   UNDEFINED, RELU, LEAKYRELU, SIGMOID, GELU, GELU_TANH, TANH,
+   RECIPROCAL, SQRT, NEG, EXP, LOG, SIN, COS, ABS, SOFTPLUS, ATAN, FLOOR, ASINH, ACOSH, ATANH, CLIP
+};
+enum class EBasicUnaryOperator { kReciprocal, kSqrt, kNeg, kExp, kLog, kSin, kCos, kAbs, kSoftplus, kAtan, kFloor, kAsinh, kAcosh, kAtanh };
+
+// one link of a chain of one-to-one operators fused behind a producer (alpha: LeakyRelu slope or Clip minimum, beta: Clip maximum)
+struct PostOp {
+   EActivationType act = EActivationType::UNDEFINED;
+   float alpha = 0.f, beta = 0.f;
+};
+constexpr std::size_t kMaxPostOps = 4; // SOFIE_MAX_POST_OPS of the runtime
 
 // Options of RModel::GenerateGPU_HIP: the subset of the reference's bit flags (core/inc/SOFIE/RModel_Base.hxx:19-33)
 // that applies to this backend, with the reference's values.

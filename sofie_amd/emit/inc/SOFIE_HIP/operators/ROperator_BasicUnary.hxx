@@ -1,7 +1,9 @@
-// Stand-alone activation operators (Relu, LeakyRelu, Sigmoid, Gelu, Tanh): the emitters of
-// core/inc/SOFIE/operators/ROperator_Relu.hxx, _LeakyRelu.hxx, _Sigmoid.hxx, _Gelu.hxx, _Tanh.hxx as one
-// class; each emits one sofie_hip_unary_f32 call, unless the generator has fused it into the producing
-// Gemm or Conv.
+// One-to-one float operators: the activations (core/inc/SOFIE/operators/ROperator_Relu.hxx, _LeakyRelu.hxx,
+// _Sigmoid.hxx, _Gelu.hxx, _Tanh.hxx), the basic unary operators (ROperator_BasicUnary.hxx) and Clip
+// (ROperator_Clip.hxx) as one class.  The generator folds such an operator into the Gemm or Conv that produces
+// its input, or into the one-to-one operator before it (the reference's elementwise fusion,
+// core/inc/SOFIE/operators/ROperator_ALPAKA.hxx:57-76); what remains emits one sofie_hip_unary_f32 or
+// sofie_hip_unary_chain_f32 call.
 #ifndef SOFIE_HIP_ROPERATOR_BASICUNARY
 #define SOFIE_HIP_ROPERATOR_BASICUNARY
 
@@ -11,8 +13,8 @@ namespace SOFIE_HIP {
 
 class ROperator_Activation : public ROperator {
 public:
-   ROperator_Activation(EActivationType act, float alpha, std::string nameX, std::string nameY)
-      : fAct(act), fAlpha(alpha), fNX(UTILITY::Clean_name(nameX)), fNY(UTILITY::Clean_name(nameY))
+   ROperator_Activation(EActivationType act, float alpha, std::string nameX, std::string nameY, float beta = 0.f)
+      : fAct(act), fAlpha(alpha), fBeta(beta), fNX(UTILITY::Clean_name(nameX)), fNY(UTILITY::Clean_name(nameY))
    {
       fInputTensorNames = {fNX};
       fOutputTensorNames = {fNY};
@@ -20,7 +22,21 @@ public:
    }
    EActivationType Activation() const { return fAct; }
    float Alpha() const { return fAlpha; }
+   float Beta() const { return fBeta; }
    const std::string &OutputName() const { return fNY; }
+   // this operator followed by the ones folded into it
+   std::vector<PostOp> Chain() const
+   {
+      std::vector<PostOp> c{PostOp{fAct, fAlpha, fBeta}};
+      c.insert(c.end(), fPost.begin(), fPost.end());
+      return c;
+   }
+   void AddPostOp(const PostOp &op, const std::string &newOutput)
+   {
+      fPost.push_back(op);
+      fNY = newOutput;
+      fOutputTensorNames = {fNY};
+   }
 
    void Initialize(RModel &model) override
    {
@@ -39,15 +55,28 @@ public:
    {
       opName = "op_" + opName;
       std::stringstream out;
-      out << "\n" << SP << "//------ " << ActivationEnumName(fAct) << " " << opName << "\n";
-      out << SP << "detail::Check(sofie_hip_unary_f32(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << BatchScaled(fDynamic, ConvertShapeToLength(fShape))
-          << ", " << ActivationEnumName(fAct) << ", " << FloatLiteral(fAlpha) << "), \"" << opName << " activation\");\n";
+      out << "\n" << SP << "//------ " << ActivationEnumName(fAct);
+      for (auto &p : fPost)
+         out << " -> " << ActivationEnumName(p.act);
+      out << " " << opName << "\n";
+      if (fPost.empty() && fAct != EActivationType::CLIP) {
+         out << SP << "detail::Check(sofie_hip_unary_f32(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", "
+             << BatchScaled(fDynamic, ConvertShapeToLength(fShape)) << ", " << ActivationEnumName(fAct) << ", " << FloatLiteral(fAlpha) << "), \""
+             << opName << " activation\");\n";
+         return out.str();
+      }
+      out << SP << "{\n";
+      out << SP << "   " << PostOpsDeclaration("ops", Chain()) << "\n";
+      out << SP << "   " << "detail::Check(sofie_hip_unary_chain_f32(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", "
+          << BatchScaled(fDynamic, ConvertShapeToLength(fShape)) << ", &ops), \"" << opName << " one-to-one chain\");\n";
+      out << SP << "}\n";
       return out.str();
    }
 
 protected:
    EActivationType fAct;
-   float fAlpha;
+   float fAlpha, fBeta = 0.f;
+   std::vector<PostOp> fPost;
    std::string fNX, fNY;
    std::vector<std::size_t> fShape;
    ETensorType fType = ETensorType::FLOAT;
@@ -80,6 +109,41 @@ struct ROperator_Gelu : ROperator_Activation {
       if (approximate != "tanh" && approximate != "none")
          throw std::runtime_error("SOFIE Gelu Op: unknown approximation " + approximate);
    }
+};
+
+// ROperator_BasicUnary<T, Op> of the reference (core/inc/SOFIE/operators/ROperator_BasicUnary.hxx:106-170)
+inline EActivationType BasicUnaryActivation(EBasicUnaryOperator op)
+{
+   switch (op) {
+   case EBasicUnaryOperator::kReciprocal: return EActivationType::RECIPROCAL;
+   case EBasicUnaryOperator::kSqrt: return EActivationType::SQRT;
+   case EBasicUnaryOperator::kNeg: return EActivationType::NEG;
+   case EBasicUnaryOperator::kExp: return EActivationType::EXP;
+   case EBasicUnaryOperator::kLog: return EActivationType::LOG;
+   case EBasicUnaryOperator::kSin: return EActivationType::SIN;
+   case EBasicUnaryOperator::kCos: return EActivationType::COS;
+   case EBasicUnaryOperator::kAbs: return EActivationType::ABS;
+   case EBasicUnaryOperator::kSoftplus: return EActivationType::SOFTPLUS;
+   case EBasicUnaryOperator::kAtan: return EActivationType::ATAN;
+   case EBasicUnaryOperator::kFloor: return EActivationType::FLOOR;
+   case EBasicUnaryOperator::kAsinh: return EActivationType::ASINH;
+   case EBasicUnaryOperator::kAcosh: return EActivationType::ACOSH;
+   default: return EActivationType::ATANH;
+   }
+}
+template <typename T, EBasicUnaryOperator Op>
+struct ROperator_BasicUnary : ROperator_Activation {
+   ROperator_BasicUnary(std::string x, std::string y) : ROperator_Activation(BasicUnaryActivation(Op), 0.f, x, y) {}
+};
+// Clip with constant bounds: Y = max(min, min(max, X)) (core/inc/SOFIE/operators/ROperator_Clip.hxx:18, 92-100)
+template <typename T>
+struct ROperator_Clip : ROperator_Activation {
+   ROperator_Clip(std::string x, std::string y, T minVal, T maxVal) : ROperator_Activation(EActivationType::CLIP, minVal, x, y, maxVal) {}
+};
+// Identity: a copy that the generator folds away wherever it follows another operator
+template <typename T>
+struct ROperator_Identity : ROperator_Activation {
+   ROperator_Identity(std::string x, std::string y) : ROperator_Activation(EActivationType::UNDEFINED, 0.f, x, y) {}
 };
 
 } // namespace SOFIE_HIP

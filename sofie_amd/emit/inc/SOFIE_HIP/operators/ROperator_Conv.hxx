@@ -133,6 +133,13 @@ public:
       fNY = newOutput;
       fOutputTensorNames = {fNY};
    }
+   std::size_t PostOpCount() const { return fPost.size(); }
+   void AddPostOp(const PostOp &op, const std::string &newOutput)
+   {
+      fPost.push_back(op);
+      fNY = newOutput;
+      fOutputTensorNames = {fNY};
+   }
    void Initialize(RModel &model) override
    {
       if (!model.CheckIfTensorAlreadyExist(fNX))
@@ -162,9 +169,11 @@ public:
       out << "\n" << SP << "//----  operator Conv " << opName << " --> " << ConvertShapeToString(fGeo.OutputShape()) << "\n";
       out << SP << "{\n";
       out << SP << "   " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n" << fGeo.BatchLine(fDynamic, SP + "   ");
+      if (!fPost.empty())
+         out << SP << "   " << PostOpsDeclaration("post", fPost) << "\n";
       out << SP << "   " << "detail::Check(sofie_hip_conv_f32(fCtx, &d, tensor_" << fNX << ", tensor_" << fNW << ", "
           << (fNB.empty() ? "nullptr" : "tensor_" + fNB) << ", " << ActivationEnumName(fActivation) << ", " << FloatLiteral(fActAlpha)
-          << ", tensor_" << fNY << "), \"" << opName << " Conv\");\n";
+          << ", tensor_" << fNY << ", " << (fPost.empty() ? "nullptr" : "&post") << "), \"" << opName << " Conv\");\n";
       out << SP << "}\n";
       return out.str();
    }
@@ -177,6 +186,7 @@ private:
    std::string fNX, fNW, fNB, fNY;
    EActivationType fActivation = EActivationType::UNDEFINED;
    float fActAlpha = 0.01f;
+   std::vector<PostOp> fPost;
    ConvGeometry fGeo;
    bool fDynamic = false;
 };

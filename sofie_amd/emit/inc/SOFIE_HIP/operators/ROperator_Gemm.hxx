@@ -21,9 +21,27 @@ inline const char *ActivationEnumName(EActivationType a)
    case EActivationType::GELU: return "SOFIE_ACT_GELU";
    case EActivationType::GELU_TANH: return "SOFIE_ACT_GELU_TANH";
    case EActivationType::TANH: return "SOFIE_ACT_TANH";
+   case EActivationType::RECIPROCAL: return "SOFIE_ACT_RECIPROCAL";
+   case EActivationType::SQRT: return "SOFIE_ACT_SQRT";
+   case EActivationType::NEG: return "SOFIE_ACT_NEG";
+   case EActivationType::EXP: return "SOFIE_ACT_EXP";
+   case EActivationType::LOG: return "SOFIE_ACT_LOG";
+   case EActivationType::SIN: return "SOFIE_ACT_SIN";
+   case EActivationType::COS: return "SOFIE_ACT_COS";
+   case EActivationType::ABS: return "SOFIE_ACT_ABS";
+   case EActivationType::SOFTPLUS: return "SOFIE_ACT_SOFTPLUS";
+   case EActivationType::ATAN: return "SOFIE_ACT_ATAN";
+   case EActivationType::FLOOR: return "SOFIE_ACT_FLOOR";
+   case EActivationType::ASINH: return "SOFIE_ACT_ASINH";
+   case EActivationType::ACOSH: return "SOFIE_ACT_ACOSH";
+   case EActivationType::ATANH: return "SOFIE_ACT_ATANH";
+   case EActivationType::CLIP: return "SOFIE_ACT_CLIP";
    default: return "SOFIE_ACT_NONE";
    }
 }
+
+// true for the activations an operator's own `act` field can hold (one parameter at most)
+inline bool IsProducerActivation(EActivationType a) { return a >= EActivationType::RELU && a <= EActivationType::TANH; }
 
 inline std::string FloatLiteral(float v)
 {
@@ -33,6 +51,23 @@ inline std::string FloatLiteral(float v)
    if (t.find_first_of(".eEn") == std::string::npos)
       t += ".0";
    return t + "f";
+}
+
+// `sofie_post_ops <name>{...};` for a chain of fused one-to-one operators
+inline std::string PostOpsDeclaration(const std::string &name, const std::vector<PostOp> &ops)
+{
+   std::ostringstream s;
+   s << "sofie_post_ops " << name << "{" << ops.size() << ", {";
+   for (std::size_t i = 0; i < kMaxPostOps; ++i)
+      s << (i < ops.size() ? ActivationEnumName(ops[i].act) : "SOFIE_ACT_NONE") << (i + 1 < kMaxPostOps ? ", " : "");
+   s << "}, {";
+   for (std::size_t i = 0; i < kMaxPostOps; ++i)
+      s << FloatLiteral(i < ops.size() ? ops[i].alpha : 0.f) << (i + 1 < kMaxPostOps ? ", " : "");
+   s << "}, {";
+   for (std::size_t i = 0; i < kMaxPostOps; ++i)
+      s << FloatLiteral(i < ops.size() ? ops[i].beta : 0.f) << (i + 1 < kMaxPostOps ? ", " : "");
+   s << "}};";
+   return s.str();
 }
 
 template <typename T>
@@ -66,6 +101,14 @@ public:
    {
       fActivation = a;
       fActAlpha = alpha;
+      fNY = newOutput;
+      fOutputTensorNames = {fNY};
+   }
+   // further one-to-one operators behind the activation, applied in the kernel's store in this order
+   std::size_t PostOpCount() const { return fPost.size(); }
+   void AddPostOp(const PostOp &op, const std::string &newOutput)
+   {
+      fPost.push_back(op);
       fNY = newOutput;
       fOutputTensorNames = {fNY};
    }
@@ -208,6 +251,8 @@ public:
       out << SP << "   " << "d.act = " << ActivationEnumName(fActivation) << "; d.act_alpha = " << FloatLiteral(fActAlpha) << ";\n";
       out << SP << "   " << "d.Y = tensor_" << fNY << "; d.batch = " << BatchScaledInt(fDynamicStack, fBatch) << "; d.strideA = " << fStrideA << "; d.strideB = "
           << fStrideB << "; d.strideC = " << fStrideC << "; d.strideY = " << (fBatch > 1 || fDynamicStack ? fM * fN : 0) << ";\n";
+      if (!fPost.empty())
+         out << SP << "   " << PostOpsDeclaration("post", fPost) << " d.post = &post;\n";
       out << SP << "   " << "detail::Check(sofie_hip_gemm_f32(fCtx, &d), \"" << opName << " Gemm\");\n";
       out << SP << "}\n";
       return out.str();
@@ -219,6 +264,7 @@ private:
    std::string fNA, fNB, fNC, fNY;
    EActivationType fActivation = EActivationType::UNDEFINED;
    float fActAlpha = 0.01f;
+   std::vector<PostOp> fPost;
    std::vector<std::size_t> fShapeA, fShapeB;
    std::size_t fM = 0, fN = 0, fK = 0, fBatch = 1, fStrideA = 0, fStrideB = 0, fStrideC = 0;
    std::string fBiasMode;

@@ -198,23 +198,41 @@ void RModel::FuseGemmActivations()
             continue;
          ROperator *next = fOperators[cons[0]].get();
          auto *act = dynamic_cast<ROperator_Activation *>(next);
-         if (auto *g = dynamic_cast<ROperator_Gemm<float> *>(op)) {
-            if (act && !g->HasActivation()) {
-               g->FuseActivation(act->Activation(), act->Alpha(), act->OutputName());
-               changed = true;
+         const bool plainRelu = act && act->Activation() == EActivationType::RELU && act->Chain().size() == 1;
+         // A one-to-one float operator behind a Gemm, a Conv or another one-to-one operator joins its producer: as the
+         // producer's own activation when that slot is free and nothing is queued behind it, else as the next link of the
+         // chain the kernel applies in its store (at most kMaxPostOps links).
+         auto absorb = [&](auto *producer) {
+            if (!act)
+               return false;
+            if (!producer->HasActivation() && producer->PostOpCount() == 0 && IsProducerActivation(act->Activation())) {
+               producer->FuseActivation(act->Activation(), act->Alpha(), act->OutputName());
+               return true;
             }
+            auto links = act->Chain();
+            if (producer->PostOpCount() + links.size() > kMaxPostOps)
+               return false;
+            for (auto &l : links)
+               producer->AddPostOp(l, act->OutputName());
+            return true;
+         };
+         if (auto *g = dynamic_cast<ROperator_Gemm<float> *>(op)) {
+            changed = absorb(g);
          } else if (auto *c = dynamic_cast<ROperator_Conv<float> *>(op)) {
-            if (act && !c->HasActivation()) {
-               c->FuseActivation(act->Activation(), act->Alpha(), act->OutputName());
+            changed = absorb(c);
+         } else if (auto *u = dynamic_cast<ROperator_Activation *>(op)) {
+            if (act && u->Chain().size() + act->Chain().size() <= kMaxPostOps) {
+               for (auto &l : act->Chain())
+                  u->AddPostOp(l, act->OutputName());
                changed = true;
             }
          } else if (auto *bn = dynamic_cast<ROperator_BatchNormalization<float> *>(op)) {
-            if (act && act->Activation() == EActivationType::RELU && !bn->HasActivation()) {
+            if (plainRelu && !bn->HasActivation()) {
                bn->FuseRelu(act->OutputName());
                changed = true;
             }
          } else if (auto *qc = dynamic_cast<ROperator_QConv *>(op)) {
-            if (act && act->Activation() == EActivationType::RELU && !qc->HasRelu()) {
+            if (plainRelu && !qc->HasRelu()) {
                qc->FuseRelu(act->OutputName());
                changed = true;
             }
@@ -226,11 +244,11 @@ void RModel::FuseGemmActivations()
                changed = true;
             }
          } else if (auto *q = dynamic_cast<ROperator_QGemm *>(op)) {
-            if (q->OutputKind() == ROperator_QGemm::Out::I8_REQUANT && act && act->Activation() == EActivationType::RELU && !q->ReluOnOutput()) {
+            if (q->OutputKind() == ROperator_QGemm::Out::I8_REQUANT && plainRelu && !q->ReluOnOutput()) {
                q->SetReluOnOutput(); // Relu on the requantised int8 value: max(sat8(x), 0)
                q->SetOutputName(act->OutputName());
                changed = true;
-            } else if (q->OutputKind() == ROperator_QGemm::Out::I32 && act && act->Activation() == EActivationType::RELU && !q->ReluOnAccumulator()) {
+            } else if (q->OutputKind() == ROperator_QGemm::Out::I32 && plainRelu && !q->ReluOnAccumulator()) {
                q->SetReluOnAccumulator();
                q->SetOutputName(act->OutputName());
                changed = true;

@@ -4,6 +4,7 @@
 #include <fstream>
 #include <iostream>
 #include <iterator>
+#include <limits>
 #include <map>
 
 namespace SOFIE_HIP {
@@ -389,6 +390,25 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          model->AddOperator(std::make_unique<ROperator_LeakyRelu<float>>(attrF(n, "alpha", 0.01f), n.in[0], n.out[0]));
       } else if (n.op == "Gelu") {
          model->AddOperator(std::make_unique<ROperator_Gelu<float>>(attrS(n, "approximate", "none"), n.in[0], n.out[0]));
+      } else if (n.op == "Reciprocal" || n.op == "Sqrt" || n.op == "Neg" || n.op == "Exp" || n.op == "Log" || n.op == "Sin" || n.op == "Cos" ||
+                 n.op == "Abs" || n.op == "Softplus" || n.op == "Atan" || n.op == "Floor" || n.op == "Asinh" || n.op == "Acosh" || n.op == "Atanh") {
+         // the reference's ROperator_BasicUnary family (parsers/src/ParseBasicUnary.cxx)
+         static const std::map<std::string, EActivationType> kinds = {
+            {"Reciprocal", EActivationType::RECIPROCAL}, {"Sqrt", EActivationType::SQRT}, {"Neg", EActivationType::NEG}, {"Exp", EActivationType::EXP},
+            {"Log", EActivationType::LOG}, {"Sin", EActivationType::SIN}, {"Cos", EActivationType::COS}, {"Abs", EActivationType::ABS},
+            {"Softplus", EActivationType::SOFTPLUS}, {"Atan", EActivationType::ATAN}, {"Floor", EActivationType::FLOOR},
+            {"Asinh", EActivationType::ASINH}, {"Acosh", EActivationType::ACOSH}, {"Atanh", EActivationType::ATANH}};
+         model->AddOperator(std::make_unique<ROperator_Activation>(kinds.at(n.op), 0.f, n.in[0], n.out[0]));
+      } else if (n.op == "Identity") {
+         model->AddOperator(std::make_unique<ROperator_Identity<float>>(n.in[0], n.out[0]));
+      } else if (n.op == "Clip") {
+         // bounds: attributes up to opset 10, optional scalar initializers (inputs 1 and 2) from opset 11 on; absent = unbounded
+         float lo = attrF(n, "min", std::numeric_limits<float>::lowest()), hi = attrF(n, "max", std::numeric_limits<float>::max());
+         if (n.in.size() > 1 && !n.in[1].empty())
+            lo = model->GetScalarInitializer(n.in[1]);
+         if (n.in.size() > 2 && !n.in[2].empty())
+            hi = model->GetScalarInitializer(n.in[2]);
+         model->AddOperator(std::make_unique<ROperator_Clip<float>>(n.in[0], n.out[0], lo, hi));
       } else if (n.op == "Add") {
          model->AddOperator(std::make_unique<ROperator_BasicBinary<float, Add>>(n.in[0], n.in[1], n.out[0]));
       } else if (n.op == "Conv") {

@@ -17,11 +17,26 @@ class SofieHipError(RuntimeError):
 
 
 # activation / bias / output codes of include/sofie_hip.h
-ACT_NONE, ACT_RELU, ACT_LEAKYRELU, ACT_SIGMOID, ACT_GELU, ACT_GELU_TANH, ACT_TANH = range(7)
+(ACT_NONE, ACT_RELU, ACT_LEAKYRELU, ACT_SIGMOID, ACT_GELU, ACT_GELU_TANH, ACT_TANH, ACT_RECIPROCAL, ACT_SQRT, ACT_NEG, ACT_EXP, ACT_LOG,
+ ACT_SIN, ACT_COS, ACT_ABS, ACT_SOFTPLUS, ACT_ATAN, ACT_FLOOR, ACT_ASINH, ACT_ACOSH, ACT_ATANH, ACT_CLIP) = range(22)
+MAX_POST_OPS = 4
 BIAS_NONE, BIAS_ROW, BIAS_COL, BIAS_SCALAR, BIAS_FULL = range(5)
 I8OUT_I32, I8OUT_F32, I8OUT_I8, I8OUT_I8_DQQ = range(4)
 F8OUT_BF16, F8OUT_F32 = range(2)
 LAYOUT_NCHW, LAYOUT_NHWC = range(2)
+
+
+class PostOps(C.Structure):
+    _fields_ = [("count", C.c_int32), ("op", C.c_int32 * MAX_POST_OPS), ("alpha", C.c_float * MAX_POST_OPS), ("beta", C.c_float * MAX_POST_OPS)]
+
+    @classmethod
+    def of(cls, ops):
+        """ops: [(code, alpha, beta)]"""
+        p = cls()
+        p.count = len(ops)
+        for i, (o, a, b) in enumerate(ops[:MAX_POST_OPS]):
+            p.op[i], p.alpha[i], p.beta[i] = o, a, b
+        return p
 
 
 class GemmF32Desc(C.Structure):
@@ -29,7 +44,7 @@ class GemmF32Desc(C.Structure):
                 ("lda", C.c_int32), ("ldb", C.c_int32), ("ldy", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float),
                 ("A", C.c_void_p), ("B", C.c_void_p), ("C", C.c_void_p), ("bias_mode", C.c_int32), ("act", C.c_int32),
                 ("act_alpha", C.c_float), ("Y", C.c_void_p), ("batch", C.c_int32), ("strideA", C.c_int64),
-                ("strideB", C.c_int64), ("strideC", C.c_int64), ("strideY", C.c_int64)]
+                ("strideB", C.c_int64), ("strideC", C.c_int64), ("strideY", C.c_int64), ("post", C.POINTER(PostOps))]
 
 
 class GemmI8Desc(C.Structure):
@@ -94,7 +109,8 @@ SYMBOLS = {
     "sofie_hip_dequantize_linear_i32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_float]),
     "sofie_hip_unary_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_int32, C.c_float]),
     "sofie_hip_add_f32": (C.c_int, [_P, C.POINTER(AddDesc)]),
-    "sofie_hip_conv_f32": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P, _P, C.c_int32, C.c_float, _P]),
+    "sofie_hip_conv_f32": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P, _P, C.c_int32, C.c_float, _P, C.POINTER(PostOps)]),
+    "sofie_hip_unary_chain_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.POINTER(PostOps)]),
     "sofie_hip_conv_i8": (C.c_int, [_P, C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
     "sofie_hip_conv_i8_workspace": (C.c_size_t, [C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
     "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),

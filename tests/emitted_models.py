@@ -184,6 +184,31 @@ def dynamic_matmul_batched():
                 outputs=[("Y", np.float32, ["N", 4, 6])], init={})
 
 
+def elementwise_chains(batch=6):
+    """One-to-one operators behind a Gemm, behind a Conv and behind a graph input: the generator folds them into the
+    producer's store (its own activation + at most four further links) or into one pass over the data."""
+    W = (util.normal(7401, 20 * 12) * np.float32(0.3)).reshape(20, 12)
+    B = util.normal(7402, 12) * np.float32(0.1)
+    Wc = (util.normal(7403, 5 * 3 * 9) * np.float32(0.2)).reshape(5, 3, 3, 3)
+    init = {"W": W, "B": B, "Wc": Wc, "lo": np.array(0.5, np.float32), "hi": np.array(3.0, np.float32)}
+    nodes = [
+        # Gemm -> LeakyRelu (the Gemm's activation) -> Exp -> Clip -> Sqrt -> Log (four links) -> Neg (one more pass)
+        ow.node("Gemm", ["X", "W", "B"], ["g0"]), ow.node("LeakyRelu", ["g0"], ["g1"], alpha=0.1), ow.node("Exp", ["g1"], ["g2"]),
+        ow.node("Clip", ["g2", "lo", "hi"], ["g3"]), ow.node("Sqrt", ["g3"], ["g4"]), ow.node("Log", ["g4"], ["g5"]),
+        ow.node("Neg", ["g5"], ["Y"]),
+        # Conv -> Tanh -> Abs -> Softplus -> Reciprocal
+        ow.node("Conv", ["I", "Wc"], ["c0"], kernel_shape=[3, 3], pads=[1, 1, 1, 1]), ow.node("Tanh", ["c0"], ["c1"]),
+        ow.node("Abs", ["c1"], ["c2"]), ow.node("Softplus", ["c2"], ["c3"]), ow.node("Reciprocal", ["c3"], ["Z"]),
+        # a graph input through Sin -> Exp -> Atan -> Floor -> Identity -> Asinh: one chain of four, then one of two
+        ow.node("Sin", ["X"], ["s0"]), ow.node("Exp", ["s0"], ["s1"]), ow.node("Atan", ["s1"], ["s2"]), ow.node("Floor", ["s2"], ["s3"]),
+        ow.node("Identity", ["s3"], ["s4"]), ow.node("Asinh", ["s4"], ["V"]),
+    ]
+    X = util.normal(7404, batch * 20).reshape(batch, 20)
+    I = util.normal(7405, 2 * 3 * 6 * 6).reshape(2, 3, 6, 6)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 20]), ("I", np.float32, [2, 3, 6, 6])],
+                outputs=[("Y", np.float32, [batch, 12]), ("Z", np.float32, [2, 5, 6, 6]), ("V", np.float32, [batch, 20])], init=init, feeds=[X, I])
+
+
 DYNAMIC_MODELS = {
     "DynamicLinear": dynamic_linear,
     "DynamicMatMulBatched": dynamic_matmul_batched,
@@ -328,6 +353,34 @@ extern "C" unsigned long pool_bytes(void *s) { return static_cast<Session *>(s)-
 '''
 
 
+# a model with several float outputs: infer returns std::vector<std::vector<float>>, handed back concatenated
+MULTI_OUTPUT_HARNESS = r'''
+#include "%(model)s_GPU_HIP.hxx"
+#include <cstring>
+extern "C" int run_model(const char *weights, const float *const *inputs, float *output, unsigned long output_len, char *err, int errlen)
+{
+   try {
+      SOFIE_%(model)s::Session s(weights);
+      auto ys = s.infer(%(args)s);
+      unsigned long at = 0;
+      for (auto &y : ys) {
+         if (at + y.size() > output_len)
+            throw std::runtime_error("outputs have more elements than expected");
+         std::memcpy(output + at, y.data(), y.size() * sizeof(float));
+         at += y.size();
+      }
+      if (at != output_len)
+         throw std::runtime_error("outputs have " + std::to_string(at) + " elements");
+      return 0;
+   } catch (const std::exception &e) {
+      std::strncpy(err, e.what(), errlen - 1);
+      err[errlen - 1] = 0;
+      return 1;
+   }
+}
+'''
+
+
 def _run(cmd):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
@@ -386,6 +439,14 @@ def build_all(jobs=8):
         p = os.path.join(OUT, m + ".onnx")
         ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)
         dynamic.append((m, p, len(spec["inputs"])))
+    spec = elementwise_chains()
+    p = os.path.join(OUT, "ElementwiseChains.onnx")
+    ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name="ElementwiseChains")
+    _run([EMIT, p, OUT])
+    src = os.path.join(OUT, "ElementwiseChains_harness.cxx")
+    with open(src, "w") as f:
+        f.write(MULTI_OUTPUT_HARNESS % dict(model="ElementwiseChains", args="inputs[0], inputs[1]"))
+    compile_shared(src, os.path.join(OUT, "libElementwiseChains.so"))
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(lambda w: emit_and_compile(*w), work))
         list(ex.map(lambda w: emit_and_compile_dynamic(*w), dynamic))
@@ -395,7 +456,7 @@ def build_all(jobs=8):
     for m in API_MODELS:
         compile_harness(m, 1)
     compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
-    return [w[0] for w in work] + list(API_MODELS)
+    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains"]
 
 
 if __name__ == "__main__":

@@ -87,6 +87,9 @@ class OracleBackend:
     def unary(self, x, act, alpha):
         return self.ob.unary(x, act, alpha)
 
+    def chain(self, x, ops):
+        return self.ob.unary_chain(x, ops)
+
     def conv(self, X, W, b, geo):
         return self.ob.conv_f32(X, W, b, pads=geo["pads"], strides=geo["strides"], dils=geo["dils"], group=geo["group"])
 
@@ -133,6 +136,17 @@ class HipBackend:
         self.rt.sync()
         return u.to_host(dy)
 
+    def chain(self, x, ops):
+        from sofie_amd.runtime import PostOps
+        u = self.u
+        dx = u.to_dev(np.ascontiguousarray(x, dtype=np.float32))
+        dy = u.dev_empty(x.shape, np.float32)
+        import torch
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_unary_chain_f32", u.ptr(dy), u.ptr(dx), C.c_size_t(x.size), C.byref(PostOps.of(ops)))
+        self.rt.sync()
+        return u.to_host(dy)
+
     def conv(self, X, W, b, geo):
         from oracle.binding import conv_out_hw
         R, u = self.R, self.u
@@ -149,7 +163,7 @@ class HipBackend:
         dY = u.dev_empty((N, Cout, OH, OW), np.float32)
         import torch
         torch.cuda.synchronize()
-        self.rt.call("sofie_hip_conv_f32", C.byref(d), u.ptr(dX), u.ptr(dW), u.ptr(db), 0, C.c_float(0), u.ptr(dY))
+        self.rt.call("sofie_hip_conv_f32", C.byref(d), u.ptr(dX), u.ptr(dW), u.ptr(db), 0, C.c_float(0), u.ptr(dY), None)
         self.rt.sync()
         return u.to_host(dY)
 
@@ -187,7 +201,12 @@ class HipBackend:
         return u.to_host(dY)
 
 
-def run(g, inputs, be):
+# codes of include/sofie_hip.h for the reference's basic unary operators
+BASIC_UNARY = {"Reciprocal": 7, "Sqrt": 8, "Neg": 9, "Exp": 10, "Log": 11, "Sin": 12, "Cos": 13, "Abs": 14, "Softplus": 15, "Atan": 16,
+               "Floor": 17, "Asinh": 18, "Acosh": 19, "Atanh": 20}
+
+
+def run(g, inputs, be, all_outputs=False):
     env = dict(g["initializers"])
     for (name, _), a in zip(g["inputs"], inputs):
         env[name] = a
@@ -203,6 +222,14 @@ def run(g, inputs, be):
             y = be.unary(x[0], 2, a.get("alpha", 0.01))
         elif op == "Gelu":
             y = be.unary(x[0], 5 if a.get("approximate", "none") == "tanh" else 4, 0.0)
+        elif op in BASIC_UNARY:
+            y = be.unary(x[0], BASIC_UNARY[op], 0.0)
+        elif op == "Identity":
+            y = np.array(x[0], copy=True)
+        elif op == "Clip":
+            lo = float(np.asarray(x[1]).ravel()[0]) if len(x) > 1 and x[1] is not None else a.get("min", float(np.finfo(np.float32).min))
+            hi = float(np.asarray(x[2]).ravel()[0]) if len(x) > 2 and x[2] is not None else a.get("max", float(np.finfo(np.float32).max))
+            y = be.chain(x[0], [(21, lo, hi)])
         elif op == "Conv":
             X, W = x[0], x[1]
             b = x[2] if len(x) > 2 else None
@@ -223,4 +250,6 @@ def run(g, inputs, be):
         else:
             raise NotImplementedError(op)
         env[n["outputs"][0]] = y
+    if all_outputs:
+        return [env[o[0]] for o in g["outputs"]]
     return env[g["outputs"][0][0]]

@@ -263,6 +263,29 @@ def test_view_based_infer_binds_the_callers_memory(emitted):
     assert "void infer(std::span<ViewConstF1D const> inputs, std::span<ViewF1D> outputs, std::size_t N)" in txt
 
 
+def test_one_to_one_operators_join_their_producer(emitted, tmp_path):
+    body = ops_body(read(emitted, "ElementwiseChains"))
+    # Gemm: LeakyRelu is its activation, Exp/Clip/Sqrt/Log ride in its store, the sixth operator is a pass of its own
+    assert "d.act = SOFIE_ACT_LEAKYRELU" in body
+    assert "sofie_post_ops post{4, {SOFIE_ACT_EXP, SOFIE_ACT_CLIP, SOFIE_ACT_SQRT, SOFIE_ACT_LOG}, {0.0f, 0.5f, 0.0f, 0.0f}, {0.0f, 3.0f, 0.0f, 0.0f}}; d.post = &post;" in body
+    assert "sofie_hip_unary_f32(fCtx, tensor_Y, tensor_g5, 72, SOFIE_ACT_NEG" in body
+    # Conv: Tanh + three links
+    assert "sofie_post_ops post{3, {SOFIE_ACT_ABS, SOFIE_ACT_SOFTPLUS, SOFIE_ACT_RECIPROCAL, SOFIE_ACT_NONE}" in body
+    assert "SOFIE_ACT_TANH, 0.0f, tensor_Z, &post)" in body
+    # no producer to join: chains of at most four in one pass each
+    assert "sofie_post_ops ops{4, {SOFIE_ACT_SIN, SOFIE_ACT_EXP, SOFIE_ACT_ATAN, SOFIE_ACT_FLOOR}" in body
+    # the chain of the reference's custom-memory model (Gemm -> Relu -> Sigmoid -> Tanh) is one launch
+    body = ops_body(read(emitted, "CustomMemoryChain"))
+    assert body.count("detail::Check(") == 1 and "sofie_post_ops post{2, {SOFIE_ACT_SIGMOID, SOFIE_ACT_TANH" in body
+    # a graph output in the middle of a chain stops the folding there
+    nodes = [ow.node("Gemm", ["X", "W"], ["G"]), ow.node("Relu", ["G"], ["R"]), ow.node("Exp", ["R"], ["Y"])]
+    r = _emit(tmp_path, nodes, [("X", np.float32, [2, 3])], [("R", np.float32, [2, 4]), ("Y", np.float32, [2, 4])], {"W": np.ones((3, 4), np.float32)})
+    assert r.returncode == 0, r.stdout
+    txt = open(os.path.join(str(tmp_path), [f for f in os.listdir(str(tmp_path)) if f.endswith(".hxx")][0])).read()
+    body = ops_body(txt)
+    assert "d.act = SOFIE_ACT_RELU" in body and "d.post" not in body and "SOFIE_ACT_EXP" in body and body.count("detail::Check(") == 2
+
+
 def test_asymmetric_zero_point_is_refused(tmp_path):
     init = {"W": np.ones((4, 3, 1, 1), dtype=np.int8), "s": np.array(0.5, dtype=np.float32), "z": np.zeros((), dtype=np.int8),
             "z1": np.array(3, dtype=np.int8), "sx": np.array(0.1, dtype=np.float32)}

@@ -205,3 +205,18 @@ def test_infer_on_views_of_device_memory_equals_infer_on_host_pointers(rt, model
     rc = lib.run_model_views(weights, ptrs, lens, len(arrs), got.ctypes.data_as(ctypes.c_void_p), ctypes.c_ulong(out_len), misalign, err, 1024)
     assert rc == 0, err.value.decode()
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32)) and np.abs(want).max() > 0
+
+
+def test_emitted_elementwise_chains(rt):
+    """One-to-one operators folded behind a Gemm, behind a Conv and behind one another (the reference's elementwise fusion,
+    core/inc/SOFIE/operators/ROperator_ALPAKA.hxx:57-76), against the same operators run one by one on the CPU."""
+    spec = em.elementwise_chains()
+    g = onnx_lite.load(os.path.join(em.OUT, "ElementwiseChains.onnx"))
+    want = np.concatenate([w.ravel() for w in gr.run(g, spec["feeds"], gr.OracleBackend(), all_outputs=True)])
+    print("emitted ElementwiseChains", flush=True)
+    got = run_emitted("ElementwiseChains", spec["feeds"], want.size)
+    assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(1.0, np.abs(want)))
+    txt = open(os.path.join(em.OUT, "ElementwiseChains_GPU_HIP.hxx")).read()
+    body = txt[txt.index("void doInfer("):txt.index("void infer_nosync(")]
+    # 18 operators in the graph, 5 launches
+    assert body.count("detail::Check(") == 5 and body.count("sofie_hip_unary_chain_f32") == 2 and body.count("sofie_hip_unary_f32") == 1

@@ -162,7 +162,7 @@ def test_conv_f32(rt, case, with_bias, act):
     db = None if b is None else util.to_dev(b)
     dY = util.dev_empty((N, Cout, d.OH, d.OW), np.float32)
     print("conv_f32", case, flush=True)
-    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(dX), util.ptr(dW), util.ptr(db), act, C.c_float(0), util.ptr(dY))
+    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(dX), util.ptr(dW), util.ptr(db), act, C.c_float(0), util.ptr(dY), None)
     rt.sync()
     want = ob.conv_f32(X, Wt, b, pads=pads, strides=strides, dils=dils, group=group, act=act)
     assert np.allclose(util.to_host(dY), want, rtol=1e-5, atol=1e-5)
@@ -194,3 +194,107 @@ def test_batchnorm_same_three_roundings_as_the_cpu_loop(rt, shape, relu):
             int(np.prod(shape[2:])), relu)
     rt.sync()
     assert np.array_equal(util.to_host(dY).view(np.uint32), want.view(np.uint32))
+
+
+# ---- the other one-to-one operators and chains of them -------------------------------------------------------
+
+def unary_domain(code, n, seed):
+    """Inputs inside each operator's domain, away from its singularities."""
+    u = util.uniform01(seed, n)
+    z = util.normal(seed + 1, n, 2.0)
+    return {R.ACT_RECIPROCAL: np.where(z >= 0, 0.1 + np.abs(z), -0.1 - np.abs(z)), R.ACT_SQRT: u * 9, R.ACT_LOG: 0.01 + u * 50,
+            R.ACT_ACOSH: 1 + u * 20, R.ACT_ATANH: (u - 0.5) * 1.9, R.ACT_EXP: z * 1.5, R.ACT_SOFTPLUS: z * 12}.get(code, z).astype(np.float32)
+
+
+BASIC_UNARY = [R.ACT_RECIPROCAL, R.ACT_SQRT, R.ACT_NEG, R.ACT_EXP, R.ACT_LOG, R.ACT_SIN, R.ACT_COS, R.ACT_ABS, R.ACT_SOFTPLUS, R.ACT_ATAN,
+               R.ACT_FLOOR, R.ACT_ASINH, R.ACT_ACOSH, R.ACT_ATANH]
+
+
+@pytest.mark.parametrize("code", BASIC_UNARY)
+@pytest.mark.parametrize("n", [5, 4096 + 3])
+def test_basic_unary_operators(rt, code, n):
+    x = unary_domain(code, n, 300 + code)
+    dx = util.to_dev(x)
+    dy = util.dev_empty((n,), np.float32)
+    rt.call("sofie_hip_unary_f32", util.ptr(dy), util.ptr(dx), C.c_size_t(n), code, C.c_float(0))
+    rt.sync()
+    want = ob.unary(x, code, 0.0)
+    got = util.to_host(dy)
+    assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(1.0, np.abs(want)))
+    if code in (R.ACT_NEG, R.ACT_ABS, R.ACT_FLOOR, R.ACT_SQRT, R.ACT_RECIPROCAL):     # correctly rounded on both sides
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def run_chain(rt, x, ops):
+    dx = util.to_dev(x)
+    dy = util.dev_empty(x.shape, np.float32)
+    rt.call("sofie_hip_unary_chain_f32", util.ptr(dy), util.ptr(dx), C.c_size_t(x.size), C.byref(R.PostOps.of(ops)))
+    rt.sync()
+    return util.to_host(dy)
+
+
+def test_unary_chain_is_the_composition(rt):
+    x = util.normal(400, 1000 + 3, 2.0)
+    ops = [(R.ACT_LEAKYRELU, 0.1, 0.0), (R.ACT_EXP, 0.0, 0.0), (R.ACT_CLIP, 0.5, 3.0), (R.ACT_LOG, 0.0, 0.0)]
+    got = run_chain(rt, x, ops)
+    want = ob.unary_chain(x, ops)
+    assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(1.0, np.abs(want)))
+    assert want.min() >= np.log(np.float32(0.5)) - 1e-6 and want.max() <= np.log(np.float32(3.0)) + 1e-6
+    # Clip alone is exact, bounds included; an empty chain and a chain of NONE copy
+    clip = run_chain(rt, x, [(R.ACT_CLIP, -0.25, 0.75)])
+    assert np.array_equal(clip, np.maximum(np.float32(-0.25), np.minimum(np.float32(0.75), x)))
+    assert np.array_equal(run_chain(rt, x, []), x) and np.array_equal(run_chain(rt, x, [(R.ACT_NONE, 0, 0)] * 4), x)
+
+
+def test_chain_errors(rt):
+    x = util.to_dev(np.zeros(8, np.float32))
+    bad = R.PostOps.of([(R.ACT_RELU, 0, 0)])
+    bad.count = 5
+    with pytest.raises(R.SofieHipError, match="more than 4"):
+        rt.call("sofie_hip_unary_chain_f32", util.ptr(x), util.ptr(x), C.c_size_t(8), C.byref(bad))
+    with pytest.raises(R.SofieHipError, match="unknown operator 22"):
+        rt.call("sofie_hip_unary_chain_f32", util.ptr(x), util.ptr(x), C.c_size_t(8), C.byref(R.PostOps.of([(22, 0, 0)])))
+    with pytest.raises(R.SofieHipError, match="NULL"):
+        rt.call("sofie_hip_unary_chain_f32", util.ptr(x), util.ptr(x), C.c_size_t(8), None)
+
+
+@pytest.mark.parametrize("kernel", ["tiles64", "wave8x8"])
+@pytest.mark.parametrize("M,N,K", [(6, 12, 20), (70, 33, 129)])
+def test_gemm_with_a_chain_in_its_store(rt, M, N, K, kernel, monkeypatch):
+    monkeypatch.setenv("SOFIE_HIP_F32_SKINNY", "1" if kernel == "wave8x8" else "0")
+    A = util.normal(410, M * K).reshape(M, K)
+    B = util.normal(411, K * N, 0.1).reshape(K, N)
+    bias = util.normal(412, N)
+    ops = [(R.ACT_SIGMOID, 0, 0), (R.ACT_TANH, 0, 0), (R.ACT_CLIP, 0.2, 0.6), (R.ACT_SQRT, 0, 0)]
+    dA, dB, dC = util.to_dev(A), util.to_dev(B), util.to_dev(bias)
+    dY = util.dev_empty((M, N), np.float32)
+    post = R.PostOps.of(ops)
+    d = R.GemmF32Desc()
+    d.M, d.N, d.K, d.alpha, d.beta, d.batch = M, N, K, 1.0, 1.0, 1
+    d.A, d.B, d.C, d.Y = util.ptr(dA), util.ptr(dB), util.ptr(dC), util.ptr(dY)
+    d.bias_mode, d.act, d.act_alpha = R.BIAS_ROW, R.ACT_LEAKYRELU, 0.1
+    d.post = C.pointer(post)
+    print("gemm_f32 with post ops", M, N, K, kernel, flush=True)
+    rt.call("sofie_hip_gemm_f32", C.byref(d))
+    rt.sync()
+    lin = ob.gemm_f32(A, B, bias, M=M, N=N, K=K, bias_mode=1, act=R.ACT_LEAKYRELU, act_alpha=0.1)
+    want = ob.unary_chain(lin, ops)
+    got = util.to_host(dY)
+    # the chain is a contraction here (sigmoid, tanh), so the GEMM's summation-order freedom stays below 1e-5 absolute
+    assert np.abs(got - want).max() <= 1e-5 and want.std() > 0.01
+
+
+def test_conv_with_a_chain_in_its_store(rt):
+    N, Cc, H, W, Cout = 2, 3, 9, 7, 5
+    X = util.uniform01(420, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.normal(421, Cout * Cc * 9, 0.3).reshape(Cout, Cc, 3, 3)
+    b = util.normal(422, Cout)
+    ops = [(R.ACT_ABS, 0, 0), (R.ACT_SOFTPLUS, 0, 0), (R.ACT_RECIPROCAL, 0, 0)]
+    d = conv_desc(N, Cc, H, W, Cout, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1)
+    dX, dW, db = util.to_dev(X), util.to_dev(Wt), util.to_dev(b)
+    dY = util.dev_empty((N, Cout, d.OH, d.OW), np.float32)
+    post = R.PostOps.of(ops)
+    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(dX), util.ptr(dW), util.ptr(db), R.ACT_TANH, C.c_float(0), util.ptr(dY), C.byref(post))
+    rt.sync()
+    want = ob.unary_chain(ob.conv_f32(X, Wt, b, pads=(1, 1, 1, 1), strides=(1, 1), dils=(1, 1), group=1, act=R.ACT_TANH), ops)
+    assert np.abs(util.to_host(dY) - want).max() <= 1e-5 and want.std() > 0.01

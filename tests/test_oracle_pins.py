@@ -306,3 +306,52 @@ def test_batchnorm_closed_forms():
     assert np.allclose(fused, gamma / np.sqrt(var + np.float32(1e-3)), rtol=1e-6)
     yr, _ = ob.batchnorm(X, gamma, beta, mean, var, eps=1e-3, relu=1)
     assert np.array_equal(yr, np.where(y > 0, y, np.float32(0)))
+
+
+# ---- the other one-to-one operators: pinned by numpy's routines and by identities ----------------------------
+
+def test_basic_unary_operators_against_library_routines_and_identities():
+    """Codes 7..21 (ROperator_BasicUnary.hxx:17-103, ROperator_Clip.hxx:18).  numpy's float32 routines are an independent
+    implementation; the identities catch a swapped code (exp for log, sin for cos, asinh for acosh ...)."""
+    from tests import util
+    z = util.normal(501, 4000, 2.0)
+    u = util.uniform01(502, 4000)
+    pos = (0.01 + 50 * u).astype(np.float32)
+    lib = {7: (np.where(z >= 0, 0.1 + np.abs(z), -0.1 - np.abs(z)).astype(np.float32), lambda x: np.float32(1) / x), 8: (9 * u, np.sqrt),
+           9: (z, np.negative), 10: (z, np.exp), 11: (pos, np.log), 12: (z, np.sin), 13: (z, np.cos), 14: (z, np.abs),
+           15: (12 * z, lambda x: np.where(x >= 20, x, np.log1p(np.exp(x.astype(np.float64))))), 16: (z, np.arctan), 17: (3 * z, np.floor),
+           18: (z, np.arcsinh), 19: ((1 + 20 * u).astype(np.float32), np.arccosh), 20: (((u - 0.5) * 1.9).astype(np.float32), np.arctanh)}
+    for code, (x, f) in lib.items():
+        x = x.astype(np.float32)
+        got = ob.unary(x, code, 0.0)
+        want = f(x.astype(np.float64) if code not in (7,) else x).astype(np.float64)
+        assert np.all(np.abs(got - want) <= 2e-6 * np.maximum(1.0, np.abs(want))), code
+    # identities
+    assert np.allclose(ob.unary(ob.unary(pos, 11, 0), 10, 0), pos, rtol=2e-5)                     # exp(log x) = x
+    s, c = ob.unary(z, 12, 0).astype(np.float64), ob.unary(z, 13, 0).astype(np.float64)
+    assert np.allclose(s * s + c * c, 1.0, atol=1e-6)                                               # sin^2 + cos^2 = 1
+    assert np.allclose(np.sinh(ob.unary(z, 18, 0).astype(np.float64)), z, rtol=1e-5, atol=1e-6)     # sinh(asinh x) = x
+    big = (1 + 20 * u).astype(np.float32)
+    assert np.allclose(np.cosh(ob.unary(big, 19, 0).astype(np.float64)), big, rtol=1e-5)            # cosh(acosh x) = x
+    assert np.allclose(np.tan(ob.unary(z, 16, 0).astype(np.float64)), z, rtol=1e-5, atol=1e-6)      # tan(atan x) = x
+    assert np.array_equal(ob.unary(np.array([25.0, 20.0], np.float32), 15, 0), np.array([25.0, 20.0], np.float32))  # softplus: identity from 20 on
+    assert abs(float(ob.unary(np.array([0.0], np.float32), 15, 0)[0]) - np.log(2.0)) < 1e-7
+    # Clip: the lower bound wins when the bounds cross (max(lo, min(hi, x))), bounds are attained exactly
+    x = np.array([-2, -0.25, 0, 0.75, 3], np.float32)
+    assert np.array_equal(ob.unary_chain(x, [(21, -0.25, 0.75)]), np.array([-0.25, -0.25, 0, 0.75, 0.75], np.float32))
+    assert np.array_equal(ob.unary_chain(x, [(21, 1.0, 0.5)]), np.full(5, 1.0, np.float32))
+
+
+def test_unary_chain_is_applied_left_to_right():
+    from tests import util
+    x = util.normal(503, 100, 1.0)
+    ops = [(2, 0.1, 0.0), (10, 0.0, 0.0), (21, 0.5, 3.0), (11, 0.0, 0.0)]          # LeakyRelu, Exp, Clip, Log
+    want = x.copy()
+    for o in ops:
+        want = ob.unary_chain(want, [o])
+    assert np.array_equal(ob.unary_chain(x, ops), want)
+    ref = np.log(np.clip(np.exp(np.where(x >= 0, x, np.float32(0.1) * x).astype(np.float64)), 0.5, 3.0))
+    assert np.allclose(want, ref, rtol=1e-5, atol=1e-6)
+    # not commutative: the reverse order gives something else
+    assert not np.allclose(ob.unary_chain(x, ops[::-1]), want, equal_nan=True)
+    assert np.array_equal(ob.unary_chain(x, []), x)
