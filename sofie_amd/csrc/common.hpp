@@ -47,7 +47,7 @@ inline int launch_status(const char *what)
 // ---- scalar formulas shared by every epilogue --------------------------------------------------
 
 // Activation on fp32, the reference's CPU formulas (see sofie_hip.h for the citations).
-__device__ __forceinline__ float apply_act(float v, int act, float alpha, float beta = 0.0f)
+__device__ __forceinline__ float apply_activation(float v, int act, float alpha)
 {
    switch (act) {
    case SOFIE_ACT_RELU: return (v > 0.0f) ? v : 0.0f;
@@ -56,6 +56,15 @@ __device__ __forceinline__ float apply_act(float v, int act, float alpha, float 
    case SOFIE_ACT_GELU: return 0.5f * v * (1.0f + erff(v * 0.7071067811865475f));
    case SOFIE_ACT_GELU_TANH: return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
    case SOFIE_ACT_TANH: return tanhf(v);
+   default: return v;
+   }
+}
+
+// The other one-to-one operators (codes above SOFIE_ACT_TANH).  Kept out of line: the kernels that carry an
+// epilogue stay as small as they were with the six activations, and pay a call only when a model uses these.
+static __device__ __noinline__ float apply_basic_unary(float v, int act, float alpha, float beta)
+{
+   switch (act) {
    case SOFIE_ACT_RECIPROCAL: return 1.0f / v;
    case SOFIE_ACT_SQRT: return sqrtf(v);
    case SOFIE_ACT_NEG: return -v;
@@ -75,19 +84,42 @@ __device__ __forceinline__ float apply_act(float v, int act, float alpha, float 
    }
 }
 
+__device__ __forceinline__ float apply_act(float v, int act, float alpha, float beta = 0.0f)
+{
+   return act <= SOFIE_ACT_TANH ? apply_activation(v, act, alpha) : apply_basic_unary(v, act, alpha, beta);
+}
+
 // An operator's own activation followed by the caller's chain of one-to-one operators, by value in the kernel
-// arguments; `count` is the same for every lane, so the loop does not diverge.
+// arguments.  The links are named fields, not arrays: every access has a fixed offset, so the chain stays in
+// scalar registers (an array indexed by a loop counter would be copied to private memory).
 struct PostChain {
    int count = 0;
-   int op[SOFIE_MAX_POST_OPS + 1];
-   float alpha[SOFIE_MAX_POST_OPS + 1];
-   float beta[SOFIE_MAX_POST_OPS + 1];
+   int op0 = 0, op1 = 0, op2 = 0, op3 = 0, op4 = 0;
+   float a0 = 0, a1 = 0, a2 = 0, a3 = 0, a4 = 0;
+   float b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0;
 };
+static_assert(SOFIE_MAX_POST_OPS == 4, "PostChain holds the activation and four links");
+
+// links 1..4, out of line (a model with more than one link behind an operator pays one call per element)
+static __device__ __noinline__ float apply_chain_tail(float v, int count, int op1, float a1, float b1, int op2, float a2, float b2, int op3,
+                                               float a3, float b3, int op4, float a4, float b4)
+{
+   v = apply_act(v, op1, a1, b1);
+   if (count > 2)
+      v = apply_act(v, op2, a2, b2);
+   if (count > 3)
+      v = apply_act(v, op3, a3, b3);
+   if (count > 4)
+      v = apply_act(v, op4, a4, b4);
+   return v;
+}
 
 __device__ __forceinline__ float apply_chain(float v, const PostChain &c)
 {
-   for (int i = 0; i < c.count; ++i)
-      v = apply_act(v, c.op[i], c.alpha[i], c.beta[i]);
+   if (c.count > 0)
+      v = apply_act(v, c.op0, c.a0, c.b0);
+   if (c.count > 1)
+      v = apply_chain_tail(v, c.count, c.op1, c.a1, c.b1, c.op2, c.a2, c.b2, c.op3, c.a3, c.b3, c.op4, c.a4, c.b4);
    return v;
 }
 
@@ -95,32 +127,43 @@ __device__ __forceinline__ float apply_chain(float v, const PostChain &c)
 // code, or -1 for a bad count) if anything is out of range.
 inline bool make_post_chain(PostChain &c, int act, float act_alpha, const sofie_post_ops *post, int &bad)
 {
-   c.count = 0;
+   c = PostChain();
+   int ops[SOFIE_MAX_POST_OPS + 1];
+   float al[SOFIE_MAX_POST_OPS + 1], be[SOFIE_MAX_POST_OPS + 1];
+   int n = 0;
    bad = act;
    if (act < SOFIE_ACT_NONE || act > SOFIE_ACT_LAST)
       return false;
    if (act != SOFIE_ACT_NONE) {
-      c.op[0] = act;
-      c.alpha[0] = act_alpha;
-      c.beta[0] = 0.0f;
-      c.count = 1;
+      ops[n] = act;
+      al[n] = act_alpha;
+      be[n] = 0.0f;
+      ++n;
    }
-   if (!post)
-      return true;
-   bad = -1;
-   if (post->count < 0 || post->count > SOFIE_MAX_POST_OPS)
-      return false;
-   for (int i = 0; i < post->count; ++i) {
-      bad = post->op[i];
-      if (post->op[i] < SOFIE_ACT_NONE || post->op[i] > SOFIE_ACT_LAST)
+   if (post) {
+      bad = -1;
+      if (post->count < 0 || post->count > SOFIE_MAX_POST_OPS)
          return false;
-      if (post->op[i] == SOFIE_ACT_NONE)
-         continue;
-      c.op[c.count] = post->op[i];
-      c.alpha[c.count] = post->alpha[i];
-      c.beta[c.count] = post->beta[i];
-      ++c.count;
+      for (int i = 0; i < post->count; ++i) {
+         bad = post->op[i];
+         if (post->op[i] < SOFIE_ACT_NONE || post->op[i] > SOFIE_ACT_LAST)
+            return false;
+         if (post->op[i] == SOFIE_ACT_NONE)
+            continue;
+         ops[n] = post->op[i];
+         al[n] = post->alpha[i];
+         be[n] = post->beta[i];
+         ++n;
+      }
    }
+   for (int i = n; i <= SOFIE_MAX_POST_OPS; ++i) {
+      ops[i] = SOFIE_ACT_NONE;
+      al[i] = be[i] = 0.0f;
+   }
+   c.count = n;
+   c.op0 = ops[0]; c.op1 = ops[1]; c.op2 = ops[2]; c.op3 = ops[3]; c.op4 = ops[4];
+   c.a0 = al[0]; c.a1 = al[1]; c.a2 = al[2]; c.a3 = al[3]; c.a4 = al[4];
+   c.b0 = be[0]; c.b1 = be[1]; c.b2 = be[2]; c.b3 = be[3]; c.b4 = be[4];
    return true;
 }
 

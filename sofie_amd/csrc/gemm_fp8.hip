@@ -113,7 +113,7 @@ struct F8Epilogue {
          v[i] = mul_nofma(a[i], scale);
          if (bias)
             v[i] = v[i] + p.b[4 * q + i];
-         v[i] = (act == SOFIE_ACT_GELU) ? gelu_erf_fast(v[i]) : apply_act(v[i], act, 0.0f);
+         v[i] = (act == SOFIE_ACT_GELU) ? gelu_erf_fast(v[i]) : apply_activation(v[i], act, 0.0f);
       }
       if (OUT == SOFIE_F8OUT_F32) {
 #pragma unroll
