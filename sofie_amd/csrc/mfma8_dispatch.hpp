@@ -75,6 +75,20 @@ static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *
             return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
          return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
       case 128:
+#ifdef SOFIE_HIP_TUNING
+         if (variant == 51)
+            return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 52)
+            return launch_mfma8_dma<MMA, 128, 128, 64, 2, 2, 8, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 53)
+            return launch_mfma8_dma<MMA, 128, 128, 64, 2, 2, 6, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 54)
+            return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI, 4>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 55)
+            return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI, 1>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 56)
+            return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 4, EPI, 4>(stream, A, Bt, M, N, K, lda, ldb, ep);
+#endif
          if (variant == 1 || !k128)
             return launch_mfma8_dma<MMA, 128, 128, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
          return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
