@@ -15,6 +15,14 @@ static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *
       return launch_mfma8_auto<MMA, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile);
    const int tile = pick_tile(M, N, force_tile);
    const bool k128 = (K % 128 == 0);
+   if constexpr (MMA::KSTEP * 2 <= 64) {
+      // Short reductions over many tiles: the 256 x 128 tile with a ring of three slabs fits twice on a CU, and one
+      // workgroup's prologue and store overlap the other's K loop (8192 x 4096 x 512: 829 -> 1019 TOP/s, 8192 x 1024 x 1024:
+      // 1003 -> 1091; no gain from K = 2048 on).  258 asks for it by force.
+      const long long tiles_256x128 = (long long)((M + 255) / 256) * ((N + 127) / 128);
+      if (force_tile == 258 || (!force_tile && variant == 0 && K <= 1024 && N >= 128 && tiles_256x128 >= 512))
+         return launch_mfma8_dma_src<MMA, 256, 128, 64, 2, 2, 3, EPI, 0, RowMajorRows, 2>(stream, RowMajorRows{A, lda}, Bt, M, N, K, ldb, ep);
+   }
    if constexpr (MMA::KSTEP * 2 > 64) {
       // two K-steps per slab are the minimum: a 64-byte K-step needs 128-byte slabs
       if (!k128)
@@ -115,10 +123,15 @@ static int launch_mfma8_conv(hipStream_t stream, const ConvRows &a, int Cg, cons
    const bool pairs = (Cg % 128 == 0);
    int tile = force_tile;
    if (!tile)
-      // Short reductions (a 3x3 convolution over 64 or 128 channels) spend as long in the tile store as in the K loop:
-      // 128 x 128 tiles leave room for two workgroups per CU, so one's store overlaps the other's MFMAs.
-      // 257 = the 256 x 128 tile, by request only.
-      tile = (N > 128 && K > 1536 && tiles(256, 256) >= 256) ? 256 : (N > 64 && tiles(128, 128) >= 192) ? 128 : 64;
+      // Short reductions (a 3x3 convolution over 64 or 128 channels) spend as long in a tile's prologue and store as in its
+      // K loop.  258 = the 256 x 128 tile with a ring of three slabs (72 KB) and 229 registers per lane: two workgroups
+      // share a CU and one's prologue and store overlap the other's MFMAs (measured on 1M rows: K = 576, N = 128
+      // 157 -> 134 us, K = 1152, N = 256 479 -> 355 us; K = 2304 is better off with the 256 x 256 tile, 760 vs 807 us).
+      // 128 x 128 tiles also fit twice.  257 = the 256 x 128 tile with a ring of five, by request only.
+      tile = (N > 128 && K > 1536 && tiles(256, 256) >= 256) ? 256
+             : (N >= 128 && tiles(256, 128) >= 512)          ? 258
+             : (N > 64 && tiles(128, 128) >= 192)            ? 128
+                                                             : 64;
    switch (tile) {
    case 256:
       if (pairs)
@@ -128,6 +141,12 @@ static int launch_mfma8_conv(hipStream_t stream, const ConvRows &a, int Cg, cons
       if (pairs)
          return launch_mfma8_pair_src<MfmaI8, 256, 128, 64, 2, 2, 5, EPI, 0, ConvRows>(stream, a, Wp, M, N, K, K, ep);
       return launch_mfma8_dma_src<MfmaI8, 256, 128, 64, 2, 2, 4, EPI, 0, ConvRows>(stream, a, Wp, M, N, K, K, ep);
+   case 258: return launch_mfma8_dma_src<MfmaI8, 256, 128, 64, 2, 2, 3, EPI, 0, ConvRows, 2>(stream, a, Wp, M, N, K, K, ep);
+#ifdef SOFIE_HIP_TUNING
+   case 259: return launch_mfma8_dma_src<MfmaI8, 256, 128, 64, 2, 2, 4, EPI, 0, ConvRows, 1>(stream, a, Wp, M, N, K, K, ep);
+   case 260: return launch_mfma8_dma_src<MfmaI8, 128, 256, 64, 2, 2, 3, EPI, 0, ConvRows, 2>(stream, a, Wp, M, N, K, K, ep);
+   case 129: return launch_mfma8_dma_src<MfmaI8, 128, 128, 64, 2, 2, 4, EPI, 0, ConvRows, 2>(stream, a, Wp, M, N, K, K, ep);
+#endif
    case 128: return launch_mfma8_dma_src<MfmaI8, 128, 128, 64, 2, 2, 4, EPI, 0, ConvRows>(stream, a, Wp, M, N, K, K, ep);
    case 64: return launch_mfma8_dma_src<MfmaI8, 64, 64, 64, 2, 2, 4, EPI, 0, ConvRows>(stream, a, Wp, M, N, K, K, ep);
    default: return fail(SOFIE_HIP_ERR_INVALID, "conv: unknown tile %d", force_tile);

@@ -202,8 +202,9 @@ static int launch_mfma8(hipStream_t stream, const int8_t *A, const int8_t *Bt, i
 // Tile choice: the largest one that still gives every one of the 256 CUs a workgroup.
 inline int pick_tile(int M, int N, int force_tile)
 {
-   if (force_tile)
+   if (force_tile == 256 || force_tile == 128 || force_tile == 64)
       return force_tile;
+   // any other request (the convolution's extra tile shapes) leaves the plain product to the heuristic
    auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
    // a tile wider than the matrix would spend its matrix-core time on columns that do not exist
    if (N > 128 && tiles(256, 256) >= 256)

@@ -26,8 +26,10 @@ __device__ __forceinline__ void wait_vmcnt()
    __builtin_amdgcn_s_waitcnt((N & 0xf) | ((N >> 4) << 14) | (0x7 << 4) | (0xf << 8));
 }
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(ASRC A, RowMajorRows Bt, int M, int N,
+// OCC: workgroups meant to share a CU (waves per SIMD); 2 halves the register budget to 256 per lane so that one
+// workgroup's tile store overlaps the other's K loop.
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows, int OCC = 1>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64, OCC) void mfma8_gemm_dma_kernel(ASRC A, RowMajorRows Bt, int M, int N,
                                                                                 int K, EPI ep, int tiles_m, int tiles_n, int sw)
 {
    constexpr int NW = WAVES_M * WAVES_N;
@@ -197,7 +199,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_dma_kernel(A
    });
 }
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows>
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows, int OCC = 1>
 static int launch_mfma8_dma_src(hipStream_t stream, const ASRC &a, const int8_t *Bt, int M, int N, int K, int ldb,
                             const EPI &ep)
 {
@@ -210,10 +212,10 @@ static int launch_mfma8_dma_src(hipStream_t stream, const ASRC &a, const int8_t 
    constexpr size_t ring = (size_t)STAGES * (BM + BN) * BK;
    constexpr size_t store = (size_t)WAVES_M * WAVES_N * tile_store_lds_bytes(BN / WAVES_N);
    constexpr size_t smem = ring > store ? ring : store;
-   static_assert(smem <= 160 * 1024, "LDS ring larger than the CU's LDS");
+   static_assert(smem * OCC <= 160 * 1024, "LDS ring larger than the CU's LDS");
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
    RowMajorRows b{Bt, ldb};
-   auto kern = mfma8_gemm_dma_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG, ASRC>;
+   auto kern = mfma8_gemm_dma_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG, ASRC, OCC>;
    static bool configured[64] = {};
    if (int st = configure_lds_once(kern, smem, configured))
       return st;

@@ -97,7 +97,7 @@ def test_global_avg_pool_i8_both_layouts(rt, N, Cc, H, W):
         assert np.array_equal(util.to_host(dY).view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("tile", [256, 257, 128, 64])
+@pytest.mark.parametrize("tile", [256, 257, 258, 128, 64])
 @pytest.mark.parametrize("case", [
     (2, 128, 12, 12, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),      # paired-slab kernels (channels % 128 == 0)
     (3, 64, 11, 9, 96, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),         # 64-byte slabs, ragged Cout

@@ -54,7 +54,7 @@ def test_int32_accumulate_matches_oracle(rt, M, N, K):
     assert np.array_equal(got, (A.astype(np.int64) @ Bt.astype(np.int64).T).astype(np.int32))
 
 
-@pytest.mark.parametrize("tile", [64, 128, 256])
+@pytest.mark.parametrize("tile", [64, 128, 256, 258])     # 258: the 256 x 128 tile that shares a CU with a second workgroup
 @pytest.mark.parametrize("M,N,K", [(300, 520, 1024), (96, 160, 80), (513, 257, 2048 + 48)])
 def test_every_tile_configuration(rt, tile, M, N, K):
     A = util.int8_sym(11, M * K).reshape(M, K)
@@ -172,3 +172,12 @@ def test_full_size_8192_sampled_rows_and_linearity(rt):
     g2 = run_gemm(rt, A2, Bt, M, N, K, transB=1, out=R.I8OUT_I32)
     assert np.array_equal(g, g1 + g2)
     torch.cuda.empty_cache()
+
+
+def test_short_reduction_over_many_tiles_takes_the_shared_cu_tile(rt):
+    """K <= 1024 with at least 512 tiles of 256 x 128: the heuristic's own choice of the two-per-CU tile (ragged M and N)."""
+    M, N, K = 8192 + 37, 2048 + 5, 512
+    A = util.int8_sym(13, M * K).reshape(M, K)
+    Bt = util.int8_sym(14, N * K).reshape(N, K)
+    got = run_gemm(rt, A, Bt, M, N, K, transB=1, out=R.I8OUT_I32)
+    assert np.array_equal(got, ob.matmul_integer(A, Bt, M=M, N=N, K=K, transB=1, omp=True))
