@@ -128,7 +128,7 @@ enum {
  * (core/inc/SOFIE/operators/ROperator_Gemm.hxx:419-741, core/src/utils/SOFIE_common_helpers.cxx:296-332)
  * and, on the alpaka path, blas.gemm / blas.gemmrelu / blas.gemmStridedBatched + GemmBiasAddKernel
  * (ROperator_Gemm.hxx:743-764, 931-1103).
- *   Y[b] = act( alpha * op(A[b]) * op(B[b]) + beta_eff * broadcast(C) ),  b < batch
+ *   Y[b] = post( act( alpha * op(A[b]) * op(B[b]) + beta_eff * broadcast(C) + residual[b] ) ),  b < batch
  * Tensors are row-major as ONNX defines them: op(A) is [M,K], op(B) is [K,N], Y is [M,N].
  * transA: A is stored [K,M]; transB: B is stored [N,K].  beta_eff is 1 for the broadcast cases and
  * `beta` for SOFIE_BIAS_FULL, which is the reference's behaviour (ROperator_Gemm.hxx:580). */
@@ -147,6 +147,9 @@ typedef struct sofie_gemm_f32_desc {
    int32_t batch; /* stacked MatMul count (>=1); strides in elements, 0 = operand shared */
    int64_t strideA, strideB, strideC, strideY;
    const sofie_post_ops *post; /* applied after `act`; NULL = none */
+   /* A tensor of Y's shape (same ldy and strideY) added before `act`: an Add of another activation tensor behind the product
+    * (a residual connection), which the reference runs as a separate ROperator_BasicBinary.  NULL = none. */
+   const float *residual;
 } sofie_gemm_f32_desc;
 int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d);
 
@@ -262,7 +265,8 @@ typedef struct sofie_conv_desc {
 } sofie_conv_desc;
 int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float *X, const float *W,
                        const float *bias /* [Cout] or NULL */, int32_t act, float act_alpha, float *Y,
-                       const sofie_post_ops *post /* applied after `act`; NULL = none */);
+                       const sofie_post_ops *post /* applied after `act`; NULL = none */,
+                       const float *residual /* [N,Cout,OH,OW] added before `act`, or NULL */);
 /* int8 form (no counterpart in the reference): acc = conv_i32(X_i8, W_i8) + bias_i32[co], then by `out`
  *   SOFIE_I8OUT_I8   Y_i8  = sat8(rne(float(acc)*scale[co])), then max(.,0) if relu
  *   SOFIE_I8OUT_F32  Y_f32 = float(acc)*scale[co], then max(.,0) if relu

@@ -27,6 +27,8 @@ struct F32Epilogue {
    int bias_mode;
    long long ldc;
    PostChain chain; // the activation, then the caller's chain of one-to-one operators
+   const float *R;  // tensor of Y's shape added before the activation, or nullptr
+   long long ldr;
 };
 
 __device__ __forceinline__ float f32_epilogue(const F32Epilogue &ep, float acc, int m, int n)
@@ -39,6 +41,8 @@ __device__ __forceinline__ float f32_epilogue(const F32Epilogue &ep, float acc, 
    case SOFIE_BIAS_FULL: v += ep.beta * ep.C[m * ep.ldc + n]; break;
    default: break;
    }
+   if (ep.R)
+      v += ep.R[m * ep.ldr + n];
    return apply_chain(v, ep.chain);
 }
 
@@ -103,6 +107,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmOperandA la, GemmOper
    lb.p += b * strideB;
    if (ep.C)
       ep.C += b * strideC;
+   if (ep.R)
+      ep.R += b * strideY;
    Y += b * strideY;
    const int m0 = blockIdx.x * F32_BM, n0 = blockIdx.y * F32_BN;
    float acc[4][4];
@@ -143,6 +149,8 @@ __global__ __launch_bounds__(64) void gemm_f32_skinny_kernel(GemmOperandA la, Ge
    lb.p += b * strideB;
    if (ep.C)
       ep.C += b * strideC;
+   if (ep.R)
+      ep.R += b * strideY;
    Y += b * strideY;
    const int lane = threadIdx.x;
    const int tm = lane >> 3, tn = lane & 7;
@@ -259,7 +267,7 @@ struct ConvOperandB {
 };
 
 __global__ __launch_bounds__(256) void conv_f32_kernel(ConvOperandA la, const float *Wt, const float *bias, float *Y, int M,
-                                                        int Cout_g, int Kg, int Cg, int Cout, int OHW, PostChain chain)
+                                                        int Cout_g, int Kg, int Cg, int Cout, int OHW, PostChain chain, const float *R)
 {
    const int g = blockIdx.z;
    la.c_first = g * Cg;
@@ -282,7 +290,10 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(ConvOperandA la, const fl
             float v = acc[i][j];
             if (bias)
                v += bias[co];
-            Y[((size_t)img * Cout + co) * OHW + pix] = apply_chain(v, chain);
+            const size_t at = ((size_t)img * Cout + co) * OHW + pix;
+            if (R)
+               v += R[at];
+            Y[at] = apply_chain(v, chain);
          }
       }
    }
@@ -322,6 +333,8 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d)
    ep.C = d->bias_mode == SOFIE_BIAS_NONE ? nullptr : d->C;
    ep.bias_mode = d->bias_mode;
    ep.ldc = N;
+   ep.R = d->residual;
+   ep.ldr = ldy;
    const unsigned gy = (M + F32_BM - 1) / F32_BM, gx = (N + F32_BN - 1) / F32_BN;
    SOFIE_HIP_REQUIRE(gx <= 65535 && d->batch <= 65535, "sofie_hip_gemm_f32: N or batch too large for one launch");
    // few 64x64 tiles: one-wave workgroups with 8x8 tiles reach every CU (SOFIE_HIP_F32_SKINNY=0/1 overrides)
@@ -352,7 +365,7 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d)
 }
 
 int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float *X, const float *W, const float *bias,
-                       int32_t act, float act_alpha, float *Y, const sofie_post_ops *post)
+                       int32_t act, float act_alpha, float *Y, const sofie_post_ops *post, const float *residual)
 {
    SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_conv_f32: NULL argument");
    SOFIE_HIP_REQUIRE(d->N >= 0 && d->C > 0 && d->H > 0 && d->W > 0 && d->Cout > 0 && d->kh > 0 && d->kw > 0,
@@ -382,7 +395,7 @@ int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float
    const unsigned gy = (unsigned)((M + F32_BM - 1) / F32_BM), gx = (Cout_g + F32_BN - 1) / F32_BN;
    SOFIE_HIP_REQUIRE(gx <= 65535 && d->group <= 65535, "sofie_hip_conv_f32: too many channels or groups for one launch");
    hipLaunchKernelGGL(conv_f32_kernel, dim3(gy, gx, (unsigned)d->group), dim3(256), 0, ctx->stream, la, W, bias, Y, (int)M, Cout_g, Kg,
-                      Cg, d->Cout, OH * OW, chain);
+                      Cg, d->Cout, OH * OW, chain, residual);
    return launch_status("conv_f32_kernel");
 }
 

@@ -140,7 +140,27 @@ public:
       fNY = newOutput;
       fOutputTensorNames = {fNY};
    }
+   // see ROperator_Gemm::SetResidual
+   bool HasResidual() const { return !fNR.empty(); }
+   void SetResidual(const std::string &name, const std::string &newOutput)
+   {
+      fNR = UTILITY::Clean_name(name);
+      fInputTensorNames.push_back(fNR);
+      fNY = newOutput;
+      fOutputTensorNames = {fNY};
+   }
+   std::vector<std::size_t> OutputShape() const { return fGeo.OutputShape(); }
+   bool IsBatched() const { return fDynamic; }
+
    void Initialize(RModel &model) override
+   {
+      ResolveShapes(model);
+      if (!fNR.empty() && (!model.CheckIfTensorAlreadyExist(fNR) || model.GetTensorType(fNR) != ETensorType::FLOAT ||
+                           model.GetTensorShape(fNR) != fGeo.OutputShape() || model.IsDynamicTensor(fNR) != fDynamic))
+         throw std::runtime_error("SOFIE Conv Op: residual tensor " + fNR + " does not have the shape of the output");
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fGeo.OutputShape(), fDynamic);
+   }
+   void ResolveShapes(RModel &model)
    {
       if (!model.CheckIfTensorAlreadyExist(fNX))
          throw std::runtime_error("SOFIE Conv op Input Tensor " + fNX + " is not found in model");
@@ -158,7 +178,6 @@ public:
             throw std::runtime_error("SOFIE Conv op " + fNY + " : invalid shape for Bias tensor " + fNB + " : " + ConvertShapeToString(shapeB));
       }
       fDynamic = model.IsDynamicTensor(fNX);
-      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fGeo.OutputShape(), fDynamic);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
@@ -173,7 +192,8 @@ public:
          out << SP << "   " << PostOpsDeclaration("post", fPost) << "\n";
       out << SP << "   " << "detail::Check(sofie_hip_conv_f32(fCtx, &d, tensor_" << fNX << ", tensor_" << fNW << ", "
           << (fNB.empty() ? "nullptr" : "tensor_" + fNB) << ", " << ActivationEnumName(fActivation) << ", " << FloatLiteral(fActAlpha)
-          << ", tensor_" << fNY << ", " << (fPost.empty() ? "nullptr" : "&post") << "), \"" << opName << " Conv\");\n";
+          << ", tensor_" << fNY << ", " << (fPost.empty() ? "nullptr" : "&post") << ", " << (fNR.empty() ? "nullptr" : "tensor_" + fNR) << "), \""
+          << opName << " Conv\");\n";
       out << SP << "}\n";
       return out.str();
    }
@@ -183,7 +203,7 @@ private:
    std::vector<std::size_t> fAttrDilations;
    std::size_t fAttrGroup;
    std::vector<std::size_t> fAttrKernelShape, fAttrPads, fAttrStrides;
-   std::string fNX, fNW, fNB, fNY;
+   std::string fNX, fNW, fNB, fNY, fNR;
    EActivationType fActivation = EActivationType::UNDEFINED;
    float fActAlpha = 0.01f;
    std::vector<PostOp> fPost;

@@ -113,7 +113,29 @@ public:
       fOutputTensorNames = {fNY};
    }
 
+   // A tensor of the product's shape that an Add behind this operator adds to it (a residual connection): it joins
+   // the kernel's store, before the activation.  The generator calls this when the shapes agree (OutputShape below).
+   bool HasResidual() const { return !fNR.empty(); }
+   void SetResidual(const std::string &name, const std::string &newOutput)
+   {
+      fNR = UTILITY::Clean_name(name);
+      fInputTensorNames.push_back(fNR);
+      fNY = newOutput;
+      fOutputTensorNames = {fNY};
+   }
+   const std::vector<std::size_t> &OutputShape() const { return fShapeY; }
+   bool IsBatched() const { return fDynamic; }
+
    void Initialize(RModel &model) override
+   {
+      ResolveShapes(model);
+      if (!fNR.empty() && (!model.CheckIfTensorAlreadyExist(fNR) || model.GetTensorType(fNR) != ETensorType::FLOAT ||
+                           model.GetTensorShape(fNR) != fShapeY || model.IsDynamicTensor(fNR) != fDynamic))
+         throw std::runtime_error("SOFIE Gemm Op: residual tensor " + fNR + " does not have the shape of the product");
+      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShapeY, fDynamic);
+   }
+   // shape inference only (registers nothing): sets M, N, K, the bias mode and OutputShape()
+   void ResolveShapes(RModel &model)
    {
       if (!model.CheckIfTensorAlreadyExist(fNA) || !model.CheckIfTensorAlreadyExist(fNB))
          throw std::runtime_error("SOFIE Gemm Op Input Tensor " + fNA + " or " + fNB + " is not found in model");
@@ -230,7 +252,7 @@ public:
          shapeY.erase(shapeY.end() - 2);
       if (appendOne)
          shapeY.pop_back();
-      model.AddIntermediateTensor(fNY, ETensorType::FLOAT, shapeY, fDynamic);
+      fShapeY = shapeY;
    }
 
    std::string Generate_GPU_HIP(std::string opName) override
@@ -253,6 +275,8 @@ public:
           << fStrideB << "; d.strideC = " << fStrideC << "; d.strideY = " << (fBatch > 1 || fDynamicStack ? fM * fN : 0) << ";\n";
       if (!fPost.empty())
          out << SP << "   " << PostOpsDeclaration("post", fPost) << " d.post = &post;\n";
+      if (!fNR.empty())
+         out << SP << "   " << "d.residual = tensor_" << fNR << ";\n";
       out << SP << "   " << "detail::Check(sofie_hip_gemm_f32(fCtx, &d), \"" << opName << " Gemm\");\n";
       out << SP << "}\n";
       return out.str();
@@ -261,7 +285,8 @@ public:
 private:
    float fAttrAlpha = 1.0, fAttrBeta = 1.0;
    int64_t fAttrTransA = 0, fAttrTransB = 0;
-   std::string fNA, fNB, fNC, fNY;
+   std::string fNA, fNB, fNC, fNY, fNR;
+   std::vector<std::size_t> fShapeY;
    EActivationType fActivation = EActivationType::UNDEFINED;
    float fActAlpha = 0.01f;
    std::vector<PostOp> fPost;

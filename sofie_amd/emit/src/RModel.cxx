@@ -272,6 +272,63 @@ void RModel::FuseGemmActivations()
    }
 }
 
+// Gemm or Conv whose only reader is an Add with a tensor of the same shape that already exists (a graph input, a weight, or
+// the output of an earlier operator): the Add joins the kernel's store, before the activation, and an activation behind the Add
+// can then join as well.  Runs just before operator i is initialised, when the shapes of everything before it are known.
+void RModel::TryFuseResidual(std::size_t i)
+{
+   ROperator *op = fOperators[i].get();
+   auto *g = dynamic_cast<ROperator_Gemm<float> *>(op);
+   auto *c = dynamic_cast<ROperator_Conv<float> *>(op);
+   if ((!g && !c) || op->GetOutputTensorNames().size() != 1)
+      return;
+   if (g ? (g->HasActivation() || g->PostOpCount() || g->HasResidual()) : (c->HasActivation() || c->PostOpCount() || c->HasResidual()))
+      return;
+   const std::string y = op->GetOutputTensorNames()[0];
+   if (IsOutputTensor(y))
+      return;
+   std::size_t reader = fOperators.size(), readers = 0;
+   for (std::size_t j = 0; j < fOperators.size(); ++j)
+      for (auto &in : fOperators[j]->GetInputTensorNames())
+         if (in == y) {
+            reader = j;
+            ++readers;
+         }
+   if (readers != 1 || reader <= i)
+      return;
+   auto *add = dynamic_cast<ROperator_BasicBinary<float, Add> *>(fOperators[reader].get());
+   if (!add)
+      return;
+   const auto &in = add->GetInputTensorNames();
+   const std::string other = in[0] == y ? in[1] : in[0];
+   if (other == y || !CheckIfTensorAlreadyExist(other) || GetTensorType(other) != ETensorType::FLOAT)
+      return;
+   std::vector<std::size_t> shapeY;
+   bool batched = false;
+   try {
+      if (g) {
+         g->ResolveShapes(*this);
+         shapeY = g->OutputShape();
+         batched = g->IsBatched();
+      } else {
+         c->ResolveShapes(*this);
+         shapeY = c->OutputShape();
+         batched = c->IsBatched();
+      }
+   } catch (const std::exception &) {
+      return; // the operator's own Initialize reports the problem
+   }
+   if (GetTensorShape(other) != shapeY || IsDynamicTensor(other) != batched)
+      return; // a broadcasting Add stays an operator of its own
+   const std::string sum = add->GetOutputTensorNames()[0];
+   if (g)
+      g->SetResidual(other, sum);
+   else
+      c->SetResidual(other, sum);
+   fOperators.erase(fOperators.begin() + reader);
+   FuseGemmActivations(); // what followed the Add may now join the same store
+}
+
 bool RModel::IsOutputTensor(const std::string &name) const
 {
    return std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), UTILITY::Clean_name(name)) != fOutputTensorNames.end();
@@ -314,6 +371,7 @@ void RModel::Initialize(int batchSize)
          fInputTensorNames.push_back(kv.first);
    FuseGemmActivations();
    for (std::size_t i = 0; i < fOperators.size(); ++i) {
+      TryFuseResidual(i);
       fOperators[i]->SetOpOrder(i);
       fOperators[i]->Initialize(*this);
       // an operator that reads a batched tensor has to say what it makes of the batch

@@ -83,6 +83,16 @@ int main(int argc, char **argv)
       f8.AddOutputTensorNameList({"Y"});
       f8.GenerateGPU_HIP();
       f8.OutputGenerated(std::string(argv[1]) + "/ApiFp8Gemm_GPU_HIP.hxx");
+      // the same product with the batch left to the Session (maximum given to the constructor, default 48)
+      RModel f8d("ApiDynamicFp8Gemm");
+      f8d.AddInputTensorInfo("X", ETensorType::FLOAT, std::vector<Dim>{Dim(std::string("batch"), 48), Dim(256)});
+      f8d.AddInputTensorName("X");
+      f8d.AddInitializedTensor("W", ETensorType::FLOAT8E4M3FN, {96, 256}, w8.data());
+      f8d.AddInitializedTensor("B", ETensorType::FLOAT, {96}, bias.data());
+      f8d.AddOperator(std::make_unique<ROperator_Fp8Gemm>(0.03125f, 0.0078125f, 1, "X", "W", "B", EActivationType::GELU, ETensorType::FLOAT, "Y"));
+      f8d.AddOutputTensorNameList({"Y"});
+      f8d.GenerateGPU_HIP();
+      f8d.OutputGenerated(std::string(argv[1]) + "/ApiDynamicFp8Gemm_GPU_HIP.hxx");
    } catch (const std::exception &e) {
       std::cerr << "error: " << e.what() << "\n";
       return 1;

@@ -44,7 +44,8 @@ class GemmF32Desc(C.Structure):
                 ("lda", C.c_int32), ("ldb", C.c_int32), ("ldy", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float),
                 ("A", C.c_void_p), ("B", C.c_void_p), ("C", C.c_void_p), ("bias_mode", C.c_int32), ("act", C.c_int32),
                 ("act_alpha", C.c_float), ("Y", C.c_void_p), ("batch", C.c_int32), ("strideA", C.c_int64),
-                ("strideB", C.c_int64), ("strideC", C.c_int64), ("strideY", C.c_int64), ("post", C.POINTER(PostOps))]
+                ("strideB", C.c_int64), ("strideC", C.c_int64), ("strideY", C.c_int64), ("post", C.POINTER(PostOps)),
+                ("residual", C.c_void_p)]
 
 
 class GemmI8Desc(C.Structure):
@@ -109,7 +110,7 @@ SYMBOLS = {
     "sofie_hip_dequantize_linear_i32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_float]),
     "sofie_hip_unary_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_int32, C.c_float]),
     "sofie_hip_add_f32": (C.c_int, [_P, C.POINTER(AddDesc)]),
-    "sofie_hip_conv_f32": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P, _P, C.c_int32, C.c_float, _P, C.POINTER(PostOps)]),
+    "sofie_hip_conv_f32": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P, _P, C.c_int32, C.c_float, _P, C.POINTER(PostOps), _P]),
     "sofie_hip_unary_chain_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.POINTER(PostOps)]),
     "sofie_hip_conv_i8": (C.c_int, [_P, C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
     "sofie_hip_conv_i8_workspace": (C.c_size_t, [C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),

@@ -209,7 +209,34 @@ def elementwise_chains(batch=6):
                 outputs=[("Y", np.float32, [batch, 12]), ("Z", np.float32, [2, 5, 6, 6]), ("V", np.float32, [batch, 20])], init=init, feeds=[X, I])
 
 
-DYNAMIC_MODELS = {
+def dynamic_residual():
+    """Run-time batch through a broadcasting Add: Y = Relu(X * W + Z) + b with X[N,6], Z[N,5] both batched and b[5] broadcast."""
+    W = (util.normal(7501, 6 * 5) * np.float32(0.4)).reshape(6, 5)
+    b = util.normal(7502, 5)
+    nodes = [ow.node("MatMul", ["X", "W"], ["P"]), ow.node("Add", ["P", "Z"], ["S"]), ow.node("Relu", ["S"], ["R"]), ow.node("Add", ["b", "R"], ["Y"])]
+    return dict(nodes=nodes, inputs=[("X", np.float32, ["N", 6]), ("Z", np.float32, ["N", 5])], outputs=[("Y", np.float32, ["N", 5])],
+                init={"W": W, "b": b}, consts=dict(W=W, b=b))
+
+
+def residual_block(batch=2):
+    """Conv -> Add(shortcut) -> Relu -> GlobalAveragePool -> Flatten -> Gemm -> Add(second input) -> Sigmoid: both Adds have
+    operands of equal shape, so each joins the store of the operator before it, ahead of the activation."""
+    Wc = (util.normal(7601, 8 * 8 * 9) * np.float32(0.15)).reshape(8, 8, 3, 3)
+    Bc = util.normal(7602, 8) * np.float32(0.1)
+    W = (util.normal(7603, 8 * 4) * np.float32(0.5)).reshape(8, 4)
+    b = util.normal(7604, 4) * np.float32(0.2)
+    nodes = [ow.node("Conv", ["X", "Wc", "Bc"], ["c0"], kernel_shape=[3, 3], pads=[1, 1, 1, 1]), ow.node("Add", ["c0", "X"], ["s0"]),
+             ow.node("Relu", ["s0"], ["r0"]), ow.node("GlobalAveragePool", ["r0"], ["p"]), ow.node("Flatten", ["p"], ["f"], axis=1),
+             ow.node("Gemm", ["f", "W", "b"], ["g"]), ow.node("Add", ["Z", "g"], ["s1"]), ow.node("Sigmoid", ["s1"], ["Y"])]
+    X = util.normal(7605, batch * 8 * 6 * 6).reshape(batch, 8, 6, 6)
+    Z = util.normal(7606, batch * 4).reshape(batch, 4)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 8, 6, 6]), ("Z", np.float32, [batch, 4])], outputs=[("Y", np.float32, [batch, 4])],
+                init={"Wc": Wc, "Bc": Bc, "W": W, "b": b}, feeds=[X, Z])
+
+
+DYNAMIC_MODELS = {    "Dynamic_ResidualBlock": lambda: with_named_batch(residual_block(2), "N"),
+    "DynamicResidual": dynamic_residual,
+
     "DynamicLinear": dynamic_linear,
     "DynamicMatMulBatched": dynamic_matmul_batched,
     "Dynamic_int8_MLP": lambda: with_named_batch(int8_mlp([64, 128, 96, 32], 48), "batch_size"),
@@ -218,6 +245,7 @@ DYNAMIC_MODELS = {
 }
 
 CONFIG_MODELS = {
+    "ResidualBlock": lambda: residual_block(2),
     "QLinearMatMulRelu": lambda: qlinear_matmul_relu(),
     "ConvIntegerDequantize": lambda: conv_integer_dequantize(),
     "ConvBatchNormRelu": lambda: conv_batchnorm_relu(2),
@@ -455,6 +483,10 @@ def build_all(jobs=8):
     _run([os.path.join(os.path.dirname(EMIT), "sofie_hip_emit_example"), OUT])
     for m in API_MODELS:
         compile_harness(m, 1)
+    src = os.path.join(OUT, "ApiDynamicFp8Gemm_harness.cxx")
+    with open(src, "w") as f:
+        f.write(DYNAMIC_HARNESS % dict(model="ApiDynamicFp8Gemm", args="inputs[0]"))
+    compile_shared(src, os.path.join(OUT, "libApiDynamicFp8Gemm.so"))
     compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
     return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains"]
 

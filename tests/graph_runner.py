@@ -163,7 +163,7 @@ class HipBackend:
         dY = u.dev_empty((N, Cout, OH, OW), np.float32)
         import torch
         torch.cuda.synchronize()
-        self.rt.call("sofie_hip_conv_f32", C.byref(d), u.ptr(dX), u.ptr(dW), u.ptr(db), 0, C.c_float(0), u.ptr(dY), None)
+        self.rt.call("sofie_hip_conv_f32", C.byref(d), u.ptr(dX), u.ptr(dW), u.ptr(db), 0, C.c_float(0), u.ptr(dY), None, None)
         self.rt.sync()
         return u.to_host(dY)
 
@@ -224,6 +224,9 @@ def run(g, inputs, be, all_outputs=False):
             y = be.unary(x[0], 5 if a.get("approximate", "none") == "tanh" else 4, 0.0)
         elif op in BASIC_UNARY:
             y = be.unary(x[0], BASIC_UNARY[op], 0.0)
+        elif op == "Flatten":
+            ax = a.get("axis", 1)
+            y = np.ascontiguousarray(x[0]).reshape(int(np.prod(x[0].shape[:ax], dtype=np.int64)), -1)
         elif op == "Identity":
             y = np.array(x[0], copy=True)
         elif op == "Clip":

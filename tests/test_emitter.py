@@ -271,7 +271,7 @@ def test_one_to_one_operators_join_their_producer(emitted, tmp_path):
     assert "sofie_hip_unary_f32(fCtx, tensor_Y, tensor_g5, 72, SOFIE_ACT_NEG" in body
     # Conv: Tanh + three links
     assert "sofie_post_ops post{3, {SOFIE_ACT_ABS, SOFIE_ACT_SOFTPLUS, SOFIE_ACT_RECIPROCAL, SOFIE_ACT_NONE}" in body
-    assert "SOFIE_ACT_TANH, 0.0f, tensor_Z, &post)" in body
+    assert "SOFIE_ACT_TANH, 0.0f, tensor_Z, &post, nullptr)" in body
     # no producer to join: chains of at most four in one pass each
     assert "sofie_post_ops ops{4, {SOFIE_ACT_SIN, SOFIE_ACT_EXP, SOFIE_ACT_ATAN, SOFIE_ACT_FLOOR}" in body
     # the chain of the reference's custom-memory model (Gemm -> Relu -> Sigmoid -> Tanh) is one launch
@@ -284,6 +284,28 @@ def test_one_to_one_operators_join_their_producer(emitted, tmp_path):
     txt = open(os.path.join(str(tmp_path), [f for f in os.listdir(str(tmp_path)) if f.endswith(".hxx")][0])).read()
     body = ops_body(txt)
     assert "d.act = SOFIE_ACT_RELU" in body and "d.post" not in body and "SOFIE_ACT_EXP" in body and body.count("detail::Check(") == 2
+
+
+def test_equal_shaped_adds_join_the_store_of_their_producer(emitted, tmp_path):
+    body = ops_body(read(emitted, "ResidualBlock"))
+    # 8 operators in the graph, 4 launches: Conv(+Add+Relu), GlobalAveragePool, Flatten, Gemm(+Add+Sigmoid)
+    assert body.count("detail::Check(") == 4 and "sofie_hip_add_f32" not in body and "sofie_hip_unary_f32" not in body
+    assert "SOFIE_ACT_RELU, 0.0f, tensor_r0, nullptr, tensor_X)" in body
+    assert "d.residual = tensor_Z;" in body and "d.act = SOFIE_ACT_SIGMOID" in body
+    # a broadcasting Add (bias-like operand of another shape) and an Add behind an activation stay operators of their own
+    body = ops_body(read(emitted, "DynamicResidual"))
+    assert body.count("sofie_hip_add_f32") == 1 and "d.residual = tensor_Z;" in body and "d.act = SOFIE_ACT_RELU" in body
+    nodes = [ow.node("Gemm", ["X", "W"], ["G"]), ow.node("Relu", ["G"], ["R"]), ow.node("Add", ["R", "Z"], ["Y"])]
+    r = _emit(tmp_path, nodes, [("X", np.float32, [2, 3]), ("Z", np.float32, [2, 4])], [("Y", np.float32, [2, 4])], {"W": np.ones((3, 4), np.float32)})
+    assert r.returncode == 0, r.stdout
+    txt = open(os.path.join(str(tmp_path), "m_GPU_HIP.hxx")).read()
+    assert "d.residual" not in txt and "sofie_hip_add_f32" in txt and "d.act = SOFIE_ACT_RELU" in txt
+    # the other operand must exist before the product runs: here it is computed later, so nothing is folded
+    nodes = [ow.node("Gemm", ["X", "W"], ["G"]), ow.node("Tanh", ["Z"], ["T"]), ow.node("Add", ["G", "T"], ["Y"])]
+    r = _emit(tmp_path, nodes, [("X", np.float32, [2, 3]), ("Z", np.float32, [2, 4])], [("Y", np.float32, [2, 4])], {"W": np.ones((3, 4), np.float32)}, name="late")
+    assert r.returncode == 0, r.stdout
+    txt = open(os.path.join(str(tmp_path), "late_GPU_HIP.hxx")).read()
+    assert "d.residual" not in txt and "sofie_hip_add_f32" in txt
 
 
 def test_asymmetric_zero_point_is_refused(tmp_path):

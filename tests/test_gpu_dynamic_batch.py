@@ -139,3 +139,45 @@ def test_dynamic_conv_batchnorm_relu(rt):
             got = s.infer(n, [x[:n]], want.size)
             w = want[:n].ravel()
             assert got.size == w.size and np.abs(got - w).max() <= 1e-5 * max(1.0, float(np.abs(w).max()))
+
+
+def test_dynamic_batch_through_broadcasting_adds(rt):
+    c = em.dynamic_residual()["consts"]
+    x, z = util.normal(8401, 9 * 6).reshape(9, 6), util.normal(8402, 9 * 5).reshape(9, 5)
+    with DynamicSession("DynamicResidual", 9) as s:
+        for n in (9, 4, 1):
+            want = np.maximum(x[:n].astype(np.float64) @ c["W"].astype(np.float64) + z[:n], 0) + c["b"]
+            got = s.infer(n, [x[:n], z[:n]], 45)
+            assert got.size == n * 5 and np.abs(got.reshape(n, 5) - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
+
+
+def test_dynamic_fp8_gemm_within_the_stated_bound(rt):
+    from oracle import binding as ob
+    K, N = 256, 96
+    s, w8 = 2024, np.empty(N * K, dtype=np.uint8)
+    for i in range(N * K):                      # the code sequence of sofie_amd/emit/tools/emit_example_api.cxx
+        s = (s * 1664525 + 1013904223) & 0xFFFFFFFF
+        w8[i] = (s >> 24) & 0xBE
+    w8 = w8.reshape(N, K)
+    bias = (0.25 * ((np.arange(N) % 7) - 3)).astype(np.float32)
+    x = util.normal(8501, 40 * K).reshape(40, K)
+    xs, wsc = np.float32(0.03125), np.float32(0.0078125)
+    with DynamicSession("ApiDynamicFp8Gemm", 40) as sess:
+        for n in (40, 7):
+            a8 = ob.quantize_fp8(x[:n], xs)
+            want, abs_sum = ob.gemm_fp8(a8, w8, M=n, N=N, K=K, transB=1, bias=bias, scale=np.float32(xs * wsc), act=4, out=1, want_abs_sum=True)
+            got = sess.infer(n, [x[:n]], 40 * N).reshape(n, N)
+            bound = 1.2 * 2.0 ** -14 * abs_sum.astype(np.float64) * float(xs * wsc) + 1e-6     # the bound of the static FP8 test
+            assert np.all(np.abs(got.astype(np.float64) - want) <= bound) and np.abs(want).max() > 0.5
+
+
+def test_dynamic_residual_block(rt):
+    spec = em.residual_block(2)
+    g = onnx_lite.load(os.path.join(em.OUT, "ResidualBlock.onnx"))
+    x = np.concatenate([spec["feeds"][0], util.normal(8601, 3 * 8 * 6 * 6).reshape(3, 8, 6, 6)])
+    z = np.concatenate([spec["feeds"][1], util.normal(8602, 3 * 4).reshape(3, 4)])
+    with DynamicSession("Dynamic_ResidualBlock", 5) as s:
+        for n in (5, 2):
+            want = gr.run(g, [x[:n], z[:n]], gr.OracleBackend()).ravel()
+            got = s.infer(n, [x[:n], z[:n]], 20)
+            assert got.size == want.size == n * 4 and np.abs(got - want).max() <= 1e-5

@@ -220,3 +220,13 @@ def test_emitted_elementwise_chains(rt):
     body = txt[txt.index("void doInfer("):txt.index("void infer_nosync(")]
     # 18 operators in the graph, 5 launches
     assert body.count("detail::Check(") == 5 and body.count("sofie_hip_unary_chain_f32") == 2 and body.count("sofie_hip_unary_f32") == 1
+
+
+def test_emitted_residual_block(rt):
+    """Adds of equal-shaped tensors behind a Conv and a Gemm ride in those operators' stores (tests/emitted_models.residual_block)."""
+    spec = em.residual_block(2)
+    g = onnx_lite.load(os.path.join(em.OUT, "ResidualBlock.onnx"))
+    want = gr.run(g, spec["feeds"], gr.OracleBackend()).ravel()
+    print("emitted ResidualBlock", flush=True)
+    got = run_emitted("ResidualBlock", spec["feeds"], want.size)
+    assert np.abs(got - want).max() <= 1e-5 and want.std() > 0.01

@@ -41,16 +41,16 @@ def test_conv_argument_checks(rt):
     d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1
     d.group, d.OH, d.OW = 1, 4, 4
     X, W, Y = util.to_dev(np.zeros((1, 4, 6, 6), np.float32)), util.to_dev(np.zeros((6, 4, 3, 3), np.float32)), util.dev_empty((1, 6, 4, 4), np.float32)
-    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(X), util.ptr(W), None, 0, C.c_float(0), util.ptr(Y), None)
+    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(X), util.ptr(W), None, 0, C.c_float(0), util.ptr(Y), None, None)
     d.OH = 5                                            # the caller's shape inference disagrees
     with pytest.raises(SofieHipError, match="does not match the descriptor"):
-        rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(X), util.ptr(W), None, 0, C.c_float(0), util.ptr(Y), None)
+        rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(X), util.ptr(W), None, 0, C.c_float(0), util.ptr(Y), None, None)
     d.OH, d.group = 4, 3                                # groups that do not divide the channels
     with pytest.raises(SofieHipError, match="does not divide"):
-        rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(X), util.ptr(W), None, 0, C.c_float(0), util.ptr(Y), None)
+        rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(X), util.ptr(W), None, 0, C.c_float(0), util.ptr(Y), None, None)
     d.group, d.kh = 1, 9                                # kernel larger than the padded image
     with pytest.raises(SofieHipError, match="larger than the padded image"):
-        rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(X), util.ptr(W), None, 0, C.c_float(0), util.ptr(Y), None)
+        rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(X), util.ptr(W), None, 0, C.c_float(0), util.ptr(Y), None, None)
     d.kh = 3
     a = R.ConvI8Args()
     a.X, a.W, a.Y, a.out = util.ptr(X), util.ptr(W), util.ptr(Y), R.I8OUT_I8   # int8 output without a scale

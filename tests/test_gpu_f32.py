@@ -162,7 +162,7 @@ def test_conv_f32(rt, case, with_bias, act):
     db = None if b is None else util.to_dev(b)
     dY = util.dev_empty((N, Cout, d.OH, d.OW), np.float32)
     print("conv_f32", case, flush=True)
-    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(dX), util.ptr(dW), util.ptr(db), act, C.c_float(0), util.ptr(dY), None)
+    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(dX), util.ptr(dW), util.ptr(db), act, C.c_float(0), util.ptr(dY), None, None)
     rt.sync()
     want = ob.conv_f32(X, Wt, b, pads=pads, strides=strides, dils=dils, group=group, act=act)
     assert np.allclose(util.to_host(dY), want, rtol=1e-5, atol=1e-5)
@@ -294,7 +294,51 @@ def test_conv_with_a_chain_in_its_store(rt):
     dX, dW, db = util.to_dev(X), util.to_dev(Wt), util.to_dev(b)
     dY = util.dev_empty((N, Cout, d.OH, d.OW), np.float32)
     post = R.PostOps.of(ops)
-    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(dX), util.ptr(dW), util.ptr(db), R.ACT_TANH, C.c_float(0), util.ptr(dY), C.byref(post))
+    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(dX), util.ptr(dW), util.ptr(db), R.ACT_TANH, C.c_float(0), util.ptr(dY), C.byref(post), None)
     rt.sync()
     want = ob.unary_chain(ob.conv_f32(X, Wt, b, pads=(1, 1, 1, 1), strides=(1, 1), dils=(1, 1), group=1, act=R.ACT_TANH), ops)
     assert np.abs(util.to_host(dY) - want).max() <= 1e-5 and want.std() > 0.01
+
+
+@pytest.mark.parametrize("kernel", ["tiles64", "wave8x8"])
+@pytest.mark.parametrize("M,N,K,batch", [(6, 12, 20, 1), (70, 33, 129, 1), (9, 10, 16, 3)])
+def test_gemm_with_a_residual_operand(rt, M, N, K, batch, kernel, monkeypatch):
+    """Y = act(alpha A B + bias + R): the Add of a same-shaped tensor behind the product, inside the store, before the activation."""
+    monkeypatch.setenv("SOFIE_HIP_F32_SKINNY", "1" if kernel == "wave8x8" else "0")
+    A = util.normal(430, batch * M * K).reshape(batch, M, K)
+    B = util.normal(431, K * N, 0.1).reshape(K, N)
+    bias = util.normal(432, N)
+    Rr = util.normal(433, batch * M * N).reshape(batch, M, N)
+    dA, dB, dC, dR = util.to_dev(A), util.to_dev(B), util.to_dev(bias), util.to_dev(Rr)
+    dY = util.dev_empty((batch, M, N), np.float32)
+    d = R.GemmF32Desc()
+    d.M, d.N, d.K, d.alpha, d.beta, d.batch = M, N, K, 1.0, 1.0, batch
+    d.strideA, d.strideB, d.strideC, d.strideY = M * K, 0, 0, M * N
+    d.A, d.B, d.C, d.Y, d.residual = util.ptr(dA), util.ptr(dB), util.ptr(dC), util.ptr(dY), util.ptr(dR)
+    d.bias_mode, d.act = R.BIAS_ROW, R.ACT_RELU
+    print("gemm_f32 with residual", M, N, K, batch, kernel, flush=True)
+    rt.call("sofie_hip_gemm_f32", C.byref(d))
+    rt.sync()
+    got = util.to_host(dY)
+    for b in range(batch):
+        lin = ob.gemm_f32(A[b], B, bias, M=M, N=N, K=K, bias_mode=1, act=0)
+        want = ob.unary(ob.add_broadcast(lin, Rr[b]), R.ACT_RELU, 0.0)
+        mag = np.abs(A[b]).astype(np.float64) @ np.abs(B).astype(np.float64) + 1.0
+        assert close(got[b], want.astype(np.float64), mag)
+    assert (got > 0).any() and (got == 0).any()
+
+
+def test_conv_with_a_residual_operand(rt):
+    N, Cc, H, W, Cout = 2, 8, 6, 6, 8
+    X = util.normal(440, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.normal(441, Cout * Cc * 9, 0.15).reshape(Cout, Cc, 3, 3)
+    b = util.normal(442, Cout)
+    d = conv_desc(N, Cc, H, W, Cout, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1)
+    dX, dW, db = util.to_dev(X), util.to_dev(Wt), util.to_dev(b)
+    dY = util.dev_empty((N, Cout, d.OH, d.OW), np.float32)
+    rt.call("sofie_hip_conv_f32", C.byref(d), util.ptr(dX), util.ptr(dW), util.ptr(db), R.ACT_RELU, C.c_float(0), util.ptr(dY), None, util.ptr(dX))
+    rt.sync()
+    lin = ob.conv_f32(X, Wt, b, pads=(1, 1, 1, 1), strides=(1, 1), dils=(1, 1), group=1, act=0)
+    want = ob.unary(ob.add_broadcast(lin, X), R.ACT_RELU, 0.0)
+    got = util.to_host(dY)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-5) and (got > 0).any() and (got == 0).any()
