@@ -84,6 +84,20 @@ inline std::size_t ConvertShapeToLength(const std::vector<std::size_t> &shape)
    return n;
 }
 
+// the same with a limit: a shape whose element count does not fit 2^40 is refused (a corrupt file, or a product that
+// would overflow the byte arithmetic of the memory plan)
+inline std::size_t CheckedShapeLength(const std::vector<std::size_t> &shape, const std::string &what)
+{
+   const std::size_t limit = std::size_t(1) << 40;
+   std::size_t n = 1;
+   for (auto d : shape) {
+      if (d != 0 && n > limit / d)
+         throw std::runtime_error("SOFIE: tensor " + what + " has more than 2^40 elements");
+      n *= d;
+   }
+   return n;
+}
+
 inline std::string ConvertShapeToString(const std::vector<std::size_t> &shape)
 {
    std::string s = "{ ";

@@ -31,6 +31,7 @@ void RModel::AddInputTensorInfo(std::string input_name, ETensorType type, std::v
    input_name = UTILITY::Clean_name(input_name);
    if (CheckIfTensorAlreadyExist(input_name))
       throw std::runtime_error("SOFIE: input tensor with name " + input_name + " already exists \n");
+   CheckedShapeLength(shape, input_name);
    fInputTensorInfos[input_name] = TensorInfo{type, shape};
 }
 
@@ -84,6 +85,7 @@ void RModel::AddIntermediateTensor(std::string tensor_name, ETensorType type, st
    tensor_name = UTILITY::Clean_name(tensor_name);
    if (CheckIfTensorAlreadyExist(tensor_name))
       throw std::runtime_error("SOFIE: intermediate tensor with name " + tensor_name + " already exists \n");
+   CheckedShapeLength(shape, tensor_name);
    if (batched && (shape.empty() || shape[0] != 1))
       throw std::runtime_error("SOFIE: tensor " + tensor_name + " does not carry the run-time batch as its leading dimension");
    fIntermediateTensorInfos[tensor_name] = TensorInfo{type, shape};

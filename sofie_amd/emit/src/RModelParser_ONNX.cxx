@@ -59,6 +59,8 @@ private:
          if (fP >= fEnd)
             throw std::runtime_error("SOFIE ONNX parser: truncated varint");
          uint8_t b = *fP++;
+         if (shift > 63)
+            throw std::runtime_error("SOFIE ONNX parser: varint longer than 10 bytes");
          r |= (uint64_t)(b & 0x7f) << shift;
          if (!(b & 0x80))
             return r;
@@ -306,10 +308,15 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
    for (auto &t : inits) {
       isInit[t.name] = true;
       const ETensorType ty = static_cast<ETensorType>(t.dtype);
-      const size_t len = ConvertShapeToLength(t.dims);
+      const size_t len = CheckedShapeLength(t.dims, t.name);
       const size_t esz = GetTypeSize(ty);
       if (esz == 0)
          throw std::runtime_error("SOFIE ONNX parser: initializer " + t.name + " has an unsupported data type " + std::to_string(t.dtype));
+      // the payload decides how much is allocated, not the dimensions the file claims
+      const size_t have = !t.raw.empty() ? t.raw.size() / esz : ty == ETensorType::FLOAT ? t.floats.size() : t.ints.size();
+      if (have != len)
+         throw std::runtime_error("SOFIE ONNX parser: initializer " + t.name + " holds " + std::to_string(have) + " values, its shape asks for " +
+                                  std::to_string(len));
       std::vector<uint8_t> data(len * esz);
       if (!t.raw.empty()) {
          if (t.raw.size() != data.size())
@@ -354,6 +361,18 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
       const Node &n = nodes[i];
       if (verbose)
          std::cout << "SOFIE HIP parser: " << n.op << " " << n.name << "\n";
+      {
+         // a node must name the inputs its operator reads below and one output, whatever the file claims
+         static const std::map<std::string, size_t> minInputs = {
+            {"Gemm", 2}, {"MatMul", 2}, {"Add", 2}, {"Conv", 2}, {"QuantizeLinear", 2}, {"DequantizeLinear", 2}, {"BatchNormalization", 5},
+            {"MatMulInteger", 2}, {"ConvInteger", 2}, {"QLinearConv", 8}, {"QLinearMatMul", 8}};
+         auto f = minInputs.find(n.op);
+         const size_t need = f == minInputs.end() ? 1 : f->second;
+         if (n.in.size() < need || n.out.empty())
+            throw std::runtime_error("SOFIE ONNX parser: node " + n.op + (n.name.empty() ? "" : " (" + n.name + ")") + " has " +
+                                     std::to_string(n.in.size()) + " inputs and " + std::to_string(n.out.size()) + " outputs; at least " +
+                                     std::to_string(need) + " and 1 are needed");
+      }
       if (n.op == "Gemm") {
          if (n.in.size() > 2 && !n.in[2].empty())
             model->AddOperator(std::make_unique<ROperator_Gemm<float>>(attrF(n, "alpha", 1.f), attrF(n, "beta", 1.f), attrI(n, "transA", 0),

@@ -308,6 +308,33 @@ def test_equal_shaped_adds_join_the_store_of_their_producer(emitted, tmp_path):
     assert "d.residual" not in txt and "sofie_hip_add_f32" in txt
 
 
+def test_corrupt_files_are_refused_with_a_message(tmp_path):
+    """Damaged ONNX files end in an error message and exit status 1, never in a crash: a node without outputs, a varint that
+    never ends, an initializer whose shape promises more values than the file holds, a truncated file."""
+    good = ow.model([ow.node("Relu", ["X"], ["Y"])], [("X", np.float32, [1, 4])], [("Y", np.float32, [1, 4])], {"W": np.ones((2, 2), np.float32)})
+
+    def run(data, name):
+        p = os.path.join(str(tmp_path), name + ".onnx")
+        open(p, "wb").write(data)
+        return subprocess.run([em.EMIT, p, str(tmp_path)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+
+    assert run(good, "good").returncode == 0
+    r = run(ow.model([ow.node("Relu", ["X"], [])], [("X", np.float32, [1, 4])], [("Y", np.float32, [1, 4])], {}), "no_output")
+    assert r.returncode == 1 and "0 outputs" in r.stdout
+    r = run(ow.model([ow.node("Gemm", ["X"], ["Y"])], [("X", np.float32, [1, 4])], [("Y", np.float32, [1, 4])], {}), "one_input")
+    assert r.returncode == 1 and "at least 2" in r.stdout
+    r = run(b"\x08" + b"\xff" * 12, "varint")
+    assert r.returncode == 1 and "varint" in r.stdout
+    for cut in (1, len(good) // 3, len(good) - 3):
+        r = run(good[:cut], "cut%d" % cut)
+        assert r.returncode in (0, 1) and (r.returncode == 0 or "error" in r.stdout)
+    # the shape of the initializer claims 2^50 values
+    t = ow._vi(1, 1 << 50) + ow._vi(1, 2) + ow._vi(2, 1) + ow._ld(8, b"W") + ow._ld(9, np.ones(4, np.float32).tobytes())
+    g = ow._ld(1, ow.node("Relu", ["X"], ["Y"])) + ow._ld(2, b"g") + ow._ld(5, t) + ow._ld(11, ow.value_info("X", 1, [1, 4])) + ow._ld(12, ow.value_info("Y", 1, [1, 4]))
+    r = run(ow._vi(1, 8) + ow._ld(7, g), "huge")
+    assert r.returncode == 1 and ("2^40" in r.stdout or "values" in r.stdout)
+
+
 def test_asymmetric_zero_point_is_refused(tmp_path):
     init = {"W": np.ones((4, 3, 1, 1), dtype=np.int8), "s": np.array(0.5, dtype=np.float32), "z": np.zeros((), dtype=np.int8),
             "z1": np.array(3, dtype=np.int8), "sx": np.array(0.1, dtype=np.float32)}
