@@ -132,8 +132,45 @@ public:
       if (!fNR.empty() && (!model.CheckIfTensorAlreadyExist(fNR) || model.GetTensorType(fNR) != ETensorType::FLOAT ||
                            model.GetTensorShape(fNR) != fShapeY || model.IsDynamicTensor(fNR) != fDynamic))
          throw std::runtime_error("SOFIE Gemm Op: residual tensor " + fNR + " does not have the shape of the product");
+      // A product of weights only is computed now and becomes a constant of the model, with the loops of the reference
+      // (core/inc/SOFIE/operators/ROperator_Gemm.hxx:317-373: plain 2-D operands, C of the product's own shape, Relu at most)
+      const bool canFold = !fDynamic && fShapeA.size() <= 2 && fBatch == 1 && model.IsInitializedTensor(fNA) && model.IsInitializedTensor(fNB) &&
+                           (fNC.empty() || (model.IsInitializedTensor(fNC) && fBiasMode == std::string("SOFIE_BIAS_FULL"))) && fNR.empty() &&
+                           fPost.empty() && (fActivation == EActivationType::UNDEFINED || fActivation == EActivationType::RELU);
+      if (canFold) {
+         const float *dataA = static_cast<const float *>(model.GetInitializedTensorData(fNA).get());
+         const float *dataB = static_cast<const float *>(model.GetInitializedTensorData(fNB).get());
+         const std::size_t m = fM, n = fN, k = fK;
+         std::vector<float> dataY(m * n, 0.f);
+         for (std::size_t i = 0; i < m; i++) {
+            for (std::size_t j = 0; j < n; j++) {
+               float sum = 0.f;
+               for (std::size_t p = 0; p < k; p++) {
+                  const float aVal = fAttrTransA ? dataA[p * m + i] : dataA[i * k + p];
+                  const float bVal = fAttrTransB ? dataB[j * k + p] : dataB[p * n + j];
+                  volatile float prod = aVal * bVal; // one rounding per operation, no fused multiply-add
+                  sum += prod;
+               }
+               dataY[i * n + j] = fAttrAlpha * sum;
+            }
+         }
+         if (!fNC.empty()) {
+            const float *dataC = static_cast<const float *>(model.GetInitializedTensorData(fNC).get());
+            for (std::size_t idx = 0; idx < dataY.size(); idx++) {
+               volatile float scaled = fAttrBeta * dataC[idx];
+               dataY[idx] += scaled;
+            }
+         }
+         if (fActivation == EActivationType::RELU)
+            for (auto &v : dataY)
+               v = std::max(v, 0.f);
+         model.AddConstantTensor(fNY, ETensorType::FLOAT, fShapeY, dataY.data());
+         fIsOutputConstant = true;
+         return;
+      }
       model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShapeY, fDynamic);
    }
+   bool IsOutputConstant() const { return fIsOutputConstant; }
    // shape inference only (registers nothing): sets M, N, K, the bias mode and OutputShape()
    void ResolveShapes(RModel &model)
    {
@@ -260,6 +297,8 @@ public:
       opName = "op_" + opName;
       if (fM == 0)
          throw std::runtime_error("SOFIE Gemm Op called to Generate without being initialized first");
+      if (fIsOutputConstant)
+         return "\n" + SP + "//--------- Gemm " + opName + " -> " + fNY + ": a product of weights, computed when the code was generated\n";
       std::stringstream out;
       out << "\n" << SP << "//--------- Gemm " << opName << " " << ConvertShapeToString(fShapeA) << " * " << ConvertShapeToString(fShapeB)
           << " -> " << fNY << "\n";
@@ -293,7 +332,7 @@ private:
    std::vector<std::size_t> fShapeA, fShapeB;
    std::size_t fM = 0, fN = 0, fK = 0, fBatch = 1, fStrideA = 0, fStrideB = 0, fStrideC = 0;
    std::string fBiasMode;
-   bool fDynamic = false, fDynamicRows = false, fDynamicStack = false;
+   bool fDynamic = false, fDynamicRows = false, fDynamicStack = false, fIsOutputConstant = false;
 };
 
 } // namespace SOFIE_HIP

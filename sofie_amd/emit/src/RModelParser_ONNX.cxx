@@ -355,6 +355,94 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
    auto attrV = [](const Node &n, const char *k) { auto f = n.attrs.find(k); return f == n.attrs.end() ? std::vector<size_t>{} : ToSizes(f->second.ints); };
 
    std::vector<bool> consumed(nodes.size(), false);
+
+   // ---- parse-time rewrites of the reference (parsers/src/RModelParser_ONNX.cxx:1116-1140, 1186-1207) ----
+   // Element types as far as the rewrites need them: graph inputs and initializers are known, an operator's output
+   // takes the type its definition gives it.
+   std::map<std::string, int> typeOf;
+   for (auto &t : inits)
+      typeOf[t.name] = t.dtype;
+   for (auto &v : inputs)
+      if (!typeOf.count(v.name))
+         typeOf[v.name] = v.elem_type;
+   std::map<std::string, size_t> rankOf;
+   for (auto &t : inits)
+      rankOf[t.name] = t.dims.size();
+   for (auto &v : inputs)
+      if (!rankOf.count(v.name))
+         rankOf[v.name] = v.shape.size();
+   auto isGraphOutput = [&](const std::string &name) {
+      for (auto &o : outputs)
+         if (o.name == name)
+            return true;
+      return false;
+   };
+   auto singleReader = [&](const std::string &name) -> size_t {
+      size_t found = nodes.size(), count = 0;
+      for (size_t j = 0; j < nodes.size(); ++j)
+         for (auto &in : nodes[j].in)
+            if (in == name) {
+               found = j;
+               ++count;
+            }
+      return count == 1 ? found : nodes.size();
+   };
+   std::map<std::string, std::string> transposedFrom; // output of an absorbed Transpose -> its input
+   for (size_t i = 0; i < nodes.size(); ++i) {
+      Node &n = nodes[i];
+      if (n.in.empty() || n.out.empty())
+         continue;
+      const int inType = typeOf.count(n.in[0]) ? typeOf[n.in[0]] : 0;
+      // a Cast to the type its input already has changes nothing: its output becomes another name of the input
+      if (n.op == "Cast" && n.in.size() == 1 && n.out.size() == 1 && !isGraphOutput(n.out[0]) && inType != 0 &&
+          attrI(n, "to", -1) == inType) {
+         for (size_t j = i + 1; j < nodes.size(); ++j)
+            for (auto &in : nodes[j].in)
+               if (in == n.out[0])
+                  in = n.in[0];
+         consumed[i] = true;
+         continue;
+      }
+      // Transpose of the last two axes whose only reader is a MatMul: the product reads the operand transposed
+      if (n.op == "Transpose" && n.in.size() == 1 && n.out.size() == 1 && !isGraphOutput(n.out[0]) && inType == 1) {
+         const size_t reader = singleReader(n.out[0]);
+         bool lastTwo = false;
+         auto perm = n.attrs.find("perm");
+         if (perm == n.attrs.end()) {
+            lastTwo = rankOf.count(n.in[0]) && rankOf[n.in[0]] == 2; // the default reverses every axis: a matrix transpose at rank 2 only
+         } else {
+            const auto &p = perm->second.ints;
+            lastTwo = p.size() >= 2;
+            for (size_t a = 0; lastTwo && a + 2 < p.size(); ++a)
+               lastTwo = p[a] == (int64_t)a;
+            lastTwo = lastTwo && p[p.size() - 2] == (int64_t)p.size() - 1 && p[p.size() - 1] == (int64_t)p.size() - 2;
+         }
+         if (lastTwo && reader < nodes.size() && nodes[reader].op == "MatMul" && nodes[reader].in.size() == 2) {
+            transposedFrom[n.out[0]] = n.in[0];
+            consumed[i] = true;
+            continue;
+         }
+      }
+      // element type and rank of what this node produces
+      int outType = inType;
+      if (n.op == "QuantizeLinear" || n.op == "QLinearConv" || n.op == "QLinearMatMul")
+         outType = 3;
+      else if (n.op == "MatMulInteger" || n.op == "ConvInteger")
+         outType = 6;
+      else if (n.op == "DequantizeLinear")
+         outType = 1;
+      else if (n.op == "Cast")
+         outType = (int)attrI(n, "to", 0);
+      typeOf[n.out[0]] = outType;
+      if (rankOf.count(n.in[0]) && (n.op == "Relu" || n.op == "Cast" || n.op == "Transpose" || n.op == "Identity"))
+         rankOf[n.out[0]] = rankOf[n.in[0]];
+   }
+   uses.clear(); // the aliases and absorbed nodes changed who reads what
+   for (size_t j = 0; j < nodes.size(); ++j)
+      if (!consumed[j])
+         for (auto &in : nodes[j].in)
+            uses[in]++;
+
    for (size_t i = 0; i < nodes.size(); ++i) {
       if (consumed[i])
          continue;
@@ -391,13 +479,16 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
                      addIdx = j;
                   break;
                }
+         // operands that an absorbed Transpose produced are read transposed from its input
+         const bool tA = transposedFrom.count(n.in[0]) != 0, tB = transposedFrom.count(n.in[1]) != 0;
+         const std::string opA = tA ? transposedFrom[n.in[0]] : n.in[0], opB = tB ? transposedFrom[n.in[1]] : n.in[1];
          if (addIdx < nodes.size()) {
             const Node &a = nodes[addIdx];
             const std::string &bias = a.in[0] == n.out[0] ? a.in[1] : a.in[0];
-            model->AddOperator(std::make_unique<ROperator_Gemm<float>>(1.f, 1.f, 0, 0, n.in[0], n.in[1], bias, a.out[0]));
+            model->AddOperator(std::make_unique<ROperator_Gemm<float>>(1.f, 1.f, tA ? 1 : 0, tB ? 1 : 0, opA, opB, bias, a.out[0]));
             consumed[addIdx] = true;
          } else {
-            model->AddOperator(std::make_unique<ROperator_Gemm<float>>(1.f, 0.f, 0, 0, n.in[0], n.in[1], n.out[0]));
+            model->AddOperator(std::make_unique<ROperator_Gemm<float>>(1.f, 0.f, tA ? 1 : 0, tB ? 1 : 0, opA, opB, n.out[0]));
          }
       } else if (n.op == "Relu") {
          model->AddOperator(std::make_unique<ROperator_Relu<float>>(n.in[0], n.out[0]));
@@ -431,10 +522,24 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
       } else if (n.op == "Add") {
          model->AddOperator(std::make_unique<ROperator_BasicBinary<float, Add>>(n.in[0], n.in[1], n.out[0]));
       } else if (n.op == "Conv") {
-         const std::string bias = n.in.size() > 2 ? n.in[2] : "";
+         std::string bias = n.in.size() > 2 ? n.in[2] : "";
+         std::string out = n.out[0];
+         // Conv without a bias whose only reader adds a one-dimensional initializer: that initializer is taken as the
+         // convolution's per-channel bias, as the reference's parser does (IsConvBiasAdd, RModelParser_ONNX.cxx:1065-1075, 1203-1207)
+         if (n.in.size() <= 2 && uses[n.out[0]] == 1 && !isGraphOutput(n.out[0])) {
+            const size_t j = singleReader(n.out[0]);
+            if (j < nodes.size() && !consumed[j] && nodes[j].op == "Add" && nodes[j].in.size() == 2 && !nodes[j].out.empty()) {
+               const std::string &other = nodes[j].in[0] == n.out[0] ? nodes[j].in[1] : nodes[j].in[0];
+               if (isInit.count(other) && rankOf.count(other) && rankOf[other] == 1) {
+                  bias = other;
+                  out = nodes[j].out[0];
+                  consumed[j] = true;
+               }
+            }
+         }
          model->AddOperator(std::make_unique<ROperator_Conv<float>>(attrS(n, "auto_pad", "NOTSET"), attrV(n, "dilations"), (size_t)attrI(n, "group", 1),
                                                                     attrV(n, "kernel_shape"), attrV(n, "pads"), attrV(n, "strides"), n.in[0],
-                                                                    n.in[1], bias, n.out[0]));
+                                                                    n.in[1], bias, out));
       } else if (n.op == "GlobalAveragePool") {
          model->AddOperator(std::make_unique<ROperator_Pool<float>>(GlobalAveragePool, n.in[0], n.out[0]));
       } else if (n.op == "QuantizeLinear") {

@@ -234,6 +234,33 @@ def residual_block(batch=2):
                 init={"Wc": Wc, "Bc": Bc, "W": W, "b": b}, feeds=[X, Z])
 
 
+def parse_rewrites():
+    """What the reference's parser rewrites before any operator is built (parsers/src/RModelParser_ONNX.cxx:1116-1140, 1186-1207) and
+    what its Gemm folds (ROperator_Gemm.hxx:317-373): a Cast to the same type, Transpose -> MatMul, MatMul + Add, Conv + Add of a
+    one-dimensional initializer (taken as the per-channel bias), a Gemm of weights only."""
+    W2 = (util.normal(7701, 5 * 6) * np.float32(0.3)).reshape(5, 6)
+    b1 = util.normal(7702, 5)
+    W3 = (util.normal(7703, 6 * 3) * np.float32(0.3)).reshape(6, 3)
+    Ka, Kb, Kc = util.normal(7704, 8).reshape(4, 2), util.normal(7705, 6).reshape(2, 3), util.normal(7706, 12).reshape(4, 3)
+    Wc = (util.normal(7707, 3 * 2) * np.float32(0.5)).reshape(3, 2, 1, 1)
+    cb = util.normal(7708, 3)
+    nodes = [
+        ow.node("Cast", ["X"], ["Xc"], to=1), ow.node("Transpose", ["W2"], ["Wt"], perm=[1, 0]), ow.node("MatMul", ["Xc", "Wt"], ["m1"]),
+        ow.node("Add", ["m1", "b1"], ["Y1"]),
+        ow.node("Transpose", ["A2"], ["At"]), ow.node("MatMul", ["At", "W3"], ["m2"]),
+        ow.node("Gemm", ["Ka", "Kb", "Kc"], ["K"], alpha=0.5, beta=2.0), ow.node("Relu", ["K"], ["Kr"]), ow.node("Add", ["m2", "Kr"], ["Y2"]),
+        ow.node("Conv", ["I", "Wc"], ["c"], kernel_shape=[1, 1], pads=[0, 0, 0, 0]), ow.node("Add", ["c", "cb"], ["Y3"]),
+    ]
+    X, A2, I = util.normal(7709, 24).reshape(4, 6), util.normal(7710, 24).reshape(6, 4), util.normal(7711, 18).reshape(1, 2, 3, 3)
+    # expected values, straight from the definitions (the Conv + Add as the reference reads it: one bias per channel)
+    K = np.maximum(0.5 * (Ka.astype(np.float64) @ Kb) + 2.0 * Kc, 0)
+    want = [X.astype(np.float64) @ W2.T + b1, A2.T.astype(np.float64) @ W3 + K,
+            np.einsum("nchw,oc->nohw", I.astype(np.float64), Wc[:, :, 0, 0]) + cb.reshape(1, 3, 1, 1)]
+    return dict(nodes=nodes, inputs=[("X", np.float32, [4, 6]), ("A2", np.float32, [6, 4]), ("I", np.float32, [1, 2, 3, 3])],
+                outputs=[("Y1", np.float32, [4, 5]), ("Y2", np.float32, [4, 3]), ("Y3", np.float32, [1, 3, 3, 3])],
+                init={"W2": W2, "b1": b1, "W3": W3, "Ka": Ka, "Kb": Kb, "Kc": Kc, "Wc": Wc, "cb": cb}, feeds=[X, A2, I], want=want)
+
+
 DYNAMIC_MODELS = {    "Dynamic_ResidualBlock": lambda: with_named_batch(residual_block(2), "N"),
     "DynamicResidual": dynamic_residual,
 
@@ -467,14 +494,15 @@ def build_all(jobs=8):
         p = os.path.join(OUT, m + ".onnx")
         ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)
         dynamic.append((m, p, len(spec["inputs"])))
-    spec = elementwise_chains()
-    p = os.path.join(OUT, "ElementwiseChains.onnx")
-    ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name="ElementwiseChains")
-    _run([EMIT, p, OUT])
-    src = os.path.join(OUT, "ElementwiseChains_harness.cxx")
-    with open(src, "w") as f:
-        f.write(MULTI_OUTPUT_HARNESS % dict(model="ElementwiseChains", args="inputs[0], inputs[1]"))
-    compile_shared(src, os.path.join(OUT, "libElementwiseChains.so"))
+    for m, make, n_in in (("ElementwiseChains", elementwise_chains, 2), ("ParseRewrites", parse_rewrites, 3)):
+        spec = make()
+        p = os.path.join(OUT, m + ".onnx")
+        ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)
+        _run([EMIT, p, OUT])
+        src = os.path.join(OUT, m + "_harness.cxx")
+        with open(src, "w") as f:
+            f.write(MULTI_OUTPUT_HARNESS % dict(model=m, args=", ".join("inputs[%d]" % i for i in range(n_in))))
+        compile_shared(src, os.path.join(OUT, "lib%s.so" % m))
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(lambda w: emit_and_compile(*w), work))
         list(ex.map(lambda w: emit_and_compile_dynamic(*w), dynamic))
@@ -488,7 +516,7 @@ def build_all(jobs=8):
         f.write(DYNAMIC_HARNESS % dict(model="ApiDynamicFp8Gemm", args="inputs[0]"))
     compile_shared(src, os.path.join(OUT, "libApiDynamicFp8Gemm.so"))
     compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
-    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains"]
+    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites"]
 
 
 if __name__ == "__main__":

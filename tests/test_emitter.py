@@ -335,6 +335,25 @@ def test_corrupt_files_are_refused_with_a_message(tmp_path):
     assert r.returncode == 1 and ("2^40" in r.stdout or "values" in r.stdout)
 
 
+def test_parse_time_rewrites_of_the_reference(emitted, tmp_path):
+    txt = read(emitted, "ParseRewrites")
+    body = ops_body(txt)
+    # 11 nodes, 4 launches: Cast aliased, both Transposes absorbed as transA / transB, MatMul + Add -> Gemm with bias,
+    # the Gemm of weights folded (with its Relu) into a constant, Conv + Add(1-D initializer) -> Conv with bias
+    assert body.count("detail::Check(") == 4
+    assert "d.transA = 0; d.transB = 1;" in body and "d.A = tensor_X; d.B = tensor_W2; d.C = tensor_b1; d.bias_mode = SOFIE_BIAS_ROW;" in body
+    assert "d.transA = 1; d.transB = 0;" in body and "d.A = tensor_A2;" in body
+    assert "computed when the code was generated" in body and "tensor_Kr" in txt and "static const float host[12]" in txt
+    assert "tensor_I, tensor_Wc, tensor_cb, SOFIE_ACT_NONE" in body
+    assert "Transpose" not in body and "Cast" not in body
+    # a Cast that changes the type, and a Transpose that is a graph output, are not rewritten away: they are refused by name
+    r = _emit(tmp_path, [ow.node("Cast", ["X"], ["Y"], to=7)], [("X", np.float32, [1, 4])], [("Y", np.int64, [1, 4])], {})
+    assert r.returncode != 0 and "Cast" in r.stdout
+    r = _emit(tmp_path, [ow.node("Transpose", ["X"], ["T"]), ow.node("MatMul", ["T", "W"], ["Y"])], [("X", np.float32, [3, 2])],
+              [("T", np.float32, [2, 3]), ("Y", np.float32, [2, 4])], {"W": np.ones((3, 4), np.float32)})
+    assert r.returncode != 0 and "Transpose" in r.stdout
+
+
 def test_asymmetric_zero_point_is_refused(tmp_path):
     init = {"W": np.ones((4, 3, 1, 1), dtype=np.int8), "s": np.array(0.5, dtype=np.float32), "z": np.zeros((), dtype=np.int8),
             "z1": np.array(3, dtype=np.int8), "sx": np.array(0.1, dtype=np.float32)}

@@ -230,3 +230,13 @@ def test_emitted_residual_block(rt):
     print("emitted ResidualBlock", flush=True)
     got = run_emitted("ResidualBlock", spec["feeds"], want.size)
     assert np.abs(got - want).max() <= 1e-5 and want.std() > 0.01
+
+
+def test_emitted_parse_time_rewrites(rt):
+    """Cast to the same type, Transpose -> MatMul, MatMul + Add, Conv + Add(1-D initializer), a Gemm of weights only:
+    the rewrites of the reference's parser and the fold of its Gemm, against the definitions in float64."""
+    spec = em.parse_rewrites()
+    want = np.concatenate([w.ravel() for w in spec["want"]])
+    print("emitted ParseRewrites", flush=True)
+    got = run_emitted("ParseRewrites", spec["feeds"], want.size)
+    assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
