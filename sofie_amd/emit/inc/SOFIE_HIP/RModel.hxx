@@ -47,6 +47,12 @@ public:
    bool CheckIfTensorAlreadyExist(const std::string &tensor_name) const;
    bool IsInitializedTensor(const std::string &name) const;
    bool IsInputTensor(const std::string &name) const;
+   // an initialized tensor computed at generation time (embedded in the header, not in the weight file)
+   bool IsConstantTensor(const std::string &name) const
+   {
+      auto f = fInitializedTensors.find(UTILITY::Clean_name(name));
+      return f != fInitializedTensors.end() && f->second.constant;
+   }
    const std::vector<std::size_t> &GetTensorShape(const std::string &name) const;
    ETensorType GetTensorType(const std::string &name) const;
    std::shared_ptr<void> GetInitializedTensorData(const std::string &name) const;
@@ -116,6 +122,7 @@ private:
    std::unordered_map<std::string, std::size_t> fOffsets;
    std::unordered_map<std::string, int> fTensorLayout;
    std::size_t fArenaBytes = 0, fPoolBytes = 0, fStaticBytes = 0, fBatchEntryBytes = 0;
+   std::size_t fPoolBase = 0, fPoolFreeBytes = 0, fPoolLargestFreeBlock = 0;
    std::unordered_map<std::string, std::vector<Dim>> fInputDimShapes;
    std::unordered_map<std::string, bool> fBatched;
    std::string fBatchParam;

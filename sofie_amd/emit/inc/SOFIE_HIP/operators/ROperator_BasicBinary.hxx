@@ -46,11 +46,37 @@ public:
                                      " cannot be broadcast");
          fShapeY[i] = std::max(fShapeA[i], fShapeB[i]);
       }
+      // two constants: the sum is computed now (core/inc/SOFIE/operators/ROperator_BasicBinary.hxx:191-257)
+      if (model.IsConstantTensor(fNA) && model.IsConstantTensor(fNB) && model.GetTensorType(fNA) == ETensorType::FLOAT &&
+          model.GetTensorType(fNB) == ETensorType::FLOAT) {
+         const float *a = static_cast<const float *>(model.GetInitializedTensorData(fNA).get());
+         const float *b = static_cast<const float *>(model.GetInitializedTensorData(fNB).get());
+         std::vector<float> y(ConvertShapeToLength(fShapeY));
+         std::vector<std::size_t> idx(r, 0);
+         for (std::size_t i = 0; i < y.size(); ++i) {
+            std::size_t ia = 0, ib = 0;
+            for (std::size_t d = 0; d < r; ++d) {
+               ia = ia * fShapeA[d] + (fShapeA[d] == 1 ? 0 : idx[d]);
+               ib = ib * fShapeB[d] + (fShapeB[d] == 1 ? 0 : idx[d]);
+            }
+            y[i] = a[ia] + b[ib];
+            for (std::size_t d = r; d-- > 0;) {
+               if (++idx[d] < fShapeY[d])
+                  break;
+               idx[d] = 0;
+            }
+         }
+         model.AddConstantTensor(fNY, ETensorType::FLOAT, fShapeY, y.data());
+         fIsOutputConstant = true;
+         return;
+      }
       model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShapeY, fDynA || fDynB);
    }
    std::string Generate_GPU_HIP(std::string opName) override
    {
       opName = "op_" + opName;
+      if (fIsOutputConstant)
+         return "\n" + SP + "//------ Add " + opName + " -> " + fNY + ": a sum of constants, computed when the code was generated\n";
       std::stringstream out;
       auto list = [](const std::vector<std::size_t> &v, bool batched) {
          std::string s = "{";
@@ -70,7 +96,7 @@ public:
 private:
    std::string fNA, fNB, fNY;
    std::vector<std::size_t> fShapeA, fShapeB, fShapeY;
-   bool fDynA = false, fDynB = false;
+   bool fDynA = false, fDynB = false, fIsOutputConstant = false;
 };
 
 } // namespace SOFIE_HIP

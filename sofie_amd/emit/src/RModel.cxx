@@ -289,6 +289,8 @@ void RModel::TryFuseResidual(std::size_t i)
    const std::string y = op->GetOutputTensorNames()[0];
    if (IsOutputTensor(y))
       return;
+   if (g && IsInitializedTensor(op->GetInputTensorNames()[0]) && IsInitializedTensor(op->GetInputTensorNames()[1]))
+      return; // a product of weights: left whole, so that it can be folded into a constant
    std::size_t reader = fOperators.size(), readers = 0;
    for (std::size_t j = 0; j < fOperators.size(); ++j)
       for (auto &in : fOperators[j]->GetInputTensorNames())
@@ -474,6 +476,9 @@ void RModel::PlanMemory()
       fOffsets[names[t]] = poolBase + r.offsets[t];
    }
    fPoolBytes = r.total_bytes; // per batch entry when the batch is a run-time parameter
+   fPoolBase = poolBase;
+   fPoolFreeBytes = r.total_free_bytes;
+   fPoolLargestFreeBlock = r.largest_free_block;
    fStaticBytes = off;
    fBatchEntryBytes = dyn ? entryOff + r.total_bytes : 0;
    fArenaBytes = dyn ? off + entryAlign * fBatchEntryBytes : poolBase + r.total_bytes; // dynamic: the smallest Session (capacity 16)
@@ -799,7 +804,7 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    std::transform(guard.begin(), guard.end(), guard.begin(), [](unsigned char c) { return std::toupper(c); });
    gc << "//Code generated automatically by SOFIE (gfx950 HIP backend)\n";
    gc << "#ifndef " << guard << "_GPU_HIP\n#define " << guard << "_GPU_HIP\n\n";
-   gc << "#include <array>\n#include <cstddef>\n#include <cstdint>\n#include <cstdlib>\n#include <fstream>\n#include <stdexcept>\n#include <string>\n"
+   gc << "#include <array>\n#include <cstddef>\n#include <cstdint>\n#include <cstdlib>\n#include <fstream>\n#include <stdexcept>\n#include <string>\n#include <string_view>\n"
          "#include <tuple>\n#include <type_traits>\n#include <vector>\n#if __cplusplus >= 202002L\n#include <span>\n#endif\n#include \"sofie_hip.h\"\n";
    if (customMemory)
       gc << "#include <functional>\n";
@@ -979,6 +984,32 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
       << (dyn ? "fCapacity * kIntermediatePoolBytesPerBatchEntry" : "kIntermediatePoolBytes") << "; }\n";
    if (dyn)
       gc << "   std::size_t GetMaxBatch() const { return fMaxBatch; }\n";
+   // statistics of the pool of intermediate tensors, as the reference's GPU sessions report them (core/src/RModel_ALPAKA.cxx:1262-1269)
+   {
+      const std::string scale = dyn ? "fCapacity * " : "";
+      gc << "   std::size_t GetTotalFreeMemory() const { return " << scale << fPoolFreeBytes << "; }\n";
+      gc << "   std::size_t GetLargestFreeBlock() const { return " << scale << fPoolLargestFreeBlock << "; }\n";
+      gc << "   double GetFragmentation() const { return " << (fPoolFreeBytes == 0 ? std::string("0.0") : "1.0 - " + std::to_string(fPoolLargestFreeBlock) + ".0 / " + std::to_string(fPoolFreeBytes) + ".0")
+         << "; }\n";
+      // zero the intermediate tensors (the reference's resetState, core/src/RModel_ALPAKA.cxx:1543-1568) and the weights
+      // (SetWeightsToZero, core/src/RModel.cxx:1632-1643)
+      gc << "   void resetState()\n   {\n";
+      const std::string base = dyn ? "static_cast<char *>(sofie_hip_arena_ptr(fCtx, 0)) + kStaticBytes + fCapacity * " + std::to_string(fPoolBase)
+                                   : "static_cast<char *>(sofie_hip_arena_ptr(fCtx, 0)) + " + std::to_string(fPoolBase);
+      if (fPoolBytes && !customMemory)
+         gc << "      detail::Check(sofie_hip_fill_zero(fCtx, " << base << ", " << scale << fPoolBytes << "), \"resetState\");\n";
+      else
+         for (auto &p : fPlan)
+            if (p.pooled)
+               gc << "      detail::Check(sofie_hip_fill_zero(fCtx, " << p.name << ", " << (p.perBatch ? scale : "") << p.bytes << "), \"resetState\");\n";
+      gc << "      detail::Check(sofie_hip_sync(fCtx), \"resetState\");\n   }\n";
+      gc << "   void SetWeightsToZero()\n   {\n";
+      for (auto &kv : fInitializedTensors)
+         if (!kv.second.constant && kv.second.type == ETensorType::FLOAT && ConvertShapeToLength(kv.second.shape))
+            gc << "      detail::Check(sofie_hip_fill_zero(fCtx, tensor_" << kv.first << ", " << ConvertShapeToLength(kv.second.shape) * 4
+               << "), \"SetWeightsToZero\");\n";
+      gc << "      detail::Check(sofie_hip_sync(fCtx), \"SetWeightsToZero\");\n   }\n";
+   }
    // device-resident use: where to write the inputs and read the outputs around infer_nosync()
    for (auto &n : fInputTensorNames)
       gc << "   " << ConvertTypeToString(fInputTensorInfos[n].type) << " *device_input_" << n << "() const { return tensor_" << n << "; }\n";
@@ -1139,15 +1170,38 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    }
    gc << "   }\n";
    gc << "}; // end of Session\n\n";
+   // the shapes of the graph tensors in the reference's form (core/src/RModel.cxx:2036-2112,
+   // core/src/utils/SOFIE_common_helpers.cxx:880-907): a run-time dimension carries its parameter's name
+   gc << "struct SingleDim {\n   enum class Kind { Static, Symbolic };\n   Kind kind;\n   std::size_t dim;\n   std::string_view name;\n"
+         "   constexpr SingleDim(std::size_t v) : kind(Kind::Static), dim(v), name() {}\n"
+         "   constexpr SingleDim(const char *v) : kind(Kind::Symbolic), dim(0), name(v) {}\n};\n"
+         "struct TensorDims {\n   const SingleDim *data;\n   std::size_t size;\n   constexpr std::size_t total_size() const\n   {\n"
+         "      std::size_t result = 1;\n      for (std::size_t i = 0; i < size; ++i)\n         result *= data[i].dim;\n      return result;\n   }\n};\n"
+         "template <class Arr>\nconstexpr TensorDims makeDims(Arr const &arr)\n{\n   return TensorDims{arr.data(), arr.size()};\n}\n\n";
+   std::set<std::string> dimsEmitted;
    auto dimsArray = [&](const std::string &what, const std::vector<std::string> &names) {
-      gc << "// " << what << " tensor shapes" << (dyn ? " (0 stands for the run-time parameter " + fBatchParam + ")" : "") << "\n";
+      gc << "// " << what << " tensor dimensions\n";
+      bool anyDynamic = false;
       for (auto &n : names) {
          const auto &s = GetTensorShape(n);
-         gc << "constexpr std::array<std::size_t, " << s.size() << "> dim_" << n << "{";
-         for (std::size_t i = 0; i < s.size(); ++i)
-            gc << (i == 0 && IsDynamicTensor(n) ? 0 : s[i]) << (i + 1 < s.size() ? ", " : "");
+         anyDynamic = anyDynamic || IsDynamicTensor(n);
+         if (!dimsEmitted.insert(n).second)
+            continue; // a graph output that is also an input, or listed twice
+         gc << "constexpr std::array<SingleDim, " << s.size() << "> dim_" << n << "{";
+         for (std::size_t i = 0; i < s.size(); ++i) {
+            if (i == 0 && IsDynamicTensor(n)) {
+               gc << "SingleDim{\"" << fBatchParam << "\"}";
+            } else
+               gc << "SingleDim{" << s[i] << "}";
+            gc << (i + 1 < s.size() ? ", " : "");
+         }
          gc << "};\n";
       }
+      gc << "constexpr std::array<TensorDims, " << names.size() << "> " << what << "TensorDims{";
+      for (std::size_t i = 0; i < names.size(); ++i)
+         gc << "makeDims(dim_" << names[i] << ")" << (i + 1 < names.size() ? ", " : "");
+      gc << "};\n";
+      gc << "constexpr bool hasDynamic" << (what == "input" ? "Input" : "Output") << "Tensors{" << (anyDynamic ? "true" : "false") << "};\n\n";
    };
    dimsArray("input", fInputTensorNames);
    dimsArray("output", fOutputTensorNames);

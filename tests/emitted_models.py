@@ -236,29 +236,32 @@ def residual_block(batch=2):
 
 def parse_rewrites():
     """What the reference's parser rewrites before any operator is built (parsers/src/RModelParser_ONNX.cxx:1116-1140, 1186-1207) and
-    what its Gemm folds (ROperator_Gemm.hxx:317-373): a Cast to the same type, Transpose -> MatMul, MatMul + Add, Conv + Add of a
-    one-dimensional initializer (taken as the per-channel bias), a Gemm of weights only."""
+    what its operators fold (ROperator_Gemm.hxx:317-373, ROperator_BasicBinary.hxx:191-257): a Cast to the same type, Transpose -> MatMul,
+    MatMul + Add, Conv + Add of a one-dimensional initializer (taken as the per-channel bias), a Gemm of weights only, a sum of constants."""
     W2 = (util.normal(7701, 5 * 6) * np.float32(0.3)).reshape(5, 6)
     b1 = util.normal(7702, 5)
     W3 = (util.normal(7703, 6 * 3) * np.float32(0.3)).reshape(6, 3)
     Ka, Kb, Kc = util.normal(7704, 8).reshape(4, 2), util.normal(7705, 6).reshape(2, 3), util.normal(7706, 12).reshape(4, 3)
+    Kbt, Kd = np.ascontiguousarray(Kb.T), util.normal(7712, 12).reshape(4, 3)
     Wc = (util.normal(7707, 3 * 2) * np.float32(0.5)).reshape(3, 2, 1, 1)
     cb = util.normal(7708, 3)
     nodes = [
         ow.node("Cast", ["X"], ["Xc"], to=1), ow.node("Transpose", ["W2"], ["Wt"], perm=[1, 0]), ow.node("MatMul", ["Xc", "Wt"], ["m1"]),
         ow.node("Add", ["m1", "b1"], ["Y1"]),
         ow.node("Transpose", ["A2"], ["At"]), ow.node("MatMul", ["At", "W3"], ["m2"]),
-        ow.node("Gemm", ["Ka", "Kb", "Kc"], ["K"], alpha=0.5, beta=2.0), ow.node("Relu", ["K"], ["Kr"]), ow.node("Add", ["m2", "Kr"], ["Y2"]),
+        ow.node("Gemm", ["Ka", "Kb", "Kc"], ["K"], alpha=0.5, beta=2.0), ow.node("Relu", ["K"], ["Kr"]),       # folded, Relu included
+        ow.node("Gemm", ["Ka", "Kbt", "Kd"], ["K2"], transB=1), ow.node("Add", ["Kr", "K2"], ["Ks"]),             # a sum of two folded products
+        ow.node("Add", ["m2", "Ks"], ["Y2"]),
         ow.node("Conv", ["I", "Wc"], ["c"], kernel_shape=[1, 1], pads=[0, 0, 0, 0]), ow.node("Add", ["c", "cb"], ["Y3"]),
     ]
     X, A2, I = util.normal(7709, 24).reshape(4, 6), util.normal(7710, 24).reshape(6, 4), util.normal(7711, 18).reshape(1, 2, 3, 3)
     # expected values, straight from the definitions (the Conv + Add as the reference reads it: one bias per channel)
-    K = np.maximum(0.5 * (Ka.astype(np.float64) @ Kb) + 2.0 * Kc, 0)
-    want = [X.astype(np.float64) @ W2.T + b1, A2.T.astype(np.float64) @ W3 + K,
+    Ks = np.maximum(0.5 * (Ka.astype(np.float64) @ Kb) + 2.0 * Kc, 0) + (Ka.astype(np.float64) @ Kb + Kd)
+    want = [X.astype(np.float64) @ W2.T + b1, A2.T.astype(np.float64) @ W3 + Ks,
             np.einsum("nchw,oc->nohw", I.astype(np.float64), Wc[:, :, 0, 0]) + cb.reshape(1, 3, 1, 1)]
     return dict(nodes=nodes, inputs=[("X", np.float32, [4, 6]), ("A2", np.float32, [6, 4]), ("I", np.float32, [1, 2, 3, 3])],
                 outputs=[("Y1", np.float32, [4, 5]), ("Y2", np.float32, [4, 3]), ("Y3", np.float32, [1, 3, 3, 3])],
-                init={"W2": W2, "b1": b1, "W3": W3, "Ka": Ka, "Kb": Kb, "Kc": Kc, "Wc": Wc, "cb": cb}, feeds=[X, A2, I], want=want)
+                init={"W2": W2, "b1": b1, "W3": W3, "Ka": Ka, "Kb": Kb, "Kbt": Kbt, "Kc": Kc, "Kd": Kd, "Wc": Wc, "cb": cb}, feeds=[X, A2, I], want=want)
 
 
 DYNAMIC_MODELS = {    "Dynamic_ResidualBlock": lambda: with_named_batch(residual_block(2), "N"),
@@ -403,6 +406,27 @@ extern "C" long dyn_infer(void *s, unsigned long batch, const float *const *inpu
       return -1;
    }
 }
+extern "C" int dyn_maintenance(void *s, int what, char *err, int errlen)
+{
+   try {
+      if (what == 0)
+         static_cast<Session *>(s)->resetState();
+      else
+         static_cast<Session *>(s)->SetWeightsToZero();
+      return 0;
+   } catch (const std::exception &e) {
+      return fail(err, errlen, e.what());
+   }
+}
+extern "C" double pool_statistics(void *s, unsigned long *free_bytes, unsigned long *largest)
+{
+   *free_bytes = static_cast<Session *>(s)->GetTotalFreeMemory();
+   *largest = static_cast<Session *>(s)->GetLargestFreeBlock();
+   return static_cast<Session *>(s)->GetFragmentation();
+}
+static_assert(SOFIE_%(model)s::inputTensorDims.size() >= 1 && SOFIE_%(model)s::hasDynamicInputTensors &&
+              SOFIE_%(model)s::inputTensorDims[0].data[0].kind == SOFIE_%(model)s::SingleDim::Kind::Symbolic,
+              "the leading dimension of the first input is the run-time parameter");
 extern "C" unsigned long arena_bytes(unsigned long max_batch) { return Session::ArenaBytes(max_batch); }
 extern "C" unsigned long pool_bytes(void *s) { return static_cast<Session *>(s)->GetIntermediateMemoryPoolSize(); }
 '''

@@ -200,6 +200,8 @@ def test_run_time_batch_signatures_follow_the_reference_convention(emitted):
     assert "d.M = static_cast<std::int32_t>(sofie_batch * 1); d.N = 3; d.K = 4;" in txt
     assert "sofie_hip_upload(fCtx, tensor_X, host_X, N * 16)" in txt and "out_0(N * 3)" in txt
     assert "kArenaBytes" not in txt and "ArenaBytes(fMaxBatch)" in txt
+    # shapes of the graph tensors in the reference's form: the parameter by name
+    assert 'dim_X{SingleDim{"N"}, SingleDim{4}}' in txt and "inputTensorDims{makeDims(dim_X)}" in txt and "hasDynamicOutputTensors{true}" in txt
     # the int8 chain: every row count scales, the re-laid-out weights do not
     txt = read(emitted, "Dynamic_int8_MLP")
     assert txt.count("d.M = static_cast<std::int32_t>(sofie_batch * 1)") == 3
@@ -213,7 +215,7 @@ def test_a_batch_given_at_generation_makes_a_static_session(emitted, tmp_path):
     txt = open(os.path.join(str(tmp_path), "DynamicLinear_GPU_HIP.hxx")).read()
     assert "sofie_batch" not in txt and "kArenaBytes" in txt and "d.M = 4; d.N = 3; d.K = 4;" in txt
     assert re.search(r"std::vector<float> infer\(float const ?\* ?host_X\)", txt)
-    assert "dim_X{4, 4}" in txt
+    assert "dim_X{SingleDim{4}, SingleDim{4}}" in txt and "hasDynamicInputTensors{false}" in txt
 
 
 def test_per_batch_entry_plan_scales_without_overlap(emitted, tmp_path):
@@ -346,6 +348,7 @@ def test_parse_time_rewrites_of_the_reference(emitted, tmp_path):
     assert "computed when the code was generated" in body and "tensor_Kr" in txt and "static const float host[12]" in txt
     assert "tensor_I, tensor_Wc, tensor_cb, SOFIE_ACT_NONE" in body
     assert "Transpose" not in body and "Cast" not in body
+    assert "-> K2: a product of weights" in body and "-> Ks: a sum of constants" in body and "d.residual" not in body
     # a Cast that changes the type, and a Transpose that is a graph output, are not rewritten away: they are refused by name
     r = _emit(tmp_path, [ow.node("Cast", ["X"], ["Y"], to=7)], [("X", np.float32, [1, 4])], [("Y", np.int64, [1, 4])], {})
     assert r.returncode != 0 and "Cast" in r.stdout

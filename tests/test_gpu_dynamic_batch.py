@@ -181,3 +181,23 @@ def test_dynamic_residual_block(rt):
             want = gr.run(g, [x[:n], z[:n]], gr.OracleBackend()).ravel()
             got = s.infer(n, [x[:n], z[:n]], 20)
             assert got.size == want.size == n * 4 and np.abs(got - want).max() <= 1e-5
+
+
+def test_reset_state_and_weights_to_zero(rt):
+    """resetState zeroes the pool of intermediates (the next inference is unaffected), SetWeightsToZero the float weights
+    (core/src/RModel_ALPAKA.cxx:1543-1568, core/src/RModel.cxx:1632-1643)."""
+    spec = em.int8_cnn(2, 12)
+    x = spec["feeds"][0]
+    with DynamicSession("Dynamic_int8_CNN", 2) as s:
+        s.lib.dyn_maintenance.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_int]
+        s.lib.pool_statistics.restype = ctypes.c_double
+        s.lib.pool_statistics.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_ulong), ctypes.POINTER(ctypes.c_ulong)]
+        first = s.infer(2, [x], 20).copy()
+        assert s.lib.dyn_maintenance(s.h, 0, s.err, 1024) == 0, s.err.value.decode()
+        assert np.array_equal(s.infer(2, [x], 20), first)
+        free, largest = ctypes.c_ulong(), ctypes.c_ulong()
+        frag = s.lib.pool_statistics(s.h, ctypes.byref(free), ctypes.byref(largest))
+        assert 0.0 <= frag < 1.0 and largest.value <= free.value <= s.lib.pool_bytes(s.h)
+        # the float weights of this model are the final Gemm's: zeroed, the output is the (zeroed) bias
+        assert s.lib.dyn_maintenance(s.h, 1, s.err, 1024) == 0, s.err.value.decode()
+        assert np.array_equal(s.infer(2, [x], 20), np.zeros(20, np.float32))
