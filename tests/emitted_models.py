@@ -264,6 +264,37 @@ def parse_rewrites():
                 init={"W2": W2, "b1": b1, "W3": W3, "Ka": Ka, "Kb": Kb, "Kbt": Kbt, "Kc": Kc, "Kd": Kd, "Wc": Wc, "cb": cb}, feeds=[X, A2, I], want=want)
 
 
+# Models of the reference's own tests whose expected outputs are literals in those tests (tests/cpu/TestCustomModelsFromONNX.cxx:509-527,
+# 1672-1700; the graphs are those of tests/models/generators/generate_input_models.py:1795-1838, 3411-3464, restated here as data).
+def reference_constant_folding_cases():
+    f = np.float32
+    return {
+        "Gemm_ConstantFolding": dict(
+            nodes=[ow.node("Gemm", ["A", "B", "C"], ["Y"], alpha=1.0, beta=1.0, transA=0, transB=0)], inputs=[], outputs=[("Y", f, [2, 2])],
+            init={"A": np.array([[1, 2, 3], [4, 5, 6]], f), "B": np.array([[7, 8], [9, 10], [11, 12]], f), "C": np.ones((2, 2), f)},
+            feeds=[], want=[[59, 65, 140, 155]]),
+        "Gemm_ConstantFolding_Shared": dict(
+            nodes=[ow.node("Gemm", ["A1", "B", "C1"], ["Y1"], alpha=1.0, beta=1.0, transA=0, transB=0),
+                   ow.node("Gemm", ["A2", "B", "C2"], ["Y2"], alpha=1.0, beta=1.0, transA=0, transB=0)],
+            inputs=[("A2", f, [2, 2])], outputs=[("Y1", f, [2, 2]), ("Y2", f, [2, 2])],
+            init={"A1": np.array([[1, 2], [3, 4]], f), "B": np.eye(2, dtype=f), "C1": np.ones((2, 2), f), "C2": np.full((2, 2), 10, f)},
+            feeds=[np.array([[5, 6], [7, 8]], f)], want=[[2, 3, 4, 5], [15, 16, 17, 18]]),
+        "MatMul_1D_Constant": dict(
+            nodes=[ow.node("MatMul", ["A", "B"], ["Y"])], inputs=[], outputs=[("Y", f, [2])],
+            init={"A": np.array([1, 2, 3], f), "B": np.array([[1, 2], [3, 4], [5, 6]], f)}, feeds=[], want=[[22, 28]]),
+    }
+
+
+def reference_stacked_matmul_cases():
+    f = np.float32
+    return {
+        "MatMul_Stacked": dict(nodes=[ow.node("MatMul", ["input1", "input2"], ["output"])], inputs=[("input1", f, ["N", 2, 2]), ("input2", f, [2, 1])],
+                               outputs=[("output", f, ["N", 2, 1])], init={}, feeds=[np.arange(1, 9, dtype=f), np.array([2, 3], f)], want=[8, 18, 28, 38]),
+        "MatMul_Stacked2": dict(nodes=[ow.node("MatMul", ["input1", "input2"], ["output"])], inputs=[("input1", f, ["N", 2, 2]), ("input2", f, ["N", 2, 1])],
+                                outputs=[("output", f, ["N", 2, 1])], init={}, feeds=[np.arange(1, 9, dtype=f), np.array([2, 3, 3, 2], f)], want=[8, 18, 27, 37]),
+    }
+
+
 DYNAMIC_MODELS = {    "Dynamic_ResidualBlock": lambda: with_named_batch(residual_block(2), "N"),
     "DynamicResidual": dynamic_residual,
 
@@ -436,20 +467,22 @@ extern "C" unsigned long pool_bytes(void *s) { return static_cast<Session *>(s)-
 MULTI_OUTPUT_HARNESS = r'''
 #include "%(model)s_GPU_HIP.hxx"
 #include <cstring>
+static void flatten(const std::vector<float> &y, std::vector<float> &all) { all.insert(all.end(), y.begin(), y.end()); }
+static void flatten(const std::vector<std::vector<float>> &ys, std::vector<float> &all)
+{
+   for (auto &y : ys)
+      flatten(y, all);
+}
 extern "C" int run_model(const char *weights, const float *const *inputs, float *output, unsigned long output_len, char *err, int errlen)
 {
+   (void)inputs;
    try {
       SOFIE_%(model)s::Session s(weights);
-      auto ys = s.infer(%(args)s);
-      unsigned long at = 0;
-      for (auto &y : ys) {
-         if (at + y.size() > output_len)
-            throw std::runtime_error("outputs have more elements than expected");
-         std::memcpy(output + at, y.data(), y.size() * sizeof(float));
-         at += y.size();
-      }
-      if (at != output_len)
-         throw std::runtime_error("outputs have " + std::to_string(at) + " elements");
+      std::vector<float> all;
+      flatten(s.infer(%(args)s), all);
+      if (all.size() != output_len)
+         throw std::runtime_error("outputs have " + std::to_string(all.size()) + " elements");
+      std::memcpy(output, all.data(), all.size() * sizeof(float));
       return 0;
    } catch (const std::exception &e) {
       std::strncpy(err, e.what(), errlen - 1);
@@ -518,7 +551,14 @@ def build_all(jobs=8):
         p = os.path.join(OUT, m + ".onnx")
         ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)
         dynamic.append((m, p, len(spec["inputs"])))
-    for m, make, n_in in (("ElementwiseChains", elementwise_chains, 2), ("ParseRewrites", parse_rewrites, 3)):
+    folded = reference_constant_folding_cases()
+    multi = [("ElementwiseChains", elementwise_chains, 2), ("ParseRewrites", parse_rewrites, 3)]
+    multi += [(m, (lambda spec=spec: spec), len(spec["inputs"])) for m, spec in folded.items()]
+    for m, spec in reference_stacked_matmul_cases().items():
+        p = os.path.join(OUT, m + ".onnx")
+        ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)
+        emit_and_compile_dynamic(m, p, len(spec["inputs"]))
+    for m, make, n_in in multi:
         spec = make()
         p = os.path.join(OUT, m + ".onnx")
         ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)

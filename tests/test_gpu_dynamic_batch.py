@@ -201,3 +201,12 @@ def test_reset_state_and_weights_to_zero(rt):
         # the float weights of this model are the final Gemm's: zeroed, the output is the (zeroed) bias
         assert s.lib.dyn_maintenance(s.h, 1, s.err, 1024) == 0, s.err.value.decode()
         assert np.array_equal(s.infer(2, [x], 20), np.zeros(20, np.float32))
+
+
+@pytest.mark.parametrize("model", ["MatMul_Stacked", "MatMul_Stacked2"])
+def test_stacked_matmul_cases_of_the_reference(rt, model):
+    """tests/cpu/TestCustomModelsFromONNX.cxx:1679-1700: Session(file, 2), infer(2, input1, input2) with the expected literals."""
+    spec = em.reference_stacked_matmul_cases()[model]
+    with DynamicSession(model, 2) as s:
+        got = s.infer(2, spec["feeds"], 8)
+    assert np.array_equal(got, np.asarray(spec["want"], np.float32))

@@ -240,3 +240,17 @@ def test_emitted_parse_time_rewrites(rt):
     print("emitted ParseRewrites", flush=True)
     got = run_emitted("ParseRewrites", spec["feeds"], want.size)
     assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+
+
+@pytest.mark.parametrize("model", ["Gemm_ConstantFolding", "Gemm_ConstantFolding_Shared", "MatMul_1D_Constant"])
+def test_constant_folding_cases_of_the_reference(rt, model):
+    """The reference's own tests with their literal expectations (tests/cpu/TestCustomModelsFromONNX.cxx:509-527, 1672-1677):
+    products of weights are folded when the code is generated, a Session without inputs still answers."""
+    spec = em.reference_constant_folding_cases()[model]
+    want = np.concatenate([np.asarray(w, np.float32) for w in spec["want"]])
+    print("emitted", model, flush=True)
+    got = run_emitted(model, spec["feeds"], want.size)
+    assert np.abs(got - want).max() <= 1e-3                 # DEFAULT_TOLERANCE of the reference's tests
+    assert np.array_equal(got, want)                        # small integers: exact in fp32 in any order
+    txt = open(os.path.join(em.OUT, model + "_GPU_HIP.hxx")).read()
+    assert "computed when the code was generated" in txt
