@@ -98,7 +98,8 @@ enum {
    SOFIE_ACT_ACOSH = 19,
    SOFIE_ACT_ATANH = 20,
    SOFIE_ACT_CLIP = 21,      /* max(alpha, min(beta, x))              */
-   SOFIE_ACT_LAST = 21
+   SOFIE_ACT_SELU = 22,      /* beta * (max(0,x) + min(0, alpha*(exp(x)-1))), beta = gamma; core/inc/SOFIE/operators/ROperator_Selu.hxx:56-62 */
+   SOFIE_ACT_LAST = 22
 };
 
 /* A chain of one-to-one operators applied, in order, to every element an operator stores: what the reference's

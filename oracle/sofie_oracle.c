@@ -14,7 +14,10 @@
  *                             tests; float64 brute force.
  *   im2col / conv_f32         golden outputs of the reference's 18 Conv* fixtures; 7-loop direct
  *                             convolution in float64.
- *   relu/sigmoid/gelu/...     Gelu / GeluTanh golden outputs; closed forms.
+ *   relu/sigmoid/gelu/...     Gelu / GeluTanh / LinearWithSelu golden outputs; closed forms.
+ *   basic_unary, unary_chain  numpy's float32 routines (an independent implementation) and identities
+ *                             (exp(log x) = x, sin^2 + cos^2 = 1, sinh(asinh x) = x, ...); Clip bounds; Selu
+ *                             through the LinearWithSelu golden output.
  *   global_avg_pool           GlobalAvgPool2d golden output.
  *   organize_memory           the reference's MemoryPlanner.inc compiled as oracle/_ref and run on the
  *                             same lifetimes; known totals of the Linear_16 plan.
@@ -138,6 +141,7 @@ ORACLE_API void oracle_basic_unary(float *out, const float *in, size_t n, int op
       case 19: y = acoshf(x); break;
       case 20: y = atanhf(x); break;
       case 21: y = fmaxf(alpha, fminf(beta, x)); break;
+      case 22: y = beta * (fmaxf(0.0f, x) + fminf(0.0f, alpha * (expf(x) - 1.0f))); break; /* Selu, ROperator_Selu.hxx:56-62; beta = gamma */
       default: break;
       }
       out[i] = y;
@@ -155,7 +159,7 @@ ORACLE_API void oracle_unary(float *out, const float *in, size_t n, int act, flo
    case 5: oracle_gelu_tanh(out, in, n); break;
    case 6: oracle_tanh(out, in, n); break;
    default:
-      if (act >= 7 && act <= 21)
+      if (act >= 7 && act <= 22)
          oracle_basic_unary(out, in, n, act, alpha, 0.0f);
       else if (out != in)
          memmove(out, in, n * sizeof(float));
@@ -168,7 +172,7 @@ ORACLE_API void oracle_unary_chain(float *out, const float *in, size_t n, int co
    if (out != in)
       memmove(out, in, n * sizeof(float));
    for (int i = 0; i < count; ++i) {
-      if (op[i] >= 7 && op[i] <= 21)
+      if (op[i] >= 7 && op[i] <= 22)
          oracle_basic_unary(out, out, n, op[i], alpha[i], beta[i]);
       else
          oracle_unary(out, out, n, op[i], alpha[i]);

@@ -59,7 +59,7 @@ public:
       for (auto &p : fPost)
          out << " -> " << ActivationEnumName(p.act);
       out << " " << opName << "\n";
-      if (fPost.empty() && fAct != EActivationType::CLIP) {
+      if (fPost.empty() && fAct != EActivationType::CLIP && fAct != EActivationType::SELU) { // those two carry a second parameter
          out << SP << "detail::Check(sofie_hip_unary_f32(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", "
              << BatchScaled(fDynamic, ConvertShapeToLength(fShape)) << ", " << ActivationEnumName(fAct) << ", " << FloatLiteral(fAlpha) << "), \""
              << opName << " activation\");\n";
@@ -139,6 +139,12 @@ struct ROperator_BasicUnary : ROperator_Activation {
 template <typename T>
 struct ROperator_Clip : ROperator_Activation {
    ROperator_Clip(std::string x, std::string y, T minVal, T maxVal) : ROperator_Activation(EActivationType::CLIP, minVal, x, y, maxVal) {}
+};
+// Selu: gamma * (max(0, x) + min(0, alpha * (exp(x) - 1))) (core/inc/SOFIE/operators/ROperator_Selu.hxx:16-62)
+template <typename T>
+struct ROperator_Selu : ROperator_Activation {
+   ROperator_Selu(std::string x, std::string y) : ROperator_Selu(1.67326319217681884765625f, 1.05070102214813232421875f, x, y) {}
+   ROperator_Selu(float alpha, float gamma, std::string x, std::string y) : ROperator_Activation(EActivationType::SELU, alpha, x, y, gamma) {}
 };
 // Identity: a copy that the generator folds away wherever it follows another operator
 template <typename T>

@@ -36,6 +36,7 @@ inline const char *ActivationEnumName(EActivationType a)
    case EActivationType::ACOSH: return "SOFIE_ACT_ACOSH";
    case EActivationType::ATANH: return "SOFIE_ACT_ATANH";
    case EActivationType::CLIP: return "SOFIE_ACT_CLIP";
+   case EActivationType::SELU: return "SOFIE_ACT_SELU";
    default: return "SOFIE_ACT_NONE";
    }
 }

@@ -509,6 +509,9 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
             {"Softplus", EActivationType::SOFTPLUS}, {"Atan", EActivationType::ATAN}, {"Floor", EActivationType::FLOOR},
             {"Asinh", EActivationType::ASINH}, {"Acosh", EActivationType::ACOSH}, {"Atanh", EActivationType::ATANH}};
          model->AddOperator(std::make_unique<ROperator_Activation>(kinds.at(n.op), 0.f, n.in[0], n.out[0]));
+      } else if (n.op == "Selu") {
+         model->AddOperator(std::make_unique<ROperator_Selu<float>>(attrF(n, "alpha", 1.67326319217681884765625f),
+                                                                    attrF(n, "gamma", 1.05070102214813232421875f), n.in[0], n.out[0]));
       } else if (n.op == "Identity") {
          model->AddOperator(std::make_unique<ROperator_Identity<float>>(n.in[0], n.out[0]));
       } else if (n.op == "Clip") {

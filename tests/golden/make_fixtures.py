@@ -41,7 +41,7 @@ def vector_literal(path, test_name, var):
 IOTA, ONES = {"kind": "iota"}, {"kind": "ones"}
 MODELS = {
     "Linear_16": ("all_ones", [ONES]), "Linear_32": ("all_ones", [ONES]), "Linear_64": ("all_ones", [ONES]),
-    "LinearWithSigmoid": ("all_ones", [ONES]),
+    "LinearWithSigmoid": ("all_ones", [ONES]), "LinearWithSelu": ("all_ones", [ONES]),
     "ConvWithPadding": (None, [IOTA]), "ConvWithoutPadding": (None, [IOTA]), "ConvWithAutopadSameLower": (None, [IOTA]),
     "ConvWithAutopadSameUpper": (None, [IOTA]), "ConvWithStridesPadding": (None, [IOTA]),
     "ConvWithStridesNoPadding": (None, [IOTA]), "ConvWithAsymmetricPadding": (None, [IOTA]),

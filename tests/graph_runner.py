@@ -227,6 +227,8 @@ def run(g, inputs, be, all_outputs=False):
         elif op == "Flatten":
             ax = a.get("axis", 1)
             y = np.ascontiguousarray(x[0]).reshape(int(np.prod(x[0].shape[:ax], dtype=np.int64)), -1)
+        elif op == "Selu":
+            y = be.chain(x[0], [(22, a.get("alpha", 1.6732631921768188), a.get("gamma", 1.0507010221481323))])
         elif op == "Identity":
             y = np.array(x[0], copy=True)
         elif op == "Clip":

@@ -252,8 +252,8 @@ def test_chain_errors(rt):
     bad.count = 5
     with pytest.raises(R.SofieHipError, match="more than 4"):
         rt.call("sofie_hip_unary_chain_f32", util.ptr(x), util.ptr(x), C.c_size_t(8), C.byref(bad))
-    with pytest.raises(R.SofieHipError, match="unknown operator 22"):
-        rt.call("sofie_hip_unary_chain_f32", util.ptr(x), util.ptr(x), C.c_size_t(8), C.byref(R.PostOps.of([(22, 0, 0)])))
+    with pytest.raises(R.SofieHipError, match="unknown operator 99"):
+        rt.call("sofie_hip_unary_chain_f32", util.ptr(x), util.ptr(x), C.c_size_t(8), C.byref(R.PostOps.of([(99, 0, 0)])))
     with pytest.raises(R.SofieHipError, match="NULL"):
         rt.call("sofie_hip_unary_chain_f32", util.ptr(x), util.ptr(x), C.c_size_t(8), None)
 
@@ -342,3 +342,12 @@ def test_conv_with_a_residual_operand(rt):
     want = ob.unary(ob.add_broadcast(lin, X), R.ACT_RELU, 0.0)
     got = util.to_host(dY)
     assert np.allclose(got, want, rtol=1e-5, atol=1e-5) and (got > 0).any() and (got == 0).any()
+
+
+def test_selu(rt):
+    x = util.normal(450, 1000 + 3, 2.0)
+    alpha, gamma = 1.6732631921768188, 1.0507010221481323
+    got = run_chain(rt, x, [(R.ACT_SELU, alpha, gamma)])
+    want = ob.unary_chain(x, [(R.ACT_SELU, alpha, gamma)])
+    ref = gamma * (np.maximum(0, x.astype(np.float64)) + np.minimum(0, alpha * (np.exp(x.astype(np.float64)) - 1)))
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6) and np.allclose(want, ref, rtol=1e-5, atol=1e-6)
