@@ -304,6 +304,17 @@ def main():
     y = np.empty((batch, dims[-1]), dtype=np.float32)
     rt.call("sofie_hip_download", y.ctypes.data_as(C.c_void_p), sess.y_ptr, C.c_size_t(y.nbytes))
     rt.sync()
+    # host <-> device transfers of one batch, reported next to the resident figure (pageable host memory, as infer(host ptr) uses it)
+    def median_ms(fn):
+        t = []
+        for _ in range(7):
+            t0 = time.perf_counter()
+            fn()
+            rt.sync()
+            t.append((time.perf_counter() - t0) * 1e3)
+        return round(sorted(t)[3], 4)
+    h2d_ms = median_ms(lambda: sess.upload_input(x))
+    d2h_ms = median_ms(lambda: rt.call("sofie_hip_download", y.ctypes.data_as(C.c_void_p), sess.y_ptr, C.c_size_t(y.nbytes)))
     if args.no_cpu:
         cpu, parity = None, None
     else:
@@ -338,6 +349,8 @@ def main():
                                "per-tensor symmetric scales, input resident in HBM (benchmark configuration 2)",
                    "global_batch": batch, "launches_per_step": 4, "wall_ms_per_step": round(wall / args.steps, 5),
                    "ms_per_step_of_5_regions": repeats, "median_ms_per_step": sorted(repeats)[2],
+                   "h2d_ms_per_batch": h2d_ms, "d2h_ms_per_batch": d2h_ms,
+                   "inferences_per_s_with_transfers": round(batch / ((ms_per_step + h2d_ms + d2h_ms) * 1e-3), 1),
                    "parity_vs_oracle_rows": args.cpu_rows, "parity_bit_exact": parity,
                    "mlp_tops": round(ops_per_inference_batch / (ms_per_step * 1e-3) / 1e12, 2),
                    "mlp_algorithmic_bytes": algo_bytes,
