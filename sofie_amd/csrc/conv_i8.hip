@@ -157,6 +157,17 @@ static bool conv_i8_implicit_shape(const sofie_conv_desc *d, int x_layout)
           d->C % 16 == 0 && reach < (1LL << 31) && rows < (1LL << 31);
 }
 
+// The whole reduction (taps x channels per group) fits one 64-byte slab: the rows are gathered inside the GEMM kernel.
+static bool conv_i8_gather_shape(const sofie_conv_desc *d)
+{
+   if (d->group <= 0 || d->C % d->group != 0)
+      return false;
+   const long long K = (long long)(d->C / d->group) * d->kh * d->kw;
+   const char *force = getenv("SOFIE_HIP_CONV_EXPLICIT");
+   return !(force && atoi(force)) && K <= 64 && (long long)(d->kh - 1) * d->dil_h <= 127 && (long long)(d->kw - 1) * d->dil_w <= 127 &&
+          (long long)d->C * d->H * d->W < (1LL << 31) && (long long)d->N * d->OH * d->OW < (1LL << 31);
+}
+
 size_t sofie_hip_conv_i8_workspace(const sofie_conv_desc *d, const sofie_conv_i8_args *a)
 {
    if (!d || !a || d->group <= 0)
@@ -164,7 +175,7 @@ size_t sofie_hip_conv_i8_workspace(const sofie_conv_desc *d, const sofie_conv_i8
    size_t K = (size_t)(d->C / d->group) * d->kh * d->kw;
    size_t Kp = (K + 15) & ~(size_t)15;
    // the column matrix of one image, unless the kernel reads the activations directly
-   size_t need = conv_i8_implicit_shape(d, a->x_layout) ? 0 : round256((size_t)d->OH * d->OW * Kp);
+   size_t need = (conv_i8_implicit_shape(d, a->x_layout) || conv_i8_gather_shape(d)) ? 0 : round256((size_t)d->OH * d->OW * Kp);
    if (!a->w_is_packed)
       need += sofie_hip_conv_weight_i8_packed_bytes(d);
    return need;
@@ -249,6 +260,48 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
          }
          return SOFIE_HIP_OK;
       }
+   }
+   // Few input channels (the first layer of an image network): K = taps x channels <= 64 is one slab, gathered in the kernel.
+   if (conv_i8_gather_shape(d) && (((uintptr_t)Wp & 15) == 0)) {
+      const long long rows = (long long)d->N * OHW;
+      const bool nhwc = a->x_layout == SOFIE_LAYOUT_NHWC;
+      for (int grp = 0; grp < d->group; ++grp) {
+         GatherConvRows src;
+         src.X = a->X + (nhwc ? (size_t)grp * g.Cg : (size_t)grp * g.Cg * d->H * d->W);
+         src.H = d->H; src.W = d->W; src.OH = g.OH; src.OW = g.OW;
+         src.stride_h = d->stride_h; src.stride_w = d->stride_w; src.pad_h0 = d->pad_h0; src.pad_w0 = d->pad_w0;
+         src.pix_mul = nhwc ? d->C : 1;
+         src.img_stride = (long long)d->C * d->H * d->W;
+         src.K = g.K;
+         for (int k = 0; k < 64; ++k) {
+            src.koff[k] = 0;
+            src.dy[k] = src.dx[k] = 0;
+            if (k < g.K) {
+               const int ci = k % g.Cg, tap = k / g.Cg; // the order of the packed weights: tap-major, channel-minor
+               const int dy = (tap / d->kw) * d->dil_h, dx = (tap % d->kw) * d->dil_w;
+               src.dy[k] = (signed char)dy;
+               src.dx[k] = (signed char)dx;
+               src.koff[k] = nhwc ? (dy * d->W + dx) * d->C + ci : ci * d->H * d->W + dy * d->W + dx;
+            }
+         }
+         I8Epilogue ep;
+         ep.bias = a->bias;
+         ep.scale = a->scale;
+         ep.scale_scalar = 1.0f;
+         ep.q_scale = 1.0f;
+         ep.relu_acc = (a->out == SOFIE_I8OUT_I32) ? a->relu : 0;
+         ep.relu_out = (a->out == SOFIE_I8OUT_I32) ? 0 : a->relu;
+         ep.out = a->out;
+         ep.ldy = d->Cout;
+         ep.N = Cout_g;
+         ep.n_offset = grp * Cout_g;
+         ep.nchw_ohw = (a->y_layout == SOFIE_LAYOUT_NHWC) ? 0 : OHW;
+         ep.Y = a->Y;
+         st = conv_i8_gather(ctx->stream, src, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.Kp, ep);
+         if (st)
+            return st;
+      }
+      return SOFIE_HIP_OK;
    }
    const size_t per_image = (size_t)OHW * g.Kp;
    SOFIE_HIP_REQUIRE(ws != nullptr && ws_left >= per_image,

@@ -51,6 +51,17 @@ int conv_i8_implicit(hipStream_t stream, const ConvRows &src, int Cg, const int8
    return launch_mfma8_conv<I8Epilogue>(stream, src, Cg, Wp, M, N, K, ep, force_tile);
 }
 
+int conv_i8_gather(hipStream_t stream, const GatherConvRows &src, const int8_t *Wp, int M, int N, int Kp, I8Epilogue ep)
+{
+   const size_t esz = ep.out == SOFIE_I8OUT_I32 || ep.out == SOFIE_I8OUT_F32 ? 4 : 1;
+   ep.N = N;
+   ep.stage_ok = (ep.nchw_ohw == 0) && (((size_t)ep.ldy * esz) % 16 == 0) && (((size_t)ep.n_offset * esz) % 16 == 0) &&
+                 (((uintptr_t)ep.Y & 15) == 0);
+   ep.vec_param = (ep.n_offset % 4 == 0) && (!ep.bias || ((uintptr_t)ep.bias & 15) == 0) &&
+                  (!ep.scale || ((uintptr_t)ep.scale & 15) == 0);
+   return launch_mfma8_gather<I8Epilogue>(stream, src, Wp, M, N, Kp, ep);
+}
+
 // SOFIE_HIP_I8_TILE=256|128|64 forces a tile configuration (tuning and tests); unset = heuristic.
 int forced_i8_tile()
 {

@@ -131,6 +131,8 @@ struct I8Epilogue {
 int gemm_i8_nt(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep,
                int force_tile);
 int forced_i8_tile();
+// Convolution whose whole reduction fits one 64-byte slab (few input channels): rows gathered byte by byte, one launch.
+int conv_i8_gather(hipStream_t stream, const GatherConvRows &src, const int8_t *Wp, int M, int N, int Kp, I8Epilogue ep);
 // Convolution as an implicit GEMM: rows of A come from `src`, Wp is [N][K] with K = taps * Cg.
 int conv_i8_implicit(hipStream_t stream, const ConvRows &src, int Cg, const int8_t *Wp, int M, int N, int K, I8Epilogue ep,
                      int force_tile);

@@ -112,6 +112,7 @@ __device__ __forceinline__ int lds_chunk_offset(int r, int c)
 //   init(st, i, m0, row, cbyte, M)   load i of this lane fills tile row `row` with the 16 bytes at slab offset cbyte
 //   load_ptr(st, i, koff)     global address of those bytes for the slab that starts at reduction offset koff
 struct RowMajorRows {
+   static constexpr bool kGather = false;
    const int8_t *base;
    int ld;
    __device__ __forceinline__ const int8_t *row(int r) const { return base + (size_t)r * (size_t)ld; }
@@ -133,6 +134,43 @@ struct RowMajorRows {
    {
       return (st.tile + koff) + st.off[i];
    }
+};
+
+// Rows of a convolution over few input channels (an RGB image: K = 3 * 3 * 3 = 27): GEMM row = output pixel, K = (tap, channel),
+// K <= 64, so one 64-byte slab holds the whole reduction.  A lane gathers the bytes of ITS pixel one k at a time; for a
+// given k the 64 lanes of a wave read 64 neighbouring pixels, i.e. (almost) consecutive bytes of one input plane.  The
+// per-k offsets are tables in the kernel arguments, indexed by compile-time constants after unrolling.
+struct GatherConvRows {
+   static constexpr bool kGather = true;
+   const int8_t *X;
+   int H, W, OH, OW, stride_h, stride_w, pad_h0, pad_w0;
+   int pix_mul;          // elements between horizontally adjacent pixels: 1 (NCHW) or C (NHWC)
+   long long img_stride; // elements per image
+   int K;
+   int koff[64];         // offset of (channel, ky, kx) from the pixel at (ih0, iw0)
+   signed char dy[64], dx[64];
+   struct row_ref {
+      const int8_t *origin; // address of channel 0 at (ih0, iw0); only dereferenced where the tap lies inside the image
+      int ih0, iw0;
+   };
+   __device__ __forceinline__ row_ref ref_of(int m, int M) const
+   {
+      const int r = m < M ? m : M - 1; // rows past the edge re-read the last row (their outputs are not stored)
+      const int ohw = OH * OW;
+      const int img = r / ohw, rem = r - img * ohw;
+      const int oh = rem / OW, ow = rem - oh * OW;
+      row_ref f;
+      f.ih0 = oh * stride_h - pad_h0;
+      f.iw0 = ow * stride_w - pad_w0;
+      f.origin = X + (long long)img * img_stride + ((long long)f.ih0 * W + f.iw0) * pix_mul;
+      return f;
+   }
+};
+// The same with the padded reduction length (16, 32, 48 or 64) as a compile-time constant: the gather loop has no
+// run-time bounds.  Entries from K up to KP are padding and read as zero.
+template <int KP>
+struct GatherConvRowsT : GatherConvRows {
+   static constexpr int kKP = KP;
 };
 
 // 256 zero bytes: what a load of a padded (out-of-image) position reads.

@@ -44,8 +44,8 @@ constexpr size_t mfma8_general_lds_bytes()
    return ring > store ? ring : store;
 }
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool ALIGNED, class EPI>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_kernel(RowMajorRows A, RowMajorRows Bt, int M, int N,
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool ALIGNED, class EPI, class ASRC = RowMajorRows>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_kernel(ASRC A, RowMajorRows Bt, int M, int N,
                                                                             int K, EPI ep, int tiles_m, int tiles_n, int sw)
 {
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
@@ -82,10 +82,44 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_kernel(RowMa
    // global -> register staging: chunk id = t + i*NTHREADS -> (row, chunk)
    v4i ra[A_LD], rb[B_LD];
    const int8_t *a_row[A_LD], *b_row[B_LD];
+   if constexpr (!ASRC::kGather) {
 #pragma unroll
-   for (int i = 0; i < A_LD; ++i) {
-      int gr = m0 + (t + i * NTHREADS) / CPR;
-      a_row[i] = A.row(gr < M ? gr : M - 1);
+      for (int i = 0; i < A_LD; ++i) {
+         int gr = m0 + (t + i * NTHREADS) / CPR;
+         a_row[i] = A.row(gr < M ? gr : M - 1);
+      }
+   } else {
+      // the whole reduction is one slab: every lane gathers the 64 bytes of its own row (pixel)
+      static_assert(!ASRC::kGather || (BM == NTHREADS && BK == 64), "the gathered source fills one row per thread of one 64-byte slab");
+      const auto ref = A.ref_of(m0 + t, M);
+      unsigned w[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+         w[i] = 0;
+      // every load is issued unconditionally (a tap outside the image reads the first byte of the tensor instead and is
+      // masked afterwards), so that the loads of a row are in flight together instead of one memory round trip per tap
+      constexpr int KP = ASRC::kKP;
+      unsigned v[KP];
+      unsigned ok_lo = 0, ok_hi = 0; // bit k: tap k lies inside the image
+#pragma unroll
+      for (int k = 0; k < KP; ++k) {
+         const int ih = ref.ih0 + A.dy[k], iw = ref.iw0 + A.dx[k];
+         const bool in = k < A.K && (unsigned)ih < (unsigned)A.H && (unsigned)iw < (unsigned)A.W; // k >= K: padding of the reduction
+         if (k < 32)
+            ok_lo |= in ? (1u << (k & 31)) : 0u;
+         else
+            ok_hi |= in ? (1u << (k & 31)) : 0u;
+         const int8_t *p = in ? ref.origin + A.koff[k] : A.X;
+         v[k] = (unsigned char)*p;
+      }
+#pragma unroll
+      for (int k = 0; k < KP; ++k) {
+         const unsigned bit = ((k < 32 ? ok_lo : ok_hi) >> (k & 31)) & 1u;
+         w[k / 4] |= (bit ? v[k] : 0u) << (8 * (k % 4));
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+         *(v4i *)(sA + lds_chunk_offset<BK>(t, c)) = v4i{(int)w[4 * c], (int)w[4 * c + 1], (int)w[4 * c + 2], (int)w[4 * c + 3]};
    }
 #pragma unroll
    for (int i = 0; i < B_LD; ++i) {
@@ -93,18 +127,22 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_kernel(RowMa
       b_row[i] = Bt.row(gr < N ? gr : N - 1);
    }
    auto load_global = [&](int k0) {
+      if constexpr (!ASRC::kGather) {
 #pragma unroll
-      for (int i = 0; i < A_LD; ++i)
-         ra[i] = load_chunk<ALIGNED>(a_row[i], k0 + ((t + i * NTHREADS) % CPR) * 16, K);
+         for (int i = 0; i < A_LD; ++i)
+            ra[i] = load_chunk<ALIGNED>(a_row[i], k0 + ((t + i * NTHREADS) % CPR) * 16, K);
+      }
 #pragma unroll
       for (int i = 0; i < B_LD; ++i)
          rb[i] = load_chunk<ALIGNED>(b_row[i], k0 + ((t + i * NTHREADS) % CPR) * 16, K);
    };
    auto store_lds = [&](int stage) {
+      if constexpr (!ASRC::kGather) {
 #pragma unroll
-      for (int i = 0; i < A_LD; ++i) {
-         int id = t + i * NTHREADS;
-         *(v4i *)(sA + stage * BM * BK + lds_chunk_offset<BK>(id / CPR, id % CPR)) = ra[i];
+         for (int i = 0; i < A_LD; ++i) {
+            int id = t + i * NTHREADS;
+            *(v4i *)(sA + stage * BM * BK + lds_chunk_offset<BK>(id / CPR, id % CPR)) = ra[i];
+         }
       }
 #pragma unroll
       for (int i = 0; i < B_LD; ++i) {
@@ -212,6 +250,43 @@ inline int pick_tile(int M, int N, int force_tile)
    if (N > 64 && tiles(128, 128) >= 192)
       return 128;
    return 64;
+}
+
+// Convolution over few input channels as ONE launch: 256 x 64 tiles (one output pixel per thread in the gather), a single
+// 64-byte slab.  Wp is the packed weight [N][Kp], Kp = the reduction length rounded up to 16, at most 64.
+template <class EPI, int KP>
+static int launch_mfma8_gather_kp(hipStream_t stream, const GatherConvRows &a, const int8_t *Wp, int M, int N, const EPI &ep)
+{
+   constexpr int BM = 256, BN = 64, BK = 64;
+   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+   const long long nwg = (long long)tiles_m * tiles_n;
+   if (nwg > 0x7fffffffLL)
+      return fail(SOFIE_HIP_ERR_INVALID, "conv: too many tiles");
+   constexpr size_t smem = mfma8_general_lds_bytes<BM, BN, BK, 4, 1>();
+   auto kern = mfma8_gemm_kernel<MfmaI8, BM, BN, BK, 4, 1, true, EPI, GatherConvRowsT<KP>>;
+   static bool configured[64] = {};
+   if (int st = configure_lds_once(kern, smem, configured))
+      return st;
+   GatherConvRowsT<KP> src;
+   static_cast<GatherConvRows &>(src) = a;
+   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), smem, stream, src, RowMajorRows{Wp, KP}, M, N, KP, ep, tiles_m, tiles_n, 0);
+   return launch_status("mfma8_gemm_kernel (gathered convolution)");
+}
+
+// Convolution over few input channels as ONE launch: 256 x 64 tiles (one output pixel per thread in the gather), a single
+// 64-byte slab.  Wp is the packed weight [N][Kp], Kp = the reduction length rounded up to 16, at most 64.
+template <class EPI>
+static int launch_mfma8_gather(hipStream_t stream, const GatherConvRows &a, const int8_t *Wp, int M, int N, int Kp, const EPI &ep)
+{
+   if (a.K > Kp)
+      return fail(SOFIE_HIP_ERR_INVALID, "conv: the gathered form needs a reduction of at most 64 bytes");
+   switch (Kp) {
+   case 16: return launch_mfma8_gather_kp<EPI, 16>(stream, a, Wp, M, N, ep);
+   case 32: return launch_mfma8_gather_kp<EPI, 32>(stream, a, Wp, M, N, ep);
+   case 48: return launch_mfma8_gather_kp<EPI, 48>(stream, a, Wp, M, N, ep);
+   case 64: return launch_mfma8_gather_kp<EPI, 64>(stream, a, Wp, M, N, ep);
+   default: return fail(SOFIE_HIP_ERR_INVALID, "conv: the gathered form needs a reduction of at most 64 bytes");
+   }
 }
 
 template <class MMA, class EPI>

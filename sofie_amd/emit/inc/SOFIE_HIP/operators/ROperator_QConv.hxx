@@ -139,9 +139,15 @@ public:
       return fXLayout == kLayoutNHWC && (cg & (cg - 1)) == 0 && cg >= 64 && taps <= 32 && fGeo.C % 16 == 0 && xbytes < 2.0e9 &&
              (double)fGeo.N * fGeo.OH * fGeo.OW < 2.0e9 && taps <= 32;
    }
+   // the runtime's rule for gathering the rows inside the kernel: the whole reduction fits one 64-byte slab
+   bool GatheredGemm() const
+   {
+      return (fGeo.C / fGeo.group) * fGeo.kh * fGeo.kw <= 64 && (fGeo.kh - 1) * fGeo.dil_h <= 127 && (fGeo.kw - 1) * fGeo.dil_w <= 127 &&
+             (double)fGeo.C * fGeo.H * fGeo.W < 2.0e9 && (double)fGeo.N * fGeo.OH * fGeo.OW < 2.0e9;
+   }
    std::size_t GetWorkspaceBytes() override
    {
-      if (ImplicitGemm())
+      if (ImplicitGemm() || GatheredGemm())
          return 0;
       const std::size_t per_image = (fGeo.OH * fGeo.OW * PackedK() + 255) / 256 * 256;
       std::size_t images = std::max<std::size_t>(1, (std::size_t(64) << 20) / per_image);
@@ -154,7 +160,7 @@ public:
       opName = "op_" + opName;
       std::stringstream out;
       out << "\n" << SP << "//----  operator " << (fInt32Out ? "ConvInteger " : "QLinearConv ") << opName << " --> " << ConvertShapeToString(fGeo.OutputShape())
-          << (fYLayout == kLayoutNHWC ? " (stored NHWC)" : "") << (ImplicitGemm() ? ", implicit GEMM" : ", column matrix") << "\n";
+          << (fYLayout == kLayoutNHWC ? " (stored NHWC)" : "") << (ImplicitGemm() ? ", implicit GEMM" : GatheredGemm() ? ", rows gathered in the kernel" : ", column matrix") << "\n";
       out << SP << "{\n";
       out << SP << "   " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n" << fGeo.BatchLine(fDynamic, SP + "   ");
       out << SP << "   " << "sofie_conv_i8_args a{};\n";

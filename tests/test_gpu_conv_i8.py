@@ -60,7 +60,12 @@ def run_conv(rt, X, Wt, bias, scale, case, relu, out, x_layout, y_layout, packed
 
 @pytest.mark.parametrize("case", CASES)
 @pytest.mark.parametrize("x_layout,y_layout,packed", [(0, 0, 0), (1, 1, 1), (0, 1, 0), (1, 0, 1)])
-def test_conv_i8_requant_bit_exact(rt, case, x_layout, y_layout, packed):
+@pytest.mark.parametrize("column_matrix", [0, 1])
+def test_conv_i8_requant_bit_exact(rt, case, x_layout, y_layout, packed, column_matrix, monkeypatch):
+    # column_matrix = 1 forces the explicit int8 im2col + GEMM; 0 lets the runtime choose: reductions of at most 64 bytes
+    # (the first six cases) are gathered inside the GEMM kernel, 64-channel NHWC input takes the implicit GEMM
+    if column_matrix:
+        monkeypatch.setenv("SOFIE_HIP_CONV_EXPLICIT", "1")
     N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
     X = util.int8_sym(50, N * Cc * H * W).reshape(N, Cc, H, W)
     Wt = util.int8_sym(51, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
@@ -121,3 +126,20 @@ def test_conv_i8_implicit_gemm_every_tile(rt, case, tile, monkeypatch):
     monkeypatch.delenv("SOFIE_HIP_I8_TILE")
     got2 = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, R.LAYOUT_NHWC, R.LAYOUT_NCHW, 1)
     assert np.array_equal(got2, want)
+
+
+def test_first_layer_of_an_image_network_needs_no_workspace(rt):
+    """3 input channels, 3x3: K = 27 fits one slab, the rows are gathered in the kernel (NCHW in, NHWC out, a ragged last tile)."""
+    case = (3, 3, 21, 19, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1)
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    d = conv_desc(N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group)
+    a = R.ConvI8Args()
+    a.x_layout, a.y_layout, a.w_is_packed = R.LAYOUT_NCHW, R.LAYOUT_NHWC, 1
+    assert rt.lib.sofie_hip_conv_i8_workspace(C.byref(d), C.byref(a)) == 0
+    X = util.int8_sym(90, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.int8_sym(91, Cout * Cc * 9).reshape(Cout, Cc, 3, 3)
+    bias = util.int32_range(92, Cout, -500, 500)
+    scale = ((0.5 + util.uniform01(93, Cout)) / np.float32(127.0 * np.sqrt(27))).astype(np.float32)
+    want = ob.conv_i8(X, Wt, bias, scale, pads=pads, strides=strides, dils=dils, group=group, relu=1, out=2, omp=True)
+    got = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, R.LAYOUT_NCHW, R.LAYOUT_NHWC, 1, ws_images=0)
+    assert np.array_equal(got, want) and (want > 0).any()
