@@ -304,6 +304,26 @@ int sofie_hip_pack_conv_weight_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, 
  * Y[n,c] = (sum over the HW plane of X[n,c,:]) / float(HW); the fp32 sum is a tree reduction, so it
  * agrees with the reference's sequential loop to rounding only. */
 int sofie_hip_global_avg_pool_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t NC, int32_t HW);
+/* MaxPool / AveragePool over 1-D and 2-D windows of an NCHW tensor, the loops of ROperator_Pool<float>::Generate
+ * (core/inc/SOFIE/operators/ROperator_Pool.hxx:286-412): the window of output (oh, ow) starts at
+ * (oh*stride_h - pad_h0, ow*stride_w - pad_w0) and spans kh x kw positions (for a dilated MaxPool kh, kw are the DILATED
+ * extents and every position inside is visited, as the reference does); positions outside the image are skipped.
+ * MaxPool: the largest value met (-inf for an empty window; NaN never wins `x > value`).  AveragePool: the fp32 sum in
+ * row-major window order, divided by float(nsum): nsum = kh*kw when `dynamic_divisor` is 0, else per dimension
+ * min(start + k, hi) - lo with hi = size (+ end padding if count_include_pad), lo = start (clamped at 0 unless
+ * count_include_pad) -- the reference's windowExtent (:328-333).  1-D pooling passes H = OH = kh = 1. */
+enum { SOFIE_POOL_MAX = 0, SOFIE_POOL_AVERAGE = 1 };
+typedef struct sofie_pool_desc {
+   int32_t planes; /* N * C */
+   int32_t H, W, OH, OW;
+   int32_t kh, kw;
+   int32_t pad_h0, pad_w0, pad_h1, pad_w1;
+   int32_t stride_h, stride_w;
+   int32_t mode; /* SOFIE_POOL_* */
+   int32_t count_include_pad;
+   int32_t dynamic_divisor; /* the reference sets it when any padding is non-zero or ceil_mode is on */
+} sofie_pool_desc;
+int sofie_hip_pool_f32(sofie_hip_ctx *ctx, const sofie_pool_desc *d, float *Y, const float *X);
 /* int8 input, fp32 output: Y = (float(sum_i32) * scale) / float(HW), exact sum -- not in the reference. */
 int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y /* [N,C] */, const int8_t *X, int32_t N, int32_t C, int32_t HW,
                                  int32_t x_layout /* SOFIE_LAYOUT_* */, float scale);

@@ -128,6 +128,52 @@ def global_avg_pool(X):
     return Y
 
 
+def pool_axes(in_shape, kernel_shape, pads=None, strides=None, dilations=None, auto_pad="NOTSET", ceil_mode=0):
+    """Per spatial axis (in, out, window, stride, pad_begin, pad_end): the attribute resolution and output extent of
+    core/inc/SOFIE/operators/ROperator_Pool.hxx:107-171 (window = dilated extent, SAME_* padding, ceil_mode limit)."""
+    nd = len(in_shape)
+    axes = []
+    for d in range(nd):
+        n_in = int(in_shape[d])
+        k = int(kernel_shape[d]) if kernel_shape else n_in
+        dil = int(dilations[d]) if dilations else 1
+        stride = int(strides[d]) if strides else 1
+        window = k + (dil - 1) * (k - 1)
+        pb = pe = 0
+        if auto_pad == "NOTSET":
+            if pads:
+                pb, pe = int(pads[d]), int(pads[d + nd])
+        elif auto_pad in ("SAME_UPPER", "SAME_LOWER"):
+            out_same = (n_in + stride - 1) // stride
+            total = max(0, (out_same - 1) * stride + window - n_in)
+            pb, pe = (total // 2, total - total // 2) if auto_pad == "SAME_UPPER" else (total - total // 2, total // 2)
+        elif auto_pad != "VALID":
+            raise ValueError("invalid auto_pad " + auto_pad)
+        n = n_in + pb + pe - window
+        out = min((n + stride - 1) // stride, (n_in - 1 + pb) // stride) + 1 if ceil_mode else n // stride + 1
+        axes.append((n_in, out, window, stride, pb, pe))
+    return axes
+
+
+def pool(X, mode, kernel_shape, pads=None, strides=None, dilations=None, auto_pad="NOTSET", ceil_mode=0, count_include_pad=0):
+    """MaxPool (mode "max") / AveragePool (mode "average") of an [N, C, W] or [N, C, H, W] tensor."""
+    X = _f32(X)
+    axes = pool_axes(X.shape[2:], kernel_shape, pads, strides, dilations, auto_pad, ceil_mode)
+    if len(axes) == 1:
+        axes = [(1, 1, 1, 1, 0, 0)] + axes
+    (H, OH, kh, sh, ph0, ph1), (W, OW, kw, sw, pw0, pw1) = axes
+    planes = X.shape[0] * X.shape[1]
+    Y = np.empty(X.shape[:2] + ((OH, OW) if X.ndim == 4 else (OW,)), dtype=np.float32)
+    lib = load()
+    lib.oracle_pool2d.restype = C.c_long
+    per_plane = lib.oracle_pool2d(_ptr(Y), _ptr(X), planes, H, W, kh, kw, ph0, pw0, ph1, pw1, sh, sw, 1 if mode == "max" else 0,
+                                  int(ceil_mode), int(count_include_pad))
+    # the loops' own count of window positions must be the inferred output shape
+    if planes and per_plane != OH * OW:
+        raise AssertionError("pool: the loops wrote %d outputs per plane, the shape says %d" % (per_plane, OH * OW))
+    return Y
+
+
 def batchnorm(X, scale, bias, mean, var, eps=1e-5, relu=0):
     X = _f32(X)
     Cc = X.shape[1]

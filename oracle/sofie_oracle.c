@@ -19,6 +19,11 @@
  *                             (exp(log x) = x, sin^2 + cos^2 = 1, sinh(asinh x) = x, ...); Clip bounds; Selu
  *                             through the LinearWithSelu golden output.
  *   global_avg_pool           GlobalAvgPool2d golden output.
+ *   pool2d                    MaxPool1d, MaxPool2d, AvgPool, AvgPoolPad, AvgPoolCountIncludePad golden outputs;
+ *                             a float64 restatement of the ONNX definition over random geometries (ceil_mode and
+ *                             both divisor conventions included); torch's max_pool / avg_pool; window = image is
+ *                             global_avg_pool.  The reference's ceil-mode and asymmetric-padding models come
+ *                             without data files: those cases rest on the definition alone.
  *   organize_memory           the reference's MemoryPlanner.inc compiled as oracle/_ref and run on the
  *                             same lifetimes; known totals of the Linear_16 plan.
  *   quantize/dequantize, gemm_i8, conv_i8, e4m3 codec, gemm_fp8
@@ -334,6 +339,62 @@ ORACLE_API void oracle_global_avg_pool(float *Y, const float *X, int NC, int HW)
       value /= (float)HW;
       Y[p] = value;
    }
+}
+
+/* MaxPool / AveragePool in 2-D (1-D: H = kh = 1), the generated loops of core/inc/SOFIE/operators/ROperator_Pool.hxx:
+ * bounds hmin = -pad_begin, hmax = H + pad_end - kh + 1 (ceil_mode: + stride instead of + 1, clipped to H) (:286-300);
+ * window start walks hmin, hmin + stride, ... < hmax (:373-374); MaxPool keeps `xval > value` from -INFINITY (:376,
+ * 394-396); AveragePool sums in window order and divides by float(nsum), nsum = kh*kw without padding and ceil_mode, else
+ * the product of the per-axis extents min(i + kh, hi) - lo (:323-333, 379-384, 403-405).  Returns the number of outputs
+ * written per plane (the caller's output shape must agree). */
+static int oracle_pool_extent(int var, int kern, int size, int pad_end, int include_pad)
+{
+   int hi = include_pad ? size + pad_end : size;
+   int lo = include_pad ? var : (var > 0 ? var : 0);
+   return (var + kern < hi ? var + kern : hi) - lo;
+}
+ORACLE_API long oracle_pool2d(float *Y, const float *X, int planes, int H, int W, int kh, int kw, int pad_h0, int pad_w0, int pad_h1, int pad_w1,
+                              int stride_h, int stride_w, int is_max, int ceil_mode, int count_include_pad)
+{
+   int hmin = -pad_h0, wmin = -pad_w0;
+   int hmax = H + pad_h1 - kh + (ceil_mode ? stride_h : 1);
+   int wmax = W + pad_w1 - kw + (ceil_mode ? stride_w : 1);
+   if (ceil_mode && hmax > H)
+      hmax = H;
+   if (ceil_mode && wmax > W)
+      wmax = W;
+   int dynamic_divisor = ceil_mode || pad_h0 > 0 || pad_w0 > 0 || pad_h1 > 0 || pad_w1 > 0;
+   size_t out = 0;
+   for (int n = 0; n < planes; ++n) {
+      const float *x = X + (size_t)n * H * W;
+      for (int i = hmin; i < hmax; i += stride_h) {
+         for (int j = wmin; j < wmax; j += stride_w) {
+            float value = is_max ? -INFINITY : 0;
+            int nsum = kh * kw;
+            if (!is_max && dynamic_divisor)
+               nsum = oracle_pool_extent(i, kh, H, pad_h1, count_include_pad) * oracle_pool_extent(j, kw, W, pad_w1, count_include_pad);
+            for (int l = i; l < i + kh; l++) {
+               if (l < 0 || l >= H)
+                  continue;
+               for (int m = j; m < j + kw; m++) {
+                  if (m < 0 || m >= W)
+                     continue;
+                  float xval = x[l * W + m];
+                  if (is_max) {
+                     if (xval > value)
+                        value = xval;
+                  } else {
+                     value += xval;
+                  }
+               }
+            }
+            if (!is_max)
+               value /= (float)nsum;
+            Y[out++] = value;
+         }
+      }
+   }
+   return planes ? (long)(out / (size_t)planes) : 0;
 }
 
 /* BatchNormalization at inference (core/inc/SOFIE/operators/ROperator_BatchNormalization.hxx:92-109, 139-148):

@@ -73,6 +73,48 @@ __global__ __launch_bounds__(256) void unary_f32_kernel(float *dst, const float 
    }
 }
 
+// One output element per thread (grid-stride); neighbouring lanes take neighbouring ow, so the window rows they read
+// overlap and lie next to each other in memory.  The sum of an average runs in the reference's order (window rows
+// outermost), one fp32 addition at a time, so the result has the bits of the reference's scalar loop.
+__global__ __launch_bounds__(256) void pool_f32_kernel(float *__restrict__ Y, const float *__restrict__ X, sofie_pool_desc d, size_t total)
+{
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += stride) {
+      const int ow = (int)(idx % (size_t)d.OW);
+      const size_t t = idx / (size_t)d.OW;
+      const int oh = (int)(t % (size_t)d.OH);
+      const size_t plane = t / (size_t)d.OH;
+      const int i = oh * d.stride_h - d.pad_h0, j = ow * d.stride_w - d.pad_w0;
+      const float *x = X + plane * (size_t)d.H * (size_t)d.W;
+      float value = d.mode == SOFIE_POOL_MAX ? -INFINITY : 0.0f;
+      for (int l = i; l < i + d.kh; ++l) {
+         if (l < 0 || l >= d.H)
+            continue;
+         for (int m = j; m < j + d.kw; ++m) {
+            if (m < 0 || m >= d.W)
+               continue;
+            const float xv = x[(size_t)l * d.W + m];
+            if (d.mode == SOFIE_POOL_MAX) {
+               if (xv > value)
+                  value = xv;
+            } else {
+               value += xv;
+            }
+         }
+      }
+      if (d.mode == SOFIE_POOL_AVERAGE) {
+         int nsum = d.kh * d.kw;
+         if (d.dynamic_divisor) {
+            const int hi_h = d.count_include_pad ? d.H + d.pad_h1 : d.H, hi_w = d.count_include_pad ? d.W + d.pad_w1 : d.W;
+            const int lo_h = d.count_include_pad ? i : (i > 0 ? i : 0), lo_w = d.count_include_pad ? j : (j > 0 ? j : 0);
+            nsum = ((i + d.kh < hi_h ? i + d.kh : hi_h) - lo_h) * ((j + d.kw < hi_w ? j + d.kw : hi_w) - lo_w);
+         }
+         value = __fdiv_rn(value, (float)nsum);
+      }
+      Y[idx] = value;
+   }
+}
+
 struct AddShape {
    int rank;
    long long y[6], sa[6], sb[6]; // output dims, element strides of A and B (0 where broadcast)
@@ -309,6 +351,26 @@ int sofie_hip_batchnorm_f32(sofie_hip_ctx *ctx, float *Y, const float *X, const 
    const size_t n = (size_t)N * (size_t)C * (size_t)spatial;
    hipLaunchKernelGGL(batchnorm_f32_kernel, dim3(grid_for(n)), dim3(256), 0, ctx->stream, Y, X, fused_scale, mean, bias, n, C, spatial, relu);
    return launch_status("batchnorm_f32_kernel");
+}
+
+int sofie_hip_pool_f32(sofie_hip_ctx *ctx, const sofie_pool_desc *d, float *Y, const float *X)
+{
+   SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_pool_f32: NULL argument");
+   SOFIE_HIP_REQUIRE(d->planes >= 0 && d->H > 0 && d->W > 0 && d->OH > 0 && d->OW > 0 && d->kh > 0 && d->kw > 0, "sofie_hip_pool_f32: bad shape");
+   SOFIE_HIP_REQUIRE(d->stride_h > 0 && d->stride_w > 0, "sofie_hip_pool_f32: bad stride");
+   SOFIE_HIP_REQUIRE(d->pad_h0 >= 0 && d->pad_w0 >= 0 && d->pad_h1 >= 0 && d->pad_w1 >= 0, "sofie_hip_pool_f32: negative padding");
+   SOFIE_HIP_REQUIRE(d->mode == SOFIE_POOL_MAX || d->mode == SOFIE_POOL_AVERAGE, "sofie_hip_pool_f32: unknown mode %d", d->mode);
+   // every window start must lie where the reference's loops put it: the last one begins inside the padded image
+   SOFIE_HIP_REQUIRE((long long)(d->OH - 1) * d->stride_h - d->pad_h0 < d->H + d->pad_h1 &&
+                        (long long)(d->OW - 1) * d->stride_w - d->pad_w0 < d->W + d->pad_w1,
+                     "sofie_hip_pool_f32: the output shape %dx%d does not fit the padded input", d->OH, d->OW);
+   const long long total = (long long)d->planes * d->OH * d->OW;
+   SOFIE_HIP_REQUIRE(total < (1LL << 40) && (long long)d->planes * d->H * d->W < (1LL << 40), "sofie_hip_pool_f32: tensor too large");
+   if (total == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(Y && X, "sofie_hip_pool_f32: NULL pointer");
+   hipLaunchKernelGGL(pool_f32_kernel, dim3(grid_for((size_t)total)), dim3(256), 0, ctx->stream, Y, X, *d, (size_t)total);
+   return launch_status("pool_f32_kernel");
 }
 
 int sofie_hip_global_avg_pool_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t NC, int32_t HW)

@@ -545,6 +545,23 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
                                                                     n.in[1], bias, out));
       } else if (n.op == "GlobalAveragePool") {
          model->AddOperator(std::make_unique<ROperator_Pool<float>>(GlobalAveragePool, n.in[0], n.out[0]));
+      } else if (n.op == "MaxPool" || n.op == "AveragePool") {
+         // attributes as parsers/src/ParsePool.cxx:37-63 reads them: count_include_pad belongs to AveragePool,
+         // storage_order and dilations to MaxPool
+         const bool isMax = n.op == "MaxPool";
+         if (n.out.size() > 1 && !n.out[1].empty())
+            throw std::runtime_error("SOFIE ONNX parser: MaxPool " + n.name + " asks for the Indices output, which is not supported");
+         RAttributes_Pool attr;
+         attr.auto_pad = attrS(n, "auto_pad", "NOTSET");
+         attr.ceil_mode = (int)attrI(n, "ceil_mode", 0);
+         attr.count_include_pad = isMax ? 0 : (int)attrI(n, "count_include_pad", 0);
+         attr.storage_order = isMax ? (int)attrI(n, "storage_order", 0) : 0;
+         if (isMax)
+            attr.dilations = attrV(n, "dilations");
+         attr.kernel_shape = attrV(n, "kernel_shape");
+         attr.pads = attrV(n, "pads");
+         attr.strides = attrV(n, "strides");
+         model->AddOperator(std::make_unique<ROperator_Pool<float>>(isMax ? MaxPool : AveragePool, attr, n.in[0], n.out[0]));
       } else if (n.op == "QuantizeLinear") {
          model->AddOperator(std::make_unique<ROperator_QuantizeLinear>(n.in[0], n.in[1], n.out[0]));
       } else if (n.op == "DequantizeLinear") {

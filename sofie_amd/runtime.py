@@ -75,6 +75,14 @@ class ConvDesc(C.Structure):
                 ("dil_h", C.c_int32), ("dil_w", C.c_int32), ("group", C.c_int32), ("OH", C.c_int32), ("OW", C.c_int32)]
 
 
+class PoolDesc(C.Structure):
+    _fields_ = [(name, C.c_int32) for name in ("planes", "H", "W", "OH", "OW", "kh", "kw", "pad_h0", "pad_w0", "pad_h1", "pad_w1",
+                                               "stride_h", "stride_w", "mode", "count_include_pad", "dynamic_divisor")]
+
+
+POOL_MAX, POOL_AVERAGE = 0, 1
+
+
 class ConvI8Args(C.Structure):
     _fields_ = [("X", C.c_void_p), ("W", C.c_void_p), ("bias", C.c_void_p), ("scale", C.c_void_p),
                 ("relu", C.c_int32), ("out", C.c_int32), ("x_layout", C.c_int32), ("y_layout", C.c_int32),
@@ -116,6 +124,7 @@ SYMBOLS = {
     "sofie_hip_conv_i8_workspace": (C.c_size_t, [C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
     "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),
     "sofie_hip_global_avg_pool_f32": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32]),
+    "sofie_hip_pool_f32": (C.c_int, [_P, _P, _P, _P]),
     "sofie_hip_batchnorm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "sofie_hip_global_avg_pool_i8": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float]),
     "sofie_hip_conv_weight_i8_packed_bytes": (C.c_size_t, [C.POINTER(ConvDesc)]),

@@ -128,6 +128,21 @@ def conv_batchnorm_relu(batch=2):
     return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 3, 10, 10])], outputs=[("Y", np.float32, [batch, 8, 1, 1])], init=init, feeds=[X])
 
 
+def conv_pool_stack(batch=2):
+    """Conv 3x3 -> Relu -> MaxPool 3x3 / stride 2 / pad 1 (the stem of a residual network) -> AveragePool 2x2 / stride 2 with
+    ceil_mode over an odd image (the last window hangs over the edge) -> Flatten -> Gemm."""
+    init = {"W": util.normal(6201, 6 * 3 * 9, 0.3).reshape(6, 3, 3, 3), "b": util.normal(6202, 6, 0.1),
+            "F": util.normal(6203, 6 * 3 * 3 * 5, 0.2).reshape(54, 5), "c": util.normal(6204, 5, 0.1)}
+    nodes = [ow.node("Conv", ["X", "W", "b"], ["C"], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1]),
+             ow.node("Relu", ["C"], ["R"]),
+             ow.node("MaxPool", ["R"], ["M"], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[2, 2]),
+             ow.node("AveragePool", ["M"], ["A"], kernel_shape=[2, 2], strides=[2, 2], ceil_mode=1),
+             ow.node("Flatten", ["A"], ["L"], axis=1),
+             ow.node("Gemm", ["L", "F", "c"], ["Y"])]
+    X = util.normal(6205, batch * 3 * 10 * 10).reshape(batch, 3, 10, 10)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 3, 10, 10])], outputs=[("Y", np.float32, [batch, 5])], init=init, feeds=[X])
+
+
 def qlinear_matmul_relu(M=16, K=64, N=48):
     """QuantizeLinear -> QLinearMatMul (per-column weight scales) -> Relu (int8) -> DequantizeLinear."""
     W = util.int8_sym(7101, K * N).reshape(K, N)
@@ -303,6 +318,7 @@ DYNAMIC_MODELS = {    "Dynamic_ResidualBlock": lambda: with_named_batch(residual
     "Dynamic_int8_MLP": lambda: with_named_batch(int8_mlp([64, 128, 96, 32], 48), "batch_size"),
     "Dynamic_int8_CNN": lambda: with_named_batch(int8_cnn(2, 12), "N"),
     "Dynamic_ConvBatchNormRelu": lambda: with_named_batch(conv_batchnorm_relu(2), "bs"),
+    "Dynamic_ConvPoolStack": lambda: with_named_batch(conv_pool_stack(2), "N"),
 }
 
 CONFIG_MODELS = {
@@ -310,6 +326,7 @@ CONFIG_MODELS = {
     "QLinearMatMulRelu": lambda: qlinear_matmul_relu(),
     "ConvIntegerDequantize": lambda: conv_integer_dequantize(),
     "ConvBatchNormRelu": lambda: conv_batchnorm_relu(2),
+    "ConvPoolStack": lambda: conv_pool_stack(2),
     "Config5_int8_CNN_small": lambda: int8_cnn(2, 12),
     "Config1_fp32_MLP": lambda: fp32_mlp(64),
     "Config2_int8_MLP_small": lambda: int8_mlp([64, 128, 96, 32], 48),

@@ -48,6 +48,7 @@ MODELS = {
     "ConvWithDilation": (None, [IOTA]), "ConvWithBias": (None, [IOTA]), "ConvBatch2": (None, [IOTA]),
     "ConvBatch4": (None, [IOTA]), "ConvBatch8": (None, [IOTA]), "ConvGroup2": (None, [IOTA]), "ConvGroup4": (None, [IOTA]),
     "ConvBatch4Group2": (None, [IOTA]), "Conv1d": (None, [IOTA]), "GlobalAvgPool2d": (None, [IOTA]),
+    "AvgPoolPad": (None, [IOTA]), "AvgPoolCountIncludePad": (None, [IOTA]),
 }
 
 
@@ -73,6 +74,10 @@ def main():
     for model in ("Gelu", "GeluTanh"):
         add(model, arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx"))["outputs"],
             [{"kind": "values", "values": vector_literal(un, model, "input")}])
+    pool = os.path.join(REF, "alpaka/TestAlpakaPool.cxx")
+    for model in ("MaxPool1d", "MaxPool2d", "AvgPool"):
+        add(model, arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx"))["output"],
+            [{"kind": "values", "values": vector_literal(pool, model, "input")}])
     lin = os.path.join(REF, "alpaka/TestAlpakaLinear.cxx")
     add("LinearWithLeakyRelu", arrays_in(os.path.join(REF, "models/onnx/references/LinearWithLeakyRelu.ref.hxx"))["outputs"],
         [{"kind": "values", "values": vector_literal(lin, "LinearWithLeakyRelu", "input")}])

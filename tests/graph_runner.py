@@ -96,6 +96,10 @@ class OracleBackend:
     def gap(self, X):
         return self.ob.global_avg_pool(X)
 
+    def pool(self, X, mode, a):
+        return self.ob.pool(X, mode, a.get("kernel_shape"), a.get("pads"), a.get("strides"), a.get("dilations"), a.get("auto_pad", "NOTSET"),
+                            a.get("ceil_mode", 0), a.get("count_include_pad", 0))
+
     def add(self, A, B):
         return self.ob.add_broadcast(A, B)
 
@@ -179,6 +183,13 @@ class HipBackend:
         self.rt.sync()
         return u.to_host(dY).reshape((N, Cc) + (1,) * (X.ndim - 2))
 
+    def pool(self, X, mode, a):
+        from oracle import binding as ob
+        R, u = self.R, self.u
+        axes = ob.pool_axes(X.shape[2:], a.get("kernel_shape"), a.get("pads"), a.get("strides"), a.get("dilations"), a.get("auto_pad", "NOTSET"),
+                            a.get("ceil_mode", 0))
+        return hip_pool(self.rt, X, mode, axes, a.get("ceil_mode", 0), a.get("count_include_pad", 0))
+
     def add(self, A, B):
         R, u = self.R, self.u
         ysh = np.broadcast_shapes(A.shape, B.shape)
@@ -199,6 +210,26 @@ class HipBackend:
         self.rt.call("sofie_hip_add_f32", C.byref(d))
         self.rt.sync()
         return u.to_host(dY)
+
+
+def hip_pool(rt, X, mode, axes, ceil_mode=0, count_include_pad=0):
+    """sofie_hip_pool_f32 on an [N, C, (H,) W] array; axes = per spatial axis (in, out, window, stride, pad_begin, pad_end)."""
+    import torch
+    from sofie_amd import runtime as R
+    from tests import util as u
+    if len(axes) == 1:
+        axes = [(1, 1, 1, 1, 0, 0)] + list(axes)
+    (H, OH, kh, sh, ph0, ph1), (W, OW, kw, sw, pw0, pw1) = axes
+    d = R.PoolDesc(planes=X.shape[0] * X.shape[1], H=H, W=W, OH=OH, OW=OW, kh=kh, kw=kw, pad_h0=ph0, pad_w0=pw0, pad_h1=ph1, pad_w1=pw1,
+                   stride_h=sh, stride_w=sw, mode=R.POOL_MAX if mode == "max" else R.POOL_AVERAGE, count_include_pad=int(count_include_pad),
+                   dynamic_divisor=int(bool(ceil_mode) or any(v > 0 for v in (ph0, ph1, pw0, pw1))))
+    ysh = X.shape[:2] + ((OH, OW) if X.ndim == 4 else (OW,))
+    dX = u.to_dev(np.ascontiguousarray(X, dtype=np.float32))
+    dY = u.dev_empty(ysh, np.float32)
+    torch.cuda.synchronize()
+    rt.call("sofie_hip_pool_f32", C.byref(d), u.ptr(dY), u.ptr(dX))
+    rt.sync()
+    return u.to_host(dY)
 
 
 # codes of include/sofie_hip.h for the reference's basic unary operators
@@ -247,6 +278,8 @@ def run(g, inputs, be, all_outputs=False):
                 y = y[:, :, 0, :]
         elif op == "GlobalAveragePool":
             y = be.gap(x[0])
+        elif op in ("MaxPool", "AveragePool"):
+            y = be.pool(x[0], "max" if op == "MaxPool" else "average", a)
         elif op == "BatchNormalization":
             from oracle import binding as ob
             y, _ = ob.batchnorm(x[0], x[1], x[2], x[3], x[4], eps=a.get("epsilon", 1e-5))

@@ -437,3 +437,33 @@ def test_safetensors_payload_is_validated_before_any_device_work(emitted, tmp_pa
     rc, msg, _ = attempt(dict(reversed(list(good.items()))), metadata={"producer": "test"})
     if not torch.cuda.is_available():
         assert rc == 1 and "SOFIE HIP runtime error in Session" in msg
+
+
+def test_pool_attributes_resolve_to_the_reference_shapes(emitted, tmp_path):
+    """Output extents of the reference's shape inference (ROperator_Pool.hxx:107-171) as they appear in the emitted call."""
+    def emit_pool(op, shape, name, **attrs):
+        r = _emit(tmp_path, [ow.node(op, ["X"], ["Y"], **attrs)], [("X", np.float32, shape)], [("Y", np.float32, shape)], {}, name=name)
+        return r, (open(os.path.join(str(tmp_path), name + "_GPU_HIP.hxx")).read() if r.returncode == 0 else "")
+    # the reference's own test shapes: 6 -> 2 (MaxPool1d_CeilMode_Overhang), 5x5 -> 3x3 (MaxPool2d_CeilMode), 4x4 -> 3x5 (AsymPad)
+    r, txt = emit_pool("MaxPool", [1, 1, 6], "overhang", kernel_shape=[2], strides=[3], ceil_mode=1)
+    assert r.returncode == 0 and "d.H = 1; d.W = 6; d.OH = 1; d.OW = 2;" in txt and "SOFIE_POOL_MAX" in txt
+    r, txt = emit_pool("MaxPool", [1, 1, 5, 5], "ceil2d", kernel_shape=[2, 2], strides=[2, 2], ceil_mode=1)
+    assert r.returncode == 0 and "d.OH = 3; d.OW = 3;" in txt
+    r, txt = emit_pool("MaxPool", [1, 1, 4, 4], "asym", kernel_shape=[2, 2], pads=[0, 1, 0, 1], strides=[1, 1])
+    assert r.returncode == 0 and "d.OH = 3; d.OW = 5;" in txt and "d.pad_h0 = 0; d.pad_w0 = 1; d.pad_h1 = 0; d.pad_w1 = 1;" in txt
+    # SAME_UPPER puts the odd sample at the end; without padding and ceil_mode the divisor is the constant kh*kw
+    r, txt = emit_pool("AveragePool", [2, 3, 7, 7], "same", kernel_shape=[2, 2], strides=[2, 2], auto_pad="SAME_UPPER", count_include_pad=1)
+    assert r.returncode == 0 and "d.OH = 4; d.OW = 4;" in txt and "d.pad_h0 = 0; d.pad_w0 = 0; d.pad_h1 = 1; d.pad_w1 = 1;" in txt
+    assert "d.count_include_pad = 1; d.dynamic_divisor = 1;" in txt and "d.planes = 6;" in txt
+    r, txt = emit_pool("AveragePool", [2, 3, 8, 8], "plain", kernel_shape=[2, 2], strides=[2, 2])
+    assert r.returncode == 0 and "d.dynamic_divisor = 0;" in txt
+    # refusals name the operator
+    r, _ = emit_pool("MaxPool", [1, 1, 4, 4, 4], "three_d", kernel_shape=[2, 2, 2])
+    assert r.returncode != 0 and "MaxPool" in r.stdout and "spatial" in r.stdout
+    r, _ = emit_pool("MaxPool", [1, 1, 4, 4], "column_major", kernel_shape=[2, 2], storage_order=1)
+    assert r.returncode != 0 and "storage_order" in r.stdout
+    r, _ = emit_pool("AveragePool", [1, 1, 4, 4], "too_big", kernel_shape=[6, 6])
+    assert r.returncode != 0 and "larger than the padded input" in r.stdout
+    r = _emit(tmp_path, [ow.node("MaxPool", ["X"], ["Y", "I"], kernel_shape=[2, 2])], [("X", np.float32, [1, 1, 4, 4])],
+              [("Y", np.float32, [1, 1, 3, 3])], {}, name="indices")
+    assert r.returncode != 0 and "Indices" in r.stdout

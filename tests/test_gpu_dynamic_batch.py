@@ -141,6 +141,20 @@ def test_dynamic_conv_batchnorm_relu(rt):
             assert got.size == w.size and np.abs(got - w).max() <= 1e-5 * max(1.0, float(np.abs(w).max()))
 
 
+def test_dynamic_conv_pool_stack(rt):
+    spec = em.conv_pool_stack(2)
+    g = onnx_lite.load(os.path.join(em.OUT, "ConvPoolStack.onnx"))     # the same weights with a fixed batch of 2
+    x2 = spec["feeds"][0]
+    x = np.concatenate([x2, util.normal(8302, 3 * x2[:1].size).reshape((3,) + x2.shape[1:])])
+    want = gr.run(g, [x], gr.OracleBackend())
+    with DynamicSession("Dynamic_ConvPoolStack", 5) as s:
+        for n in (5, 2, 1):
+            print("Dynamic_ConvPoolStack batch", n, flush=True)
+            got = s.infer(n, [x[:n]], want.size)
+            w = want[:n].ravel()
+            assert got.size == w.size and np.abs(got - w).max() <= 1e-5 * max(1.0, float(np.abs(w).max()))
+
+
 def test_dynamic_batch_through_broadcasting_adds(rt):
     c = em.dynamic_residual()["consts"]
     x, z = util.normal(8401, 9 * 6).reshape(9, 6), util.normal(8402, 9 * 5).reshape(9, 5)

@@ -128,6 +128,19 @@ def test_emitted_conv_batchnorm_relu(rt):
     assert "BatchNorm + ReLU" in txt and "sofie_hip_unary_f32" not in txt   # the Relu is folded into the normalisation
 
 
+def test_emitted_conv_pool_stack(rt):
+    spec = em.conv_pool_stack(2)
+    g = onnx_lite.load(os.path.join(em.OUT, "ConvPoolStack.onnx"))
+    want = gr.run(g, spec["feeds"], gr.OracleBackend()).ravel()
+    print("emitted ConvPoolStack", flush=True)
+    got = run_emitted("ConvPoolStack", spec["feeds"], want.size)
+    assert want.size == 10 and np.abs(want).max() > 1e-2
+    assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+    txt = open(os.path.join(em.OUT, "ConvPoolStack_GPU_HIP.hxx")).read()
+    # 10x10 -> MaxPool(3, stride 2, pad 1) -> 5x5 -> AveragePool(2, stride 2, ceil) -> 3x3, its divisor following the window
+    assert "d.OH = 5; d.OW = 5;" in txt and "d.OH = 3; d.OW = 3;" in txt and "d.dynamic_divisor = 1" in txt
+
+
 def test_safetensors_session_reproduces_the_golden_output(rt, tmp_path):
     from safetensors.numpy import load_file, save_file
     g, inputs, expected = gr.load_fixture("Linear_16")

@@ -9,7 +9,8 @@ import pytest
 
 from tests import graph_runner as gr
 
-FOUR_DECIMALS = ("Gelu", "GeluTanh", "LinearWithLeakyRelu")  # references printed with 4 decimals
+# references printed with 4 decimals
+FOUR_DECIMALS = ("Gelu", "GeluTanh", "LinearWithLeakyRelu", "AvgPool", "MaxPool1d", "MaxPool2d", "AvgPoolPad", "AvgPoolCountIncludePad")
 
 
 def golden_tolerance(model, expected):

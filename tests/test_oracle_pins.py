@@ -355,3 +355,91 @@ def test_unary_chain_is_applied_left_to_right():
     # not commutative: the reverse order gives something else
     assert not np.allclose(ob.unary_chain(x, ops[::-1]), want, equal_nan=True)
     assert np.array_equal(ob.unary_chain(x, []), x)
+
+
+def _pool_by_definition(X, mode, k, pads, strides, ceil_mode, include_pad):
+    """ONNX MaxPool / AveragePool written from the specification: pad the image (-inf for max; zeros plus a validity
+    mask for the average), slice each window, reduce in float64."""
+    N, Cc, H, W = X.shape
+    (kh, kw), (ph0, pw0, ph1, pw1), (sh, sw) = k, pads, strides
+
+    def extent(n, p0, p1, kk, s):
+        span = n + p0 + p1 - kk
+        out = -(-span // s) + 1 if ceil_mode else span // s + 1
+        if ceil_mode and (out - 1) * s >= n + p0:   # a window may not start in the end padding
+            out -= 1
+        return out
+    OH, OW = extent(H, ph0, ph1, kh, sh), extent(W, pw0, pw1, kw, sw)
+    big_h, big_w = (OH - 1) * sh + kh, (OW - 1) * sw + kw     # the padded canvas every window fits into
+    canvas = np.full((N, Cc, max(big_h, H + ph0), max(big_w, W + pw0)), -np.inf if mode == "max" else 0.0)
+    real = np.zeros(canvas.shape[2:], dtype=bool)     # true input samples
+    padded = np.zeros(canvas.shape[2:], dtype=bool)   # input plus the declared padding
+    canvas[:, :, ph0:ph0 + H, pw0:pw0 + W] = X
+    real[ph0:ph0 + H, pw0:pw0 + W] = True
+    padded[:H + ph0 + ph1, :W + pw0 + pw1] = True
+    Y = np.empty((N, Cc, OH, OW))
+    for oh, ow in itertools.product(range(OH), range(OW)):
+        win = canvas[:, :, oh * sh:oh * sh + kh, ow * sw:ow * sw + kw]
+        if mode == "max":
+            Y[:, :, oh, ow] = win.max(axis=(2, 3))
+        else:
+            count = (padded if include_pad else real)[oh * sh:oh * sh + kh, ow * sw:ow * sw + kw].sum()
+            Y[:, :, oh, ow] = win.sum(axis=(2, 3)) / count
+    return Y
+
+
+@pytest.mark.parametrize("mode", ["max", "average"])
+def test_pool_equals_the_definition_on_a_sweep_of_geometries(mode):
+    rng = np.random.default_rng(11)
+    seen_ceil_overhang = 0
+    for case in range(120):
+        H, W = rng.integers(3, 12, 2)
+        kh, kw = rng.integers(1, 5, 2)
+        sh, sw = rng.integers(1, 4, 2)
+        pads = tuple(int(min(p, kk - 1)) for p, kk in zip(rng.integers(0, 3, 4), (kh, kw, kh, kw)))  # ONNX: pad < kernel
+        ceil_mode, include_pad = int(case % 2), int((case // 2) % 2)
+        X = rng.standard_normal((2, 3, H, W)).astype(np.float32)
+        want = _pool_by_definition(X.astype(np.float64), mode, (kh, kw), pads, (sh, sw), ceil_mode, include_pad)
+        got = ob.pool(X, mode, [kh, kw], list(pads), [sh, sw], None, "NOTSET", ceil_mode, include_pad)
+        assert got.shape == want.shape, (case, H, W, kh, kw, sh, sw, pads, ceil_mode)
+        if mode == "max":
+            np.testing.assert_array_equal(got, want.astype(np.float32))
+        else:
+            np.testing.assert_allclose(got, want, rtol=2e-6, atol=2e-6)
+        seen_ceil_overhang += int(ceil_mode and ((H + pads[0] + pads[2] - kh) % sh or (W + pads[1] + pads[3] - kw) % sw))
+    assert seen_ceil_overhang > 10   # the sweep does reach windows that hang over the end
+
+
+def test_pool_against_the_library_routine():
+    """torch's pooling is an independent implementation of the same definition (floor mode)."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(12)
+    X = rng.standard_normal((2, 4, 9, 11)).astype(np.float32)
+    t = torch.from_numpy(X)
+    np.testing.assert_array_equal(ob.pool(X, "max", [3, 2], [1, 0, 1, 0], [2, 1]), F.max_pool2d(t, (3, 2), (2, 1), (1, 0)).numpy())
+    for include in (0, 1):
+        want = F.avg_pool2d(t, (3, 3), (2, 2), (1, 1), count_include_pad=bool(include)).numpy()
+        np.testing.assert_allclose(ob.pool(X, "average", [3, 3], [1, 1, 1, 1], [2, 2], count_include_pad=include), want, rtol=2e-6, atol=2e-6)
+    X1 = rng.standard_normal((3, 2, 17)).astype(np.float32)
+    np.testing.assert_array_equal(ob.pool(X1, "max", [3], None, [2]), F.max_pool1d(torch.from_numpy(X1), 3, 2).numpy())
+
+
+def test_pool_special_cases():
+    X = np.arange(2 * 3 * 4 * 5, dtype=np.float32).reshape(2, 3, 4, 5)
+    # a window that is the image is GlobalAveragePool; a 1x1 window with stride 1 is the identity
+    np.testing.assert_array_equal(ob.pool(X, "average", [4, 5]), ob.global_avg_pool(X))
+    np.testing.assert_array_equal(ob.pool(X, "max", [1, 1]), X)
+    np.testing.assert_array_equal(ob.pool(X, "average", [1, 1]), X)
+    # NaN never wins `x > value`; a window of NaNs only stays at -inf (the reference's comparison, not IEEE maximum)
+    Xn = np.array([[[np.nan, 1.0, np.nan, np.nan]]], dtype=np.float32)
+    np.testing.assert_array_equal(ob.pool(Xn, "max", [2], None, [2]), np.array([[[1.0, -np.inf]]], dtype=np.float32))
+    # SAME_UPPER puts the odd padding sample at the end, SAME_LOWER at the beginning
+    assert ob.pool_axes([5], [2], None, [1], None, "SAME_UPPER")[0][4:] == (0, 1)
+    assert ob.pool_axes([5], [2], None, [1], None, "SAME_LOWER")[0][4:] == (1, 0)
+    # the reference pools over the whole dilated extent: kernel 2 with dilation 2 is a dense window of 3
+    np.testing.assert_array_equal(ob.pool(X, "max", [2, 2], None, [1, 1], [2, 2]), ob.pool(X, "max", [3, 3]))
+    # ceil_mode with the window hanging over the end (the reference's MaxPool1d_CeilMode_Overhang shape: 6 -> 2)
+    X6 = np.array([[[1, 2, 3, 4, 5, 6]]], dtype=np.float32)
+    np.testing.assert_array_equal(ob.pool(X6, "max", [2], None, [3], ceil_mode=1), np.array([[[2, 5]]], dtype=np.float32))
+    np.testing.assert_array_equal(ob.pool(X6, "average", [2], None, [3], ceil_mode=1), np.array([[[1.5, 4.5]]], dtype=np.float32))
