@@ -37,24 +37,29 @@ def _run(cmd, cwd=None):
         raise RuntimeError("command failed (%d): %s" % (r.returncode, " ".join(cmd)))
 
 
-def build_hip_library(jobs=8):
-    """Compiles every HIP source for gfx950 and links sofie_amd/lib/libsofie_hip.so."""
+def build_hip_library(jobs=8, tuning=False):
+    """Compiles every HIP source for gfx950 and links sofie_amd/lib/libsofie_hip.so.  tuning=True builds, beside it, the
+    library with the ablation and alternative-tile kernels (-DSOFIE_HIP_TUNING) that SOFIE_HIP_GEMM_VARIANT and
+    SOFIE_HIP_I8_TILE select, as sofie_amd/lib/tuning/libsofie_hip.so; nothing loads that one by default."""
     from concurrent.futures import ThreadPoolExecutor
-    os.makedirs(LIB_DIR, exist_ok=True)
-    obj_dir = os.path.join(ROOT, "build", "obj")
+    lib_dir = os.path.join(LIB_DIR, "tuning") if tuning else LIB_DIR
+    lib = os.path.join(lib_dir, "libsofie_hip.so")
+    os.makedirs(lib_dir, exist_ok=True)
+    obj_dir = os.path.join(ROOT, "build", "obj_tuning" if tuning else "obj")
     os.makedirs(obj_dir, exist_ok=True)
+    flags = HIPCC_FLAGS + (["-DSOFIE_HIP_TUNING"] if tuning else [])
     hipcc = _hipcc()
     sources = [s for s in HIP_SOURCES if os.path.exists(os.path.join(CSRC, s))]
     objs = [os.path.join(obj_dir, s.replace(".hip", ".o")) for s in sources]
 
     def compile_one(pair):
         src, obj = pair
-        _run([hipcc] + HIPCC_FLAGS + ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-c", os.path.join(CSRC, src), "-o", obj])
+        _run([hipcc] + flags + ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-c", os.path.join(CSRC, src), "-o", obj])
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(compile_one, zip(sources, objs)))
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
-    return LIB
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs)
+    return lib
 
 
 def build_oracle():
@@ -70,5 +75,8 @@ def build_all():
 
 
 if __name__ == "__main__":
-    build_all()
+    if "--tuning" in sys.argv[1:]:
+        build_hip_library(tuning=True)
+    else:
+        build_all()
     sys.exit(0)

@@ -96,11 +96,21 @@ static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *
             return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI, 1>(stream, A, Bt, M, N, K, lda, ldb, ep);
          if (variant == 56)
             return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 4, EPI, 4>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 57)
+            return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI, 7>(stream, A, Bt, M, N, K, lda, ldb, ep);
 #endif
          if (variant == 1 || !k128)
             return launch_mfma8_dma<MMA, 128, 128, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
          return launch_mfma8_dma<MMA, 128, 128, 128, 2, 2, 3, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
       case 64:
+#ifdef SOFIE_HIP_TUNING
+         if (variant == 54)
+            return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI, 4>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 55)
+            return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI, 1>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 57)
+            return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI, 7>(stream, A, Bt, M, N, K, lda, ldb, ep);
+#endif
          if (variant == 1 || !k128)
             return launch_mfma8_dma<MMA, 64, 64, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
          return launch_mfma8_dma<MMA, 64, 64, 128, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
