@@ -173,7 +173,8 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d);
  * The MFMA kernel wants both operands K-contiguous; a B given as [K,N] is transposed into
  * `workspace` (K*N bytes, 256-B aligned) on every call.  A constant B (a weight) is better re-laid
  * out once at Session construction with sofie_hip_transpose_i8 and then passed with transB = 1. */
-enum { SOFIE_I8OUT_I32 = 0, SOFIE_I8OUT_F32 = 1, SOFIE_I8OUT_I8 = 2, SOFIE_I8OUT_I8_DQQ = 3 };
+enum { SOFIE_I8OUT_I32 = 0, SOFIE_I8OUT_F32 = 1, SOFIE_I8OUT_I8 = 2, SOFIE_I8OUT_I8_DQQ = 3,
+       SOFIE_I8OUT_I8_PLANE_SUMS = 4 /* sofie_hip_conv_i8 only, see there */ };
 typedef struct sofie_gemm_i8_desc {
    int32_t M, N, K;
    int32_t transA, transB;
@@ -272,6 +273,12 @@ int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float
  *   SOFIE_I8OUT_I8   Y_i8  = sat8(rne(float(acc)*scale[co])), then max(.,0) if relu
  *   SOFIE_I8OUT_F32  Y_f32 = float(acc)*scale[co], then max(.,0) if relu
  *   SOFIE_I8OUT_I32  Y_i32 = relu ? max(acc,0) : acc
+ *   SOFIE_I8OUT_I8_PLANE_SUMS  the int8 feature map of SOFIE_I8OUT_I8 is not stored; Y is int32 [N, Cout] and receives
+ *                    Y[n,co] += sum over the OH*OW output pixels of that int8 value (integer additions from the kernel's store,
+ *                    exact in any order).  The caller clears Y first (sofie_hip_fill_zero).  For a GlobalAveragePool that is
+ *                    the only reader of a convolution: the largest activation of the network is neither written nor read
+ *                    back.  Needs OH*OW to be a multiple of 256 and a shape that takes no column matrix (workspace 0), else
+ *                    the call is refused; y_layout is ignored.
  * Activations are NCHW (the ONNX layout) or NHWC (channels fastest), chosen per tensor: a chain of
  * convolutions keeps NHWC between its layers.  W is the ONNX weight [Cout, C/group, kh, kw], or, with
  * w_is_packed, the re-laid-out form sofie_hip_pack_conv_weight_i8 writes once at Session construction
@@ -327,6 +334,11 @@ int sofie_hip_pool_f32(sofie_hip_ctx *ctx, const sofie_pool_desc *d, float *Y, c
 /* int8 input, fp32 output: Y = (float(sum_i32) * scale) / float(HW), exact sum -- not in the reference. */
 int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y /* [N,C] */, const int8_t *X, int32_t N, int32_t C, int32_t HW,
                                  int32_t x_layout /* SOFIE_LAYOUT_* */, float scale);
+/* The same average when a convolution has already added the planes up (sofie_hip_conv_i8 with
+ * SOFIE_I8OUT_I8_PLANE_SUMS): Y[i] = (float(sums[i]) * scale) / float(HW) -- the bits sofie_hip_global_avg_pool_i8 gives
+ * on the feature map that was never stored. */
+int sofie_hip_plane_sums_to_average(sofie_hip_ctx *ctx, float *Y /* [NC] */, const int32_t *sums /* [NC] */, int32_t NC, int32_t HW,
+                                    float scale);
 
 /* BatchNormalization at inference, for models whose normalisation was not folded into the weights
  * (core/inc/SOFIE/operators/ROperator_BatchNormalization.hxx:139-158): X is [N, C, spatial...],

@@ -188,8 +188,15 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
    int st = check_conv(d, g, "sofie_hip_conv_i8");
    if (st)
       return st;
-   SOFIE_HIP_REQUIRE(a->out == SOFIE_I8OUT_I32 || a->out == SOFIE_I8OUT_F32 || a->out == SOFIE_I8OUT_I8,
+   SOFIE_HIP_REQUIRE(a->out == SOFIE_I8OUT_I32 || a->out == SOFIE_I8OUT_F32 || a->out == SOFIE_I8OUT_I8 || a->out == SOFIE_I8OUT_I8_PLANE_SUMS,
                      "sofie_hip_conv_i8: unknown output kind %d", a->out);
+   // Plane sums ride in the tile store of the matrix-core kernels: a wave's tile (at most 128 rows of a 256-row tile) must lie in one
+   // image and hold valid rows only.
+   const bool plane_sums = a->out == SOFIE_I8OUT_I8_PLANE_SUMS;
+   const int out_kind = plane_sums ? SOFIE_I8OUT_I8 : a->out;
+   SOFIE_HIP_REQUIRE(!plane_sums || ((g.OH * g.OW) % 256 == 0 && (conv_i8_implicit_shape(d, a->x_layout) || conv_i8_gather_shape(d))),
+                     "sofie_hip_conv_i8: plane sums need output planes of a multiple of 256 pixels (got %d) and a shape the kernel reads "
+                     "without a column matrix", g.OH * g.OW);
    SOFIE_HIP_REQUIRE((a->x_layout == SOFIE_LAYOUT_NCHW || a->x_layout == SOFIE_LAYOUT_NHWC) &&
                         (a->y_layout == SOFIE_LAYOUT_NCHW || a->y_layout == SOFIE_LAYOUT_NHWC),
                      "sofie_hip_conv_i8: unknown layout");
@@ -216,7 +223,7 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
    }
    const int OHW = g.OH * g.OW;
    const int Cout_g = d->Cout / d->group;
-   const size_t esz = a->out == SOFIE_I8OUT_I8 ? 1 : 4;
+   const size_t esz = out_kind == SOFIE_I8OUT_I8 ? 1 : 4;
 
    // Implicit GEMM: the kernel reads the NHWC activations directly, one launch per group over the whole batch.
    // Needs K slabs that lie inside one input pixel (channels per group a power of two >= 64) and 32-bit offsets.
@@ -246,13 +253,14 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
             ep.scale = a->scale;
             ep.scale_scalar = 1.0f;
             ep.q_scale = 1.0f;
-            ep.relu_acc = (a->out == SOFIE_I8OUT_I32) ? a->relu : 0;
-            ep.relu_out = (a->out == SOFIE_I8OUT_I32) ? 0 : a->relu;
-            ep.out = a->out;
+            ep.relu_acc = (out_kind == SOFIE_I8OUT_I32) ? a->relu : 0;
+            ep.relu_out = (out_kind == SOFIE_I8OUT_I32) ? 0 : a->relu;
+            ep.out = out_kind;
             ep.ldy = d->Cout;
             ep.N = Cout_g;
             ep.n_offset = grp * Cout_g;
-            ep.nchw_ohw = (a->y_layout == SOFIE_LAYOUT_NHWC) ? 0 : OHW;
+            ep.nchw_ohw = (a->y_layout == SOFIE_LAYOUT_NHWC || plane_sums) ? 0 : OHW;
+            ep.rows_per_plane = plane_sums ? OHW : 0;
             ep.Y = a->Y;
             st = conv_i8_implicit(ctx->stream, src, g.Cg, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.K, ep, forced_i8_tile());
             if (st)
@@ -289,13 +297,14 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
          ep.scale = a->scale;
          ep.scale_scalar = 1.0f;
          ep.q_scale = 1.0f;
-         ep.relu_acc = (a->out == SOFIE_I8OUT_I32) ? a->relu : 0;
-         ep.relu_out = (a->out == SOFIE_I8OUT_I32) ? 0 : a->relu;
-         ep.out = a->out;
+         ep.relu_acc = (out_kind == SOFIE_I8OUT_I32) ? a->relu : 0;
+         ep.relu_out = (out_kind == SOFIE_I8OUT_I32) ? 0 : a->relu;
+         ep.out = out_kind;
          ep.ldy = d->Cout;
          ep.N = Cout_g;
          ep.n_offset = grp * Cout_g;
-         ep.nchw_ohw = (a->y_layout == SOFIE_LAYOUT_NHWC) ? 0 : OHW;
+         ep.nchw_ohw = (a->y_layout == SOFIE_LAYOUT_NHWC || plane_sums) ? 0 : OHW;
+         ep.rows_per_plane = plane_sums ? OHW : 0;
          ep.Y = a->Y;
          st = conv_i8_gather(ctx->stream, src, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.Kp, ep);
          if (st)
@@ -303,6 +312,7 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
       }
       return SOFIE_HIP_OK;
    }
+   SOFIE_HIP_REQUIRE(!plane_sums, "sofie_hip_conv_i8: plane sums need 16-byte aligned activations and weights");
    const size_t per_image = (size_t)OHW * g.Kp;
    SOFIE_HIP_REQUIRE(ws != nullptr && ws_left >= per_image,
                      "sofie_hip_conv_i8: the activations are not 16-byte aligned; a workspace of %zu bytes is needed for the column matrix",
@@ -340,9 +350,9 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
          ep.scale = a->scale;
          ep.scale_scalar = 1.0f;
          ep.q_scale = 1.0f;
-         ep.relu_acc = (a->out == SOFIE_I8OUT_I32) ? a->relu : 0;
-         ep.relu_out = (a->out == SOFIE_I8OUT_I32) ? 0 : a->relu;
-         ep.out = a->out;
+         ep.relu_acc = (out_kind == SOFIE_I8OUT_I32) ? a->relu : 0;
+         ep.relu_out = (out_kind == SOFIE_I8OUT_I32) ? 0 : a->relu;
+         ep.out = out_kind;
          ep.ldy = d->Cout;
          ep.stage_ok = 0;
          ep.vec_param = 0;

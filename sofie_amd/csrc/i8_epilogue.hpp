@@ -20,6 +20,8 @@ struct I8Epilogue {
    int N;         // number of valid columns
    int nchw_ohw;  // 0: Y[m*ldy + n]; else m = (img, pix) and Y[(img*ldy + n)*nchw_ohw + pix], ldy = Cout
    int n_offset;  // added to n for bias/scale/Y addressing (grouped convolution)
+   int rows_per_plane = 0; // non-zero (with out = SOFIE_I8OUT_I8): the int8 values of the rows of a plane are added up instead of stored;
+                       // Y is int32 [M / rows_per_plane][ldy]
 
    template <class F>
    __device__ __forceinline__ void dispatch(F f) const
@@ -35,6 +37,18 @@ struct I8Epilogue {
    static constexpr int out_bytes()
    {
       return (OUT == SOFIE_I8OUT_I32 || OUT == SOFIE_I8OUT_F32) ? 4 : 1;
+   }
+   static constexpr bool kCanSumRows = true;
+   __device__ __forceinline__ bool sums_rows() const { return rows_per_plane != 0; }
+   // sums of columns n..n+3 over a wave tile's rows, which start at row m and lie in one plane: integer additions, so the
+   // order in which the tiles arrive does not matter
+   __device__ __forceinline__ void add_row_sums(int m, int n, int N_, const int (&s)[4]) const
+   {
+      int *dst = (int *)Y + (size_t)(m / rows_per_plane) * (size_t)ldy + n + n_offset;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+         if (n + e < N_)
+            atomicAdd(dst + e, s[e]);
    }
    __device__ __forceinline__ bool rows_vectorizable() const { return stage_ok != 0; }
    __device__ __forceinline__ char *out_base() const { return (char *)Y; }

@@ -237,6 +237,12 @@ struct ConvRows {
    }
 };
 
+// Can epilogue EPI add the rows of a tile up instead of storing them?  (EPI::kCanSumRows, if the epilogue has it.)
+template <class EPI, class = void>
+struct epi_can_sum_rows : std::false_type {};
+template <class EPI>
+struct epi_can_sum_rows<EPI, std::enable_if_t<EPI::kCanSumRows>> : std::true_type {};
+
 // LDS bytes one wave needs for the tile store below (TN = columns of the wave tile).
 constexpr int tile_store_lds_bytes(int TN) { return 32 * (TN * 4 + 16); }
 
@@ -272,6 +278,19 @@ __device__ __forceinline__ void tile_store_convert_first(const EPI &ep, ACC (&ac
    char *out = ep.out_base();
    const bool vec = ep.rows_vectorizable();
 
+   // Row sums (an epilogue that can, asked at run time, 1-byte elements): instead of storing the converted elements, the wave
+   // adds them up column by column over all MT * 32 rows of its tile (the caller guarantees that those rows are valid and
+   // belong to one plane) and hands the epilogue 4 column sums per lane.  A lane takes dword `sum_dw` of every RG-th row of
+   // the parked block.
+   constexpr int DPR = TN / 4;                         // dwords per parked row
+   constexpr int RG = (64 / DPR) > 0 ? (64 / DPR) : 1; // rows read per pass
+   constexpr bool CAN_SUM = epi_can_sum_rows<EPI>::value && ESZ == 1 && DPR <= 64 && 64 % DPR == 0 && 32 % RG == 0;
+   bool sums = false;
+   if constexpr (CAN_SUM)
+      sums = ep.sums_rows();
+   const int sum_dw = lane % DPR, sum_rg = lane / DPR;
+   int colsum[4] = {0, 0, 0, 0};
+
    // the lane's columns are the same in every 32-row block: their constants are fetched once
    typename EPI::template col_params<4> prm[NT][4];
    static_for<NT>([&](auto cj) {
@@ -303,7 +322,16 @@ __device__ __forceinline__ void tile_store_convert_first(const EPI &ep, ACC (&ac
       });
       __builtin_amdgcn_wave_barrier();
       const int m_first = m_base + i * 32;
-      if (vec) {
+      if (CAN_SUM && sums) {
+#pragma unroll 4
+         for (int row = sum_rg; row < 32; row += RG) {
+            const int v = *(const int *)(wsm + row * ROWB + sum_dw * 4);
+            colsum[0] += (v << 24) >> 24;
+            colsum[1] += (v << 16) >> 24;
+            colsum[2] += (v << 8) >> 24;
+            colsum[3] += v >> 24;
+         }
+      } else if (vec) {
          constexpr int CPL = 16 / ESZ;          // columns per lane
          constexpr int LPR = TN / CPL;          // lanes per row
          constexpr int RPP = 64 / LPR;          // rows per pass
@@ -353,6 +381,18 @@ __device__ __forceinline__ void tile_store_convert_first(const EPI &ep, ACC (&ac
       }
       __builtin_amdgcn_wave_barrier();
    });
+   if constexpr (CAN_SUM) {
+      if (sums) {
+         // lanes that share a dword column hold the sums of different rows: fold them onto the lanes of row group 0
+#pragma unroll
+         for (int d = DPR; d < 64; d *= 2)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+               colsum[e] += __shfl_xor(colsum[e], d, 64);
+         if (sum_rg == 0)
+            ep.add_row_sums(m_base, n_base + sum_dw * 4, N, colsum);
+      }
+   }
 }
 
 // The other order, for stores whose conversion is long (an erf per element): the raw 32-bit accumulators are parked and

@@ -106,6 +106,7 @@ private:
    void Initialize(int batchSize);
    void FuseGemmActivations();
    void TryFuseResidual(std::size_t i);
+   void TryFusePlaneSums(std::size_t i);
    void PlanMemory();
    void GenerateSessionCode(std::underlying_type_t<Options> options);
    void WriteWeightFile(const std::string &filename) const;

@@ -7,6 +7,9 @@
 //                A Relu that follows is folded into the store.  Between two quantised convolutions the
 //                activation is kept NHWC (channels fastest), which is what the matrix-core kernel reads in place.
 //   DequantizeLinear + GlobalAveragePool on an int8 map  ->  one kernel: exact int32 sum, then * scale / HW.
+//                When that map comes from a QLinearConv which nothing else reads, and the runtime can do it (planes of a
+//                multiple of 256 pixels, no column matrix), the convolution adds the planes up in its own store: the map
+//                is neither written nor read back, and a small kernel turns the sums into the average.
 //   Flatten      a device copy (the tensors here are a few KB).
 #ifndef SOFIE_HIP_ROPERATOR_QCONV
 #define SOFIE_HIP_ROPERATOR_QCONV
@@ -55,6 +58,31 @@ public:
       fOutputTensorNames = {fNY};
    }
    const std::string &OutputName() const { return fNY; }
+
+   // Whether the runtime would add the output planes up in the kernel's store (sofie_hip_conv_i8 with
+   // SOFIE_I8OUT_I8_PLANE_SUMS): callable before Initialize, once the input's shape and layout are known.
+   bool CanSumPlanes(RModel &model)
+   {
+      if (fInt32Out || !model.CheckIfTensorAlreadyExist(fNX) || !model.CheckIfTensorAlreadyExist(fNW))
+         return false;
+      try {
+         fGeo.Resolve(fAttrAutopad, fAttrDilations, fAttrGroup, fAttrKernelShape, fAttrPads, fAttrStrides, model.GetTensorShape(fNX),
+                      model.GetTensorShape(fNW));
+      } catch (const std::exception &) {
+         return false; // Initialize reports the problem
+      }
+      fXLayout = model.GetTensorLayout(fNX);
+      return (fGeo.OH * fGeo.OW) % 256 == 0 && (ImplicitGemm() || GatheredGemm());
+   }
+   // The GlobalAveragePool(DequantizeLinear(Y, scale)) that was the only reader of Y becomes this operator's output.
+   void SumPlanes(float dequantScale, const std::string &pooledOutput)
+   {
+      fSumPlanes = true;
+      fPoolScale = dequantScale;
+      fNPooled = pooledOutput;
+      fOutputTensorNames = {fNPooled};
+   }
+   bool SumsPlanes() const { return fSumPlanes; }
 
    void Initialize(RModel &model) override
    {
@@ -105,6 +133,12 @@ public:
              ConvertShapeToLength(model.GetTensorShape(fNB)) != fGeo.Cout)
             throw std::runtime_error("SOFIE QLinearConv Op: bias " + fNB + " must be an int32 initializer of " + std::to_string(fGeo.Cout) + " elements");
       }
+      if (fSumPlanes) {
+         if (!((fGeo.OH * fGeo.OW) % 256 == 0 && (ImplicitGemm() || GatheredGemm())))
+            throw std::runtime_error("SOFIE QLinearConv Op: " + fNY + " cannot be summed plane by plane in the convolution");
+         model.AddIntermediateTensor(fNPooled, ETensorType::FLOAT, {fGeo.N, fGeo.Cout, 1, 1}, fDynamic);
+         return;
+      }
       // channels-last output when every reader understands it
       fYLayout = kLayoutNHWC;
       if (model.IsOutputTensor(fNY))
@@ -147,6 +181,8 @@ public:
    }
    std::size_t GetWorkspaceBytes() override
    {
+      if (fSumPlanes) // the int32 plane sums [N][Cout]; with a run-time batch N is 1 here and the bytes are per batch entry
+         return (fGeo.N * fGeo.Cout * 4 + 255) / 256 * 256;
       if (ImplicitGemm() || GatheredGemm())
          return 0;
       const std::size_t per_image = (fGeo.OH * fGeo.OW * PackedK() + 255) / 256 * 256;
@@ -160,15 +196,27 @@ public:
       opName = "op_" + opName;
       std::stringstream out;
       out << "\n" << SP << "//----  operator " << (fInt32Out ? "ConvInteger " : "QLinearConv ") << opName << " --> " << ConvertShapeToString(fGeo.OutputShape())
-          << (fYLayout == kLayoutNHWC ? " (stored NHWC)" : "") << (ImplicitGemm() ? ", implicit GEMM" : GatheredGemm() ? ", rows gathered in the kernel" : ", column matrix") << "\n";
+          << (fSumPlanes ? " (not stored: planes summed for the GlobalAveragePool)" : fYLayout == kLayoutNHWC ? " (stored NHWC)" : "")
+          << (ImplicitGemm() ? ", implicit GEMM" : GatheredGemm() ? ", rows gathered in the kernel" : ", column matrix") << "\n";
       out << SP << "{\n";
       out << SP << "   " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n" << fGeo.BatchLine(fDynamic, SP + "   ");
       out << SP << "   " << "sofie_conv_i8_args a{};\n";
       out << SP << "   " << "a.X = tensor_" << fNX << "; a.W = packed_" << fNW << "; a.w_is_packed = 1; a.bias = "
           << (fNB.empty() ? "nullptr" : "tensor_" + fNB) << "; a.scale = " << (fInt32Out ? std::string("nullptr") : "tensor_" + fNM) << ";\n";
-      out << SP << "   " << "a.relu = " << (fRelu ? 1 : 0) << "; a.out = " << (fInt32Out ? "SOFIE_I8OUT_I32" : "SOFIE_I8OUT_I8") << "; a.x_layout = "
-          << (fXLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.y_layout = "
-          << (fYLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.Y = tensor_" << fNY << ";\n";
+      out << SP << "   " << "a.relu = " << (fRelu ? 1 : 0) << "; a.out = " << (fSumPlanes ? "SOFIE_I8OUT_I8_PLANE_SUMS" : fInt32Out ? "SOFIE_I8OUT_I32" : "SOFIE_I8OUT_I8")
+          << "; a.x_layout = " << (fXLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.y_layout = "
+          << (fYLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.Y = " << (fSumPlanes ? ws : "tensor_" + fNY) << ";\n";
+      if (fSumPlanes) {
+         // rows of Cout int32 sums, one per image; cleared, filled by the convolution's store, then averaged
+         const std::string count = BatchScaledInt(fDynamic, fGeo.N * fGeo.Cout);
+         out << SP << "   " << "detail::Check(sofie_hip_fill_zero(fCtx, " << ws << ", static_cast<std::size_t>(" << count << ") * 4), \"" << opName
+             << " clear plane sums\");\n";
+         out << SP << "   " << "detail::Check(sofie_hip_conv_i8(fCtx, &d, &a), \"" << opName << " QLinearConv\");\n";
+         out << SP << "   " << "detail::Check(sofie_hip_plane_sums_to_average(fCtx, tensor_" << fNPooled << ", static_cast<const int32_t *>(static_cast<const void *>(" << ws
+             << ")), " << count << ", " << fGeo.OH * fGeo.OW << ", " << FloatLiteral(fPoolScale) << "), \"" << opName << " GlobalAveragePool\");\n";
+         out << SP << "}\n";
+         return out.str();
+      }
       if (GetWorkspaceBytes())
          out << SP << "   " << "a.workspace = " << ws << "; a.workspace_bytes = " << BatchScaled(fDynamic, GetWorkspaceBytes()) << ";\n";
       out << SP << "   " << "detail::Check(sofie_hip_conv_i8(fCtx, &d, &a), \"" << opName << " QLinearConv\");\n";
@@ -182,7 +230,9 @@ private:
    std::size_t fAttrGroup;
    std::vector<std::size_t> fAttrKernelShape, fAttrPads, fAttrStrides;
    std::string fNX, fNXS, fNXZ, fNW, fNWS, fNWZ, fNYS, fNYZ, fNB, fNY, fNM;
-   bool fRelu = false, fInt32Out = false, fDynamic = false;
+   bool fRelu = false, fInt32Out = false, fDynamic = false, fSumPlanes = false;
+   float fPoolScale = 1.0f;
+   std::string fNPooled;
    int fXLayout = kLayoutNCHW, fYLayout = kLayoutNCHW;
    ConvGeometry fGeo;
 };
@@ -197,6 +247,8 @@ public:
       fOutputTensorNames = {fNY};
       fKind = OperatorKind::QPOOL;
    }
+   const std::string &ScaleName() const { return fNS; }
+   const std::string &OutputName() const { return fNY; }
    void Initialize(RModel &model) override
    {
       if (!model.CheckIfTensorAlreadyExist(fNX))

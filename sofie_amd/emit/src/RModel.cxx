@@ -333,6 +333,33 @@ void RModel::TryFuseResidual(std::size_t i)
    FuseGemmActivations(); // what followed the Add may now join the same store
 }
 
+// A quantised convolution whose only reader is the fused DequantizeLinear + GlobalAveragePool, and whose shape the runtime can
+// sum plane by plane in the kernel's store: the pooling joins the convolution and the feature map is never stored.  Runs just
+// before operator i is initialised, like TryFuseResidual.
+void RModel::TryFusePlaneSums(std::size_t i)
+{
+   auto *qc = dynamic_cast<ROperator_QConv *>(fOperators[i].get());
+   if (!qc || qc->SumsPlanes())
+      return;
+   const std::string y = qc->OutputName();
+   if (IsOutputTensor(y))
+      return;
+   std::size_t reader = fOperators.size(), readers = 0;
+   for (std::size_t j = 0; j < fOperators.size(); ++j)
+      for (auto &in : fOperators[j]->GetInputTensorNames())
+         if (in == y) {
+            reader = j;
+            ++readers;
+         }
+   if (readers != 1 || reader <= i)
+      return;
+   auto *pool = dynamic_cast<ROperator_QGlobalAveragePool *>(fOperators[reader].get());
+   if (!pool || !qc->CanSumPlanes(*this))
+      return;
+   qc->SumPlanes(GetScalarInitializer(pool->ScaleName()), pool->OutputName());
+   fOperators.erase(fOperators.begin() + reader);
+}
+
 bool RModel::IsOutputTensor(const std::string &name) const
 {
    return std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), UTILITY::Clean_name(name)) != fOutputTensorNames.end();
@@ -376,6 +403,7 @@ void RModel::Initialize(int batchSize)
    FuseGemmActivations();
    for (std::size_t i = 0; i < fOperators.size(); ++i) {
       TryFuseResidual(i);
+      TryFusePlaneSums(i);
       fOperators[i]->SetOpOrder(i);
       fOperators[i]->Initialize(*this);
       // an operator that reads a batched tensor has to say what it makes of the batch

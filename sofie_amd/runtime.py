@@ -21,7 +21,7 @@ class SofieHipError(RuntimeError):
  ACT_SIN, ACT_COS, ACT_ABS, ACT_SOFTPLUS, ACT_ATAN, ACT_FLOOR, ACT_ASINH, ACT_ACOSH, ACT_ATANH, ACT_CLIP, ACT_SELU) = range(23)
 MAX_POST_OPS = 4
 BIAS_NONE, BIAS_ROW, BIAS_COL, BIAS_SCALAR, BIAS_FULL = range(5)
-I8OUT_I32, I8OUT_F32, I8OUT_I8, I8OUT_I8_DQQ = range(4)
+I8OUT_I32, I8OUT_F32, I8OUT_I8, I8OUT_I8_DQQ, I8OUT_I8_PLANE_SUMS = range(5)
 F8OUT_BF16, F8OUT_F32 = range(2)
 LAYOUT_NCHW, LAYOUT_NHWC = range(2)
 
@@ -125,6 +125,7 @@ SYMBOLS = {
     "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),
     "sofie_hip_global_avg_pool_f32": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32]),
     "sofie_hip_pool_f32": (C.c_int, [_P, _P, _P, _P]),
+    "sofie_hip_plane_sums_to_average": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_float]),
     "sofie_hip_batchnorm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "sofie_hip_global_avg_pool_i8": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float]),
     "sofie_hip_conv_weight_i8_packed_bytes": (C.c_size_t, [C.POINTER(ConvDesc)]),

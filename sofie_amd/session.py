@@ -128,7 +128,9 @@ class Int8CNNSession:
     (= s_in * s_w[co] / s_out), pads (h0,w0,h1,w1), strides, dils.  fc_w is fp32 [C_last, n_out], fc_b [n_out].
     """
 
-    def __init__(self, rt, batch, in_shape, in_scale, convs, last_scale, fc_w, fc_b):
+    def __init__(self, rt, batch, in_shape, in_scale, convs, last_scale, fc_w, fc_b, pool_in_conv=True):
+        """pool_in_conv: let the last convolution add its planes up in its store (the feature map the average reads is then
+        neither written nor read back) whenever the runtime takes that shape; False keeps the two kernels apart."""
         self.rt = rt
         self.batch = N = int(batch)
         Cin, H, W = in_shape
@@ -175,6 +177,7 @@ class Int8CNNSession:
         stage = max(cv["W"].size for cv in convs)
         self.off_stage = take(stage)
         self.off_pool = take(4 * N * self.out_shape[0])
+        self.off_sums = take(4 * N * self.out_shape[0])
         self.off_fcw = take(4 * fc_w.size)
         self.off_fcb = take(4 * fc_b.size)
         self.off_y = take(4 * N * self.n_out)
@@ -211,6 +214,12 @@ class Int8CNNSession:
             self.conv_args.append(a)
             src, src_layout = dst, R.LAYOUT_NHWC
         self.off_last = src
+        # the last convolution may hand the average its plane sums instead of the feature map
+        last_d, last_a = self.conv_descs[-1], self.conv_args[-1]
+        self.pool_in_conv = bool(pool_in_conv) and (last_d.OH * last_d.OW) % 256 == 0 and \
+            lib.sofie_hip_conv_i8_workspace(C.byref(last_d), C.byref(last_a)) == 0
+        if self.pool_in_conv:
+            last_a.out, last_a.Y = R.I8OUT_I8_PLANE_SUMS, p(self.off_sums)
         upload(self.off_fcw, fc_w.astype(np.float32))
         upload(self.off_fcb, fc_b.astype(np.float32))
         g = R.GemmF32Desc()
@@ -238,11 +247,17 @@ class Int8CNNSession:
         Cin, H, W = self.in_shape
         rt.call("sofie_hip_quantize_linear", self.p(self.off_xq), self.x_ptr, C.c_size_t(self.batch * Cin * H * W),
                 C.c_float(float(self.in_scale)))
+        c, h, w = self.out_shape
+        if self.pool_in_conv:
+            rt.call("sofie_hip_fill_zero", self.p(self.off_sums), C.c_size_t(4 * self.batch * c))
         for d, a in zip(self.conv_descs, self.conv_args):
             rt.call("sofie_hip_conv_i8", C.byref(d), C.byref(a))
-        c, h, w = self.out_shape
-        rt.call("sofie_hip_global_avg_pool_i8", self.p(self.off_pool), self.p(self.off_last), self.batch, c, h * w, R.LAYOUT_NHWC,
-                C.c_float(float(self.last_scale)))
+        if self.pool_in_conv:
+            rt.call("sofie_hip_plane_sums_to_average", self.p(self.off_pool), self.p(self.off_sums), self.batch * c, h * w,
+                    C.c_float(float(self.last_scale)))
+        else:
+            rt.call("sofie_hip_global_avg_pool_i8", self.p(self.off_pool), self.p(self.off_last), self.batch, c, h * w, R.LAYOUT_NHWC,
+                    C.c_float(float(self.last_scale)))
         rt.call("sofie_hip_gemm_f32", C.byref(self.fc))
 
     def infer(self, x):

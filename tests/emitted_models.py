@@ -319,6 +319,7 @@ DYNAMIC_MODELS = {    "Dynamic_ResidualBlock": lambda: with_named_batch(residual
     "Dynamic_int8_CNN": lambda: with_named_batch(int8_cnn(2, 12), "N"),
     "Dynamic_ConvBatchNormRelu": lambda: with_named_batch(conv_batchnorm_relu(2), "bs"),
     "Dynamic_ConvPoolStack": lambda: with_named_batch(conv_pool_stack(2), "N"),
+    "Dynamic_int8_CNN_plane_sums": lambda: with_named_batch(int8_cnn(2, 16, (3, 64, 128)), "N"),
 }
 
 CONFIG_MODELS = {
@@ -328,6 +329,7 @@ CONFIG_MODELS = {
     "ConvBatchNormRelu": lambda: conv_batchnorm_relu(2),
     "ConvPoolStack": lambda: conv_pool_stack(2),
     "Config5_int8_CNN_small": lambda: int8_cnn(2, 12),
+    "Int8_CNN_plane_sums": lambda: int8_cnn(2, 16, (3, 64, 128)),   # planes of 256 pixels: the last convolution sums them itself
     "Config1_fp32_MLP": lambda: fp32_mlp(64),
     "Config2_int8_MLP_small": lambda: int8_mlp([64, 128, 96, 32], 48),
     "Config2_int8_MLP_mid": lambda: int8_mlp([256, 512, 512, 256], 256),

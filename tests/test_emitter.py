@@ -179,6 +179,23 @@ def test_quantised_cnn_keeps_channels_last_and_reads_activations_in_place(emitte
     assert ctor.count("sofie_hip_pack_conv_weight_i8(") == 4
 
 
+def test_global_average_pool_joins_a_convolution_whose_planes_the_runtime_can_sum(emitted):
+    txt = read(emitted, "Int8_CNN_plane_sums")
+    body = ops_body(txt)
+    assert body.count("sofie_hip_conv_i8(") == 2 and body.count("a.out = SOFIE_I8OUT_I8_PLANE_SUMS") == 1
+    assert "sofie_hip_global_avg_pool_i8(" not in body and body.count("sofie_hip_plane_sums_to_average(") == 1
+    # cleared, summed into, averaged: in that order, on the operator's own workspace (2 images x 128 channels of int32)
+    order = [body.index(k) for k in ("sofie_hip_fill_zero(fCtx, workspace_op_2, static_cast<std::size_t>(256) * 4)", "a.Y = workspace_op_2",
+                                     "sofie_hip_conv_i8(fCtx, &d, &a), \"op_2", "sofie_hip_plane_sums_to_average(fCtx, tensor_")]
+    assert order[1] < order[0] < order[2] < order[3]
+    assert ", 256, 256, " in body[order[3]:order[3] + 300]        # 256 sums, planes of 256 pixels
+    # planes of 144 pixels (12 x 12) stay with the stand-alone kernel
+    assert "PLANE_SUMS" not in read(emitted, "Config5_int8_CNN_small")
+    # with a run-time batch the sums are a per-batch-entry workspace and the counts scale with the batch
+    dyn = ops_body(read(emitted, "Dynamic_int8_CNN_plane_sums"))
+    assert "a.out = SOFIE_I8OUT_I8_PLANE_SUMS" in dyn and "sofie_batch * 128" in dyn
+
+
 def test_qlinear_matmul_and_conv_integer_become_one_launch_each(emitted):
     txt = read(emitted, "QLinearMatMulRelu")
     body = ops_body(txt)

@@ -11,24 +11,28 @@ from tests.refmodels import make_int8_cnn, int8_cnn_oracle
 pytestmark = pytest.mark.gpu
 
 
-def session(rt, m):
-    return Int8CNNSession(rt, m["batch"], m["in_shape"], m["in_scale"], m["convs"], m["last_scale"], m["fc_w"], m["fc_b"])
+def session(rt, m, pool_in_conv=True):
+    return Int8CNNSession(rt, m["batch"], m["in_shape"], m["in_scale"], m["convs"], m["last_scale"], m["fc_w"], m["fc_b"], pool_in_conv)
 
 
-@pytest.mark.parametrize("batch,hw,channels", [(3, 8, (3, 16, 32)), (2, 12, (3, 64, 128, 256, 256)), (5, 16, (3, 64, 128))])
-def test_cnn_chain_matches_cpu_chain(rt, batch, hw, channels):
+# pooled: whether the last convolution can add its planes up in its store (planes of a multiple of 256 pixels)
+@pytest.mark.parametrize("batch,hw,channels,pooled", [(3, 8, (3, 16, 32), False), (2, 12, (3, 64, 128, 256, 256), False), (5, 16, (3, 64, 128), True),
+                                                      (2, 32, (3, 64, 128, 256), True), (3, 16, (3, 24), True)])
+@pytest.mark.parametrize("pool_in_conv", [False, True])
+def test_cnn_chain_matches_cpu_chain(rt, batch, hw, channels, pooled, pool_in_conv):
     from sofie_amd import Runtime
     m = make_int8_cnn(batch, hw, channels)
-    print("cnn_i8", batch, hw, channels, flush=True)
+    print("cnn_i8", batch, hw, channels, pool_in_conv, flush=True)
     rt = Runtime(0)   # a Session owns its context's arena: one context per Session
     try:
-        _check(rt, m, batch)
+        _check(rt, m, batch, pool_in_conv, pooled)
     finally:
         rt.close()
 
 
-def _check(rt, m, batch):
-    s = session(rt, m)
+def _check(rt, m, batch, pool_in_conv, pooled):
+    s = session(rt, m, pool_in_conv)
+    assert s.pool_in_conv == (pool_in_conv and pooled)
     got = s.infer(m["x"])
     want = int8_cnn_oracle(m, m["x"])
     # the last feature map, int8 NHWC on the device, bit-exact
@@ -37,10 +41,17 @@ def _check(rt, m, batch):
     for cv in m["convs"]:
         h = ob.conv_i8(h, cv["W"], cv["bias"], cv["scale"], pads=cv["pads"], strides=cv["strides"], dils=cv["dils"], relu=1, out=2, omp=True)
     c, oh, ow = s.out_shape
-    fm = np.empty((batch, oh, ow, c), dtype=np.int8)
-    rt.call("sofie_hip_download", fm.ctypes.data_as(C.c_void_p), s.p(s.off_last), C.c_size_t(fm.nbytes))
-    rt.sync()
-    assert np.array_equal(fm.transpose(0, 3, 1, 2), h)
+    if s.pool_in_conv:
+        # the last map is never stored: its plane sums are what the device holds
+        sums = np.empty((batch, c), dtype=np.int32)
+        rt.call("sofie_hip_download", sums.ctypes.data_as(C.c_void_p), s.p(s.off_sums), C.c_size_t(sums.nbytes))
+        rt.sync()
+        assert np.array_equal(sums, h.astype(np.int64).sum(axis=(2, 3)).astype(np.int32))
+    else:
+        fm = np.empty((batch, oh, ow, c), dtype=np.int8)
+        rt.call("sofie_hip_download", fm.ctypes.data_as(C.c_void_p), s.p(s.off_last), C.c_size_t(fm.nbytes))
+        rt.sync()
+        assert np.array_equal(fm.transpose(0, 3, 1, 2), h)
     assert h.any() and (h > 0).mean() > 0.05          # the maps are not degenerate
     assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
     # a second inference on the same session reuses every buffer and gives the same bits

@@ -143,3 +143,78 @@ def test_first_layer_of_an_image_network_needs_no_workspace(rt):
     want = ob.conv_i8(X, Wt, bias, scale, pads=pads, strides=strides, dils=dils, group=group, relu=1, out=2, omp=True)
     got = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, R.LAYOUT_NCHW, R.LAYOUT_NHWC, 1, ws_images=0)
     assert np.array_equal(got, want) and (want > 0).any()
+
+
+def run_conv_plane_sums(rt, X, Wt, bias, scale, case, relu, x_layout, forced_tile=None, monkeypatch=None):
+    """sofie_hip_conv_i8 with SOFIE_I8OUT_I8_PLANE_SUMS into a cleared int32 [N, Cout], then the average."""
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    d = conv_desc(N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group)
+    Xd = X if x_layout == R.LAYOUT_NCHW else np.ascontiguousarray(X.transpose(0, 2, 3, 1))
+    dX, dW, db, ds = util.to_dev(Xd), util.to_dev(Wt), util.to_dev(bias), util.to_dev(scale)
+    dS = util.to_dev(np.full((N, Cout), 123456, np.int32))     # stale contents: the caller's clear is part of the contract
+    dY = util.dev_empty((N, Cout), np.float32)
+    nb = rt.lib.sofie_hip_conv_weight_i8_packed_bytes(C.byref(d))
+    dWp = util.dev_empty((nb,), np.int8)
+    rt.call("sofie_hip_pack_conv_weight_i8", C.byref(d), util.ptr(dWp), util.ptr(dW))
+    a = R.ConvI8Args()
+    a.X, a.W, a.bias, a.scale, a.Y = util.ptr(dX), util.ptr(dWp), util.ptr(db), util.ptr(ds), util.ptr(dS)
+    a.relu, a.out, a.x_layout, a.y_layout, a.w_is_packed = relu, R.I8OUT_I8_PLANE_SUMS, x_layout, x_layout, 1
+    assert rt.lib.sofie_hip_conv_i8_workspace(C.byref(d), C.byref(a)) == 0
+    import torch
+    torch.cuda.synchronize()
+    print("conv_i8 plane sums", case, relu, x_layout, forced_tile, flush=True)
+    rt.call("sofie_hip_fill_zero", util.ptr(dS), C.c_size_t(N * Cout * 4))
+    rt.call("sofie_hip_conv_i8", C.byref(d), C.byref(a))
+    rt.call("sofie_hip_plane_sums_to_average", util.ptr(dY), util.ptr(dS), N * Cout, d.OH * d.OW, C.c_float(0.037))
+    rt.sync()
+    return util.to_host(dS), util.to_host(dY)
+
+
+PLANE_SUM_CASES = [
+    # implicit GEMM (NHWC, 64 or 128 channels per group), planes of 256 and 1024 pixels
+    ((3, 64, 16, 16, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1), R.LAYOUT_NHWC),
+    ((2, 128, 32, 32, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1), R.LAYOUT_NHWC),
+    ((2, 128, 32, 32, 96, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1), 2), R.LAYOUT_NHWC),     # grouped, 48 columns per group
+    ((5, 64, 33, 33, 64, 3, 3, (1, 1, 1, 1), (2, 2), (1, 1), 1), R.LAYOUT_NHWC),      # stride 2: 17 x 17 = 289 -> refused below
+    # rows gathered in the kernel (3 channels), either input layout
+    ((4, 3, 16, 32, 40, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1), R.LAYOUT_NCHW),
+    ((4, 3, 16, 32, 40, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1), R.LAYOUT_NHWC),
+]
+
+
+@pytest.mark.parametrize("case,x_layout", PLANE_SUM_CASES)
+@pytest.mark.parametrize("relu", [0, 1])
+@pytest.mark.parametrize("tile", [0, 64, 128, 256, 258])
+def test_conv_i8_plane_sums_equal_the_sums_of_the_stored_map(rt, case, x_layout, relu, tile, monkeypatch):
+    """The int8 feature map is never stored: the sums the kernel adds up in its store must be the sums of the map the
+    oracle computes, and the average the bits of the oracle's DequantizeLinear + GlobalAveragePool on that map."""
+    if tile:
+        monkeypatch.setenv("SOFIE_HIP_I8_TILE", str(tile))
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    X = util.int8_sym(70, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.int8_sym(71, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
+    bias = util.int32_range(72, Cout, -2000, 2000)
+    K = (Cc // group) * kh * kw
+    scale = ((0.5 + util.uniform01(73, Cout)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    OH = (H + pads[0] + pads[2] - dils[0] * (kh - 1) - 1) // strides[0] + 1
+    OW = (W + pads[1] + pads[3] - dils[1] * (kw - 1) - 1) // strides[1] + 1
+    if (OH * OW) % 256:
+        with pytest.raises(R.SofieHipError, match="multiple of 256"):
+            run_conv_plane_sums(rt, X, Wt, bias, scale, case, relu, x_layout)
+        return
+    sums, avg = run_conv_plane_sums(rt, X, Wt, bias, scale, case, relu, x_layout, tile)
+    fmap = ob.conv_i8(X, Wt, bias, scale, pads=pads, strides=strides, dils=dils, group=group, relu=relu, out=2, omp=True)
+    want_sums = fmap.astype(np.int64).sum(axis=(2, 3))
+    assert np.array_equal(sums, want_sums.astype(np.int32))
+    assert np.abs(want_sums).max() > 100          # the case does exercise the sums
+    want_avg = ob.global_avg_pool_i8(fmap, 0.037)
+    assert np.array_equal(avg.view(np.uint32), want_avg.view(np.uint32))
+
+
+def test_conv_i8_plane_sums_refuse_a_column_matrix_shape(rt):
+    case = (2, 16, 16, 16, 32, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1)     # 144-byte reduction over NCHW input: needs a column matrix
+    N, Cc, H, W, Cout, kh, kw, *_ = case
+    X = util.int8_sym(74, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.int8_sym(75, Cout * Cc * kh * kw).reshape(Cout, Cc, kh, kw)
+    with pytest.raises((R.SofieHipError, AssertionError)):
+        run_conv_plane_sums(rt, X, Wt, np.zeros(Cout, np.int32), np.ones(Cout, np.float32), case, 0, R.LAYOUT_NCHW)

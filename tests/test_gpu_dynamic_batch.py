@@ -127,6 +127,20 @@ def test_dynamic_int8_cnn_matches_cpu_chain_for_every_batch(rt):
             assert np.abs(want).max() > 1e-3
 
 
+def test_dynamic_int8_cnn_with_plane_sums_for_every_batch(rt):
+    from tests.refmodels import int8_cnn_oracle
+    spec = em.int8_cnn(2, 16, (3, 64, 128))
+    x = np.concatenate([spec["feeds"][0], util.uniform01(8202, 3 * 3 * 16 * 16).reshape(3, 3, 16, 16)])
+    with DynamicSession("Dynamic_int8_CNN_plane_sums", 5) as s:
+        for n in (5, 2, 1, 5):
+            want = int8_cnn_oracle(spec["consts"], x[:n]).ravel()
+            print("Dynamic_int8_CNN_plane_sums batch", n, flush=True)
+            got = s.infer(n, [x[:n]], 50)
+            assert got.size == want.size == n * 10
+            assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+            assert np.abs(want).max() > 1e-3
+
+
 def test_dynamic_conv_batchnorm_relu(rt):
     spec = em.conv_batchnorm_relu(2)
     g = onnx_lite.load(os.path.join(em.OUT, "ConvBatchNormRelu.onnx"))     # the same weights with a fixed batch of 2

@@ -76,6 +76,19 @@ def test_emitted_int8_cnn_matches_cpu_chain(rt):
     assert np.abs(want).max() > 1e-3
 
 
+def test_emitted_int8_cnn_whose_last_convolution_sums_its_planes(rt):
+    """Planes of 256 pixels: the GlobalAveragePool joins the last QLinearConv, whose feature map is never stored."""
+    from tests.refmodels import int8_cnn_oracle
+    spec = em.int8_cnn(2, 16, (3, 64, 128))
+    want = int8_cnn_oracle(spec["consts"], spec["feeds"][0]).ravel()
+    print("emitted Int8_CNN_plane_sums", flush=True)
+    got = run_emitted("Int8_CNN_plane_sums", spec["feeds"], want.size)
+    assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+    assert np.abs(want).max() > 1e-3
+    txt = open(os.path.join(em.OUT, "Int8_CNN_plane_sums_GPU_HIP.hxx")).read()
+    assert txt.count("SOFIE_I8OUT_I8_PLANE_SUMS") == 1 and "sofie_hip_plane_sums_to_average" in txt and "sofie_hip_global_avg_pool_i8" not in txt
+
+
 def test_model_built_through_the_api_external_stream_option(rt):
     # Y = Relu(X[1,3] * ones[3,1] + 0.5): ones -> 3.5 (the reference's tests/alpaka/TestAlpakaExternalStream.cxx:34-37)
     got = run_emitted("ApiGemmRelu", [np.ones((1, 3), np.float32)], 1)
