@@ -153,6 +153,13 @@ typedef struct sofie_gemm_f32_desc {
    const float *residual;
 } sofie_gemm_f32_desc;
 int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d);
+/* `count` products of which each reads what the one before wrote (layers[l].A == layers[l-1].Y): the Gemm + activation
+ * sequence the reference emits for an MLP, one blas call and one Relu pass per layer (ROperator_Gemm.hxx:685-741).  The
+ * results are those of `count` calls of sofie_hip_gemm_f32 in order, every Y written.  At small M (up to 256 rows, no transA,
+ * no stacking, rows of at most 2048 to 8192 floats) the whole chain is ONE launch, the activations passing from layer to
+ * layer through LDS; otherwise the call is the loop over the layers. */
+#define SOFIE_MAX_GEMM_CHAIN 16
+int sofie_hip_gemm_chain_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *layers, int32_t count);
 
 /* ---- int8 Gemm (MatMulInteger + fused requantisation) -------------------------------------- */
 /* No counterpart exists in the reference (ROperator_Gemm is float only,

@@ -301,6 +301,134 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(ConvOperandA la, const fl
 
 } // namespace sofie_hip
 
+namespace sofie_hip {
+
+// ---- a chain of small products in one launch -----------------------------------------------------------------
+// Layer l+1 reads what layer l wrote (an MLP at small batch): per layer launches cost more than the arithmetic, so one
+// workgroup takes RB rows through every layer, the rows of activations staying in LDS between layers (each layer's
+// output is also written to its Y, as separate launches would).  The weights stream from L2 once per workgroup:
+//   transB (W stored [N][K], the ONNX export of a Linear layer): a wave takes 4 outputs at a time, its lanes stride over k
+//     (coalesced 256-byte reads of each weight row), then the 64 partial sums are folded with shuffles;
+//   else (W stored [K][N]): a thread owns output n and walks k (lanes read consecutive n of one weight row).
+struct ChainLayerArgs {
+   const float *B;
+   long long ldb;
+   int transB, N, K;
+   float *Y;
+   long long ldy;
+   F32Epilogue ep;
+};
+struct ChainArgs {
+   int count, M;
+   const float *A;
+   long long lda;
+   ChainLayerArgs layer[SOFIE_MAX_GEMM_CHAIN];
+};
+
+// 16 waves per workgroup: what a layer costs is the round trips to L2 for its weights, and the waves' loads overlap
+constexpr int CHAIN_THREADS = 1024;
+
+template <int RB>
+__global__ __launch_bounds__(CHAIN_THREADS) void gemm_chain_f32_kernel(ChainArgs a, int width)
+{
+   extern __shared__ float chain_lds[]; // two buffers of RB rows x width
+   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+   const int m0 = blockIdx.x * RB;
+   const int rows = (a.M - m0) < RB ? (a.M - m0) : RB;
+   float *in = chain_lds, *out = chain_lds + RB * width;
+   // rows beyond the matrix are kept at zero so that the loops below need no row test
+   if (rows < RB) {
+      for (int i = t; i < 2 * RB * width; i += CHAIN_THREADS)
+         chain_lds[i] = 0.0f;
+      __syncthreads();
+   }
+   const int K0 = a.layer[0].K;
+   for (int r = 0; r < rows; ++r)
+      for (int k = t; k < K0; k += CHAIN_THREADS)
+         in[r * width + k] = a.A[(long long)(m0 + r) * a.lda + k];
+   __syncthreads();
+   for (int l = 0; l < a.count; ++l) {
+      const ChainLayerArgs &L = a.layer[l];
+      const int N = L.N, K = L.K;
+      const float *__restrict__ B = L.B;
+      if (L.transB) {
+         for (int n0 = wave * 4; n0 < N; n0 += CHAIN_THREADS / 16) {
+            float acc[4][RB];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+               for (int r = 0; r < RB; ++r)
+                  acc[j][r] = 0.0f;
+            // rows of W past N are read as row N-1 and their sums dropped
+            const float *w0 = B + (long long)(n0 + 0 < N ? n0 + 0 : N - 1) * L.ldb;
+            const float *w1 = B + (long long)(n0 + 1 < N ? n0 + 1 : N - 1) * L.ldb;
+            const float *w2 = B + (long long)(n0 + 2 < N ? n0 + 2 : N - 1) * L.ldb;
+            const float *w3 = B + (long long)(n0 + 3 < N ? n0 + 3 : N - 1) * L.ldb;
+            // (issuing the loads of eight guarded k-positions at once instead, with no remainder loop, measured slower)
+#pragma unroll 8
+            for (int k = lane; k < K; k += 64) {
+               const float w[4] = {w0[k], w1[k], w2[k], w3[k]};
+#pragma unroll
+               for (int r = 0; r < RB; ++r) {
+                  const float x = in[r * width + k];
+#pragma unroll
+                  for (int j = 0; j < 4; ++j)
+                     acc[j][r] = fmaf(w[j], x, acc[j][r]);
+               }
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1)
+#pragma unroll
+               for (int j = 0; j < 4; ++j)
+#pragma unroll
+                  for (int r = 0; r < RB; ++r)
+                     acc[j][r] += __shfl_xor(acc[j][r], off, 64);
+            // every lane now holds the 4 x RB sums: lane j finishes output n0 + j
+            const int n = n0 + lane;
+            if (lane < 4 && n < N) {
+#pragma unroll
+               for (int r = 0; r < RB; ++r) {
+                  if (r < rows) {
+                     const float s = lane == 0 ? acc[0][r] : lane == 1 ? acc[1][r] : lane == 2 ? acc[2][r] : acc[3][r];
+                     const float v = f32_epilogue(L.ep, s, m0 + r, n);
+                     out[r * width + n] = v;
+                     L.Y[(long long)(m0 + r) * L.ldy + n] = v;
+                  }
+               }
+            }
+         }
+      } else {
+         for (int n = t; n < N; n += CHAIN_THREADS) {
+            float acc[RB];
+#pragma unroll
+            for (int r = 0; r < RB; ++r)
+               acc[r] = 0.0f;
+#pragma unroll 8
+            for (int k = 0; k < K; ++k) {
+               const float w = B[(long long)k * L.ldb + n];
+#pragma unroll
+               for (int r = 0; r < RB; ++r)
+                  acc[r] = fmaf(w, in[r * width + k], acc[r]);
+            }
+#pragma unroll
+            for (int r = 0; r < RB; ++r) {
+               if (r < rows) {
+                  const float v = f32_epilogue(L.ep, acc[r], m0 + r, n);
+                  out[r * width + n] = v;
+                  L.Y[(long long)(m0 + r) * L.ldy + n] = v;
+               }
+            }
+         }
+      }
+      __syncthreads();
+      float *tmp = in;
+      in = out;
+      out = tmp;
+   }
+}
+
+} // namespace sofie_hip
+
 using namespace sofie_hip;
 
 extern "C" {
@@ -362,6 +490,69 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d)
    hipLaunchKernelGGL(gemm_f32_kernel, dim3(gy, gx, (unsigned)d->batch), dim3(256), 0, ctx->stream, la, lb, M, N, K, d->Y, ldy, ep,
                       (long long)d->strideA, (long long)d->strideB, (long long)d->strideC, (long long)d->strideY);
    return launch_status("gemm_f32_kernel");
+}
+
+int sofie_hip_gemm_chain_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *layers, int32_t count)
+{
+   SOFIE_HIP_REQUIRE(ctx && layers, "sofie_hip_gemm_chain_f32: NULL argument");
+   SOFIE_HIP_REQUIRE(count >= 1 && count <= SOFIE_MAX_GEMM_CHAIN, "sofie_hip_gemm_chain_f32: %d layers (1..%d allowed)", count, SOFIE_MAX_GEMM_CHAIN);
+   for (int l = 1; l < count; ++l)
+      SOFIE_HIP_REQUIRE(layers[l].A == layers[l - 1].Y && layers[l].A != nullptr, "sofie_hip_gemm_chain_f32: layer %d does not read the output of layer %d", l, l - 1);
+   // One launch when the batch is small enough that launches, not arithmetic, set the time, and the rows fit in LDS.
+   const char *force = getenv("SOFIE_HIP_F32_CHAIN");
+   const int M = layers[0].M;
+   bool fused = count >= 2 && M >= 1 && (force ? atoi(force) != 0 : M <= 256);
+   int width = layers[0].K;
+   ChainArgs a;
+   a.count = count;
+   a.M = M;
+   a.A = layers[0].A;
+   a.lda = layers[0].lda ? layers[0].lda : layers[0].K;
+   for (int l = 0; l < count && fused; ++l) {
+      const sofie_gemm_f32_desc &d = layers[l];
+      const long long ldb = d.ldb ? d.ldb : (d.transB ? d.K : d.N), ldy = d.ldy ? d.ldy : d.N;
+      fused = d.M == M && d.N >= 1 && d.K >= 1 && !d.transA && d.batch == 1 && d.A && d.B && d.Y && ldb >= (d.transB ? d.K : d.N) && ldy >= d.N &&
+              d.bias_mode >= SOFIE_BIAS_NONE && d.bias_mode <= SOFIE_BIAS_FULL && (d.bias_mode == SOFIE_BIAS_NONE || d.C != nullptr) &&
+              (l == 0 ? a.lda >= d.K : (d.K == layers[l - 1].N && (d.lda ? d.lda : d.K) == (layers[l - 1].ldy ? layers[l - 1].ldy : layers[l - 1].N)));
+      if (!fused)
+         break;
+      ChainLayerArgs &L = a.layer[l];
+      L.B = d.B;
+      L.ldb = ldb;
+      L.transB = d.transB ? 1 : 0;
+      L.N = d.N;
+      L.K = d.K;
+      L.Y = d.Y;
+      L.ldy = ldy;
+      int bad = 0;
+      fused = make_post_chain(L.ep.chain, d.act, d.act_alpha, d.post, bad);
+      L.ep.alpha = d.alpha;
+      L.ep.beta = d.beta;
+      L.ep.C = d.bias_mode == SOFIE_BIAS_NONE ? nullptr : d.C;
+      L.ep.bias_mode = d.bias_mode;
+      L.ep.ldc = d.N;
+      L.ep.R = d.residual;
+      L.ep.ldr = ldy;
+      width = d.N > width ? d.N : width;
+   }
+   const int RB = M <= 64 ? 1 : M <= 128 ? 2 : 4;
+   width = (width + 3) / 4 * 4;
+   if (fused && (long long)RB * width <= 8192) {
+      const size_t lds = (size_t)2 * RB * width * sizeof(float);
+      const dim3 grid((unsigned)((M + RB - 1) / RB));
+      if (RB == 1)
+         hipLaunchKernelGGL(gemm_chain_f32_kernel<1>, grid, dim3(CHAIN_THREADS), lds, ctx->stream, a, width);
+      else if (RB == 2)
+         hipLaunchKernelGGL(gemm_chain_f32_kernel<2>, grid, dim3(CHAIN_THREADS), lds, ctx->stream, a, width);
+      else
+         hipLaunchKernelGGL(gemm_chain_f32_kernel<4>, grid, dim3(CHAIN_THREADS), lds, ctx->stream, a, width);
+      return launch_status("gemm_chain_f32_kernel");
+   }
+   // anything else (and every malformed descriptor, which the single product reports): one launch per layer
+   for (int l = 0; l < count; ++l)
+      if (int st = sofie_hip_gemm_f32(ctx, &layers[l]))
+         return st;
+   return SOFIE_HIP_OK;
 }
 
 int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float *X, const float *W, const float *bias,

@@ -35,6 +35,7 @@ struct PostOp {
    float alpha = 0.f, beta = 0.f;
 };
 constexpr std::size_t kMaxPostOps = 4; // SOFIE_MAX_POST_OPS of the runtime
+constexpr std::size_t kMaxGemmChain = 16; // SOFIE_MAX_GEMM_CHAIN of the runtime
 
 // Options of RModel::GenerateGPU_HIP: the subset of the reference's bit flags (core/inc/SOFIE/RModel_Base.hxx:19-33)
 // that applies to this backend, with the reference's values.

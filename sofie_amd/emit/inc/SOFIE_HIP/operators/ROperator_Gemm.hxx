@@ -301,26 +301,38 @@ public:
       if (fIsOutputConstant)
          return "\n" + SP + "//--------- Gemm " + opName + " -> " + fNY + ": a product of weights, computed when the code was generated\n";
       std::stringstream out;
-      out << "\n" << SP << "//--------- Gemm " << opName << " " << ConvertShapeToString(fShapeA) << " * " << ConvertShapeToString(fShapeB)
-          << " -> " << fNY << "\n";
+      out << "\n" << SP << "//--------- Gemm " << opName << " " << Title() << "\n";
       out << SP << "{\n";
       out << SP << "   " << "sofie_gemm_f32_desc d{};\n";
-      out << SP << "   " << "d.M = " << BatchScaledInt(fDynamicRows, fM) << "; d.N = " << fN << "; d.K = " << fK << "; d.transA = " << (fAttrTransA ? 1 : 0)
-          << "; d.transB = " << (fAttrTransB ? 1 : 0) << ";\n";
-      out << SP << "   " << "d.alpha = " << FloatLiteral(fAttrAlpha) << "; d.beta = " << FloatLiteral(fAttrBeta) << ";\n";
-      out << SP << "   " << "d.A = tensor_" << fNA << "; d.B = tensor_" << fNB << "; d.C = " << (fNC.empty() ? "nullptr" : "tensor_" + fNC)
-          << "; d.bias_mode = " << fBiasMode << ";\n";
-      out << SP << "   " << "d.act = " << ActivationEnumName(fActivation) << "; d.act_alpha = " << FloatLiteral(fActAlpha) << ";\n";
-      out << SP << "   " << "d.Y = tensor_" << fNY << "; d.batch = " << BatchScaledInt(fDynamicStack, fBatch) << "; d.strideA = " << fStrideA << "; d.strideB = "
-          << fStrideB << "; d.strideC = " << fStrideC << "; d.strideY = " << (fBatch > 1 || fDynamicStack ? fM * fN : 0) << ";\n";
-      if (!fPost.empty())
-         out << SP << "   " << PostOpsDeclaration("post", fPost) << " d.post = &post;\n";
-      if (!fNR.empty())
-         out << SP << "   " << "d.residual = tensor_" << fNR << ";\n";
+      out << DescriptorStatements("d", "post");
       out << SP << "   " << "detail::Check(sofie_hip_gemm_f32(fCtx, &d), \"" << opName << " Gemm\");\n";
       out << SP << "}\n";
       return out.str();
    }
+   std::string Title() const { return ConvertShapeToString(fShapeA) + " * " + ConvertShapeToString(fShapeB) + " -> " + fNY; }
+   // the statements that fill the sofie_gemm_f32_desc named `d` (a post-operator block, if any, is declared as `post`)
+   std::string DescriptorStatements(const std::string &d, const std::string &post) const
+   {
+      std::stringstream out;
+      out << SP << "   " << d << ".M = " << BatchScaledInt(fDynamicRows, fM) << "; " << d << ".N = " << fN << "; " << d << ".K = " << fK << "; " << d
+          << ".transA = " << (fAttrTransA ? 1 : 0) << "; " << d << ".transB = " << (fAttrTransB ? 1 : 0) << ";\n";
+      out << SP << "   " << d << ".alpha = " << FloatLiteral(fAttrAlpha) << "; " << d << ".beta = " << FloatLiteral(fAttrBeta) << ";\n";
+      out << SP << "   " << d << ".A = tensor_" << fNA << "; " << d << ".B = tensor_" << fNB << "; " << d << ".C = " << (fNC.empty() ? "nullptr" : "tensor_" + fNC)
+          << "; " << d << ".bias_mode = " << fBiasMode << ";\n";
+      out << SP << "   " << d << ".act = " << ActivationEnumName(fActivation) << "; " << d << ".act_alpha = " << FloatLiteral(fActAlpha) << ";\n";
+      out << SP << "   " << d << ".Y = tensor_" << fNY << "; " << d << ".batch = " << BatchScaledInt(fDynamicStack, fBatch) << "; " << d << ".strideA = " << fStrideA
+          << "; " << d << ".strideB = " << fStrideB << "; " << d << ".strideC = " << fStrideC << "; " << d << ".strideY = "
+          << (fBatch > 1 || fDynamicStack ? fM * fN : 0) << ";\n";
+      if (!fPost.empty())
+         out << SP << "   " << PostOpsDeclaration(post, fPost) << " " << d << ".post = &" << post << ";\n";
+      if (!fNR.empty())
+         out << SP << "   " << d << ".residual = tensor_" << fNR << ";\n";
+      return out.str();
+   }
+   // Can this product stand in a chain handed to sofie_hip_gemm_chain_f32 (it exists at run time and is a plain 2-D product)?
+   bool IsChainLink() const { return fM != 0 && !fIsOutputConstant && fBatch == 1 && !fDynamicStack && !fAttrTransA; }
+   const std::string &NameA() const { return fNA; }
+   const std::string &NameY() const { return fNY; }
 
 private:
    float fAttrAlpha = 1.0, fAttrBeta = 1.0;

@@ -1067,8 +1067,33 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    gc << ")\n   {";
    if (dyn)
       gc << "\n      (void)sofie_batch;";
-   for (std::size_t i = 0; i < fOperators.size(); ++i)
-      gc << fOperators[i]->Generate_GPU_HIP(std::to_string(i));
+   for (std::size_t i = 0; i < fOperators.size(); ++i) {
+      // Consecutive products of which each reads what the one before wrote (the layers of an MLP) go to the runtime as one
+      // call: at small batch it runs them in a single launch, otherwise layer by layer -- the results are the same.
+      std::vector<ROperator_Gemm<float> *> chain;
+      for (std::size_t j = i; j < fOperators.size() && chain.size() < kMaxGemmChain; ++j) {
+         auto *g = dynamic_cast<ROperator_Gemm<float> *>(fOperators[j].get());
+         if (!g || !g->IsChainLink() || (!chain.empty() && g->NameA() != chain.back()->NameY()))
+            break;
+         chain.push_back(g);
+      }
+      if (chain.size() < 2) {
+         gc << fOperators[i]->Generate_GPU_HIP(std::to_string(i));
+         continue;
+      }
+      const std::string last = std::to_string(i + chain.size() - 1);
+      const std::string SP = "      "; // the operators' indentation inside doInfer
+      gc << "\n" << SP << "//--------- Gemm chain op_" << i << " .. op_" << last << "\n";
+      gc << SP << "{\n";
+      gc << SP << "   " << "sofie_gemm_f32_desc chain[" << chain.size() << "]{};\n";
+      for (std::size_t l = 0; l < chain.size(); ++l) {
+         gc << SP << "   " << "// op_" << (i + l) << " " << chain[l]->Title() << "\n";
+         gc << chain[l]->DescriptorStatements("chain[" + std::to_string(l) + "]", "post_" + std::to_string(l));
+      }
+      gc << SP << "   " << "detail::Check(sofie_hip_gemm_chain_f32(fCtx, chain, " << chain.size() << "), \"op_" << i << " .. op_" << last << " Gemm chain\");\n";
+      gc << SP << "}\n";
+      i += chain.size() - 1;
+   }
    gc << "   }\n\n";
    auto boundArgs = [&](const std::string &inPrefix, const std::string &outPrefix) {
       std::string a = dyn ? "static_cast<std::int64_t>(" + bp + ")" : "";

@@ -125,6 +125,7 @@ SYMBOLS = {
     "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),
     "sofie_hip_global_avg_pool_f32": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32]),
     "sofie_hip_pool_f32": (C.c_int, [_P, _P, _P, _P]),
+    "sofie_hip_gemm_chain_f32": (C.c_int, [_P, _P, C.c_int32]),
     "sofie_hip_plane_sums_to_average": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_float]),
     "sofie_hip_batchnorm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "sofie_hip_global_avg_pool_i8": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float]),

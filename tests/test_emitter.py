@@ -89,9 +89,10 @@ def test_session_api_of_the_generated_header(emitted):
 def test_gemm_relu_pairs_are_fused(emitted):
     txt = read(emitted, "Linear_16")
     body = ops_body(txt)
-    assert body.count("sofie_hip_gemm_f32") == 10
+    # ten layers, each reading its predecessor: one chain call
+    assert body.count("sofie_hip_gemm_chain_f32(fCtx, chain, 10)") == 1 and "sofie_hip_gemm_f32(" not in body
     assert "sofie_hip_unary_f32" not in body          # every Relu went into a Gemm epilogue
-    assert body.count("SOFIE_ACT_RELU") == 9
+    assert body.count(".act = SOFIE_ACT_RELU") == 9
     txt = read(emitted, "LinearWithSigmoid")
     assert "SOFIE_ACT_SIGMOID" in txt
 
