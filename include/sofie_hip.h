@@ -99,7 +99,9 @@ enum {
    SOFIE_ACT_ATANH = 20,
    SOFIE_ACT_CLIP = 21,      /* max(alpha, min(beta, x))              */
    SOFIE_ACT_SELU = 22,      /* beta * (max(0,x) + min(0, alpha*(exp(x)-1))), beta = gamma; core/inc/SOFIE/operators/ROperator_Selu.hxx:56-62 */
-   SOFIE_ACT_LAST = 22
+   SOFIE_ACT_ELU = 23,       /* x >= 0 ? x : alpha * (exp(x) - 1); core/inc/SOFIE/operators/ROperator_Elu.hxx:69-74 */
+   SOFIE_ACT_ERF = 24,       /* std::erf(x); core/inc/SOFIE/operators/ROperator_Erf.hxx */
+   SOFIE_ACT_LAST = 24
 };
 
 /* A chain of one-to-one operators applied, in order, to every element an operator stores: what the reference's
@@ -346,6 +348,13 @@ int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y /* [N,C] */, const
  * on the feature map that was never stored. */
 int sofie_hip_plane_sums_to_average(sofie_hip_ctx *ctx, float *Y /* [NC] */, const int32_t *sums /* [NC] */, int32_t NC, int32_t HW,
                                     float scale);
+
+/* Softmax / LogSoftmax along one axis of a tensor seen as [outer, axis_len, inner] (ROperator_Softmax::Generate,
+ * core/inc/SOFIE/operators/ROperator_Softmax.hxx:82-198): vmax = max over the axis, e = exp(x - vmax), sum = sum of e;
+ * Softmax gives e * (1.0f / sum) when the axis is the last one (inner == 1, :114-117) and e / sum otherwise (:188); LogSoftmax
+ * gives x - vmax - log(sum).  The sum is a tree over the axis here, a sequential loop in the reference: results agree to
+ * the rounding of that sum, which for the loop grows with the axis length (1e-7 relative at 10 classes, 6e-5 at 70000). */
+int sofie_hip_softmax_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int64_t outer, int32_t axis_len, int64_t inner, int32_t log_softmax);
 
 /* BatchNormalization at inference, for models whose normalisation was not folded into the weights
  * (core/inc/SOFIE/operators/ROperator_BatchNormalization.hxx:139-158): X is [N, C, spatial...],

@@ -174,6 +174,15 @@ def pool(X, mode, kernel_shape, pads=None, strides=None, dilations=None, auto_pa
     return Y
 
 
+def softmax(X, axis=-1, log=False):
+    X = _f32(X)
+    axis = axis + X.ndim if axis < 0 else axis
+    outer, A, inner = int(np.prod(X.shape[:axis], dtype=np.int64)), X.shape[axis], int(np.prod(X.shape[axis + 1:], dtype=np.int64))
+    Y = np.empty_like(X)
+    load().oracle_softmax(_ptr(Y), _ptr(X), C.c_long(outer), C.c_int(A), C.c_long(inner), C.c_int(1 if log else 0))
+    return Y
+
+
 def batchnorm(X, scale, bias, mean, var, eps=1e-5, relu=0):
     X = _f32(X)
     Cc = X.shape[1]

@@ -16,9 +16,12 @@
  *                             convolution in float64.
  *   relu/sigmoid/gelu/...     Gelu / GeluTanh / LinearWithSelu golden outputs; closed forms.
  *   basic_unary, unary_chain  numpy's float32 routines (an independent implementation) and identities
- *                             (exp(log x) = x, sin^2 + cos^2 = 1, sinh(asinh x) = x, ...); Clip bounds; Selu
- *                             through the LinearWithSelu golden output.
+ *                             (exp(log x) = x, sin^2 + cos^2 = 1, sinh(asinh x) = x, ...); Clip bounds; the golden
+ *                             outputs Sqrt, Reciprocal, Exp, Log, Neg, Elu, SeluNonDefaultCoeffs, LinearWithSelu of the
+ *                             reference's tests; Erf against scipy's erf.
  *   global_avg_pool           GlobalAvgPool2d golden output.
+ *   softmax                   Softmax1d / 2d / 3d / 4d golden outputs; scipy's softmax and log_softmax in float64; rows sum
+ *                             to 1; invariance under a shift of the input.
  *   pool2d                    MaxPool1d, MaxPool2d, AvgPool, AvgPoolPad, AvgPoolCountIncludePad golden outputs;
  *                             a float64 restatement of the ONNX definition over random geometries (ceil_mode and
  *                             both divisor conventions included); torch's max_pool / avg_pool; window = image is
@@ -147,6 +150,8 @@ ORACLE_API void oracle_basic_unary(float *out, const float *in, size_t n, int op
       case 20: y = atanhf(x); break;
       case 21: y = fmaxf(alpha, fminf(beta, x)); break;
       case 22: y = beta * (fmaxf(0.0f, x) + fminf(0.0f, alpha * (expf(x) - 1.0f))); break; /* Selu, ROperator_Selu.hxx:56-62; beta = gamma */
+      case 23: y = x >= 0.0f ? x : alpha * (expf(x) - 1.0f); break; /* Elu, ROperator_Elu.hxx:69-74 */
+      case 24: y = erff(x); break;                                  /* Erf, ROperator_Erf.hxx: std::erf */
       default: break;
       }
       out[i] = y;
@@ -164,7 +169,7 @@ ORACLE_API void oracle_unary(float *out, const float *in, size_t n, int act, flo
    case 5: oracle_gelu_tanh(out, in, n); break;
    case 6: oracle_tanh(out, in, n); break;
    default:
-      if (act >= 7 && act <= 22)
+      if (act >= 7 && act <= 24)
          oracle_basic_unary(out, in, n, act, alpha, 0.0f);
       else if (out != in)
          memmove(out, in, n * sizeof(float));
@@ -177,7 +182,7 @@ ORACLE_API void oracle_unary_chain(float *out, const float *in, size_t n, int co
    if (out != in)
       memmove(out, in, n * sizeof(float));
    for (int i = 0; i < count; ++i) {
-      if (op[i] >= 7 && op[i] <= 22)
+      if (op[i] >= 7 && op[i] <= 24)
          oracle_basic_unary(out, out, n, op[i], alpha[i], beta[i]);
       else
          oracle_unary(out, out, n, op[i], alpha[i]);
@@ -395,6 +400,40 @@ ORACLE_API long oracle_pool2d(float *Y, const float *X, int planes, int H, int W
       }
    }
    return planes ? (long)(out / (size_t)planes) : 0;
+}
+
+/* Softmax / LogSoftmax over the middle dimension of [outer, A, inner], the loops of ROperator_Softmax::Generate
+ * (core/inc/SOFIE/operators/ROperator_Softmax.hxx): last axis (:92-119) y = exp(x - vmax), sum += y in order, then
+ * y *= 1.0f / sum (or x - vmax - log(sum)); any other axis (:121-198) the same with y /= sum. */
+ORACLE_API void oracle_softmax(float *Y, const float *X, long outer, int A, long inner, int log_softmax)
+{
+   for (long o = 0; o < outer; ++o) {
+      for (long in = 0; in < inner; ++in) {
+         const float *x = X + (size_t)o * A * inner + in;
+         float *y = Y + (size_t)o * A * inner + in;
+         float vmax = x[0];
+         for (int i = 1; i < A; ++i)
+            if (x[(size_t)i * inner] > vmax)
+               vmax = x[(size_t)i * inner];
+         float sum = 0.0f;
+         for (int i = 0; i < A; ++i) {
+            y[(size_t)i * inner] = expf(x[(size_t)i * inner] - vmax);
+            sum += y[(size_t)i * inner];
+         }
+         if (log_softmax) {
+            float log_sum = logf(sum);
+            for (int i = 0; i < A; ++i)
+               y[(size_t)i * inner] = x[(size_t)i * inner] - vmax - log_sum;
+         } else if (inner == 1) {
+            float inv_sum = 1.0f / sum;
+            for (int i = 0; i < A; ++i)
+               y[i] *= inv_sum;
+         } else {
+            for (int i = 0; i < A; ++i)
+               y[(size_t)i * inner] /= sum;
+         }
+      }
+   }
 }
 
 /* BatchNormalization at inference (core/inc/SOFIE/operators/ROperator_BatchNormalization.hxx:92-109, 139-148):

@@ -81,6 +81,8 @@ static __device__ __noinline__ float apply_basic_unary(float v, int act, float a
    case SOFIE_ACT_ATANH: return atanhf(v);
    case SOFIE_ACT_CLIP: return fmaxf(alpha, fminf(beta, v));
    case SOFIE_ACT_SELU: return beta * (fmaxf(0.0f, v) + fminf(0.0f, alpha * (expf(v) - 1.0f)));
+   case SOFIE_ACT_ELU: return v >= 0.0f ? v : alpha * (expf(v) - 1.0f);
+   case SOFIE_ACT_ERF: return erff(v);
    default: return v;
    }
 }

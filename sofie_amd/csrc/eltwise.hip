@@ -172,6 +172,48 @@ __global__ __launch_bounds__(256) void gap_i8_nhwc_kernel(float *__restrict__ Y,
    }
 }
 
+// Softmax over the middle dimension of [outer, A, inner]: one wave per (outer, inner) line, lanes stride over the axis
+// (consecutive lanes read consecutive elements when inner == 1), three passes over a line that stays in cache.
+__global__ __launch_bounds__(256) void softmax_f32_kernel(float *__restrict__ Y, const float *__restrict__ X, long long lines, int A, long long inner,
+                                                          int log_softmax)
+{
+   const int lane = threadIdx.x & 63;
+   const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6), nwaves = (long long)gridDim.x * 4;
+   for (long long line = wave; line < lines; line += nwaves) {
+      const long long o = line / inner, in = line - o * inner;
+      const float *x = X + o * A * inner + in;
+      float *y = Y + o * A * inner + in;
+      float vmax = -INFINITY;
+      for (int i = lane; i < A; i += 64) {
+         const float v = x[i * inner];
+         vmax = v > vmax ? v : vmax;
+      }
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) {
+         const float other = __shfl_xor(vmax, off, 64);
+         vmax = other > vmax ? other : vmax;
+      }
+      float sum = 0.0f;
+      for (int i = lane; i < A; i += 64)
+         sum += expf(x[i * inner] - vmax);
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1)
+         sum += __shfl_xor(sum, off, 64);
+      if (log_softmax) {
+         const float log_sum = logf(sum);
+         for (int i = lane; i < A; i += 64)
+            y[i * inner] = x[i * inner] - vmax - log_sum;
+      } else if (inner == 1) {
+         const float inv_sum = 1.0f / sum;
+         for (int i = lane; i < A; i += 64)
+            y[i] = mul_nofma(expf(x[i] - vmax), inv_sum);
+      } else {
+         for (int i = lane; i < A; i += 64)
+            y[i * inner] = __fdiv_rn(expf(x[i * inner] - vmax), sum);
+      }
+   }
+}
+
 // The last step of an average whose integer plane sums already exist (a convolution added them up in its store).
 __global__ __launch_bounds__(256) void plane_sums_to_average_kernel(float *__restrict__ Y, const int32_t *__restrict__ sums, int NC, int HW,
                                                                     float scale)
@@ -415,6 +457,21 @@ int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y, const int8_t *X, 
    const int NC = N * C;
    hipLaunchKernelGGL((gap_kernel<int8_t, int>), dim3((NC + 3) / 4), dim3(256), 0, ctx->stream, Y, X, NC, HW, scale);
    return launch_status("gap_kernel");
+}
+
+int sofie_hip_softmax_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int64_t outer, int32_t axis_len, int64_t inner, int32_t log_softmax)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_softmax_f32: ctx is NULL");
+   SOFIE_HIP_REQUIRE(outer >= 0 && axis_len > 0 && inner > 0, "sofie_hip_softmax_f32: bad shape");
+   SOFIE_HIP_REQUIRE(outer < (1LL << 40) && inner < (1LL << 40) && (double)outer * axis_len * (double)inner < 1.0e12, "sofie_hip_softmax_f32: tensor too large");
+   const long long lines = (long long)outer * inner;
+   if (lines == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(Y && X, "sofie_hip_softmax_f32: NULL pointer");
+   const long long blocks = (lines + 3) / 4;
+   hipLaunchKernelGGL(softmax_f32_kernel, dim3((unsigned)(blocks < 256 * 64 ? blocks : 256 * 64)), dim3(256), 0, ctx->stream, Y, X, lines, axis_len,
+                      (long long)inner, log_softmax);
+   return launch_status("softmax_f32_kernel");
 }
 
 int sofie_hip_plane_sums_to_average(sofie_hip_ctx *ctx, float *Y, const int32_t *sums, int32_t NC, int32_t HW, float scale)

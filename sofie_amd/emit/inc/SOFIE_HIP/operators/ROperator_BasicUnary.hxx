@@ -146,6 +146,16 @@ struct ROperator_Selu : ROperator_Activation {
    ROperator_Selu(std::string x, std::string y) : ROperator_Selu(1.67326319217681884765625f, 1.05070102214813232421875f, x, y) {}
    ROperator_Selu(float alpha, float gamma, std::string x, std::string y) : ROperator_Activation(EActivationType::SELU, alpha, x, y, gamma) {}
 };
+// Elu: x >= 0 ? x : alpha * (exp(x) - 1) (core/inc/SOFIE/operators/ROperator_Elu.hxx:16-74)
+template <typename T>
+struct ROperator_Elu : ROperator_Activation {
+   ROperator_Elu(float alpha, std::string x, std::string y) : ROperator_Activation(EActivationType::ELU, alpha, x, y) {}
+};
+// Erf: std::erf(x) (core/inc/SOFIE/operators/ROperator_Erf.hxx)
+template <typename T>
+struct ROperator_Erf : ROperator_Activation {
+   ROperator_Erf(std::string x, std::string y) : ROperator_Activation(EActivationType::ERF, 0.f, x, y) {}
+};
 // Identity: a copy that the generator folds away wherever it follows another operator
 template <typename T>
 struct ROperator_Identity : ROperator_Activation {

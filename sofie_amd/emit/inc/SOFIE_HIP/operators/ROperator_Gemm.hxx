@@ -37,6 +37,8 @@ inline const char *ActivationEnumName(EActivationType a)
    case EActivationType::ATANH: return "SOFIE_ACT_ATANH";
    case EActivationType::CLIP: return "SOFIE_ACT_CLIP";
    case EActivationType::SELU: return "SOFIE_ACT_SELU";
+   case EActivationType::ELU: return "SOFIE_ACT_ELU";
+   case EActivationType::ERF: return "SOFIE_ACT_ERF";
    default: return "SOFIE_ACT_NONE";
    }
 }

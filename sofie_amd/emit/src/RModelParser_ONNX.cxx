@@ -512,6 +512,10 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
       } else if (n.op == "Selu") {
          model->AddOperator(std::make_unique<ROperator_Selu<float>>(attrF(n, "alpha", 1.67326319217681884765625f),
                                                                     attrF(n, "gamma", 1.05070102214813232421875f), n.in[0], n.out[0]));
+      } else if (n.op == "Elu") {
+         model->AddOperator(std::make_unique<ROperator_Elu<float>>(attrF(n, "alpha", 1.0f), n.in[0], n.out[0]));
+      } else if (n.op == "Erf") {
+         model->AddOperator(std::make_unique<ROperator_Erf<float>>(n.in[0], n.out[0]));
       } else if (n.op == "Identity") {
          model->AddOperator(std::make_unique<ROperator_Identity<float>>(n.in[0], n.out[0]));
       } else if (n.op == "Clip") {
@@ -545,6 +549,8 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
                                                                     n.in[1], bias, out));
       } else if (n.op == "GlobalAveragePool") {
          model->AddOperator(std::make_unique<ROperator_Pool<float>>(GlobalAveragePool, n.in[0], n.out[0]));
+      } else if (n.op == "Softmax" || n.op == "LogSoftmax") {
+         model->AddOperator(std::make_unique<ROperator_Softmax>(attrI(n, "axis", -1), n.in[0], n.out[0], n.op == "LogSoftmax"));
       } else if (n.op == "MaxPool" || n.op == "AveragePool") {
          // attributes as parsers/src/ParsePool.cxx:37-63 reads them: count_include_pad belongs to AveragePool,
          // storage_order and dilations to MaxPool

@@ -143,6 +143,23 @@ def conv_pool_stack(batch=2):
     return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 3, 10, 10])], outputs=[("Y", np.float32, [batch, 5])], init=init, feeds=[X])
 
 
+def classifier_head(batch=4):
+    """Gemm -> Relu -> Gemm -> Softmax over the classes, and a LogSoftmax of the same logits as a second output."""
+    init = {"W1": util.normal(6301, 20 * 32, 0.2).reshape(20, 32), "b1": util.normal(6302, 32, 0.1),
+            "W2": util.normal(6303, 32 * 7, 0.3).reshape(32, 7), "b2": util.normal(6304, 7, 0.1)}
+    nodes = [ow.node("Gemm", ["X", "W1", "b1"], ["H"]), ow.node("Relu", ["H"], ["R"]), ow.node("Gemm", ["R", "W2", "b2"], ["L"]),
+             ow.node("Softmax", ["L"], ["P"], axis=1), ow.node("LogSoftmax", ["L"], ["Q"], axis=-1)]
+    X = util.normal(6305, batch * 20).reshape(batch, 20)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 20])], outputs=[("P", np.float32, [batch, 7]), ("Q", np.float32, [batch, 7])], init=init,
+                feeds=[X])
+
+
+def softmax_head(batch=4):
+    """Gemm -> Softmax over the classes (one output)."""
+    spec = classifier_head(batch)
+    return dict(spec, nodes=[spec["nodes"][0], spec["nodes"][1], spec["nodes"][2], spec["nodes"][3]], outputs=[spec["outputs"][0]])
+
+
 def qlinear_matmul_relu(M=16, K=64, N=48):
     """QuantizeLinear -> QLinearMatMul (per-column weight scales) -> Relu (int8) -> DequantizeLinear."""
     W = util.int8_sym(7101, K * N).reshape(K, N)
@@ -319,6 +336,7 @@ DYNAMIC_MODELS = {    "Dynamic_ResidualBlock": lambda: with_named_batch(residual
     "Dynamic_int8_CNN": lambda: with_named_batch(int8_cnn(2, 12), "N"),
     "Dynamic_ConvBatchNormRelu": lambda: with_named_batch(conv_batchnorm_relu(2), "bs"),
     "Dynamic_ConvPoolStack": lambda: with_named_batch(conv_pool_stack(2), "N"),
+    "Dynamic_SoftmaxHead": lambda: with_named_batch(softmax_head(4), "N"),
     "Dynamic_int8_CNN_plane_sums": lambda: with_named_batch(int8_cnn(2, 16, (3, 64, 128)), "N"),
 }
 
@@ -571,7 +589,7 @@ def build_all(jobs=8):
         ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)
         dynamic.append((m, p, len(spec["inputs"])))
     folded = reference_constant_folding_cases()
-    multi = [("ElementwiseChains", elementwise_chains, 2), ("ParseRewrites", parse_rewrites, 3)]
+    multi = [("ElementwiseChains", elementwise_chains, 2), ("ParseRewrites", parse_rewrites, 3), ("ClassifierHead", classifier_head, 1)]
     multi += [(m, (lambda spec=spec: spec), len(spec["inputs"])) for m, spec in folded.items()]
     for m, spec in reference_stacked_matmul_cases().items():
         p = os.path.join(OUT, m + ".onnx")
@@ -599,7 +617,7 @@ def build_all(jobs=8):
         f.write(DYNAMIC_HARNESS % dict(model="ApiDynamicFp8Gemm", args="inputs[0]"))
     compile_shared(src, os.path.join(OUT, "libApiDynamicFp8Gemm.so"))
     compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
-    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites"]
+    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead"]
 
 
 if __name__ == "__main__":

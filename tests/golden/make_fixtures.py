@@ -71,13 +71,17 @@ def main():
     add("ConvGroupBatch", arrays_in(os.path.join(REF, "models/onnx/references/ConvGroupBatch.ref.hxx"))["output"],
         [{"kind": "values", "values": arrays_in(os.path.join(REF, "models/onnx/references/ConvGroupBatch_input.ref.hxx"))["data"]}])
     un = os.path.join(REF, "alpaka/TestAlpakaElementwiseUnary.cxx")
-    for model in ("Gelu", "GeluTanh"):
-        add(model, arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx"))["outputs"],
+    for model in ("Gelu", "GeluTanh", "Sqrt", "Reciprocal", "Exp", "Log", "Neg", "Elu", "SeluNonDefaultCoeffs"):
+        add(model, next(iter(arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx")).values())),
             [{"kind": "values", "values": vector_literal(un, model, "input")}])
     pool = os.path.join(REF, "alpaka/TestAlpakaPool.cxx")
     for model in ("MaxPool1d", "MaxPool2d", "AvgPool"):
         add(model, arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx"))["output"],
             [{"kind": "values", "values": vector_literal(pool, model, "input")}])
+    norm = os.path.join(REF, "alpaka/TestAlpakaNormalization.cxx")
+    for model in ("Softmax1d", "Softmax2d", "Softmax3d", "Softmax4d"):
+        add(model, arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx"))["output"],
+            [{"kind": "values", "values": vector_literal(norm, model, "input_vec")}])
     lin = os.path.join(REF, "alpaka/TestAlpakaLinear.cxx")
     add("LinearWithLeakyRelu", arrays_in(os.path.join(REF, "models/onnx/references/LinearWithLeakyRelu.ref.hxx"))["outputs"],
         [{"kind": "values", "values": vector_literal(lin, "LinearWithLeakyRelu", "input")}])

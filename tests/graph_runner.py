@@ -100,6 +100,9 @@ class OracleBackend:
         return self.ob.pool(X, mode, a.get("kernel_shape"), a.get("pads"), a.get("strides"), a.get("dilations"), a.get("auto_pad", "NOTSET"),
                             a.get("ceil_mode", 0), a.get("count_include_pad", 0))
 
+    def softmax(self, X, axis, log):
+        return self.ob.softmax(X, axis, log)
+
     def add(self, A, B):
         return self.ob.add_broadcast(A, B)
 
@@ -190,6 +193,18 @@ class HipBackend:
                             a.get("ceil_mode", 0))
         return hip_pool(self.rt, X, mode, axes, a.get("ceil_mode", 0), a.get("count_include_pad", 0))
 
+    def softmax(self, X, axis, log):
+        import torch
+        u = self.u
+        axis = axis + X.ndim if axis < 0 else axis
+        outer, A, inner = int(np.prod(X.shape[:axis], dtype=np.int64)), X.shape[axis], int(np.prod(X.shape[axis + 1:], dtype=np.int64))
+        dX = u.to_dev(np.ascontiguousarray(X, dtype=np.float32))
+        dY = u.dev_empty(X.shape, np.float32)
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_softmax_f32", u.ptr(dY), u.ptr(dX), outer, A, inner, 1 if log else 0)
+        self.rt.sync()
+        return u.to_host(dY)
+
     def add(self, A, B):
         R, u = self.R, self.u
         ysh = np.broadcast_shapes(A.shape, B.shape)
@@ -260,6 +275,10 @@ def run(g, inputs, be, all_outputs=False):
             y = np.ascontiguousarray(x[0]).reshape(int(np.prod(x[0].shape[:ax], dtype=np.int64)), -1)
         elif op == "Selu":
             y = be.chain(x[0], [(22, a.get("alpha", 1.6732631921768188), a.get("gamma", 1.0507010221481323))])
+        elif op == "Elu":
+            y = be.chain(x[0], [(23, a.get("alpha", 1.0), 0.0)])
+        elif op == "Erf":
+            y = be.unary(x[0], 24, 0.0)
         elif op == "Identity":
             y = np.array(x[0], copy=True)
         elif op == "Clip":
@@ -278,6 +297,8 @@ def run(g, inputs, be, all_outputs=False):
                 y = y[:, :, 0, :]
         elif op == "GlobalAveragePool":
             y = be.gap(x[0])
+        elif op in ("Softmax", "LogSoftmax"):
+            y = be.softmax(x[0], a.get("axis", -1), op == "LogSoftmax")
         elif op in ("MaxPool", "AveragePool"):
             y = be.pool(x[0], "max" if op == "MaxPool" else "average", a)
         elif op == "BatchNormalization":

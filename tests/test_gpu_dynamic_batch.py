@@ -141,6 +141,19 @@ def test_dynamic_int8_cnn_with_plane_sums_for_every_batch(rt):
             assert np.abs(want).max() > 1e-3
 
 
+def test_dynamic_softmax_head(rt):
+    spec = em.softmax_head(4)
+    g = onnx_lite.load(os.path.join(em.OUT, "ClassifierHead.onnx"))     # the same weights with a fixed batch
+    x = np.concatenate([spec["feeds"][0], util.normal(8303, 5 * 20).reshape(5, 20)])
+    want = gr.run(g, [x], gr.OracleBackend(), all_outputs=True)[0]
+    with DynamicSession("Dynamic_SoftmaxHead", 9) as s:
+        for n in (9, 4, 1):
+            print("Dynamic_SoftmaxHead batch", n, flush=True)
+            got = s.infer(n, [x[:n]], want.size)
+            w = want[:n].ravel()
+            assert got.size == w.size and np.all(np.abs(got - w) <= 1e-5 * w + 1e-7)
+
+
 def test_dynamic_conv_batchnorm_relu(rt):
     spec = em.conv_batchnorm_relu(2)
     g = onnx_lite.load(os.path.join(em.OUT, "ConvBatchNormRelu.onnx"))     # the same weights with a fixed batch of 2

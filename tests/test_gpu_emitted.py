@@ -248,6 +248,19 @@ def test_emitted_elementwise_chains(rt):
     assert body.count("detail::Check(") == 5 and body.count("sofie_hip_unary_chain_f32") == 2 and body.count("sofie_hip_unary_f32") == 1
 
 
+def test_emitted_classifier_head_with_softmax_and_logsoftmax(rt):
+    spec = em.classifier_head(4)
+    g = onnx_lite.load(os.path.join(em.OUT, "ClassifierHead.onnx"))
+    P, Q = gr.run(g, spec["feeds"], gr.OracleBackend(), all_outputs=True)
+    print("emitted ClassifierHead", flush=True)
+    got = run_emitted("ClassifierHead", spec["feeds"], P.size + Q.size)
+    gp, gq = got[:P.size].reshape(P.shape), got[P.size:].reshape(Q.shape)
+    assert np.all(np.abs(gp - P) <= 1e-5 * P + 1e-7) and np.allclose(gp.sum(axis=1), 1.0, atol=1e-5)
+    assert np.all(np.abs(gq - Q) <= 1e-5 * np.abs(Q) + 1e-5) and P.std() > 0.01
+    txt = open(os.path.join(em.OUT, "ClassifierHead_GPU_HIP.hxx")).read()
+    assert txt.count("sofie_hip_softmax_f32(") == 2 and "sofie_hip_gemm_chain_f32(fCtx, chain, 2)" in txt
+
+
 def test_emitted_residual_block(rt):
     """Adds of equal-shaped tensors behind a Conv and a Gemm ride in those operators' stores (tests/emitted_models.residual_block)."""
     spec = em.residual_block(2)

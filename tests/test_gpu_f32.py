@@ -351,3 +351,13 @@ def test_selu(rt):
     want = ob.unary_chain(x, [(R.ACT_SELU, alpha, gamma)])
     ref = gamma * (np.maximum(0, x.astype(np.float64)) + np.minimum(0, alpha * (np.exp(x.astype(np.float64)) - 1)))
     assert np.allclose(got, want, rtol=1e-5, atol=1e-6) and np.allclose(want, ref, rtol=1e-5, atol=1e-6)
+
+
+def test_elu_and_erf(rt):
+    x = util.normal(451, 1000 + 3, 2.0)
+    got = run_chain(rt, x, [(R.ACT_ELU, 0.7, 0.0)])
+    want = ob.unary_chain(x, [(R.ACT_ELU, 0.7, 0.0)])
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6) and np.array_equal(got[x >= 0], x[x >= 0]) and (got < 0).any()
+    got = run_chain(rt, x, [(R.ACT_ERF, 0.0, 0.0), (R.ACT_ELU, 1.0, 0.0)])
+    want = ob.unary_chain(x, [(R.ACT_ERF, 0.0, 0.0), (R.ACT_ELU, 1.0, 0.0)])
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6) and want.std() > 0.1

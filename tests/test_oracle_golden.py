@@ -10,11 +10,20 @@ import pytest
 from tests import graph_runner as gr
 
 # references printed with 4 decimals
-FOUR_DECIMALS = ("Gelu", "GeluTanh", "LinearWithLeakyRelu", "AvgPool", "MaxPool1d", "MaxPool2d", "AvgPoolPad", "AvgPoolCountIncludePad")
+FOUR_DECIMALS = ("Gelu", "GeluTanh", "LinearWithLeakyRelu", "AvgPool", "MaxPool1d", "MaxPool2d", "AvgPoolPad", "AvgPoolCountIncludePad",
+                 "Exp", "Log", "Neg", "Elu", "SeluNonDefaultCoeffs", "Softmax3d", "Softmax4d")
+
+
+# Inputs AND outputs printed with 4 decimals, the outputs computed from the unrounded inputs: the rounding of an input
+# reaches the output multiplied by the operator's slope (1/x^2 = 25 at x = 0.2), so these two are held to the
+# tolerance of the reference's own test (DEFAULT_TOLERANCE = 1e-3, tests/alpaka/TestAlpakaCommon.h:10).
+INPUT_ROUNDED = ("Reciprocal", "Sqrt")
 
 
 def golden_tolerance(model, expected):
     """Half a unit of the last printed digit of the reference file, plus fp32 rounding of the result."""
+    if model in INPUT_ROUNDED:
+        return 1e-3
     if model in FOUR_DECIMALS:
         return 0.6e-4
     return 2e-5 + 2e-6 * float(np.abs(expected).max())

@@ -443,3 +443,32 @@ def test_pool_special_cases():
     X6 = np.array([[[1, 2, 3, 4, 5, 6]]], dtype=np.float32)
     np.testing.assert_array_equal(ob.pool(X6, "max", [2], None, [3], ceil_mode=1), np.array([[[2, 5]]], dtype=np.float32))
     np.testing.assert_array_equal(ob.pool(X6, "average", [2], None, [3], ceil_mode=1), np.array([[[1.5, 4.5]]], dtype=np.float32))
+
+
+def test_erf_and_elu_against_library_routines():
+    from scipy import special
+    x = np.linspace(-4, 4, 4001).astype(np.float32)
+    np.testing.assert_allclose(ob.unary(x, 24), special.erf(x.astype(np.float64)), rtol=0, atol=2e-7)
+    assert ob.unary(np.array([0.0, np.inf, -np.inf], np.float32), 24).tolist() == [0.0, 1.0, -1.0]
+    elu = ob.unary_chain(x, [(23, 0.7, 0.0)])
+    want = np.where(x >= 0, x, np.float32(0.7) * np.expm1(x.astype(np.float64)))
+    np.testing.assert_allclose(elu, want, rtol=0, atol=2e-7)
+    assert np.array_equal(elu[x >= 0], x[x >= 0])     # the positive half is the identity, bit for bit
+
+
+def test_softmax_against_the_library_routine_and_its_invariants():
+    from scipy import special
+    rng = np.random.default_rng(31)
+    for shape, axis in [((7,), 0), ((5, 11), -1), ((3, 4, 6), 1), ((2, 3, 4, 2), -2), ((4, 1000), 1), ((2, 5, 3), 0)]:
+        X = (3 * rng.standard_normal(shape)).astype(np.float32)
+        got = ob.softmax(X, axis)
+        np.testing.assert_allclose(got, special.softmax(X.astype(np.float64), axis=axis), rtol=3e-6, atol=1e-9)
+        np.testing.assert_allclose(got.sum(axis=axis), 1.0, rtol=0, atol=2e-6)
+        np.testing.assert_allclose(ob.softmax(X, axis, log=True), special.log_softmax(X.astype(np.float64), axis=axis), rtol=5e-7, atol=2e-6)
+        # a shift that is exact in fp32 leaves x - vmax, and with it every bit of the result, unchanged
+        Xq = (np.round(X * 1024) / 1024).astype(np.float32)
+        assert np.array_equal(ob.softmax(Xq, axis), ob.softmax(Xq + np.float32(8.0), axis))
+    # large inputs do not overflow (the maximum is subtracted first), and a one-element axis gives exactly 1
+    big = np.array([[1000.0, 999.0, -1000.0]], dtype=np.float32)
+    np.testing.assert_allclose(ob.softmax(big), [[1 / (1 + np.exp(-1.0)), np.exp(-1.0) / (1 + np.exp(-1.0)), 0.0]], rtol=2e-7)
+    assert ob.softmax(np.array([[3.5], [-2.0]], np.float32)).tolist() == [[1.0], [1.0]]
