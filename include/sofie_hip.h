@@ -257,6 +257,19 @@ typedef struct sofie_add_desc {
    float *Y;
 } sofie_add_desc;
 int sofie_hip_add_f32(sofie_hip_ctx *ctx, const sofie_add_desc *d);
+/* The other members of the family, same broadcasting (BinaryOperatorTrait<T, Op>::Op, ROperator_BasicBinary.hxx:22-53: a - b,
+ * a * b, a / b, std::pow(a, b)), and the pairwise steps of the n-ary operators (NaryOperatorTraits, ROperator_BasicNary.hxx:19-100:
+ * std::max / std::min keep the FIRST operand unless the second is strictly larger / smaller, Sum adds left to right, Mean
+ * divides that sum by float(count)): an n-ary operator is a left fold of these, ADD_DIV with `param` = count being Mean's last step.
+ * Pow goes through the device's powf (a few ulp from the host library's); every other result is the IEEE one. */
+enum {
+   SOFIE_BINARY_ADD = 0, SOFIE_BINARY_SUB = 1, SOFIE_BINARY_MUL = 2, SOFIE_BINARY_DIV = 3, SOFIE_BINARY_POW = 4,
+   SOFIE_BINARY_MAX = 5, /* a < b ? b : a */
+   SOFIE_BINARY_MIN = 6, /* b < a ? b : a */
+   SOFIE_BINARY_ADD_DIV = 7, /* (a + b) / param */
+   SOFIE_BINARY_LAST = 7
+};
+int sofie_hip_binary_f32(sofie_hip_ctx *ctx, const sofie_add_desc *d, int32_t op, float param);
 
 /* ---- Conv as GEMM --------------------------------------------------------------------------- */
 /* Replaces ROperator_Conv<float>::Generate: weight re-layout + per-image Im2col + Gemm_Call

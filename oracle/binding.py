@@ -87,6 +87,19 @@ def add_broadcast(A, B):
     return Y
 
 
+def binary_broadcast(A, B, op, param=0.0):
+    """op: the SOFIE_BINARY_* code of include/sofie_hip.h."""
+    A, B = _f32(A), _f32(B)
+    yshape = np.broadcast_shapes(A.shape, B.shape)
+    rank = len(yshape)
+    ash = (1,) * (rank - A.ndim) + A.shape
+    bsh = (1,) * (rank - B.ndim) + B.shape
+    Y = np.empty(yshape, dtype=np.float32)
+    arr = lambda s: (C.c_int64 * 6)(*(list(s) + [1] * (6 - len(s))))
+    load().oracle_binary_broadcast(C.c_int(rank), arr(yshape), arr(ash), arr(bsh), _ptr(A), _ptr(B), _ptr(Y), C.c_int(op), C.c_float(param))
+    return Y
+
+
 def conv_out_hw(H, W, kh, kw, pads, strides, dils):
     OH = (H + pads[0] + pads[2] - (dils[0] * (kh - 1) + 1)) // strides[0] + 1
     OW = (W + pads[1] + pads[3] - (dils[1] * (kw - 1) + 1)) // strides[1] + 1

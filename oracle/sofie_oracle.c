@@ -19,6 +19,8 @@
  *                             (exp(log x) = x, sin^2 + cos^2 = 1, sinh(asinh x) = x, ...); Clip bounds; the golden
  *                             outputs Sqrt, Reciprocal, Exp, Log, Neg, Elu, SeluNonDefaultCoeffs, LinearWithSelu of the
  *                             reference's tests; Erf against scipy's erf.
+ *   binary_broadcast          Add, AddBroadcast1..7, Sub, Mul, Div, Pow, Pow_broadcast and the Max / Min / Mean / Sum
+ *                             MultidirectionalBroadcast golden outputs; numpy's broadcasting arithmetic.
  *   global_avg_pool           GlobalAvgPool2d golden output.
  *   softmax                   Softmax1d / 2d / 3d / 4d golden outputs; scipy's softmax and log_softmax in float64; rows sum
  *                             to 1; invariance under a shift of the input.
@@ -243,6 +245,45 @@ ORACLE_API void oracle_add_broadcast(int rank, const int64_t *yshape, const int6
          ib += idx * sb[d];
       }
       Y[i] = A[ia] + B[ib];
+   }
+}
+
+/* The other binary operators with the same loops (BinaryOperatorTrait<T, Op>::Op, ROperator_BasicBinary.hxx:22-53) and the
+ * pairwise steps of the n-ary ones (NaryOperatorTraits, ROperator_BasicNary.hxx:19-100: std::max({..}) / std::min({..}) are
+ * left folds that keep the first of equal elements; Sum adds left to right; Mean divides that sum by T(count)).
+ * op: 0 a+b, 1 a-b, 2 a*b, 3 a/b, 4 powf(a,b), 5 std::max(a,b), 6 std::min(a,b), 7 (a+b)/param. */
+ORACLE_API void oracle_binary_broadcast(int rank, const int64_t *yshape, const int64_t *ashape, const int64_t *bshape, const float *A,
+                                        const float *B, float *Y, int op, float param)
+{
+   int64_t sa[6], sb[6], n = 1, ca = 1, cb = 1;
+   for (int d = rank - 1; d >= 0; --d) {
+      sa[d] = (ashape[d] == 1 && yshape[d] != 1) ? 0 : ca;
+      sb[d] = (bshape[d] == 1 && yshape[d] != 1) ? 0 : cb;
+      ca *= ashape[d];
+      cb *= bshape[d];
+      n *= yshape[d];
+   }
+   for (int64_t i = 0; i < n; ++i) {
+      int64_t rest = i, ia = 0, ib = 0;
+      for (int d = rank - 1; d >= 0; --d) {
+         int64_t idx = rest % yshape[d];
+         rest /= yshape[d];
+         ia += idx * sa[d];
+         ib += idx * sb[d];
+      }
+      const float a = A[ia], b = B[ib];
+      float y;
+      switch (op) {
+      case 1: y = a - b; break;
+      case 2: y = a * b; break;
+      case 3: y = a / b; break;
+      case 4: y = powf(a, b); break;
+      case 5: y = a < b ? b : a; break;
+      case 6: y = b < a ? b : a; break;
+      case 7: y = (a + b) / param; break;
+      default: y = a + b; break;
+      }
+      Y[i] = y;
    }
 }
 

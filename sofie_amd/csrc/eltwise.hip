@@ -120,6 +120,37 @@ struct AddShape {
    long long y[6], sa[6], sb[6]; // output dims, element strides of A and B (0 where broadcast)
 };
 
+__device__ __forceinline__ float binary_op(float a, float b, int op, float param)
+{
+   switch (op) {
+   case SOFIE_BINARY_SUB: return a - b;
+   case SOFIE_BINARY_MUL: return mul_nofma(a, b);
+   case SOFIE_BINARY_DIV: return __fdiv_rn(a, b);
+   case SOFIE_BINARY_POW: return powf(a, b);
+   case SOFIE_BINARY_MAX: return a < b ? b : a;
+   case SOFIE_BINARY_MIN: return b < a ? b : a;
+   case SOFIE_BINARY_ADD_DIV: return __fdiv_rn(a + b, param);
+   default: return a + b;
+   }
+}
+
+__global__ __launch_bounds__(256) void binary_f32_kernel(float *__restrict__ Y, const float *__restrict__ A, const float *__restrict__ B, size_t n,
+                                                          AddShape sh, int op, float param)
+{
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+      size_t rest = i;
+      long long ia = 0, ib = 0;
+      for (int d = sh.rank - 1; d >= 0; --d) {
+         long long idx = (long long)(rest % (size_t)sh.y[d]);
+         rest /= (size_t)sh.y[d];
+         ia += idx * sh.sa[d];
+         ib += idx * sh.sb[d];
+      }
+      Y[i] = binary_op(A[ia], B[ib], op, param);
+   }
+}
+
 __global__ __launch_bounds__(256) void add_f32_kernel(float *__restrict__ Y, const float *__restrict__ A,
                                                        const float *__restrict__ B, size_t n, AddShape sh)
 {
@@ -366,7 +397,13 @@ int sofie_hip_unary_chain_f32(sofie_hip_ctx *ctx, float *dst, const float *src, 
 
 int sofie_hip_add_f32(sofie_hip_ctx *ctx, const sofie_add_desc *d)
 {
+   return sofie_hip_binary_f32(ctx, d, SOFIE_BINARY_ADD, 0.0f);
+}
+
+int sofie_hip_binary_f32(sofie_hip_ctx *ctx, const sofie_add_desc *d, int32_t op, float param)
+{
    SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_add_f32: NULL argument");
+   SOFIE_HIP_REQUIRE(op >= SOFIE_BINARY_ADD && op <= SOFIE_BINARY_LAST, "sofie_hip_binary_f32: unknown operator %d", op);
    SOFIE_HIP_REQUIRE(d->rank >= 0 && d->rank <= 6, "sofie_hip_add_f32: rank %d not in [0,6]", d->rank);
    AddShape sh;
    sh.rank = d->rank;
@@ -387,8 +424,12 @@ int sofie_hip_add_f32(sofie_hip_ctx *ctx, const sofie_add_desc *d)
    if (n == 0)
       return SOFIE_HIP_OK;
    SOFIE_HIP_REQUIRE(d->A && d->B && d->Y, "sofie_hip_add_f32: NULL pointer");
-   hipLaunchKernelGGL(add_f32_kernel, dim3(grid_for(n)), dim3(256), 0, ctx->stream, d->Y, d->A, d->B, n, sh);
-   return launch_status("add_f32_kernel");
+   if (op == SOFIE_BINARY_ADD) {
+      hipLaunchKernelGGL(add_f32_kernel, dim3(grid_for(n)), dim3(256), 0, ctx->stream, d->Y, d->A, d->B, n, sh);
+      return launch_status("add_f32_kernel");
+   }
+   hipLaunchKernelGGL(binary_f32_kernel, dim3(grid_for(n)), dim3(256), 0, ctx->stream, d->Y, d->A, d->B, n, sh, op, param);
+   return launch_status("binary_f32_kernel");
 }
 
 int sofie_hip_batchnorm_f32(sofie_hip_ctx *ctx, float *Y, const float *X, const float *fused_scale, const float *mean,

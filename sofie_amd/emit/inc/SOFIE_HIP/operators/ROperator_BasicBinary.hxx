@@ -1,21 +1,66 @@
-// Broadcast Add (core/inc/SOFIE/operators/ROperator_BasicBinary.hxx, the Add instance): one
-// sofie_hip_add_f32 call with the multidirectional broadcast resolved at generation time.
+// The broadcasting binary operators Add, Sub, Mul, Div, Pow (core/inc/SOFIE/operators/ROperator_BasicBinary.hxx:22-53) and, as
+// left folds of pairwise steps, the n-ary Max, Min, Sum, Mean (ROperator_BasicNary.hxx:19-100): one runtime call per step with
+// the multidirectional broadcast resolved at generation time.
 #ifndef SOFIE_HIP_ROPERATOR_BASICBINARY
 #define SOFIE_HIP_ROPERATOR_BASICBINARY
 
 #include "SOFIE_HIP/operators/ROperator_Gemm.hxx"
 
+#include <cmath>
+
 namespace SOFIE_HIP {
 
-enum EBasicBinaryOperator { Add };
+// Add .. Pow as in the reference; the last three are the pairwise steps of the n-ary operators
+enum EBasicBinaryOperator { Add, Sub, Mul, Div, Pow, PairMax, PairMin, AddThenDivide };
+
+inline const char *BinaryRuntimeCode(EBasicBinaryOperator op)
+{
+   switch (op) {
+   case Sub: return "SOFIE_BINARY_SUB";
+   case Mul: return "SOFIE_BINARY_MUL";
+   case Div: return "SOFIE_BINARY_DIV";
+   case Pow: return "SOFIE_BINARY_POW";
+   case PairMax: return "SOFIE_BINARY_MAX";
+   case PairMin: return "SOFIE_BINARY_MIN";
+   case AddThenDivide: return "SOFIE_BINARY_ADD_DIV";
+   default: return "SOFIE_BINARY_ADD";
+   }
+}
+inline const char *BinaryName(EBasicBinaryOperator op)
+{
+   switch (op) {
+   case Sub: return "Sub";
+   case Mul: return "Mul";
+   case Div: return "Div";
+   case Pow: return "Pow";
+   case PairMax: return "Max";
+   case PairMin: return "Min";
+   case AddThenDivide: return "Mean (last step)";
+   default: return "Add";
+   }
+}
+// the value the generated code computes, for folding two constants (the host's arithmetic is the reference's)
+inline float BinaryValue(EBasicBinaryOperator op, float a, float b, float param)
+{
+   switch (op) {
+   case Sub: return a - b;
+   case Mul: return a * b;
+   case Div: return a / b;
+   case Pow: return std::pow(a, b);
+   case PairMax: return a < b ? b : a;
+   case PairMin: return b < a ? b : a;
+   case AddThenDivide: return (a + b) / param;
+   default: return a + b;
+   }
+}
 
 template <typename T, EBasicBinaryOperator Op>
 class ROperator_BasicBinary final : public ROperator {
-   static_assert(std::is_same<T, float>::value && Op == Add, "only the float Add is on this backend's path");
+   static_assert(std::is_same<T, float>::value, "the float operators are on this backend's path");
 
 public:
-   ROperator_BasicBinary(std::string nameA, std::string nameB, std::string nameY)
-      : fNA(UTILITY::Clean_name(nameA)), fNB(UTILITY::Clean_name(nameB)), fNY(UTILITY::Clean_name(nameY))
+   ROperator_BasicBinary(std::string nameA, std::string nameB, std::string nameY, float param = 0.f)
+      : fNA(UTILITY::Clean_name(nameA)), fNB(UTILITY::Clean_name(nameB)), fNY(UTILITY::Clean_name(nameY)), fParam(param)
    {
       fInputTensorNames = {fNA, fNB};
       fOutputTensorNames = {fNY};
@@ -59,7 +104,7 @@ public:
                ia = ia * fShapeA[d] + (fShapeA[d] == 1 ? 0 : idx[d]);
                ib = ib * fShapeB[d] + (fShapeB[d] == 1 ? 0 : idx[d]);
             }
-            y[i] = a[ia] + b[ib];
+            y[i] = BinaryValue(Op, a[ia], b[ib], fParam);
             for (std::size_t d = r; d-- > 0;) {
                if (++idx[d] < fShapeY[d])
                   break;
@@ -76,7 +121,7 @@ public:
    {
       opName = "op_" + opName;
       if (fIsOutputConstant)
-         return "\n" + SP + "//------ Add " + opName + " -> " + fNY + ": a sum of constants, computed when the code was generated\n";
+         return "\n" + SP + "//------ " + BinaryName(Op) + " " + opName + " -> " + fNY + ": constants only, computed when the code was generated\n";
       std::stringstream out;
       auto list = [](const std::vector<std::size_t> &v, bool batched) {
          std::string s = "{";
@@ -84,11 +129,15 @@ public:
             s += BatchScaled(batched && i == 0, i < v.size() ? v[i] : 1) + (i < 5 ? ", " : "");
          return s + "}";
       };
-      out << "\n" << SP << "//------ Add " << opName << " --> " << ConvertShapeToString(fShapeY) << "\n";
+      out << "\n" << SP << "//------ " << BinaryName(Op) << " " << opName << " --> " << ConvertShapeToString(fShapeY) << "\n";
       out << SP << "{\n";
       out << SP << "   " << "sofie_add_desc d{" << fShapeY.size() << ", " << list(fShapeY, fDynA || fDynB) << ", " << list(fShapeA, fDynA) << ", " << list(fShapeB, fDynB)
           << ", tensor_" << fNA << ", tensor_" << fNB << ", tensor_" << fNY << "};\n";
-      out << SP << "   " << "detail::Check(sofie_hip_add_f32(fCtx, &d), \"" << opName << " Add\");\n";
+      if (Op == Add)
+         out << SP << "   " << "detail::Check(sofie_hip_add_f32(fCtx, &d), \"" << opName << " Add\");\n";
+      else
+         out << SP << "   " << "detail::Check(sofie_hip_binary_f32(fCtx, &d, " << BinaryRuntimeCode(Op) << ", " << FloatLiteral(fParam) << "), \"" << opName << " "
+             << BinaryName(Op) << "\");\n";
       out << SP << "}\n";
       return out.str();
    }
@@ -96,6 +145,7 @@ public:
 private:
    std::string fNA, fNB, fNY;
    std::vector<std::size_t> fShapeA, fShapeB, fShapeY;
+   float fParam = 0.f;
    bool fDynA = false, fDynB = false, fIsOutputConstant = false;
 };
 

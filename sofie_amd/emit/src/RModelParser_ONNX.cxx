@@ -452,7 +452,7 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
       {
          // a node must name the inputs its operator reads below and one output, whatever the file claims
          static const std::map<std::string, size_t> minInputs = {
-            {"Gemm", 2}, {"MatMul", 2}, {"Add", 2}, {"Conv", 2}, {"QuantizeLinear", 2}, {"DequantizeLinear", 2}, {"BatchNormalization", 5},
+            {"Gemm", 2}, {"MatMul", 2}, {"Add", 2}, {"Sub", 2}, {"Mul", 2}, {"Div", 2}, {"Pow", 2}, {"Conv", 2}, {"QuantizeLinear", 2}, {"DequantizeLinear", 2}, {"BatchNormalization", 5},
             {"MatMulInteger", 2}, {"ConvInteger", 2}, {"QLinearConv", 8}, {"QLinearMatMul", 8}};
          auto f = minInputs.find(n.op);
          const size_t need = f == minInputs.end() ? 1 : f->second;
@@ -528,6 +528,36 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          model->AddOperator(std::make_unique<ROperator_Clip<float>>(n.in[0], n.out[0], lo, hi));
       } else if (n.op == "Add") {
          model->AddOperator(std::make_unique<ROperator_BasicBinary<float, Add>>(n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "Sub") {
+         model->AddOperator(std::make_unique<ROperator_BasicBinary<float, Sub>>(n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "Mul") {
+         model->AddOperator(std::make_unique<ROperator_BasicBinary<float, Mul>>(n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "Div") {
+         model->AddOperator(std::make_unique<ROperator_BasicBinary<float, Div>>(n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "Pow") {
+         model->AddOperator(std::make_unique<ROperator_BasicBinary<float, Pow>>(n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "Max" || n.op == "Min" || n.op == "Sum" || n.op == "Mean") {
+         // the reference's ROperator_BasicNary (parsers/src/ParseBasicNary.cxx) as a left fold of pairwise steps: std::max({a, b, c})
+         // is max(max(a, b), c), a + b + c is (a + b) + c, and Mean's last step also divides by the number of operands
+         const size_t count = n.in.size();
+         if (count == 1) {
+            model->AddOperator(std::make_unique<ROperator_Identity<float>>(n.in[0], n.out[0]));
+         } else {
+            std::string acc = n.in[0];
+            for (size_t i = 1; i < count; ++i) {
+               const bool last = i + 1 == count;
+               const std::string out = last ? n.out[0] : n.out[0] + "_fold" + std::to_string(i);
+               if (n.op == "Max")
+                  model->AddOperator(std::make_unique<ROperator_BasicBinary<float, PairMax>>(acc, n.in[i], out));
+               else if (n.op == "Min")
+                  model->AddOperator(std::make_unique<ROperator_BasicBinary<float, PairMin>>(acc, n.in[i], out));
+               else if (n.op == "Mean" && last)
+                  model->AddOperator(std::make_unique<ROperator_BasicBinary<float, AddThenDivide>>(acc, n.in[i], out, static_cast<float>(count)));
+               else
+                  model->AddOperator(std::make_unique<ROperator_BasicBinary<float, Add>>(acc, n.in[i], out));
+               acc = out;
+            }
+         }
       } else if (n.op == "Conv") {
          std::string bias = n.in.size() > 2 ? n.in[2] : "";
          std::string out = n.out[0];

@@ -81,6 +81,7 @@ class PoolDesc(C.Structure):
 
 
 POOL_MAX, POOL_AVERAGE = 0, 1
+BINARY_ADD, BINARY_SUB, BINARY_MUL, BINARY_DIV, BINARY_POW, BINARY_MAX, BINARY_MIN, BINARY_ADD_DIV = range(8)
 
 
 class ConvI8Args(C.Structure):
@@ -125,6 +126,7 @@ SYMBOLS = {
     "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),
     "sofie_hip_global_avg_pool_f32": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32]),
     "sofie_hip_pool_f32": (C.c_int, [_P, _P, _P, _P]),
+    "sofie_hip_binary_f32": (C.c_int, [_P, _P, C.c_int32, C.c_float]),
     "sofie_hip_softmax_f32": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, C.c_int64, C.c_int32]),
     "sofie_hip_gemm_chain_f32": (C.c_int, [_P, _P, C.c_int32]),
     "sofie_hip_plane_sums_to_average": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_float]),

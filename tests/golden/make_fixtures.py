@@ -5,6 +5,8 @@ Reads (never imports or runs) files under /root/reference/tests:
   models/onnx/<Model>.onnx                 binary model files  -> copied to tests/golden/models/
   models/onnx/references/<Model>.ref.hxx   expected outputs    -> numbers extracted into fixtures.json
   alpaka/TestAlpaka*.cxx                   literal input vectors of a few tests -> numbers extracted
+  models/generators/generate_input_models.py   its TEST_INPUTS table (the inputs the expected outputs were made from), read
+                                           as text: the numbers of each f32([...], shape) entry are extracted
 Run in the build container only:  python tests/golden/make_fixtures.py
 """
 import json
@@ -35,6 +37,48 @@ def vector_literal(path, test_name, var):
     m = re.search(r"std::vector<float>\s+%s\s*\(\s*\{(.*?)\}\s*\)" % var, text[start:], re.S)
     body = re.sub(r"(?<=[\d.])f\b", "", m.group(1))
     return [float(x) for x in re.findall(NUM, body)]
+
+
+def _matching(text, start, open_ch, close_ch):
+    """Index just past the bracket that closes the one at text[start]."""
+    depth = 0
+    for i in range(start, len(text)):
+        if text[i] == open_ch:
+            depth += 1
+        elif text[i] == close_ch:
+            depth -= 1
+            if depth == 0:
+                return i + 1
+    raise ValueError("unbalanced brackets")
+
+
+def test_inputs_table(path, model):
+    """The entries of TEST_INPUTS["model"] in the generator script, as [{"kind": "values", "values": [...], "shape": [...]}].
+    Only f32(list, shape) entries are understood; anything else (seeded random inputs, integer tensors) returns None."""
+    text = open(path).read()
+    table = text.index("TEST_INPUTS = {")
+    m = re.search(r'\n    "%s": \[' % re.escape(model), text[table:])
+    if not m:
+        return None
+    lst = table + m.end() - 1
+    body = text[lst:_matching(text, lst, "[", "]")]
+    out, pos = [], 1
+    while True:
+        c = re.search(r"\b(\w+)\(", body[pos:])
+        if not c:
+            break
+        call_open = pos + c.end() - 1
+        call_end = _matching(body, call_open, "(", ")")
+        if c.group(1) != "f32":
+            return None
+        inner = body[call_open + 1:call_end - 1]
+        vals_open = inner.index("[")
+        vals_end = _matching(inner, vals_open, "[", "]")
+        values = [float(x) for x in re.findall(NUM, inner[vals_open:vals_end])]
+        shape = [int(x) for x in re.findall(r"\d+", inner[vals_end:])]
+        out.append({"kind": "values", "values": values, "shape": shape})
+        pos = call_end
+    return out
 
 
 # model -> (expected-array name or None for "the only one", input spec)
@@ -82,6 +126,17 @@ def main():
     for model in ("Softmax1d", "Softmax2d", "Softmax3d", "Softmax4d"):
         add(model, arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx"))["output"],
             [{"kind": "values", "values": vector_literal(norm, model, "input_vec")}])
+    # models whose inputs are entries of the generator script's TEST_INPUTS table
+    gen = os.path.join(REF, "models/generators/generate_input_models.py")
+    # (Sub and MaxPool2d_AsymPad are left out: their .ref.hxx files were made from other inputs than the table holds -- 1.5 - 0.25 is
+    # not the 1 the file expects -- and the matching outputs exist only in files the reference generates at test time.)
+    for model in ("Add", "AddBroadcast2", "AddBroadcast3", "AddBroadcast4", "AddBroadcast5", "AddBroadcast6", "AddBroadcast7", "Mul", "Div", "Pow",
+                  "Pow_broadcast", "MaxMultidirectionalBroadcast", "MinMultidirectionalBroadcast", "MeanMultidirectionalBroadcast",
+                  "SumMultidirectionalBroadcast", "Tanh", "Erf"):
+        inputs = test_inputs_table(gen, model)
+        if inputs is None:
+            raise RuntimeError("no literal inputs for " + model)
+        add(model, next(iter(arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx")).values())), inputs)
     lin = os.path.join(REF, "alpaka/TestAlpakaLinear.cxx")
     add("LinearWithLeakyRelu", arrays_in(os.path.join(REF, "models/onnx/references/LinearWithLeakyRelu.ref.hxx"))["outputs"],
         [{"kind": "values", "values": vector_literal(lin, "LinearWithLeakyRelu", "input")}])

@@ -106,6 +106,9 @@ class OracleBackend:
     def add(self, A, B):
         return self.ob.add_broadcast(A, B)
 
+    def binary(self, A, B, op, param=0.0):
+        return self.ob.binary_broadcast(A, B, op, param)
+
 
 class HipBackend:
     """Every operator goes through the C-ABI on device buffers."""
@@ -206,7 +209,11 @@ class HipBackend:
         return u.to_host(dY)
 
     def add(self, A, B):
+        return self.binary(A, B, None)
+
+    def binary(self, A, B, op, param=0.0):
         R, u = self.R, self.u
+        A, B = np.ascontiguousarray(A, dtype=np.float32), np.ascontiguousarray(B, dtype=np.float32)
         ysh = np.broadcast_shapes(A.shape, B.shape)
         rank = len(ysh)
         d = R.AddDesc()
@@ -222,7 +229,10 @@ class HipBackend:
         d.A, d.B, d.Y = u.ptr(dA), u.ptr(dB), u.ptr(dY)
         import torch
         torch.cuda.synchronize()
-        self.rt.call("sofie_hip_add_f32", C.byref(d))
+        if op is None:
+            self.rt.call("sofie_hip_add_f32", C.byref(d))
+        else:
+            self.rt.call("sofie_hip_binary_f32", C.byref(d), op, C.c_float(param))
         self.rt.sync()
         return u.to_host(dY)
 
@@ -246,6 +256,10 @@ def hip_pool(rt, X, mode, axes, ceil_mode=0, count_include_pad=0):
     rt.sync()
     return u.to_host(dY)
 
+
+# SOFIE_BINARY_* codes of include/sofie_hip.h
+BINARY = {"Sub": 1, "Mul": 2, "Div": 3, "Pow": 4}
+NARY = {"Max": 5, "Min": 6, "Sum": 0, "Mean": 0}
 
 # codes of include/sofie_hip.h for the reference's basic unary operators
 BASIC_UNARY = {"Reciprocal": 7, "Sqrt": 8, "Neg": 9, "Exp": 10, "Log": 11, "Sin": 12, "Cos": 13, "Abs": 14, "Softplus": 15, "Atan": 16,
@@ -306,6 +320,16 @@ def run(g, inputs, be, all_outputs=False):
             y, _ = ob.batchnorm(x[0], x[1], x[2], x[3], x[4], eps=a.get("epsilon", 1e-5))
         elif op == "Add":
             y = be.add(x[0], x[1])
+        elif op in BINARY:
+            y = be.binary(x[0], x[1], BINARY[op])
+        elif op in NARY:
+            # a left fold of pairwise steps; Mean's last step divides by the number of operands
+            y = x[0] if len(x) > 1 else be.binary(x[0], x[0], NARY["Max"])
+            for i in range(1, len(x)):
+                last = i == len(x) - 1
+                y = be.binary(y, x[i], 7 if (op == "Mean" and last) else NARY[op], float(len(x)))
+            if op == "Mean" and len(x) == 1:
+                y = np.array(x[0], copy=True)
         else:
             raise NotImplementedError(op)
         env[n["outputs"][0]] = y

@@ -367,7 +367,7 @@ def test_parse_time_rewrites_of_the_reference(emitted, tmp_path):
     assert "computed when the code was generated" in body and "tensor_Kr" in txt and "static const float host[12]" in txt
     assert "tensor_I, tensor_Wc, tensor_cb, SOFIE_ACT_NONE" in body
     assert "Transpose" not in body and "Cast" not in body
-    assert "-> K2: a product of weights" in body and "-> Ks: a sum of constants" in body and "d.residual" not in body
+    assert "-> K2: a product of weights" in body and "-> Ks: constants only" in body and "d.residual" not in body
     # a Cast that changes the type, and a Transpose that is a graph output, are not rewritten away: they are refused by name
     r = _emit(tmp_path, [ow.node("Cast", ["X"], ["Y"], to=7)], [("X", np.float32, [1, 4])], [("Y", np.int64, [1, 4])], {})
     assert r.returncode != 0 and "Cast" in r.stdout

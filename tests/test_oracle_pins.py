@@ -472,3 +472,27 @@ def test_softmax_against_the_library_routine_and_its_invariants():
     big = np.array([[1000.0, 999.0, -1000.0]], dtype=np.float32)
     np.testing.assert_allclose(ob.softmax(big), [[1 / (1 + np.exp(-1.0)), np.exp(-1.0) / (1 + np.exp(-1.0)), 0.0]], rtol=2e-7)
     assert ob.softmax(np.array([[3.5], [-2.0]], np.float32)).tolist() == [[1.0], [1.0]]
+
+
+def test_binary_operators_against_numpy_and_the_library_semantics():
+    rng = np.random.default_rng(41)
+    A = (2 * rng.standard_normal((3, 1, 5, 4))).astype(np.float32)
+    B = (2 * rng.standard_normal((6, 1, 4))).astype(np.float32)
+    B[np.abs(B) < 0.05] = 0.5
+    assert np.array_equal(ob.binary_broadcast(A, B, 0), A + B)
+    assert np.array_equal(ob.binary_broadcast(A, B, 1), A - B)
+    assert np.array_equal(ob.binary_broadcast(A, B, 2), A * B)
+    assert np.array_equal(ob.binary_broadcast(A, B, 3), A / B)
+    np.testing.assert_allclose(ob.binary_broadcast(np.abs(A) + 0.1, B, 4), np.power((np.abs(A) + 0.1).astype(np.float64), B.astype(np.float64)), rtol=3e-7)
+    assert np.array_equal(ob.binary_broadcast(A, B, 5), np.maximum(A, B)) and np.array_equal(ob.binary_broadcast(A, B, 6), np.minimum(A, B))
+    assert np.array_equal(ob.binary_broadcast(A, B, 7, 3.0), ((A + B) / np.float32(3.0)).astype(np.float32))
+    # std::max / std::min return their FIRST argument unless the second is strictly larger / smaller (C++ [alg.min.max]):
+    # a NaN in first place stays, a NaN in second place never wins, and of two zeros the first one's sign survives
+    nan, one = np.array([np.nan], np.float32), np.array([1.0], np.float32)
+    assert np.isnan(ob.binary_broadcast(nan, one, 5)[0]) and ob.binary_broadcast(one, nan, 5)[0] == 1.0
+    assert np.isnan(ob.binary_broadcast(nan, one, 6)[0]) and ob.binary_broadcast(one, nan, 6)[0] == 1.0
+    mz, pz = np.array([-0.0], np.float32), np.array([0.0], np.float32)
+    assert np.signbit(ob.binary_broadcast(mz, pz, 5)[0]) and not np.signbit(ob.binary_broadcast(pz, mz, 5)[0])
+    # pow special values of the C library: x^0 = 1 for any x, 1^y = 1, a negative base with a non-integer exponent is NaN
+    p = ob.binary_broadcast(np.array([np.nan, 1.0, -8.0, -8.0, 0.0], np.float32), np.array([0.0, np.nan, 1.0 / 3, 2.0, -1.0], np.float32), 4)
+    assert p[0] == 1.0 and p[1] == 1.0 and np.isnan(p[2]) and p[3] == 64.0 and np.isposinf(p[4])
