@@ -65,6 +65,14 @@ int sofie_hip_copy(sofie_hip_ctx *ctx, void *dst_device, const void *src_device,
 int sofie_hip_fill_zero(sofie_hip_ctx *ctx, void *dst_device, size_t bytes); /* resetState, RModel_ALPAKA.cxx:1546-1568 */
 int sofie_hip_sync(sofie_hip_ctx *ctx);                                      /* alpaka::wait(queue) */
 
+/* Data movement of the shape operators.  Transpose (ROperator_Transpose::Generate, core/inc/SOFIE/operators/ROperator_Transpose.hxx):
+ * Y[i_perm[0], ..., i_perm[r-1]] = X[i_0, ..., i_{r-1}], i.e. output axis k is input axis perm[k]; `shape` is the INPUT shape, rank <= 6,
+ * 4-byte elements.  copy_rows moves `rows` pieces of `row_bytes` bytes from a pitched source to a pitched destination (Concat
+ * along an inner axis, ROperator_Concat.hxx: each input contributes one piece per outer index); pitches and row_bytes multiples of 4. */
+int sofie_hip_transpose_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t rank, const int64_t *shape, const int32_t *perm);
+int sofie_hip_copy_rows(sofie_hip_ctx *ctx, void *dst_device, size_t dst_pitch_bytes, const void *src_device, size_t src_pitch_bytes, size_t rows,
+                        size_t row_bytes);
+
 /* ---- activation / epilogue vocabulary ------------------------------------------------------ */
 /* Scalar formulas follow the reference's CPU emitters:
  *   RELU      x > 0 ? x : 0            core/src/utils/SOFIE_common_helpers.cxx:325-332

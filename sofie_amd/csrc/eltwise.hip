@@ -120,6 +120,36 @@ struct AddShape {
    long long y[6], sa[6], sb[6]; // output dims, element strides of A and B (0 where broadcast)
 };
 
+struct TransposeShape {
+   int rank;
+   long long y[6], sx[6]; // output dims and, per OUTPUT axis, the element stride of the input axis it reads
+};
+
+// One output element per thread (grid-stride): writes are coalesced, reads are strided by the permutation.
+__global__ __launch_bounds__(256) void transpose_f32_kernel(float *__restrict__ Y, const float *__restrict__ X, size_t n, TransposeShape sh)
+{
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+      size_t rest = i;
+      long long ix = 0;
+      for (int d = sh.rank - 1; d >= 0; --d) {
+         ix += (long long)(rest % (size_t)sh.y[d]) * sh.sx[d];
+         rest /= (size_t)sh.y[d];
+      }
+      Y[i] = X[ix];
+   }
+}
+
+__global__ __launch_bounds__(256) void copy_rows_kernel(uint32_t *__restrict__ dst, size_t dst_pitch, const uint32_t *__restrict__ src, size_t src_pitch,
+                                                         size_t rows, size_t row_words)
+{
+   const size_t n = rows * row_words, stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+      const size_t r = i / row_words, c = i - r * row_words;
+      dst[r * dst_pitch + c] = src[r * src_pitch + c];
+   }
+}
+
 __device__ __forceinline__ float binary_op(float a, float b, int op, float param)
 {
    switch (op) {
@@ -498,6 +528,48 @@ int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y, const int8_t *X, 
    const int NC = N * C;
    hipLaunchKernelGGL((gap_kernel<int8_t, int>), dim3((NC + 3) / 4), dim3(256), 0, ctx->stream, Y, X, NC, HW, scale);
    return launch_status("gap_kernel");
+}
+
+int sofie_hip_transpose_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t rank, const int64_t *shape, const int32_t *perm)
+{
+   SOFIE_HIP_REQUIRE(ctx && shape && perm, "sofie_hip_transpose_f32: NULL argument");
+   SOFIE_HIP_REQUIRE(rank >= 1 && rank <= 6, "sofie_hip_transpose_f32: rank %d not in [1,6]", rank);
+   long long in_stride[6];
+   size_t n = 1;
+   unsigned seen = 0;
+   for (int d = rank - 1; d >= 0; --d) {
+      SOFIE_HIP_REQUIRE(shape[d] >= 0 && shape[d] < (1LL << 40), "sofie_hip_transpose_f32: bad dimension");
+      in_stride[d] = (long long)n;
+      n *= (size_t)shape[d];
+      SOFIE_HIP_REQUIRE(n < (1ULL << 40), "sofie_hip_transpose_f32: tensor too large");
+   }
+   TransposeShape sh;
+   sh.rank = rank;
+   for (int k = 0; k < rank; ++k) {
+      SOFIE_HIP_REQUIRE(perm[k] >= 0 && perm[k] < rank && !(seen & (1u << perm[k])), "sofie_hip_transpose_f32: perm is not a permutation of 0..%d", rank - 1);
+      seen |= 1u << perm[k];
+      sh.y[k] = shape[perm[k]];
+      sh.sx[k] = in_stride[perm[k]];
+   }
+   if (n == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(Y && X, "sofie_hip_transpose_f32: NULL pointer");
+   hipLaunchKernelGGL(transpose_f32_kernel, dim3(grid_for(n)), dim3(256), 0, ctx->stream, Y, X, n, sh);
+   return launch_status("transpose_f32_kernel");
+}
+
+int sofie_hip_copy_rows(sofie_hip_ctx *ctx, void *dst, size_t dst_pitch_bytes, const void *src, size_t src_pitch_bytes, size_t rows, size_t row_bytes)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_copy_rows: ctx is NULL");
+   SOFIE_HIP_REQUIRE(row_bytes % 4 == 0 && dst_pitch_bytes % 4 == 0 && src_pitch_bytes % 4 == 0, "sofie_hip_copy_rows: sizes must be multiples of 4 bytes");
+   SOFIE_HIP_REQUIRE(dst_pitch_bytes >= row_bytes && src_pitch_bytes >= row_bytes, "sofie_hip_copy_rows: a pitch is smaller than the row");
+   SOFIE_HIP_REQUIRE(rows < (1ULL << 40) && row_bytes < (1ULL << 40) && (double)rows * (double)row_bytes < 1.0e13, "sofie_hip_copy_rows: too large");
+   if (rows == 0 || row_bytes == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(dst && src && (((uintptr_t)dst | (uintptr_t)src) & 3) == 0, "sofie_hip_copy_rows: NULL or misaligned pointer");
+   hipLaunchKernelGGL(copy_rows_kernel, dim3(grid_for(rows * (row_bytes / 4))), dim3(256), 0, ctx->stream, (uint32_t *)dst, dst_pitch_bytes / 4,
+                      (const uint32_t *)src, src_pitch_bytes / 4, rows, row_bytes / 4);
+   return launch_status("copy_rows_kernel");
 }
 
 int sofie_hip_softmax_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int64_t outer, int32_t axis_len, int64_t inner, int32_t log_softmax)

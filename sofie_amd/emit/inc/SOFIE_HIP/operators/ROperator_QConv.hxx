@@ -10,7 +10,6 @@
 //                When that map comes from a QLinearConv which nothing else reads, and the runtime can do it (planes of a
 //                multiple of 256 pixels, no column matrix), the convolution adds the planes up in its own store: the map
 //                is neither written nor read back, and a small kernel turns the sums into the average.
-//   Flatten      a device copy (the tensors here are a few KB).
 #ifndef SOFIE_HIP_ROPERATOR_QCONV
 #define SOFIE_HIP_ROPERATOR_QCONV
 
@@ -285,51 +284,6 @@ private:
    std::vector<std::size_t> fShapeX;
    float fScale = 1.0f;
    int fLayout = kLayoutNCHW;
-   bool fDynamic = false;
-};
-
-// Flatten(axis): [d0..dn) -> [prod(d0..axis), prod(axis..n)], same bytes; emitted as a copy
-class ROperator_Flatten final : public ROperator {
-public:
-   ROperator_Flatten(int axis, std::string nameX, std::string nameY) : fAxis(axis), fNX(UTILITY::Clean_name(nameX)), fNY(UTILITY::Clean_name(nameY))
-   {
-      fInputTensorNames = {fNX};
-      fOutputTensorNames = {fNY};
-   }
-   void Initialize(RModel &model) override
-   {
-      if (!model.CheckIfTensorAlreadyExist(fNX))
-         throw std::runtime_error("SOFIE Reshape Op Input Tensor " + fNX + "  is not found in model");
-      if (model.GetTensorLayout(fNX) != kLayoutNCHW)
-         throw std::runtime_error("SOFIE Flatten Op: input tensor " + fNX + " is stored channels-last");
-      const auto shape = model.GetTensorShape(fNX);
-      int axis = fAxis < 0 ? fAxis + (int)shape.size() : fAxis;
-      if (axis < 0 || axis > (int)shape.size())
-         throw std::runtime_error("SOFIE Flatten Op: axis out of range for " + fNX);
-      std::size_t a = 1, b = 1;
-      for (int i = 0; i < (int)shape.size(); ++i)
-         (i < axis ? a : b) *= shape[i];
-      fType = model.GetTensorType(fNX);
-      fBytes = a * b * GetTypeSize(fType);
-      fDynamic = model.IsDynamicTensor(fNX);
-      if (fDynamic && axis < 1)
-         throw std::runtime_error("SOFIE Flatten Op: axis 0 would fold the run-time batch of " + fNX + " into the second dimension");
-      model.AddIntermediateTensor(fNY, fType, {a, b}, fDynamic);
-   }
-   std::string Generate_GPU_HIP(std::string opName) override
-   {
-      opName = "op_" + opName;
-      std::stringstream out;
-      out << "\n" << SP << "//----  Flatten " << opName << "\n";
-      out << SP << "detail::Check(sofie_hip_copy(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << BatchScaled(fDynamic, fBytes) << "), \"" << opName << " Flatten\");\n";
-      return out.str();
-   }
-
-private:
-   int fAxis;
-   std::string fNX, fNY;
-   ETensorType fType = ETensorType::FLOAT;
-   std::size_t fBytes = 0;
    bool fDynamic = false;
 };
 

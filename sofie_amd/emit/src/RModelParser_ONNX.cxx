@@ -651,7 +651,25 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          op->SetRequantize(mname, false);
          model->AddOperator(std::move(op));
       } else if (n.op == "Flatten") {
-         model->AddOperator(std::make_unique<ROperator_Flatten>((int)attrI(n, "axis", 1), n.in[0], n.out[0]));
+         model->AddOperator(std::make_unique<ROperator_Reshape>(Flatten, (int)attrI(n, "axis", 1), n.in[0], "", n.out[0]));
+      } else if (n.op == "Reshape") {
+         if (n.in.size() < 2)
+            throw std::runtime_error("SOFIE ONNX parser: Reshape " + n.name + " needs the shape as its second input");
+         model->AddOperator(std::make_unique<ROperator_Reshape>(Reshape, (int)attrI(n, "allowzero", 0), n.in[0], n.in[1], n.out[0]));
+      } else if (n.op == "Squeeze" || n.op == "Unsqueeze") {
+         // the axes are an input from opset 13 on, an attribute before (parsers/src/ParseReshape.cxx:19-51)
+         const ReshapeOpMode mode = n.op == "Squeeze" ? Squeeze : Unsqueeze;
+         if (n.in.size() > 1 && !n.in[1].empty()) {
+            model->AddOperator(std::make_unique<ROperator_Reshape>(mode, 0, n.in[0], n.in[1], n.out[0]));
+         } else {
+            auto f = n.attrs.find("axes");
+            model->AddOperator(std::make_unique<ROperator_Reshape>(mode, f == n.attrs.end() ? std::vector<int64_t>{} : f->second.ints, n.in[0], n.out[0]));
+         }
+      } else if (n.op == "Transpose") {
+         auto f = n.attrs.find("perm");
+         model->AddOperator(std::make_unique<ROperator_Transpose<float>>(f == n.attrs.end() ? std::vector<int64_t>{} : f->second.ints, n.in[0], n.out[0]));
+      } else if (n.op == "Concat") {
+         model->AddOperator(std::make_unique<ROperator_Concat>(n.in, (int)attrI(n, "axis", 0), 0, n.out[0]));
       } else if (n.op == "MatMulInteger") {
          model->AddOperator(MakeMatMulInteger(n.in[0], n.in[1], n.out[0]));
       } else {

@@ -154,6 +154,21 @@ def classifier_head(batch=4):
                 feeds=[X])
 
 
+def shape_plumbing(batch=3):
+    """Reshape (with 0 and -1), Transpose, Squeeze / Unsqueeze (axes as input and as attribute), Concat and Flatten around a Gemm:
+    X [b, 2, 3, 4] -> Transpose(0, 2, 1, 3) -> Reshape [0, 3, -1] -> Concat with Z [b, 3, 2] along the last axis -> Unsqueeze(1) -> Squeeze(1)
+    -> Flatten -> Gemm."""
+    init = {"shape": np.array([0, 3, -1], np.int64), "ax1": np.array([1], np.int64), "W": util.normal(6401, 30 * 6, 0.2).reshape(30, 6),
+            "b": util.normal(6402, 6, 0.1)}
+    nodes = [ow.node("Transpose", ["X"], ["T"], perm=[0, 2, 1, 3]), ow.node("Reshape", ["T", "shape"], ["R"]),
+             ow.node("Concat", ["R", "Z"], ["C"], axis=-1), ow.node("Unsqueeze", ["C", "ax1"], ["U"]), ow.node("Squeeze", ["U"], ["S"], axes=[1]),
+             ow.node("Flatten", ["S"], ["F"], axis=1), ow.node("Gemm", ["F", "W", "b"], ["Y"])]
+    X = util.normal(6403, batch * 24).reshape(batch, 2, 3, 4)
+    Z = util.normal(6404, batch * 6).reshape(batch, 3, 2)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 2, 3, 4]), ("Z", np.float32, [batch, 3, 2])], outputs=[("Y", np.float32, [batch, 6])],
+                init=init, feeds=[X, Z])
+
+
 def softmax_head(batch=4):
     """Gemm -> Softmax over the classes (one output)."""
     spec = classifier_head(batch)
@@ -337,6 +352,7 @@ DYNAMIC_MODELS = {    "Dynamic_ResidualBlock": lambda: with_named_batch(residual
     "Dynamic_ConvBatchNormRelu": lambda: with_named_batch(conv_batchnorm_relu(2), "bs"),
     "Dynamic_ConvPoolStack": lambda: with_named_batch(conv_pool_stack(2), "N"),
     "Dynamic_SoftmaxHead": lambda: with_named_batch(softmax_head(4), "N"),
+    "Dynamic_ShapePlumbing": lambda: with_named_batch(shape_plumbing(3), "N"),
     "Dynamic_int8_CNN_plane_sums": lambda: with_named_batch(int8_cnn(2, 16, (3, 64, 128)), "N"),
 }
 
@@ -346,6 +362,7 @@ CONFIG_MODELS = {
     "ConvIntegerDequantize": lambda: conv_integer_dequantize(),
     "ConvBatchNormRelu": lambda: conv_batchnorm_relu(2),
     "ConvPoolStack": lambda: conv_pool_stack(2),
+    "ShapePlumbing": lambda: shape_plumbing(3),
     "Config5_int8_CNN_small": lambda: int8_cnn(2, 12),
     "Int8_CNN_plane_sums": lambda: int8_cnn(2, 16, (3, 64, 128)),   # planes of 256 pixels: the last convolution sums them itself
     "Config1_fp32_MLP": lambda: fp32_mlp(64),

@@ -103,6 +103,13 @@ class OracleBackend:
     def softmax(self, X, axis, log):
         return self.ob.softmax(X, axis, log)
 
+    # pure data movement: numpy is the definition
+    def transpose(self, X, perm):
+        return np.ascontiguousarray(np.transpose(X, perm))
+
+    def concat(self, xs, axis):
+        return np.ascontiguousarray(np.concatenate(xs, axis=axis))
+
     def add(self, A, B):
         return self.ob.add_broadcast(A, B)
 
@@ -196,6 +203,41 @@ class HipBackend:
                             a.get("ceil_mode", 0))
         return hip_pool(self.rt, X, mode, axes, a.get("ceil_mode", 0), a.get("count_include_pad", 0))
 
+    def transpose(self, X, perm):
+        import torch
+        u = self.u
+        X = np.ascontiguousarray(X, dtype=np.float32)
+        shape = (C.c_int64 * 6)(*(list(X.shape) + [1] * (6 - X.ndim)))
+        p = (C.c_int32 * 6)(*(list(perm) + list(range(X.ndim, 6))))
+        dX = u.to_dev(X)
+        dY = u.dev_empty(tuple(X.shape[i] for i in perm), np.float32)
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_transpose_f32", u.ptr(dY), u.ptr(dX), X.ndim, shape, p)
+        self.rt.sync()
+        return u.to_host(dY)
+
+    def concat(self, xs, axis):
+        import torch
+        u = self.u
+        xs = [np.ascontiguousarray(x, dtype=np.float32) for x in xs]
+        axis = axis + xs[0].ndim if axis < 0 else axis
+        outer = int(np.prod(xs[0].shape[:axis], dtype=np.int64))
+        inner = int(np.prod(xs[0].shape[axis + 1:], dtype=np.int64))
+        total = sum(x.shape[axis] for x in xs)
+        ysh = xs[0].shape[:axis] + (total,) + xs[0].shape[axis + 1:]
+        dY = u.dev_empty(ysh, np.float32)
+        devs = [u.to_dev(x) for x in xs]
+        torch.cuda.synchronize()
+        off = 0
+        for x, dx in zip(xs, devs):
+            row = x.shape[axis] * inner * 4
+            if row:
+                self.rt.call("sofie_hip_copy_rows", C.c_void_p(u.ptr(dY).value + off), C.c_size_t(total * inner * 4), u.ptr(dx), C.c_size_t(row), C.c_size_t(outer),
+                             C.c_size_t(row))
+            off += row
+        self.rt.sync()
+        return u.to_host(dY)
+
     def softmax(self, X, axis, log):
         import torch
         u = self.u
@@ -287,6 +329,21 @@ def run(g, inputs, be, all_outputs=False):
         elif op == "Flatten":
             ax = a.get("axis", 1)
             y = np.ascontiguousarray(x[0]).reshape(int(np.prod(x[0].shape[:ax], dtype=np.int64)), -1)
+        elif op == "Reshape":
+            shape = [int(v) for v in np.asarray(x[1]).ravel()]
+            shape = [x[0].shape[i] if (v == 0 and not a.get("allowzero", 0)) else v for i, v in enumerate(shape)]
+            y = np.ascontiguousarray(x[0]).reshape(shape)
+        elif op in ("Squeeze", "Unsqueeze"):
+            axes = [int(v) for v in np.asarray(x[1]).ravel()] if len(x) > 1 and x[1] is not None else list(a.get("axes", []))
+            if op == "Squeeze":
+                y = np.squeeze(x[0], axis=tuple(axes) if axes else None)
+            else:
+                y = np.expand_dims(x[0], axis=tuple(axes))
+            y = np.ascontiguousarray(y)
+        elif op == "Transpose":
+            y = be.transpose(x[0], a.get("perm", list(range(x[0].ndim))[::-1]))
+        elif op == "Concat":
+            y = be.concat(x, a.get("axis", 0))
         elif op == "Selu":
             y = be.chain(x[0], [(22, a.get("alpha", 1.6732631921768188), a.get("gamma", 1.0507010221481323))])
         elif op == "Elu":

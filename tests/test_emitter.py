@@ -368,12 +368,14 @@ def test_parse_time_rewrites_of_the_reference(emitted, tmp_path):
     assert "tensor_I, tensor_Wc, tensor_cb, SOFIE_ACT_NONE" in body
     assert "Transpose" not in body and "Cast" not in body
     assert "-> K2: a product of weights" in body and "-> Ks: constants only" in body and "d.residual" not in body
-    # a Cast that changes the type, and a Transpose that is a graph output, are not rewritten away: they are refused by name
+    # a Cast that changes the type is not rewritten away: it is refused by name
     r = _emit(tmp_path, [ow.node("Cast", ["X"], ["Y"], to=7)], [("X", np.float32, [1, 4])], [("Y", np.int64, [1, 4])], {})
     assert r.returncode != 0 and "Cast" in r.stdout
+    # a Transpose that is also a graph output stays an operator of its own (a gather kernel), and the MatMul reads its result
     r = _emit(tmp_path, [ow.node("Transpose", ["X"], ["T"]), ow.node("MatMul", ["T", "W"], ["Y"])], [("X", np.float32, [3, 2])],
-              [("T", np.float32, [2, 3]), ("Y", np.float32, [2, 4])], {"W": np.ones((3, 4), np.float32)})
-    assert r.returncode != 0 and "Transpose" in r.stdout
+              [("T", np.float32, [2, 3]), ("Y", np.float32, [2, 4])], {"W": np.ones((3, 4), np.float32)}, name="kept")
+    kept = open(os.path.join(str(tmp_path), "kept_GPU_HIP.hxx")).read()
+    assert r.returncode == 0 and "sofie_hip_transpose_f32(" in kept and "d.A = tensor_T;" in kept and "d.transA = 0;" in kept
 
 
 def test_asymmetric_zero_point_is_refused(tmp_path):

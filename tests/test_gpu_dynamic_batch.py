@@ -141,6 +141,20 @@ def test_dynamic_int8_cnn_with_plane_sums_for_every_batch(rt):
             assert np.abs(want).max() > 1e-3
 
 
+def test_dynamic_shape_plumbing(rt):
+    spec = em.shape_plumbing(3)
+    x = np.concatenate([spec["feeds"][0], util.normal(8304, 2 * 24).reshape(2, 2, 3, 4)])
+    z = np.concatenate([spec["feeds"][1], util.normal(8305, 2 * 6).reshape(2, 3, 2)])
+    with DynamicSession("Dynamic_ShapePlumbing", 5) as s:
+        for n in (5, 3, 1):
+            # the static model's Reshape keeps the batch through its leading 0, so the same graph evaluates any batch on the CPU
+            g = onnx_lite.load(os.path.join(em.OUT, "ShapePlumbing.onnx"))
+            want = gr.run(g, [x[:n], z[:n]], gr.OracleBackend()).ravel()
+            print("Dynamic_ShapePlumbing batch", n, flush=True)
+            got = s.infer(n, [x[:n], z[:n]], want.size)
+            assert got.size == want.size == n * 6 and np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+
+
 def test_dynamic_softmax_head(rt):
     spec = em.softmax_head(4)
     g = onnx_lite.load(os.path.join(em.OUT, "ClassifierHead.onnx"))     # the same weights with a fixed batch

@@ -261,6 +261,15 @@ def test_emitted_classifier_head_with_softmax_and_logsoftmax(rt):
     assert txt.count("sofie_hip_softmax_f32(") == 2 and "sofie_hip_gemm_chain_f32(fCtx, chain, 2)" in txt
 
 
+def test_emitted_shape_plumbing(rt):
+    spec = em.shape_plumbing(3)
+    g = onnx_lite.load(os.path.join(em.OUT, "ShapePlumbing.onnx"))
+    want = gr.run(g, spec["feeds"], gr.OracleBackend()).ravel()
+    print("emitted ShapePlumbing", flush=True)
+    got = run_emitted("ShapePlumbing", spec["feeds"], want.size)
+    assert want.size == 18 and np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max())) and want.std() > 0.05
+
+
 def test_emitted_residual_block(rt):
     """Adds of equal-shaped tensors behind a Conv and a Gemm ride in those operators' stores (tests/emitted_models.residual_block)."""
     spec = em.residual_block(2)
