@@ -377,6 +377,13 @@ int sofie_hip_plane_sums_to_average(sofie_hip_ctx *ctx, float *Y /* [NC] */, con
  * the rounding of that sum, which for the loop grows with the axis length (1e-7 relative at 10 classes, 6e-5 at 70000). */
 int sofie_hip_softmax_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int64_t outer, int32_t axis_len, int64_t inner, int32_t log_softmax);
 
+/* LayerNormalization over the trailing dimensions of a tensor seen as [rows, L] (ROperator_LayerNormalization::Generate,
+ * core/inc/SOFIE/operators/ROperator_LayerNormalization.hxx:247-312): mean = sum(x) / L, invStdDev = 1 / sqrt(sum((x - mean)^2) / L + epsilon),
+ * Y = scale[j] * invStdDev * (x - mean) + bias[j].  scale and bias hold L elements (bias may be NULL); mean_out / inv_std_out, when not
+ * NULL, receive the per-row statistics (the operator's optional outputs).  The two sums are trees here, loops in the reference. */
+int sofie_hip_layernorm_f32(sofie_hip_ctx *ctx, float *Y, const float *X, const float *scale, const float *bias, int64_t rows, int32_t L,
+                            float epsilon, float *mean_out, float *inv_std_out);
+
 /* BatchNormalization at inference, for models whose normalisation was not folded into the weights
  * (core/inc/SOFIE/operators/ROperator_BatchNormalization.hxx:139-158): X is [N, C, spatial...],
  *   Y = (X - mean[c]) * fused_scale[c] + bias[c],   fused_scale[c] = scale[c] / sqrt(var[c] + eps) formed by the generator,

@@ -196,6 +196,18 @@ def softmax(X, axis=-1, log=False):
     return Y
 
 
+def layernorm(X, scale, bias=None, axis=-1, eps=1e-5, stats=False):
+    X, scale = _f32(X), _f32(scale)
+    axis = axis + X.ndim if axis < 0 else axis
+    rows, L = int(np.prod(X.shape[:axis], dtype=np.int64)), int(np.prod(X.shape[axis:], dtype=np.int64))
+    b = None if bias is None else _f32(bias)
+    assert scale.size == L and (b is None or b.size == L)
+    Y = np.empty_like(X)
+    mean, inv = np.empty(rows, np.float32), np.empty(rows, np.float32)
+    load().oracle_layernorm(_ptr(Y), _ptr(X), _ptr(scale), _ptr(b), C.c_long(rows), C.c_int(L), C.c_float(eps), _ptr(mean), _ptr(inv))
+    return (Y, mean, inv) if stats else Y
+
+
 def batchnorm(X, scale, bias, mean, var, eps=1e-5, relu=0):
     X = _f32(X)
     Cc = X.shape[1]

@@ -21,6 +21,8 @@
  *                             reference's tests; Erf against scipy's erf.
  *   binary_broadcast          Add, AddBroadcast1..7, Sub, Mul, Div, Pow, Pow_broadcast and the Max / Min / Mean / Sum
  *                             MultidirectionalBroadcast golden outputs; numpy's broadcasting arithmetic.
+ *   layernorm                 LayerNormalization2d / 4d golden outputs; the float64 definition; rows of zero mean and unit
+ *                             variance before scale and bias.
  *   global_avg_pool           GlobalAvgPool2d golden output.
  *   softmax                   Softmax1d / 2d / 3d / 4d golden outputs; scipy's softmax and log_softmax in float64; rows sum
  *                             to 1; invariance under a shift of the input.
@@ -473,6 +475,37 @@ ORACLE_API void oracle_softmax(float *Y, const float *X, long outer, int A, long
             for (int i = 0; i < A; ++i)
                y[(size_t)i * inner] /= sum;
          }
+      }
+   }
+}
+
+/* LayerNormalization over [rows, L], the loops of ROperator_LayerNormalization::Generate
+ * (core/inc/SOFIE/operators/ROperator_LayerNormalization.hxx:247-312): mean += x in order, mean /= L; sum += tmp*tmp with
+ * tmp = x - mean; invStdDev = 1 / std::sqrt(sum / L + epsilon); Y = scale * invStdDev * (x - mean) [+ bias]. */
+ORACLE_API void oracle_layernorm(float *Y, const float *X, const float *scale, const float *bias, long rows, int L, float epsilon, float *mean_out,
+                                 float *inv_std_out)
+{
+   for (long r = 0; r < rows; ++r) {
+      const float *x = X + (size_t)r * L;
+      float mean = 0.0f;
+      for (int j = 0; j < L; ++j)
+         mean += x[j];
+      mean /= (float)L;
+      float sum = 0.0f;
+      for (int j = 0; j < L; ++j) {
+         float tmp = x[j] - mean;
+         sum += tmp * tmp;
+      }
+      float invStdDev = 1 / sqrtf(sum / (float)L + epsilon);
+      if (mean_out)
+         mean_out[r] = mean;
+      if (inv_std_out)
+         inv_std_out[r] = invStdDev;
+      for (int j = 0; j < L; ++j) {
+         float v = scale[j] * invStdDev * (x[j] - mean);
+         if (bias)
+            v += bias[j];
+         Y[(size_t)r * L + j] = v;
       }
    }
 }

@@ -275,6 +275,47 @@ __global__ __launch_bounds__(256) void softmax_f32_kernel(float *__restrict__ Y,
    }
 }
 
+// LayerNormalization: one wave per row of L elements, lanes stride over the row; mean, then the centred sum of squares, then the output.
+__global__ __launch_bounds__(256) void layernorm_f32_kernel(float *__restrict__ Y, const float *__restrict__ X, const float *__restrict__ scale,
+                                                            const float *__restrict__ bias, long long rows, int L, float epsilon,
+                                                            float *__restrict__ mean_out, float *__restrict__ inv_std_out)
+{
+   const int lane = threadIdx.x & 63;
+   const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6), nwaves = (long long)gridDim.x * 4;
+   for (long long row = wave; row < rows; row += nwaves) {
+      const float *x = X + row * L;
+      float *y = Y + row * L;
+      float mean = 0.0f;
+      for (int j = lane; j < L; j += 64)
+         mean += x[j];
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1)
+         mean += __shfl_xor(mean, off, 64);
+      mean = __fdiv_rn(mean, (float)L);
+      float sum = 0.0f;
+      for (int j = lane; j < L; j += 64) {
+         const float tmp = x[j] - mean;
+         sum += mul_nofma(tmp, tmp);
+      }
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1)
+         sum += __shfl_xor(sum, off, 64);
+      const float inv_std = __fdiv_rn(1.0f, __fsqrt_rn(__fdiv_rn(sum, (float)L) + epsilon));
+      if (lane == 0) {
+         if (mean_out)
+            mean_out[row] = mean;
+         if (inv_std_out)
+            inv_std_out[row] = inv_std;
+      }
+      for (int j = lane; j < L; j += 64) {
+         float v = mul_nofma(mul_nofma(scale[j], inv_std), x[j] - mean);
+         if (bias)
+            v += bias[j];
+         y[j] = v;
+      }
+   }
+}
+
 // The last step of an average whose integer plane sums already exist (a convolution added them up in its store).
 __global__ __launch_bounds__(256) void plane_sums_to_average_kernel(float *__restrict__ Y, const int32_t *__restrict__ sums, int NC, int HW,
                                                                     float scale)
@@ -585,6 +626,21 @@ int sofie_hip_softmax_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int64_t 
    hipLaunchKernelGGL(softmax_f32_kernel, dim3((unsigned)(blocks < 256 * 64 ? blocks : 256 * 64)), dim3(256), 0, ctx->stream, Y, X, lines, axis_len,
                       (long long)inner, log_softmax);
    return launch_status("softmax_f32_kernel");
+}
+
+int sofie_hip_layernorm_f32(sofie_hip_ctx *ctx, float *Y, const float *X, const float *scale, const float *bias, int64_t rows, int32_t L, float epsilon,
+                            float *mean_out, float *inv_std_out)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_layernorm_f32: ctx is NULL");
+   SOFIE_HIP_REQUIRE(rows >= 0 && L > 0 && rows < (1LL << 40) && (double)rows * L < 1.0e12, "sofie_hip_layernorm_f32: bad shape");
+   SOFIE_HIP_REQUIRE(epsilon >= 0.0f, "sofie_hip_layernorm_f32: epsilon is negative");
+   if (rows == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(Y && X && scale, "sofie_hip_layernorm_f32: NULL pointer");
+   const long long blocks = (rows + 3) / 4;
+   hipLaunchKernelGGL(layernorm_f32_kernel, dim3((unsigned)(blocks < 256 * 64 ? blocks : 256 * 64)), dim3(256), 0, ctx->stream, Y, X, scale, bias, (long long)rows, L,
+                      epsilon, mean_out, inv_std_out);
+   return launch_status("layernorm_f32_kernel");
 }
 
 int sofie_hip_plane_sums_to_average(sofie_hip_ctx *ctx, float *Y, const int32_t *sums, int32_t NC, int32_t HW, float scale)

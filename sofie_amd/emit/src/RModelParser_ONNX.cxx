@@ -579,6 +579,12 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
                                                                     n.in[1], bias, out));
       } else if (n.op == "GlobalAveragePool") {
          model->AddOperator(std::make_unique<ROperator_Pool<float>>(GlobalAveragePool, n.in[0], n.out[0]));
+      } else if (n.op == "LayerNormalization") {
+         if (n.in.size() < 2)
+            throw std::runtime_error("SOFIE ONNX parser: LayerNormalization " + n.name + " needs X and Scale");
+         model->AddOperator(std::make_unique<ROperator_LayerNormalization<float>>(
+            (int)attrI(n, "axis", -1), attrF(n, "epsilon", 1e-5f), (size_t)attrI(n, "stash_type", 1), n.in[0], n.in[1], n.in.size() > 2 ? n.in[2] : "", n.out[0],
+            n.out.size() > 1 ? n.out[1] : "", n.out.size() > 2 ? n.out[2] : ""));
       } else if (n.op == "Softmax" || n.op == "LogSoftmax") {
          model->AddOperator(std::make_unique<ROperator_Softmax>(attrI(n, "axis", -1), n.in[0], n.out[0], n.op == "LogSoftmax"));
       } else if (n.op == "MaxPool" || n.op == "AveragePool") {

@@ -126,6 +126,7 @@ SYMBOLS = {
     "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),
     "sofie_hip_global_avg_pool_f32": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32]),
     "sofie_hip_pool_f32": (C.c_int, [_P, _P, _P, _P]),
+    "sofie_hip_layernorm_f32": (C.c_int, [_P, _P, _P, _P, _P, C.c_int64, C.c_int32, C.c_float, _P, _P]),
     "sofie_hip_transpose_f32": (C.c_int, [_P, _P, _P, C.c_int32, _P, _P]),
     "sofie_hip_copy_rows": (C.c_int, [_P, _P, C.c_size_t, _P, C.c_size_t, C.c_size_t, C.c_size_t]),
     "sofie_hip_binary_f32": (C.c_int, [_P, _P, C.c_int32, C.c_float]),

@@ -169,6 +169,16 @@ def shape_plumbing(batch=3):
                 init=init, feeds=[X, Z])
 
 
+def layernorm_block(batch=3):
+    """Gemm -> LayerNormalization over the features (with its Mean as a second output) -> Gelu -> Gemm: the shape of a transformer's feed-forward entry."""
+    init = {"W1": util.normal(6501, 12 * 16, 0.3).reshape(12, 16), "b1": util.normal(6502, 16, 0.1), "g": (1 + 0.2 * util.normal(6503, 16)).astype(np.float32),
+            "beta": util.normal(6504, 16, 0.1), "W2": util.normal(6505, 16 * 4, 0.3).reshape(16, 4)}
+    nodes = [ow.node("Gemm", ["X", "W1", "b1"], ["H"]), ow.node("LayerNormalization", ["H", "g", "beta"], ["N", "M"], axis=-1, epsilon=1e-5),
+             ow.node("Gelu", ["N"], ["A"]), ow.node("MatMul", ["A", "W2"], ["Y"])]
+    X = util.normal(6506, batch * 12).reshape(batch, 12)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 12])], outputs=[("Y", np.float32, [batch, 4]), ("M", np.float32, [batch, 1])], init=init, feeds=[X])
+
+
 def softmax_head(batch=4):
     """Gemm -> Softmax over the classes (one output)."""
     spec = classifier_head(batch)
@@ -606,7 +616,8 @@ def build_all(jobs=8):
         ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=m)
         dynamic.append((m, p, len(spec["inputs"])))
     folded = reference_constant_folding_cases()
-    multi = [("ElementwiseChains", elementwise_chains, 2), ("ParseRewrites", parse_rewrites, 3), ("ClassifierHead", classifier_head, 1)]
+    multi = [("ElementwiseChains", elementwise_chains, 2), ("ParseRewrites", parse_rewrites, 3), ("ClassifierHead", classifier_head, 1),
+             ("LayerNormBlock", layernorm_block, 1)]
     multi += [(m, (lambda spec=spec: spec), len(spec["inputs"])) for m, spec in folded.items()]
     for m, spec in reference_stacked_matmul_cases().items():
         p = os.path.join(OUT, m + ".onnx")
@@ -634,7 +645,7 @@ def build_all(jobs=8):
         f.write(DYNAMIC_HARNESS % dict(model="ApiDynamicFp8Gemm", args="inputs[0]"))
     compile_shared(src, os.path.join(OUT, "libApiDynamicFp8Gemm.so"))
     compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
-    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead"]
+    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead", "LayerNormBlock"]
 
 
 if __name__ == "__main__":

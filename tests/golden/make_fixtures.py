@@ -72,9 +72,13 @@ def test_inputs_table(path, model):
         if c.group(1) != "f32":
             return None
         inner = body[call_open + 1:call_end - 1]
-        vals_open = inner.index("[")
-        vals_end = _matching(inner, vals_open, "[", "]")
+        vals_open = inner.index("[") if "[" in inner else 0
+        vals_end = _matching(inner, vals_open, "[", "]") if "[" in inner else 0
         values = [float(x) for x in re.findall(NUM, inner[vals_open:vals_end])]
+        ar = re.match(r"\s*np\.arange\(\s*(%s)\s*,\s*(%s)\s*\)" % (NUM, NUM), inner)
+        if ar:      # f32(np.arange(a, b), shape): the integers from a to b - 1
+            values = [float(v) for v in range(int(float(ar.group(1))), int(float(ar.group(2))))]
+            vals_end = ar.end()
         shape = [int(x) for x in re.findall(r"\d+", inner[vals_end:])]
         out.append({"kind": "values", "values": values, "shape": shape})
         pos = call_end
@@ -137,6 +141,11 @@ def main():
         if inputs is None:
             raise RuntimeError("no literal inputs for " + model)
         add(model, next(iter(arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx")).values())), inputs)
+    for model in ("LayerNormalization2d", "LayerNormalization4d"):      # expected outputs in <Model>.hxx, not .ref.hxx
+        shutil.copyfile(os.path.join(REF, "models/onnx", model + ".onnx"), os.path.join(HERE, "models", model + ".onnx"))
+        os.chmod(os.path.join(HERE, "models", model + ".onnx"), 0o644)
+        fixtures[model] = {"inputs": test_inputs_table(gen, model), "expected": arrays_in(os.path.join(REF, "models/onnx/references", model + ".hxx"))["output"],
+                           "source": "tests/models/onnx/%s.onnx + references/%s.hxx" % (model, model)}
     lin = os.path.join(REF, "alpaka/TestAlpakaLinear.cxx")
     add("LinearWithLeakyRelu", arrays_in(os.path.join(REF, "models/onnx/references/LinearWithLeakyRelu.ref.hxx"))["outputs"],
         [{"kind": "values", "values": vector_literal(lin, "LinearWithLeakyRelu", "input")}])

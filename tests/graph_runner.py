@@ -103,6 +103,9 @@ class OracleBackend:
     def softmax(self, X, axis, log):
         return self.ob.softmax(X, axis, log)
 
+    def layernorm(self, X, scale, bias, axis, eps):
+        return self.ob.layernorm(X, scale, bias, axis, eps)
+
     # pure data movement: numpy is the definition
     def transpose(self, X, perm):
         return np.ascontiguousarray(np.transpose(X, perm))
@@ -202,6 +205,21 @@ class HipBackend:
         axes = ob.pool_axes(X.shape[2:], a.get("kernel_shape"), a.get("pads"), a.get("strides"), a.get("dilations"), a.get("auto_pad", "NOTSET"),
                             a.get("ceil_mode", 0))
         return hip_pool(self.rt, X, mode, axes, a.get("ceil_mode", 0), a.get("count_include_pad", 0))
+
+    def layernorm(self, X, scale, bias, axis, eps, stats=False):
+        import torch
+        u = self.u
+        X = np.ascontiguousarray(X, dtype=np.float32)
+        axis = axis + X.ndim if axis < 0 else axis
+        rows, L = int(np.prod(X.shape[:axis], dtype=np.int64)), int(np.prod(X.shape[axis:], dtype=np.int64))
+        dX, dS = u.to_dev(X), u.to_dev(np.ascontiguousarray(scale, dtype=np.float32))
+        dB = None if bias is None else u.to_dev(np.ascontiguousarray(bias, dtype=np.float32))
+        dY, dM, dI = u.dev_empty(X.shape, np.float32), u.dev_empty((rows,), np.float32), u.dev_empty((rows,), np.float32)
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_layernorm_f32", u.ptr(dY), u.ptr(dX), u.ptr(dS), u.ptr(dB), rows, L, C.c_float(eps), u.ptr(dM) if stats else None,
+                     u.ptr(dI) if stats else None)
+        self.rt.sync()
+        return (u.to_host(dY), u.to_host(dM), u.to_host(dI)) if stats else u.to_host(dY)
 
     def transpose(self, X, perm):
         import torch
@@ -368,6 +386,8 @@ def run(g, inputs, be, all_outputs=False):
                 y = y[:, :, 0, :]
         elif op == "GlobalAveragePool":
             y = be.gap(x[0])
+        elif op == "LayerNormalization":
+            y = be.layernorm(x[0], x[1], x[2] if len(x) > 2 else None, a.get("axis", -1), a.get("epsilon", 1e-5))
         elif op in ("Softmax", "LogSoftmax"):
             y = be.softmax(x[0], a.get("axis", -1), op == "LogSoftmax")
         elif op in ("MaxPool", "AveragePool"):

@@ -8,6 +8,8 @@ import os
 import numpy as np
 import pytest
 
+from oracle import binding as ob
+from sofie_amd import runtime as R
 from tests import emitted_models as em
 from tests import graph_runner as gr
 from tests import onnx_lite
@@ -259,6 +261,19 @@ def test_emitted_classifier_head_with_softmax_and_logsoftmax(rt):
     assert np.all(np.abs(gq - Q) <= 1e-5 * np.abs(Q) + 1e-5) and P.std() > 0.01
     txt = open(os.path.join(em.OUT, "ClassifierHead_GPU_HIP.hxx")).read()
     assert txt.count("sofie_hip_softmax_f32(") == 2 and "sofie_hip_gemm_chain_f32(fCtx, chain, 2)" in txt
+
+
+def test_emitted_layernorm_block(rt):
+    spec = em.layernorm_block(3)
+    X = spec["feeds"][0]
+    i = spec["init"]
+    H = ob.gemm_f32(X, i["W1"], i["b1"], M=3, N=16, K=12, bias_mode=1)
+    N, mean, _ = ob.layernorm(H, i["g"], i["beta"], -1, 1e-5, stats=True)
+    Y = ob.gemm_f32(ob.unary(N, R.ACT_GELU), i["W2"], None, M=3, N=4, K=16)
+    print("emitted LayerNormBlock", flush=True)
+    got = run_emitted("LayerNormBlock", spec["feeds"], 12 + 3)
+    assert np.abs(got[:12] - Y.ravel()).max() <= 3e-5 * max(1.0, float(np.abs(Y).max())) and np.allclose(got[12:], mean, rtol=1e-5, atol=1e-6)
+    assert Y.std() > 0.05
 
 
 def test_emitted_shape_plumbing(rt):

@@ -11,7 +11,7 @@ from tests import graph_runner as gr
 
 # references printed with 4 decimals
 FOUR_DECIMALS = ("Gelu", "GeluTanh", "LinearWithLeakyRelu", "AvgPool", "MaxPool1d", "MaxPool2d", "AvgPoolPad", "AvgPoolCountIncludePad",
-                 "Exp", "Log", "Neg", "Elu", "SeluNonDefaultCoeffs", "Softmax3d", "Softmax4d")
+                 "Exp", "Log", "Neg", "Elu", "SeluNonDefaultCoeffs", "Softmax3d", "Softmax4d", "LayerNormalization2d", "LayerNormalization4d")
 
 
 # Inputs AND outputs printed with 4 decimals, the outputs computed from the unrounded inputs: the rounding of an input

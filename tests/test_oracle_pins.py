@@ -496,3 +496,26 @@ def test_binary_operators_against_numpy_and_the_library_semantics():
     # pow special values of the C library: x^0 = 1 for any x, 1^y = 1, a negative base with a non-integer exponent is NaN
     p = ob.binary_broadcast(np.array([np.nan, 1.0, -8.0, -8.0, 0.0], np.float32), np.array([0.0, np.nan, 1.0 / 3, 2.0, -1.0], np.float32), 4)
     assert p[0] == 1.0 and p[1] == 1.0 and np.isnan(p[2]) and p[3] == 64.0 and np.isposinf(p[4])
+
+
+def test_layernorm_against_the_definition():
+    rng = np.random.default_rng(51)
+    for shape, axis in [((3, 4), -1), ((2, 3, 4, 5), 2), ((5, 1000), 1), ((4, 6, 7), 1)]:
+        X = (2 * rng.standard_normal(shape) + 0.5).astype(np.float32)
+        ax = axis + len(shape) if axis < 0 else axis
+        norm_shape = shape[ax:]
+        scale, bias = rng.standard_normal(norm_shape).astype(np.float32), rng.standard_normal(norm_shape).astype(np.float32)
+        Y, mean, inv = ob.layernorm(X, scale, bias, axis, 1e-5, stats=True)
+        x64 = X.astype(np.float64).reshape(-1, int(np.prod(norm_shape)))
+        m = x64.mean(axis=1, keepdims=True)
+        v = ((x64 - m) ** 2).mean(axis=1, keepdims=True)
+        want = (x64 - m) / np.sqrt(v + 1e-5) * scale.astype(np.float64).ravel() + bias.astype(np.float64).ravel()
+        np.testing.assert_allclose(Y.reshape(want.shape), want, rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(mean, m.ravel(), rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(inv, 1 / np.sqrt(v.ravel() + 1e-5), rtol=1e-5)
+        # unit scale, no bias: every row comes out with zero mean and (up to epsilon) unit variance
+        Z = ob.layernorm(X, np.ones(norm_shape, np.float32), None, axis, 1e-5).reshape(want.shape)
+        assert np.abs(Z.mean(axis=1)).max() < 1e-5 and np.abs(Z.var(axis=1) - 1).max() < 1e-3
+    # a constant row has zero variance: the output is the bias, and invStdDev is 1 / sqrt(epsilon)
+    Y, mean, inv = ob.layernorm(np.full((1, 8), 3.0, np.float32), np.ones(8, np.float32), np.arange(8, dtype=np.float32), -1, 1e-4, stats=True)
+    assert Y.ravel().tolist() == list(range(8)) and mean[0] == 3.0 and abs(inv[0] - 100.0) < 1e-3
