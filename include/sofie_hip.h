@@ -377,6 +377,15 @@ int sofie_hip_plane_sums_to_average(sofie_hip_ctx *ctx, float *Y /* [NC] */, con
  * the rounding of that sum, which for the loop grows with the axis length (1e-7 relative at 10 classes, 6e-5 at 70000). */
 int sofie_hip_softmax_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int64_t outer, int32_t axis_len, int64_t inner, int32_t log_softmax);
 
+/* The Reduce family over the middle dimension of a tensor seen as [outer, A, inner] (ROperator_Reduce<Op>::Generate,
+ * core/inc/SOFIE/operators/ROperator_Reduce.hxx:349-400: start value 0, 1 for Prod, lowest() for Max, max() for Min; y += x, y += x*x,
+ * y *= x, y = std::max(y, x), y = std::min(y, x) over the reduced elements in increasing order; Mean then divides by float(A), L2 takes
+ * std::sqrt).  Reduced axes that are adjacent fold into one A.  Few long lines (inner == 1, A >= 64, fewer than 16384 outputs) are
+ * reduced by a wave each, as a tree: sums and products then agree with the loop to rounding only; every other case runs the loop's order. */
+enum { SOFIE_REDUCE_SUM = 0, SOFIE_REDUCE_MEAN = 1, SOFIE_REDUCE_SUM_SQUARE = 2, SOFIE_REDUCE_PROD = 3, SOFIE_REDUCE_L2 = 4, SOFIE_REDUCE_MAX = 5,
+       SOFIE_REDUCE_MIN = 6 };
+int sofie_hip_reduce_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int64_t outer, int32_t A, int64_t inner, int32_t op);
+
 /* LayerNormalization over the trailing dimensions of a tensor seen as [rows, L] (ROperator_LayerNormalization::Generate,
  * core/inc/SOFIE/operators/ROperator_LayerNormalization.hxx:247-312): mean = sum(x) / L, invStdDev = 1 / sqrt(sum((x - mean)^2) / L + epsilon),
  * Y = scale[j] * invStdDev * (x - mean) + bias[j].  scale and bias hold L elements (bias may be NULL); mean_out / inv_std_out, when not

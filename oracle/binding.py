@@ -196,6 +196,28 @@ def softmax(X, axis=-1, log=False):
     return Y
 
 
+def reduce_block(shape, axes):
+    """(outer, A, inner) of a reduction over adjacent axes of `shape` (dimensions of 1 may lie between them); None if the axes are not adjacent."""
+    rank = len(shape)
+    ax = sorted(a + rank if a < 0 else a for a in axes) if axes else list(range(rank))
+    if any(shape[i] != 1 for i in range(ax[0], ax[-1] + 1) if i not in ax):
+        return None
+    return (int(np.prod(shape[:ax[0]], dtype=np.int64)), int(np.prod(shape[ax[0]:ax[-1] + 1], dtype=np.int64)),
+            int(np.prod(shape[ax[-1] + 1:], dtype=np.int64)))
+
+
+def reduce(X, op, axes=None, keepdims=1):
+    """op: the SOFIE_REDUCE_* code; axes must be adjacent."""
+    X = _f32(X)
+    outer, A, inner = reduce_block(X.shape, axes)
+    Y = np.empty(outer * inner, dtype=np.float32)
+    load().oracle_reduce(_ptr(Y), _ptr(X), C.c_long(outer), C.c_int(A), C.c_long(inner), C.c_int(op))
+    rank = X.ndim
+    ax = sorted(a + rank if a < 0 else a for a in axes) if axes else list(range(rank))
+    shape = [1 if i in ax else d for i, d in enumerate(X.shape)] if keepdims else [d for i, d in enumerate(X.shape) if i not in ax]
+    return Y.reshape(shape)
+
+
 def layernorm(X, scale, bias=None, axis=-1, eps=1e-5, stats=False):
     X, scale = _f32(X), _f32(scale)
     axis = axis + X.ndim if axis < 0 else axis

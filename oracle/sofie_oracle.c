@@ -21,6 +21,8 @@
  *                             reference's tests; Erf against scipy's erf.
  *   binary_broadcast          Add, AddBroadcast1..7, Sub, Mul, Div, Pow, Pow_broadcast and the Max / Min / Mean / Sum
  *                             MultidirectionalBroadcast golden outputs; numpy's broadcasting arithmetic.
+ *   reduce                    ReduceMean, ReduceProd, ReduceL2, ReduceMax, ReduceMax_axis0, ReduceMax_mid golden outputs; numpy's
+ *                             reductions in float64.
  *   layernorm                 LayerNormalization2d / 4d golden outputs; the float64 definition; rows of zero mean and unit
  *                             variance before scale and bias.
  *   global_avg_pool           GlobalAvgPool2d golden output.
@@ -475,6 +477,35 @@ ORACLE_API void oracle_softmax(float *Y, const float *X, long outer, int A, long
             for (int i = 0; i < A; ++i)
                y[(size_t)i * inner] /= sum;
          }
+      }
+   }
+}
+
+/* The Reduce family over the middle dimension of [outer, A, inner]: ROperator_Reduce<Op>::Generate
+ * (core/inc/SOFIE/operators/ROperator_Reduce.hxx:349-400), whose three loop nests (reduced axes last, first, in the middle) all visit
+ * the reduced elements of an output in increasing order.  op: 0 Sum, 1 Mean, 2 SumSquare, 3 Prod, 4 L2, 5 Max, 6 Min. */
+ORACLE_API void oracle_reduce(float *Y, const float *X, long outer, int A, long inner, int op)
+{
+   for (long o = 0; o < outer; ++o) {
+      for (long in = 0; in < inner; ++in) {
+         const float *x = X + (size_t)o * A * inner + in;
+         float y = op == 3 ? 1.0f : op == 5 ? -3.402823466e+38f : op == 6 ? 3.402823466e+38f : 0.0f;
+         for (int a = 0; a < A; ++a) {
+            float v = x[(size_t)a * inner];
+            switch (op) {
+            case 2:
+            case 4: y += v * v; break;
+            case 3: y *= v; break;
+            case 5: y = y < v ? v : y; break; /* std::max(y, v) */
+            case 6: y = v < y ? v : y; break; /* std::min(y, v) */
+            default: y += v; break;
+            }
+         }
+         if (op == 1)
+            y /= (float)A;
+         else if (op == 4)
+            y = sqrtf(y);
+         Y[(size_t)o * inner + in] = y;
       }
    }
 }

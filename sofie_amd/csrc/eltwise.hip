@@ -2,6 +2,7 @@
 // broadcast Add, GlobalAveragePool.  Each thread moves 16 bytes of the widest operand per step and
 // the grid strides over the tensor, so the launches stay coalesced for any length.
 #include "common.hpp"
+#include <cfloat>
 
 namespace sofie_hip {
 
@@ -275,6 +276,63 @@ __global__ __launch_bounds__(256) void softmax_f32_kernel(float *__restrict__ Y,
    }
 }
 
+__device__ __forceinline__ float reduce_start(int op)
+{
+   return op == SOFIE_REDUCE_PROD ? 1.0f : op == SOFIE_REDUCE_MAX ? -FLT_MAX : op == SOFIE_REDUCE_MIN ? FLT_MAX : 0.0f;
+}
+__device__ __forceinline__ float reduce_step(float y, float x, int op)
+{
+   switch (op) {
+   case SOFIE_REDUCE_SUM_SQUARE:
+   case SOFIE_REDUCE_L2: return y + mul_nofma(x, x);
+   case SOFIE_REDUCE_PROD: return mul_nofma(y, x);
+   case SOFIE_REDUCE_MAX: return y < x ? x : y;
+   case SOFIE_REDUCE_MIN: return x < y ? x : y;
+   default: return y + x;
+   }
+}
+// folds two partial results (the tree form): partial sums of squares add, everything else combines as a step does
+__device__ __forceinline__ float reduce_merge(float a, float b, int op)
+{
+   return (op == SOFIE_REDUCE_SUM_SQUARE || op == SOFIE_REDUCE_L2) ? a + b : reduce_step(a, b, op);
+}
+__device__ __forceinline__ float reduce_finish(float y, int A, int op)
+{
+   return op == SOFIE_REDUCE_MEAN ? __fdiv_rn(y, (float)A) : op == SOFIE_REDUCE_L2 ? sqrtf(y) : y;
+}
+
+// One output per thread, the reduced elements in increasing order: the reference's loop (neighbouring threads read neighbouring `inner`).
+__global__ __launch_bounds__(256) void reduce_f32_kernel(float *__restrict__ Y, const float *__restrict__ X, size_t outputs, int A, long long inner, int op)
+{
+   const size_t stride = (size_t)gridDim.x * blockDim.x;
+   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < outputs; i += stride) {
+      const size_t o = i / (size_t)inner, in = i - o * (size_t)inner;
+      const float *x = X + o * (size_t)A * (size_t)inner + in;
+      float y = reduce_start(op);
+      for (int a = 0; a < A; ++a)
+         y = reduce_step(y, x[(size_t)a * (size_t)inner], op);
+      Y[i] = reduce_finish(y, A, op);
+   }
+}
+
+// Long contiguous lines: one wave per line, lanes stride over it, then a shuffle tree.
+__global__ __launch_bounds__(256) void reduce_lines_f32_kernel(float *__restrict__ Y, const float *__restrict__ X, long long lines, int A, int op)
+{
+   const int lane = threadIdx.x & 63;
+   const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6), nwaves = (long long)gridDim.x * 4;
+   for (long long line = wave; line < lines; line += nwaves) {
+      const float *x = X + line * A;
+      float y = reduce_start(op);
+      for (int a = lane; a < A; a += 64)
+         y = reduce_step(y, x[a], op);
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1)
+         y = reduce_merge(y, __shfl_xor(y, off, 64), op);
+      if (lane == 0)
+         Y[line] = reduce_finish(y, A, op);
+   }
+}
+
 // LayerNormalization: one wave per row of L elements, lanes stride over the row; mean, then the centred sum of squares, then the output.
 __global__ __launch_bounds__(256) void layernorm_f32_kernel(float *__restrict__ Y, const float *__restrict__ X, const float *__restrict__ scale,
                                                             const float *__restrict__ bias, long long rows, int L, float epsilon,
@@ -300,7 +358,7 @@ __global__ __launch_bounds__(256) void layernorm_f32_kernel(float *__restrict__ 
 #pragma unroll
       for (int off = 32; off >= 1; off >>= 1)
          sum += __shfl_xor(sum, off, 64);
-      const float inv_std = __fdiv_rn(1.0f, __fsqrt_rn(__fdiv_rn(sum, (float)L) + epsilon));
+      const float inv_std = __fdiv_rn(1.0f, sqrtf(__fdiv_rn(sum, (float)L) + epsilon));
       if (lane == 0) {
          if (mean_out)
             mean_out[row] = mean;
@@ -626,6 +684,24 @@ int sofie_hip_softmax_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int64_t 
    hipLaunchKernelGGL(softmax_f32_kernel, dim3((unsigned)(blocks < 256 * 64 ? blocks : 256 * 64)), dim3(256), 0, ctx->stream, Y, X, lines, axis_len,
                       (long long)inner, log_softmax);
    return launch_status("softmax_f32_kernel");
+}
+
+int sofie_hip_reduce_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int64_t outer, int32_t A, int64_t inner, int32_t op)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_reduce_f32: ctx is NULL");
+   SOFIE_HIP_REQUIRE(op >= SOFIE_REDUCE_SUM && op <= SOFIE_REDUCE_MIN, "sofie_hip_reduce_f32: unknown operator %d", op);
+   SOFIE_HIP_REQUIRE(outer >= 0 && A > 0 && inner > 0 && outer < (1LL << 40) && inner < (1LL << 40) && (double)outer * A * (double)inner < 1.0e12,
+                     "sofie_hip_reduce_f32: bad shape");
+   const long long outputs = (long long)outer * inner;
+   if (outputs == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(Y && X, "sofie_hip_reduce_f32: NULL pointer");
+   if (inner == 1 && A >= 64 && outputs < 16384) {
+      hipLaunchKernelGGL(reduce_lines_f32_kernel, dim3((unsigned)((outputs + 3) / 4)), dim3(256), 0, ctx->stream, Y, X, outputs, A, op);
+      return launch_status("reduce_lines_f32_kernel");
+   }
+   hipLaunchKernelGGL(reduce_f32_kernel, dim3(grid_for((size_t)outputs)), dim3(256), 0, ctx->stream, Y, X, (size_t)outputs, A, (long long)inner, op);
+   return launch_status("reduce_f32_kernel");
 }
 
 int sofie_hip_layernorm_f32(sofie_hip_ctx *ctx, float *Y, const float *X, const float *scale, const float *bias, int64_t rows, int32_t L, float epsilon,

@@ -30,6 +30,8 @@ public:
    virtual std::size_t GetWorkspaceBytes() { return 0; }
    // in a model with a run-time batch: true if GetWorkspaceBytes() is the need of ONE batch entry
    virtual bool WorkspacePerBatchEntry() const { return false; }
+   // true for an operator that reads a tensor with a run-time batch and folds the batch away (a reduction over it): its outputs carry none
+   virtual bool ConsumesBatch() const { return false; }
    virtual OperatorKind GetKind() const { return fKind; }
    const std::vector<std::string> &GetInputTensorNames() const { return fInputTensorNames; }
    const std::vector<std::string> &GetOutputTensorNames() const { return fOutputTensorNames; }

@@ -412,7 +412,7 @@ void RModel::Initialize(int batchSize)
          batchedIn = batchedIn || IsDynamicTensor(in);
       for (auto &y : fOperators[i]->GetOutputTensorNames())
          batchedOut = batchedOut || IsDynamicTensor(y);
-      if (batchedIn && !batchedOut)
+      if (batchedIn && !batchedOut && !fOperators[i]->ConsumesBatch())
          throw std::runtime_error("SOFIE: operator " + std::to_string(i) + " (output " + fOperators[i]->GetOutputTensorNames().at(0) +
                                   ") does not support a run-time batch; generate with a fixed batch size");
    }

@@ -585,6 +585,28 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          model->AddOperator(std::make_unique<ROperator_LayerNormalization<float>>(
             (int)attrI(n, "axis", -1), attrF(n, "epsilon", 1e-5f), (size_t)attrI(n, "stash_type", 1), n.in[0], n.in[1], n.in.size() > 2 ? n.in[2] : "", n.out[0],
             n.out.size() > 1 ? n.out[1] : "", n.out.size() > 2 ? n.out[2] : ""));
+      } else if (n.op.rfind("Reduce", 0) == 0) {
+         // keepdims = 1 and the axes attribute (before opset 13 / 18) or the axes input (parsers/src/ParseReduce.cxx:41-62)
+         auto f = n.attrs.find("axes");
+         const std::vector<int64_t> axes = f == n.attrs.end() ? std::vector<int64_t>{} : f->second.ints;
+         const int keepdims = (int)attrI(n, "keepdims", 1);
+         const std::string axesName = n.in.size() > 1 ? n.in[1] : "";
+         if (n.op == "ReduceMean")
+            model->AddOperator(std::make_unique<ROperator_Reduce<ReduceMean>>(keepdims, axes, n.in[0], axesName, n.out[0]));
+         else if (n.op == "ReduceSum")
+            model->AddOperator(std::make_unique<ROperator_Reduce<ReduceSum>>(keepdims, axes, n.in[0], axesName, n.out[0]));
+         else if (n.op == "ReduceSumSquare")
+            model->AddOperator(std::make_unique<ROperator_Reduce<ReduceSumSquare>>(keepdims, axes, n.in[0], axesName, n.out[0]));
+         else if (n.op == "ReduceProd")
+            model->AddOperator(std::make_unique<ROperator_Reduce<ReduceProd>>(keepdims, axes, n.in[0], axesName, n.out[0]));
+         else if (n.op == "ReduceL2")
+            model->AddOperator(std::make_unique<ROperator_Reduce<ReduceL2>>(keepdims, axes, n.in[0], axesName, n.out[0]));
+         else if (n.op == "ReduceMax")
+            model->AddOperator(std::make_unique<ROperator_Reduce<ReduceMax>>(keepdims, axes, n.in[0], axesName, n.out[0]));
+         else if (n.op == "ReduceMin")
+            model->AddOperator(std::make_unique<ROperator_Reduce<ReduceMin>>(keepdims, axes, n.in[0], axesName, n.out[0]));
+         else
+            throw std::runtime_error("SOFIE - Reduce op mode not supported.");
       } else if (n.op == "Softmax" || n.op == "LogSoftmax") {
          model->AddOperator(std::make_unique<ROperator_Softmax>(attrI(n, "axis", -1), n.in[0], n.out[0], n.op == "LogSoftmax"));
       } else if (n.op == "MaxPool" || n.op == "AveragePool") {

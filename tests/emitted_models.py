@@ -179,6 +179,19 @@ def layernorm_block(batch=3):
     return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 12])], outputs=[("Y", np.float32, [batch, 4]), ("M", np.float32, [batch, 1])], init=init, feeds=[X])
 
 
+def reduce_block(batch=3, named=None):
+    """ReduceMean over the last axis (kept) -> Sub (centring) -> ReduceL2 with the axes as an input; a ReduceMax over the middle axis and a ReduceSum
+    over the batch itself as further outputs.  `named` leaves the batch as a run-time parameter."""
+    b = named if named else batch
+    init = {"ax": np.array([-1], np.int64)}
+    nodes = [ow.node("ReduceMean", ["X"], ["M"], axes=[2], keepdims=1), ow.node("Sub", ["X", "M"], ["C"]),
+             ow.node("ReduceL2", ["C", "ax"], ["Y1"], keepdims=0), ow.node("ReduceMax", ["X"], ["Y2"], axes=[1], keepdims=0),
+             ow.node("ReduceSum", ["X"], ["Y3"], axes=[0], keepdims=1)]
+    X = (util.normal(6601, batch * 24) + np.float32(0.25)).reshape(batch, 4, 6)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [b, 4, 6])], outputs=[("Y1", np.float32, [b, 4]), ("Y2", np.float32, [b, 6]), ("Y3", np.float32, [1, 4, 6])],
+                init=init, feeds=[X])
+
+
 def softmax_head(batch=4):
     """Gemm -> Softmax over the classes (one output)."""
     spec = classifier_head(batch)
@@ -363,6 +376,7 @@ DYNAMIC_MODELS = {    "Dynamic_ResidualBlock": lambda: with_named_batch(residual
     "Dynamic_ConvPoolStack": lambda: with_named_batch(conv_pool_stack(2), "N"),
     "Dynamic_SoftmaxHead": lambda: with_named_batch(softmax_head(4), "N"),
     "Dynamic_ShapePlumbing": lambda: with_named_batch(shape_plumbing(3), "N"),
+    "Dynamic_ReduceBlock": lambda: reduce_block(3, "N"),
     "Dynamic_int8_CNN_plane_sums": lambda: with_named_batch(int8_cnn(2, 16, (3, 64, 128)), "N"),
 }
 
@@ -478,6 +492,12 @@ static int fail(char *err, int errlen, const char *what)
    err[errlen - 1] = 0;
    return 1;
 }
+static void flatten(const std::vector<float> &y, std::vector<float> &all) { all.insert(all.end(), y.begin(), y.end()); }
+[[maybe_unused]] static void flatten(const std::vector<std::vector<float>> &ys, std::vector<float> &all)
+{
+   for (auto &y : ys)
+      flatten(y, all);
+}
 extern "C" void *dyn_open(const char *weights, unsigned long max_batch, char *err, int errlen)
 {
    try {
@@ -491,7 +511,8 @@ extern "C" void dyn_close(void *s) { delete static_cast<Session *>(s); }
 extern "C" long dyn_infer(void *s, unsigned long batch, const float *const *inputs, float *output, unsigned long capacity, char *err, int errlen)
 {
    try {
-      auto y = static_cast<Session *>(s)->infer(batch, %(args)s);
+      std::vector<float> y;
+      flatten(static_cast<Session *>(s)->infer(batch, %(args)s), y);      // several outputs come back one after the other
       if (y.size() > capacity)
          throw std::runtime_error("output has " + std::to_string(y.size()) + " elements");
       std::memcpy(output, y.data(), y.size() * sizeof(float));
@@ -617,7 +638,7 @@ def build_all(jobs=8):
         dynamic.append((m, p, len(spec["inputs"])))
     folded = reference_constant_folding_cases()
     multi = [("ElementwiseChains", elementwise_chains, 2), ("ParseRewrites", parse_rewrites, 3), ("ClassifierHead", classifier_head, 1),
-             ("LayerNormBlock", layernorm_block, 1)]
+             ("LayerNormBlock", layernorm_block, 1), ("ReduceBlock", reduce_block, 1)]
     multi += [(m, (lambda spec=spec: spec), len(spec["inputs"])) for m, spec in folded.items()]
     for m, spec in reference_stacked_matmul_cases().items():
         p = os.path.join(OUT, m + ".onnx")
@@ -645,7 +666,7 @@ def build_all(jobs=8):
         f.write(DYNAMIC_HARNESS % dict(model="ApiDynamicFp8Gemm", args="inputs[0]"))
     compile_shared(src, os.path.join(OUT, "libApiDynamicFp8Gemm.so"))
     compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
-    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead", "LayerNormBlock"]
+    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead", "LayerNormBlock", "ReduceBlock"]
 
 
 if __name__ == "__main__":

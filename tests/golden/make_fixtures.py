@@ -39,6 +39,15 @@ def vector_literal(path, test_name, var):
     return [float(x) for x in re.findall(NUM, body)]
 
 
+def array_literal(path, test_name, var):
+    """The numbers of `std::vector<float> var = { ... }` or `float var[] = { ... }` inside TEST_F(..., test_name)."""
+    text = open(path).read()
+    start = text.index("TEST_F(SofieAlpakaTest, %s)" % test_name)
+    m = re.search(r"(?:std::vector<float>|float)\s+%s\s*(?:\[\])?\s*=\s*\{(.*?)\}" % var, text[start:], re.S)
+    body = re.sub(r"(?<=[\d.])f\b", "", m.group(1))
+    return [float(x) for x in re.findall(NUM, body)]
+
+
 def _matching(text, start, open_ch, close_ch):
     """Index just past the bracket that closes the one at text[start]."""
     depth = 0
@@ -146,6 +155,16 @@ def main():
         os.chmod(os.path.join(HERE, "models", model + ".onnx"), 0o644)
         fixtures[model] = {"inputs": test_inputs_table(gen, model), "expected": arrays_in(os.path.join(REF, "models/onnx/references", model + ".hxx"))["output"],
                            "source": "tests/models/onnx/%s.onnx + references/%s.hxx" % (model, model)}
+    red = os.path.join(REF, "alpaka/TestAlpakaReduce.cxx")
+    for model, var in (("ReduceMean", "input"), ("ReduceProd", "input"), ("ReduceL2", "input"), ("ReduceMax", "input"), ("ReduceMax_axis0", "vals"),
+                       ("ReduceMax_mid", "vals")):
+        add(model, arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx"))["output"],
+            [{"kind": "values", "values": array_literal(red, model, var)}])
+    for model in ("ReduceSum", "ReduceSumSquare"):      # expected outputs are literals of the test itself
+        shutil.copyfile(os.path.join(REF, "models/onnx", model + ".onnx"), os.path.join(HERE, "models", model + ".onnx"))
+        os.chmod(os.path.join(HERE, "models", model + ".onnx"), 0o644)
+        fixtures[model] = {"inputs": [{"kind": "values", "values": array_literal(red, model, "input")}], "expected": array_literal(red, model, "correct"),
+                           "source": "tests/models/onnx/%s.onnx + tests/alpaka/TestAlpakaReduce.cxx" % model}
     lin = os.path.join(REF, "alpaka/TestAlpakaLinear.cxx")
     add("LinearWithLeakyRelu", arrays_in(os.path.join(REF, "models/onnx/references/LinearWithLeakyRelu.ref.hxx"))["outputs"],
         [{"kind": "values", "values": vector_literal(lin, "LinearWithLeakyRelu", "input")}])

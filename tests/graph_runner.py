@@ -106,6 +106,9 @@ class OracleBackend:
     def layernorm(self, X, scale, bias, axis, eps):
         return self.ob.layernorm(X, scale, bias, axis, eps)
 
+    def reduce(self, X, op, axes, keepdims):
+        return self.ob.reduce(X, op, axes, keepdims)
+
     # pure data movement: numpy is the definition
     def transpose(self, X, perm):
         return np.ascontiguousarray(np.transpose(X, perm))
@@ -205,6 +208,20 @@ class HipBackend:
         axes = ob.pool_axes(X.shape[2:], a.get("kernel_shape"), a.get("pads"), a.get("strides"), a.get("dilations"), a.get("auto_pad", "NOTSET"),
                             a.get("ceil_mode", 0))
         return hip_pool(self.rt, X, mode, axes, a.get("ceil_mode", 0), a.get("count_include_pad", 0))
+
+    def reduce(self, X, op, axes, keepdims):
+        import torch
+        from oracle import binding as ob
+        u = self.u
+        X = np.ascontiguousarray(X, dtype=np.float32)
+        outer, A, inner = ob.reduce_block(X.shape, axes)
+        dX, dY = u.to_dev(X), u.dev_empty((outer * inner,), np.float32)
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_reduce_f32", u.ptr(dY), u.ptr(dX), outer, A, inner, op)
+        self.rt.sync()
+        ax = sorted(a + X.ndim if a < 0 else a for a in axes) if axes else list(range(X.ndim))
+        shape = [1 if i in ax else d for i, d in enumerate(X.shape)] if keepdims else [d for i, d in enumerate(X.shape) if i not in ax]
+        return u.to_host(dY).reshape(shape)
 
     def layernorm(self, X, scale, bias, axis, eps, stats=False):
         import torch
@@ -317,6 +334,9 @@ def hip_pool(rt, X, mode, axes, ceil_mode=0, count_include_pad=0):
     return u.to_host(dY)
 
 
+# SOFIE_REDUCE_* codes of include/sofie_hip.h
+REDUCE = {"ReduceSum": 0, "ReduceMean": 1, "ReduceSumSquare": 2, "ReduceProd": 3, "ReduceL2": 4, "ReduceMax": 5, "ReduceMin": 6}
+
 # SOFIE_BINARY_* codes of include/sofie_hip.h
 BINARY = {"Sub": 1, "Mul": 2, "Div": 3, "Pow": 4}
 NARY = {"Max": 5, "Min": 6, "Sum": 0, "Mean": 0}
@@ -386,6 +406,9 @@ def run(g, inputs, be, all_outputs=False):
                 y = y[:, :, 0, :]
         elif op == "GlobalAveragePool":
             y = be.gap(x[0])
+        elif op in REDUCE:
+            axes = [int(v) for v in np.asarray(x[1]).ravel()] if len(x) > 1 and x[1] is not None else list(a.get("axes", []))
+            y = be.reduce(x[0], REDUCE[op], axes, a.get("keepdims", 1))
         elif op == "LayerNormalization":
             y = be.layernorm(x[0], x[1], x[2] if len(x) > 2 else None, a.get("axis", -1), a.get("epsilon", 1e-5))
         elif op in ("Softmax", "LogSoftmax"):

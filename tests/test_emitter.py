@@ -487,3 +487,20 @@ def test_pool_attributes_resolve_to_the_reference_shapes(emitted, tmp_path):
     r = _emit(tmp_path, [ow.node("MaxPool", ["X"], ["Y", "I"], kernel_shape=[2, 2])], [("X", np.float32, [1, 1, 4, 4])],
               [("Y", np.float32, [1, 1, 3, 3])], {}, name="indices")
     assert r.returncode != 0 and "Indices" in r.stdout
+
+
+def test_reduce_shapes_axes_and_refusals(tmp_path):
+    f = np.float32
+    # keepdims = 0 over the two middle axes, the axes as an input; negative axes; everything reduced when no axes are given
+    r = _emit(tmp_path, [ow.node("ReduceSum", ["X", "ax"], ["Y"], keepdims=0), ow.node("ReduceMean", ["X"], ["Z"], axes=[-1]), ow.node("ReduceProd", ["X"], ["P"], keepdims=0)],
+              [("X", f, [2, 3, 4, 5])], [("Y", f, [2, 5]), ("Z", f, [2, 3, 4, 1]), ("P", f, [])], {"ax": np.array([1, 2], np.int64)}, name="red")
+    assert r.returncode == 0, r.stdout
+    txt = open(os.path.join(str(tmp_path), "red_GPU_HIP.hxx")).read()
+    assert "tensor_X, 2, 12, 5, SOFIE_REDUCE_SUM)" in txt and "tensor_X, 24, 5, 1, SOFIE_REDUCE_MEAN)" in txt and "tensor_X, 1, 120, 1, SOFIE_REDUCE_PROD)" in txt
+    # axes that are not adjacent, an axis out of range, axes computed at run time
+    r = _emit(tmp_path, [ow.node("ReduceMax", ["X"], ["Y"], axes=[0, 2])], [("X", f, [2, 3, 4])], [("Y", f, [1, 3, 1])], {}, name="gap")
+    assert r.returncode != 0 and "ReduceMax" in r.stdout and "not adjacent" in r.stdout
+    r = _emit(tmp_path, [ow.node("ReduceMin", ["X"], ["Y"], axes=[3])], [("X", f, [2, 3, 4])], [("Y", f, [2, 3, 4])], {}, name="range")
+    assert r.returncode != 0 and "invalid axes values 3" in r.stdout
+    r = _emit(tmp_path, [ow.node("ReduceL2", ["X", "A"], ["Y"])], [("X", f, [2, 3]), ("A", np.int64, [1])], [("Y", f, [2, 1])], {}, name="runtime_axes")
+    assert r.returncode != 0 and "int64 initializer" in r.stdout

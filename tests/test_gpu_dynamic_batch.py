@@ -7,6 +7,7 @@ import os
 import numpy as np
 import pytest
 
+from sofie_amd import runtime as R
 from tests import emitted_models as em
 from tests import graph_runner as gr
 from tests import onnx_lite
@@ -153,6 +154,20 @@ def test_dynamic_shape_plumbing(rt):
             print("Dynamic_ShapePlumbing batch", n, flush=True)
             got = s.infer(n, [x[:n], z[:n]], want.size)
             assert got.size == want.size == n * 6 and np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+
+
+def test_dynamic_reduce_block_keeps_or_consumes_the_batch(rt):
+    from oracle import binding as ob
+    x = np.concatenate([em.reduce_block(3)["feeds"][0], util.normal(8306, 4 * 24).reshape(4, 4, 6)])
+    with DynamicSession("Dynamic_ReduceBlock", 7) as s:
+        for n in (7, 3, 1):
+            X = x[:n]
+            C = ob.binary_broadcast(X, ob.reduce(X, R.REDUCE_MEAN, [2], 1), 1)
+            # Y1 and Y2 keep the batch; Y3 sums over it (the reference's DynamicReduceMaxFirst reduces over the run-time dimension in the same way)
+            want = np.concatenate([ob.reduce(C, R.REDUCE_L2, [-1], 0).ravel(), ob.reduce(X, R.REDUCE_MAX, [1], 0).ravel(), ob.reduce(X, R.REDUCE_SUM, [0], 1).ravel()])
+            print("Dynamic_ReduceBlock batch", n, flush=True)
+            got = s.infer(n, [X], want.size)
+            assert got.size == want.size == n * 10 + 24 and np.array_equal(got, want)
 
 
 def test_dynamic_softmax_head(rt):

@@ -276,6 +276,20 @@ def test_emitted_layernorm_block(rt):
     assert Y.std() > 0.05
 
 
+def test_emitted_reduce_block(rt):
+    spec = em.reduce_block(3)
+    X = spec["feeds"][0]
+    C = ob.binary_broadcast(X, ob.reduce(X, R.REDUCE_MEAN, [2], 1), 1)
+    want = np.concatenate([ob.reduce(C, R.REDUCE_L2, [-1], 0).ravel(), ob.reduce(X, R.REDUCE_MAX, [1], 0).ravel(), ob.reduce(X, R.REDUCE_SUM, [0], 1).ravel()])
+    print("emitted ReduceBlock", flush=True)
+    got = run_emitted("ReduceBlock", spec["feeds"], want.size)
+    assert want.size == 12 + 18 + 24 and np.array_equal(got, want) and want.std() > 0.3
+    # float64 numpy as a second opinion on the whole graph
+    x64 = X.astype(np.float64)
+    ref = np.concatenate([np.sqrt(((x64 - x64.mean(axis=2, keepdims=True)) ** 2).sum(axis=2)).ravel(), x64.max(axis=1).ravel(), x64.sum(axis=0).ravel()])
+    assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
+
+
 def test_emitted_shape_plumbing(rt):
     spec = em.shape_plumbing(3)
     g = onnx_lite.load(os.path.join(em.OUT, "ShapePlumbing.onnx"))

@@ -519,3 +519,34 @@ def test_layernorm_against_the_definition():
     # a constant row has zero variance: the output is the bias, and invStdDev is 1 / sqrt(epsilon)
     Y, mean, inv = ob.layernorm(np.full((1, 8), 3.0, np.float32), np.ones(8, np.float32), np.arange(8, dtype=np.float32), -1, 1e-4, stats=True)
     assert Y.ravel().tolist() == list(range(8)) and mean[0] == 3.0 and abs(inv[0] - 100.0) < 1e-3
+
+
+def test_reduce_against_numpy_in_float64():
+    rng = np.random.default_rng(77)
+    np_ops = {0: lambda x, ax: x.sum(axis=ax), 1: lambda x, ax: x.mean(axis=ax), 2: lambda x, ax: (x * x).sum(axis=ax), 3: lambda x, ax: x.prod(axis=ax),
+              4: lambda x, ax: np.sqrt((x * x).sum(axis=ax)), 5: lambda x, ax: x.max(axis=ax), 6: lambda x, ax: x.min(axis=ax)}
+    for shape, axes in [((1, 2, 3), [1]), ((3, 4), [0]), ((2, 3, 4), [1]), ((2, 3, 4), [-1]), ((2, 3, 4, 5), [1, 2]), ((4, 512), [1]), ((5, 7), None),
+                        ((6, 1, 5), [0, 2])]:
+        X = rng.uniform(0.5, 1.5, shape).astype(np.float32) * rng.choice([-1.0, 1.0], shape).astype(np.float32)
+        ax = tuple(range(len(shape))) if axes is None else tuple(a % len(shape) for a in axes)
+        for op, f in np_ops.items():
+            for keep in (0, 1):
+                want = f(X.astype(np.float64), ax)
+                got = ob.reduce(X, op, axes, keep)
+                want = np.expand_dims(want, ax) if keep else want
+                assert got.shape == np.shape(want), (shape, axes, op, keep)
+                if op >= 5:
+                    assert np.array_equal(got, want.astype(np.float32))
+                else:
+                    np.testing.assert_allclose(got, want, rtol=3e-6, atol=3e-6 * np.abs(X).sum(axis=ax).max() if op != 3 else 0)
+    # the reference's own literal cases: ReduceSum {24}, ReduceSumSquare {38, 66}, ReduceMin {5, 2, 3}, ReduceMean over the first axis of iota(12) = {4, 5, 6, 7},
+    # ReduceL2Large rows of r + 1 over 512 columns = (r + 1) * sqrt(512)
+    x = np.array([5, 2, 3, 5, 5, 4], np.float32).reshape(1, 2, 3)
+    assert ob.reduce(x, 0, [0, 1, 2], 1).ravel().tolist() == [24.0] and ob.reduce(x, 2, [2], 0).ravel().tolist() == [38.0, 66.0]
+    assert ob.reduce(x, 6, [1], 0).ravel().tolist() == [5.0, 2.0, 3.0]
+    assert ob.reduce(np.arange(12, dtype=np.float32).reshape(3, 4), 1, [0], 0).tolist() == [4.0, 5.0, 6.0, 7.0]
+    big = np.repeat(np.arange(1, 5, dtype=np.float32)[:, None], 512, axis=1)
+    np.testing.assert_allclose(ob.reduce(big, 4, [1], 0), np.arange(1, 5) * np.sqrt(512.0), rtol=1e-6)
+    # empty-product and start values: a reduced length of 1 returns the element (its square, its absolute value for L2)
+    one = np.array([[-3.0]], np.float32)
+    assert [float(ob.reduce(one, op, [1], 0)[0]) for op in range(7)] == [-3.0, -3.0, 9.0, -3.0, 3.0, -3.0, -3.0]
