@@ -109,7 +109,10 @@ enum {
    SOFIE_ACT_SELU = 22,      /* beta * (max(0,x) + min(0, alpha*(exp(x)-1))), beta = gamma; core/inc/SOFIE/operators/ROperator_Selu.hxx:56-62 */
    SOFIE_ACT_ELU = 23,       /* x >= 0 ? x : alpha * (exp(x) - 1); core/inc/SOFIE/operators/ROperator_Elu.hxx:69-74 */
    SOFIE_ACT_ERF = 24,       /* std::erf(x); core/inc/SOFIE/operators/ROperator_Erf.hxx */
-   SOFIE_ACT_LAST = 24
+   SOFIE_ACT_HARDSIGMOID = 25, /* max(0, min(1, alpha * x + beta)); core/inc/SOFIE/operators/ROperator_HardSigmoid.hxx:71-74 */
+   SOFIE_ACT_HARDSWISH = 26,   /* x * fmax(0, fmin(1, (1/6) * x + 1/2)), 1/6 rounded to float; core/inc/SOFIE/operators/ROperator_HardSwish.hxx:56-60 */
+   SOFIE_ACT_SWISH = 27,       /* x / (1 + exp(-x)); core/inc/SOFIE/operators/ROperator_Swish.hxx:54-56 */
+   SOFIE_ACT_LAST = 27
 };
 
 /* A chain of one-to-one operators applied, in order, to every element an operator stores: what the reference's

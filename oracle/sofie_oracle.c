@@ -158,6 +158,13 @@ ORACLE_API void oracle_basic_unary(float *out, const float *in, size_t n, int op
       case 22: y = beta * (fmaxf(0.0f, x) + fminf(0.0f, alpha * (expf(x) - 1.0f))); break; /* Selu, ROperator_Selu.hxx:56-62; beta = gamma */
       case 23: y = x >= 0.0f ? x : alpha * (expf(x) - 1.0f); break; /* Elu, ROperator_Elu.hxx:69-74 */
       case 24: y = erff(x); break;                                  /* Erf, ROperator_Erf.hxx: std::erf */
+      case 25: y = fmaxf(0.0f, fminf(1.0f, alpha * x + beta)); break; /* HardSigmoid, ROperator_HardSigmoid.hxx:71-74 */
+      case 26: {                                                    /* HardSwish, ROperator_HardSwish.hxx:56-60 */
+         float h = 0x1.5555555555555p-3f * x + 0x1p-1f;
+         y = x * fmaxf(0.0f, fminf(1.0f, h));
+         break;
+      }
+      case 27: y = x / (1 + expf(-x)); break;                       /* Swish, ROperator_Swish.hxx:54-56 */
       default: break;
       }
       out[i] = y;
@@ -175,7 +182,7 @@ ORACLE_API void oracle_unary(float *out, const float *in, size_t n, int act, flo
    case 5: oracle_gelu_tanh(out, in, n); break;
    case 6: oracle_tanh(out, in, n); break;
    default:
-      if (act >= 7 && act <= 24)
+      if (act >= 7 && act <= 27)
          oracle_basic_unary(out, in, n, act, alpha, 0.0f);
       else if (out != in)
          memmove(out, in, n * sizeof(float));
@@ -188,7 +195,7 @@ ORACLE_API void oracle_unary_chain(float *out, const float *in, size_t n, int co
    if (out != in)
       memmove(out, in, n * sizeof(float));
    for (int i = 0; i < count; ++i) {
-      if (op[i] >= 7 && op[i] <= 24)
+      if (op[i] >= 7 && op[i] <= 27)
          oracle_basic_unary(out, out, n, op[i], alpha[i], beta[i]);
       else
          oracle_unary(out, out, n, op[i], alpha[i]);

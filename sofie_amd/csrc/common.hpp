@@ -83,6 +83,9 @@ static __device__ __noinline__ float apply_basic_unary(float v, int act, float a
    case SOFIE_ACT_SELU: return beta * (fmaxf(0.0f, v) + fminf(0.0f, alpha * (expf(v) - 1.0f)));
    case SOFIE_ACT_ELU: return v >= 0.0f ? v : alpha * (expf(v) - 1.0f);
    case SOFIE_ACT_ERF: return erff(v);
+   case SOFIE_ACT_HARDSIGMOID: return fmaxf(0.0f, fminf(1.0f, alpha * v + beta));
+   case SOFIE_ACT_HARDSWISH: return v * fmaxf(0.0f, fminf(1.0f, 0x1.5555555555555p-3f * v + 0.5f));
+   case SOFIE_ACT_SWISH: return v / (1.0f + expf(-v));
    default: return v;
    }
 }

@@ -25,7 +25,7 @@ enum class ETensorType {
 // (EBasicUnaryOperator, core/inc/SOFIE/operators/ROperator_BasicUnary.hxx:11, and Clip)
 enum class EActivationType {
    UNDEFINED, RELU, LEAKYRELU, SIGMOID, GELU, GELU_TANH, TANH,
-   RECIPROCAL, SQRT, NEG, EXP, LOG, SIN, COS, ABS, SOFTPLUS, ATAN, FLOOR, ASINH, ACOSH, ATANH, CLIP, SELU, ELU, ERF
+   RECIPROCAL, SQRT, NEG, EXP, LOG, SIN, COS, ABS, SOFTPLUS, ATAN, FLOOR, ASINH, ACOSH, ATANH, CLIP, SELU, ELU, ERF, HARDSIGMOID, HARDSWISH, SWISH
 };
 enum class EBasicUnaryOperator { kReciprocal, kSqrt, kNeg, kExp, kLog, kSin, kCos, kAbs, kSoftplus, kAtan, kFloor, kAsinh, kAcosh, kAtanh };
 

@@ -156,6 +156,21 @@ template <typename T>
 struct ROperator_Erf : ROperator_Activation {
    ROperator_Erf(std::string x, std::string y) : ROperator_Activation(EActivationType::ERF, 0.f, x, y) {}
 };
+// HardSigmoid: max(0, min(1, alpha * x + beta)), alpha = 0.2, beta = 0.5 (core/inc/SOFIE/operators/ROperator_HardSigmoid.hxx:15-25, 71-74)
+template <typename T>
+struct ROperator_HardSigmoid : ROperator_Activation {
+   ROperator_HardSigmoid(float alpha, float beta, std::string x, std::string y) : ROperator_Activation(EActivationType::HARDSIGMOID, alpha, x, y, beta) {}
+};
+// HardSwish: x * max(0, min(1, x / 6 + 1 / 2)) (core/inc/SOFIE/operators/ROperator_HardSwish.hxx:56-60)
+template <typename T>
+struct ROperator_HardSwish : ROperator_Activation {
+   ROperator_HardSwish(std::string x, std::string y) : ROperator_Activation(EActivationType::HARDSWISH, 0.f, x, y) {}
+};
+// Swish: x / (1 + exp(-x)) (core/inc/SOFIE/operators/ROperator_Swish.hxx:54-56)
+template <typename T>
+struct ROperator_Swish : ROperator_Activation {
+   ROperator_Swish(std::string x, std::string y) : ROperator_Activation(EActivationType::SWISH, 0.f, x, y) {}
+};
 // Identity: a copy that the generator folds away wherever it follows another operator
 template <typename T>
 struct ROperator_Identity : ROperator_Activation {

@@ -39,6 +39,9 @@ inline const char *ActivationEnumName(EActivationType a)
    case EActivationType::SELU: return "SOFIE_ACT_SELU";
    case EActivationType::ELU: return "SOFIE_ACT_ELU";
    case EActivationType::ERF: return "SOFIE_ACT_ERF";
+   case EActivationType::HARDSIGMOID: return "SOFIE_ACT_HARDSIGMOID";
+   case EActivationType::HARDSWISH: return "SOFIE_ACT_HARDSWISH";
+   case EActivationType::SWISH: return "SOFIE_ACT_SWISH";
    default: return "SOFIE_ACT_NONE";
    }
 }

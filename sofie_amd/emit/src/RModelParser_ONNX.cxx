@@ -516,6 +516,12 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          model->AddOperator(std::make_unique<ROperator_Elu<float>>(attrF(n, "alpha", 1.0f), n.in[0], n.out[0]));
       } else if (n.op == "Erf") {
          model->AddOperator(std::make_unique<ROperator_Erf<float>>(n.in[0], n.out[0]));
+      } else if (n.op == "HardSigmoid") {      // parsers/src/ParseHardSigmoid.cxx:20-33
+         model->AddOperator(std::make_unique<ROperator_HardSigmoid<float>>(attrF(n, "alpha", 0.2f), attrF(n, "beta", 0.5f), n.in[0], n.out[0]));
+      } else if (n.op == "HardSwish") {
+         model->AddOperator(std::make_unique<ROperator_HardSwish<float>>(n.in[0], n.out[0]));
+      } else if (n.op == "Swish") {
+         model->AddOperator(std::make_unique<ROperator_Swish<float>>(n.in[0], n.out[0]));
       } else if (n.op == "Identity") {
          model->AddOperator(std::make_unique<ROperator_Identity<float>>(n.in[0], n.out[0]));
       } else if (n.op == "Clip") {

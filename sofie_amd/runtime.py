@@ -18,7 +18,7 @@ class SofieHipError(RuntimeError):
 
 # activation / bias / output codes of include/sofie_hip.h
 (ACT_NONE, ACT_RELU, ACT_LEAKYRELU, ACT_SIGMOID, ACT_GELU, ACT_GELU_TANH, ACT_TANH, ACT_RECIPROCAL, ACT_SQRT, ACT_NEG, ACT_EXP, ACT_LOG,
- ACT_SIN, ACT_COS, ACT_ABS, ACT_SOFTPLUS, ACT_ATAN, ACT_FLOOR, ACT_ASINH, ACT_ACOSH, ACT_ATANH, ACT_CLIP, ACT_SELU, ACT_ELU, ACT_ERF) = range(25)
+ ACT_SIN, ACT_COS, ACT_ABS, ACT_SOFTPLUS, ACT_ATAN, ACT_FLOOR, ACT_ASINH, ACT_ACOSH, ACT_ATANH, ACT_CLIP, ACT_SELU, ACT_ELU, ACT_ERF, ACT_HARDSIGMOID, ACT_HARDSWISH, ACT_SWISH) = range(28)
 MAX_POST_OPS = 4
 BIAS_NONE, BIAS_ROW, BIAS_COL, BIAS_SCALAR, BIAS_FULL = range(5)
 I8OUT_I32, I8OUT_F32, I8OUT_I8, I8OUT_I8_DQQ, I8OUT_I8_PLANE_SUMS = range(5)

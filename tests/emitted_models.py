@@ -192,6 +192,19 @@ def reduce_block(batch=3, named=None):
                 init=init, feeds=[X])
 
 
+def hard_activations(batch=4):
+    """Gemm -> HardSwish -> Gemm -> Swish -> HardSigmoid (non-default alpha / beta), and a Conv -> HardSwish on a second input: every one of them
+    rides in the store of the product before it."""
+    init = {"W1": util.normal(6701, 12 * 24, 0.6).reshape(12, 24), "b1": util.normal(6702, 24, 0.5), "W2": util.normal(6703, 24 * 5, 0.5).reshape(24, 5),
+            "b2": util.normal(6704, 5, 0.3), "K": util.normal(6705, 4 * 3 * 3 * 3, 0.5).reshape(4, 3, 3, 3)}
+    nodes = [ow.node("Gemm", ["X", "W1", "b1"], ["H"]), ow.node("HardSwish", ["H"], ["A"]), ow.node("Gemm", ["A", "W2", "b2"], ["L"]),
+             ow.node("Swish", ["L"], ["S"]), ow.node("HardSigmoid", ["S"], ["Y"], alpha=0.25, beta=0.4),
+             ow.node("Conv", ["Z", "K"], ["C"], kernel_shape=[3, 3], pads=[1, 1, 1, 1]), ow.node("HardSwish", ["C"], ["V"])]
+    X, Z = util.normal(6706, batch * 12, 1.5).reshape(batch, 12), util.normal(6707, batch * 3 * 6 * 6, 1.5).reshape(batch, 3, 6, 6)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 12]), ("Z", np.float32, [batch, 3, 6, 6])],
+                outputs=[("Y", np.float32, [batch, 5]), ("V", np.float32, [batch, 4, 6, 6])], init=init, feeds=[X, Z])
+
+
 def softmax_head(batch=4):
     """Gemm -> Softmax over the classes (one output)."""
     spec = classifier_head(batch)
@@ -638,7 +651,7 @@ def build_all(jobs=8):
         dynamic.append((m, p, len(spec["inputs"])))
     folded = reference_constant_folding_cases()
     multi = [("ElementwiseChains", elementwise_chains, 2), ("ParseRewrites", parse_rewrites, 3), ("ClassifierHead", classifier_head, 1),
-             ("LayerNormBlock", layernorm_block, 1), ("ReduceBlock", reduce_block, 1)]
+             ("LayerNormBlock", layernorm_block, 1), ("ReduceBlock", reduce_block, 1), ("HardActivations", hard_activations, 2)]
     multi += [(m, (lambda spec=spec: spec), len(spec["inputs"])) for m, spec in folded.items()]
     for m, spec in reference_stacked_matmul_cases().items():
         p = os.path.join(OUT, m + ".onnx")
@@ -666,7 +679,7 @@ def build_all(jobs=8):
         f.write(DYNAMIC_HARNESS % dict(model="ApiDynamicFp8Gemm", args="inputs[0]"))
     compile_shared(src, os.path.join(OUT, "libApiDynamicFp8Gemm.so"))
     compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
-    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead", "LayerNormBlock", "ReduceBlock"]
+    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead", "LayerNormBlock", "ReduceBlock", "HardActivations"]
 
 
 if __name__ == "__main__":

@@ -388,6 +388,12 @@ def run(g, inputs, be, all_outputs=False):
             y = be.chain(x[0], [(23, a.get("alpha", 1.0), 0.0)])
         elif op == "Erf":
             y = be.unary(x[0], 24, 0.0)
+        elif op == "HardSigmoid":
+            y = be.chain(x[0], [(25, a.get("alpha", 0.2), a.get("beta", 0.5))])
+        elif op == "HardSwish":
+            y = be.unary(x[0], 26, 0.0)
+        elif op == "Swish":
+            y = be.unary(x[0], 27, 0.0)
         elif op == "Identity":
             y = np.array(x[0], copy=True)
         elif op == "Clip":

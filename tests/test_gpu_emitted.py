@@ -276,6 +276,19 @@ def test_emitted_layernorm_block(rt):
     assert Y.std() > 0.05
 
 
+def test_emitted_hard_activations_ride_in_the_stores(rt):
+    spec = em.hard_activations(4)
+    g = onnx_lite.load(os.path.join(em.OUT, "HardActivations.onnx"))
+    Y, V = gr.run(g, spec["feeds"], gr.OracleBackend(), all_outputs=True)
+    print("emitted HardActivations", flush=True)
+    got = run_emitted("HardActivations", spec["feeds"], Y.size + V.size)
+    gy, gv = got[:Y.size].reshape(Y.shape), got[Y.size:].reshape(V.shape)
+    assert np.abs(gy - Y).max() <= 1e-5 and np.abs(gv - V).max() <= 1e-5 * max(1.0, float(np.abs(V).max()))
+    assert 0.0 <= Y.min() and Y.max() <= 1.0 and Y.std() > 0.05 and (V == 0).any() and V.max() > 3.0       # both clamps of HardSwish are reached
+    txt = open(os.path.join(em.OUT, "HardActivations_GPU_HIP.hxx")).read()
+    assert "sofie_hip_unary" not in txt and txt.count("SOFIE_ACT_HARDSWISH") == 2 and "SOFIE_ACT_SWISH" in txt and "SOFIE_ACT_HARDSIGMOID" in txt
+
+
 def test_emitted_reduce_block(rt):
     spec = em.reduce_block(3)
     X = spec["feeds"][0]

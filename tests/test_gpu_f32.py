@@ -344,6 +344,24 @@ def test_conv_with_a_residual_operand(rt):
     assert np.allclose(got, want, rtol=1e-5, atol=1e-5) and (got > 0).any() and (got == 0).any()
 
 
+def test_hard_sigmoid_hard_swish_and_swish(rt):
+    x = np.concatenate([util.normal(452, 1000 + 3, 2.5), np.array([-3.0, 3.0, -2.5, 2.5, 0.0, -0.0], np.float32)])
+    for ops, exact in [([(R.ACT_HARDSIGMOID, 0.2, 0.5)], True), ([(R.ACT_HARDSIGMOID, 0.37, 0.1)], True), ([(R.ACT_HARDSWISH, 0.0, 0.0)], True),
+                       ([(R.ACT_SWISH, 0.0, 0.0)], False), ([(R.ACT_SWISH, 0.0, 0.0), (R.ACT_HARDSWISH, 0.0, 0.0), (R.ACT_HARDSIGMOID, 0.2, 0.5)], False)]:
+        got, want = run_chain(rt, x, ops), ob.unary_chain(x, ops)
+        if exact:       # multiplications, additions and clamps only: the device computes the reference's bits
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), ops
+        else:
+            assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(1.0, np.abs(want))), ops
+    x64 = x.astype(np.float64)
+    assert np.allclose(run_chain(rt, x, [(R.ACT_SWISH, 0.0, 0.0)]), x64 / (1 + np.exp(-x64)), rtol=1e-5, atol=1e-6)
+    # the single-operator entry point takes the codes too (HardSigmoid's beta only through the chain)
+    dx, dy = util.to_dev(x), util.dev_empty(x.shape, np.float32)
+    rt.call("sofie_hip_unary_f32", util.ptr(dy), util.ptr(dx), C.c_size_t(x.size), R.ACT_HARDSWISH, C.c_float(0))
+    rt.sync()
+    assert np.array_equal(util.to_host(dy).view(np.uint32), ob.unary(x, R.ACT_HARDSWISH, 0.0).view(np.uint32))
+
+
 def test_selu(rt):
     x = util.normal(450, 1000 + 3, 2.0)
     alpha, gamma = 1.6732631921768188, 1.0507010221481323

@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 from oracle import binding as ob
+from sofie_amd import runtime as R
 from tests import util
 
 
@@ -550,3 +551,22 @@ def test_reduce_against_numpy_in_float64():
     # empty-product and start values: a reduced length of 1 returns the element (its square, its absolute value for L2)
     one = np.array([[-3.0]], np.float32)
     assert [float(ob.reduce(one, op, [1], 0)[0]) for op in range(7)] == [-3.0, -3.0, 9.0, -3.0, 3.0, -3.0, -3.0]
+
+
+def test_hard_sigmoid_hard_swish_and_swish_against_their_definitions():
+    x = np.concatenate([np.linspace(-8, 8, 1601), [-3.0, 3.0, -2.5, 2.5, 0.0]]).astype(np.float32)
+    x64 = x.astype(np.float64)
+    hs = ob.unary_chain(x, [(R.ACT_HARDSIGMOID, 0.2, 0.5)])
+    np.testing.assert_allclose(hs, np.clip(0.2 * x64 + 0.5, 0, 1), atol=1e-7)
+    assert hs[x <= -2.5].max() == 0.0 and hs[x >= 2.5].min() == 1.0 and hs[-1] == 0.5       # saturates exactly; 0 -> beta
+    other = ob.unary_chain(x, [(R.ACT_HARDSIGMOID, 0.5, 0.25)])                              # the attributes are used, not the defaults
+    np.testing.assert_allclose(other, np.clip(0.5 * x64 + 0.25, 0, 1), atol=1e-7)
+    hw = ob.unary_chain(x, [(R.ACT_HARDSWISH, 0.0, 0.0)])
+    np.testing.assert_allclose(hw, x64 * np.clip(x64 / 6 + 0.5, 0, 1), rtol=2e-7, atol=2e-7)
+    assert np.array_equal(hw[x >= 3], x[x >= 3]) and np.all(hw[x <= -3] == 0)                # identity above 3, zero below -3
+    sw = ob.unary_chain(x, [(R.ACT_SWISH, 0.0, 0.0)])
+    np.testing.assert_allclose(sw, x64 / (1 + np.exp(-x64)), rtol=3e-7, atol=1e-7)
+    # Swish is x * Sigmoid(x), and Swish(x) - Swish(-x) = x
+    sg = ob.unary(x, R.ACT_SIGMOID, 0.0)
+    np.testing.assert_allclose(sw, x * sg, rtol=3e-7, atol=1e-7)
+    np.testing.assert_allclose(sw - ob.unary_chain(-x, [(R.ACT_SWISH, 0.0, 0.0)]), x, atol=1e-6)
