@@ -70,6 +70,13 @@ int sofie_hip_sync(sofie_hip_ctx *ctx);                                      /* 
  * 4-byte elements.  copy_rows moves `rows` pieces of `row_bytes` bytes from a pitched source to a pitched destination (Concat
  * along an inner axis, ROperator_Concat.hxx: each input contributes one piece per outer index); pitches and row_bytes multiples of 4. */
 int sofie_hip_transpose_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t rank, const int64_t *shape, const int32_t *perm);
+/* The same kernel with the strides spelled out: Y[i_0, ..., i_{r-1}] = X[in_offset + sum_k i_k * in_strides[k]], Y dense of shape out_shape,
+ * rank <= 6, strides in elements (0 repeats an axis, a negative one walks it backwards).  It carries Slice (ROperator_Slice::Generate,
+ * core/inc/SOFIE/operators/ROperator_Slice.hxx: offset = sum start * stride, stride = step * stride), Split (ROperator_Split.hxx: one slice
+ * per output), Expand (ROperator_Expand.hxx: stride 0 on the broadcast axes) and Tile (ROperator_Tile.hxx: every axis seen as [repeat, length]
+ * with strides [0, stride]).  Every element read must lie inside [0, in_elements): checked on the host before the launch. */
+int sofie_hip_strided_gather_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t rank, const int64_t *out_shape, const int64_t *in_strides,
+                                 int64_t in_offset, int64_t in_elements);
 int sofie_hip_copy_rows(sofie_hip_ctx *ctx, void *dst_device, size_t dst_pitch_bytes, const void *src_device, size_t src_pitch_bytes, size_t rows,
                         size_t row_bytes);
 

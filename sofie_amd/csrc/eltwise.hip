@@ -657,6 +657,37 @@ int sofie_hip_transpose_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_
    return launch_status("transpose_f32_kernel");
 }
 
+int sofie_hip_strided_gather_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t rank, const int64_t *out_shape, const int64_t *in_strides,
+                                 int64_t in_offset, int64_t in_elements)
+{
+   SOFIE_HIP_REQUIRE(ctx && out_shape && in_strides, "sofie_hip_strided_gather_f32: NULL argument");
+   SOFIE_HIP_REQUIRE(rank >= 1 && rank <= 6, "sofie_hip_strided_gather_f32: rank %d not in [1,6]", rank);
+   SOFIE_HIP_REQUIRE(in_elements >= 0 && in_elements < (1LL << 40) && in_offset >= 0, "sofie_hip_strided_gather_f32: bad input size or offset");
+   TransposeShape sh;
+   sh.rank = rank;
+   size_t n = 1;
+   long long lo = in_offset, hi = in_offset; // the smallest and the largest input index the output reads
+   for (int k = 0; k < rank; ++k) {
+      SOFIE_HIP_REQUIRE(out_shape[k] >= 0 && out_shape[k] < (1LL << 40), "sofie_hip_strided_gather_f32: bad dimension");
+      SOFIE_HIP_REQUIRE(in_strides[k] > -(1LL << 40) && in_strides[k] < (1LL << 40), "sofie_hip_strided_gather_f32: bad stride");
+      n *= (size_t)out_shape[k];
+      SOFIE_HIP_REQUIRE(n < (1ULL << 40), "sofie_hip_strided_gather_f32: tensor too large");
+      sh.y[k] = out_shape[k];
+      sh.sx[k] = in_strides[k];
+   }
+   if (n == 0)
+      return SOFIE_HIP_OK;
+   for (int k = 0; k < rank; ++k) {
+      const double span = (double)(out_shape[k] - 1) * (double)in_strides[k];
+      SOFIE_HIP_REQUIRE(span > -1.0e15 && span < 1.0e15, "sofie_hip_strided_gather_f32: axis %d reaches outside the input", k);
+      (in_strides[k] < 0 ? lo : hi) += (long long)(out_shape[k] - 1) * in_strides[k];
+   }
+   SOFIE_HIP_REQUIRE(lo >= 0 && hi < in_elements, "sofie_hip_strided_gather_f32: reads elements %lld..%lld of an input of %lld", lo, hi, (long long)in_elements);
+   SOFIE_HIP_REQUIRE(Y && X, "sofie_hip_strided_gather_f32: NULL pointer");
+   hipLaunchKernelGGL(transpose_f32_kernel, dim3(grid_for(n)), dim3(256), 0, ctx->stream, Y, X + in_offset, n, sh);
+   return launch_status("transpose_f32_kernel");
+}
+
 int sofie_hip_copy_rows(sofie_hip_ctx *ctx, void *dst, size_t dst_pitch_bytes, const void *src, size_t src_pitch_bytes, size_t rows, size_t row_bytes)
 {
    SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_copy_rows: ctx is NULL");

@@ -699,6 +699,33 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
             auto f = n.attrs.find("axes");
             model->AddOperator(std::make_unique<ROperator_Reshape>(mode, f == n.attrs.end() ? std::vector<int64_t>{} : f->second.ints, n.in[0], n.out[0]));
          }
+      } else if (n.op == "Slice") {
+         // starts / ends / axes / steps are inputs from opset 10 on, attributes before (parsers/src/ParseSlice.cxx:19-47)
+         if (n.in.size() > 1) {
+            model->AddOperator(std::make_unique<ROperator_Slice<float, int64_t>>(n.in[0], std::vector<std::string>(n.in.begin() + 1, n.in.end()), n.out[0]));
+         } else {
+            auto ints = [&](const char *name) {
+               auto f = n.attrs.find(name);
+               return f == n.attrs.end() ? std::vector<int64_t>{} : f->second.ints;
+            };
+            model->AddOperator(std::make_unique<ROperator_Slice<float, int64_t>>(n.in[0], ints("starts"), ints("ends"), ints("axes"), n.out[0]));
+         }
+      } else if (n.op == "Split") {
+         for (auto &kv : n.attrs)
+            if (kv.first != "axis" && kv.first != "num_outputs")
+               throw std::runtime_error("SOFIE ONNX Parser Split operator: attribute" + kv.first + "is not yet supported");
+         model->AddOperator(std::make_unique<ROperator_Split>(n.in[0], n.in.size() > 1 ? n.in[1] : "", (int)attrI(n, "axis", 0), n.out));
+      } else if (n.op == "Expand" || n.op == "Tile") {
+         if (n.in.size() < 2)
+            throw std::runtime_error("SOFIE ONNX parser: " + n.op + " " + n.name + " needs its second input");
+         if (n.op == "Expand")
+            model->AddOperator(std::make_unique<ROperator_Expand<float>>(n.in[0], n.in[1], n.out[0]));
+         else
+            model->AddOperator(std::make_unique<ROperator_Tile<float>>(n.in[1], n.in[0], n.out[0]));
+      } else if (n.op == "Gather") {
+         if (n.in.size() < 2)
+            throw std::runtime_error("SOFIE ONNX parser: Gather " + n.name + " needs its indices");
+         model->AddOperator(std::make_unique<ROperator_Gather>(attrI(n, "axis", 0), n.in[0], n.in[1], n.out[0]));
       } else if (n.op == "Transpose") {
          auto f = n.attrs.find("perm");
          model->AddOperator(std::make_unique<ROperator_Transpose<float>>(f == n.attrs.end() ? std::vector<int64_t>{} : f->second.ints, n.in[0], n.out[0]));

@@ -130,6 +130,7 @@ SYMBOLS = {
     "sofie_hip_reduce_f32": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, C.c_int64, C.c_int32]),
     "sofie_hip_layernorm_f32": (C.c_int, [_P, _P, _P, _P, _P, C.c_int64, C.c_int32, C.c_float, _P, _P]),
     "sofie_hip_transpose_f32": (C.c_int, [_P, _P, _P, C.c_int32, _P, _P]),
+    "sofie_hip_strided_gather_f32": (C.c_int, [_P, _P, _P, C.c_int32, _P, _P, C.c_int64, C.c_int64]),
     "sofie_hip_copy_rows": (C.c_int, [_P, _P, C.c_size_t, _P, C.c_size_t, C.c_size_t, C.c_size_t]),
     "sofie_hip_binary_f32": (C.c_int, [_P, _P, C.c_int32, C.c_float]),
     "sofie_hip_softmax_f32": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, C.c_int64, C.c_int32]),

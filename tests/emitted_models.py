@@ -205,6 +205,21 @@ def hard_activations(batch=4):
                 outputs=[("Y", np.float32, [batch, 5]), ("V", np.float32, [batch, 4, 6, 6])], init=init, feeds=[X, Z])
 
 
+def indexing_block(batch=3, named=None):
+    """Split of [b, 6, 8] along the last axis into 3 + 3 + 2 columns (no sizes given: the last part is the short one), a Slice that walks the middle axis
+    backwards in steps of 2, a Gather of three rows (one counted from the end), a Tile of a part and an Expand of a gathered row; four outputs."""
+    b = named if named else batch
+    i64 = lambda *v: np.array(v, np.int64)
+    init = {"st": i64(-1, 1), "en": i64(-100, 7), "ax": i64(1, 2), "sp": i64(-2, 1), "idx": i64(4, -1, 0), "rep": i64(1, 2, 3), "one": i64(2), "shape": i64(1, 5, 8)}
+    nodes = [ow.node("Split", ["X"], ["A", "B", "Cc"], axis=-1), ow.node("Slice", ["X", "st", "en", "ax", "sp"], ["S"]),
+             ow.node("Gather", ["X", "idx"], ["G"], axis=1), ow.node("Tile", ["Cc", "rep"], ["T"]),
+             ow.node("Gather", ["X", "one"], ["R"], axis=1), ow.node("Expand", ["R", "shape"], ["E"]), ow.node("Add", ["A", "B"], ["AB"])]
+    X = util.normal(6801, batch * 48).reshape(batch, 6, 8)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [b, 6, 8])],
+                outputs=[("AB", np.float32, [b, 6, 3]), ("S", np.float32, [b, 3, 6]), ("G", np.float32, [b, 3, 8]), ("T", np.float32, [b, 12, 6]), ("E", np.float32, [b, 5, 8])],
+                init=init, feeds=[X])
+
+
 def softmax_head(batch=4):
     """Gemm -> Softmax over the classes (one output)."""
     spec = classifier_head(batch)
@@ -390,6 +405,7 @@ DYNAMIC_MODELS = {    "Dynamic_ResidualBlock": lambda: with_named_batch(residual
     "Dynamic_SoftmaxHead": lambda: with_named_batch(softmax_head(4), "N"),
     "Dynamic_ShapePlumbing": lambda: with_named_batch(shape_plumbing(3), "N"),
     "Dynamic_ReduceBlock": lambda: reduce_block(3, "N"),
+    "Dynamic_IndexingBlock": lambda: indexing_block(3, "N"),
     "Dynamic_int8_CNN_plane_sums": lambda: with_named_batch(int8_cnn(2, 16, (3, 64, 128)), "N"),
 }
 
@@ -651,7 +667,7 @@ def build_all(jobs=8):
         dynamic.append((m, p, len(spec["inputs"])))
     folded = reference_constant_folding_cases()
     multi = [("ElementwiseChains", elementwise_chains, 2), ("ParseRewrites", parse_rewrites, 3), ("ClassifierHead", classifier_head, 1),
-             ("LayerNormBlock", layernorm_block, 1), ("ReduceBlock", reduce_block, 1), ("HardActivations", hard_activations, 2)]
+             ("LayerNormBlock", layernorm_block, 1), ("ReduceBlock", reduce_block, 1), ("HardActivations", hard_activations, 2), ("IndexingBlock", indexing_block, 1)]
     multi += [(m, (lambda spec=spec: spec), len(spec["inputs"])) for m, spec in folded.items()]
     for m, spec in reference_stacked_matmul_cases().items():
         p = os.path.join(OUT, m + ".onnx")
@@ -679,7 +695,7 @@ def build_all(jobs=8):
         f.write(DYNAMIC_HARNESS % dict(model="ApiDynamicFp8Gemm", args="inputs[0]"))
     compile_shared(src, os.path.join(OUT, "libApiDynamicFp8Gemm.so"))
     compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
-    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead", "LayerNormBlock", "ReduceBlock", "HardActivations"]
+    return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead", "LayerNormBlock", "ReduceBlock", "HardActivations", "IndexingBlock"]
 
 
 if __name__ == "__main__":

@@ -21,12 +21,12 @@ NUM = r"[-+]?(?:\d+\.?\d*|\.\d+)(?:[eE][-+]?\d+)?"
 
 
 def arrays_in(path):
-    """{name: [floats]} for every `float name[...] = {...};` in a C++ header."""
+    """{name: [floats]} for every `float name[...] = {...};` and `std::vector<float> name = {...};` in a C++ header."""
     text = open(path).read()
     out = {}
-    for m in re.finditer(r"float\s+(\w+)\s*\[[^\]]*\]\s*=\s*\{(.*?)\}\s*;", text, re.S):
-        body = re.sub(r"//[^\n]*", "", m.group(2))
-        out[m.group(1)] = [float(x) for x in re.findall(NUM, re.sub(r"(?<=[\d.])f\b", "", body))]
+    for m in re.finditer(r"(?:float\s+(\w+)\s*\[[^\]]*\]|std::vector<float>\s+(\w+))\s*=\s*\{(.*?)\}\s*;", text, re.S):
+        body = re.sub(r"//[^\n]*", "", m.group(3))
+        out[m.group(1) or m.group(2)] = [float(x) for x in re.findall(NUM, re.sub(r"(?<=[\d.])f\b", "", body))]
     return out
 
 
@@ -155,6 +155,19 @@ def main():
         os.chmod(os.path.join(HERE, "models", model + ".onnx"), 0o644)
         fixtures[model] = {"inputs": test_inputs_table(gen, model), "expected": arrays_in(os.path.join(REF, "models/onnx/references", model + ".hxx"))["output"],
                            "source": "tests/models/onnx/%s.onnx + references/%s.hxx" % (model, model)}
+    for model in ("ExpandSameSize", "ExpandDiffSize", "Tile5D", "Gather2d", "GatherAxis0", "GatherAxis1", "GatherAxis2", "GatherAxis3", "GatherNegativeIndices"):
+        inputs = test_inputs_table(gen, model)
+        if inputs is None:
+            raise RuntimeError("no literal inputs for " + model)
+        add(model, next(iter(arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx")).values())), inputs)
+    # Slice: input and output side by side in the .ref.hxx.  The reference's tests reach them through the namespace inside the file, and two of
+    # the files hold each other's namespace (Slice_Neg.ref.hxx declares Slice_Default_Steps and the reverse): the namespace names the model.
+    for name in ("Slice", "Slice_Default_Axis", "Slice_Default_Steps", "Slice_Neg"):
+        path = os.path.join(REF, "models/onnx/references", name + ".ref.hxx")
+        model = re.search(r"namespace\s+(\w+)", open(path).read()).group(1)
+        arrays = arrays_in(path)
+        add(model, arrays["output"], [{"kind": "values", "values": arrays["input"]}])
+        fixtures[model]["source"] = "tests/models/onnx/%s.onnx + references/%s.ref.hxx (namespace %s)" % (model, name, model)
     red = os.path.join(REF, "alpaka/TestAlpakaReduce.cxx")
     for model, var in (("ReduceMean", "input"), ("ReduceProd", "input"), ("ReduceL2", "input"), ("ReduceMax", "input"), ("ReduceMax_axis0", "vals"),
                        ("ReduceMax_mid", "vals")):

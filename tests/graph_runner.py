@@ -113,6 +113,13 @@ class OracleBackend:
     def transpose(self, X, perm):
         return np.ascontiguousarray(np.transpose(X, perm))
 
+    def view(self, X, v):
+        """`v`, a numpy view of X (a slice, a broadcast), as a dense tensor"""
+        return np.ascontiguousarray(v)
+
+    def take(self, X, indices, axis):
+        return np.ascontiguousarray(np.take(X, indices, axis=axis))
+
     def concat(self, xs, axis):
         return np.ascontiguousarray(np.concatenate(xs, axis=axis))
 
@@ -251,6 +258,44 @@ class HipBackend:
         self.rt.sync()
         return u.to_host(dY)
 
+    def view(self, X, v):
+        """The strided read that makes the numpy view `v` of the contiguous X dense: shape, element strides and offset are the view's own."""
+        import torch
+        u = self.u
+        assert X.flags["C_CONTIGUOUS"] and X.dtype == np.float32 and v.dtype == np.float32
+        dims = [(d, s // 4) for d, s in zip(v.shape, v.strides) if d != 1] or [(1, 0)]       # axes of one element carry no stride
+        i = 0
+        while i + 1 < len(dims):        # neighbours that walk the input in one stride fold into one axis, as in the emitted Tile
+            if dims[i][1] == dims[i + 1][0] * dims[i + 1][1]:
+                dims[i:i + 2] = [(dims[i][0] * dims[i + 1][0], dims[i + 1][1])]
+            else:
+                i += 1
+        assert len(dims) <= 6
+        offset = (v.__array_interface__["data"][0] - X.__array_interface__["data"][0]) // 4
+        shape = (C.c_int64 * 6)(*([d for d, _ in dims] + [1] * (6 - len(dims))))
+        strides = (C.c_int64 * 6)(*([s for _, s in dims] + [0] * (6 - len(dims))))
+        dX, dY = u.to_dev(X), u.dev_empty(v.shape, np.float32)
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_strided_gather_f32", u.ptr(dY), u.ptr(dX), len(dims), shape, strides, offset, X.size)
+        self.rt.sync()
+        return u.to_host(dY)
+
+    def take(self, X, indices, axis):
+        """one pitched copy per index, as the emitted Gather makes them"""
+        import torch
+        u = self.u
+        X = np.ascontiguousarray(X, dtype=np.float32)
+        idx = np.asarray(indices, dtype=np.int64)
+        flat = [int(i) + X.shape[axis] if i < 0 else int(i) for i in idx.ravel()]
+        outer, inner = int(np.prod(X.shape[:axis], dtype=np.int64)), int(np.prod(X.shape[axis + 1:], dtype=np.int64))
+        dX, dY = u.to_dev(X), u.dev_empty(X.shape[:axis] + idx.shape + X.shape[axis + 1:], np.float32)
+        torch.cuda.synchronize()
+        for k, i in enumerate(flat):
+            self.rt.call("sofie_hip_copy_rows", C.c_void_p(u.ptr(dY).value + k * inner * 4), C.c_size_t(len(flat) * inner * 4),
+                         C.c_void_p(u.ptr(dX).value + i * inner * 4), C.c_size_t(X.shape[axis] * inner * 4), C.c_size_t(outer), C.c_size_t(inner * 4))
+        self.rt.sync()
+        return u.to_host(dY)
+
     def concat(self, xs, axis):
         import torch
         u = self.u
@@ -382,6 +427,44 @@ def run(g, inputs, be, all_outputs=False):
             y = be.transpose(x[0], a.get("perm", list(range(x[0].ndim))[::-1]))
         elif op == "Concat":
             y = be.concat(x, a.get("axis", 0))
+        elif op == "Slice":
+            X = np.ascontiguousarray(x[0], dtype=np.float32)
+            par = [[int(v) for v in np.asarray(t).ravel()] if t is not None else None for t in x[1:]] if len(x) > 1 else [a["starts"], a["ends"], a.get("axes")]
+            par += [None] * (4 - len(par))
+            starts, ends, axes, steps = par[0], par[1], par[2] or list(range(len(par[0]))), par[3] or [1] * len(par[0])
+            sl = [slice(None)] * X.ndim
+            for s, e, ax, st in zip(starts, ends, axes, steps):       # Python's slices clamp as ONNX's do; an end below -dim means "to the front"
+                d = X.shape[ax]
+                sl[ax] = slice(max(s, -d) if st > 0 else s, None if (st < 0 and e < -d) else e, st)
+            y = be.view(X, X[tuple(sl)])
+        elif op == "Split":
+            X = np.ascontiguousarray(x[0], dtype=np.float32)
+            ax = a.get("axis", 0) % X.ndim
+            k = len(n["outputs"])
+            if len(x) > 1 and x[1] is not None:
+                sizes = [int(v) for v in np.asarray(x[1]).ravel()]
+            else:
+                per = -(-X.shape[ax] // k)
+                sizes = [per] * (k - 1) + [X.shape[ax] - per * (k - 1)]
+            start = 0
+            for name, sz in zip(n["outputs"], sizes):
+                sl = [slice(None)] * X.ndim
+                sl[ax] = slice(start, start + sz)
+                env[name] = be.view(X, X[tuple(sl)])
+                start += sz
+            continue
+        elif op == "Expand":
+            X = np.ascontiguousarray(x[0], dtype=np.float32)
+            target = np.broadcast_shapes(X.shape, tuple(int(v) for v in np.asarray(x[1]).ravel()))
+            y = be.view(X, np.broadcast_to(X, target))
+        elif op == "Tile":
+            X = np.ascontiguousarray(x[0], dtype=np.float32)
+            reps = [int(v) for v in np.asarray(x[1]).ravel()]
+            pairs = np.broadcast_to(X.reshape([v for d in X.shape for v in (1, d)]), [v for r, d in zip(reps, X.shape) for v in (r, d)])
+            y = be.view(X, pairs).reshape([r * d for r, d in zip(reps, X.shape)])
+            assert np.array_equal(y, np.tile(X, reps)) or not isinstance(be, OracleBackend)
+        elif op == "Gather":
+            y = be.take(np.ascontiguousarray(x[0], dtype=np.float32), np.asarray(x[1]), a.get("axis", 0) % np.ndim(x[0]))
         elif op == "Selu":
             y = be.chain(x[0], [(22, a.get("alpha", 1.6732631921768188), a.get("gamma", 1.0507010221481323))])
         elif op == "Elu":

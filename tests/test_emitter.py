@@ -504,3 +504,24 @@ def test_reduce_shapes_axes_and_refusals(tmp_path):
     assert r.returncode != 0 and "invalid axes values 3" in r.stdout
     r = _emit(tmp_path, [ow.node("ReduceL2", ["X", "A"], ["Y"])], [("X", f, [2, 3]), ("A", np.int64, [1])], [("Y", f, [2, 1])], {}, name="runtime_axes")
     assert r.returncode != 0 and "int64 initializer" in r.stdout
+
+
+def test_indexing_operators_shapes_and_refusals(tmp_path):
+    f, i64 = np.float32, lambda *v: np.array(v, np.int64)
+    # Slice before opset 10 (attributes), ends beyond the axis clamp; Split in unequal parts; Gather with a scalar index drops the axis
+    r = _emit(tmp_path, [ow.node("Slice", ["X"], ["S"], starts=[1], ends=[1000], axes=[1]), ow.node("Split", ["X", "parts"], ["A", "B"], axis=0),
+                         ow.node("Gather", ["X", "i"], ["G"], axis=1)],
+              [("X", f, [4, 5])], [("S", f, [4, 4]), ("A", f, [1, 5]), ("B", f, [3, 5]), ("G", f, [4])], {"parts": i64(1, 3), "i": np.array(3, np.int64)}, name="idx")
+    assert r.returncode == 0, r.stdout
+    txt = open(os.path.join(str(tmp_path), "idx_GPU_HIP.hxx")).read()
+    assert "shape[6] = {4, 4, 1, 1, 1, 1}" in txt and "strides, 1, 20)" in txt and "strides, 5, 20)" in txt and "+ 12, 20, 4, 4)" in txt
+    for nodes, init, words in [
+            ([ow.node("Slice", ["X", "s", "e"], ["Y"])], {"s": i64(2), "e": i64(2)}, "empty"),
+            ([ow.node("Slice", ["X", "s", "e", "a", "t"], ["Y"])], {"s": i64(0), "e": i64(2), "a": i64(0), "t": i64(0)}, "step 0"),
+            ([ow.node("Split", ["X", "p"], ["Y", "Z"])], {"p": i64(1, 2)}, "Sum of split sizes"),
+            ([ow.node("Expand", ["X", "p"], ["Y"])], {"p": i64(3, 5)}, "cannot be broadcast"),
+            ([ow.node("Tile", ["X", "p"], ["Y"])], {"p": i64(2)}, "one repeat per axis"),
+            ([ow.node("Gather", ["X", "p"], ["Y"])], {"p": i64(4)}, "index 4 is out of range"),
+            ([ow.node("Gather", ["X", "X2"], ["Y"])], {}, "int64 initializer")]:
+        r = _emit(tmp_path, nodes, [("X", f, [4, 5]), ("X2", f, [4, 5])], [("Y", f, [4, 5])], init, name="bad")
+        assert r.returncode != 0 and words in r.stdout, (words, r.stdout)

@@ -170,6 +170,17 @@ def test_dynamic_reduce_block_keeps_or_consumes_the_batch(rt):
             assert got.size == want.size == n * 10 + 24 and np.array_equal(got, want)
 
 
+def test_dynamic_indexing_block(rt):
+    from tests.test_gpu_emitted import indexing_block_expected
+    x = np.concatenate([em.indexing_block(3)["feeds"][0], util.normal(8307, 2 * 48).reshape(2, 6, 8)])
+    with DynamicSession("Dynamic_IndexingBlock", 5) as s:
+        for n in (5, 2, 1):
+            want = indexing_block_expected(x[:n])
+            print("Dynamic_IndexingBlock batch", n, flush=True)
+            got = s.infer(n, [x[:n]], want.size)
+            assert got.size == want.size and np.array_equal(got, want)
+
+
 def test_dynamic_softmax_head(rt):
     spec = em.softmax_head(4)
     g = onnx_lite.load(os.path.join(em.OUT, "ClassifierHead.onnx"))     # the same weights with a fixed batch

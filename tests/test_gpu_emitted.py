@@ -289,6 +289,27 @@ def test_emitted_hard_activations_ride_in_the_stores(rt):
     assert "sofie_hip_unary" not in txt and txt.count("SOFIE_ACT_HARDSWISH") == 2 and "SOFIE_ACT_SWISH" in txt and "SOFIE_ACT_HARDSIGMOID" in txt
 
 
+def indexing_block_expected(X):
+    """numpy's own indexing, output after output"""
+    A, B, Cc = X[:, :, 0:3], X[:, :, 3:6], X[:, :, 6:8]
+    S = X[:, ::-2, 1:7]
+    G = X[:, [4, -1, 0], :]
+    T = np.tile(Cc, (1, 2, 3))
+    E = np.broadcast_to(X[:, [2], :], (X.shape[0], 5, 8))
+    return np.concatenate([np.ascontiguousarray(v, dtype=np.float32).ravel() for v in (A + B, S, G, T, E)])
+
+
+def test_emitted_indexing_block(rt):
+    spec = em.indexing_block(3)
+    want = indexing_block_expected(spec["feeds"][0])
+    print("emitted IndexingBlock", flush=True)
+    got = run_emitted("IndexingBlock", spec["feeds"], want.size)
+    assert want.size == 3 * (18 + 18 + 24 + 72 + 40) and np.array_equal(got, want)
+    g = onnx_lite.load(os.path.join(em.OUT, "IndexingBlock.onnx"))
+    outs = gr.run(g, spec["feeds"], gr.OracleBackend(), all_outputs=True)      # the graph runner's reading of the same operators agrees
+    assert np.array_equal(np.concatenate([o.ravel() for o in outs]), want)
+
+
 def test_emitted_reduce_block(rt):
     spec = em.reduce_block(3)
     X = spec["feeds"][0]
