@@ -23,15 +23,26 @@ __global__ __launch_bounds__(256) void quantize_linear_kernel(int8_t *__restrict
    const size_t stride = (size_t)gridDim.x * blockDim.x;
    size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
    if (vec) {
+      // four 16-byte loads per lane are issued before the first is used (a lane's pieces lie a workgroup's width apart, so every
+      // wave instruction reads and writes whole lines): the kernel is a single round trip to memory, and a quarter of the waves run it
       const size_t n4 = n / 4;
-      for (; i < n4; i += stride) {
-         float4 v = ((const float4 *)src)[i];
-         int q0 = quantize_rne_sat8(__fdiv_rn(v.x, scale));
-         int q1 = quantize_rne_sat8(__fdiv_rn(v.y, scale));
-         int q2 = quantize_rne_sat8(__fdiv_rn(v.z, scale));
-         int q3 = quantize_rne_sat8(__fdiv_rn(v.w, scale));
-         ((uint32_t *)dst)[i] = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) |
-                                ((uint32_t)(q3 & 0xff) << 24);
+      for (size_t base = blockIdx.x * (size_t)blockDim.x * 4 + threadIdx.x; base < n4; base += stride * 4) {
+         float4 v[4];
+#pragma unroll
+         for (int j = 0; j < 4; ++j) {
+            const size_t k = base + (size_t)j * blockDim.x;
+            v[j] = k < n4 ? ((const float4 *)src)[k] : make_float4(0.f, 0.f, 0.f, 0.f);
+         }
+#pragma unroll
+         for (int j = 0; j < 4; ++j) {
+            const size_t k = base + (size_t)j * blockDim.x;
+            int q0 = quantize_rne_sat8(__fdiv_rn(v[j].x, scale));
+            int q1 = quantize_rne_sat8(__fdiv_rn(v[j].y, scale));
+            int q2 = quantize_rne_sat8(__fdiv_rn(v[j].z, scale));
+            int q3 = quantize_rne_sat8(__fdiv_rn(v[j].w, scale));
+            if (k < n4)
+               ((uint32_t *)dst)[k] = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) | ((uint32_t)(q3 & 0xff) << 24);
+         }
       }
       i = n4 * 4 + (blockIdx.x * (size_t)blockDim.x + threadIdx.x);
       if (i < n)
@@ -468,7 +479,7 @@ int sofie_hip_quantize_linear(sofie_hip_ctx *ctx, int8_t *dst, const float *src,
    SOFIE_HIP_REQUIRE(dst && src, "sofie_hip_quantize_linear: NULL pointer");
    SOFIE_HIP_REQUIRE(scale > 0.0f, "sofie_hip_quantize_linear: scale must be positive");
    const int vec = (((uintptr_t)src & 15) == 0) && (((uintptr_t)dst & 3) == 0);
-   hipLaunchKernelGGL(quantize_linear_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(256), 0, ctx->stream, dst, src, n, scale, vec);
+   hipLaunchKernelGGL(quantize_linear_kernel, dim3(grid_for(vec ? (n + 15) / 16 : n)), dim3(256), 0, ctx->stream, dst, src, n, scale, vec);
    return launch_status("quantize_linear_kernel");
 }
 

@@ -21,3 +21,14 @@ def rt():
     r = Runtime(0)
     yield r
     r.close()
+
+
+@pytest.fixture(scope="session", autouse=True)
+def _torch_initialises_the_gpu_first(request):
+    """torch brings its own copy of the HIP runtime: whichever of torch and libsofie_hip.so touches the GPU first decides which copy the process uses.
+    The GPU tests share device memory between the two, so torch goes first whatever test file happens to run first."""
+    if any(item.get_closest_marker("gpu") for item in request.session.items):
+        import torch
+        if torch.cuda.is_available():
+            torch.cuda.init()
+    yield
