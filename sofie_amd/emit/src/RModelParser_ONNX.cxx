@@ -163,6 +163,7 @@ struct Attr {
    int64_t i = 0;
    float f = 0;
    std::vector<int64_t> ints;
+   Slice tensor; // a TensorProto (the `value` of a Constant node), inside the file's buffer
    bool has_i = false, has_f = false, has_s = false;
 };
 
@@ -194,6 +195,7 @@ Node ParseNode(Slice s)
             case 2: a.f = AsFloat((uint32_t)g.v); a.has_f = true; break;
             case 3: a.i = (int64_t)g.v; a.has_i = true; break;
             case 4: a.s = Str(g.bytes); a.has_s = true; break;
+            case 5: a.tensor = g.bytes; break;
             case 8:
                for (auto v : PackedInts(g))
                   a.ints.push_back(v);
@@ -302,6 +304,36 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          else if (f.no == 12)
             outputs.push_back(ParseValueInfo(f.bytes));
       }
+   }
+   // A Constant node is an initializer under its output's name (the reference registers it as one when parsing,
+   // parsers/src/ParseConstant.cxx): exporters write the shapes, axes and indices of Reshape / Slice / Gather this way.
+   for (auto it = nodes.begin(); it != nodes.end();) {
+      if (it->op != "Constant") {
+         ++it;
+         continue;
+      }
+      if (it->out.size() != 1)
+         throw std::runtime_error("SOFIE ONNX parser: Constant " + it->name + " must have one output");
+      Tensor t;
+      auto has = [&](const char *a) { return it->attrs.count(a) != 0; };
+      if (has("value") && it->attrs["value"].tensor.p) {
+         t = ParseTensor(it->attrs["value"].tensor);
+      } else if (has("value_float")) {
+         t.dtype = static_cast<int>(ETensorType::FLOAT);
+         t.floats = {it->attrs["value_float"].f};
+      } else if (has("value_int")) {
+         t.dtype = static_cast<int>(ETensorType::INT64);
+         t.ints = {it->attrs["value_int"].i};
+      } else if (has("value_ints")) {
+         t.dtype = static_cast<int>(ETensorType::INT64);
+         t.ints = it->attrs["value_ints"].ints;
+         t.dims = {t.ints.size()};
+      } else {
+         throw std::runtime_error("SOFIE ONNX parser: Constant " + it->name + " has no value, value_float, value_int or value_ints attribute");
+      }
+      t.name = it->out[0];
+      inits.push_back(std::move(t));
+      it = nodes.erase(it);
    }
    auto model = std::make_unique<RModel>(modelName.empty() ? filename : modelName);
    std::map<std::string, bool> isInit;

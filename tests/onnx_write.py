@@ -48,6 +48,8 @@ def attribute(name, value):
         a += _vi(3, value) + _vi(20, 2)
     elif isinstance(value, str):
         a += _ld(4, value.encode()) + _vi(20, 3)
+    elif isinstance(value, np.ndarray):      # a tensor attribute (the value of a Constant node)
+        a += _ld(5, tensor("", value)) + _vi(20, 4)
     else:
         a += b"".join(_vi(8, int(v)) for v in value) + _vi(20, 7)
     return a

@@ -525,3 +525,25 @@ def test_indexing_operators_shapes_and_refusals(tmp_path):
             ([ow.node("Gather", ["X", "X2"], ["Y"])], {}, "int64 initializer")]:
         r = _emit(tmp_path, nodes, [("X", f, [4, 5]), ("X2", f, [4, 5])], [("Y", f, [4, 5])], init, name="bad")
         assert r.returncode != 0 and words in r.stdout, (words, r.stdout)
+
+
+def test_constant_nodes_become_initializers(tmp_path):
+    """Exporters hand Reshape its shape, Slice its bounds and a Gemm its weights through Constant nodes: the parser registers each as an initializer
+    under the node's output name (parsers/src/ParseConstant.cxx), so the emitted code equals that of the same graph with initializers."""
+    f = np.float32
+    W = np.arange(12, dtype=f).reshape(4, 3)
+    nodes = [ow.node("Constant", [], ["W"], value=W), ow.node("Constant", [], ["shape"], value=np.array([2, 6], np.int64)),
+             ow.node("Constant", [], ["st"], value_ints=[1]), ow.node("Constant", [], ["en"], value_ints=[3]),
+             ow.node("MatMul", ["X", "W"], ["Y"]), ow.node("Reshape", ["Y", "shape"], ["R"]), ow.node("Slice", ["R", "st", "en"], ["S"])]
+    r = _emit(tmp_path, nodes, [("X", f, [4, 4])], [("S", f, [1, 6])], {}, name="viaconst")
+    assert r.returncode == 0, r.stdout
+    a = open(os.path.join(str(tmp_path), "viaconst_GPU_HIP.hxx")).read()
+    same = [n for n in nodes if n not in nodes[:4]]
+    r = _emit(tmp_path, same, [("X", f, [4, 4])], [("S", f, [1, 6])], {"W": W, "shape": np.array([2, 6], np.int64), "st": np.array([1], np.int64), "en": np.array([3], np.int64)},
+              name="viainit")
+    assert r.returncode == 0, r.stdout
+    b = open(os.path.join(str(tmp_path), "viainit_GPU_HIP.hxx")).read()
+    assert ops_body(a) == ops_body(b) and "sofie_hip_strided_gather_f32" in a and "strides, 6, 12)" in a
+    assert open(os.path.join(str(tmp_path), "viaconst_GPU_HIP.dat")).read().split()[-12:] == open(os.path.join(str(tmp_path), "viainit_GPU_HIP.dat")).read().split()[-12:]
+    r = _emit(tmp_path, [ow.node("Constant", [], ["W"]), ow.node("Relu", ["X"], ["Y"])], [("X", f, [4])], [("Y", f, [4])], {}, name="novalue")
+    assert r.returncode != 0 and "has no value" in r.stdout
