@@ -51,6 +51,8 @@ struct I8Epilogue {
             atomicAdd(dst + e, s[e]);
    }
    __device__ __forceinline__ bool rows_vectorizable() const { return stage_ok != 0; }
+   // row-major output with 16-byte aligned rows, every element stored (what the register tile store handles)
+   bool stores_plain_rows() const { return stage_ok != 0 && nchw_ohw == 0 && rows_per_plane == 0; }
    __device__ __forceinline__ char *out_base() const { return (char *)Y; }
    __device__ __forceinline__ size_t out_index(int m, int n) const
    {
@@ -107,6 +109,13 @@ struct I8Epilogue {
             p.s[i] = scale ? scale[nn] : scale_scalar;
          }
       }
+   }
+
+   // bias and scale of the single column n (n < N)
+   __device__ __forceinline__ void load_column(int n, int &b, float &sc) const
+   {
+      b = bias ? bias[n + n_offset] : 0;
+      sc = scale ? scale[n + n_offset] : scale_scalar;
    }
 
    // converts columns 4q..4q+3 of the lane's columns (exact int32 dot products) into 4*out_bytes() bytes

@@ -33,12 +33,38 @@ struct MfmaI8 {
    typedef int elem_t;
    static constexpr int KSTEP = 32; // K bytes per MFMA
    static constexpr int CHUNKS = 1; // 16-byte chunks per lane and operand
+   static constexpr int ROWS = 32;  // rows (and columns) of the output block; lane = lk * ROWS + row
+   static constexpr int LK = 2;     // lanes that share a row
+   static constexpr int ACC = 16;   // accumulator registers per lane
    struct frag_t {
       v4i c[1];
    };
    static __device__ __forceinline__ acc_t mma(const frag_t &a, const frag_t &b, acc_t c)
    {
       return __builtin_amdgcn_mfma_i32_32x32x32_i8(a.c[0], b.c[0], c, 0, 0, 0);
+   }
+};
+
+// int8 with 16 x 16 output blocks: v_mfma_i32_16x16x64_i8, 16 bytes of K per lane and step, four lanes per row.  Per multiply-add
+// it moves half as many accumulator registers as the 32 x 32 form; under the board's power limit (operands that toggle)
+// it sustains about a sixth more, provided two waves share the SIMD (one wave alone cannot issue it back to back).
+struct MfmaI8x16 {
+   typedef v4i acc_t;
+   typedef int elem_t;
+   static constexpr int KSTEP = 64;
+   static constexpr int CHUNKS = 1;
+   static constexpr int ROWS = 16;
+   static constexpr int LK = 4;
+   static constexpr int ACC = 4;
+   // XOR applied to the chunk index of row r in a slab of 64-byte rows so that this instruction's fragment read (lane = lk*16 + row,
+   // chunk lk) is free of bank conflicts: measured 240 B/clk per CU against 126 B/clk with the (r/4)%4 of the 32-row fragments
+   static __device__ __forceinline__ int lds_swizzle(int r) { return (r >> 1) & 3; }
+   struct frag_t {
+      v4i c[1];
+   };
+   static __device__ __forceinline__ acc_t mma(const frag_t &a, const frag_t &b, acc_t c)
+   {
+      return __builtin_amdgcn_mfma_i32_16x16x64_i8(a.c[0], b.c[0], c, 0, 0, 0);
    }
 };
 
@@ -49,6 +75,9 @@ struct MfmaF8 {
    typedef float elem_t;
    static constexpr int KSTEP = 64;
    static constexpr int CHUNKS = 2;
+   static constexpr int ROWS = 32;
+   static constexpr int LK = 2;
+   static constexpr int ACC = 16;
    struct frag_t {
       v4i c[2];
    };

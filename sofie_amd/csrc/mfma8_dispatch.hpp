@@ -1,6 +1,6 @@
 // Kernel choice for the int8 / FP8 GEMM and the int8 convolution: which tile, which pipelined kernel, or the general one.
 #pragma once
-#include "mfma8_gemm_pair.hpp"
+#include "mfma8_gemm_persist.hpp"
 
 namespace sofie_hip {
 
@@ -16,6 +16,10 @@ static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *
    const int tile = pick_tile(M, N, force_tile);
    const bool k128 = (K % 128 == 0);
    if constexpr (MMA::KSTEP * 2 <= 64) {
+      // Large products that divide into whole 256 x 256 tiles: the persistent kernel (512 asks for it by force)
+      if ((force_tile == 512 || (!force_tile && variant == 0 && tile == 256)) && mfma8_persist_applies(A, Bt, M, N, K, lda, ldb) &&
+          ep.stores_plain_rows())
+         return launch_mfma8_persist<MfmaI8x16, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
       // Short reductions over many tiles: the 256 x 128 tile with a ring of three slabs fits twice on a CU, and one
       // workgroup's prologue and store overlap the other's K loop (8192 x 4096 x 512: 829 -> 1019 TOP/s, 8192 x 1024 x 1024:
       // 1003 -> 1091; no gain from K = 2048 on).  258 asks for it by force.
@@ -78,6 +82,12 @@ static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *
             return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 128>(stream, A, Bt, M, N, K, lda, ldb, ep);
          if (variant == 38)
             return launch_mfma8_pair<MMA, 256, 256, 64, 2, 2, 5, EPI, 19>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 61)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 4, 5, EPI, 0>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 62)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 4, 2, 5, EPI, 0>(stream, A, Bt, M, N, K, lda, ldb, ep);
+         if (variant == 63)
+            return launch_mfma8_pair<MMA, 256, 256, 64, 2, 4, 5, EPI, 16>(stream, A, Bt, M, N, K, lda, ldb, ep);
 #endif
          if (variant == 1 || !k128)
             return launch_mfma8_dma<MMA, 256, 256, 64, 2, 2, 4, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);

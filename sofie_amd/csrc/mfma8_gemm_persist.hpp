@@ -1,0 +1,325 @@
+// Persistent tile loop of the int8 / FP8 GEMM for large shapes that divide evenly into 256 x 256 tiles.
+//
+// One workgroup of EIGHT waves per CU (two per SIMD, 256 registers each) walks a list of output tiles; the K loop runs
+// straight through the tile boundaries:
+//   * the ring of five 64-byte K slabs (paired as in mfma8_gemm_pair.hpp: the two halves of a 128-byte line are
+//     requested back to back) never drains: while the last slabs of a tile are multiplied, the first slabs of the
+//     workgroup's next tile are already landing;
+//   * a wave owns a 128 x 64 piece of the tile (128 accumulator registers), so two waves share a SIMD: while one waits
+//     (barrier, LDS, the tile store), the matrix core runs the other's MFMAs;
+//   * the tile store needs no LDS (the ring takes all 160 KB): the lanes exchange the converted elements through
+//     v_permlane16_swap / v_permlane32_swap until every lane holds 16 consecutive output bytes, and store them.
+//
+// Step t of the loop multiplies slab t (its fragments are in registers) while the fragments of slab t + 1 are read from
+// LDS into the other register buffer, and, on even t, the eight loads of the pair of slabs t + 4, t + 5 are issued.
+// One workgroup barrier opens each step.  Before it a wave has waited for its own LDS reads of slab t (so after the
+// barrier the ring slot of slab t may be overwritten: that is where slab t + 5 goes) and, on odd t, for its own loads
+// of the pair that starts at slab t + 1 (so after the barrier that pair is complete for every wave).
+#pragma once
+#include "mfma8_gemm_pair.hpp"
+
+namespace sofie_hip {
+
+// Tile store straight from the accumulator registers.  With the Bt fragment as the first MFMA operand a lane holds, per
+// register group g, 4 consecutive columns  n = j*R + g*4*LK + lk*4 + (0..3)  of row  m = i*R + lr   (R = rows of the MFMA
+// block, lr = lane % R, lk = lane / R, LK = 64 / R).
+//   4-byte elements: those are 16 bytes, stored as they are (the LK lanes of a row cover 16*LK consecutive bytes).
+//   1-byte elements, R = 16, four column blocks per wave (NT = 4): the four lanes of a row hold a 4 x 4 matrix of dwords
+//   (lane lk, block j) -> columns j*16 + lk*4; transposing it (two swap stages) leaves lane lk with the dwords of
+//   columns lk*16 .. lk*16 + 15: one 16-byte store per lane and 16-row block.
+// The per-column constants of the epilogue (bias, scale) arrive one column per lane (lane l holds those of column
+// n_base + l; the wave tile is 64 columns wide) and are handed to the lanes that need them by ds_bpermute: two loads per
+// tile instead of one round trip to memory per group of columns.
+template <int MODE, class MMA, int MT, int NT, class EPI, class ACC>
+__device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int lane, int col_bias,
+                                                          float col_scale)
+{
+   constexpr int ESZ = EPI::template out_bytes<MODE>();
+   constexpr int R = MMA::ROWS, LK = MMA::LK, G = MMA::ACC / 4;
+   static_assert(NT * R == 64, "one column constant per lane");
+   const int lr = lane % R, lk = lane / R;
+   char *out = ep.out_base();
+   // byte address (for ds_bpermute) of the lane that holds the constants of this lane's first column; made opaque so that the
+   // sixteen addresses derived from it are recomputed where they are used (one addition each) instead of being kept, and
+   // spilled, across the K loop
+   int first_col_addr = lk * 16;
+   asm volatile("" : "+v"(first_col_addr));
+   auto column_constants = [&](int c0, typename EPI::template col_params<4> &prm) { // columns lk*4 + c0 .. + 3 of the wave tile
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+         prm.b[v] = __builtin_amdgcn_ds_bpermute(first_col_addr + (c0 + v) * 4, col_bias);
+         prm.s[v] = __int_as_float(__builtin_amdgcn_ds_bpermute(first_col_addr + (c0 + v) * 4, __float_as_int(col_scale)));
+      }
+   };
+   if constexpr (ESZ == 4) {
+      static_for<NT>([&](auto cj) {
+         constexpr int j = decltype(cj)::value;
+         static_for<G>([&](auto cg) {
+            constexpr int g = decltype(cg)::value;
+            constexpr int cb = j * R + g * 4 * LK;
+            const int c0 = cb + lk * 4;
+            typename EPI::template col_params<4> prm;
+            column_constants(cb, prm);
+            static_for<MT>([&](auto ci) {
+               constexpr int i = decltype(ci)::value;
+               uint32_t w[4];
+               ep.template pack4<MODE, 4>(prm, 0, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3], w);
+               *(uint4 *)(out + ep.out_index(m_base + i * R + lr, n_base + c0) * 4) = make_uint4(w[0], w[1], w[2], w[3]);
+            });
+         });
+      });
+   } else {
+      static_assert(ESZ == 1 && R == 16 && NT == 4 && G == 1, "1-byte outputs are exchanged as a 4 x 4 matrix of dwords between the four lanes of a row");
+      // IB row blocks at a time (the column constants are permuted again for each group of blocks: few registers live at once)
+      constexpr int IB = 2;
+      static_assert(MT % IB == 0, "row blocks per wave");
+      static_for<MT / IB>([&](auto cb) {
+         constexpr int i0 = decltype(cb)::value * IB;
+         uint32_t w[IB][NT];
+         static_for<NT>([&](auto cj) {
+            constexpr int j = decltype(cj)::value;
+            typename EPI::template col_params<4> prm;
+            column_constants(j * R, prm);
+            static_for<IB>([&](auto ci) {
+               constexpr int i = decltype(ci)::value;
+               ep.template pack4<MODE, 4>(prm, 0, acc[i0 + i][j][0], acc[i0 + i][j][1], acc[i0 + i][j][2], acc[i0 + i][j][3], &w[i][j]);
+            });
+         });
+         static_for<IB>([&](auto ci) {
+            constexpr int i = decltype(ci)::value;
+            // (lane lk, register j) <-> (lane j, register lk): first the high bits (rows 2,3 of 16 lanes <-> registers 2,3), then the low ones
+            auto s02 = __builtin_amdgcn_permlane32_swap(w[i][0], w[i][2], false, false);
+            auto s13 = __builtin_amdgcn_permlane32_swap(w[i][1], w[i][3], false, false);
+            auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+            auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+            *(uint4 *)(out + ep.out_index(m_base + (i0 + i) * R + lr, n_base + lk * 16)) = make_uint4(t01[0], t01[1], t23[0], t23[1]);
+         });
+      });
+   }
+}
+
+template <class MMA, class EPI>
+__global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(const int8_t *__restrict__ A, const int8_t *__restrict__ Bt, int lda, int ldb,
+                                                                  int K, EPI ep, int tiles_m, int tiles_n, int sw)
+{
+   constexpr int BM = 256, BN = 256, BK = 64, STAGES = 5, NW = 8, WAVES_N = 4;
+   constexpr int R = MMA::ROWS, LK = MMA::LK;
+   constexpr int TM = 128, TN = 64, MT = TM / R, NT = TN / R;
+   constexpr int LD = BM / 16 / NW;            // wave instructions per operand and slab (an instruction fills 16 rows of 64 bytes)
+   constexpr int STAGE_BYTES = (BM + BN) * BK; // 32 KB
+   static_assert(MMA::KSTEP == BK, "one MFMA step per slab");
+   static_assert(BM == BN && LD == 2, "the load schedule below is written for 2 + 2 wave instructions per slab");
+   typedef typename MMA::acc_t acc_t;
+   typedef typename MMA::frag_t frag_t;
+
+   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+
+   const int t = threadIdx.x;
+   const int lane = t & 63;
+   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+   const int lr = lane % R, lk = lane / R;
+   const int nwg = gridDim.x, bid = blockIdx.x;
+   const int ntiles = tiles_m * tiles_n;
+   const int my_tiles = (ntiles - bid + nwg - 1) / nwg;
+   const int KP = K / (2 * BK);
+
+   // loader: wave instruction i of an operand fills rows (i*NW + wave)*16 .. +15 of a slab; a lane supplies the chunk that
+   // belongs at its position of the swizzled layout (chunk c of row r sits at position c ^ MMA::lds_swizzle(r); the swizzle has
+   // period 16 in r, so a fragment's rows r = 16*k + lr swizzle like lr)
+   uint32_t a_off[LD], b_off[LD];
+#pragma unroll
+   for (int i = 0; i < LD; ++i) {
+      const int row = (i * NW + wave) * 16 + lane / 4;
+      const int c = (lane % 4) ^ MMA::lds_swizzle(row);
+      a_off[i] = (uint32_t)row * (uint32_t)lda + (uint32_t)c * 16u;
+      b_off[i] = (uint32_t)row * (uint32_t)ldb + (uint32_t)c * 16u;
+   }
+   // The loads run two pairs ahead of the MFMAs and cross into the next tile of the list before the current one is stored.
+   // l_a, l_b: origin of the tile being loaded; n_a, n_b: origin of the one after it, worked out once per tile (in the tile
+   // store, which needs the tile order anyway) so that the step itself has no branch.  Past the end of the list the
+   // loads start over on the last tile: filler that keeps the count of loads in flight constant; nobody reads it.
+   auto tile_origin = [&](int it, int &m0, int &n0) {
+      int tm, tn;
+      tile_of_block((it < my_tiles ? it : my_tiles - 1) * nwg + bid, ntiles, tiles_m, tiles_n, sw, tm, tn);
+      m0 = tm * BM;
+      n0 = tn * BN;
+   };
+   auto load_origin = [&](int it, const int8_t *&pa, const int8_t *&pb) {
+      int m0, n0;
+      tile_origin(it, m0, n0);
+      pa = A + (size_t)m0 * (size_t)lda;
+      pb = Bt + (size_t)n0 * (size_t)ldb;
+   };
+   int l_kp = 0; // pair (of the tile being loaded) the next loads fetch
+   const int8_t *l_a, *l_b, *n_a, *n_b;
+   load_origin(0, l_a, l_b);
+   load_origin(1, n_a, n_b);
+   // load q (0..7) of the pair: operand q/4, wave instruction (q/2)%2, half q%2 of the 128-byte line
+   auto issue_load = [&](int slot0, int slot1, auto q_c) {
+      constexpr int q = decltype(q_c)::value;
+      constexpr int opnd = q / 4, i = (q / 2) % 2, half = q % 2;
+      int8_t *dst = smem + (half ? slot1 : slot0) * STAGE_BYTES + opnd * (BM * BK) + (i * NW + wave) * 1024;
+      // uniform base (scalar registers) + 32-bit lane offset.  (The instruction's own offset field cannot supply the second
+      // half of the line: it is added to the LDS address as well.)
+      const int8_t *base = (opnd ? l_b : l_a) + (l_kp * (2 * BK) + half * BK);
+      const int8_t *src = base + (opnd ? b_off[i] : a_off[i]);
+      __builtin_amdgcn_global_load_lds((global_void_t *)src, (lds_void_t *)dst, 16, 0, 0);
+   };
+   auto advance_loader = [&]() {
+      const bool wrap = (l_kp + 1 == KP);
+      l_kp = wrap ? 0 : l_kp + 1;
+      l_a = wrap ? n_a : l_a;
+      l_b = wrap ? n_b : l_b;
+   };
+
+   const int a_frag = (wm * TM + lr) * BK, b_frag = BM * BK + (wn * TN + lr) * BK;
+   auto read_frags = [&](int slot, frag_t(&fa)[MT], frag_t(&fb)[NT]) {
+      const int8_t *base = smem + slot * STAGE_BYTES;
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+         for (int c = 0; c < MMA::CHUNKS; ++c)
+            fb[j].c[c] = *(const v4i *)(base + b_frag + j * R * BK + (((lk * MMA::CHUNKS + c) ^ MMA::lds_swizzle(lr)) << 4));
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+         for (int c = 0; c < MMA::CHUNKS; ++c)
+            fa[i].c[c] = *(const v4i *)(base + a_frag + i * R * BK + (((lk * MMA::CHUNKS + c) ^ MMA::lds_swizzle(lr)) << 4));
+   };
+
+   acc_t acc[MT][NT];
+   auto zero_acc = [&]() {
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+         for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int v = 0; v < MMA::ACC; ++v)
+               acc[i][j][v] = 0;
+   };
+   zero_acc();
+   int col_bias;
+   float col_scale;
+   {
+      int m0, n0;
+      tile_origin(0, m0, n0);
+      ep.load_column(n0 + wn * TN + lane, col_bias, col_scale);
+   }
+
+   // prologue: pairs 0 and 1 into slots 0..3
+   static_for<8>([&](auto q) { issue_load(0, 1, q); });
+   advance_loader();
+   static_for<8>([&](auto q) { issue_load(2, 3, q); });
+   advance_loader();
+   frag_t fa[2][MT], fb[2][NT];
+   wait_vmcnt<8>();
+   __builtin_amdgcn_s_barrier();
+   read_frags(0, fa[0], fb[0]);
+
+   int rslot = 1; // slot of the slab whose fragments are read during the current step
+   int lslot = 4; // slot of the first slab of the pair requested during the current (even) step
+   constexpr int NMFMA = MT * NT, NREAD = (MT + NT) * MMA::CHUNKS;
+   static_assert(NMFMA % 8 == 0 && NREAD <= 16 && NREAD >= 8, "issue pattern below: 8 groups per step");
+   for (int it = 0; it < my_tiles; ++it) {
+      for (int kp = 0; kp < KP; ++kp) {
+         // ---- even step (the scheduling fences keep the compiler from mixing the instructions of two steps)
+         __builtin_amdgcn_sched_barrier(0);
+         __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+         __builtin_amdgcn_s_barrier();
+         __builtin_amdgcn_sched_barrier(0);
+         read_frags(rslot, fa[1], fb[1]);
+         const int lslot1 = (lslot + 1 == STAGES) ? 0 : lslot + 1;
+         static_for<4>([&](auto q) { issue_load(lslot, lslot1, q); }); // the A rows of the pair; the Bt rows follow in the odd step
+#pragma unroll
+         for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+               acc[i][j] = MMA::mma(fb[0][j], fa[0][i], acc[i][j]);
+         // issue order: the compiler keeps the LDS reads ahead of the loads into LDS (it cannot tell that they touch different
+         // slots), so the reads go between the MFMAs of the first half of the step and the loads between those of the second
+         static_for<4>([&](auto gc) {
+            __builtin_amdgcn_sched_group_barrier(0x008, NMFMA / 8, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, (NREAD + 3) / 4, 0);
+         });
+         static_for<4>([&](auto gc) {
+            __builtin_amdgcn_sched_group_barrier(0x008, NMFMA / 8, 0);
+            __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+         });
+         rslot = (rslot + 1 == STAGES) ? 0 : rslot + 1;
+         // ---- odd step
+         __builtin_amdgcn_sched_barrier(0);
+         wait_vmcnt<4>();                    // all but the four loads just issued: the pair that starts with the next slab has landed
+         __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+         __builtin_amdgcn_s_barrier();
+         __builtin_amdgcn_sched_barrier(0);
+         read_frags(rslot, fa[0], fb[0]);
+         static_for<4>([&](auto q) { issue_load(lslot, lslot1, std::integral_constant<int, 4 + decltype(q)::value>{}); });
+         advance_loader();
+#pragma unroll
+         for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+               acc[i][j] = MMA::mma(fb[1][j], fa[1][i], acc[i][j]);
+         static_for<4>([&](auto gc) {
+            __builtin_amdgcn_sched_group_barrier(0x008, NMFMA / 8, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, (NREAD + 3) / 4, 0);
+         });
+         static_for<4>([&](auto gc) {
+            __builtin_amdgcn_sched_group_barrier(0x008, NMFMA / 8, 0);
+            __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+         });
+         __builtin_amdgcn_sched_barrier(0);
+         rslot = (rslot + 1 == STAGES) ? 0 : rslot + 1;
+         lslot = (lslot + 2 >= STAGES) ? lslot + 2 - STAGES : lslot + 2;
+      }
+      // the loads have moved on to tile it + 1 (K spans at least three pairs): the tile after that is it + 2
+      load_origin(it + 2, n_a, n_b);
+      int m0, n0;
+      tile_origin(it, m0, n0);
+      ep.dispatch([&](auto mode) {
+         tile_store_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, lane, col_bias, col_scale);
+      });
+      zero_acc();
+      // the column constants of the next tile: fetched now, used after its K loop
+      tile_origin(it + 1, m0, n0);
+      ep.load_column(n0 + wn * TN + lane, col_bias, col_scale);
+   }
+   wait_vmcnt<0>();
+}
+
+// Whether the persistent kernel takes this product: whole 256 x 256 tiles, K a multiple of 128, 16-byte aligned rows, at
+// least as many tiles as CUs would otherwise idle.
+inline bool mfma8_persist_applies(const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb)
+{
+   return M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0 && K >= 384 && K % 128 == 0 && lda % 16 == 0 && ldb % 16 == 0 &&
+          (((uintptr_t)A | (uintptr_t)Bt) & 15) == 0 && (long long)(M / 256) * (N / 256) <= 0x7fffffLL &&
+          (size_t)256 * (size_t)(lda > ldb ? lda : ldb) < 0xffffffffULL;
+}
+
+template <class MMA, class EPI>
+static int launch_mfma8_persist(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
+{
+   const int tiles_m = M / 256, tiles_n = N / 256;
+   const int ntiles = tiles_m * tiles_n;
+   constexpr size_t smem = (size_t)5 * 512 * 64;
+   static_assert(smem <= 160 * 1024, "LDS ring larger than the CU's LDS");
+   auto kern = mfma8_gemm_persist_kernel<MMA, EPI>;
+   static bool configured[64] = {};
+   if (int st = configure_lds_once(kern, smem, configured))
+      return st;
+   static int cus[64] = {};
+   int dev = 0;
+   SOFIE_HIP_CHECK(hipGetDevice(&dev));
+   int ncu = (dev >= 0 && dev < 64) ? cus[dev] : 0;
+   if (ncu == 0) {
+      SOFIE_HIP_CHECK(hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev));
+      if (dev >= 0 && dev < 64)
+         cus[dev] = ncu;
+   }
+   const int grid = ntiles < ncu ? ntiles : ncu;
+   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, stream, A, Bt, lda, ldb, K, ep, tiles_m, tiles_n, swizzle_mode());
+   return launch_status("mfma8_gemm_persist_kernel");
+}
+
+} // namespace sofie_hip

@@ -181,3 +181,35 @@ def test_short_reduction_over_many_tiles_takes_the_shared_cu_tile(rt):
     Bt = util.int8_sym(14, N * K).reshape(N, K)
     got = run_gemm(rt, A, Bt, M, N, K, transB=1, out=R.I8OUT_I32)
     assert np.array_equal(got, ob.matmul_integer(A, Bt, M=M, N=N, K=K, transB=1, omp=True))
+
+
+@pytest.mark.parametrize("out,relu_acc,relu_out", [(R.I8OUT_I32, 0, 0), (R.I8OUT_F32, 1, 0), (R.I8OUT_I8, 0, 1), (R.I8OUT_I8, 0, 0),
+                                                   (R.I8OUT_I8_DQQ, 1, 0)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 384), (512, 768, 512), (1280, 512, 1152), (256, 4352, 640)])
+def test_persistent_kernel_forced_on_small_shapes(rt, out, relu_acc, relu_out, M, N, K):
+    """Tile 512 asks for the persistent 256 x 256 kernel (eight waves, tile store from registers) where the heuristic would
+    not pick it: one tile, fewer tiles than CUs, more tiles than CUs (17 x 1 and 5 x 2 lists of uneven length per workgroup
+    do not occur at these sizes, so the 4352-column case gives workgroups 0..16 one tile each), K of 3, 4, 5 and 9 slab pairs."""
+    A = util.int8_sym(51 + M, M * K).reshape(M, K)
+    Bt = util.int8_sym(52 + N, N * K).reshape(N, K)
+    bias = util.int32_range(53, N, -(1 << 15), 1 << 15)
+    scale = ((0.5 + util.uniform01(54, N)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    kw = dict(bias=bias, scale=scale, q_scale=np.float32(0.041), relu_acc=relu_acc, relu_out=relu_out, out=out)
+    os.environ["SOFIE_HIP_I8_TILE"] = "512"
+    try:
+        got = run_gemm(rt, A, Bt, M, N, K, transB=1, **kw)
+    finally:
+        del os.environ["SOFIE_HIP_I8_TILE"]
+    want = ob.gemm_i8(A, Bt, M=M, N=N, K=K, transB=1, omp=True, **kw)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
+def test_persistent_kernel_more_tiles_than_cus(rt):
+    """2304 x 8192: 9 x 32 = 288 tiles on 256 CUs, so 32 workgroups take a second tile and the loads of the others run past
+    the end of their lists; per-tensor scale (no bias, no scale vector)."""
+    M, N, K = 2304, 8192, 512
+    A = util.int8_sym(61, M * K).reshape(M, K)
+    Bt = util.int8_sym(62, N * K).reshape(N, K)
+    got = run_gemm(rt, A, Bt, M, N, K, transB=1, scale_scalar=np.float32(3e-4), out=R.I8OUT_I8)
+    want = ob.gemm_i8(A, Bt, M=M, N=N, K=K, transB=1, omp=True, scale_scalar=np.float32(3e-4), out=R.I8OUT_I8)
+    assert np.array_equal(got, want)
