@@ -15,6 +15,15 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float x)
    return (uint16_t)(u >> 16);
 }
 
+// Two fp32 -> two bf16 in one dword (round to nearest even, NaN stays a quiet NaN): one v_cvt_pk_bf16_f32.
+__device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi)
+{
+   typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+   typedef float f32x2 __attribute__((ext_vector_type(2)));
+   const f32x2 v = {lo, hi};
+   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+
 // fp32 -> e4m3fn code, round to nearest even, saturating at +-448 (also +-inf); NaN -> 0x7f.
 __device__ __forceinline__ uint8_t f32_to_e4m3_rne_sat(float x)
 {
@@ -75,18 +84,30 @@ struct F8Epilogue {
    int stage_ok;
    int N;
 
+   // The store is compiled once per (output type, activation class): MODE = out | class << 1, class 0 = none, 1 = relu,
+   // 2 = gelu (erf form), 3 = any other activation, chosen per element at run time.  With the activation a compile-time
+   // constant the conversion of one element is a few instructions (about 25 for gelu); with the run-time switch every
+   // element of an unrolled tile store carries the code of all of them, and the store of a 256 x 256 tile took 26 us.
+   static constexpr int kClassNone = 0, kClassRelu = 1, kClassGelu = 2, kClassAny = 3;
    template <class F>
    __device__ __forceinline__ void dispatch(F f) const
    {
-      if (out == SOFIE_F8OUT_F32)
-         f(std::integral_constant<int, SOFIE_F8OUT_F32>{});
-      else
-         f(std::integral_constant<int, SOFIE_F8OUT_BF16>{});
+      const int cls = act == SOFIE_ACT_NONE ? kClassNone : act == SOFIE_ACT_RELU ? kClassRelu : act == SOFIE_ACT_GELU ? kClassGelu : kClassAny;
+      switch ((out == SOFIE_F8OUT_F32 ? 1 : 0) | (cls << 1)) {
+      case 0: f(std::integral_constant<int, 0>{}); break;
+      case 1: f(std::integral_constant<int, 1>{}); break;
+      case 2: f(std::integral_constant<int, 2>{}); break;
+      case 3: f(std::integral_constant<int, 3>{}); break;
+      case 4: f(std::integral_constant<int, 4>{}); break;
+      case 5: f(std::integral_constant<int, 5>{}); break;
+      case 6: f(std::integral_constant<int, 6>{}); break;
+      default: f(std::integral_constant<int, 7>{}); break;
+      }
    }
-   template <int OUT>
+   template <int MODE>
    static constexpr int out_bytes()
    {
-      return OUT == SOFIE_F8OUT_F32 ? 4 : 2;
+      return (MODE & 1) ? 4 : 2;
    }
    __device__ __forceinline__ bool rows_vectorizable() const { return stage_ok != 0; }
    __device__ __forceinline__ char *out_base() const { return (char *)Y; }
@@ -102,10 +123,21 @@ struct F8Epilogue {
       for (int i = 0; i < C; ++i)
          p.b[i] = bias ? bias[n + i < N ? n + i : N - 1] : 0.0f;
    }
+   // the constants of one column as 32-bit words (what the register tile store hands from lane to lane): the bias
+   static constexpr int kColWords = 1;
+   __device__ __forceinline__ void load_column(int n, uint32_t (&w)[kColWords]) const { w[0] = __float_as_uint(bias ? bias[n] : 0.0f); }
+   template <int C>
+   static __device__ __forceinline__ void set_column(col_params<C> &p, int i, const uint32_t (&w)[kColWords])
+   {
+      p.b[i] = __uint_as_float(w[0]);
+   }
+   // row-major output with 16-byte aligned rows (what the register tile store handles)
+   bool stores_plain_rows() const { return stage_ok != 0; }
    // v = acc*scale + bias[n]; activation in fp32; then fp32 or bf16 (round to nearest even)
-   template <int OUT, int C>
+   template <int MODE, int C>
    __device__ __forceinline__ void pack4(const col_params<C> &p, int q, float a0, float a1, float a2, float a3, uint32_t *w) const
    {
+      constexpr int cls = MODE >> 1;
       const float a[4] = {a0, a1, a2, a3};
       float v[4];
 #pragma unroll
@@ -113,15 +145,20 @@ struct F8Epilogue {
          v[i] = mul_nofma(a[i], scale);
          if (bias)
             v[i] = v[i] + p.b[4 * q + i];
-         v[i] = (act == SOFIE_ACT_GELU) ? gelu_erf_fast(v[i]) : apply_activation(v[i], act, 0.0f);
+         if constexpr (cls == kClassRelu)
+            v[i] = apply_activation(v[i], SOFIE_ACT_RELU, 0.0f);
+         else if constexpr (cls == kClassGelu)
+            v[i] = gelu_erf_fast(v[i]);
+         else if constexpr (cls == kClassAny)
+            v[i] = apply_activation(v[i], act, 0.0f);
       }
-      if (OUT == SOFIE_F8OUT_F32) {
+      if constexpr (MODE & 1) {
 #pragma unroll
          for (int i = 0; i < 4; ++i)
             w[i] = __float_as_uint(v[i]);
       } else {
-         w[0] = (uint32_t)f32_to_bf16_rne(v[0]) | ((uint32_t)f32_to_bf16_rne(v[1]) << 16);
-         w[1] = (uint32_t)f32_to_bf16_rne(v[2]) | ((uint32_t)f32_to_bf16_rne(v[3]) << 16);
+         w[0] = pack_bf16_rne(v[0], v[1]);
+         w[1] = pack_bf16_rne(v[2], v[3]);
       }
    }
 };

@@ -111,11 +111,18 @@ struct I8Epilogue {
       }
    }
 
-   // bias and scale of the single column n (n < N)
-   __device__ __forceinline__ void load_column(int n, int &b, float &sc) const
+   // The constants of ONE column as 32-bit words (what the register tile store hands from lane to lane): bias, scale.
+   static constexpr int kColWords = 2;
+   __device__ __forceinline__ void load_column(int n, uint32_t (&w)[kColWords]) const
    {
-      b = bias ? bias[n + n_offset] : 0;
-      sc = scale ? scale[n + n_offset] : scale_scalar;
+      w[0] = (uint32_t)(bias ? bias[n + n_offset] : 0);
+      w[1] = __float_as_uint(scale ? scale[n + n_offset] : scale_scalar);
+   }
+   template <int C>
+   static __device__ __forceinline__ void set_column(col_params<C> &p, int i, const uint32_t (&w)[kColWords])
+   {
+      p.b[i] = (int)w[0];
+      p.s[i] = __uint_as_float(w[1]);
    }
 
    // converts columns 4q..4q+3 of the lane's columns (exact int32 dot products) into 4*out_bytes() bytes

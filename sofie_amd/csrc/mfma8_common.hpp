@@ -78,6 +78,8 @@ struct MfmaF8 {
    static constexpr int ROWS = 32;
    static constexpr int LK = 2;
    static constexpr int ACC = 16;
+   // chunk XOR of row r in 64-byte LDS rows: conflict-free for this fragment (lane = lk*32 + row, chunks 2*lk and 2*lk + 1)
+   static __device__ __forceinline__ int lds_swizzle(int r) { return (r >> 2) & 3; }
    struct frag_t {
       v4i c[2];
    };

@@ -31,6 +31,9 @@ static int launch_mfma8_best(hipStream_t stream, const int8_t *A, const int8_t *
       // two K-steps per slab are the minimum: a 64-byte K-step needs 128-byte slabs
       if (!k128)
          return launch_mfma8_auto<MMA, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile);
+      if ((force_tile == 512 || (!force_tile && variant == 0 && tile == 256)) && mfma8_persist_applies(A, Bt, M, N, K, lda, ldb) &&
+          ep.stores_plain_rows())
+         return launch_mfma8_persist<MMA, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep);
       switch (tile) {
       case 256:
          if (variant == 1)

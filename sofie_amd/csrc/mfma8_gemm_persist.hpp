@@ -31,8 +31,8 @@ namespace sofie_hip {
 // n_base + l; the wave tile is 64 columns wide) and are handed to the lanes that need them by ds_bpermute: two loads per
 // tile instead of one round trip to memory per group of columns.
 template <int MODE, class MMA, int MT, int NT, class EPI, class ACC>
-__device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int lane, int col_bias,
-                                                          float col_scale)
+__device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int lane,
+                                                          const uint32_t (&col_words)[EPI::kColWords])
 {
    constexpr int ESZ = EPI::template out_bytes<MODE>();
    constexpr int R = MMA::ROWS, LK = MMA::LK, G = MMA::ACC / 4;
@@ -47,8 +47,11 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
    auto column_constants = [&](int c0, typename EPI::template col_params<4> &prm) { // columns lk*4 + c0 .. + 3 of the wave tile
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-         prm.b[v] = __builtin_amdgcn_ds_bpermute(first_col_addr + (c0 + v) * 4, col_bias);
-         prm.s[v] = __int_as_float(__builtin_amdgcn_ds_bpermute(first_col_addr + (c0 + v) * 4, __float_as_int(col_scale)));
+         uint32_t w[EPI::kColWords];
+#pragma unroll
+         for (int k = 0; k < EPI::kColWords; ++k)
+            w[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(first_col_addr + (c0 + v) * 4, (int)col_words[k]);
+         EPI::template set_column<4>(prm, v, w);
       }
    };
    if constexpr (ESZ == 4) {
@@ -65,6 +68,32 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
                uint32_t w[4];
                ep.template pack4<MODE, 4>(prm, 0, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3], w);
                *(uint4 *)(out + ep.out_index(m_base + i * R + lr, n_base + c0) * 4) = make_uint4(w[0], w[1], w[2], w[3]);
+            });
+         });
+      });
+   } else if constexpr (ESZ == 2) {
+      // 2-byte elements, R = 32: a lane's 4 columns of group g are 8 bytes at column g*8 + lk*4.  The two lanes of a row swap
+      // so that lane lk = 0 ends up with the 8 columns of an even group and lane lk = 1 with those of the odd group after it:
+      // 16 consecutive bytes each.
+      static_assert(R == 32 && G == 4, "2-byte outputs are exchanged between the two lanes of a row of the 32 x 32 block");
+      static_for<NT>([&](auto cj) {
+         constexpr int j = decltype(cj)::value;
+         static_for<2>([&](auto cgp) {
+            constexpr int ge = decltype(cgp)::value * 2, go = ge + 1;
+            typename EPI::template col_params<4> pe, po;
+            column_constants(j * R + ge * 4 * LK, pe);
+            column_constants(j * R + go * 4 * LK, po);
+            static_for<MT>([&](auto ci) {
+               constexpr int i = decltype(ci)::value;
+               uint32_t we[2], wo[2];
+               ep.template pack4<MODE, 4>(pe, 0, acc[i][j][4 * ge + 0], acc[i][j][4 * ge + 1], acc[i][j][4 * ge + 2], acc[i][j][4 * ge + 3], we);
+               ep.template pack4<MODE, 4>(po, 0, acc[i][j][4 * go + 0], acc[i][j][4 * go + 1], acc[i][j][4 * go + 2], acc[i][j][4 * go + 3], wo);
+               // swap(a, b): a keeps its lower 32 lanes and receives b's lower 32 lanes in its upper half; b the other way round
+               auto s0 = __builtin_amdgcn_permlane32_swap(we[0], wo[0], false, false);
+               auto s1 = __builtin_amdgcn_permlane32_swap(we[1], wo[1], false, false);
+               // lane lk: group ge + lk, columns 0..3 in s0[0], s1[0] and columns 4..7 in s0[1], s1[1]
+               const int n = n_base + j * R + (ge + lk) * 4 * LK;
+               *(uint4 *)(out + ep.out_index(m_base + i * R + lr, n) * 2) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
             });
          });
       });
@@ -199,12 +228,11 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(const int8_t *_
                acc[i][j][v] = 0;
    };
    zero_acc();
-   int col_bias;
-   float col_scale;
+   uint32_t col_words[EPI::kColWords]; // the epilogue's constants of column n0 + wn*TN + lane of the tile in work
    {
       int m0, n0;
       tile_origin(0, m0, n0);
-      ep.load_column(n0 + wn * TN + lane, col_bias, col_scale);
+      ep.load_column(n0 + wn * TN + lane, col_words);
    }
 
    // prologue: pairs 0 and 1 into slots 0..3
@@ -278,12 +306,12 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(const int8_t *_
       int m0, n0;
       tile_origin(it, m0, n0);
       ep.dispatch([&](auto mode) {
-         tile_store_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, lane, col_bias, col_scale);
+         tile_store_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, lane, col_words);
       });
       zero_acc();
       // the column constants of the next tile: fetched now, used after its K loop
       tile_origin(it + 1, m0, n0);
-      ep.load_column(n0 + wn * TN + lane, col_bias, col_scale);
+      ep.load_column(n0 + wn * TN + lane, col_words);
    }
    wait_vmcnt<0>();
 }

@@ -111,3 +111,58 @@ def test_bf16_output_with_bias_and_activation(rt, act):
     acc_err = 2.0 ** -14 * abs_sum.astype(np.float64) * float(scale)
     bound = 1.2 * acc_err + 2.0 ** -8 * np.abs(want) + 1e-6
     assert np.all(np.abs(got.astype(np.float64) - want) <= bound)
+
+
+def check_fp8_against_oracle(got_f32, A, Bt, bias, scale, act, bf16):
+    """|got - oracle| within the accumulation bound (propagated through bias and an activation of slope <= 1.13) plus the
+    rounding of the output type."""
+    M, K = A.shape
+    N = Bt.shape[0]
+    want, abs_sum = ob.gemm_fp8(A, Bt, M=M, N=N, K=K, transB=1, bias=bias, scale=scale, act=act, out=1, want_abs_sum=True, omp=True)
+    acc_err = 2.0 ** -14 * abs_sum.astype(np.float64) * float(scale)
+    bound = 1.2 * acc_err + (2.0 ** -8 if bf16 else 2.0 ** -21) * np.abs(want) + 1e-6
+    err = np.abs(got_f32.astype(np.float64) - want)
+    assert np.all(err <= bound), "worst excess %g at %s" % ((err - bound).max(), np.unravel_index(np.argmax(err - bound), err.shape))
+    return want
+
+
+@pytest.mark.parametrize("tile,M,N,K", [(64, 130, 200, 384), (64, 96, 72, 1000), (128, 300, 260, 512), (128, 257, 129, 1040),
+                                        (256, 520, 700, 640), (256, 300, 513, 2048 + 64), (512, 512, 768, 512), (512, 256, 256, 384),
+                                        (512, 1280, 512, 1152)])
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("out,act", [(1, R.ACT_NONE), (0, R.ACT_GELU)])
+def test_every_fp8_tile_configuration(rt, monkeypatch, tile, M, N, K, variant, out, act):
+    """Every tile kernel of the FP8 product, forced: 64 / 128 / 256 (pipelined kernels when K is a multiple of 128, the general one
+    otherwise; variant 1 = the alternative pipelined kernel) and 512 = the persistent kernel with the tile store from registers."""
+    if tile == 512 and variant:
+        pytest.skip("the persistent kernel has one form")
+    monkeypatch.setenv("SOFIE_HIP_F8_TILE", str(tile))
+    monkeypatch.setenv("SOFIE_HIP_GEMM_VARIANT", str(variant))
+    A, sa = make_fp8(4101 + M, M, K)
+    Bt, sb = make_fp8(4102 + N, N, K)
+    bias = util.normal(4103, N)
+    scale = np.float32(sa * sb)
+    got = run_fp8(rt, A, Bt, M, N, K, bias=bias, scale=scale, act=act, out=out)
+    if out == 0:
+        got = ob.bf16_bits_to_f32(got)
+    check_fp8_against_oracle(got, A, Bt, bias, scale, act, bf16=(out == 0))
+
+
+@pytest.mark.parametrize("n", [4096, 8192])
+def test_full_size_fp8_sampled_rows_and_columns(rt, n):
+    """benchmark configuration 4 at M=N=K=4096 and 8192 (the heuristic's own kernel choice), bias + GELU, bf16 output: sampled
+    full rows and full columns against the oracle; the accumulation bound 2^-14 sum|a b| is checked at the full K."""
+    import torch
+    M = N = K = n
+    A, sa = make_fp8(4001, M, K)
+    Bt, sb = make_fp8(4002, N, K)
+    bias = util.normal(4003, N)
+    scale = np.float32(sa * sb)
+    got = ob.bf16_bits_to_f32(run_fp8(rt, A, Bt, M, N, K, bias=bias, scale=scale, act=R.ACT_GELU, out=0))
+    rows = np.array([0, 1, 31, 32, 255, 256, n // 2 - 1, n // 2, n - 2, n - 1, 777])
+    want = check_fp8_against_oracle(got[rows], np.ascontiguousarray(A[rows]), Bt, bias, scale, R.ACT_GELU, bf16=True)
+    assert np.abs(want).max() > 0.5  # the outputs are not all in the flat part of GELU
+    cols = np.array([0, 5, 63, 64, n // 2 + 1, n - 1])
+    check_fp8_against_oracle(got[:, cols], A, np.ascontiguousarray(Bt[cols]), bias[cols], scale, R.ACT_GELU, bf16=True)
+    del got
+    torch.cuda.empty_cache()
