@@ -297,16 +297,6 @@ def main():
     avg_launch_s = gms * 1e-3 / launches
     achieved = ops_per_launch / avg_launch_s
 
-    # what the matrix cores of this board sustain with no memory traffic (constant / toggling operands)
-    import torch
-    scratch = torch.empty(1 << 20, dtype=torch.int32, device="cuda")
-    torch.cuda.synchronize()
-    probe = {}
-    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
-        v = C.c_double()
-        rt.call("sofie_hip_mfma_i8_probe", C.c_void_p(scratch.data_ptr()), C.c_size_t(scratch.numel() * 4), 20000, rnd, C.byref(v))
-        probe[name] = round(v.value / 1e12, 1)
-
     # parity of what was timed, against the oracle on the sampled rows
     y = np.empty((batch, dims[-1]), dtype=np.float32)
     rt.call("sofie_hip_download", y.ctypes.data_as(C.c_void_p), sess.y_ptr, C.c_size_t(y.nbytes))
@@ -361,12 +351,10 @@ def main():
                    "parity_vs_oracle_rows": args.cpu_rows, "parity_bit_exact": parity,
                    "mlp_tops": round(ops_per_inference_batch / (ms_per_step * 1e-3) / 1e12, 2),
                    "mlp_algorithmic_bytes": algo_bytes,
-                   "int8_mfma_register_only_tops": probe,
                    "gemm_sweep_int8_requant_bias_relu": sweep,
                    "gemm_sweep_fp8_bias_gelu_bf16": f8, **extra},
         "roofline": {"bound": "mfma", "achieved": round(achieved / 1e12, 2), "peak": INT8_PEAK / 1e12, "unit": "TFLOP/s",
                      "frac": round(achieved / INT8_PEAK, 4), "traffic": DOMINANT_KERNEL_TRAFFIC_BYTES,
-                     "frac_of_sustained_random_operand_rate": round(achieved / 1e12 / probe["random_operands"], 4),
                      "kernel": "mfma8_gemm_dma_kernel<MfmaI8, 128, 128, 128, 2, 2, 3, ...> (layers 1 and 2 of the MLP: 2 launches per inference, "
                                "avg %.2f us, %.3e int8 op per launch on average)" % (avg_launch_s * 1e6, ops_per_launch)},
         "cpu_baseline": cpu,

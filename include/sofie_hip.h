@@ -42,6 +42,13 @@ enum {
  * (core/inc/SOFIE/RModel_Base.hxx:19-33). */
 int sofie_hip_ctx_create(sofie_hip_ctx **out, int device, void *external_stream);
 int sofie_hip_ctx_destroy(sofie_hip_ctx *ctx);
+/* Kernel-choice overrides of one context, for tuning and for tests that must reach a particular kernel (no counterpart in the
+ * reference, whose GPU path has no such choice): "i8_tile" / "f8_tile" (64, 128, 256; 258 and 512 ask for the two-per-CU and the
+ * persistent kernel; 0 = heuristic), "gemm_variant" (1: alternative pipelined kernel, -1: general kernel only), "swizzle"
+ * (tile order), "conv_explicit" (1: int8 convolutions through a column matrix whenever the workspace holds one), "f32_skinny",
+ * "f32_chain" (0 / 1, -1 = heuristic).  Each is also read once, at sofie_hip_ctx_create, from the environment variable
+ * SOFIE_HIP_<NAME IN CAPITALS>; nothing reads the environment after that. */
+int sofie_hip_ctx_set_option(sofie_hip_ctx *ctx, const char *name, int32_t value);
 const char *sofie_hip_last_error(void);
 int sofie_hip_abi_version(void);
 
@@ -343,6 +350,7 @@ typedef struct sofie_conv_i8_args {
 } sofie_conv_i8_args;
 int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_conv_i8_args *a);
 size_t sofie_hip_conv_i8_workspace(const sofie_conv_desc *d, const sofie_conv_i8_args *a); /* minimum bytes */
+size_t sofie_hip_conv_i8_column_matrix_bytes(const sofie_conv_desc *d); /* column matrix of one image (what "conv_explicit" needs on top) */
 size_t sofie_hip_conv_weight_i8_packed_bytes(const sofie_conv_desc *d);
 int sofie_hip_pack_conv_weight_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, int8_t *dst, const int8_t *src);
 
@@ -411,12 +419,6 @@ int sofie_hip_batchnorm_f32(sofie_hip_ctx *ctx, float *Y, const float *X, const 
                             const float *bias, int32_t N, int32_t C, int32_t spatial, int32_t relu);
 
 /* ---- measurement helpers used by the benchmark ------------------------------------------------ */
-/* Register-only int8 MFMA loop on every CU (no counterpart in the reference): the rate the matrix
- * cores of this board sustain with no memory traffic, with constant operands (random_operands = 0)
- * or with operands that toggle every instruction (1: the board clocks down under its power limit).
- * `scratch` receives one int per lane (CUs * 256 * 4 bytes). */
-int sofie_hip_mfma_i8_probe(sofie_hip_ctx *ctx, void *scratch, size_t scratch_bytes, int32_t iters, int32_t random_operands,
-                            double *ops_per_second);
 /* hipEvent pair on the context's stream (torch's events only see torch's streams). */
 int sofie_hip_timer_start(sofie_hip_ctx *ctx);
 int sofie_hip_timer_stop(sofie_hip_ctx *ctx, float *elapsed_ms); /* records, synchronises, returns ms */

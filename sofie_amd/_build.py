@@ -9,7 +9,7 @@ CSRC = os.path.join(ROOT, "sofie_amd", "csrc")
 LIB_DIR = os.path.join(ROOT, "sofie_amd", "lib")
 LIB = os.path.join(LIB_DIR, "libsofie_hip.so")
 
-HIP_SOURCES = ["runtime.hip", "gemm_i8.hip", "gemm_f32.hip", "gemm_fp8.hip", "conv_i8.hip", "eltwise.hip", "probe.hip"]
+HIP_SOURCES = ["runtime.hip", "gemm_i8.hip", "gemm_f32.hip", "gemm_fp8.hip", "conv_i8.hip", "eltwise.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -37,17 +37,15 @@ def _run(cmd, cwd=None):
         raise RuntimeError("command failed (%d): %s" % (r.returncode, " ".join(cmd)))
 
 
-def build_hip_library(jobs=8, tuning=False):
-    """Compiles every HIP source for gfx950 and links sofie_amd/lib/libsofie_hip.so.  tuning=True builds, beside it, the
-    library with the ablation and alternative-tile kernels (-DSOFIE_HIP_TUNING) that SOFIE_HIP_GEMM_VARIANT and
-    SOFIE_HIP_I8_TILE select, as sofie_amd/lib/tuning/libsofie_hip.so; nothing loads that one by default."""
+def build_hip_library(jobs=8):
+    """Compiles every HIP source for gfx950 and links sofie_amd/lib/libsofie_hip.so."""
     from concurrent.futures import ThreadPoolExecutor
-    lib_dir = os.path.join(LIB_DIR, "tuning") if tuning else LIB_DIR
-    lib = os.path.join(lib_dir, "libsofie_hip.so")
+    lib_dir = LIB_DIR
+    lib = LIB
     os.makedirs(lib_dir, exist_ok=True)
-    obj_dir = os.path.join(ROOT, "build", "obj_tuning" if tuning else "obj")
+    obj_dir = os.path.join(ROOT, "build", "obj")
     os.makedirs(obj_dir, exist_ok=True)
-    flags = HIPCC_FLAGS + (["-DSOFIE_HIP_TUNING"] if tuning else [])
+    flags = HIPCC_FLAGS
     hipcc = _hipcc()
     sources = [s for s in HIP_SOURCES if os.path.exists(os.path.join(CSRC, s))]
     objs = [os.path.join(obj_dir, s.replace(".hip", ".o")) for s in sources]
@@ -75,8 +73,5 @@ def build_all():
 
 
 if __name__ == "__main__":
-    if "--tuning" in sys.argv[1:]:
-        build_hip_library(tuning=True)
-    else:
-        build_all()
+    build_all()
     sys.exit(0)

@@ -7,7 +7,21 @@
 #include <cstring>
 #include "sofie_hip.h"
 
+// Kernel-choice overrides of a context (tuning and tests).  Read from the environment ONCE, when the context is created
+// (SOFIE_HIP_SWIZZLE, SOFIE_HIP_I8_TILE, SOFIE_HIP_F8_TILE, SOFIE_HIP_GEMM_VARIANT, SOFIE_HIP_CONV_EXPLICIT,
+// SOFIE_HIP_F32_SKINNY, SOFIE_HIP_F32_CHAIN), afterwards changed only through sofie_hip_ctx_set_option.
+struct sofie_hip_options {
+   int swizzle = 4;       // tile order: XCD regrouping, bands of 4 tile rows
+   int i8_tile = 0;       // 0 = heuristic
+   int f8_tile = 0;
+   int gemm_variant = 0;  // alternative pipelined kernel (1), general kernel only (-1)
+   int conv_explicit = 0; // int8 convolution through a column matrix whenever the workspace holds one
+   int f32_skinny = -1;   // -1 = heuristic
+   int f32_chain = -1;
+};
+
 struct sofie_hip_ctx {
+   sofie_hip_options opt;
    int device = 0;
    hipStream_t stream = nullptr;
    bool owns_stream = false;
@@ -18,6 +32,16 @@ struct sofie_hip_ctx {
 };
 
 namespace sofie_hip {
+
+// What a launch of the int8 / FP8 GEMM kernels needs from the context: the stream and the kernel-choice overrides.
+struct LaunchCfg {
+   hipStream_t stream;
+   int tile;    // forced tile configuration, 0 = heuristic
+   int variant; // alternative of the pipelined kernel
+   int swizzle; // tile order (tile_of_block)
+};
+inline LaunchCfg launch_cfg_i8(const sofie_hip_ctx *ctx) { return LaunchCfg{ctx->stream, ctx->opt.i8_tile, ctx->opt.gemm_variant, ctx->opt.swizzle}; }
+inline LaunchCfg launch_cfg_f8(const sofie_hip_ctx *ctx) { return LaunchCfg{ctx->stream, ctx->opt.f8_tile, ctx->opt.gemm_variant, ctx->opt.swizzle}; }
 
 // Records the text returned by sofie_hip_last_error() for the calling thread and returns `code`.
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));

@@ -152,8 +152,7 @@ static bool conv_i8_implicit_shape(const sofie_conv_desc *d, int x_layout)
    for (int t = 0; t < ntaps && t < 32; ++t)
       if (((t * kw_recip) >> 16) != t / d->kw)
          return false;
-   const char *force = getenv("SOFIE_HIP_CONV_EXPLICIT");
-   return !(force && atoi(force)) && x_layout == SOFIE_LAYOUT_NHWC && (Cg & (Cg - 1)) == 0 && Cg >= 64 && ntaps <= 32 &&
+   return x_layout == SOFIE_LAYOUT_NHWC && (Cg & (Cg - 1)) == 0 && Cg >= 64 && ntaps <= 32 &&
           d->C % 16 == 0 && reach < (1LL << 31) && rows < (1LL << 31);
 }
 
@@ -163,8 +162,7 @@ static bool conv_i8_gather_shape(const sofie_conv_desc *d)
    if (d->group <= 0 || d->C % d->group != 0)
       return false;
    const long long K = (long long)(d->C / d->group) * d->kh * d->kw;
-   const char *force = getenv("SOFIE_HIP_CONV_EXPLICIT");
-   return !(force && atoi(force)) && K <= 64 && (long long)(d->kh - 1) * d->dil_h <= 127 && (long long)(d->kw - 1) * d->dil_w <= 127 &&
+   return K <= 64 && (long long)(d->kh - 1) * d->dil_h <= 127 && (long long)(d->kw - 1) * d->dil_w <= 127 &&
           (long long)d->C * d->H * d->W < (1LL << 31) && (long long)d->N * d->OH * d->OW < (1LL << 31);
 }
 
@@ -179,6 +177,14 @@ size_t sofie_hip_conv_i8_workspace(const sofie_conv_desc *d, const sofie_conv_i8
    if (!a->w_is_packed)
       need += sofie_hip_conv_weight_i8_packed_bytes(d);
    return need;
+}
+
+size_t sofie_hip_conv_i8_column_matrix_bytes(const sofie_conv_desc *d)
+{
+   if (!d || d->group <= 0)
+      return 0;
+   const size_t K = (size_t)(d->C / d->group) * d->kh * d->kw;
+   return round256((size_t)d->OH * d->OW * ((K + 15) & ~(size_t)15));
 }
 
 int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_conv_i8_args *a)
@@ -224,6 +230,9 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
    const int OHW = g.OH * g.OW;
    const int Cout_g = d->Cout / d->group;
    const size_t esz = out_kind == SOFIE_I8OUT_I8 ? 1 : 4;
+   // the context's conv_explicit option sends every shape through the column matrix, provided the caller's workspace holds
+   // one (a Session sized by sofie_hip_conv_i8_workspace keeps working, on the kernels that need none)
+   const bool column_matrix_by_option = ctx->opt.conv_explicit && !plane_sums && ws != nullptr && ws_left >= (size_t)OHW * g.Kp;
 
    // Implicit GEMM: the kernel reads the NHWC activations directly, one launch per group over the whole batch.
    // Needs K slabs that lie inside one input pixel (channels per group a power of two >= 64) and 32-bit offsets.
@@ -231,7 +240,7 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
       const int ntaps = d->kh * d->kw;
       const int kw_recip = (65536 + d->kw - 1) / d->kw;
       const long long rows = (long long)d->N * OHW;
-      const bool implicit = conv_i8_implicit_shape(d, a->x_layout) && (((uintptr_t)a->X & 15) == 0) && (((uintptr_t)Wp & 15) == 0) &&
+      const bool implicit = !column_matrix_by_option && conv_i8_implicit_shape(d, a->x_layout) && (((uintptr_t)a->X & 15) == 0) && (((uintptr_t)Wp & 15) == 0) &&
                             g.Kp == g.K;
       if (implicit) {
          int cg_shift = 0;
@@ -262,7 +271,7 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
             ep.nchw_ohw = (a->y_layout == SOFIE_LAYOUT_NHWC || plane_sums) ? 0 : OHW;
             ep.rows_per_plane = plane_sums ? OHW : 0;
             ep.Y = a->Y;
-            st = conv_i8_implicit(ctx->stream, src, g.Cg, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.K, ep, forced_i8_tile());
+            st = conv_i8_implicit(launch_cfg_i8(ctx), src, g.Cg, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.K, ep);
             if (st)
                return st;
          }
@@ -270,7 +279,7 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
       }
    }
    // Few input channels (the first layer of an image network): K = taps x channels <= 64 is one slab, gathered in the kernel.
-   if (conv_i8_gather_shape(d) && (((uintptr_t)Wp & 15) == 0)) {
+   if (!column_matrix_by_option && conv_i8_gather_shape(d) && (((uintptr_t)Wp & 15) == 0)) {
       const long long rows = (long long)d->N * OHW;
       const bool nhwc = a->x_layout == SOFIE_LAYOUT_NHWC;
       for (int grp = 0; grp < d->group; ++grp) {
@@ -306,7 +315,7 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
          ep.nchw_ohw = (a->y_layout == SOFIE_LAYOUT_NHWC || plane_sums) ? 0 : OHW;
          ep.rows_per_plane = plane_sums ? OHW : 0;
          ep.Y = a->Y;
-         st = conv_i8_gather(ctx->stream, src, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.Kp, ep);
+         st = conv_i8_gather(launch_cfg_i8(ctx), src, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.Kp, ep);
          if (st)
             return st;
       }
@@ -365,8 +374,7 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
             ep.nchw_ohw = OHW;
             ep.Y = (char *)a->Y + (size_t)img0 * d->Cout * OHW * esz;
          }
-         st = gemm_i8_nt(ctx->stream, (const int8_t *)ws, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.Kp, g.Kp, g.Kp, ep,
-                         forced_i8_tile());
+         st = gemm_i8_nt(launch_cfg_i8(ctx), (const int8_t *)ws, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.Kp, g.Kp, g.Kp, ep);
          if (st)
             return st;
       }

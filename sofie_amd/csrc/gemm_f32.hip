@@ -466,8 +466,7 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *d)
    const unsigned gy = (M + F32_BM - 1) / F32_BM, gx = (N + F32_BN - 1) / F32_BN;
    SOFIE_HIP_REQUIRE(gx <= 65535 && d->batch <= 65535, "sofie_hip_gemm_f32: N or batch too large for one launch");
    // few 64x64 tiles: one-wave workgroups with 8x8 tiles reach every CU (SOFIE_HIP_F32_SKINNY=0/1 overrides)
-   const char *force = getenv("SOFIE_HIP_F32_SKINNY");
-   const bool skinny = force ? atoi(force) != 0 : ((long long)gy * gx * d->batch < 192);
+   const bool skinny = ctx->opt.f32_skinny >= 0 ? ctx->opt.f32_skinny != 0 : ((long long)gy * gx * d->batch < 192);
    if (skinny && K > 0 && (N + SK_T - 1) / SK_T <= 65535) {
       auto aligned16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
       const bool va = !d->transA && K % 4 == 0 && lda % 4 == 0 && aligned16(d->A) && d->strideA % 4 == 0;
@@ -499,9 +498,8 @@ int sofie_hip_gemm_chain_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *laye
    for (int l = 1; l < count; ++l)
       SOFIE_HIP_REQUIRE(layers[l].A == layers[l - 1].Y && layers[l].A != nullptr, "sofie_hip_gemm_chain_f32: layer %d does not read the output of layer %d", l, l - 1);
    // One launch when the batch is small enough that launches, not arithmetic, set the time, and the rows fit in LDS.
-   const char *force = getenv("SOFIE_HIP_F32_CHAIN");
    const int M = layers[0].M;
-   bool fused = count >= 2 && M >= 1 && (force ? atoi(force) != 0 : M <= 256);
+   bool fused = count >= 2 && M >= 1 && (ctx->opt.f32_chain >= 0 ? ctx->opt.f32_chain != 0 : M <= 256);
    int width = layers[0].K;
    ChainArgs a;
    a.count = count;

@@ -1,7 +1,6 @@
 // FP8 (OCP e4m3fn) GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x64_f8f6f4, fp32 accumulate) with
 // scale + bias + activation + bf16 conversion fused into the store, and the fp32 -> e4m3fn quantiser.
 #include "mfma8_dispatch.hpp"
-#include <cstdlib>
 
 namespace sofie_hip {
 
@@ -226,9 +225,7 @@ int sofie_hip_gemm_fp8(sofie_hip_ctx *ctx, const sofie_gemm_fp8_desc *d)
       Bt = (const int8_t *)d->Y;
       lda = ldb = 16;
    }
-   const char *s = getenv("SOFIE_HIP_F8_TILE");
-   const char *v = getenv("SOFIE_HIP_GEMM_VARIANT");
-   return launch_mfma8_best<MfmaF8, F8Epilogue>(ctx->stream, A, Bt, M, N, K, lda, ldb, ep, s ? atoi(s) : 0, v ? atoi(v) : 0);
+   return launch_mfma8_best<MfmaF8, F8Epilogue>(launch_cfg_f8(ctx), A, Bt, M, N, K, lda, ldb, ep);
 }
 
 } // extern "C"

@@ -1,7 +1,6 @@
 // int8 x int8 -> int32 GEMM on the gfx950 matrix cores (v_mfma_i32_32x32x32_i8) with the
 // requantisation / dequantisation epilogue fused into the store, and the int8 re-layout kernel.
 #include "i8_epilogue.hpp"
-#include <cstdlib>
 
 namespace sofie_hip {
 
@@ -25,8 +24,7 @@ __global__ __launch_bounds__(256) void transpose_i8_kernel(int8_t *__restrict__ 
 }
 
 
-int gemm_i8_nt(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep,
-               int force_tile)
+int gemm_i8_nt(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep)
 {
    const size_t esz = ep.out == SOFIE_I8OUT_I32 || ep.out == SOFIE_I8OUT_F32 ? 4 : 1;
    ep.N = N;
@@ -34,13 +32,10 @@ int gemm_i8_nt(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int
                  (((uintptr_t)ep.Y & 15) == 0);
    ep.vec_param = (ep.n_offset % 4 == 0) && (!ep.bias || ((uintptr_t)ep.bias & 15) == 0) &&
                   (!ep.scale || ((uintptr_t)ep.scale & 15) == 0);
-   // SOFIE_HIP_GEMM_VARIANT: tuning alternative of the pipelined kernel; -1 = general kernel only
-   const char *v = getenv("SOFIE_HIP_GEMM_VARIANT");
-   return launch_mfma8_best<MfmaI8, I8Epilogue>(stream, A, Bt, M, N, K, lda, ldb, ep, force_tile, v ? atoi(v) : 0);
+   return launch_mfma8_best<MfmaI8, I8Epilogue>(lc, A, Bt, M, N, K, lda, ldb, ep);
 }
 
-int conv_i8_implicit(hipStream_t stream, const ConvRows &src, int Cg, const int8_t *Wp, int M, int N, int K, I8Epilogue ep,
-                     int force_tile)
+int conv_i8_implicit(const LaunchCfg &lc, const ConvRows &src, int Cg, const int8_t *Wp, int M, int N, int K, I8Epilogue ep)
 {
    const size_t esz = ep.out == SOFIE_I8OUT_I32 || ep.out == SOFIE_I8OUT_F32 ? 4 : 1;
    ep.N = N;
@@ -48,10 +43,10 @@ int conv_i8_implicit(hipStream_t stream, const ConvRows &src, int Cg, const int8
                  (((uintptr_t)ep.Y & 15) == 0);
    ep.vec_param = (ep.n_offset % 4 == 0) && (!ep.bias || ((uintptr_t)ep.bias & 15) == 0) &&
                   (!ep.scale || ((uintptr_t)ep.scale & 15) == 0);
-   return launch_mfma8_conv<I8Epilogue>(stream, src, Cg, Wp, M, N, K, ep, force_tile);
+   return launch_mfma8_conv<I8Epilogue>(lc, src, Cg, Wp, M, N, K, ep);
 }
 
-int conv_i8_gather(hipStream_t stream, const GatherConvRows &src, const int8_t *Wp, int M, int N, int Kp, I8Epilogue ep)
+int conv_i8_gather(const LaunchCfg &lc, const GatherConvRows &src, const int8_t *Wp, int M, int N, int Kp, I8Epilogue ep)
 {
    const size_t esz = ep.out == SOFIE_I8OUT_I32 || ep.out == SOFIE_I8OUT_F32 ? 4 : 1;
    ep.N = N;
@@ -59,14 +54,7 @@ int conv_i8_gather(hipStream_t stream, const GatherConvRows &src, const int8_t *
                  (((uintptr_t)ep.Y & 15) == 0);
    ep.vec_param = (ep.n_offset % 4 == 0) && (!ep.bias || ((uintptr_t)ep.bias & 15) == 0) &&
                   (!ep.scale || ((uintptr_t)ep.scale & 15) == 0);
-   return launch_mfma8_gather<I8Epilogue>(stream, src, Wp, M, N, Kp, ep);
-}
-
-// SOFIE_HIP_I8_TILE=256|128|64 forces a tile configuration (tuning and tests); unset = heuristic.
-int forced_i8_tile()
-{
-   const char *s = getenv("SOFIE_HIP_I8_TILE");
-   return s ? atoi(s) : 0;
+   return launch_mfma8_gather<I8Epilogue>(lc, src, Wp, M, N, Kp, ep);
 }
 
 int transpose_i8(hipStream_t stream, int8_t *dst, const int8_t *src, int rows, int cols, int ld_src, int ld_dst)
@@ -177,15 +165,7 @@ int sofie_hip_gemm_i8(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d)
       Bt = (const int8_t *)d->Y;
       lda = ldb = 16;
    }
-   return gemm_i8_nt(ctx->stream, A, Bt, M, N, K, lda, ldb, ep, forced_i8_tile());
+   return gemm_i8_nt(launch_cfg_i8(ctx), A, Bt, M, N, K, lda, ldb, ep);
 }
 
 } // extern "C"
-
-#ifdef SOFIE_HIP_TUNING
-// tuning builds only: per-workgroup timestamps of the paired-slab kernel (start, first slab landed, loop done, stored)
-extern "C" int sofie_hip_dbg_read_ts(unsigned long long *host, size_t n)
-{
-   return hipMemcpyFromSymbol(host, HIP_SYMBOL(sofie_hip::dbg_ts), n * sizeof(unsigned long long)) == hipSuccess ? 0 : 1;
-}
-#endif

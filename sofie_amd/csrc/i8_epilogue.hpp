@@ -157,14 +157,11 @@ struct I8Epilogue {
    }
 };
 
-// Y = epilogue(A[M,K] * Bt[N,K]^T); fills the derived fields of ep.  force_tile 0 = heuristic.
-int gemm_i8_nt(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep,
-               int force_tile);
-int forced_i8_tile();
+// Y = epilogue(A[M,K] * Bt[N,K]^T); fills the derived fields of ep.
+int gemm_i8_nt(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep);
 // Convolution whose whole reduction fits one 64-byte slab (few input channels): rows gathered byte by byte, one launch.
-int conv_i8_gather(hipStream_t stream, const GatherConvRows &src, const int8_t *Wp, int M, int N, int Kp, I8Epilogue ep);
+int conv_i8_gather(const LaunchCfg &lc, const GatherConvRows &src, const int8_t *Wp, int M, int N, int Kp, I8Epilogue ep);
 // Convolution as an implicit GEMM: rows of A come from `src`, Wp is [N][K] with K = taps * Cg.
-int conv_i8_implicit(hipStream_t stream, const ConvRows &src, int Cg, const int8_t *Wp, int M, int N, int K, I8Epilogue ep,
-                     int force_tile);
+int conv_i8_implicit(const LaunchCfg &lc, const ConvRows &src, int Cg, const int8_t *Wp, int M, int N, int K, I8Epilogue ep);
 
 } // namespace sofie_hip

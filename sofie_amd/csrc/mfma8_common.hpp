@@ -2,7 +2,6 @@
 // the swizzled LDS slab layout and the tile store through LDS.
 #pragma once
 #include "common.hpp"
-#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -116,13 +115,6 @@ __device__ __forceinline__ void tile_of_block(int bid, int nwg, int tiles_m, int
    const int gsz = (tiles_m - first_m) < gm ? (tiles_m - first_m) : gm;
    tm = first_m + (id % width) % gsz;
    tn = (id % width) / gsz;
-}
-
-// SOFIE_HIP_SWIZZLE overrides the tile order (tuning); default: XCD regrouping, bands of 4 tile rows.
-inline int swizzle_mode()
-{
-   const char *s = getenv("SOFIE_HIP_SWIZZLE");
-   return s ? (int)strtol(s, nullptr, 0) : 4;
 }
 
 // Byte offset of 16-byte chunk c of row r in an LDS slab of BK-byte rows.  Chunk c is stored at chunk

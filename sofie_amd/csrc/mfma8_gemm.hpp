@@ -209,7 +209,7 @@ static int configure_lds_once(KERN kern, size_t smem, bool (&configured)[64])
 }
 
 template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, class EPI>
-static int launch_mfma8(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb,
+static int launch_mfma8(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb,
                         const EPI &ep, bool aligned)
 {
    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -219,20 +219,19 @@ static int launch_mfma8(hipStream_t stream, const int8_t *A, const int8_t *Bt, i
    constexpr size_t smem = mfma8_general_lds_bytes<BM, BN, BK, WAVES_M, WAVES_N>();
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
    RowMajorRows a{A, lda}, b{Bt, ldb};
-   const int sw = swizzle_mode();
-   int st;
+      int st;
    if (aligned) {
       auto kern = mfma8_gemm_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, true, EPI>;
       static bool configured[64] = {};
       if ((st = configure_lds_once(kern, smem, configured)))
          return st;
-      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n, sw);
+      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, lc.stream, a, b, M, N, K, ep, tiles_m, tiles_n, lc.swizzle);
    } else {
       auto kern = mfma8_gemm_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, false, EPI>;
       static bool configured[64] = {};
       if ((st = configure_lds_once(kern, smem, configured)))
          return st;
-      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n, sw);
+      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, lc.stream, a, b, M, N, K, ep, tiles_m, tiles_n, lc.swizzle);
    }
    return launch_status("mfma8_gemm_kernel");
 }
@@ -255,7 +254,7 @@ inline int pick_tile(int M, int N, int force_tile)
 // Convolution over few input channels as ONE launch: 256 x 64 tiles (one output pixel per thread in the gather), a single
 // 64-byte slab.  Wp is the packed weight [N][Kp], Kp = the reduction length rounded up to 16, at most 64.
 template <class EPI, int KP>
-static int launch_mfma8_gather_kp(hipStream_t stream, const GatherConvRows &a, const int8_t *Wp, int M, int N, const EPI &ep)
+static int launch_mfma8_gather_kp(const LaunchCfg &lc, const GatherConvRows &a, const int8_t *Wp, int M, int N, const EPI &ep)
 {
    constexpr int BM = 256, BN = 64, BK = 64;
    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -269,36 +268,37 @@ static int launch_mfma8_gather_kp(hipStream_t stream, const GatherConvRows &a, c
       return st;
    GatherConvRowsT<KP> src;
    static_cast<GatherConvRows &>(src) = a;
-   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), smem, stream, src, RowMajorRows{Wp, KP}, M, N, KP, ep, tiles_m, tiles_n, 0);
+   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), smem, lc.stream, src, RowMajorRows{Wp, KP}, M, N, KP, ep, tiles_m, tiles_n, 0);
    return launch_status("mfma8_gemm_kernel (gathered convolution)");
 }
 
 // Convolution over few input channels as ONE launch: 256 x 64 tiles (one output pixel per thread in the gather), a single
 // 64-byte slab.  Wp is the packed weight [N][Kp], Kp = the reduction length rounded up to 16, at most 64.
 template <class EPI>
-static int launch_mfma8_gather(hipStream_t stream, const GatherConvRows &a, const int8_t *Wp, int M, int N, int Kp, const EPI &ep)
+static int launch_mfma8_gather(const LaunchCfg &lc, const GatherConvRows &a, const int8_t *Wp, int M, int N, int Kp, const EPI &ep)
 {
    if (a.K > Kp)
       return fail(SOFIE_HIP_ERR_INVALID, "conv: the gathered form needs a reduction of at most 64 bytes");
    switch (Kp) {
-   case 16: return launch_mfma8_gather_kp<EPI, 16>(stream, a, Wp, M, N, ep);
-   case 32: return launch_mfma8_gather_kp<EPI, 32>(stream, a, Wp, M, N, ep);
-   case 48: return launch_mfma8_gather_kp<EPI, 48>(stream, a, Wp, M, N, ep);
-   case 64: return launch_mfma8_gather_kp<EPI, 64>(stream, a, Wp, M, N, ep);
+   case 16: return launch_mfma8_gather_kp<EPI, 16>(lc, a, Wp, M, N, ep);
+   case 32: return launch_mfma8_gather_kp<EPI, 32>(lc, a, Wp, M, N, ep);
+   case 48: return launch_mfma8_gather_kp<EPI, 48>(lc, a, Wp, M, N, ep);
+   case 64: return launch_mfma8_gather_kp<EPI, 64>(lc, a, Wp, M, N, ep);
    default: return fail(SOFIE_HIP_ERR_INVALID, "conv: the gathered form needs a reduction of at most 64 bytes");
    }
 }
 
 template <class MMA, class EPI>
-static int launch_mfma8_auto(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb,
-                             const EPI &ep, int force_tile)
+static int launch_mfma8_auto(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb,
+                             const EPI &ep)
 {
+   const int force_tile = lc.tile;
    const bool aligned = (K % 16 == 0) && (lda % 16 == 0) && (ldb % 16 == 0) && (((uintptr_t)A & 15) == 0) &&
                         (((uintptr_t)Bt & 15) == 0);
    switch (pick_tile(M, N, force_tile)) {
-   case 256: return launch_mfma8<MMA, 256, 256, 64, 2, 2, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, aligned);
-   case 128: return launch_mfma8<MMA, 128, 128, 64, 2, 2, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, aligned);
-   case 64: return launch_mfma8<MMA, 64, 64, 64, 2, 2, EPI>(stream, A, Bt, M, N, K, lda, ldb, ep, aligned);
+   case 256: return launch_mfma8<MMA, 256, 256, 64, 2, 2, EPI>(lc, A, Bt, M, N, K, lda, ldb, ep, aligned);
+   case 128: return launch_mfma8<MMA, 128, 128, 64, 2, 2, EPI>(lc, A, Bt, M, N, K, lda, ldb, ep, aligned);
+   case 64: return launch_mfma8<MMA, 64, 64, 64, 2, 2, EPI>(lc, A, Bt, M, N, K, lda, ldb, ep, aligned);
    default: return fail(SOFIE_HIP_ERR_INVALID, "gemm: unknown tile %d", force_tile);
    }
 }

@@ -11,7 +11,6 @@
 //     between the MFMAs of step s, so LDS traffic of the four waves spreads over the MFMA time.
 #pragma once
 #include "mfma8_gemm.hpp"
-#include <cstdlib>
 
 namespace sofie_hip {
 
@@ -28,7 +27,7 @@ __device__ __forceinline__ void wait_vmcnt()
 
 // OCC: workgroups meant to share a CU (waves per SIMD); 2 halves the register budget to 256 per lane so that one
 // workgroup's tile store overlaps the other's K loop.
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows, int OCC = 1>
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, class ASRC = RowMajorRows, int OCC = 1>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, OCC) void mfma8_gemm_dma_kernel(ASRC A, RowMajorRows Bt, int M, int N,
                                                                                 int K, EPI ep, int tiles_m, int tiles_n, int sw)
 {
@@ -81,8 +80,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, OCC) void mfma8_gemm_dma_ker
    static_assert(LPT % KS_ == 0, "slab loads must divide over the K-steps");
    auto issue_loads = [&](int kt, int stage, auto part_c) {
       constexpr int part = decltype(part_c)::value; // 0..KS-1, or -1 for the whole slab
-      if (DBG & 1)
-         return;
       int8_t *sA = smem + stage * STAGE_BYTES;
       int8_t *sB = sA + BM * BK;
       const int koff = kt * BK;
@@ -113,8 +110,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, OCC) void mfma8_gemm_dma_ker
       issue_loads(s < KT ? s : KT - 1, s, std::integral_constant<int, -1>{});
 
    auto read_frags = [&](const int8_t *cA, const int8_t *cB, int ks, frag_t(&fa)[MT], frag_t(&fb)[NT]) {
-      if (DBG & 2)
-         return;
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -165,10 +160,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, OCC) void mfma8_gemm_dma_ker
          for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int j = 0; j < NT; ++j)
-               if (!(DBG & 4))
-                  acc[i][j] = MMA::mma(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
-               else
-                  acc[i][j][0] += fb[ks & 1][j].c[0][0] + fa[ks & 1][i].c[0][0];
+               acc[i][j] = MMA::mma(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
          // issue order within the step: MFMAs with the LDS reads and the loads slotted in between
          constexpr int NMFMA = MT * NT;
          constexpr int NREAD = (MT + NT) * MMA::CHUNKS;
@@ -199,8 +191,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, OCC) void mfma8_gemm_dma_ker
    });
 }
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows, int OCC = 1>
-static int launch_mfma8_dma_src(hipStream_t stream, const ASRC &a, const int8_t *Bt, int M, int N, int K, int ldb,
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, class ASRC = RowMajorRows, int OCC = 1>
+static int launch_mfma8_dma_src(const LaunchCfg &lc, const ASRC &a, const int8_t *Bt, int M, int N, int K, int ldb,
                             const EPI &ep)
 {
    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -215,19 +207,19 @@ static int launch_mfma8_dma_src(hipStream_t stream, const ASRC &a, const int8_t 
    static_assert(smem * OCC <= 160 * 1024, "LDS ring larger than the CU's LDS");
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
    RowMajorRows b{Bt, ldb};
-   auto kern = mfma8_gemm_dma_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG, ASRC, OCC>;
+   auto kern = mfma8_gemm_dma_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, ASRC, OCC>;
    static bool configured[64] = {};
    if (int st = configure_lds_once(kern, smem, configured))
       return st;
-   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n, swizzle_mode());
+   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, lc.stream, a, b, M, N, K, ep, tiles_m, tiles_n, lc.swizzle);
    return launch_status("mfma8_gemm_dma_kernel");
 }
 
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0>
-static int launch_mfma8_dma(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI>
+static int launch_mfma8_dma(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
 {
-   return launch_mfma8_dma_src<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG, RowMajorRows>(stream, RowMajorRows{A, lda}, Bt, M, N, K, ldb, ep);
+   return launch_mfma8_dma_src<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, RowMajorRows>(lc, RowMajorRows{A, lda}, Bt, M, N, K, ldb, ep);
 }
 
 } // namespace sofie_hip

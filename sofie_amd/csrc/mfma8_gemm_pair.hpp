@@ -16,18 +16,8 @@
 
 namespace sofie_hip {
 
-#ifdef SOFIE_HIP_TUNING
-static __device__ unsigned long long dbg_ts[8192 * 4];
-#define SOFIE_TS(slot)                                                                              \
-   do {                                                                                             \
-      if (threadIdx.x == 0 && blockIdx.x < 8192)                                                    \
-         dbg_ts[blockIdx.x * 4 + (slot)] = wall_clock64();                                          \
-   } while (0)
-#else
-#define SOFIE_TS(slot) ((void)0)
-#endif
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows>
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, class ASRC = RowMajorRows>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(ASRC A, RowMajorRows Bt, int M, int N,
                                                                                  int K, EPI ep, int tiles_m, int tiles_n, int sw)
 {
@@ -50,7 +40,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
 
    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
 
-   SOFIE_TS(0);
    int tm, tn;
    tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, sw, tm, tn);
    const int m0 = tm * BM, n0 = tn * BN;
@@ -83,8 +72,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
    // slab 2*pair + q%2, so the two halves of a cache line are requested by consecutive instructions.
    auto issue_pair = [&](int pair, int slot0, int slot1, auto q0_c, auto q1_c) {
       constexpr int Q0 = decltype(q0_c)::value, Q1 = decltype(q1_c)::value;
-      if (DBG & 1)
-         return;
       const int koff = pair * 2 * BK;
       static_for<Q1 - Q0>([&](auto qc) {
          constexpr int q = Q0 + decltype(qc)::value;
@@ -116,8 +103,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
       issue_pair(p < KP ? p : KP - 1, 2 * p, 2 * p + 1, std::integral_constant<int, 0>{}, std::integral_constant<int, 2 * LPT>{});
 
    auto read_frags = [&](const int8_t *cA, const int8_t *cB, int ks, frag_t(&fa)[MT], frag_t(&fb)[NT]) {
-      if (DBG & 2)
-         return;
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -133,7 +118,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
    frag_t fa[2][MT], fb[2][NT];
    wait_vmcnt<(AHEAD - 1) * 2 * LPT>(); // pair 0 has landed
    __builtin_amdgcn_s_barrier();
-   SOFIE_TS(1);
    read_frags(smem, smem + BM * BK, 0, fa[0], fb[0]);
    int stage = 0;              // slot of the slab being computed
    int lslot0 = STAGES - 1;    // slots the next requested pair goes to: those of slabs 2p-1 and 2p
@@ -151,12 +135,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
             if (h == 1) {
                // issued so far, newest first: parts 0..KS-2 of pair kp+AHEAD, then pairs kp+AHEAD-1 ... kp+1.
                // Pair kp+1 must have landed (its first slab is read next, its second one a slab later).
-               if (!(DBG & 8))
-                  wait_vmcnt<(AHEAD - 2) * 2 * LPT + (KS - 1) * (2 * LPT / KS)>();
+               wait_vmcnt<(AHEAD - 2) * 2 * LPT + (KS - 1) * (2 * LPT / KS)>();
             }
             __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this wave's LDS reads of the current slab are complete
-            if (!(DBG & 16))
-               __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_s_barrier();
             read_frags(smem + nxt * STAGE_BYTES, smem + nxt * STAGE_BYTES + BM * BK, 0, fa[(g + 1) & 1], fb[(g + 1) & 1]);
          } else {
             read_frags(cA, cB, ks + 1, fa[(g + 1) & 1], fb[(g + 1) & 1]);
@@ -168,10 +150,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
          for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int j = 0; j < NT; ++j)
-               if (!(DBG & 4))
-                  acc[i][j] = MMA::mma(fb[g & 1][j], fa[g & 1][i], acc[i][j]);
-               else
-                  acc[i][j][0] += fb[g & 1][j].c[0][0] + fa[g & 1][i].c[0][0];
+               acc[i][j] = MMA::mma(fb[g & 1][j], fa[g & 1][i], acc[i][j]);
          // issue order within the step: MFMAs with the LDS reads and the loads slotted in between
          constexpr int NMFMA = MT * NT;
          constexpr int NREAD = (MT + NT) * MMA::CHUNKS;
@@ -181,14 +160,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
 #pragma unroll
          for (int gg = 0; gg < GROUPS; ++gg) {
             constexpr int HALF = MPG / 2 > 0 ? MPG / 2 : 1;
-            if (NLOAD > 0 && !(DBG & (64 | 128)))
+            if (NLOAD > 0)
                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, HALF, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, RPG - RPG / 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, MPG - HALF, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, RPG / 2, 0);
-            if (NLOAD > 0 && (DBG & 64))
-               __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
          }
       });
       stage = (stage + 2 >= STAGES) ? stage + 2 - STAGES : stage + 2;
@@ -198,16 +175,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_pair_kernel(
 
    wait_vmcnt<0>();
    __syncthreads();
-   SOFIE_TS(2);
    char *wsm = (char *)smem + wave * tile_store_lds_bytes(TN);
    ep.dispatch([&](auto mode) {
       tile_store_via_lds<decltype(mode)::value, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, M, N, lane, wsm);
    });
-   SOFIE_TS(3);
 }
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0, class ASRC = RowMajorRows>
-static int launch_mfma8_pair_src(hipStream_t stream, const ASRC &a, const int8_t *Bt, int M, int N, int K, int ldb,
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, class ASRC = RowMajorRows>
+static int launch_mfma8_pair_src(const LaunchCfg &lc, const ASRC &a, const int8_t *Bt, int M, int N, int K, int ldb,
                              const EPI &ep)
 {
    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -222,19 +197,19 @@ static int launch_mfma8_pair_src(hipStream_t stream, const ASRC &a, const int8_t
    static_assert(smem <= 160 * 1024, "LDS ring larger than the CU's LDS");
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
    RowMajorRows b{Bt, ldb};
-   auto kern = mfma8_gemm_pair_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG, ASRC>;
+   auto kern = mfma8_gemm_pair_kernel<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, ASRC>;
    static bool configured[64] = {};
    if (int st = configure_lds_once(kern, smem, configured))
       return st;
-   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, stream, a, b, M, N, K, ep, tiles_m, tiles_n, swizzle_mode());
+   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NTHREADS), smem, lc.stream, a, b, M, N, K, ep, tiles_m, tiles_n, lc.swizzle);
    return launch_status("mfma8_gemm_pair_kernel");
 }
 
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI, int DBG = 0>
-static int launch_mfma8_pair(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, class EPI>
+static int launch_mfma8_pair(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
 {
-   return launch_mfma8_pair_src<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, DBG, RowMajorRows>(stream, RowMajorRows{A, lda}, Bt, M, N, K, ldb, ep);
+   return launch_mfma8_pair_src<MMA, BM, BN, BK, WAVES_M, WAVES_N, STAGES, EPI, RowMajorRows>(lc, RowMajorRows{A, lda}, Bt, M, N, K, ldb, ep);
 }
 
 } // namespace sofie_hip

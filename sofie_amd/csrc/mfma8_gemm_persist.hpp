@@ -326,7 +326,7 @@ inline bool mfma8_persist_applies(const int8_t *A, const int8_t *Bt, int M, int 
 }
 
 template <class MMA, class EPI>
-static int launch_mfma8_persist(hipStream_t stream, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
+static int launch_mfma8_persist(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
 {
    const int tiles_m = M / 256, tiles_n = N / 256;
    const int ntiles = tiles_m * tiles_n;
@@ -346,7 +346,7 @@ static int launch_mfma8_persist(hipStream_t stream, const int8_t *A, const int8_
          cus[dev] = ncu;
    }
    const int grid = ntiles < ncu ? ntiles : ncu;
-   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, stream, A, Bt, lda, ldb, K, ep, tiles_m, tiles_n, swizzle_mode());
+   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, lc.stream, A, Bt, lda, ldb, K, ep, tiles_m, tiles_n, lc.swizzle);
    return launch_status("mfma8_gemm_persist_kernel");
 }
 

@@ -1,5 +1,6 @@
 // Context, stream, arena and copy entry points of include/sofie_hip.h.
 #include "common.hpp"
+#include <cstdlib>
 #include <new>
 
 namespace sofie_hip {
@@ -39,6 +40,22 @@ extern "C" {
 const char *sofie_hip_last_error(void) { return g_last_error; }
 int sofie_hip_abi_version(void) { return SOFIE_HIP_ABI_VERSION; }
 
+namespace {
+struct OptionName {
+   const char *name, *env;
+   int sofie_hip_options::*field;
+};
+const OptionName kOptionNames[] = {
+   {"swizzle", "SOFIE_HIP_SWIZZLE", &sofie_hip_options::swizzle},
+   {"i8_tile", "SOFIE_HIP_I8_TILE", &sofie_hip_options::i8_tile},
+   {"f8_tile", "SOFIE_HIP_F8_TILE", &sofie_hip_options::f8_tile},
+   {"gemm_variant", "SOFIE_HIP_GEMM_VARIANT", &sofie_hip_options::gemm_variant},
+   {"conv_explicit", "SOFIE_HIP_CONV_EXPLICIT", &sofie_hip_options::conv_explicit},
+   {"f32_skinny", "SOFIE_HIP_F32_SKINNY", &sofie_hip_options::f32_skinny},
+   {"f32_chain", "SOFIE_HIP_F32_CHAIN", &sofie_hip_options::f32_chain},
+};
+} // namespace
+
 int sofie_hip_ctx_create(sofie_hip_ctx **out, int device, void *external_stream)
 {
    SOFIE_HIP_REQUIRE(out != nullptr, "sofie_hip_ctx_create: out is NULL");
@@ -70,8 +87,22 @@ int sofie_hip_ctx_create(sofie_hip_ctx **out, int device, void *external_stream)
       delete ctx;
       return fail(SOFIE_HIP_ERR_RUNTIME, "hipEventCreate failed");
    }
+   for (const OptionName &o : kOptionNames)
+      if (const char *v = getenv(o.env))
+         ctx->opt.*(o.field) = (int)strtol(v, nullptr, 0);
    *out = ctx;
    return SOFIE_HIP_OK;
+}
+
+int sofie_hip_ctx_set_option(sofie_hip_ctx *ctx, const char *name, int32_t value)
+{
+   SOFIE_HIP_REQUIRE(ctx && name, "sofie_hip_ctx_set_option: NULL argument");
+   for (const OptionName &o : kOptionNames)
+      if (strcmp(name, o.name) == 0) {
+         ctx->opt.*(o.field) = value;
+         return SOFIE_HIP_OK;
+      }
+   return fail(SOFIE_HIP_ERR_INVALID, "sofie_hip_ctx_set_option: unknown option '%s'", name);
 }
 
 int sofie_hip_ctx_destroy(sofie_hip_ctx *ctx)

@@ -124,6 +124,8 @@ SYMBOLS = {
     "sofie_hip_unary_chain_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.POINTER(PostOps)]),
     "sofie_hip_conv_i8": (C.c_int, [_P, C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
     "sofie_hip_conv_i8_workspace": (C.c_size_t, [C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
+    "sofie_hip_conv_i8_column_matrix_bytes": (C.c_size_t, [C.POINTER(ConvDesc)]),
+    "sofie_hip_ctx_set_option": (C.c_int, [_P, C.c_char_p, C.c_int32]),
     "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),
     "sofie_hip_global_avg_pool_f32": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32]),
     "sofie_hip_pool_f32": (C.c_int, [_P, _P, _P, _P]),
@@ -139,7 +141,6 @@ SYMBOLS = {
     "sofie_hip_batchnorm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "sofie_hip_global_avg_pool_i8": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float]),
     "sofie_hip_conv_weight_i8_packed_bytes": (C.c_size_t, [C.POINTER(ConvDesc)]),
-    "sofie_hip_mfma_i8_probe": (C.c_int, [_P, _P, C.c_size_t, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
     "sofie_hip_timer_start": (C.c_int, [_P]),
     "sofie_hip_timer_stop": (C.c_int, [_P, C.POINTER(C.c_float)]),
 }
@@ -196,6 +197,10 @@ class Runtime:
 
     def call(self, name, *args):
         self._check(getattr(self.lib, name)(self.ctx, *args))
+
+    def set_option(self, name, value):
+        """Kernel-choice override of this context (see sofie_hip_ctx_set_option)."""
+        self.call("sofie_hip_ctx_set_option", name.encode(), int(value))
 
     def sync(self):
         self.call("sofie_hip_sync")

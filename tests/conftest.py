@@ -23,6 +23,21 @@ def rt():
     r.close()
 
 
+@pytest.fixture
+def opt(rt):
+    """opt(name, value) sets a kernel-choice override on the shared context (sofie_hip_ctx_set_option); the defaults are put
+    back when the test ends."""
+    defaults = {"swizzle": 4, "i8_tile": 0, "f8_tile": 0, "gemm_variant": 0, "conv_explicit": 0, "f32_skinny": -1, "f32_chain": -1}
+    touched = []
+
+    def set_option(name, value):
+        rt.set_option(name, value)
+        touched.append(name)
+    yield set_option
+    for name in touched:
+        rt.set_option(name, defaults[name])
+
+
 @pytest.fixture(scope="session", autouse=True)
 def _torch_initialises_the_gpu_first(request):
     """torch brings its own copy of the HIP runtime: whichever of torch and libsofie_hip.so touches the GPU first decides which copy the process uses.

@@ -24,7 +24,7 @@ CASES = [
 ]
 
 
-def run_conv(rt, X, Wt, bias, scale, case, relu, out, x_layout, y_layout, packed, ws_images=None):
+def run_conv(rt, X, Wt, bias, scale, case, relu, out, x_layout, y_layout, packed, ws_images=None, column_matrix=False):
     N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
     d = conv_desc(N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group)
     Xd = X if x_layout == R.LAYOUT_NCHW else np.ascontiguousarray(X.transpose(0, 2, 3, 1))
@@ -47,6 +47,8 @@ def run_conv(rt, X, Wt, bias, scale, case, relu, out, x_layout, y_layout, packed
     need = rt.lib.sofie_hip_conv_i8_workspace(C.byref(d), C.byref(a))
     if ws_images:
         need = need * ws_images
+    if column_matrix:  # room for what the "conv_explicit" option needs on top of the minimum
+        need += rt.lib.sofie_hip_conv_i8_column_matrix_bytes(C.byref(d)) * (ws_images or 1)
     ws = util.dev_empty((need + 256,), np.int8)
     a.workspace, a.workspace_bytes = util.ptr(ws), need
     import torch
@@ -61,18 +63,18 @@ def run_conv(rt, X, Wt, bias, scale, case, relu, out, x_layout, y_layout, packed
 @pytest.mark.parametrize("case", CASES)
 @pytest.mark.parametrize("x_layout,y_layout,packed", [(0, 0, 0), (1, 1, 1), (0, 1, 0), (1, 0, 1)])
 @pytest.mark.parametrize("column_matrix", [0, 1])
-def test_conv_i8_requant_bit_exact(rt, case, x_layout, y_layout, packed, column_matrix, monkeypatch):
+def test_conv_i8_requant_bit_exact(rt, case, x_layout, y_layout, packed, column_matrix, opt):
     # column_matrix = 1 forces the explicit int8 im2col + GEMM; 0 lets the runtime choose: reductions of at most 64 bytes
     # (the first six cases) are gathered inside the GEMM kernel, 64-channel NHWC input takes the implicit GEMM
     if column_matrix:
-        monkeypatch.setenv("SOFIE_HIP_CONV_EXPLICIT", "1")
+        opt("conv_explicit", 1)
     N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
     X = util.int8_sym(50, N * Cc * H * W).reshape(N, Cc, H, W)
     Wt = util.int8_sym(51, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
     bias = util.int32_range(52, Cout, -2000, 2000)
     K = (Cc // group) * kh * kw
     scale = ((0.5 + util.uniform01(53, Cout)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
-    got = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, x_layout, y_layout, packed, ws_images=2)
+    got = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, x_layout, y_layout, packed, ws_images=2, column_matrix=bool(column_matrix))
     want = ob.conv_i8(X, Wt, bias, scale, pads=pads, strides=strides, dils=dils, group=group, relu=1, out=2, omp=True)
     assert np.array_equal(got, want)
 
@@ -109,9 +111,9 @@ def test_global_avg_pool_i8_both_layouts(rt, N, Cc, H, W):
     (2, 128, 10, 10, 64, 3, 2, (2, 0, 1, 1), (2, 1), (1, 2), 2),       # groups, stride, dilation, asymmetric pads
     (1, 64, 7, 7, 32, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1), 1),          # 1x1
 ])
-def test_conv_i8_implicit_gemm_every_tile(rt, case, tile, monkeypatch):
+def test_conv_i8_implicit_gemm_every_tile(rt, case, tile, opt):
     """NHWC input with a power-of-two channel count >= 64 takes the implicit-GEMM kernels (no column matrix)."""
-    monkeypatch.setenv("SOFIE_HIP_I8_TILE", str(tile))
+    opt("i8_tile", tile)
     N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
     X = util.int8_sym(80, N * Cc * H * W).reshape(N, Cc, H, W)
     Wt = util.int8_sym(81, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
@@ -122,9 +124,9 @@ def test_conv_i8_implicit_gemm_every_tile(rt, case, tile, monkeypatch):
     got = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, R.LAYOUT_NHWC, R.LAYOUT_NHWC, 1)
     assert np.array_equal(got, want)
     # and the explicit column-matrix path gives the same bits
-    monkeypatch.setenv("SOFIE_HIP_CONV_EXPLICIT", "1")
-    monkeypatch.delenv("SOFIE_HIP_I8_TILE")
-    got2 = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, R.LAYOUT_NHWC, R.LAYOUT_NCHW, 1)
+    opt("conv_explicit", 1)
+    opt("i8_tile", 0)
+    got2 = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, R.LAYOUT_NHWC, R.LAYOUT_NCHW, 1, column_matrix=True)
     assert np.array_equal(got2, want)
 
 
@@ -145,7 +147,7 @@ def test_first_layer_of_an_image_network_needs_no_workspace(rt):
     assert np.array_equal(got, want) and (want > 0).any()
 
 
-def run_conv_plane_sums(rt, X, Wt, bias, scale, case, relu, x_layout, forced_tile=None, monkeypatch=None):
+def run_conv_plane_sums(rt, X, Wt, bias, scale, case, relu, x_layout):
     """sofie_hip_conv_i8 with SOFIE_I8OUT_I8_PLANE_SUMS into a cleared int32 [N, Cout], then the average."""
     N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
     d = conv_desc(N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group)
@@ -162,7 +164,7 @@ def run_conv_plane_sums(rt, X, Wt, bias, scale, case, relu, x_layout, forced_til
     assert rt.lib.sofie_hip_conv_i8_workspace(C.byref(d), C.byref(a)) == 0
     import torch
     torch.cuda.synchronize()
-    print("conv_i8 plane sums", case, relu, x_layout, forced_tile, flush=True)
+    print("conv_i8 plane sums", case, relu, x_layout, flush=True)
     rt.call("sofie_hip_fill_zero", util.ptr(dS), C.c_size_t(N * Cout * 4))
     rt.call("sofie_hip_conv_i8", C.byref(d), C.byref(a))
     rt.call("sofie_hip_plane_sums_to_average", util.ptr(dY), util.ptr(dS), N * Cout, d.OH * d.OW, C.c_float(0.037))
@@ -185,11 +187,11 @@ PLANE_SUM_CASES = [
 @pytest.mark.parametrize("case,x_layout", PLANE_SUM_CASES)
 @pytest.mark.parametrize("relu", [0, 1])
 @pytest.mark.parametrize("tile", [0, 64, 128, 256, 258])
-def test_conv_i8_plane_sums_equal_the_sums_of_the_stored_map(rt, case, x_layout, relu, tile, monkeypatch):
+def test_conv_i8_plane_sums_equal_the_sums_of_the_stored_map(rt, case, x_layout, relu, tile, opt):
     """The int8 feature map is never stored: the sums the kernel adds up in its store must be the sums of the map the
     oracle computes, and the average the bits of the oracle's DequantizeLinear + GlobalAveragePool on that map."""
     if tile:
-        monkeypatch.setenv("SOFIE_HIP_I8_TILE", str(tile))
+        opt("i8_tile", tile)
     N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
     X = util.int8_sym(70, N * Cc * H * W).reshape(N, Cc, H, W)
     Wt = util.int8_sym(71, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
@@ -202,7 +204,7 @@ def test_conv_i8_plane_sums_equal_the_sums_of_the_stored_map(rt, case, x_layout,
         with pytest.raises(R.SofieHipError, match="multiple of 256"):
             run_conv_plane_sums(rt, X, Wt, bias, scale, case, relu, x_layout)
         return
-    sums, avg = run_conv_plane_sums(rt, X, Wt, bias, scale, case, relu, x_layout, tile)
+    sums, avg = run_conv_plane_sums(rt, X, Wt, bias, scale, case, relu, x_layout)
     fmap = ob.conv_i8(X, Wt, bias, scale, pads=pads, strides=strides, dils=dils, group=group, relu=relu, out=2, omp=True)
     want_sums = fmap.astype(np.int64).sum(axis=(2, 3))
     assert np.array_equal(sums, want_sums.astype(np.int32))

@@ -42,9 +42,9 @@ def close(got, want, mag, rel=1e-5):
                                                  (7, 5, 3, 1, 0), (65, 67, 33, 1, 1), (1, 1, 1, 0, 0), (130, 70, 257, 0, 0), (9, 17, 520, 0, 1), (12, 20, 600, 1, 0)])
 @pytest.mark.parametrize("bias_mode,act", [(0, 0), (1, 1), (2, 0), (3, 2), (4, 3), (1, 4)])
 @pytest.mark.parametrize("kernel", ["tiles64", "wave8x8"])
-def test_gemm_f32_matches_sofie_cpu_semantics(rt, M, N, K, transA, transB, bias_mode, act, kernel, monkeypatch):
+def test_gemm_f32_matches_sofie_cpu_semantics(rt, M, N, K, transA, transB, bias_mode, act, kernel, opt):
     # both fp32 kernels on every shape: the 64x64-tile one and the one-wave 8x8-tile one for small products
-    monkeypatch.setenv("SOFIE_HIP_F32_SKINNY", "1" if kernel == "wave8x8" else "0")
+    opt("f32_skinny", 1 if kernel == "wave8x8" else 0)
     A = util.normal(1, M * K).reshape((K, M) if transA else (M, K))
     B = util.normal(2, N * K, 0.05).reshape((N, K) if transB else (K, N))
     Cshape = {0: None, 1: (N,), 2: (M, 1), 3: (1,), 4: (M, N)}[bias_mode]
@@ -260,8 +260,8 @@ def test_chain_errors(rt):
 
 @pytest.mark.parametrize("kernel", ["tiles64", "wave8x8"])
 @pytest.mark.parametrize("M,N,K", [(6, 12, 20), (70, 33, 129)])
-def test_gemm_with_a_chain_in_its_store(rt, M, N, K, kernel, monkeypatch):
-    monkeypatch.setenv("SOFIE_HIP_F32_SKINNY", "1" if kernel == "wave8x8" else "0")
+def test_gemm_with_a_chain_in_its_store(rt, M, N, K, kernel, opt):
+    opt("f32_skinny", 1 if kernel == "wave8x8" else 0)
     A = util.normal(410, M * K).reshape(M, K)
     B = util.normal(411, K * N, 0.1).reshape(K, N)
     bias = util.normal(412, N)
@@ -302,9 +302,9 @@ def test_conv_with_a_chain_in_its_store(rt):
 
 @pytest.mark.parametrize("kernel", ["tiles64", "wave8x8"])
 @pytest.mark.parametrize("M,N,K,batch", [(6, 12, 20, 1), (70, 33, 129, 1), (9, 10, 16, 3)])
-def test_gemm_with_a_residual_operand(rt, M, N, K, batch, kernel, monkeypatch):
+def test_gemm_with_a_residual_operand(rt, M, N, K, batch, kernel, opt):
     """Y = act(alpha A B + bias + R): the Add of a same-shaped tensor behind the product, inside the store, before the activation."""
-    monkeypatch.setenv("SOFIE_HIP_F32_SKINNY", "1" if kernel == "wave8x8" else "0")
+    opt("f32_skinny", 1 if kernel == "wave8x8" else 0)
     A = util.normal(430, batch * M * K).reshape(batch, M, K)
     B = util.normal(431, K * N, 0.1).reshape(K, N)
     bias = util.normal(432, N)

@@ -131,13 +131,13 @@ def check_fp8_against_oracle(got_f32, A, Bt, bias, scale, act, bf16):
                                         (512, 1280, 512, 1152)])
 @pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("out,act", [(1, R.ACT_NONE), (0, R.ACT_GELU)])
-def test_every_fp8_tile_configuration(rt, monkeypatch, tile, M, N, K, variant, out, act):
+def test_every_fp8_tile_configuration(rt, opt, tile, M, N, K, variant, out, act):
     """Every tile kernel of the FP8 product, forced: 64 / 128 / 256 (pipelined kernels when K is a multiple of 128, the general one
     otherwise; variant 1 = the alternative pipelined kernel) and 512 = the persistent kernel with the tile store from registers."""
     if tile == 512 and variant:
         pytest.skip("the persistent kernel has one form")
-    monkeypatch.setenv("SOFIE_HIP_F8_TILE", str(tile))
-    monkeypatch.setenv("SOFIE_HIP_GEMM_VARIANT", str(variant))
+    opt("f8_tile", tile)
+    opt("gemm_variant", variant)
     A, sa = make_fp8(4101 + M, M, K)
     Bt, sb = make_fp8(4102 + N, N, K)
     bias = util.normal(4103, N)

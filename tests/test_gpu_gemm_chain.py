@@ -101,10 +101,10 @@ def test_the_benchmark_mlp_as_a_chain(rt, M, transB):
 
 
 @pytest.mark.parametrize("fused", ["0", "1"])
-def test_chain_with_every_epilogue_feature(rt, fused, monkeypatch):
+def test_chain_with_every_epilogue_feature(rt, fused, opt):
     """Odd widths, both weight layouts, alpha, every bias mode, an activation with a chain behind it, a residual: the one-launch
     form and the layer-by-layer form of the same call agree with the oracle."""
-    monkeypatch.setenv("SOFIE_HIP_F32_CHAIN", fused)
+    opt("f32_chain", int(fused))
     M = 37
     X = util.normal(930, M * 50).reshape(M, 50)
     layers = [

@@ -1,6 +1,5 @@
 """Parity of the int8 MFMA GEMM (through the C-ABI) with the CPU oracle: bit-exact."""
 import ctypes as C
-import os
 
 import numpy as np
 import pytest
@@ -56,14 +55,11 @@ def test_int32_accumulate_matches_oracle(rt, M, N, K):
 
 @pytest.mark.parametrize("tile", [64, 128, 256, 258])     # 258: the 256 x 128 tile that shares a CU with a second workgroup
 @pytest.mark.parametrize("M,N,K", [(300, 520, 1024), (96, 160, 80), (513, 257, 2048 + 48)])
-def test_every_tile_configuration(rt, tile, M, N, K):
+def test_every_tile_configuration(rt, opt, tile, M, N, K):
     A = util.int8_sym(11, M * K).reshape(M, K)
     Bt = util.int8_sym(12, N * K).reshape(N, K)
-    os.environ["SOFIE_HIP_I8_TILE"] = str(tile)
-    try:
-        got = run_gemm(rt, A, Bt, M, N, K, transB=1, out=R.I8OUT_I32)
-    finally:
-        del os.environ["SOFIE_HIP_I8_TILE"]
+    opt("i8_tile", tile)
+    got = run_gemm(rt, A, Bt, M, N, K, transB=1, out=R.I8OUT_I32)
     assert np.array_equal(got, ob.matmul_integer(A, Bt, M=M, N=N, K=K, transB=1, omp=True))
 
 
@@ -186,7 +182,7 @@ def test_short_reduction_over_many_tiles_takes_the_shared_cu_tile(rt):
 @pytest.mark.parametrize("out,relu_acc,relu_out", [(R.I8OUT_I32, 0, 0), (R.I8OUT_F32, 1, 0), (R.I8OUT_I8, 0, 1), (R.I8OUT_I8, 0, 0),
                                                    (R.I8OUT_I8_DQQ, 1, 0)])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 384), (512, 768, 512), (1280, 512, 1152), (256, 4352, 640)])
-def test_persistent_kernel_forced_on_small_shapes(rt, out, relu_acc, relu_out, M, N, K):
+def test_persistent_kernel_forced_on_small_shapes(rt, opt, out, relu_acc, relu_out, M, N, K):
     """Tile 512 asks for the persistent 256 x 256 kernel (eight waves, tile store from registers) where the heuristic would
     not pick it: one tile, fewer tiles than CUs, more tiles than CUs (17 x 1 and 5 x 2 lists of uneven length per workgroup
     do not occur at these sizes, so the 4352-column case gives workgroups 0..16 one tile each), K of 3, 4, 5 and 9 slab pairs."""
@@ -195,11 +191,8 @@ def test_persistent_kernel_forced_on_small_shapes(rt, out, relu_acc, relu_out, M
     bias = util.int32_range(53, N, -(1 << 15), 1 << 15)
     scale = ((0.5 + util.uniform01(54, N)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
     kw = dict(bias=bias, scale=scale, q_scale=np.float32(0.041), relu_acc=relu_acc, relu_out=relu_out, out=out)
-    os.environ["SOFIE_HIP_I8_TILE"] = "512"
-    try:
-        got = run_gemm(rt, A, Bt, M, N, K, transB=1, **kw)
-    finally:
-        del os.environ["SOFIE_HIP_I8_TILE"]
+    opt("i8_tile", 512)
+    got = run_gemm(rt, A, Bt, M, N, K, transB=1, **kw)
     want = ob.gemm_i8(A, Bt, M=M, N=N, K=K, transB=1, omp=True, **kw)
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
 
