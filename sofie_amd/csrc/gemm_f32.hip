@@ -533,6 +533,44 @@ int sofie_hip_gemm_chain_f32(sofie_hip_ctx *ctx, const sofie_gemm_f32_desc *laye
       L.ep.ldr = ldy;
       width = d.N > width ? d.N : width;
    }
+   // In one launch a workgroup takes ITS rows through every layer, independently of the other workgroups.  Two tensors of the
+   // chain may therefore share memory only row for row (same address, same pitch, same width: the ping-pong of equal layers,
+   // where a row is rewritten by the workgroup that owns it); any other overlap of what a layer writes with what a layer
+   // reads or writes would let one workgroup's rows land on another's.  Callers that planned the layers' tensors by
+   // per-layer lifetimes get the layer-by-layer form then.
+   if (fused) {
+      struct Range {
+         const char *lo, *hi;
+         long long pitch, width;
+      };
+      auto range = [](const void *p, long long bytes, long long pitch, long long w) {
+         return Range{(const char *)p, (const char *)p + (bytes > 0 ? bytes : 0), pitch, w};
+      };
+      auto overlap = [](const Range &x, const Range &y) { return x.lo < y.hi && y.lo < x.hi; };
+      auto same_rows = [](const Range &x, const Range &y) { return x.lo == y.lo && x.pitch == y.pitch && x.width == y.width; };
+      Range reads[2 * SOFIE_MAX_GEMM_CHAIN], writes[SOFIE_MAX_GEMM_CHAIN];
+      int nr = 0;
+      const Range input = range(layers[0].A, ((long long)(M - 1) * a.lda + layers[0].K) * 4, a.lda, layers[0].K);
+      for (int l = 0; l < count; ++l) {
+         const sofie_gemm_f32_desc &d = layers[l];
+         const long long ldy = d.ldy ? d.ldy : d.N, ybytes = ((long long)(M - 1) * ldy + d.N) * 4;
+         writes[l] = range(d.Y, ybytes, ldy, d.N);
+         if (d.bias_mode != SOFIE_BIAS_NONE)
+            reads[nr++] = range(d.C, 4LL * (d.bias_mode == SOFIE_BIAS_ROW ? d.N : d.bias_mode == SOFIE_BIAS_COL ? M : d.bias_mode == SOFIE_BIAS_FULL ? (long long)M * d.N : 1), 0, 0);
+         if (d.residual)
+            reads[nr++] = range(d.residual, ybytes, 0, 0);
+      }
+      for (int l = 0; l < count && fused; ++l) {
+         if (overlap(writes[l], input) && !same_rows(writes[l], input))
+            fused = false;
+         for (int m = 0; m < l && fused; ++m)
+            if (overlap(writes[l], writes[m]) && !same_rows(writes[l], writes[m]))
+               fused = false;
+         for (int r = 0; r < nr && fused; ++r)
+            if (overlap(writes[l], reads[r]))
+               fused = false;
+      }
+   }
    const int RB = M <= 64 ? 1 : M <= 128 ? 2 : 4;
    width = (width + 3) / 4 * 4;
    if (fused && (long long)RB * width <= 8192) {

@@ -14,6 +14,8 @@
 #include <memory>
 #include <string>
 #include <unordered_map>
+#include <set>
+#include <utility>
 #include <vector>
 
 namespace SOFIE_HIP {
@@ -108,6 +110,11 @@ private:
    void TryFuseResidual(std::size_t i);
    void TryFusePlaneSums(std::size_t i);
    void PlanMemory();
+   void PlanMemoryPass(const std::set<std::size_t> &wholeChain);
+   // Runs of consecutive Gemm operators of which each reads what the one before wrote: {first operator, count >= 2}.
+   // Such a run goes to the runtime as ONE call that may execute every layer in a single launch, so the memory plan
+   // treats it as one operator.
+   std::vector<std::pair<std::size_t, std::size_t>> GemmChains() const;
    void GenerateSessionCode(std::underlying_type_t<Options> options);
    void WriteWeightFile(const std::string &filename) const;
    void WriteSafetensorsFile(const std::string &filename) const;

@@ -428,7 +428,73 @@ void RModel::Initialize(int batchSize)
 // workspaces, placed by OrganizeMemory from their lifetimes [producer, last consumer + 1), as the reference's
 // GPU generator does (core/src/RModel_ALPAKA.cxx:360-540).
 // ---------------------------------------------------------------------------------------------------------
+std::vector<std::pair<std::size_t, std::size_t>> RModel::GemmChains() const
+{
+   std::vector<std::pair<std::size_t, std::size_t>> chains;
+   for (std::size_t i = 0; i < fOperators.size(); ++i) {
+      std::size_t n = 0;
+      const ROperator_Gemm<float> *prev = nullptr;
+      for (std::size_t j = i; j < fOperators.size() && n < kMaxGemmChain; ++j) {
+         auto *g = dynamic_cast<const ROperator_Gemm<float> *>(fOperators[j].get());
+         if (!g || !g->IsChainLink() || (prev && g->NameA() != prev->NameY()))
+            break;
+         prev = g;
+         ++n;
+      }
+      if (n >= 2) {
+         chains.emplace_back(i, n);
+         i += n - 1;
+      }
+   }
+   return chains;
+}
+
 void RModel::PlanMemory()
+{
+   std::set<std::size_t> wholeChain; // first operators of the chains whose tensors must not share memory at all
+   for (;;) {
+      PlanMemoryPass(wholeChain);
+      bool again = false;
+      for (auto &ch : GemmChains()) {
+         if (wholeChain.count(ch.first))
+            continue;
+         // what the layers of this chain read and write, with its shape
+         std::vector<std::pair<std::string, std::vector<std::size_t>>> tensors;
+         for (std::size_t i = ch.first; i < ch.first + ch.second; ++i) {
+            for (auto &n : fOperators[i]->GetInputTensorNames())
+               tensors.emplace_back("tensor_" + std::string(n), GetTensorShape(std::string(n)));
+            for (auto &n : fOperators[i]->GetOutputTensorNames())
+               tensors.emplace_back("tensor_" + std::string(n), GetTensorShape(std::string(n)));
+         }
+         bool clash = false;
+         for (std::size_t x = 0; x < tensors.size() && !clash; ++x)
+            for (std::size_t y = x + 1; y < tensors.size() && !clash; ++y) {
+               if (tensors[x].first == tensors[y].first || !fOffsets.count(tensors[x].first) || !fOffsets.count(tensors[y].first))
+                  continue;
+               const PlannedTensor *px = nullptr, *py = nullptr;
+               for (auto &e : fPlan) {
+                  if (e.name == tensors[x].first)
+                     px = &e;
+                  if (e.name == tensors[y].first)
+                     py = &e;
+               }
+               if (!px || !py || px->perBatch != py->perBatch) // the per-entry region of a run-time batch lies apart from the static one
+                  continue;
+               const bool overlap = px->offset < py->offset + py->bytes && py->offset < px->offset + px->bytes;
+               if (overlap && !(px->offset == py->offset && tensors[x].second == tensors[y].second))
+                  clash = true;
+            }
+         if (clash) {
+            wholeChain.insert(ch.first);
+            again = true;
+         }
+      }
+      if (!again)
+         break;
+   }
+}
+
+void RModel::PlanMemoryPass(const std::set<std::size_t> &wholeChain)
 {
    fPlan.clear();
    fOffsets.clear();
@@ -468,6 +534,19 @@ void RModel::PlanMemory()
       if (fIntermediateTensorInfos.count(n))
          addGraphTensor(n, fIntermediateTensorInfos[n]);
 
+   // A Gemm chain may run all its layers in one launch, every workgroup taking its rows through all the layers on its own.
+   // Tensors of the chain may then share memory only row for row (equal shapes at the same offset: the ping-pong of equal
+   // layers).  The plan is made from per-operator lifetimes first; a chain in which two tensors of different shape came to
+   // share bytes is planned again with everything it touches live from its first operator to its last (`wholeChain`).
+   std::vector<int> opFirst(fOperators.size()), opLast(fOperators.size());
+   for (std::size_t i = 0; i < fOperators.size(); ++i)
+      opFirst[i] = opLast[i] = (int)i;
+   for (auto &ch : GemmChains())
+      if (wholeChain.count(ch.first))
+         for (std::size_t i = ch.first; i < ch.first + ch.second; ++i) {
+            opFirst[i] = (int)ch.first;
+            opLast[i] = (int)(ch.first + ch.second - 1);
+         }
    std::vector<TensorLifeInfo> life;
    std::vector<std::string> names;
    for (std::size_t i = 0; i < fOperators.size(); ++i) {
@@ -479,12 +558,12 @@ void RModel::PlanMemory()
             addStatic("tensor_" + y, tensorBytes(ti));
             continue;
          }
-         int last = (int)i;
+         int last = opLast[i];
          for (std::size_t j = i + 1; j < fOperators.size(); ++j)
             for (auto &in : fOperators[j]->GetInputTensorNames())
                if (in == y)
-                  last = (int)j;
-         life.push_back({(int)i, last + 1, dyn ? alignEntry(tensorBytes(ti)) : AlignUp(tensorBytes(ti))});
+                  last = std::max(last, opLast[j]);
+         life.push_back({opFirst[i], last + 1, dyn ? alignEntry(tensorBytes(ti)) : AlignUp(tensorBytes(ti))});
          names.push_back("tensor_" + y);
       }
       if (std::size_t ws = fOperators[i]->GetWorkspaceBytes()) {
@@ -1067,16 +1146,15 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    gc << ")\n   {";
    if (dyn)
       gc << "\n      (void)sofie_batch;";
+   const auto chains = GemmChains(); // the runs the memory plan was made for
    for (std::size_t i = 0; i < fOperators.size(); ++i) {
       // Consecutive products of which each reads what the one before wrote (the layers of an MLP) go to the runtime as one
       // call: at small batch it runs them in a single launch, otherwise layer by layer -- the results are the same.
       std::vector<ROperator_Gemm<float> *> chain;
-      for (std::size_t j = i; j < fOperators.size() && chain.size() < kMaxGemmChain; ++j) {
-         auto *g = dynamic_cast<ROperator_Gemm<float> *>(fOperators[j].get());
-         if (!g || !g->IsChainLink() || (!chain.empty() && g->NameA() != chain.back()->NameY()))
-            break;
-         chain.push_back(g);
-      }
+      for (auto &ch : chains)
+         if (ch.first == i)
+            for (std::size_t j = i; j < i + ch.second; ++j)
+               chain.push_back(static_cast<ROperator_Gemm<float> *>(fOperators[j].get()));
       if (chain.size() < 2) {
          gc << fOperators[i]->Generate_GPU_HIP(std::to_string(i));
          continue;

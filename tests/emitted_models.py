@@ -154,6 +154,19 @@ def classifier_head(batch=4):
                 feeds=[X])
 
 
+def gemm_chain_widths(batch=64):
+    """X[64,32] -> Gemm(128) -> Gemm(64) -> Gemm(96) -> Softmax: three products of different widths that the generator hands to the
+    runtime as one call; planned by per-operator lifetimes, the third output would take the start of the first one's memory with a
+    different row pitch."""
+    init = {"W0": util.normal(6401, 32 * 128, 0.2).reshape(32, 128), "b0": util.normal(6402, 128, 0.1),
+            "W1": util.normal(6403, 128 * 64, 0.1).reshape(128, 64), "b1": util.normal(6404, 64, 0.1),
+            "W2": util.normal(6405, 64 * 96, 0.1).reshape(64, 96), "b2": util.normal(6406, 96, 0.1)}
+    nodes = [ow.node("Gemm", ["X", "W0", "b0"], ["Y0"]), ow.node("Gemm", ["Y0", "W1", "b1"], ["Y1"]), ow.node("Gemm", ["Y1", "W2", "b2"], ["Y2"]),
+             ow.node("Softmax", ["Y2"], ["P"], axis=1)]
+    X = util.normal(6407, batch * 32).reshape(batch, 32)
+    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 32])], outputs=[("P", np.float32, [batch, 96])], init=init, feeds=[X])
+
+
 def shape_plumbing(batch=3):
     """Reshape (with 0 and -1), Transpose, Squeeze / Unsqueeze (axes as input and as attribute), Concat and Flatten around a Gemm:
     X [b, 2, 3, 4] -> Transpose(0, 2, 1, 3) -> Reshape [0, 3, -1] -> Concat with Z [b, 3, 2] along the last axis -> Unsqueeze(1) -> Squeeze(1)
@@ -418,6 +431,7 @@ CONFIG_MODELS = {
     "ShapePlumbing": lambda: shape_plumbing(3),
     "Config5_int8_CNN_small": lambda: int8_cnn(2, 12),
     "Int8_CNN_plane_sums": lambda: int8_cnn(2, 16, (3, 64, 128)),   # planes of 256 pixels: the last convolution sums them itself
+    "GemmChainWidths": lambda: gemm_chain_widths(64),
     "Config1_fp32_MLP": lambda: fp32_mlp(64),
     "Config2_int8_MLP_small": lambda: int8_mlp([64, 128, 96, 32], 48),
     "Config2_int8_MLP_mid": lambda: int8_mlp([256, 512, 512, 256], 256),

@@ -69,6 +69,24 @@ def test_plan_alignment_and_liveness(emitted, tmp_path, model):
         assert pool <= sum(r["bytes"] for r in pooled)
 
 
+def test_tensors_of_a_gemm_chain_share_no_memory(emitted, tmp_path):
+    """Three Gemms of different widths that go to the runtime as one call (which may run them in one launch, every workgroup
+    taking its rows through all the layers): tensors of different shape would share memory under per-operator lifetimes, so
+    the chain's input, outputs and biases are planned as live for the whole chain.  (Equal shapes may share row for row: the
+    reference's ping-pong of Linear_16 stays, see test_linear16_pool_matches_the_reference_planner.)"""
+    arena, pool, rows = plan_of(os.path.join(emitted, "GemmChainWidths.onnx"), tmp_path)
+    txt = read(emitted, "GemmChainWidths")
+    assert "sofie_hip_gemm_chain_f32(fCtx, chain, 3)" in txt
+    chain = [r for r in rows if r["name"] in ("tensor_X", "tensor_Y0", "tensor_Y1", "tensor_Y2", "tensor_b0", "tensor_b1", "tensor_b2",
+                                              "tensor_W0", "tensor_W1", "tensor_W2")]
+    assert len(chain) == 10
+    for i, a in enumerate(chain):
+        for b in chain[i + 1:]:
+            assert a["offset"] + a["bytes"] <= b["offset"] or b["offset"] + b["bytes"] <= a["offset"], (a, b)
+    y = {r["name"]: r for r in rows}
+    assert y["tensor_Y0"]["first"] == 0 and y["tensor_Y0"]["last"] >= 3 and y["tensor_Y1"]["first"] == 0 and y["tensor_Y2"]["first"] == 0
+
+
 def read(emitted, model):
     return open(os.path.join(emitted, model + "_GPU_HIP.hxx")).read()
 

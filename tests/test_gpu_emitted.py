@@ -263,6 +263,17 @@ def test_emitted_classifier_head_with_softmax_and_logsoftmax(rt):
     assert txt.count("sofie_hip_softmax_f32(") == 2 and "sofie_hip_gemm_chain_f32(fCtx, chain, 2)" in txt
 
 
+def test_emitted_gemm_chain_of_different_widths(rt):
+    """Three Gemms of widths 128 / 64 / 96 emitted as one chain call, then Softmax: the Session's own memory plan under the
+    one-launch kernel."""
+    spec = em.gemm_chain_widths(64)
+    g = onnx_lite.load(os.path.join(em.OUT, "GemmChainWidths.onnx"))
+    want = gr.run(g, spec["feeds"], gr.OracleBackend()).ravel()
+    print("emitted GemmChainWidths", flush=True)
+    got = run_emitted("GemmChainWidths", spec["feeds"], want.size)
+    assert np.all(np.abs(got - want) <= 1e-5 * want + 1e-7) and want.std() > 1e-4
+
+
 def test_emitted_layernorm_block(rt):
     spec = em.layernorm_block(3)
     X = spec["feeds"][0]

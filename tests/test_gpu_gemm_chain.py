@@ -13,9 +13,10 @@ from tests import util
 pytestmark = pytest.mark.gpu
 
 
-def run_chain(rt, X, layers):
+def run_chain(rt, X, layers, alias=None):
     """layers: dicts with W (stored as given), transB, bias (or None), bias_mode, act, act_alpha, alpha, post (list or None),
-    residual (array of the output's shape or None).  Returns the device results of every layer."""
+    residual (array of the output's shape or None).  alias = {l: m}: layer l writes into the buffer of layer m < l (same
+    size).  Returns the device results of every layer."""
     n = len(layers)
     descs = (R.GemmF32Desc * n)()
     keep, outs = [], []
@@ -26,7 +27,7 @@ def run_chain(rt, X, layers):
         dW = util.to_dev(L["W"])
         dC = None if L.get("bias") is None else util.to_dev(L["bias"])
         dR = None if L.get("residual") is None else util.to_dev(L["residual"])
-        dY = util.dev_empty((M, N), np.float32)
+        dY = outs[alias[l]] if alias and l in alias else util.dev_empty((M, N), np.float32)
         d = descs[l]
         d.M, d.N, d.K, d.transA, d.transB = M, N, K, 0, int(L["transB"])
         d.alpha, d.beta, d.batch = L.get("alpha", 1.0), L.get("beta", 1.0), 1
@@ -120,6 +121,19 @@ def test_chain_with_every_epilogue_feature(rt, fused, opt):
     got = run_chain(rt, X, layers)
     want, mags = oracle_chain(X, layers)
     check(got, want, mags)
+
+
+def test_layers_that_share_memory_run_layer_by_layer(rt):
+    """A caller that planned the chain's tensors by per-layer lifetimes hands layer 2 the buffer of layer 0 (dead once layer 1 has
+    read it).  In one launch a workgroup's layer-0 rows would land on rows of layer 2 that another workgroup has finished; the
+    entry point sees the overlap and launches per layer, so layers 1 and 2 come out right."""
+    M = 64
+    X = util.normal(960, M * 32).reshape(M, 32)
+    layers = mlp_layers([32, 128, 64, 128], 961, act=R.ACT_TANH)
+    got = run_chain(rt, X, layers, alias={2: 0})
+    want, mags = oracle_chain(X, layers)
+    check(got[1:], want[1:], mags[1:])
+    assert np.array_equal(got[0], got[2])  # the shared buffer holds layer 2's result
 
 
 def test_chain_of_one_wide_rows_and_refusals(rt):
