@@ -80,7 +80,14 @@ private:
    const uint8_t *fP, *fEnd;
 };
 
-std::string Str(Slice s) { return std::string((const char *)s.p, s.n); }
+std::string Str(Slice s) { return s.p ? std::string((const char *)s.p, s.n) : std::string(); }
+// text of a string / bytes field; a field of that number written with another wire type is a malformed file
+std::string Str(const Field &f)
+{
+   if (f.wt != 2)
+      throw std::runtime_error("SOFIE ONNX parser: field " + std::to_string(f.no) + " should be length-delimited");
+   return Str(f.bytes);
+}
 
 std::vector<int64_t> PackedInts(const Field &f)
 {
@@ -89,14 +96,19 @@ std::vector<int64_t> PackedInts(const Field &f)
       out.push_back((int64_t)f.v);
       return out;
    }
-   Reader r(f.bytes);
-   // a packed field is a sequence of bare varints: reuse the reader by faking keys is not possible, so decode here
+   if (f.wt != 2)
+      throw std::runtime_error("SOFIE ONNX parser: repeated integer field " + std::to_string(f.no) + " has wire type " + std::to_string(f.wt));
+   // a packed field is a sequence of bare varints, each at most 10 bytes long
    const uint8_t *p = f.bytes.p, *e = f.bytes.p + f.bytes.n;
    while (p < e) {
       uint64_t v = 0;
       int shift = 0;
-      while (p < e) {
-         uint8_t b = *p++;
+      for (;;) {
+         if (p >= e)
+            throw std::runtime_error("SOFIE ONNX parser: truncated varint in a packed field");
+         if (shift > 63)
+            throw std::runtime_error("SOFIE ONNX parser: varint longer than 10 bytes");
+         const uint8_t b = *p++;
          v |= (uint64_t)(b & 0x7f) << shift;
          if (!(b & 0x80))
             break;
@@ -105,6 +117,25 @@ std::vector<int64_t> PackedInts(const Field &f)
       out.push_back((int64_t)v);
    }
    return out;
+}
+
+// repeated float: packed (length-delimited, 4 bytes each) or one fixed32 per occurrence
+void AppendFloats(const Field &f, std::vector<float> &out)
+{
+   if (f.wt == 5) {
+      float v;
+      const uint32_t bits = (uint32_t)f.v;
+      std::memcpy(&v, &bits, 4);
+      out.push_back(v);
+      return;
+   }
+   if (f.wt != 2 || f.bytes.n % 4 != 0)
+      throw std::runtime_error("SOFIE ONNX parser: repeated float field " + std::to_string(f.no) + " is malformed");
+   for (size_t i = 0; i + 4 <= f.bytes.n; i += 4) {
+      float v;
+      std::memcpy(&v, f.bytes.p + i, 4);
+      out.push_back(v);
+   }
 }
 
 float AsFloat(uint32_t bits)
@@ -150,7 +181,7 @@ Tensor ParseTensor(Slice s)
          for (auto v : PackedInts(f))
             t.ints.push_back(v);
          break;
-      case 8: t.name = Str(f.bytes); break;
+      case 8: t.name = Str(f); break;
       case 9: t.raw.assign(f.bytes.p, f.bytes.p + f.bytes.n); break;
       default: break;
       }
@@ -163,6 +194,7 @@ struct Attr {
    int64_t i = 0;
    float f = 0;
    std::vector<int64_t> ints;
+   std::vector<float> floats;
    Slice tensor; // a TensorProto (the `value` of a Constant node), inside the file's buffer
    bool has_i = false, has_f = false, has_s = false;
 };
@@ -180,10 +212,10 @@ Node ParseNode(Slice s)
    Field f;
    while (r.Next(f)) {
       switch (f.no) {
-      case 1: n.in.push_back(Str(f.bytes)); break;
-      case 2: n.out.push_back(Str(f.bytes)); break;
-      case 3: n.name = Str(f.bytes); break;
-      case 4: n.op = Str(f.bytes); break;
+      case 1: n.in.push_back(Str(f)); break;
+      case 2: n.out.push_back(Str(f)); break;
+      case 3: n.name = Str(f); break;
+      case 4: n.op = Str(f); break;
       case 5: {
          Attr a;
          std::string an;
@@ -191,11 +223,16 @@ Node ParseNode(Slice s)
          Field g;
          while (ra.Next(g)) {
             switch (g.no) {
-            case 1: an = Str(g.bytes); break;
+            case 1: an = Str(g); break;
             case 2: a.f = AsFloat((uint32_t)g.v); a.has_f = true; break;
             case 3: a.i = (int64_t)g.v; a.has_i = true; break;
-            case 4: a.s = Str(g.bytes); a.has_s = true; break;
-            case 5: a.tensor = g.bytes; break;
+            case 4: a.s = Str(g); a.has_s = true; break;
+            case 5:
+               if (g.wt != 2)
+                  throw std::runtime_error("SOFIE ONNX parser: attribute tensor should be length-delimited");
+               a.tensor = g.bytes;
+               break;
+            case 7: AppendFloats(g, a.floats); break;
             case 8:
                for (auto v : PackedInts(g))
                   a.ints.push_back(v);
@@ -226,7 +263,7 @@ ValueInfo ParseValueInfo(Slice s)
    Field f;
    while (r.Next(f)) {
       if (f.no == 1)
-         v.name = Str(f.bytes);
+         v.name = Str(f);
       else if (f.no == 2) {
          Reader rt(f.bytes);
          Field t;
@@ -252,7 +289,7 @@ ValueInfo ParseValueInfo(Slice s)
                                  v.dims.push_back(Dim((size_t)x.v));
                                  value = true;
                               } else if (x.no == 2) {
-                                 param = Str(x.bytes);
+                                 param = Str(x);
                               }
                            if (!value) {
                               v.shape.push_back(0);
@@ -328,8 +365,12 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          t.dtype = static_cast<int>(ETensorType::INT64);
          t.ints = it->attrs["value_ints"].ints;
          t.dims = {t.ints.size()};
+      } else if (has("value_floats")) {
+         t.dtype = static_cast<int>(ETensorType::FLOAT);
+         t.floats = it->attrs["value_floats"].floats;
+         t.dims = {t.floats.size()};
       } else {
-         throw std::runtime_error("SOFIE ONNX parser: Constant " + it->name + " has no value, value_float, value_int or value_ints attribute");
+         throw std::runtime_error("SOFIE ONNX parser: Constant " + it->name + " has no value, value_float(s) or value_int(s) attribute");
       }
       t.name = it->out[0];
       inits.push_back(std::move(t));

@@ -374,6 +374,41 @@ def test_corrupt_files_are_refused_with_a_message(tmp_path):
     assert r.returncode == 1 and ("2^40" in r.stdout or "values" in r.stdout)
 
 
+def test_packed_fields_wire_types_and_float_lists(tmp_path):
+    """The packed-integer decoder holds varints to 10 bytes like the plain one; a string field written as a varint is a malformed
+    file, not a null string; `floats` attributes (packed or one fixed32 each) are read, so a Constant given as value_floats becomes
+    an initializer."""
+    def run(data, name):
+        p = os.path.join(str(tmp_path), name + ".onnx")
+        open(p, "wb").write(data)
+        return subprocess.run([em.EMIT, p, str(tmp_path), "--name", name], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+
+    def graph(node_bytes, extra=b""):
+        g = ow._ld(1, node_bytes) + ow._ld(2, b"g") + extra + ow._ld(11, ow.value_info("X", 1, [1, 4])) + ow._ld(12, ow.value_info("Y", 1, [1, 4]))
+        return ow._vi(1, 8) + ow._ld(8, ow._ld(2, ow._vi(2, 17))) + ow._ld(7, g)
+
+    # an `ints` attribute whose packed payload is one varint of 12 continuation bytes
+    bad_ints = ow._ld(1, b"axes") + ow._ld(8, b"\xff" * 12 + b"\x01") + ow._vi(20, 7)
+    n = ow._ld(1, b"X") + ow._ld(2, b"Y") + ow._ld(4, b"Relu") + ow._ld(5, bad_ints)
+    r = run(graph(n), "overlong")
+    assert r.returncode == 1 and "varint longer than 10 bytes" in r.stdout
+    # the operator type (field 4, a string) written as a varint
+    n = ow._ld(1, b"X") + ow._ld(2, b"Y") + ow._vi(4, 7)
+    r = run(graph(n), "mistyped")
+    assert r.returncode == 1 and "length-delimited" in r.stdout
+    # Constant(value_floats) -> Add: the constant is an initializer of the generated Session, packed and unpacked encodings alike
+    import struct
+    vals = [0.5, -1.25, 3.0, 8.0]
+    for name, payload in (("packed", ow._ld(7, struct.pack("<4f", *vals))), ("unpacked", b"".join(ow._key(7, 5) + struct.pack("<f", v) for v in vals))):
+        const = ow._ld(2, b"C") + ow._ld(4, b"Constant") + ow._ld(5, ow._ld(1, b"value_floats") + payload + ow._vi(20, 6))
+        add = ow.node("Add", ["X", "C"], ["Y"])
+        g = ow._ld(1, const) + ow._ld(1, add) + ow._ld(2, b"g") + ow._ld(11, ow.value_info("X", 1, [1, 4])) + ow._ld(12, ow.value_info("Y", 1, [1, 4]))
+        r = run(ow._vi(1, 8) + ow._ld(8, ow._ld(2, ow._vi(2, 17))) + ow._ld(7, g), "floats_" + name)
+        assert r.returncode == 0, r.stdout
+        dat = open(os.path.join(str(tmp_path), "floats_%s_GPU_HIP.dat" % name)).read().split()
+        assert dat[0] == "tensor_C" and dat[1] == "4" and [float(v) for v in dat[2:6]] == vals
+
+
 def test_parse_time_rewrites_of_the_reference(emitted, tmp_path):
     txt = read(emitted, "ParseRewrites")
     body = ops_body(txt)
