@@ -4,8 +4,11 @@
 Workload (benchmark configuration 2): int8 quantised MLP 1024 -> 4096 -> 4096 -> 1024 at batch 1024,
 QuantizeLinear -> [int8 Gemm (int32 accumulate) -> Relu -> DequantizeLinear]x3, per-tensor scales,
 synthetic seeded data, fp32 input already resident in HBM.  One step = one inference over the batch.
-Prints ONE JSON line; `value` = inferences/s.  Also times the stand-alone int8 GEMM sweep
-(M=N=K in 1024/4096/8192) and the CPU oracle on a bounded sample of batch rows.
+What is timed for `value` is the Session the generator EMITS for this model (tests/emitted/Config2_int8_MLP_GPU_HIP.hxx, weights
+from a safetensors file), the way the reference's benchmark times its generated code (benchmark/src/BenchmarkEmitter.cxx.in:486-504):
+K x infer_nosync, one wait, wall clock; `value` is the MEDIAN of five such regions.
+Prints ONE JSON line; `value` = inferences/s.  Also times the stand-alone int8 and FP8 GEMM sweeps (M=N=K in 1024/4096/8192), the
+fp32 MLP and the int8 CNN, and the CPU oracle on bounded samples.
 """
 import argparse
 import ctypes as C
@@ -29,19 +32,11 @@ DOMINANT_KERNEL_TRAFFIC_BYTES = 36024320
 
 
 def build_mlp():
-    from tests import util
-    dims, batch = [1024, 4096, 4096, 1024], 1024
-    weights = [util.int8_sym(1101 + l, dims[l] * dims[l + 1]).reshape(dims[l], dims[l + 1]) for l in range(3)]
-    x = util.normal(2101, batch * dims[0]).reshape(batch, dims[0])
-    w_scales = [np.float32(1.0 / 127.0)] * 3
-    in_scales = [np.float32(np.abs(x).max() / 127.0)]
-    h = x[:8]
-    for l, w in enumerate(weights[:-1]):  # calibration of the frozen activation scales (model constants), plain numpy
-        q = np.clip(np.rint(h / in_scales[l]), -128, 127).astype(np.int32)
-        acc = np.maximum(q @ w.astype(np.int32), 0)
-        h = acc.astype(np.float32) * np.float32(in_scales[l] * w_scales[l])
-        in_scales.append(np.float32(max(h.max(), 1e-6) / 127.0))
-    return dims, batch, x, weights, w_scales, in_scales
+    """The constants of the emitted benchmark model (tests/emitted_models.bench_mlp_spec): weights, frozen scales, the input batch."""
+    from tests import emitted_models as em
+    spec = em.bench_mlp_spec()
+    c = spec["consts"]
+    return [1024, 4096, 4096, 1024], 1024, spec["feeds"][0], c["weights"], c["w_scales"], c["in_scales"]
 
 
 def time_region(rt, fn, reps):
@@ -184,17 +179,17 @@ def fp32_mlp_leg(steps=200):
             "max_rel_err_vs_oracle": err, "cpu_oracle_us_per_batch_1_core": round(cpu_s * 1e6, 1)}
 
 
-def int8_cnn_leg(steps=10):
+def int8_cnn_leg(steps=10, parity=True):
     """benchmark configuration 5: 4 x [Conv3x3 s1 p1 + folded BatchNorm + Relu] 3->64->128->256->256 on 64x64 images, batch 256,
-    global average pool, Gemm 256->10; int8 weights, per-channel scales."""
+    global average pool, Gemm 256->10; int8 weights, per-channel scales.  Parity: the CPU chain on four of the 256 images."""
     from sofie_amd import Runtime
     from sofie_amd.session import Int8CNNSession
-    from tests.refmodels import make_int8_cnn
+    from tests.refmodels import make_int8_cnn, int8_cnn_oracle
     batch = 256
     m = make_int8_cnn(batch, 64)
     rt = Runtime(0)
     s = Int8CNNSession(rt, m["batch"], m["in_shape"], m["in_scale"], m["convs"], m["last_scale"], m["fc_w"], m["fc_b"])
-    s.upload_input(m["x"])
+    got = s.infer(m["x"])
     rt.sync()
     for _ in range(3):
         s.infer_nosync()
@@ -202,8 +197,16 @@ def int8_cnn_leg(steps=10):
     rt.close()
     ops = 2.0 * batch * 64 * 64 * sum(cv["W"].size for cv in m["convs"])
     t = ms / steps * 1e-3
-    return {"ms_per_batch": round(t * 1e3, 4), "images_per_s": round(batch / t, 0), "tops": round(ops / t / 1e12, 1),
-            "frac_of_int8_peak": round(ops / t / INT8_PEAK, 4)}
+    out = {"ms_per_batch": round(t * 1e3, 4), "images_per_s": round(batch / t, 0), "tops": round(ops / t / 1e12, 1),
+           "frac_of_int8_peak": round(ops / t / INT8_PEAK, 4)}
+    if parity:
+        sample = [0, 85, 170, 255]
+        want = int8_cnn_oracle(m, np.ascontiguousarray(m["x"][sample]))
+        err = float(np.abs(got[sample] - want).max() / max(1.0, float(np.abs(want).max())))
+        out["parity_images_vs_oracle"] = sample
+        out["max_rel_err_vs_oracle"] = err
+        out["parity_within_1e-5"] = bool(err <= 1e-5)
+    return out
 
 
 def two_stream_leg(weights, w_scales, in_scales, batch, x, steps=200):
@@ -231,18 +234,51 @@ def two_stream_leg(weights, w_scales, in_scales, batch, x, steps=200):
     return {"us_per_batch": round(dt / steps * 1e6, 2), "inferences_per_s": round(batch * steps / dt, 0)}
 
 
-def cpu_baseline(x, weights, w_scales, in_scales, rows, passes=8):
+def cpu_model_name():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(x, weights, w_scales, in_scales, rows):
+    """The oracle's unfused CPU chain (oracle/sofie_oracle.c) on the host cores: all threads on the whole batch, one thread on a
+    sample of rows; and the 8192^3 int8 product with its requantising store on a slice of 1024 of its 8192 rows."""
     from oracle import binding as ob
+    from tests import util
     from tests.refmodels import int8_mlp_oracle
-    threads = ob.load(True).oracle_num_threads()
+    threads = int(ob.load(True).oracle_num_threads())
     int8_mlp_oracle(x[:2], weights, w_scales, in_scales, omp=True)  # warm the caches / thread pool
-    t0 = time.perf_counter()
-    for _ in range(passes):
+    passes, t0 = 0, time.perf_counter()
+    while passes < 8 and (passes < 2 or time.perf_counter() - t0 < 6.0):
         ref = int8_mlp_oracle(x[:rows], weights, w_scales, in_scales, omp=True)
+        passes += 1
     dt = time.perf_counter() - t0
-    return ref, {"value": round(rows * passes / dt, 2), "unit": "inferences/s", "cores": int(threads), "kind": "port",
+    rows1 = min(rows, 48)
+    t1 = time.perf_counter()
+    int8_mlp_oracle(x[:rows1], weights, w_scales, in_scales, omp=False)
+    dt1 = time.perf_counter() - t1
+    # benchmark configuration 3 at 8192^3: rows 0..1023 of A against the whole B, all threads; the full product is 8 such slices
+    n, slice_rows = 8192, 1024
+    A = util.int8_sym(3001, n * n).reshape(n, n)[:slice_rows]
+    Bt = util.int8_sym(3002, n * n).reshape(n, n)
+    bias = util.int32_range(3003, n, -(1 << 15), 1 << 15)
+    scale = ((0.5 + util.uniform01(3004, n)) / np.float32(127.0 * np.sqrt(n))).astype(np.float32)
+    t2 = time.perf_counter()
+    ob.gemm_i8(np.ascontiguousarray(A), Bt, M=slice_rows, N=n, K=n, transB=1, omp=True, bias=bias, scale=scale, relu_out=1, out=2)
+    dt2 = time.perf_counter() - t2
+    return ref, {"value": round(rows * passes / dt, 2), "unit": "inferences/s", "cores": threads, "kind": "port",
                  "sample": "%d passes over the first %d of 1024 batch rows through the unfused CPU chain (oracle/sofie_oracle.c, "
-                           "OpenMP over rows), %.1f s" % (passes, rows, dt)}
+                           "OpenMP over rows, %d threads), %.1f s" % (passes, rows, threads, dt),
+                 "one_thread_inferences_per_s": round(rows1 / dt1, 2),
+                 "one_thread_sample": "one pass over %d rows, 1 thread, %.1f s" % (rows1, dt1),
+                 "host_cpu": cpu_model_name(), "host_logical_cpus": os.cpu_count(),
+                 "int8_gemm_8192_cpu": {"slice": "rows 0..1023 of 8192 (x8 = the whole product)", "threads": threads,
+                                        "seconds_for_slice": round(dt2, 2), "extrapolated_seconds_full": round(8 * dt2, 1),
+                                        "tops_all_threads": round(2.0 * slice_rows * n * n / dt2 / 1e12, 4)}}
 
 
 def main():
@@ -268,19 +304,29 @@ def main():
     from sofie_amd.session import Int8MLPSession
 
     dims, batch, x, weights, w_scales, in_scales = build_mlp()
+    from tests import emitted_models as em
+    emitted = em.BenchSession()   # raises if the emitted Session has not been built (__graft_entry__.build())
+    emitted.upload(x)
+    emitted.run(args.warmup)
+    regions = [emitted.run(args.steps) for _ in range(5)]   # (wall ms, event ms) of K x infer_nosync + one wait
+    walls = sorted(w for w, _ in regions)
+    wall = walls[2]                                         # the median region is the one reported
+    ms_per_step = wall / args.steps
+    value = batch / (ms_per_step * 1e-3)
+    repeats = [round(w / args.steps, 5) for w, _ in regions]
+    event_ms_per_step = sorted(e for _, e in regions)[2] / args.steps
+    y_emitted = emitted.download((batch, dims[-1]))
+    emitted.close()
+    y = np.empty_like(y_emitted)
+
+    # the same calls through the Python mirror of the Session, for the per-kernel legs below
     rt = Runtime(0)
     sess = Int8MLPSession(rt, weights, w_scales, in_scales, batch)
     sess.upload_input(x)
     rt.sync()
-
-    for _ in range(args.warmup):
+    for _ in range(20):
         sess.infer_nosync()
     rt.sync()
-    ms, wall = time_region(rt, sess.infer_nosync, args.steps)
-    ms_per_step = ms / args.steps
-    value = batch / (ms_per_step * 1e-3)
-    # four more regions of the same length, for the spread (the reported figures are those of the first region)
-    repeats = [round(ms_per_step, 5)] + [round(time_region(rt, sess.infer_nosync, args.steps)[0] / args.steps, 5) for _ in range(4)]
 
     # the dominant kernel alone: layers 1 and 2 (1024x4096x1024 and 1024x4096x4096) run the same kernel
     # instantiation (128x128 tiles) and hold 83% of the arithmetic; layer 3 runs the 64x64-tile one
@@ -297,10 +343,7 @@ def main():
     avg_launch_s = gms * 1e-3 / launches
     achieved = ops_per_launch / avg_launch_s
 
-    # parity of what was timed, against the oracle on the sampled rows
-    y = np.empty((batch, dims[-1]), dtype=np.float32)
-    rt.call("sofie_hip_download", y.ctypes.data_as(C.c_void_p), sess.y_ptr, C.c_size_t(y.nbytes))
-    rt.sync()
+    # parity of what was timed (the emitted Session's output, downloaded above) against the oracle
     # host <-> device transfers of one batch, reported next to the resident figure (pageable host memory, as infer(host ptr) uses it)
     def median_ms(fn):
         t = []
@@ -316,7 +359,7 @@ def main():
         cpu, parity = None, None
     else:
         ref, cpu = cpu_baseline(x, weights, w_scales, in_scales, args.cpu_rows)
-        parity = bool(np.array_equal(y[:args.cpu_rows].view(np.uint32), ref.view(np.uint32)))
+        parity = bool(np.array_equal(y_emitted[:args.cpu_rows].view(np.uint32), ref.view(np.uint32)))
 
     sweep = [] if args.no_sweep else gemm_sweep(rt, [1024, 4096, 8192])
     f8 = [] if args.no_sweep else fp8_sweep(rt, [1024, 4096, 8192])
@@ -344,8 +387,10 @@ def main():
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": "int8 MLP 1024->4096->4096->1024, batch 1024, Q -> [i8 Gemm(i32) -> Relu -> DQ]x3, "
                                "per-tensor symmetric scales, input resident in HBM (benchmark configuration 2)",
-                   "global_batch": batch, "launches_per_step": 4, "wall_ms_per_step": round(wall / args.steps, 5),
-                   "ms_per_step_of_5_regions": repeats, "median_ms_per_step": sorted(repeats)[2],
+                   "timed": "the emitted Session (Config2_int8_MLP_GPU_HIP.hxx, safetensors weights): K x infer_nosync + one wait, wall clock, "
+                            "median of 5 regions",
+                   "global_batch": batch, "launches_per_step": 4, "event_ms_per_step": round(event_ms_per_step, 5),
+                   "ms_per_step_of_5_regions": repeats,
                    "h2d_ms_per_batch": h2d_ms, "d2h_ms_per_batch": d2h_ms,
                    "inferences_per_s_with_transfers": round(batch / ((ms_per_step + h2d_ms + d2h_ms) * 1e-3), 1),
                    "parity_vs_oracle_rows": args.cpu_rows, "parity_bit_exact": parity,

@@ -1122,7 +1122,11 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
       gc << "   " << ConvertTypeToString(fInputTensorInfos[n].type) << " *device_input_" << n << "() const { return tensor_" << n << "; }\n";
    for (auto &n : fOutputTensorNames)
       gc << "   " << ConvertTypeToString(GetTensorType(n)) << " const *device_output_" << n << "() const { return tensor_" << n << "; }\n";
-   gc << "   void *stream() const { return sofie_hip_stream(fCtx); }\n\n";
+   gc << "   void *stream() const { return sofie_hip_stream(fCtx); }\n";
+   gc << "   // the runtime context of the Session (its stream, arena and event timer), as the reference's GPU Session leaves its queue public\n";
+   gc << "   sofie_hip_ctx *context() const { return fCtx; }\n";
+   gc << "   // waits for everything enqueued on the session's stream (what follows a run of infer_nosync calls)\n";
+   gc << "   void sync() { detail::Check(sofie_hip_sync(fCtx), \"sync\"); }\n\n";
 
    // doInfer: the operators.  The graph inputs and outputs are parameters named like the members they shadow, so that the
    // same statements run on the arena's regions (infer_nosync) or on memory of the caller (the overload that takes views).

@@ -621,6 +621,81 @@ extern "C" int run_model(const char *weights, const float *const *inputs, float 
 '''
 
 
+# Benchmark harness around the emitted Session of the int8 MLP at its full size: the Session lives across calls, the input
+# stays resident on the device, and the timed region is the reference benchmark's (benchmark/src/BenchmarkEmitter.cxx.in:486-504):
+# N x infer_nosync, one wait, wall clock.
+BENCH_HARNESS = r'''
+#include "%(model)s_GPU_HIP.hxx"
+#include <chrono>
+#include <cstring>
+using Session = SOFIE_%(model)s::Session;
+static void set_error(char *err, int errlen, const char *what)
+{
+   std::strncpy(err, what, errlen - 1);
+   err[errlen - 1] = 0;
+}
+extern "C" void *bench_open(const char *weights, char *err, int errlen)
+{
+   try {
+      return new Session(weights);
+   } catch (const std::exception &e) {
+      set_error(err, errlen, e.what());
+      return nullptr;
+   }
+}
+extern "C" void bench_close(void *h) { delete static_cast<Session *>(h); }
+// uploads one batch into the Session's input region; returns 0, or 1 with the exception text in err
+extern "C" int bench_upload(void *h, const float *x, unsigned long n, char *err, int errlen)
+{
+   try {
+      Session &s = *static_cast<Session *>(h);
+      if (sofie_hip_upload(s.context(), s.device_input_%(input)s(), x, n * sizeof(float)) || sofie_hip_sync(s.context()))
+         throw std::runtime_error(sofie_hip_last_error());
+      return 0;
+   } catch (const std::exception &e) {
+      set_error(err, errlen, e.what());
+      return 1;
+   }
+}
+extern "C" int bench_download(void *h, float *y, unsigned long n, char *err, int errlen)
+{
+   try {
+      Session &s = *static_cast<Session *>(h);
+      if (sofie_hip_download(s.context(), y, s.device_output_%(output)s(), n * sizeof(float)) || sofie_hip_sync(s.context()))
+         throw std::runtime_error(sofie_hip_last_error());
+      return 0;
+   } catch (const std::exception &e) {
+      set_error(err, errlen, e.what());
+      return 1;
+   }
+}
+// `steps` inferences enqueued back to back, one wait: wall-clock milliseconds of the region (and, through *event_ms, what a pair
+// of events on the Session's stream measured); negative on failure
+extern "C" double bench_run(void *h, int steps, float *event_ms, char *err, int errlen)
+{
+   try {
+      Session &s = *static_cast<Session *>(h);
+      s.sync();
+      const auto t0 = std::chrono::steady_clock::now();
+      if (sofie_hip_timer_start(s.context()))
+         throw std::runtime_error(sofie_hip_last_error());
+      for (int i = 0; i < steps; ++i)
+         s.infer_nosync();
+      float ms = 0;
+      if (sofie_hip_timer_stop(s.context(), &ms)) // records the second event and waits for it
+         throw std::runtime_error(sofie_hip_last_error());
+      const auto t1 = std::chrono::steady_clock::now();
+      if (event_ms)
+         *event_ms = ms;
+      return std::chrono::duration<double, std::milli>(t1 - t0).count();
+   } catch (const std::exception &e) {
+      set_error(err, errlen, e.what());
+      return -1.0;
+   }
+}
+'''
+
+
 def _run(cmd):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
@@ -656,6 +731,74 @@ def compile_shared(src, lib):
           "-L" + os.path.join(ROOT, "sofie_amd", "lib"), "-lsofie_hip", "-Wl,-rpath," + os.path.join(ROOT, "sofie_amd", "lib"),
           "-Wl,-rpath,$ORIGIN/../../sofie_amd/lib"])
     return lib
+
+
+BENCH_MODEL = "Config2_int8_MLP"
+
+
+def bench_mlp_spec():
+    """benchmark configuration 2 at its full size: 1024 -> 4096 -> 4096 -> 1024, batch 1024 (same seeds as bench.py's model)."""
+    return int8_mlp([1024, 4096, 4096, 1024], 1024, seed=1100)
+
+
+def build_bench_model():
+    """Emits benchmark configuration 2 at full size with its weights in a safetensors file and compiles the benchmark harness
+    around the emitted Session: what bench.py times and what the full-size parity test runs."""
+    spec = bench_mlp_spec()
+    p = os.path.join(OUT, BENCH_MODEL + ".onnx")
+    ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=BENCH_MODEL)
+    _run([EMIT, p, OUT, "--safetensors"])
+    src = os.path.join(OUT, BENCH_MODEL + "_bench.cxx")
+    with open(src, "w") as f:
+        f.write(BENCH_HARNESS % dict(model=BENCH_MODEL, input=spec["inputs"][0][0], output=spec["outputs"][0][0]))
+    return compile_shared(src, os.path.join(OUT, "lib%s_bench.so" % BENCH_MODEL))
+
+
+class BenchSession:
+    """The emitted Session of the full-size int8 MLP behind its benchmark harness (ctypes)."""
+
+    def __init__(self):
+        import ctypes as C
+        lib_path = os.path.join(OUT, "lib%s_bench.so" % BENCH_MODEL)
+        if not os.path.exists(lib_path):
+            raise RuntimeError("%s is missing: __graft_entry__.build() emits and compiles it" % lib_path)
+        self.C = C
+        self.lib = C.CDLL(lib_path)
+        self.lib.bench_open.restype = C.c_void_p
+        self.lib.bench_open.argtypes = [C.c_char_p, C.c_char_p, C.c_int]
+        self.lib.bench_close.argtypes = [C.c_void_p]
+        self.lib.bench_upload.argtypes = [C.c_void_p, C.c_void_p, C.c_ulong, C.c_char_p, C.c_int]
+        self.lib.bench_download.argtypes = [C.c_void_p, C.c_void_p, C.c_ulong, C.c_char_p, C.c_int]
+        self.lib.bench_run.restype = C.c_double
+        self.lib.bench_run.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_float), C.c_char_p, C.c_int]
+        self.err = C.create_string_buffer(1024)
+        self.h = self.lib.bench_open(os.path.join(OUT, BENCH_MODEL + "_GPU_HIP.safetensors").encode(), self.err, 1024)
+        if not self.h:
+            raise RuntimeError("emitted Session: " + self.err.value.decode())
+
+    def close(self):
+        if self.h:
+            self.lib.bench_close(self.h)
+            self.h = None
+
+    def upload(self, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if self.lib.bench_upload(self.h, x.ctypes.data, x.size, self.err, 1024):
+            raise RuntimeError(self.err.value.decode())
+
+    def download(self, shape):
+        y = np.empty(shape, dtype=np.float32)
+        if self.lib.bench_download(self.h, y.ctypes.data, y.size, self.err, 1024):
+            raise RuntimeError(self.err.value.decode())
+        return y
+
+    def run(self, steps):
+        """steps x infer_nosync + one wait: (wall ms, event ms) of the region."""
+        ev = self.C.c_float()
+        wall = self.lib.bench_run(self.h, steps, self.C.byref(ev), self.err, 1024)
+        if wall < 0:
+            raise RuntimeError(self.err.value.decode())
+        return wall, ev.value
 
 
 def build_all(jobs=8):
@@ -709,6 +852,7 @@ def build_all(jobs=8):
         f.write(DYNAMIC_HARNESS % dict(model="ApiDynamicFp8Gemm", args="inputs[0]"))
     compile_shared(src, os.path.join(OUT, "libApiDynamicFp8Gemm.so"))
     compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
+    build_bench_model()
     return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead", "LayerNormBlock", "ReduceBlock", "HardActivations", "IndexingBlock"]
 
 

@@ -56,3 +56,44 @@ def _check(rt, m, batch, pool_in_conv, pooled):
     assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
     # a second inference on the same session reuses every buffer and gives the same bits
     assert np.array_equal(s.infer(m["x"]).view(np.uint32), got.view(np.uint32))
+
+
+@pytest.mark.parametrize("pool_in_conv", [False, True])
+def test_full_size_batch_256_on_sampled_images(pool_in_conv):
+    """benchmark configuration 5 at its real size (batch 256, 64 x 64 images, 3 -> 64 -> 128 -> 256 -> 256): the kernels the
+    heuristics pick for a million GEMM rows.  The images of a batch are independent, so the CPU chain runs on a sample of
+    them: the last int8 feature map (or its plane sums, when the last convolution adds them up in its store) bit-exact, the
+    fp32 outputs to 1e-5."""
+    from oracle import binding as ob
+    from sofie_amd import Runtime
+    batch = 256
+    m = make_int8_cnn(batch, 64)
+    sample = [0, 1, 127, 255]
+    rt = Runtime(0)
+    try:
+        s = session(rt, m, pool_in_conv)
+        assert s.pool_in_conv == pool_in_conv
+        print("cnn_i8 full size, pool_in_conv =", pool_in_conv, flush=True)
+        got = s.infer(m["x"])
+        xs = np.ascontiguousarray(m["x"][sample])
+        want = int8_cnn_oracle(m, xs)
+        h = ob.quantize_linear(xs, m["in_scale"])
+        for cv in m["convs"]:
+            h = ob.conv_i8(h, cv["W"], cv["bias"], cv["scale"], pads=cv["pads"], strides=cv["strides"], dils=cv["dils"], relu=1, out=2, omp=True)
+        c, oh, ow = s.out_shape
+        if s.pool_in_conv:
+            sums = np.empty((batch, c), dtype=np.int32)
+            rt.call("sofie_hip_download", sums.ctypes.data_as(C.c_void_p), s.p(s.off_sums), C.c_size_t(sums.nbytes))
+            rt.sync()
+            assert np.array_equal(sums[sample], h.astype(np.int64).sum(axis=(2, 3)).astype(np.int32))
+        else:
+            for k, img in enumerate(sample):
+                fm = np.empty((oh, ow, c), dtype=np.int8)
+                rt.call("sofie_hip_download", fm.ctypes.data_as(C.c_void_p), s.p(s.off_last + img * fm.nbytes), C.c_size_t(fm.nbytes))
+                rt.sync()
+                assert np.array_equal(fm.transpose(2, 0, 1), h[k]), "image %d" % img
+        assert (h > 0).mean() > 0.05
+        assert np.abs(got[sample] - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+        assert np.isfinite(got).all() and got.std() > 1e-3
+    finally:
+        rt.close()

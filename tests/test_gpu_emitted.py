@@ -65,6 +65,36 @@ def test_emitted_int8_mlp_is_bit_exact(rt, model, dims, batch):
     assert np.abs(h).max() > 0
 
 
+def test_emitted_int8_mlp_at_full_size_on_sampled_rows(rt):
+    """benchmark configuration 2 at its real size (1024 -> 4096 -> 4096 -> 1024, batch 1024) through the emitted Session that the
+    benchmark times: weights from a safetensors file, input resident on the device, infer_nosync.  The rows of a batch are
+    independent, so the unfused CPU chain runs on a sample of them: bit-exact."""
+    from oracle import binding as ob
+    spec = em.bench_mlp_spec()
+    c, X = spec["consts"], spec["feeds"][0]
+    rows = np.array([0, 1, 127, 128, 255, 256, 511, 777, 1022, 1023])
+    h = np.ascontiguousarray(X[rows])
+    for l, w in enumerate(c["weights"]):
+        q = ob.quantize_linear(h, c["in_scales"][l])
+        acc = np.maximum(ob.matmul_integer(q, w, M=len(rows), N=w.shape[1], K=w.shape[0], omp=True), 0)
+        h = ob.dequantize_linear(acc, np.float32(c["in_scales"][l] * c["w_scales"][l]))
+    print("emitted Config2_int8_MLP (full size)", flush=True)
+    s = em.BenchSession()
+    try:
+        s.upload(X)
+        s.run(1)
+        got = s.download((1024, 1024))
+        s.run(3)   # further inferences on the same Session give the same bits
+        again = s.download((1024, 1024))
+    finally:
+        s.close()
+    assert np.array_equal(got[rows].view(np.uint32), h.view(np.uint32))
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+    assert np.abs(h).max() > 0 and (got > 0).mean() > 0.1
+    txt = open(os.path.join(em.OUT, em.BENCH_MODEL + "_GPU_HIP.hxx")).read()
+    assert txt.count("sofie_hip_gemm_i8(") == 3 and "SOFIE_I8OUT_I8_DQQ" in txt and "safetensors" in txt
+
+
 def test_emitted_int8_cnn_matches_cpu_chain(rt):
     """QuantizeLinear -> 4 x [QLinearConv + Relu] -> DequantizeLinear -> GlobalAveragePool -> Flatten -> Gemm, parsed from ONNX,
     emitted, compiled: the int8 stages are bit-exact by construction of the kernels (checked operator by operator in
