@@ -228,6 +228,14 @@ typedef struct sofie_gemm_i8_desc {
 int sofie_hip_gemm_i8(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d);
 /* Bytes of workspace sofie_hip_gemm_i8 needs for this descriptor (0 if none). */
 size_t sofie_hip_gemm_i8_workspace(const sofie_gemm_i8_desc *d);
+/* sofie_hip_gemm_i8 for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The scratch for the operand re-layout (B given
+ * as [K,N], A given as [K,M]) is a static device array of SOFIE_HIP_GEMM_I8_NOALLOC_SCRATCH_BYTES that every GPU the library
+ * runs on holds until the process ends; `workspace` / `workspace_bytes` of the descriptor are ignored.  A descriptor whose
+ * re-layout needs more (sofie_hip_gemm_i8_workspace) is refused with an error.  The call allocates and frees nothing.  All
+ * calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race. */
+#define SOFIE_HIP_GEMM_I8_NOALLOC_SCRATCH_BYTES (8u << 20)
+int sofie_hip_gemm_i8_noalloc(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d);
 /* Re-layout of a [K,N] int8 matrix into [N,K] (weights, once, at Session construction; the
  * analogue of the Conv weight re-layout into tensor_<Y>_f, ROperator_Conv.hxx:456-476). */
 int sofie_hip_transpose_i8(sofie_hip_ctx *ctx, int8_t *dst, const int8_t *src, int32_t rows, int32_t cols,

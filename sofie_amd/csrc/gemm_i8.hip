@@ -1,6 +1,7 @@
 // int8 x int8 -> int32 GEMM on the gfx950 matrix cores (v_mfma_i32_32x32x32_i8) with the
 // requantisation / dequantisation epilogue fused into the store, and the int8 re-layout kernel.
 #include "i8_epilogue.hpp"
+#include <mutex>
 
 namespace sofie_hip {
 
@@ -99,7 +100,8 @@ int sofie_hip_transpose_i8(sofie_hip_ctx *ctx, int8_t *dst, const int8_t *src, i
    return transpose_i8(ctx->stream, dst, src, rows, cols, ld_src, ld_dst);
 }
 
-int sofie_hip_gemm_i8(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d)
+// The body of sofie_hip_gemm_i8 with the re-layout scratch given separately from the descriptor.
+static int gemm_i8_with_workspace(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d, void *workspace, size_t workspace_bytes)
 {
    SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_gemm_i8: NULL argument");
    SOFIE_HIP_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "sofie_hip_gemm_i8: negative dimension");
@@ -117,8 +119,8 @@ int sofie_hip_gemm_i8(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d)
                      "sofie_hip_gemm_i8: leading dimension too small");
 
    const int8_t *A = d->A, *Bt = d->B;
-   char *ws = (char *)d->workspace;
-   size_t ws_left = d->workspace_bytes;
+   char *ws = (char *)workspace;
+   size_t ws_left = workspace_bytes;
    if (K > 0 && !d->transB) {
       // B is [K,N]: the kernel wants [N,K]
       size_t need = (((size_t)K * (size_t)N) + 255) & ~(size_t)255;
@@ -166,6 +168,56 @@ int sofie_hip_gemm_i8(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d)
       lda = ldb = 16;
    }
    return gemm_i8_nt(launch_cfg_i8(ctx), A, Bt, M, N, K, lda, ldb, ep);
+}
+
+int sofie_hip_gemm_i8(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d)
+{
+   SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_gemm_i8: NULL argument");
+   return gemm_i8_with_workspace(ctx, d, d->workspace, d->workspace_bytes);
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------------------------------------------
+// The operand re-layout of sofie_hip_gemm_i8 (B given as [K,N], A given as [K,M]) needs scratch memory.  Here it lives in a
+// static device array instead of a workspace of the caller: every GPU the library runs on holds its own copy of the array
+// until the process ends.  In host code the array's name is only a stand-in; the device address comes from
+// hipGetSymbolAddress, once per device, and that pointer is what the kernels are given.
+static __device__ __align__(256) unsigned char scratch[SOFIE_HIP_GEMM_I8_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[64] = {}; // per device: the address of `scratch` there
+} // namespace
+
+int sofie_hip_gemm_i8_noalloc(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *d)
+{
+   SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_gemm_i8_noalloc: NULL argument");
+   SOFIE_HIP_REQUIRE(ctx->device >= 0 && ctx->device < 64, "sofie_hip_gemm_i8_noalloc: device %d out of range", ctx->device);
+   const size_t need = sofie_hip_gemm_i8_workspace(d);
+   SOFIE_HIP_REQUIRE(need <= (size_t)SOFIE_HIP_GEMM_I8_NOALLOC_SCRATCH_BYTES,
+                     "sofie_hip_gemm_i8_noalloc: the operand re-layout needs %zu bytes of scratch, the static buffer holds %zu "
+                     "(use sofie_hip_gemm_i8 with a workspace, or operands already laid out [M,K] and [N,K])",
+                     need, (size_t)SOFIE_HIP_GEMM_I8_NOALLOC_SCRATCH_BYTES);
+   void *ptr = nullptr;
+   {
+      std::lock_guard<std::mutex> lock(g_scratch_mutex);
+      if (!g_scratch_ptr[ctx->device]) {
+         // first call on this device: look the array's address up with that device current
+         int current = -1;
+         SOFIE_HIP_CHECK(hipGetDevice(&current));
+         if (current != ctx->device)
+            SOFIE_HIP_CHECK(hipSetDevice(ctx->device));
+         void *p = nullptr;
+         const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+         if (current != ctx->device)
+            (void)hipSetDevice(current);
+         if (e != hipSuccess || !p)
+            return fail(SOFIE_HIP_ERR_RUNTIME, "sofie_hip_gemm_i8_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+         g_scratch_ptr[ctx->device] = p;
+      }
+      ptr = g_scratch_ptr[ctx->device];
+   }
+   // the re-layout kernels overwrite every byte they later read: nothing has to start at zero
+   return gemm_i8_with_workspace(ctx, d, ptr, (size_t)SOFIE_HIP_GEMM_I8_NOALLOC_SCRATCH_BYTES);
 }
 
 } // extern "C"

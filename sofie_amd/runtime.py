@@ -126,6 +126,7 @@ SYMBOLS = {
     "sofie_hip_conv_i8_workspace": (C.c_size_t, [C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
     "sofie_hip_conv_i8_column_matrix_bytes": (C.c_size_t, [C.POINTER(ConvDesc)]),
     "sofie_hip_ctx_set_option": (C.c_int, [_P, C.c_char_p, C.c_int32]),
+    "sofie_hip_gemm_i8_noalloc": (C.c_int, [_P, C.POINTER(GemmI8Desc)]),
     "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),
     "sofie_hip_global_avg_pool_f32": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32]),
     "sofie_hip_pool_f32": (C.c_int, [_P, _P, _P, _P]),
