@@ -324,6 +324,23 @@ int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float
                        const float *bias /* [Cout] or NULL */, int32_t act, float act_alpha, float *Y,
                        const sofie_post_ops *post /* applied after `act`; NULL = none */,
                        const float *residual /* [N,Cout,OH,OW] added before `act`, or NULL */);
+/* 3-D convolution (ROperator_Conv with three spatial dimensions, core/inc/SOFIE/operators/ROperator_Conv.hxx:533-552, and
+ * UTILITY::Im2col_3d, core/src/utils/SOFIE_common_helpers.cxx:85-139): the same implicit GEMM with the reduction over
+ * (channel, kd, kh, kw).  X is [N,C,D,H,W], W is [Cout, C/group, kd, kh, kw], Y is [N,Cout,OD,OH,OW]; the pads are ordered as the
+ * ONNX attribute: {d_begin, h_begin, w_begin, d_end, h_end, w_end}. */
+typedef struct sofie_conv3d_desc {
+   int32_t N, C, D, H, W;
+   int32_t Cout, kd, kh, kw;
+   int32_t pad[6];
+   int32_t stride[3];
+   int32_t dil[3];
+   int32_t group;
+   int32_t OD, OH, OW; /* as computed by the caller's shape inference; checked */
+} sofie_conv3d_desc;
+int sofie_hip_conv3d_f32(sofie_hip_ctx *ctx, const sofie_conv3d_desc *d, const float *X, const float *W,
+                         const float *bias /* [Cout] or NULL */, int32_t act, float act_alpha, float *Y,
+                         const sofie_post_ops *post /* applied after `act`; NULL = none */,
+                         const float *residual /* of Y's shape, added before `act`, or NULL */);
 /* int8 form (no counterpart in the reference): acc = conv_i32(X_i8, W_i8) + bias_i32[co], then by `out`
  *   SOFIE_I8OUT_I8   Y_i8  = sat8(rne(float(acc)*scale[co])), then max(.,0) if relu
  *   SOFIE_I8OUT_F32  Y_f32 = float(acc)*scale[co], then max(.,0) if relu

@@ -121,6 +121,22 @@ def conv_f32(X, W, bias=None, *, pads=(0, 0, 0, 0), strides=(1, 1), dils=(1, 1),
     return Y
 
 
+def conv3d_f32(X, W, bias=None, *, pads=(0, 0, 0, 0, 0, 0), strides=(1, 1, 1), dils=(1, 1, 1), group=1, act=0, act_alpha=0.0):
+    """X [N,C,D,H,W], W [Cout,C/group,kd,kh,kw], pads (d0,h0,w0,d1,h1,w1) as the ONNX attribute orders them."""
+    X, W = _f32(X), _f32(W)
+    b = None if bias is None else _f32(bias)
+    N, Cc, D, H, Wd = X.shape
+    Cout, _, kd, kh, kw = W.shape
+    out = [(X.shape[2 + a] + pads[a] + pads[a + 3] - (dils[a] * (W.shape[2 + a] - 1) + 1)) // strides[a] + 1 for a in range(3)]
+    Y = np.zeros((N, Cout, out[0], out[1], out[2]), dtype=np.float32)
+    i3 = C.c_int * 3
+    rc = load().oracle_conv3d_f32(N, Cc, D, H, Wd, Cout, kd, kh, kw, (C.c_int * 6)(*pads), i3(*strides), i3(*dils), group, _ptr(X), _ptr(W),
+                                  _ptr(b), act, C.c_float(act_alpha), _ptr(Y))
+    if rc:
+        raise MemoryError("oracle_conv3d_f32")
+    return Y
+
+
 def im2col(x, kh, kw, pads, strides, dils):
     """x [C,H,W] -> [C*kh*kw, OH*OW]; pads (h0,w0,h1,w1)."""
     x = _f32(x)

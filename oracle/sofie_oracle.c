@@ -385,6 +385,88 @@ ORACLE_API int oracle_conv_f32(int N, int C, int H, int W, int Cout, int kh, int
    return 0;
 }
 
+/* UTILITY::Im2col_3d (core/src/utils/SOFIE_common_helpers.cxx:85-139): rows (c, kd, kh, kw), columns (od, oh, ow), zero outside
+ * the volume. */
+ORACLE_API void oracle_im2col_3d(const float *data_im, int channels, int depth, int height, int width, int kernel_d, int kernel_h,
+                                 int kernel_w, int pad_d_begin, int pad_d_end, int pad_h_begin, int pad_h_end, int pad_w_begin,
+                                 int pad_w_end, int stride_d, int stride_h, int stride_w, int dilation_d, int dilation_h,
+                                 int dilation_w, float *data_col)
+{
+   const int output_h = (height + pad_h_begin + pad_h_end - (dilation_h * (kernel_h - 1) + 1)) / stride_h + 1;
+   const int output_w = (width + pad_w_begin + pad_w_end - (dilation_w * (kernel_w - 1) + 1)) / stride_w + 1;
+   const int output_d = (depth + pad_d_begin + pad_d_end - (dilation_d * (kernel_d - 1) + 1)) / stride_d + 1;
+   const int channel_size = height * width * depth;
+   for (int channel = 0; channel < channels; ++channel, data_im += channel_size)
+      for (int kd = 0; kd < kernel_d; ++kd)
+         for (int kr = 0; kr < kernel_h; ++kr)
+            for (int kc = 0; kc < kernel_w; ++kc) {
+               int input_dep = -pad_d_begin + kd * dilation_d;
+               for (int od = 0; od < output_d; ++od, input_dep += stride_d) {
+                  int input_row = -pad_h_begin + kr * dilation_h;
+                  for (int orow = 0; orow < output_h; ++orow, input_row += stride_h) {
+                     int input_col = -pad_w_begin + kc * dilation_w;
+                     for (int oc = 0; oc < output_w; ++oc, input_col += stride_w)
+                        *(data_col++) = (in_range(input_dep, depth) && in_range(input_row, height) && in_range(input_col, width))
+                                           ? data_im[input_dep * width * height + input_row * width + input_col]
+                                           : 0.0f;
+                  }
+               }
+            }
+}
+
+/* ROperator_Conv<float>::Generate for 3-D convolutions (core/inc/SOFIE/operators/ROperator_Conv.hxx:406-642): as in 1-D / 2-D the
+ * kernel goes into the dilated layout (:442-476, zero between the taps, effective size k + (d-1)(k-1) per axis, dilation 1 from then
+ * on), then per image and group Im2col_3d with the pads in the order {d_begin, d_end, h_begin, h_end, w_begin, w_end} taken from
+ * the attribute {d_begin, h_begin, w_begin, d_end, h_end, w_end} (:533-541) and Gemm_Call(y, false, false, m = OD*OH*OW, n = Cout/g,
+ * k = Cin/g*KD*KH*KW, 1, xcol, f, beta, bias).
+ * X [N,C,D,H,W]; W [Cout, C/group, kd, kh, kw]; pads[6] = {d0,h0,w0,d1,h1,w1}; strides[3], dils[3]; Y [N,Cout,OD,OH,OW]. */
+ORACLE_API int oracle_conv3d_f32(int N, int C, int D, int H, int W, int Cout, int kd, int kh, int kw, const int *pads, const int *strides,
+                                 const int *dils, int group, const float *X, const float *Wt, const float *bias, int act, float act_alpha,
+                                 float *Y)
+{
+   const int Cg = C / group, Cout_g = Cout / group;
+   const int ekd = kd + (dils[0] - 1) * (kd - 1), ekh = kh + (dils[1] - 1) * (kh - 1), ekw = kw + (dils[2] - 1) * (kw - 1);
+   const int OD = (D + pads[0] + pads[3] - ekd) / strides[0] + 1;
+   const int OH = (H + pads[1] + pads[4] - ekh) / strides[1] + 1;
+   const int OW = (W + pads[2] + pads[5] - ekw) / strides[2] + 1;
+   const int m = OD * OH * OW, k = Cg * ekd * ekh * ekw;
+   float *f = (float *)calloc((size_t)Cout * k, sizeof(float));
+   float *xcol = (float *)malloc(sizeof(float) * (size_t)k * (size_t)m);
+   float *bcast = bias ? (float *)malloc(sizeof(float) * (size_t)Cout * m) : NULL;
+   if (!f || !xcol || (bias && !bcast)) {
+      free(f);
+      free(xcol);
+      free(bcast);
+      return 1;
+   }
+   for (int oc = 0; oc < Cout; ++oc)
+      for (int ic = 0; ic < Cg; ++ic)
+         for (int z = 0; z < kd; ++z)
+            for (int y = 0; y < kh; ++y)
+               for (int x = 0; x < kw; ++x)
+                  f[(size_t)oc * k + (size_t)ic * ekd * ekh * ekw + (size_t)z * dils[0] * ekh * ekw + (size_t)y * dils[1] * ekw +
+                    (size_t)x * dils[2]] = Wt[((((size_t)oc * Cg + ic) * kd + z) * kh + y) * kw + x];
+   if (bias)
+      for (int oc = 0; oc < Cout; ++oc)
+         for (int i = 0; i < m; ++i)
+            bcast[(size_t)oc * m + i] = bias[oc];
+   const float beta = bias ? 1.0f : 0.0f;
+   for (int n = 0; n < N; ++n)
+      for (int g = 0; g < group; ++g) {
+         const size_t x_offset = ((size_t)n * C + (size_t)g * Cg) * D * H * W;
+         const size_t g_offset = (size_t)g * Cout_g * m;
+         const size_t out_offset = (size_t)n * Cout * m + g_offset;
+         oracle_im2col_3d(X + x_offset, Cg, D, H, W, ekd, ekh, ekw, pads[0], pads[3], pads[1], pads[4], pads[2], pads[5], strides[0],
+                          strides[1], strides[2], 1, 1, 1, xcol);
+         oracle_gemm_call(Y + out_offset, 0, 0, m, Cout_g, k, 1.0f, xcol, f + (size_t)g * Cout_g * k, beta, bias ? bcast + g_offset : NULL);
+      }
+   oracle_unary(Y, Y, (size_t)N * Cout * m, act, act_alpha);
+   free(f);
+   free(xcol);
+   free(bcast);
+   return 0;
+}
+
 /* GlobalAveragePool = AveragePool with kernel == image (core/inc/SOFIE/operators/ROperator_Pool.hxx:225-237):
  * sequential fp32 sum over the plane, then `value /= float(nsum)` (:362-368). */
 ORACLE_API void oracle_global_avg_pool(float *Y, const float *X, int NC, int HW)

@@ -260,13 +260,37 @@ struct ConvOperandA {
       return X[(((size_t)img * C + c_first + ci) * H + ih) * W + iw];
    }
 };
+// The same for three spatial dimensions (the reference's Im2col_3d): row m = (image, od, oh, ow), column k = (ci, kd, kh, kw).
+struct Conv3dOperandA {
+   const float *X;
+   int C, D, H, W, kd, kh, kw, OD, OH, OW, pad_d0, pad_h0, pad_w0, stride_d, stride_h, stride_w, dil_d, dil_h, dil_w;
+   int c_first;
+   __device__ __forceinline__ float operator()(int m, int k) const
+   {
+      int ow = m % OW, t = m / OW;
+      int oh = t % OH;
+      t /= OH;
+      int od = t % OD, img = t / OD;
+      int kx = k % kw, t2 = k / kw;
+      int ky = t2 % kh;
+      t2 /= kh;
+      int kz = t2 % kd, ci = t2 / kd;
+      int id = od * stride_d - pad_d0 + kz * dil_d;
+      int ih = oh * stride_h - pad_h0 + ky * dil_h;
+      int iw = ow * stride_w - pad_w0 + kx * dil_w;
+      if ((unsigned)id >= (unsigned)D || (unsigned)ih >= (unsigned)H || (unsigned)iw >= (unsigned)W)
+         return 0.0f;
+      return X[((((size_t)img * C + c_first + ci) * D + id) * H + ih) * W + iw];
+   }
+};
 struct ConvOperandB {
    const float *Wt; // [Cout_g][Kg] rows of this group
    int Kg;
    __device__ __forceinline__ float operator()(int k, int n) const { return Wt[(size_t)n * Kg + k]; }
 };
 
-__global__ __launch_bounds__(256) void conv_f32_kernel(ConvOperandA la, const float *Wt, const float *bias, float *Y, int M,
+template <class LA>
+__global__ __launch_bounds__(256) void conv_f32_kernel(LA la, const float *Wt, const float *bias, float *Y, int M,
                                                         int Cout_g, int Kg, int Cg, int Cout, int OHW, PostChain chain, const float *R)
 {
    const int g = blockIdx.z;
@@ -621,9 +645,48 @@ int sofie_hip_conv_f32(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const float
    ConvOperandA la{X, d->C, d->H, d->W, d->kh, d->kw, OH, OW, d->pad_h0, d->pad_w0, d->stride_h, d->stride_w, d->dil_h, d->dil_w, 0};
    const unsigned gy = (unsigned)((M + F32_BM - 1) / F32_BM), gx = (Cout_g + F32_BN - 1) / F32_BN;
    SOFIE_HIP_REQUIRE(gx <= 65535 && d->group <= 65535, "sofie_hip_conv_f32: too many channels or groups for one launch");
-   hipLaunchKernelGGL(conv_f32_kernel, dim3(gy, gx, (unsigned)d->group), dim3(256), 0, ctx->stream, la, W, bias, Y, (int)M, Cout_g, Kg,
+   hipLaunchKernelGGL(conv_f32_kernel<ConvOperandA>, dim3(gy, gx, (unsigned)d->group), dim3(256), 0, ctx->stream, la, W, bias, Y, (int)M, Cout_g, Kg,
                       Cg, d->Cout, OH * OW, chain, residual);
    return launch_status("conv_f32_kernel");
+}
+
+int sofie_hip_conv3d_f32(sofie_hip_ctx *ctx, const sofie_conv3d_desc *d, const float *X, const float *W, const float *bias,
+                         int32_t act, float act_alpha, float *Y, const sofie_post_ops *post, const float *residual)
+{
+   SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_conv3d_f32: NULL argument");
+   SOFIE_HIP_REQUIRE(d->N >= 0 && d->C > 0 && d->D > 0 && d->H > 0 && d->W > 0 && d->Cout > 0 && d->kd > 0 && d->kh > 0 && d->kw > 0,
+                     "sofie_hip_conv3d_f32: bad shape");
+   SOFIE_HIP_REQUIRE(d->group > 0 && d->C % d->group == 0 && d->Cout % d->group == 0,
+                     "sofie_hip_conv3d_f32: group %d does not divide the channels", d->group);
+   const int in[3] = {d->D, d->H, d->W}, kern[3] = {d->kd, d->kh, d->kw}, want[3] = {d->OD, d->OH, d->OW};
+   int outd[3];
+   for (int a = 0; a < 3; ++a) {
+      SOFIE_HIP_REQUIRE(d->stride[a] > 0 && d->dil[a] > 0, "sofie_hip_conv3d_f32: bad stride or dilation");
+      SOFIE_HIP_REQUIRE(d->pad[a] >= 0 && d->pad[a + 3] >= 0, "sofie_hip_conv3d_f32: negative padding");
+      const int eff = d->dil[a] * (kern[a] - 1) + 1;
+      SOFIE_HIP_REQUIRE(in[a] + d->pad[a] + d->pad[a + 3] >= eff, "sofie_hip_conv3d_f32: kernel larger than the padded volume");
+      outd[a] = (in[a] + d->pad[a] + d->pad[a + 3] - eff) / d->stride[a] + 1;
+      SOFIE_HIP_REQUIRE(outd[a] == want[a], "sofie_hip_conv3d_f32: output extent %d of axis %d does not match the descriptor's %d", outd[a], a, want[a]);
+   }
+   PostChain chain;
+   int bad = 0;
+   SOFIE_HIP_REQUIRE(make_post_chain(chain, act, act_alpha, post, bad),
+                     "sofie_hip_conv3d_f32: unknown activation or post operator %d (or more than %d post operators)", bad, SOFIE_MAX_POST_OPS);
+   if (d->N == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(X && W && Y, "sofie_hip_conv3d_f32: NULL pointer");
+   const long long plane = (long long)outd[0] * outd[1] * outd[2], M = (long long)d->N * plane;
+   SOFIE_HIP_REQUIRE(M < (1LL << 31) && (long long)d->C * d->D * d->H * d->W < (1LL << 31), "sofie_hip_conv3d_f32: too many output or input elements");
+   const long long Kg64 = (long long)(d->C / d->group) * d->kd * d->kh * d->kw;
+   SOFIE_HIP_REQUIRE(Kg64 < (1LL << 31), "sofie_hip_conv3d_f32: reduction too long");
+   const int Cg = d->C / d->group, Cout_g = d->Cout / d->group, Kg = (int)Kg64;
+   Conv3dOperandA la{X, d->C, d->D, d->H, d->W, d->kd, d->kh, d->kw, outd[0], outd[1], outd[2], d->pad[0], d->pad[1], d->pad[2],
+                     d->stride[0], d->stride[1], d->stride[2], d->dil[0], d->dil[1], d->dil[2], 0};
+   const unsigned gy = (unsigned)((M + F32_BM - 1) / F32_BM), gx = (Cout_g + F32_BN - 1) / F32_BN;
+   SOFIE_HIP_REQUIRE(gx <= 65535 && d->group <= 65535, "sofie_hip_conv3d_f32: too many channels or groups for one launch");
+   hipLaunchKernelGGL(conv_f32_kernel<Conv3dOperandA>, dim3(gy, gx, (unsigned)d->group), dim3(256), 0, ctx->stream, la, W, bias, Y, (int)M,
+                      Cout_g, Kg, Cg, d->Cout, (int)plane, chain, residual);
+   return launch_status("conv_f32_kernel (3-D)");
 }
 
 } // extern "C"

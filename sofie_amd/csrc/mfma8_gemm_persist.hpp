@@ -132,7 +132,7 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(const int8_t *_
                                                                   int K, EPI ep, int tiles_m, int tiles_n, int sw)
 {
    constexpr int BM = 256, BN = 256, BK = 64, STAGES = 5, NW = 8, WAVES_N = 4;
-   constexpr int R = MMA::ROWS, LK = MMA::LK;
+   constexpr int R = MMA::ROWS;
    constexpr int TM = 128, TN = 64, MT = TM / R, NT = TN / R;
    constexpr int LD = BM / 16 / NW;            // wave instructions per operand and slab (an instruction fills 16 rows of 64 bytes)
    constexpr int STAGE_BYTES = (BM + BN) * BK; // 32 KB

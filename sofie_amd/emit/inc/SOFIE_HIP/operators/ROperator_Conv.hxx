@@ -1,7 +1,8 @@
 // Conv emitter for the gfx950 backend: the operator of core/inc/SOFIE/operators/ROperator_Conv.hxx (same
 // constructor arguments, same padding / stride / dilation / autopad rules), emitting ONE implicit-GEMM
 // launch over the whole batch (sofie_hip_conv_f32) instead of a per-image Im2col + Gemm_Call loop and a
-// per-call weight re-layout.  1-D convolutions run as 2-D with H = 1.  3-D convolutions are not emitted.
+// per-call weight re-layout.  1-D convolutions run as 2-D with H = 1; 3-D convolutions (the reference's Im2col_3d path) go to
+// sofie_hip_conv3d_f32, the same implicit GEMM with the reduction over (channel, kd, kh, kw).
 #ifndef SOFIE_HIP_ROPERATOR_CONV
 #define SOFIE_HIP_ROPERATOR_CONV
 
@@ -11,6 +12,9 @@ namespace SOFIE_HIP {
 
 struct ConvGeometry {
    std::size_t N = 0, C = 0, H = 1, W = 0, Cout = 0, kh = 1, kw = 1, OH = 1, OW = 0, group = 1;
+   // three spatial dimensions: depth first; the pads in the attribute's order {d0, h0, w0, d1, h1, w1}
+   std::size_t D = 1, kd = 1, OD = 1;
+   std::vector<std::size_t> pads3, strides3, dils3;
    std::size_t pad_h0 = 0, pad_w0 = 0, pad_h1 = 0, pad_w1 = 0, stride_h = 1, stride_w = 1, dil_h = 1, dil_w = 1;
    std::size_t dim = 2;
 
@@ -21,8 +25,8 @@ struct ConvGeometry {
                 std::vector<std::size_t> pads, std::vector<std::size_t> strides, const std::vector<std::size_t> &shapeX,
                 const std::vector<std::size_t> &shapeW)
    {
-      if (shapeX.size() < 3 || shapeX.size() > 4)
-         throw std::runtime_error("SOFIE Conv Op: this backend emits 1-D and 2-D convolutions (input of 3 or 4 dimensions)");
+      if (shapeX.size() < 3 || shapeX.size() > 5)
+         throw std::runtime_error("SOFIE Conv Op: the input must have 3, 4 or 5 dimensions (1-D, 2-D or 3-D convolution)");
       dim = shapeX.size() - 2;
       if (shapeW.size() != shapeX.size())
          throw std::runtime_error("SOFIE Conv Op Shape inference - invalid weights ");
@@ -66,6 +70,18 @@ struct ConvGeometry {
       Cout = shapeW[0];
       if (C % group != 0 || Cout % group != 0 || shapeW[1] != C / group)
          throw std::runtime_error("SOFIE Conv Op: channels, groups and weight shape do not agree");
+      if (dim == 3) {
+         D = shapeX[2]; H = shapeX[3]; W = shapeX[4]; kd = kernelShape[0]; kh = kernelShape[1]; kw = kernelShape[2];
+         pads3 = pads; strides3 = strides; dils3 = dilations;
+         std::size_t out[3];
+         for (std::size_t d = 0; d < 3; ++d) {
+            if (shapeX[2 + d] + pads[d] + pads[d + 3] < ek[d])
+               throw std::runtime_error("SOFIE Conv Op: kernel larger than the padded input");
+            out[d] = (shapeX[2 + d] + pads[d] + pads[d + 3] - ek[d]) / strides[d] + 1;
+         }
+         OD = out[0]; OH = out[1]; OW = out[2];
+         return;
+      }
       if (dim == 1) {
          H = 1; W = shapeX[2]; kh = 1; kw = kernelShape[0];
          pad_h0 = pad_h1 = 0; pad_w0 = pads[0]; pad_w1 = pads[1];
@@ -85,6 +101,8 @@ struct ConvGeometry {
    {
       if (dim == 1)
          return {N, Cout, OW};
+      if (dim == 3)
+         return {N, Cout, OD, OH, OW};
       return {N, Cout, OH, OW};
    }
    // statement that scales the descriptor's image count by the run-time batch
@@ -95,6 +113,13 @@ struct ConvGeometry {
    std::string DescInitializer() const
    {
       std::stringstream s;
+      if (dim == 3) {
+         s << "{" << N << ", " << C << ", " << D << ", " << H << ", " << W << ", " << Cout << ", " << kd << ", " << kh << ", " << kw << ", {"
+           << pads3[0] << ", " << pads3[1] << ", " << pads3[2] << ", " << pads3[3] << ", " << pads3[4] << ", " << pads3[5] << "}, {" << strides3[0]
+           << ", " << strides3[1] << ", " << strides3[2] << "}, {" << dils3[0] << ", " << dils3[1] << ", " << dils3[2] << "}, " << group << ", " << OD
+           << ", " << OH << ", " << OW << "}";
+         return s.str();
+      }
       s << "{" << N << ", " << C << ", " << H << ", " << W << ", " << Cout << ", " << kh << ", " << kw << ", " << pad_h0 << ", " << pad_w0 << ", "
         << pad_h1 << ", " << pad_w1 << ", " << stride_h << ", " << stride_w << ", " << dil_h << ", " << dil_w << ", " << group << ", " << OH
         << ", " << OW << "}";
@@ -187,10 +212,11 @@ public:
       std::stringstream out;
       out << "\n" << SP << "//----  operator Conv " << opName << " --> " << ConvertShapeToString(fGeo.OutputShape()) << "\n";
       out << SP << "{\n";
-      out << SP << "   " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n" << fGeo.BatchLine(fDynamic, SP + "   ");
+      const bool threeD = fGeo.dim == 3;
+      out << SP << "   " << (threeD ? "sofie_conv3d_desc d" : "sofie_conv_desc d") << fGeo.DescInitializer() << ";\n" << fGeo.BatchLine(fDynamic, SP + "   ");
       if (!fPost.empty())
          out << SP << "   " << PostOpsDeclaration("post", fPost) << "\n";
-      out << SP << "   " << "detail::Check(sofie_hip_conv_f32(fCtx, &d, tensor_" << fNX << ", tensor_" << fNW << ", "
+      out << SP << "   " << "detail::Check(" << (threeD ? "sofie_hip_conv3d_f32" : "sofie_hip_conv_f32") << "(fCtx, &d, tensor_" << fNX << ", tensor_" << fNW << ", "
           << (fNB.empty() ? "nullptr" : "tensor_" + fNB) << ", " << ActivationEnumName(fActivation) << ", " << FloatLiteral(fActAlpha)
           << ", tensor_" << fNY << ", " << (fPost.empty() ? "nullptr" : "&post") << ", " << (fNR.empty() ? "nullptr" : "tensor_" + fNR) << "), \""
           << opName << " Conv\");\n";

@@ -67,6 +67,8 @@ public:
       try {
          fGeo.Resolve(fAttrAutopad, fAttrDilations, fAttrGroup, fAttrKernelShape, fAttrPads, fAttrStrides, model.GetTensorShape(fNX),
                       model.GetTensorShape(fNW));
+      if (fGeo.dim == 3)
+         throw std::runtime_error("SOFIE quantised Conv Op: 3-D convolutions are emitted for float tensors only");
       } catch (const std::exception &) {
          return false; // Initialize reports the problem
       }

@@ -85,6 +85,12 @@ REDUCE_SUM, REDUCE_MEAN, REDUCE_SUM_SQUARE, REDUCE_PROD, REDUCE_L2, REDUCE_MAX, 
 BINARY_ADD, BINARY_SUB, BINARY_MUL, BINARY_DIV, BINARY_POW, BINARY_MAX, BINARY_MIN, BINARY_ADD_DIV = range(8)
 
 
+class Conv3dDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("N", "C", "D", "H", "W", "Cout", "kd", "kh", "kw")] + \
+               [("pad", C.c_int32 * 6), ("stride", C.c_int32 * 3), ("dil", C.c_int32 * 3), ("group", C.c_int32),
+                ("OD", C.c_int32), ("OH", C.c_int32), ("OW", C.c_int32)]
+
+
 class ConvI8Args(C.Structure):
     _fields_ = [("X", C.c_void_p), ("W", C.c_void_p), ("bias", C.c_void_p), ("scale", C.c_void_p),
                 ("relu", C.c_int32), ("out", C.c_int32), ("x_layout", C.c_int32), ("y_layout", C.c_int32),
@@ -121,6 +127,7 @@ SYMBOLS = {
     "sofie_hip_unary_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_int32, C.c_float]),
     "sofie_hip_add_f32": (C.c_int, [_P, C.POINTER(AddDesc)]),
     "sofie_hip_conv_f32": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P, _P, C.c_int32, C.c_float, _P, C.POINTER(PostOps), _P]),
+    "sofie_hip_conv3d_f32": (C.c_int, [_P, C.POINTER(Conv3dDesc), _P, _P, _P, C.c_int32, C.c_float, _P, C.POINTER(PostOps), _P]),
     "sofie_hip_unary_chain_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.POINTER(PostOps)]),
     "sofie_hip_conv_i8": (C.c_int, [_P, C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),
     "sofie_hip_conv_i8_workspace": (C.c_size_t, [C.POINTER(ConvDesc), C.POINTER(ConvI8Args)]),

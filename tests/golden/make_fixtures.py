@@ -104,7 +104,7 @@ MODELS = {
     "ConvWithStridesNoPadding": (None, [IOTA]), "ConvWithAsymmetricPadding": (None, [IOTA]),
     "ConvWithDilation": (None, [IOTA]), "ConvWithBias": (None, [IOTA]), "ConvBatch2": (None, [IOTA]),
     "ConvBatch4": (None, [IOTA]), "ConvBatch8": (None, [IOTA]), "ConvGroup2": (None, [IOTA]), "ConvGroup4": (None, [IOTA]),
-    "ConvBatch4Group2": (None, [IOTA]), "Conv1d": (None, [IOTA]), "GlobalAvgPool2d": (None, [IOTA]),
+    "ConvBatch4Group2": (None, [IOTA]), "Conv1d": (None, [IOTA]), "Conv3d": (None, [IOTA]), "GlobalAvgPool2d": (None, [IOTA]),
     "AvgPoolPad": (None, [IOTA]), "AvgPoolCountIncludePad": (None, [IOTA]),
 }
 

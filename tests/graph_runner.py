@@ -53,6 +53,8 @@ def conv_geometry(attrs, xshape, wshape):
         pads = [0] * (2 * dim)
     else:
         raise ValueError(auto)
+    if dim == 3:  # the pads stay in the attribute's order {d0, h0, w0, d1, h1, w1}
+        return dict(k=tuple(k), pads=tuple(pads), strides=tuple(strides), dils=tuple(dils), group=group)
     if dim == 1:  # H = 1
         return dict(k=(1, k[0]), pads=(0, pads[0], 0, pads[1]), strides=(1, strides[0]), dils=(1, dils[0]), group=group)
     return dict(k=(k[0], k[1]), pads=(pads[0], pads[1], pads[2], pads[3]), strides=tuple(strides), dils=tuple(dils), group=group)
@@ -91,6 +93,8 @@ class OracleBackend:
         return self.ob.unary_chain(x, ops)
 
     def conv(self, X, W, b, geo):
+        if X.ndim == 5:
+            return self.ob.conv3d_f32(X, W, b, pads=geo["pads"], strides=geo["strides"], dils=geo["dils"], group=geo["group"])
         return self.ob.conv_f32(X, W, b, pads=geo["pads"], strides=geo["strides"], dils=geo["dils"], group=geo["group"])
 
     def gap(self, X):
@@ -177,7 +181,27 @@ class HipBackend:
         self.rt.sync()
         return u.to_host(dy)
 
+    def conv3d(self, X, W, b, geo):
+        R, u = self.R, self.u
+        N, Cc, D, H, Wd = X.shape
+        Cout, _, kd, kh, kw = W.shape
+        out = [(X.shape[2 + a] + geo["pads"][a] + geo["pads"][a + 3] - (geo["dils"][a] * (W.shape[2 + a] - 1) + 1)) // geo["strides"][a] + 1 for a in range(3)]
+        d = R.Conv3dDesc()
+        (d.N, d.C, d.D, d.H, d.W, d.Cout, d.kd, d.kh, d.kw) = (N, Cc, D, H, Wd, Cout, kd, kh, kw)
+        d.pad, d.stride, d.dil = (C.c_int32 * 6)(*geo["pads"]), (C.c_int32 * 3)(*geo["strides"]), (C.c_int32 * 3)(*geo["dils"])
+        d.group, d.OD, d.OH, d.OW = geo["group"], out[0], out[1], out[2]
+        dX, dW = u.to_dev(X), u.to_dev(W)
+        db = None if b is None else u.to_dev(b)
+        dY = u.dev_empty((N, Cout, out[0], out[1], out[2]), np.float32)
+        import torch
+        torch.cuda.synchronize()
+        self.rt.call("sofie_hip_conv3d_f32", C.byref(d), u.ptr(dX), u.ptr(dW), u.ptr(db), 0, C.c_float(0), u.ptr(dY), None, None)
+        self.rt.sync()
+        return u.to_host(dY)
+
     def conv(self, X, W, b, geo):
+        if X.ndim == 5:
+            return self.conv3d(X, W, b, geo)
         from oracle.binding import conv_out_hw
         R, u = self.R, self.u
         N, Cc, H, Wd = X.shape

@@ -168,6 +168,54 @@ def test_conv_f32(rt, case, with_bias, act):
     assert np.allclose(util.to_host(dY), want, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("case", [
+    # N, C, (D,H,W), Cout, (kd,kh,kw), pads {d0,h0,w0,d1,h1,w1}, strides, dils, group
+    (1, 1, (3, 4, 4), 2, (2, 3, 3), (0, 1, 1, 0, 1, 1), (1, 1, 1), (1, 1, 1), 1),
+    (2, 4, (5, 6, 7), 6, (3, 2, 3), (1, 0, 2, 0, 1, 1), (2, 1, 2), (1, 1, 1), 2),
+    (1, 2, (7, 5, 6), 3, (2, 3, 2), (2, 1, 0, 1, 2, 1), (1, 2, 1), (2, 1, 2), 1),
+    (1, 6, (4, 4, 4), 6, (3, 3, 3), (1, 1, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1), 3),
+    (2, 8, (8, 12, 10), 40, (3, 3, 3), (1, 1, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1), 1),
+    (1, 3, (2, 3, 3), 2, (1, 1, 1), (0, 0, 0, 0, 0, 0), (1, 1, 1), (1, 1, 1), 1),
+])
+@pytest.mark.parametrize("with_bias,act", [(False, 0), (True, 1)])
+def test_conv3d_f32(rt, case, with_bias, act):
+    """3-D convolution: the im2col-3D + Gemm of the reference's CPU operator, restated in the oracle, against the kernel that
+    gathers the taps while it loads its tiles."""
+    N, Cc, sp, Cout, k, pads, strides, dils, group = case
+    X = util.uniform01(33, N * Cc * int(np.prod(sp))).reshape(N, Cc, *sp)
+    Wt = util.normal(34, Cout * (Cc // group) * int(np.prod(k)), 0.3).reshape(Cout, Cc // group, *k)
+    b = util.normal(35, Cout) if with_bias else None
+    out = [(sp[a] + pads[a] + pads[a + 3] - (dils[a] * (k[a] - 1) + 1)) // strides[a] + 1 for a in range(3)]
+    d = R.Conv3dDesc()
+    (d.N, d.C, d.D, d.H, d.W, d.Cout, d.kd, d.kh, d.kw) = (N, Cc, *sp, Cout, *k)
+    d.pad, d.stride, d.dil = (C.c_int32 * 6)(*pads), (C.c_int32 * 3)(*strides), (C.c_int32 * 3)(*dils)
+    d.group, d.OD, d.OH, d.OW = group, *out
+    dX, dW = util.to_dev(X), util.to_dev(Wt)
+    db = None if b is None else util.to_dev(b)
+    dY = util.dev_empty((N, Cout, *out), np.float32)
+    print("conv3d_f32", case, flush=True)
+    rt.call("sofie_hip_conv3d_f32", C.byref(d), util.ptr(dX), util.ptr(dW), util.ptr(db), act, C.c_float(0), util.ptr(dY), None, None)
+    rt.sync()
+    want = ob.conv3d_f32(X, Wt, b, pads=pads, strides=strides, dils=dils, group=group, act=act)
+    assert want.shape == (N, Cout, *out)
+    assert np.allclose(util.to_host(dY), want, rtol=1e-5, atol=1e-5)
+
+
+def test_conv3d_refuses_inconsistent_geometry(rt):
+    d = R.Conv3dDesc()
+    (d.N, d.C, d.D, d.H, d.W, d.Cout, d.kd, d.kh, d.kw) = (1, 2, 4, 4, 4, 2, 3, 3, 3)
+    d.pad, d.stride, d.dil = (C.c_int32 * 6)(*[0] * 6), (C.c_int32 * 3)(1, 1, 1), (C.c_int32 * 3)(1, 1, 1)
+    d.group, d.OD, d.OH, d.OW = 1, 2, 2, 3  # OW should be 2
+    x = util.to_dev(np.zeros(2 * 64, np.float32))
+    w = util.to_dev(np.zeros(2 * 2 * 27, np.float32))
+    y = util.dev_empty((2 * 12,), np.float32)
+    with pytest.raises(R.SofieHipError):
+        rt.call("sofie_hip_conv3d_f32", C.byref(d), util.ptr(x), util.ptr(w), None, 0, C.c_float(0), util.ptr(y), None, None)
+    d.OW, d.group = 2, 3  # 2 channels do not split into 3 groups
+    with pytest.raises(R.SofieHipError):
+        rt.call("sofie_hip_conv3d_f32", C.byref(d), util.ptr(x), util.ptr(w), None, 0, C.c_float(0), util.ptr(y), None, None)
+
+
 def test_global_avg_pool(rt):
     X = util.normal(40, 3 * 7 * 33).reshape(3, 7, 33)
     dX = util.to_dev(X)

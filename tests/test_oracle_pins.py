@@ -102,6 +102,54 @@ def test_conv_f32_equals_direct_convolution(case):
         assert np.allclose(got, direct_conv(X, Wt, bias, pads, strides, dils, group), rtol=1e-5, atol=1e-5)
 
 
+def direct_conv3d(X, W, b, pads, strides, dils, group):
+    N, Cc = X.shape[:2]
+    Cout, Cg = W.shape[:2]
+    sp, k = X.shape[2:], W.shape[2:]
+    out = [(sp[a] + pads[a] + pads[a + 3] - (dils[a] * (k[a] - 1) + 1)) // strides[a] + 1 for a in range(3)]
+    Y = np.zeros((N, Cout, *out))
+    for n, co, od, oh, ow in itertools.product(range(N), range(Cout), *[range(o) for o in out]):
+        g = co // (Cout // group)
+        s = 0.0 if b is None else float(b[co])
+        for ci, z, y, x in itertools.product(range(Cg), *[range(v) for v in k]):
+            pos = [o * strides[a] - pads[a] + t * dils[a] for a, (o, t) in enumerate(zip((od, oh, ow), (z, y, x)))]
+            if all(0 <= pos[a] < sp[a] for a in range(3)):
+                s += float(X[n, g * Cg + ci, pos[0], pos[1], pos[2]]) * float(W[co, ci, z, y, x])
+        Y[n, co, od, oh, ow] = s
+    return Y
+
+
+CONV3D_CASES = [
+    # N, C, (D,H,W), Cout, (kd,kh,kw), pads {d0,h0,w0,d1,h1,w1}, strides, dils, group
+    (1, 1, (3, 4, 4), 2, (2, 3, 3), (0, 1, 1, 0, 1, 1), (1, 1, 1), (1, 1, 1), 1),
+    (2, 4, (5, 6, 7), 6, (3, 2, 3), (1, 0, 2, 0, 1, 1), (2, 1, 2), (1, 1, 1), 2),
+    (1, 2, (7, 5, 6), 3, (2, 3, 2), (2, 1, 0, 1, 2, 1), (1, 2, 1), (2, 1, 2), 1),
+    (1, 6, (4, 4, 4), 6, (3, 3, 3), (1, 1, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1), 3),
+]
+
+
+@pytest.mark.parametrize("case", CONV3D_CASES)
+def test_conv3d_f32_equals_direct_convolution(case):
+    # every axis has its own extent, kernel, pad pair, stride and dilation somewhere in the cases, so an axis mix-up shows
+    N, Cc, sp, Cout, k, pads, strides, dils, group = case
+    X = util.normal(15, N * Cc * int(np.prod(sp))).reshape(N, Cc, *sp)
+    Wt = util.normal(16, Cout * (Cc // group) * int(np.prod(k))).reshape(Cout, Cc // group, *k)
+    b = util.normal(17, Cout)
+    for bias in (None, b):
+        got = ob.conv3d_f32(X, Wt, bias, pads=pads, strides=strides, dils=dils, group=group)
+        want = direct_conv3d(X, Wt, bias, pads, strides, dils, group)
+        assert got.shape == want.shape
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+def test_conv3d_of_depth_one_is_the_2d_convolution():
+    X = util.normal(18, 2 * 3 * 6 * 5).reshape(2, 3, 1, 6, 5)
+    Wt = util.normal(19, 4 * 3 * 3 * 2).reshape(4, 3, 1, 3, 2)
+    got = ob.conv3d_f32(X, Wt, None, pads=(0, 1, 0, 0, 2, 1), strides=(1, 2, 1), dils=(1, 1, 2), group=1)
+    want = ob.conv_f32(X[:, :, 0], Wt[:, :, 0], None, pads=(1, 0, 2, 1), strides=(2, 1), dils=(1, 2), group=1)
+    assert np.array_equal(got[:, :, 0], want)
+
+
 def test_im2col_layout():
     # rows (c,kh,kw), columns (oh,ow), zero outside the image
     x = np.arange(2 * 3 * 3, dtype=np.float32).reshape(2, 3, 3)
