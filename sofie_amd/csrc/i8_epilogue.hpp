@@ -53,6 +53,11 @@ struct I8Epilogue {
    __device__ __forceinline__ bool rows_vectorizable() const { return stage_ok != 0; }
    // row-major output with 16-byte aligned rows, every element stored (what the register tile store handles)
    bool stores_plain_rows() const { return stage_ok != 0 && nchw_ohw == 0 && rows_per_plane == 0; }
+   // plane sums (of int8 results) whose planes are made of whole groups of `rows` GEMM rows
+   bool sums_rows_of_whole_wave_tiles(int rows) const
+   {
+      return rows_per_plane != 0 && rows_per_plane % rows == 0 && (out == SOFIE_I8OUT_I8 || out == SOFIE_I8OUT_I8_DQQ) && nchw_ohw == 0;
+   }
    __device__ __forceinline__ char *out_base() const { return (char *)Y; }
    __device__ __forceinline__ size_t out_index(int m, int n) const
    {
@@ -123,6 +128,20 @@ struct I8Epilogue {
    {
       p.b[i] = (int)w[0];
       p.s[i] = __uint_as_float(w[1]);
+   }
+
+   // the int8 results of columns 4q..4q+3 as integers (what the plane sums of a convolution add up)
+   template <int OUT, int C>
+   __device__ __forceinline__ void quantize4(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, int (&r)[4]) const
+   {
+      int acc[4] = {a0, a1, a2, a3};
+      const int acc_floor = relu_acc ? 0 : (int)0x80000000;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+         acc[i] += p.b[4 * q + i];
+         acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
+         r[i] = to_i8<OUT>(acc[i], p.s[4 * q + i]);
+      }
    }
 
    // converts columns 4q..4q+3 of the lane's columns (exact int32 dot products) into 4*out_bytes() bytes

@@ -86,6 +86,13 @@ static int launch_mfma8_conv(const LaunchCfg &lc, const ConvRows &a, int Cg, con
              : (N >= 128 && tiles(256, 128) >= 512)          ? 258
              : (N > 64 && tiles(128, 128) >= 192)            ? 128
                                                              : 64;
+   // Whole 256 x 256 tiles, at least one per CU, and a store the register path handles (NHWC rows, or the plane sums of
+   // planes that hold whole wave tiles): the persistent kernel.  512 asks for it by force.
+   if ((force_tile == 512 || (!force_tile && lc.variant == 0 && tiles(256, 256) >= 256)) && mfma8_persist_conv_applies(a, Wp, M, N, K) &&
+       (ep.stores_plain_rows() || ep.sums_rows_of_whole_wave_tiles(128)))
+      return launch_mfma8_persist_src<MfmaI8x16, EPI, PersistConvRows>(lc, PersistConvRows{a}, Wp, M, N, K, K, ep);
+   if (tile == 512)
+      tile = 256;
    switch (tile) {
    case 256:
       if (pairs)

@@ -127,9 +127,137 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
    }
 }
 
-template <class MMA, class EPI>
-__global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(const int8_t *__restrict__ A, const int8_t *__restrict__ Bt, int lda, int ldb,
-                                                                  int K, EPI ep, int tiles_m, int tiles_n, int sw)
+// The plane sums of a convolution that feeds a global average pool, from the accumulator registers: the int8 results of the
+// wave tile's rows (all in one plane) are added up per column instead of stored.  A lane adds its row blocks in registers,
+// the R lanes that share columns combine by xor-shuffles, and one lane per group of 4 columns adds the sums to memory.
+template <int MODE, class MMA, int MT, int NT, class EPI, class ACC>
+__device__ __forceinline__ void tile_sum_from_registers(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int lane,
+                                                        const uint32_t (&col_words)[EPI::kColWords])
+{
+   constexpr int R = MMA::ROWS, LK = MMA::LK, G = MMA::ACC / 4;
+   static_assert(NT * R == 64, "one column constant per lane");
+   const int lr = lane % R, lk = lane / R;
+   int first_col_addr = lk * 16;
+   asm volatile("" : "+v"(first_col_addr));
+   static_for<NT>([&](auto cj) {
+      constexpr int j = decltype(cj)::value;
+      static_for<G>([&](auto cg) {
+         constexpr int g = decltype(cg)::value;
+         constexpr int cb = j * R + g * 4 * LK;
+         typename EPI::template col_params<4> prm;
+#pragma unroll
+         for (int v = 0; v < 4; ++v) {
+            uint32_t w[EPI::kColWords];
+#pragma unroll
+            for (int k = 0; k < EPI::kColWords; ++k)
+               w[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(first_col_addr + (cb + v) * 4, (int)col_words[k]);
+            EPI::template set_column<4>(prm, v, w);
+         }
+         int sum[4] = {0, 0, 0, 0};
+         static_for<MT>([&](auto ci) {
+            constexpr int i = decltype(ci)::value;
+            int q[4];
+            ep.template quantize4<MODE, 4>(prm, 0, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3], q);
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+               sum[v] += q[v];
+         });
+#pragma unroll
+         for (int d = 1; d < R; d <<= 1)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+               sum[v] += __shfl_xor(sum[v], d, 64);
+         if (lr == 0)
+            ep.add_row_sums(m_base, n_base + cb + lk * 4, ep.N, sum);
+      });
+   });
+}
+
+template <int MODE, class MMA, int MT, int NT, class EPI, class ACC>
+__device__ __forceinline__ void tile_store_or_sum_from_registers(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int lane,
+                                                                 const uint32_t (&col_words)[EPI::kColWords])
+{
+   if constexpr (epi_can_sum_rows<EPI>::value && EPI::template out_bytes<MODE>() == 1) {
+      if (ep.sums_rows()) {
+         tile_sum_from_registers<MODE, MMA, MT, NT>(ep, acc, m_base, n_base, lane, col_words);
+         return;
+      }
+   }
+   tile_store_from_registers<MODE, MMA, MT, NT>(ep, acc, m_base, n_base, lane, col_words);
+}
+
+// The A operand of the persistent kernel.  A lane issues two load instructions per slab of A (tile rows row[0], row[1], the
+// 16 bytes at slab offset cbyte[i]).  The source keeps what it needs per TILE in a tile_state (the kernel holds two: the
+// tile being loaded and the one after it) and turns (state, instruction, reduction offset of the slab) into an address.
+struct PersistPlainRows {
+   static constexpr bool kConv = false;
+   const int8_t *A;
+   int lda;
+   struct lane_state {
+      uint32_t off[2];
+   };
+   struct tile_state {
+      const int8_t *origin; // uniform
+   };
+   __device__ __forceinline__ void init_lane(lane_state &ls, int i, int row, int cbyte) const
+   {
+      ls.off[i] = (uint32_t)row * (uint32_t)lda + (uint32_t)cbyte;
+   }
+   __device__ __forceinline__ void tile(tile_state &ts, const lane_state &, int m0) const { ts.origin = A + (size_t)m0 * (size_t)lda; }
+   static __device__ __forceinline__ void take(tile_state &dst, const tile_state &src, bool yes) { dst.origin = yes ? src.origin : dst.origin; }
+   __device__ __forceinline__ const int8_t *src(const lane_state &ls, const tile_state &ts, int i, int kbyte) const
+   {
+      return (ts.origin + kbyte) + ls.off[i]; // uniform base (scalar registers) + 32-bit lane offset
+   }
+};
+
+// Rows of a convolution read straight from the NHWC activations (the addressing of ConvRows): GEMM row m is the output
+// pixel (n, oh, ow), a 64-byte slab is 64 consecutive channels of one input pixel of one filter tap, and a tap that falls
+// outside the image reads the zero page.  Per tile a lane keeps the offsets of its two pixels and one bit per (pixel, tap).
+struct PersistConvRows {
+   static constexpr bool kConv = true;
+   ConvRows g;
+   struct lane_state {
+      int row[2], swz[2]; // swz: the chunk of the 64-byte slab row this lane supplies
+   };
+   struct tile_state {
+      int32_t off[2];
+      uint32_t mask; // bit 16*i + t: tap t of pixel i lies inside the image (at most 16 taps)
+   };
+   __device__ __forceinline__ void init_lane(lane_state &ls, int i, int row, int cbyte) const
+   {
+      ls.row[i] = row;
+      ls.swz[i] = cbyte;
+   }
+   __device__ __forceinline__ void tile(tile_state &ts, const lane_state &ls, int m0) const
+   {
+      ConvRows::lane_state<2> st;
+      g.template init<2>(st, 0, m0, ls.row[0], ls.swz[0], 0x7fffffff);
+      g.template init<2>(st, 1, m0, ls.row[1], ls.swz[1], 0x7fffffff);
+      ts.off[0] = st.off[0];
+      ts.off[1] = st.off[1];
+      ts.mask = st.mask[0] | (st.mask[1] << 16);
+   }
+   static __device__ __forceinline__ void take(tile_state &dst, const tile_state &src, bool yes)
+   {
+      dst.off[0] = yes ? src.off[0] : dst.off[0];
+      dst.off[1] = yes ? src.off[1] : dst.off[1];
+      dst.mask = yes ? src.mask : dst.mask;
+   }
+   __device__ __forceinline__ const int8_t *src(const lane_state &, const tile_state &ts, int i, int kbyte) const
+   {
+      const int tap = kbyte >> g.cg_shift; // uniform
+      const int cb = kbyte & ((1 << g.cg_shift) - 1);
+      const int khi = (tap * g.kw_recip) >> 16, kwi = tap - khi * g.kw;
+      const int toff = (khi * g.dil_h * g.W + kwi * g.dil_w) * g.C + cb;
+      const int8_t *p = g.X + (ptrdiff_t)(ts.off[i] + toff);
+      return ((ts.mask >> (16 * i + tap)) & 1u) ? p : (const int8_t *)conv_zero_page;
+   }
+};
+
+template <class MMA, class EPI, class ASRC>
+__global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const int8_t *__restrict__ Bt, int ldb, int K, EPI ep, int tiles_m,
+                                                                  int tiles_n, int sw)
 {
    constexpr int BM = 256, BN = 256, BK = 64, STAGES = 5, NW = 8, WAVES_N = 4;
    constexpr int R = MMA::ROWS;
@@ -156,32 +284,51 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(const int8_t *_
    // loader: wave instruction i of an operand fills rows (i*NW + wave)*16 .. +15 of a slab; a lane supplies the chunk that
    // belongs at its position of the swizzled layout (chunk c of row r sits at position c ^ MMA::lds_swizzle(r); the swizzle has
    // period 16 in r, so a fragment's rows r = 16*k + lr swizzle like lr)
-   uint32_t a_off[LD], b_off[LD];
+   typename ASRC::lane_state a_lane;
+   uint32_t b_off[LD];
+   auto init_a_lane = [&](typename ASRC::lane_state &ls, int ln) {
+#pragma unroll
+      for (int i = 0; i < LD; ++i) {
+         const int row = (i * NW + wave) * 16 + ln / 4;
+         A.init_lane(ls, i, row, ((ln % 4) ^ MMA::lds_swizzle(row)) * 16);
+      }
+   };
+   init_a_lane(a_lane, lane);
 #pragma unroll
    for (int i = 0; i < LD; ++i) {
       const int row = (i * NW + wave) * 16 + lane / 4;
       const int c = (lane % 4) ^ MMA::lds_swizzle(row);
-      a_off[i] = (uint32_t)row * (uint32_t)lda + (uint32_t)c * 16u;
       b_off[i] = (uint32_t)row * (uint32_t)ldb + (uint32_t)c * 16u;
    }
    // The loads run two pairs ahead of the MFMAs and cross into the next tile of the list before the current one is stored.
-   // l_a, l_b: origin of the tile being loaded; n_a, n_b: origin of the one after it, worked out once per tile (in the tile
-   // store, which needs the tile order anyway) so that the step itself has no branch.  Past the end of the list the
-   // loads start over on the last tile: filler that keeps the count of loads in flight constant; nobody reads it.
+   // l_a, l_b: the tile being loaded; n_a, n_b: the one after it, worked out once per tile (in the tile store, which needs
+   // the tile order anyway) so that the step itself has no branch.  Past the end of the list the loads start over on the
+   // last tile: filler that keeps the count of loads in flight constant; nobody reads it.
    auto tile_origin = [&](int it, int &m0, int &n0) {
       int tm, tn;
       tile_of_block((it < my_tiles ? it : my_tiles - 1) * nwg + bid, ntiles, tiles_m, tiles_n, sw, tm, tn);
       m0 = tm * BM;
       n0 = tn * BN;
    };
-   auto load_origin = [&](int it, const int8_t *&pa, const int8_t *&pb) {
+   auto load_origin = [&](int it, typename ASRC::tile_state &ta, const int8_t *&pb) {
       int m0, n0;
       tile_origin(it, m0, n0);
-      pa = A + (size_t)m0 * (size_t)lda;
+      if constexpr (ASRC::kConv) {
+         // what the source keeps per lane is only needed here, once per tile: worked out again from the lane number (made
+         // opaque, so that it is not kept in registers across the K loop instead)
+         int ln = lane;
+         asm volatile("" : "+v"(ln));
+         typename ASRC::lane_state ls;
+         init_a_lane(ls, ln);
+         A.tile(ta, ls, m0);
+      } else {
+         A.tile(ta, a_lane, m0);
+      }
       pb = Bt + (size_t)n0 * (size_t)ldb;
    };
    int l_kp = 0; // pair (of the tile being loaded) the next loads fetch
-   const int8_t *l_a, *l_b, *n_a, *n_b;
+   typename ASRC::tile_state l_a, n_a;
+   const int8_t *l_b, *n_b;
    load_origin(0, l_a, l_b);
    load_origin(1, n_a, n_b);
    // load q (0..7) of the pair: operand q/4, wave instruction (q/2)%2, half q%2 of the 128-byte line
@@ -189,16 +336,19 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(const int8_t *_
       constexpr int q = decltype(q_c)::value;
       constexpr int opnd = q / 4, i = (q / 2) % 2, half = q % 2;
       int8_t *dst = smem + (half ? slot1 : slot0) * STAGE_BYTES + opnd * (BM * BK) + (i * NW + wave) * 1024;
-      // uniform base (scalar registers) + 32-bit lane offset.  (The instruction's own offset field cannot supply the second
-      // half of the line: it is added to the LDS address as well.)
-      const int8_t *base = (opnd ? l_b : l_a) + (l_kp * (2 * BK) + half * BK);
-      const int8_t *src = base + (opnd ? b_off[i] : a_off[i]);
+      // (The instruction's own offset field cannot supply the second half of the line: it is added to the LDS address as well.)
+      const int kbyte = l_kp * (2 * BK) + half * BK;
+      const int8_t *src;
+      if constexpr (opnd == 0)
+         src = A.src(a_lane, l_a, i, kbyte);
+      else
+         src = (l_b + kbyte) + b_off[i]; // uniform base (scalar registers) + 32-bit lane offset
       __builtin_amdgcn_global_load_lds((global_void_t *)src, (lds_void_t *)dst, 16, 0, 0);
    };
    auto advance_loader = [&]() {
       const bool wrap = (l_kp + 1 == KP);
       l_kp = wrap ? 0 : l_kp + 1;
-      l_a = wrap ? n_a : l_a;
+      ASRC::take(l_a, n_a, wrap);
       l_b = wrap ? n_b : l_b;
    };
 
@@ -217,6 +367,12 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(const int8_t *_
             fa[i].c[c] = *(const v4i *)(base + a_frag + i * R * BK + (((lk * MMA::CHUNKS + c) ^ MMA::lds_swizzle(lr)) << 4));
    };
 
+   uint32_t col_words[EPI::kColWords]; // the epilogue's constants of column n0 + wn*TN + lane of the tile in work
+   {
+      int m0, n0;
+      tile_origin(0, m0, n0);
+      ep.load_column(n0 + wn * TN + lane, col_words);
+   }
    acc_t acc[MT][NT];
    auto zero_acc = [&]() {
 #pragma unroll
@@ -228,12 +384,6 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(const int8_t *_
                acc[i][j][v] = 0;
    };
    zero_acc();
-   uint32_t col_words[EPI::kColWords]; // the epilogue's constants of column n0 + wn*TN + lane of the tile in work
-   {
-      int m0, n0;
-      tile_origin(0, m0, n0);
-      ep.load_column(n0 + wn * TN + lane, col_words);
-   }
 
    // prologue: pairs 0 and 1 into slots 0..3
    static_for<8>([&](auto q) { issue_load(0, 1, q); });
@@ -306,7 +456,7 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(const int8_t *_
       int m0, n0;
       tile_origin(it, m0, n0);
       ep.dispatch([&](auto mode) {
-         tile_store_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, lane, col_words);
+         tile_store_or_sum_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, lane, col_words);
       });
       zero_acc();
       // the column constants of the next tile: fetched now, used after its K loop
@@ -324,30 +474,51 @@ inline bool mfma8_persist_applies(const int8_t *A, const int8_t *Bt, int M, int 
           (((uintptr_t)A | (uintptr_t)Bt) & 15) == 0 && (long long)(M / 256) * (N / 256) <= 0x7fffffLL &&
           (size_t)256 * (size_t)(lda > ldb ? lda : ldb) < 0xffffffffULL;
 }
-
-template <class MMA, class EPI>
-static int launch_mfma8_persist(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
+// The same for a convolution read through ConvRows (whose own conditions the caller has checked: channels per group a power
+// of two >= 64, 32-bit offsets): one bit per tap and pixel must fit the lane's mask.
+inline bool mfma8_persist_conv_applies(const ConvRows &a, const int8_t *Wp, int M, int N, int K)
 {
-   const int tiles_m = M / 256, tiles_n = N / 256;
-   const int ntiles = tiles_m * tiles_n;
-   constexpr size_t smem = (size_t)5 * 512 * 64;
-   static_assert(smem <= 160 * 1024, "LDS ring larger than the CU's LDS");
-   auto kern = mfma8_gemm_persist_kernel<MMA, EPI>;
-   static bool configured[64] = {};
-   if (int st = configure_lds_once(kern, smem, configured))
-      return st;
+   return M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0 && K >= 384 && K % 128 == 0 && a.ntaps <= 16 && (((uintptr_t)a.X | (uintptr_t)Wp) & 15) == 0 &&
+          (long long)(M / 256) * (N / 256) <= 0x7fffffLL && (size_t)256 * (size_t)K < 0xffffffffULL;
+}
+
+inline int cu_count_of_current_device(int &ncu)
+{
    static int cus[64] = {};
    int dev = 0;
    SOFIE_HIP_CHECK(hipGetDevice(&dev));
-   int ncu = (dev >= 0 && dev < 64) ? cus[dev] : 0;
+   ncu = (dev >= 0 && dev < 64) ? cus[dev] : 0;
    if (ncu == 0) {
       SOFIE_HIP_CHECK(hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev));
       if (dev >= 0 && dev < 64)
          cus[dev] = ncu;
    }
+   return SOFIE_HIP_OK;
+}
+
+template <class MMA, class EPI, class ASRC>
+static int launch_mfma8_persist_src(const LaunchCfg &lc, const ASRC &a, const int8_t *Bt, int M, int N, int K, int ldb, const EPI &ep)
+{
+   const int tiles_m = M / 256, tiles_n = N / 256;
+   const int ntiles = tiles_m * tiles_n;
+   constexpr size_t smem = (size_t)5 * 512 * 64;
+   static_assert(smem <= 160 * 1024, "LDS ring larger than the CU's LDS");
+   auto kern = mfma8_gemm_persist_kernel<MMA, EPI, ASRC>;
+   static bool configured[64] = {};
+   if (int st = configure_lds_once(kern, smem, configured))
+      return st;
+   int ncu = 0;
+   if (int st = cu_count_of_current_device(ncu))
+      return st;
    const int grid = ntiles < ncu ? ntiles : ncu;
-   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, lc.stream, A, Bt, lda, ldb, K, ep, tiles_m, tiles_n, lc.swizzle);
+   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, lc.stream, a, Bt, ldb, K, ep, tiles_m, tiles_n, lc.swizzle);
    return launch_status("mfma8_gemm_persist_kernel");
+}
+
+template <class MMA, class EPI>
+static int launch_mfma8_persist(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, const EPI &ep)
+{
+   return launch_mfma8_persist_src<MMA, EPI, PersistPlainRows>(lc, PersistPlainRows{A, lda}, Bt, M, N, K, ldb, ep);
 }
 
 } // namespace sofie_hip

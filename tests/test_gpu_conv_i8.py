@@ -130,6 +130,32 @@ def test_conv_i8_implicit_gemm_every_tile(rt, case, tile, opt):
     assert np.array_equal(got2, want)
 
 
+@pytest.mark.parametrize("case", [
+    (4, 128, 16, 16, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),       # 4 tiles, K = 1152
+    (2, 256, 16, 32, 512, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),       # 8 tiles in two columns, K = 2304
+    (2, 256, 15, 17, 512, 3, 2, (2, 0, 1, 1), (2, 1), (1, 2), 2),       # groups, stride, dilation, asymmetric pads: one tile per group
+    (257, 128, 16, 16, 256, 1, 3, (0, 1, 0, 1), (1, 1), (1, 1), 1),     # 257 tiles: more than one per workgroup
+])
+@pytest.mark.parametrize("forced", [False, True])
+def test_conv_i8_persistent_kernel(rt, case, forced, opt):
+    """Convolutions whose GEMM divides into whole 256 x 256 tiles (rows = batch x output pixels, columns = output channels per
+    group) take the persistent kernel: the rows of A are gathered from the NHWC activations tap by tap, taps outside the image
+    read zeros, and the loads run on into the workgroup's next tile."""
+    if forced:
+        opt("i8_tile", 512)
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    X = util.int8_sym(84, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.int8_sym(85, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
+    bias = util.int32_range(86, Cout, -2000, 2000)
+    K = (Cc // group) * kh * kw
+    scale = ((0.5 + util.uniform01(87, Cout)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    print("conv_i8 persistent", case, forced, flush=True)
+    want = ob.conv_i8(X, Wt, bias, scale, pads=pads, strides=strides, dils=dils, group=group, relu=1, out=2, omp=True)
+    got = run_conv(rt, X, Wt, bias, scale, case, 1, R.I8OUT_I8, R.LAYOUT_NHWC, R.LAYOUT_NHWC, 1)
+    assert np.array_equal(got, want)
+    assert (want != 0).mean() > 0.2 and np.abs(want).max() > 60  # neither all zero nor saturated
+
+
 def test_first_layer_of_an_image_network_needs_no_workspace(rt):
     """3 input channels, 3x3: K = 27 fits one slab, the rows are gathered in the kernel (NCHW in, NHWC out, a ragged last tile)."""
     case = (3, 3, 21, 19, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1)
@@ -186,7 +212,7 @@ PLANE_SUM_CASES = [
 
 @pytest.mark.parametrize("case,x_layout", PLANE_SUM_CASES)
 @pytest.mark.parametrize("relu", [0, 1])
-@pytest.mark.parametrize("tile", [0, 64, 128, 256, 258])
+@pytest.mark.parametrize("tile", [0, 64, 128, 256, 258, 512])
 def test_conv_i8_plane_sums_equal_the_sums_of_the_stored_map(rt, case, x_layout, relu, tile, opt):
     """The int8 feature map is never stored: the sums the kernel adds up in its store must be the sums of the map the
     oracle computes, and the average the bits of the oracle's DequantizeLinear + GlobalAveragePool on that map."""
