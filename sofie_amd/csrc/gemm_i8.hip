@@ -1,6 +1,7 @@
 // int8 x int8 -> int32 GEMM on the gfx950 matrix cores (v_mfma_i32_32x32x32_i8) with the
 // requantisation / dequantisation epilogue fused into the store, and the int8 re-layout kernel.
 #include "i8_epilogue.hpp"
+#include <cmath>
 #include <mutex>
 
 namespace sofie_hip {
@@ -110,7 +111,8 @@ static int gemm_i8_with_workspace(sofie_hip_ctx *ctx, const sofie_gemm_i8_desc *
       return SOFIE_HIP_OK;
    SOFIE_HIP_REQUIRE(d->Y != nullptr, "sofie_hip_gemm_i8: Y is NULL");
    SOFIE_HIP_REQUIRE(d->K == 0 || (d->A && d->B), "sofie_hip_gemm_i8: A or B is NULL");
-   SOFIE_HIP_REQUIRE(d->out != SOFIE_I8OUT_I8_DQQ || d->q_scale != 0.0f, "sofie_hip_gemm_i8: q_scale is 0");
+   SOFIE_HIP_REQUIRE(d->out != SOFIE_I8OUT_I8_DQQ || (d->q_scale != 0.0f && std::isfinite(d->q_scale)),
+                     "sofie_hip_gemm_i8: q_scale is 0 or not finite");
    const int M = d->M, N = d->N, K = d->K;
    int lda = d->lda ? d->lda : (d->transA ? M : K);
    int ldb = d->ldb ? d->ldb : (d->transB ? K : N);

@@ -140,8 +140,56 @@ struct I8Epilogue {
       for (int i = 0; i < 4; ++i) {
          acc[i] += p.b[4 * q + i];
          acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
-         r[i] = to_i8<OUT>(acc[i], p.s[4 * q + i]);
+         float v = mul_nofma((float)acc[i], p.s[4 * q + i]);
+         if (OUT == SOFIE_I8OUT_I8_DQQ)
+            v = __fdiv_rn(v, q_scale);
+         r[i] = (int)i8_bits(v, (OUT == SOFIE_I8OUT_I8 && relu_out) ? 0.0f : -128.0f) - 0x4B400000; // needs the tamed scale, like pack4_short
       }
+   }
+
+   // sat8(rne(v)), clamped below at lo (-128, or 0 when a relu follows): the low byte of the returned word.  v is clamped to
+   // [lo, 127] first (the bounds are integers: clamping commutes with the rounding), then 1.5 * 2^23 is added: the sum lies
+   // in [2^23, 2^24), where floats are the integers, so the addition itself rounds to the nearest integer, ties to even (the
+   // constant is even), and leaves that integer in the low mantissa bits.  Two instructions instead of the four of
+   // quantize_rne_clamp.  NaN is clamped to lo by v_med3_f32 where quantize_rne_clamp gives 0: the caller keeps NaN out.
+   static __device__ __forceinline__ uint32_t i8_bits(float v, float lo)
+   {
+      const float c = __builtin_amdgcn_fmed3f(v, lo, 127.0f);
+      return __float_as_uint(c + 12582912.0f);
+   }
+   // pack4 for the 1-byte outputs with the short conversion.  float(acc) * s is NaN only for a scale that is NaN, or
+   // infinite against an accumulator of 0; load_column_tamed() below replaces such scales by ones that give the same results
+   // without NaN.
+   template <int OUT, int C>
+   __device__ __forceinline__ void pack4_short(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, uint32_t *w) const
+   {
+      static_assert(OUT == SOFIE_I8OUT_I8 || OUT == SOFIE_I8OUT_I8_DQQ, "1-byte outputs");
+      int acc[4] = {a0, a1, a2, a3};
+      uint32_t b[4];
+      const int acc_floor = relu_acc ? 0 : (int)0x80000000;
+      const float lo = (OUT == SOFIE_I8OUT_I8 && relu_out) ? 0.0f : -128.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+         acc[i] += p.b[4 * q + i];
+         acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
+         float v = mul_nofma((float)acc[i], p.s[4 * q + i]);
+         if (OUT == SOFIE_I8OUT_I8_DQQ)
+            v = __fdiv_rn(v, q_scale);
+         b[i] = i8_bits(v, lo);
+      }
+      const uint32_t lo2 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+      const uint32_t hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u);
+      w[0] = __builtin_amdgcn_perm(hi2, lo2, 0x05040100u);
+   }
+   // load_column with the scale made safe for pack4_short: NaN becomes 0 and +-inf the largest finite number.  The results
+   // are those of the plain scale: a NaN product is stored as 0, and so is 0 * s; a non-zero accumulator times +-inf
+   // saturates like one times +-FLT_MAX.
+   __device__ __forceinline__ void load_column_tamed(int n, uint32_t (&w)[kColWords]) const
+   {
+      load_column(n, w);
+      float s = __uint_as_float(w[1]);
+      s = (s == s) ? s : 0.0f;
+      w[1] = __float_as_uint(__builtin_amdgcn_fmed3f(s, -3.402823466e38f, 3.402823466e38f));
    }
 
    // converts columns 4q..4q+3 of the lane's columns (exact int32 dot products) into 4*out_bytes() bytes

@@ -111,7 +111,7 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
             column_constants(j * R, prm);
             static_for<IB>([&](auto ci) {
                constexpr int i = decltype(ci)::value;
-               ep.template pack4<MODE, 4>(prm, 0, acc[i0 + i][j][0], acc[i0 + i][j][1], acc[i0 + i][j][2], acc[i0 + i][j][3], &w[i][j]);
+               ep.template pack4_short<MODE, 4>(prm, 0, acc[i0 + i][j][0], acc[i0 + i][j][1], acc[i0 + i][j][2], acc[i0 + i][j][3], &w[i][j]);
             });
          });
          static_for<IB>([&](auto ci) {
@@ -371,7 +371,7 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const i
    {
       int m0, n0;
       tile_origin(0, m0, n0);
-      ep.load_column(n0 + wn * TN + lane, col_words);
+      ep.load_column_tamed(n0 + wn * TN + lane, col_words);
    }
    acc_t acc[MT][NT];
    auto zero_acc = [&]() {
@@ -461,7 +461,7 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const i
       zero_acc();
       // the column constants of the next tile: fetched now, used after its K loop
       tile_origin(it + 1, m0, n0);
-      ep.load_column(n0 + wn * TN + lane, col_words);
+      ep.load_column_tamed(n0 + wn * TN + lane, col_words);
    }
    wait_vmcnt<0>();
 }
