@@ -72,29 +72,43 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
          });
       });
    } else if constexpr (ESZ == 2) {
-      // 2-byte elements, R = 32: a lane's 4 columns of group g are 8 bytes at column g*8 + lk*4.  The two lanes of a row swap
-      // so that lane lk = 0 ends up with the 8 columns of an even group and lane lk = 1 with those of the odd group after it:
-      // 16 consecutive bytes each.
+      // 2-byte elements, R = 32: a lane's 4 columns of group g are 8 bytes at column g*8 + lk*4 of the 32-column block.  First
+      // the two lanes of a row swap so that lane lk holds the 8 columns (16 bytes) of group 2p + lk, for p = 0 and p = 1: the
+      // four 16-byte chunks of the block's 64-byte row segment, two per lane.  Then the lanes of rows 0..15 and of rows 16..31
+      // swap chunks, so that one register holds all four chunks of rows 0..15 and the other those of rows 16..31: a wave
+      // instruction writes whole 64-byte segments (stored pairwise instead, every segment would be written as two halves).
       static_assert(R == 32 && G == 4, "2-byte outputs are exchanged between the two lanes of a row of the 32 x 32 block");
+      const int q16 = lane >> 4;
+      const int chunk = ((q16 & 1) << 1) | (q16 >> 1); // which chunk a lane ends up with: lanes 0-15: 0, 16-31: 2, 32-47: 1, 48-63: 3
       static_for<NT>([&](auto cj) {
          constexpr int j = decltype(cj)::value;
-         static_for<2>([&](auto cgp) {
-            constexpr int ge = decltype(cgp)::value * 2, go = ge + 1;
-            typename EPI::template col_params<4> pe, po;
-            column_constants(j * R + ge * 4 * LK, pe);
-            column_constants(j * R + go * 4 * LK, po);
-            static_for<MT>([&](auto ci) {
-               constexpr int i = decltype(ci)::value;
+         typename EPI::template col_params<4> prm[4];
+         static_for<4>([&](auto cg) { column_constants(j * R + decltype(cg)::value * 4 * LK, prm[decltype(cg)::value]); });
+         static_for<MT>([&](auto ci) {
+            constexpr int i = decltype(ci)::value;
+            uint32_t lo[4], hi[4]; // the 16 bytes of group lk (lo) and of group 2 + lk (hi)
+            static_for<2>([&](auto cp) {
+               constexpr int ge = decltype(cp)::value * 2, go = ge + 1;
                uint32_t we[2], wo[2];
-               ep.template pack4<MODE, 4>(pe, 0, acc[i][j][4 * ge + 0], acc[i][j][4 * ge + 1], acc[i][j][4 * ge + 2], acc[i][j][4 * ge + 3], we);
-               ep.template pack4<MODE, 4>(po, 0, acc[i][j][4 * go + 0], acc[i][j][4 * go + 1], acc[i][j][4 * go + 2], acc[i][j][4 * go + 3], wo);
+               ep.template pack4<MODE, 4>(prm[ge], 0, acc[i][j][4 * ge + 0], acc[i][j][4 * ge + 1], acc[i][j][4 * ge + 2], acc[i][j][4 * ge + 3], we);
+               ep.template pack4<MODE, 4>(prm[go], 0, acc[i][j][4 * go + 0], acc[i][j][4 * go + 1], acc[i][j][4 * go + 2], acc[i][j][4 * go + 3], wo);
                // swap(a, b): a keeps its lower 32 lanes and receives b's lower 32 lanes in its upper half; b the other way round
                auto s0 = __builtin_amdgcn_permlane32_swap(we[0], wo[0], false, false);
                auto s1 = __builtin_amdgcn_permlane32_swap(we[1], wo[1], false, false);
-               // lane lk: group ge + lk, columns 0..3 in s0[0], s1[0] and columns 4..7 in s0[1], s1[1]
-               const int n = n_base + j * R + (ge + lk) * 4 * LK;
-               *(uint4 *)(out + ep.out_index(m_base + i * R + lr, n) * 2) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+               uint32_t *dst = decltype(cp)::value ? hi : lo;
+               dst[0] = s0[0], dst[1] = s1[0], dst[2] = s0[1], dst[3] = s1[1];
             });
+            uint32_t top[4], bot[4];
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+               // swap(a, b) of 16-lane rows: a = {a.row0, b.row0, a.row2, b.row2}, b = {a.row1, b.row1, a.row3, b.row3}
+               auto t = __builtin_amdgcn_permlane16_swap(lo[d], hi[d], false, false);
+               top[d] = t[0];
+               bot[d] = t[1];
+            }
+            const int n = n_base + j * R + chunk * 8;
+            *(uint4 *)(out + ep.out_index(m_base + i * R + (lane & 15), n) * 2) = make_uint4(top[0], top[1], top[2], top[3]);
+            *(uint4 *)(out + ep.out_index(m_base + i * R + 16 + (lane & 15), n) * 2) = make_uint4(bot[0], bot[1], bot[2], bot[3]);
          });
       });
    } else {
