@@ -281,6 +281,39 @@ def organize_memory(begin, end, size, lib=None, fn="oracle_organize_memory"):
             "largest_free_block": lfree.value}
 
 
+def plan_memory_greedy(ops, sizes, model_outputs=()):
+    """The reference's CPU-path pool planner.  ops: one (outputs, inputs) pair of tensor-id lists per operator, in execution
+    order (inputs that are model inputs or weights: any id < 0); sizes[t]: bytes of tensor t; model_outputs: ids never released.
+    A tensor is released after the last operator that reads it (core/src/RModel.cxx:220-249); one that nothing reads has its
+    producer as last use (:773-782) but keeps its chunk, because only an operator's inputs are ever released (:606-613).  Returns {"offsets": [...], "pool_bytes": n}."""
+    n_t = len(sizes)
+    last = [-2] * n_t
+    for i, (outs, ins) in enumerate(ops):
+        for t in ins:
+            if t >= 0:
+                last[t] = i
+    for i, (outs, ins) in enumerate(ops):
+        for t in outs:
+            if last[t] == -2:
+                last[t] = i
+    for t in model_outputs:
+        last[t] = -1
+    out_ptr, out_ids, in_ptr, in_ids = [0], [], [0], []
+    for outs, ins in ops:
+        out_ids += list(outs)
+        in_ids += list(ins)
+        out_ptr.append(len(out_ids))
+        in_ptr.append(len(in_ids))
+    arr = lambda v: (C.c_int * max(1, len(v)))(*v)
+    off = (C.c_size_t * n_t)()
+    pool = C.c_size_t()
+    rc = load().oracle_plan_memory_greedy(len(ops), arr(out_ptr), arr(out_ids), arr(in_ptr), arr(in_ids), n_t,
+                                          (C.c_size_t * n_t)(*sizes), arr(last), off, C.byref(pool))
+    if rc:
+        raise MemoryError("oracle_plan_memory_greedy")
+    return {"offsets": list(off), "pool_bytes": pool.value, "last_use": last}
+
+
 def quantize_linear(x, scale):
     x = _f32(x)
     q = np.empty(x.shape, dtype=np.int8)

@@ -664,6 +664,170 @@ ORACLE_API void oracle_batchnorm(float *Y, const float *X, const float *fused_sc
 typedef struct {
    size_t off, size;
 } free_block;
+/* ---- the CPU path's pool planner -------------------------------------------------------------------------------
+ * RModel::AllocateIntermediateMemory / CheckAndFlushIntermediateMemory (core/src/RModel.cxx:492-595, 597-674), driven
+ * operator by operator as RModel::Generate does (:1474-1482): the outputs of an operator, largest first, each go into the
+ * first free chunk that holds them (cut from the chunk's END), or grow the last chunk of the pool if that one is free, or
+ * are appended; then every input whose last reader this operator is gives its chunk back, merging with free neighbours.
+ * The pool is the end of the last chunk (GenerateIntermediateMemoryPool, :975-984).  The GPU backend plans with
+ * OrganizeMemory (above), not with this; the function exists to pin the reference's other answer (Linear_16: 6400 B).
+ *   ops: operator i produces tensors out_ids[out_ptr[i] .. out_ptr[i+1]) and reads in_ids[in_ptr[i] .. in_ptr[i+1]);
+ *   last_use[t]: index of the operator after which t is released if t is among that operator's inputs, or -1 (a model
+ *   output: never released). */
+typedef struct {
+   size_t off, size;
+   int name; /* tensor id, or -1 for a free chunk */
+} pool_chunk;
+typedef struct {
+   size_t off, size;
+} free_chunk;
+
+static int chunk_find(const pool_chunk *c, int n, size_t off)
+{
+   for (int i = 0; i < n; ++i)
+      if (c[i].off == off)
+         return i;
+   return -1;
+}
+/* total_stack[off] = {name, size}: replaces the entry at off or inserts one, keeping the offsets ascending */
+static void chunk_set(pool_chunk *c, int *n, size_t off, int name, size_t size)
+{
+   int i = chunk_find(c, *n, off);
+   if (i < 0) {
+      i = *n;
+      while (i > 0 && c[i - 1].off > off) {
+         c[i] = c[i - 1];
+         --i;
+      }
+      ++*n;
+   }
+   c[i].off = off, c[i].name = name, c[i].size = size;
+}
+static void chunk_erase(pool_chunk *c, int *n, size_t off)
+{
+   int i = chunk_find(c, *n, off);
+   if (i < 0)
+      return;
+   for (; i + 1 < *n; ++i)
+      c[i] = c[i + 1];
+   --*n;
+}
+static void free_insert(free_chunk *f, int *n, size_t off, size_t size)
+{
+   int i = *n;
+   while (i > 0 && f[i - 1].off > off) {
+      f[i] = f[i - 1];
+      --i;
+   }
+   f[i].off = off, f[i].size = size;
+   ++*n;
+}
+static void free_erase(free_chunk *f, int *n, int i)
+{
+   for (; i + 1 < *n; ++i)
+      f[i] = f[i + 1];
+   --*n;
+}
+
+ORACLE_API int oracle_plan_memory_greedy(int n_ops, const int *out_ptr, const int *out_ids, const int *in_ptr, const int *in_ids,
+                                         int n_tensors, const size_t *size, const int *last_use, size_t *offset, size_t *pool_bytes)
+{
+   pool_chunk *total = (pool_chunk *)malloc(sizeof(pool_chunk) * (size_t)(2 * n_tensors + 2));
+   free_chunk *avail = (free_chunk *)malloc(sizeof(free_chunk) * (size_t)(2 * n_tensors + 2));
+   int *order = (int *)malloc(sizeof(int) * (size_t)(n_tensors + 1));
+   if (!total || !avail || !order) {
+      free(total), free(avail), free(order);
+      return 1;
+   }
+   int nt = 0, na = 0;
+   for (int op = 0; op < n_ops; ++op) {
+      /* outputs ordered by size, largest first (:524-525; equal sizes keep their order here) */
+      int no = 0;
+      for (int k = out_ptr[op]; k < out_ptr[op + 1]; ++k) {
+         int t = out_ids[k], i = no++;
+         while (i > 0 && size[order[i - 1]] < size[t]) {
+            order[i] = order[i - 1];
+            --i;
+         }
+         order[i] = t;
+      }
+      for (int k = 0; k < no; ++k) {
+         const int t = order[k];
+         const size_t sz = size[t];
+         int done = 0;
+         for (int a = 0; a < na; ++a) {
+            if (avail[a].size >= sz) {
+               /* cut from the end of the free chunk (:540-547) */
+               const size_t at = avail[a].off, loc = at + avail[a].size - sz;
+               total[chunk_find(total, nt, at)].size -= sz;
+               chunk_set(total, &nt, loc, t, sz);
+               offset[t] = loc;
+               avail[a].size -= sz;
+               if (avail[a].size == 0)
+                  free_erase(avail, &na, a);
+               done = 1;
+               break;
+            } else if (a == na - 1 && total[nt - 1].off == avail[a].off) {
+               /* the last free chunk is the last of the pool: it grows (:560-568) */
+               chunk_set(total, &nt, avail[a].off, t, sz);
+               offset[t] = avail[a].off;
+               free_erase(avail, &na, a);
+               done = 1;
+               break;
+            }
+         }
+         if (!done) {
+            const size_t at = nt ? total[nt - 1].off + total[nt - 1].size : 0;
+            chunk_set(total, &nt, at, t, sz);
+            offset[t] = at;
+         }
+      }
+      for (int k = in_ptr[op]; k < in_ptr[op + 1]; ++k) {
+         const int t = in_ids[k];
+         if (t < 0 || last_use[t] != op)
+            continue;
+         int c = -1;
+         for (int i = 0; i < nt; ++i)
+            if (total[i].name == t) {
+               c = i;
+               break;
+            }
+         if (c < 0)
+            continue;
+         const size_t coff = total[c].off, csz = total[c].size;
+         int g = 0; /* first free chunk above coff */
+         while (g < na && avail[g].off <= coff)
+            ++g;
+         const int sm = g - 1; /* last free chunk below */
+         if (sm >= 0 && avail[sm].off + avail[sm].size == coff) {
+            avail[sm].size += csz;
+            total[chunk_find(total, nt, avail[sm].off)].size += csz;
+            if (g < na && avail[sm].off + avail[sm].size == avail[g].off) {
+               const size_t goff = avail[g].off;
+               avail[sm].size += avail[g].size;
+               total[chunk_find(total, nt, avail[sm].off)].size += total[chunk_find(total, nt, goff)].size;
+               chunk_erase(total, &nt, goff);
+               free_erase(avail, &na, g);
+            }
+            chunk_erase(total, &nt, coff);
+         } else if (g < na && coff + csz == avail[g].off) {
+            const size_t goff = avail[g].off, merged = csz + avail[g].size;
+            free_erase(avail, &na, g);
+            free_insert(avail, &na, coff, merged);
+            total[c].size += total[chunk_find(total, nt, goff)].size;
+            chunk_erase(total, &nt, goff);
+            total[chunk_find(total, nt, coff)].name = -1;
+         } else {
+            free_insert(avail, &na, coff, csz);
+            total[c].name = -1;
+         }
+      }
+   }
+   *pool_bytes = nt ? total[nt - 1].off + total[nt - 1].size : 0;
+   free(total), free(avail), free(order);
+   return 0;
+}
+
 typedef struct {
    int t, type, idx;
 } mem_event;

@@ -160,6 +160,88 @@ def test_im2col_layout():
     assert col[4].tolist() == [0, 0, 9, 10, 12, 13]           # c=1,kh=0,kw=0
 
 
+# ---- the CPU path's greedy pool planner ------------------------------------------------------------------------
+
+def check_greedy_plan(ops, sizes, plan, model_outputs=()):
+    """Tensors alive at the same time do not share bytes, and everything lies inside the pool.  A tensor is alive from its
+    producer until after its last reader (until the end for a model output)."""
+    prod = {t: i for i, (outs, ins) in enumerate(ops) for t in outs}
+    last = plan["last_use"]
+    end = lambda t: len(ops) if last[t] < 0 else last[t]
+    off = plan["offsets"]
+    for a in prod:
+        assert off[a] + sizes[a] <= plan["pool_bytes"]
+        for b in prod:
+            if a < b and prod[a] <= end(b) and prod[b] <= end(a):  # alive together at some operator (released AFTER the last reader ran)
+                assert off[a] + sizes[a] <= off[b] or off[b] + sizes[b] <= off[a], (a, b)
+
+
+def test_greedy_planner_linear16_is_two_buffers_of_3200():
+    # the reference's CPU Session of Linear_16: 10 Gemm(+Relu) operators, outputs 9 x [16,50] and [16,10], fp32;
+    # its generated pool is std::vector<char>(6400): two 3200-byte buffers used in turn
+    sizes = [3200] * 9 + [640]
+    ops = [([i], [i - 1]) for i in range(10)]  # operator 0 reads the model input (id -1)
+    plan = ob.plan_memory_greedy(ops, sizes, model_outputs=[9])
+    assert plan["pool_bytes"] == 6400
+    assert plan["offsets"][:9] == [0, 3200] * 4 + [0]
+    assert plan["offsets"][9] == 3200 + 3200 - 640   # cut from the END of the free chunk
+    check_greedy_plan(ops, sizes, plan, [9])
+
+
+def test_greedy_planner_hand_worked_cases():
+    # outputs of one operator are placed largest first; a tensor nothing reads is released by its own producer
+    ops = [([0, 1], [-1]), ([2], [1]), ([3], [2, 0])]
+    sizes = [100, 300, 50, 400]
+    plan = ob.plan_memory_greedy(ops, sizes, model_outputs=[3])
+    # op 0: tensor 1 (300) at 0, tensor 0 (100) at 300.  op 1: tensor 2 (50) appended at 400, then tensor 1 is released: free [0,300).
+    # op 2: tensor 3 (400) does not fit [0,300), which is not the last chunk either: appended at 450; pool 850.
+    assert plan["offsets"] == [300, 0, 400, 450] and plan["pool_bytes"] == 850
+    # a free last chunk grows: A(100) released, then B(500) takes its place and the pool is 500, not 600
+    ops = [([0], [-1]), ([1], [0]), ([2], [1])]
+    plan = ob.plan_memory_greedy(ops, [100, 64, 500], model_outputs=[2])
+    # op 1: tensor 1 appended at 100, tensor 0 released: free [0,100).  op 2: 500 > 100 and the free chunk is not the last one:
+    # appended at 164; then tensor 1 released and merged with [0,100): free [0,164)
+    assert plan["offsets"] == [0, 100, 164] and plan["pool_bytes"] == 664
+    ops = [([0], [-1]), ([1], [-1]), ([2], [0, 1]), ([3], [2])]
+    plan = ob.plan_memory_greedy(ops, [100, 200, 40, 900], model_outputs=[3])
+    # op 2: tensor 2 at 300; tensors 0 and 1 released and merged: free [0,300).  op 3: 900 > 300; the free chunk [0,300) is the last
+    # free one but not the last of the pool ([300,340) is tensor 2): appended at 340; pool 1240
+    assert plan["offsets"] == [0, 100, 300, 340] and plan["pool_bytes"] == 1240
+    ops = [([0], [-1]), ([1], [0]), ([2], [-1])]
+    plan = ob.plan_memory_greedy(ops, [100, 50, 700], model_outputs=[2])
+    # a tensor nobody reads is never given back (only an operator's INPUTS are released): tensor 1 stays at [100,150), the free
+    # chunk [0,100) is not the last of the pool, tensor 2 is appended at 150
+    assert plan["offsets"] == [0, 100, 150] and plan["pool_bytes"] == 850
+    ops = [([0], [-1]), ([1], [0]), ([2], [1]), ([3], [2])]
+    plan = ob.plan_memory_greedy(ops, [100, 50, 30, 500], model_outputs=[3])
+    # op 1: tensor 1 at 100, tensor 0 released: free [0,100).  op 2: tensor 2 (30) is cut from the END of that chunk: [70,100); tensor 1
+    # released: free [0,70) and [100,150).  op 3: 500 fits neither, but [100,150) is the last free chunk AND the last of the pool:
+    # it grows in place; pool 600
+    assert plan["offsets"] == [0, 100, 70, 100] and plan["pool_bytes"] == 600
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_greedy_planner_never_overlaps_live_tensors(seed):
+    rng = np.random.default_rng(seed)
+    n_ops = int(rng.integers(3, 25))
+    ops, sizes, made = [], [], []
+    for i in range(n_ops):
+        k = int(rng.integers(1, 4))
+        outs = list(range(len(sizes), len(sizes) + k))
+        sizes += [int(rng.integers(1, 40)) * 16 for _ in range(k)]
+        ins = [int(t) for t in rng.choice(made, size=min(len(made), int(rng.integers(0, 4))), replace=False)] if made else [-1]
+        ops.append((outs, ins or [-1]))
+        made += outs
+    outputs = [made[-1]]
+    plan = ob.plan_memory_greedy(ops, sizes, model_outputs=outputs)
+    check_greedy_plan(ops, sizes, plan, outputs)
+    # never smaller than what is alive at once, never larger than everything laid end to end
+    prod = {t: i for i, (outs, ins) in enumerate(ops) for t in outs}
+    last = plan["last_use"]
+    peak = max(sum(sizes[t] for t in prod if prod[t] <= i and (last[t] < 0 or last[t] >= i)) for i in range(n_ops))
+    assert peak <= plan["pool_bytes"] <= sum(sizes)
+
+
 # ---- memory planner -----------------------------------------------------------------------------------------
 
 def check_plan(begin, end, size, plan):
