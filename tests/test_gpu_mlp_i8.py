@@ -97,7 +97,8 @@ def test_inference_captured_in_a_hip_graph_replays_correctly():
             sess.upload_input(inp)
             rt.call("sofie_hip_fill_zero", sess.y_ptr, C.c_size_t(y.nbytes))   # eager work between the replays
             rt.sync()
-            graph.replay()
+            with torch.cuda.stream(stream):   # a replay goes to torch's CURRENT stream: make that the one the download follows
+                graph.replay()
             stream.synchronize()
             got = fetch()
             assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), "replay %d" % replay
