@@ -404,6 +404,20 @@ typedef struct sofie_pool_desc {
    int32_t dynamic_divisor; /* the reference sets it when any padding is non-zero or ceil_mode is on */
 } sofie_pool_desc;
 int sofie_hip_pool_f32(sofie_hip_ctx *ctx, const sofie_pool_desc *d, float *Y, const float *X);
+/* The same over three spatial axes, slowest first (the third branch of ROperator_Pool::Generate,
+ * core/inc/SOFIE/operators/ROperator_Pool.hxx:293-300, 421-475): the window is visited axis 0, then 1, then 2, the divisor of an
+ * average is the product of the three window extents (:433-438).  k is the window per axis (the dilated extent). */
+typedef struct sofie_pool3d_desc {
+   int32_t planes; /* N * C */
+   int32_t in[3], out[3];
+   int32_t k[3];
+   int32_t pad_begin[3], pad_end[3];
+   int32_t stride[3];
+   int32_t mode; /* SOFIE_POOL_* */
+   int32_t count_include_pad;
+   int32_t dynamic_divisor;
+} sofie_pool3d_desc;
+int sofie_hip_pool3d_f32(sofie_hip_ctx *ctx, const sofie_pool3d_desc *d, float *Y, const float *X);
 /* int8 input, fp32 output: Y = (float(sum_i32) * scale) / float(HW), exact sum -- not in the reference. */
 int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y /* [N,C] */, const int8_t *X, int32_t N, int32_t C, int32_t HW,
                                  int32_t x_layout /* SOFIE_LAYOUT_* */, float scale);

@@ -185,9 +185,20 @@ def pool_axes(in_shape, kernel_shape, pads=None, strides=None, dilations=None, a
 
 
 def pool(X, mode, kernel_shape, pads=None, strides=None, dilations=None, auto_pad="NOTSET", ceil_mode=0, count_include_pad=0):
-    """MaxPool (mode "max") / AveragePool (mode "average") of an [N, C, W] or [N, C, H, W] tensor."""
+    """MaxPool (mode "max") / AveragePool (mode "average") of an [N, C, W], [N, C, H, W] or [N, C, D, H, W] tensor."""
     X = _f32(X)
     axes = pool_axes(X.shape[2:], kernel_shape, pads, strides, dilations, auto_pad, ceil_mode)
+    if len(axes) == 3:
+        planes = X.shape[0] * X.shape[1]
+        Y = np.empty(X.shape[:2] + tuple(a[1] for a in axes), dtype=np.float32)
+        i3 = lambda col: (C.c_int * 3)(*[a[col] for a in axes])
+        lib = load()
+        lib.oracle_pool3d.restype = C.c_long
+        per_plane = lib.oracle_pool3d(_ptr(Y), _ptr(X), planes, i3(0), i3(2), i3(4), i3(5), i3(3), 1 if mode == "max" else 0, int(ceil_mode),
+                                      int(count_include_pad))
+        if planes and per_plane != axes[0][1] * axes[1][1] * axes[2][1]:
+            raise AssertionError("pool: the loops wrote %d outputs per plane, the shape says %s" % (per_plane, [a[1] for a in axes]))
+        return Y
     if len(axes) == 1:
         axes = [(1, 1, 1, 1, 0, 0)] + axes
     (H, OH, kh, sh, ph0, ph1), (W, OW, kw, sw, pw0, pw1) = axes

@@ -480,7 +480,7 @@ ORACLE_API void oracle_global_avg_pool(float *Y, const float *X, int NC, int HW)
    }
 }
 
-/* MaxPool / AveragePool in 2-D (1-D: H = kh = 1), the generated loops of core/inc/SOFIE/operators/ROperator_Pool.hxx:
+/* MaxPool / AveragePool in 2-D (1-D: H = kh = 1; 3-D: oracle_pool3d below), the generated loops of core/inc/SOFIE/operators/ROperator_Pool.hxx:
  * bounds hmin = -pad_begin, hmax = H + pad_end - kh + 1 (ceil_mode: + stride instead of + 1, clipped to H) (:286-300);
  * window start walks hmin, hmin + stride, ... < hmax (:373-374); MaxPool keeps `xval > value` from -INFINITY (:376,
  * 394-396); AveragePool sums in window order and divides by float(nsum), nsum = kh*kw without padding and ceil_mode, else
@@ -532,6 +532,60 @@ ORACLE_API long oracle_pool2d(float *Y, const float *X, int planes, int H, int W
             Y[out++] = value;
          }
       }
+   }
+   return planes ? (long)(out / (size_t)planes) : 0;
+}
+
+/* The same over three spatial axes (core/inc/SOFIE/operators/ROperator_Pool.hxx:293-300 bounds of the third axis, :421-475 the
+ * generated loops): window starts i, j, k walk the three axes slowest first, the window is visited l, m, p in that order, the
+ * divisor of an average is the product of the three extents (:433-438).  in/k/pad_begin/pad_end/stride are per axis. */
+ORACLE_API long oracle_pool3d(float *Y, const float *X, int planes, const int *in, const int *k, const int *pad_begin, const int *pad_end,
+                              const int *stride, int is_max, int ceil_mode, int count_include_pad)
+{
+   int lo[3], hi[3], dynamic_divisor = ceil_mode;
+   for (int a = 0; a < 3; ++a) {
+      lo[a] = -pad_begin[a];
+      hi[a] = in[a] + pad_end[a] - k[a] + (ceil_mode ? stride[a] : 1);
+      if (ceil_mode && hi[a] > in[a])
+         hi[a] = in[a];
+      dynamic_divisor |= pad_begin[a] > 0 || pad_end[a] > 0;
+   }
+   const size_t s0 = (size_t)in[1] * in[2], s1 = (size_t)in[2];
+   size_t out = 0;
+   for (int n = 0; n < planes; ++n) {
+      const float *x = X + (size_t)n * in[0] * s0;
+      for (int i = lo[0]; i < hi[0]; i += stride[0])
+         for (int j = lo[1]; j < hi[1]; j += stride[1])
+            for (int kk = lo[2]; kk < hi[2]; kk += stride[2]) {
+               float value = is_max ? -INFINITY : 0;
+               int nsum = k[0] * k[1] * k[2];
+               if (!is_max && dynamic_divisor)
+                  nsum = oracle_pool_extent(i, k[0], in[0], pad_end[0], count_include_pad) *
+                         oracle_pool_extent(j, k[1], in[1], pad_end[1], count_include_pad) *
+                         oracle_pool_extent(kk, k[2], in[2], pad_end[2], count_include_pad);
+               for (int l = i; l < i + k[0]; l++) {
+                  if (l < 0 || l >= in[0])
+                     continue;
+                  for (int m = j; m < j + k[1]; m++) {
+                     if (m < 0 || m >= in[1])
+                        continue;
+                     for (int p = kk; p < kk + k[2]; p++) {
+                        if (p < 0 || p >= in[2])
+                           continue;
+                        float xval = x[l * s0 + m * s1 + p];
+                        if (is_max) {
+                           if (xval > value)
+                              value = xval;
+                        } else {
+                           value += xval;
+                        }
+                     }
+                  }
+               }
+               if (!is_max)
+                  value /= (float)nsum;
+               Y[out++] = value;
+            }
    }
    return planes ? (long)(out / (size_t)planes) : 0;
 }

@@ -85,41 +85,54 @@ __global__ __launch_bounds__(256) void unary_f32_kernel(float *dst, const float 
    }
 }
 
-// One output element per thread (grid-stride); neighbouring lanes take neighbouring ow, so the window rows they read
-// overlap and lie next to each other in memory.  The sum of an average runs in the reference's order (window rows
-// outermost), one fp32 addition at a time, so the result has the bits of the reference's scalar loop.
-__global__ __launch_bounds__(256) void pool_f32_kernel(float *__restrict__ Y, const float *__restrict__ X, sofie_pool_desc d, size_t total)
+// One output element per thread (grid-stride); neighbouring lanes take neighbouring outputs of the fastest axis, so the
+// window rows they read overlap and lie next to each other in memory.  Three spatial axes, slowest first (a 2-D pooling has a
+// first axis of extent 1): the window is visited axis 0, then 1, then 2, one fp32 addition at a time -- the order of the
+// reference's generated loops, so an average has the bits of the reference's scalar loop.
+__global__ __launch_bounds__(256) void pool_f32_kernel(float *__restrict__ Y, const float *__restrict__ X, sofie_pool3d_desc d, size_t total)
 {
    const size_t stride = (size_t)gridDim.x * blockDim.x;
+   const size_t s0 = (size_t)d.in[1] * (size_t)d.in[2], s1 = (size_t)d.in[2];
    for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += stride) {
-      const int ow = (int)(idx % (size_t)d.OW);
-      const size_t t = idx / (size_t)d.OW;
-      const int oh = (int)(t % (size_t)d.OH);
-      const size_t plane = t / (size_t)d.OH;
-      const int i = oh * d.stride_h - d.pad_h0, j = ow * d.stride_w - d.pad_w0;
-      const float *x = X + plane * (size_t)d.H * (size_t)d.W;
+      const int o2 = (int)(idx % (size_t)d.out[2]);
+      size_t t = idx / (size_t)d.out[2];
+      const int o1 = (int)(t % (size_t)d.out[1]);
+      t /= (size_t)d.out[1];
+      const int o0 = (int)(t % (size_t)d.out[0]);
+      const size_t plane = t / (size_t)d.out[0];
+      const int i = o0 * d.stride[0] - d.pad_begin[0], j = o1 * d.stride[1] - d.pad_begin[1], k = o2 * d.stride[2] - d.pad_begin[2];
+      const float *x = X + plane * (size_t)d.in[0] * s0;
       float value = d.mode == SOFIE_POOL_MAX ? -INFINITY : 0.0f;
-      for (int l = i; l < i + d.kh; ++l) {
-         if (l < 0 || l >= d.H)
+      for (int l = i; l < i + d.k[0]; ++l) {
+         if (l < 0 || l >= d.in[0])
             continue;
-         for (int m = j; m < j + d.kw; ++m) {
-            if (m < 0 || m >= d.W)
+         for (int m = j; m < j + d.k[1]; ++m) {
+            if (m < 0 || m >= d.in[1])
                continue;
-            const float xv = x[(size_t)l * d.W + m];
-            if (d.mode == SOFIE_POOL_MAX) {
-               if (xv > value)
-                  value = xv;
-            } else {
-               value += xv;
+            for (int p = k; p < k + d.k[2]; ++p) {
+               if (p < 0 || p >= d.in[2])
+                  continue;
+               const float xv = x[(size_t)l * s0 + (size_t)m * s1 + p];
+               if (d.mode == SOFIE_POOL_MAX) {
+                  if (xv > value)
+                     value = xv;
+               } else {
+                  value += xv;
+               }
             }
          }
       }
       if (d.mode == SOFIE_POOL_AVERAGE) {
-         int nsum = d.kh * d.kw;
+         int nsum = d.k[0] * d.k[1] * d.k[2];
          if (d.dynamic_divisor) {
-            const int hi_h = d.count_include_pad ? d.H + d.pad_h1 : d.H, hi_w = d.count_include_pad ? d.W + d.pad_w1 : d.W;
-            const int lo_h = d.count_include_pad ? i : (i > 0 ? i : 0), lo_w = d.count_include_pad ? j : (j > 0 ? j : 0);
-            nsum = ((i + d.kh < hi_h ? i + d.kh : hi_h) - lo_h) * ((j + d.kw < hi_w ? j + d.kw : hi_w) - lo_w);
+            const int start[3] = {i, j, k};
+            nsum = 1;
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+               const int hi = d.count_include_pad ? d.in[a] + d.pad_end[a] : d.in[a];
+               const int lo = d.count_include_pad ? start[a] : (start[a] > 0 ? start[a] : 0);
+               nsum *= (start[a] + d.k[a] < hi ? start[a] + d.k[a] : hi) - lo;
+            }
          }
          value = __fdiv_rn(value, (float)nsum);
       }
@@ -585,6 +598,30 @@ int sofie_hip_batchnorm_f32(sofie_hip_ctx *ctx, float *Y, const float *X, const 
    return launch_status("batchnorm_f32_kernel");
 }
 
+int sofie_hip_pool3d_f32(sofie_hip_ctx *ctx, const sofie_pool3d_desc *d, float *Y, const float *X)
+{
+   SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_pool3d_f32: NULL argument");
+   SOFIE_HIP_REQUIRE(d->planes >= 0, "sofie_hip_pool3d_f32: bad shape");
+   SOFIE_HIP_REQUIRE(d->mode == SOFIE_POOL_MAX || d->mode == SOFIE_POOL_AVERAGE, "sofie_hip_pool3d_f32: unknown mode %d", d->mode);
+   long long total = d->planes, in_total = d->planes;
+   for (int a = 0; a < 3; ++a) {
+      SOFIE_HIP_REQUIRE(d->in[a] > 0 && d->out[a] > 0 && d->k[a] > 0, "sofie_hip_pool3d_f32: bad shape");
+      SOFIE_HIP_REQUIRE(d->stride[a] > 0, "sofie_hip_pool3d_f32: bad stride");
+      SOFIE_HIP_REQUIRE(d->pad_begin[a] >= 0 && d->pad_end[a] >= 0, "sofie_hip_pool3d_f32: negative padding");
+      // every window start must lie where the reference's loops put it: the last one begins inside the padded volume
+      SOFIE_HIP_REQUIRE((long long)(d->out[a] - 1) * d->stride[a] - d->pad_begin[a] < d->in[a] + d->pad_end[a],
+                        "sofie_hip_pool3d_f32: the output extent %d of axis %d does not fit the padded input", d->out[a], a);
+      total *= d->out[a];
+      in_total *= d->in[a];
+      SOFIE_HIP_REQUIRE(total < (1LL << 40) && in_total < (1LL << 40), "sofie_hip_pool3d_f32: tensor too large");
+   }
+   if (total == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(Y && X, "sofie_hip_pool3d_f32: NULL pointer");
+   hipLaunchKernelGGL(pool_f32_kernel, dim3(grid_for((size_t)total)), dim3(256), 0, ctx->stream, Y, X, *d, (size_t)total);
+   return launch_status("pool_f32_kernel");
+}
+
 int sofie_hip_pool_f32(sofie_hip_ctx *ctx, const sofie_pool_desc *d, float *Y, const float *X)
 {
    SOFIE_HIP_REQUIRE(ctx && d, "sofie_hip_pool_f32: NULL argument");
@@ -596,13 +633,17 @@ int sofie_hip_pool_f32(sofie_hip_ctx *ctx, const sofie_pool_desc *d, float *Y, c
    SOFIE_HIP_REQUIRE((long long)(d->OH - 1) * d->stride_h - d->pad_h0 < d->H + d->pad_h1 &&
                         (long long)(d->OW - 1) * d->stride_w - d->pad_w0 < d->W + d->pad_w1,
                      "sofie_hip_pool_f32: the output shape %dx%d does not fit the padded input", d->OH, d->OW);
-   const long long total = (long long)d->planes * d->OH * d->OW;
-   SOFIE_HIP_REQUIRE(total < (1LL << 40) && (long long)d->planes * d->H * d->W < (1LL << 40), "sofie_hip_pool_f32: tensor too large");
-   if (total == 0)
-      return SOFIE_HIP_OK;
-   SOFIE_HIP_REQUIRE(Y && X, "sofie_hip_pool_f32: NULL pointer");
-   hipLaunchKernelGGL(pool_f32_kernel, dim3(grid_for((size_t)total)), dim3(256), 0, ctx->stream, Y, X, *d, (size_t)total);
-   return launch_status("pool_f32_kernel");
+   // a volume of depth one
+   sofie_pool3d_desc v{};
+   v.planes = d->planes;
+   v.in[0] = 1, v.in[1] = d->H, v.in[2] = d->W;
+   v.out[0] = 1, v.out[1] = d->OH, v.out[2] = d->OW;
+   v.k[0] = 1, v.k[1] = d->kh, v.k[2] = d->kw;
+   v.pad_begin[0] = 0, v.pad_begin[1] = d->pad_h0, v.pad_begin[2] = d->pad_w0;
+   v.pad_end[0] = 0, v.pad_end[1] = d->pad_h1, v.pad_end[2] = d->pad_w1;
+   v.stride[0] = 1, v.stride[1] = d->stride_h, v.stride[2] = d->stride_w;
+   v.mode = d->mode, v.count_include_pad = d->count_include_pad, v.dynamic_divisor = d->dynamic_divisor;
+   return sofie_hip_pool3d_f32(ctx, &v, Y, X);
 }
 
 int sofie_hip_global_avg_pool_f32(sofie_hip_ctx *ctx, float *Y, const float *X, int32_t NC, int32_t HW)

@@ -1,5 +1,5 @@
-// MaxPool, AveragePool and GlobalAveragePool over one or two spatial dimensions
-// (core/inc/SOFIE/operators/ROperator_Pool.hxx: attributes :17-26, shape inference :89-189, generated loops :286-412).
+// MaxPool, AveragePool and GlobalAveragePool over one, two or three spatial dimensions
+// (core/inc/SOFIE/operators/ROperator_Pool.hxx: attributes :17-26, shape inference :89-189, generated loops :286-475).
 // The operator resolves attributes to one window description per spatial axis and emits one runtime call; the runtime
 // kernel visits the window in the order of the reference's generated loops.
 #ifndef SOFIE_HIP_ROPERATOR_POOL
@@ -62,8 +62,8 @@ public:
          shapeY.resize(fShapeX.size(), 1);
       } else {
          const std::size_t nd = fShapeX.size() - 2;
-         if (nd > 2)
-            throw std::runtime_error("SOFIE " + Name() + " Op : this backend pools over 1 or 2 spatial dimensions, tensor " + fNX + " has " +
+         if (nd > 3)
+            throw std::runtime_error("SOFIE " + Name() + " Op : pooling over 1, 2 or 3 spatial dimensions, tensor " + fNX + " has " +
                                      std::to_string(nd));
          if (fAttr.storage_order != 0)
             throw std::runtime_error("SOFIE " + Name() + " Op : storage_order = 1 is not supported");
@@ -86,6 +86,24 @@ public:
             hw *= fShapeX[i];
          out << SP << "detail::Check(sofie_hip_global_avg_pool_f32(fCtx, tensor_" << fNY << ", tensor_" << fNX << ", " << planes << ", " << hw << "), \""
              << opName << " GlobalAveragePool\");\n";
+         return out.str();
+      }
+      // the divisor of an average follows the window over the border whenever there is padding or ceil_mode
+      // (ROperator_Pool.hxx:323-327)
+      bool dynamicDivisor3 = fAttr.ceil_mode != 0;
+      for (auto &a : fAxes)
+         dynamicDivisor3 |= a.padBegin > 0 || a.padEnd > 0;
+      if (fAxes.size() == 3) {
+         auto triple = [&](auto field) {
+            return "{" + std::to_string(field(fAxes[0])) + ", " + std::to_string(field(fAxes[1])) + ", " + std::to_string(field(fAxes[2])) + "}";
+         };
+         out << SP << "{\n";
+         out << SP << "   " << "sofie_pool3d_desc d{" << planes << ", " << triple([](const Axis &a) { return a.in; }) << ", " << triple([](const Axis &a) { return a.out; })
+             << ", " << triple([](const Axis &a) { return a.window; }) << ", " << triple([](const Axis &a) { return a.padBegin; }) << ", "
+             << triple([](const Axis &a) { return a.padEnd; }) << ", " << triple([](const Axis &a) { return a.stride; }) << ", "
+             << (fMode == MaxPool ? "SOFIE_POOL_MAX" : "SOFIE_POOL_AVERAGE") << ", " << (fAttr.count_include_pad ? 1 : 0) << ", " << (dynamicDivisor3 ? 1 : 0) << "};\n";
+         out << SP << "   " << "detail::Check(sofie_hip_pool3d_f32(fCtx, &d, tensor_" << fNY << ", tensor_" << fNX << "), \"" << opName << " " << Name() << "\");\n";
+         out << SP << "}\n";
          return out.str();
       }
       // 1-D pooling runs as a 2-D pooling over images of one row

@@ -80,6 +80,12 @@ class PoolDesc(C.Structure):
                                                "stride_h", "stride_w", "mode", "count_include_pad", "dynamic_divisor")]
 
 
+class Pool3dDesc(C.Structure):
+    _fields_ = [("planes", C.c_int32), ("in_", C.c_int32 * 3), ("out", C.c_int32 * 3), ("k", C.c_int32 * 3), ("pad_begin", C.c_int32 * 3),
+                ("pad_end", C.c_int32 * 3), ("stride", C.c_int32 * 3), ("mode", C.c_int32), ("count_include_pad", C.c_int32),
+                ("dynamic_divisor", C.c_int32)]
+
+
 POOL_MAX, POOL_AVERAGE = 0, 1
 REDUCE_SUM, REDUCE_MEAN, REDUCE_SUM_SQUARE, REDUCE_PROD, REDUCE_L2, REDUCE_MAX, REDUCE_MIN = range(7)
 BINARY_ADD, BINARY_SUB, BINARY_MUL, BINARY_DIV, BINARY_POW, BINARY_MAX, BINARY_MIN, BINARY_ADD_DIV = range(8)
@@ -137,6 +143,7 @@ SYMBOLS = {
     "sofie_hip_pack_conv_weight_i8": (C.c_int, [_P, C.POINTER(ConvDesc), _P, _P]),
     "sofie_hip_global_avg_pool_f32": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32]),
     "sofie_hip_pool_f32": (C.c_int, [_P, _P, _P, _P]),
+    "sofie_hip_pool3d_f32": (C.c_int, [_P, _P, _P, _P]),
     "sofie_hip_reduce_f32": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, C.c_int64, C.c_int32]),
     "sofie_hip_layernorm_f32": (C.c_int, [_P, _P, _P, _P, _P, C.c_int64, C.c_int32, C.c_float, _P, _P]),
     "sofie_hip_transpose_f32": (C.c_int, [_P, _P, _P, C.c_int32, _P, _P]),

@@ -132,7 +132,7 @@ def main():
         add(model, next(iter(arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx")).values())),
             [{"kind": "values", "values": vector_literal(un, model, "input")}])
     pool = os.path.join(REF, "alpaka/TestAlpakaPool.cxx")
-    for model in ("MaxPool1d", "MaxPool2d", "AvgPool"):
+    for model in ("MaxPool1d", "MaxPool2d", "MaxPool3d", "AvgPool"):
         add(model, arrays_in(os.path.join(REF, "models/onnx/references", model + ".ref.hxx"))["output"],
             [{"kind": "values", "values": vector_literal(pool, model, "input")}])
     norm = os.path.join(REF, "alpaka/TestAlpakaNormalization.cxx")

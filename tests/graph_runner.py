@@ -384,10 +384,21 @@ class HipBackend:
 
 
 def hip_pool(rt, X, mode, axes, ceil_mode=0, count_include_pad=0):
-    """sofie_hip_pool_f32 on an [N, C, (H,) W] array; axes = per spatial axis (in, out, window, stride, pad_begin, pad_end)."""
+    """sofie_hip_pool_f32 on an [N, C, (H,) W] array, sofie_hip_pool3d_f32 on [N, C, D, H, W]; axes = per spatial axis (in, out, window, stride, pad_begin, pad_end)."""
     import torch
     from sofie_amd import runtime as R
     from tests import util as u
+    if len(axes) == 3:
+        col = lambda c: (C.c_int32 * 3)(*[a[c] for a in axes])
+        d = R.Pool3dDesc(planes=X.shape[0] * X.shape[1], in_=col(0), out=col(1), k=col(2), stride=col(3), pad_begin=col(4), pad_end=col(5),
+                         mode=R.POOL_MAX if mode == "max" else R.POOL_AVERAGE, count_include_pad=int(count_include_pad),
+                         dynamic_divisor=int(bool(ceil_mode) or any(a[4] > 0 or a[5] > 0 for a in axes)))
+        dX = u.to_dev(np.ascontiguousarray(X, dtype=np.float32))
+        dY = u.dev_empty(X.shape[:2] + tuple(a[1] for a in axes), np.float32)
+        torch.cuda.synchronize()
+        rt.call("sofie_hip_pool3d_f32", C.byref(d), u.ptr(dY), u.ptr(dX))
+        rt.sync()
+        return u.to_host(dY)
     if len(axes) == 1:
         axes = [(1, 1, 1, 1, 0, 0)] + list(axes)
     (H, OH, kh, sh, ph0, ph1), (W, OW, kw, sw, pw0, pw1) = axes

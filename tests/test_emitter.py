@@ -530,8 +530,11 @@ def test_pool_attributes_resolve_to_the_reference_shapes(emitted, tmp_path):
     assert "d.count_include_pad = 1; d.dynamic_divisor = 1;" in txt and "d.planes = 6;" in txt
     r, txt = emit_pool("AveragePool", [2, 3, 8, 8], "plain", kernel_shape=[2, 2], strides=[2, 2])
     assert r.returncode == 0 and "d.dynamic_divisor = 0;" in txt
+    # three spatial axes are one call with the axes slowest first: {in}, {out}, {window}, {pad begin}, {pad end}, {stride}
+    r, txt = emit_pool("MaxPool", [1, 2, 4, 5, 6], "three_d", kernel_shape=[2, 2, 3], strides=[2, 1, 3], pads=[0, 1, 0, 0, 0, 0])
+    assert r.returncode == 0 and "sofie_pool3d_desc d{2, {4, 5, 6}, {2, 5, 2}, {2, 2, 3}, {0, 1, 0}, {0, 0, 0}, {2, 1, 3}, SOFIE_POOL_MAX, 0, 1};" in txt
     # refusals name the operator
-    r, _ = emit_pool("MaxPool", [1, 1, 4, 4, 4], "three_d", kernel_shape=[2, 2, 2])
+    r, _ = emit_pool("MaxPool", [1, 1, 4, 4, 4, 4], "four_d", kernel_shape=[2, 2, 2, 2])
     assert r.returncode != 0 and "MaxPool" in r.stdout and "spatial" in r.stdout
     r, _ = emit_pool("MaxPool", [1, 1, 4, 4], "column_major", kernel_shape=[2, 2], storage_order=1)
     assert r.returncode != 0 and "storage_order" in r.stdout

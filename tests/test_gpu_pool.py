@@ -49,6 +49,23 @@ def test_pool_auto_pad_and_one_dimension(rt, mode, auto_pad):
     assert same_bits(got, want)
 
 
+@pytest.mark.parametrize("mode", ["max", "average"])
+def test_pool_over_three_axes_is_bit_exact(rt, mode):
+    """Volumes [N, C, D, H, W]: every axis with its own extent, window, stride and padding, both divisor conventions, ceil_mode."""
+    rng = np.random.default_rng(23)
+    for case in range(40):
+        sp = [int(v) for v in rng.integers(2, 11, 3)]
+        k = [int(min(v, n)) for v, n in zip(rng.integers(1, 4, 3), sp)]
+        st = [int(v) for v in rng.integers(1, 4, 3)]
+        pads = [int(min(p, kk - 1)) for p, kk in zip(rng.integers(0, 3, 6), k + k)]
+        X = rng.standard_normal((int(rng.integers(1, 3)), int(rng.integers(1, 5)), *sp)).astype(np.float32)
+        got, want = both(rt, X, mode, k, pads, st, None, "NOTSET", case % 2, (case // 2) % 2)
+        assert same_bits(got, want), case
+    X = util.normal(9104, 2 * 8 * 16 * 40 * 40).reshape(2, 8, 16, 40, 40)
+    got, want = both(rt, X, mode, [2, 3, 3], [0, 1, 1, 0, 1, 1], [2, 2, 2])
+    assert got.shape == (2, 8, 8, 20, 20) and same_bits(got, want)
+
+
 def test_pool_at_the_size_of_a_network_stem(rt):
     """64 x 64 planes of 112 x 112 -> MaxPool 3x3 / 2 / pad 1 -> 56 x 56: more outputs than one pass of the grid covers."""
     X = util.normal(9103, 64 * 64 * 112 * 112).reshape(64, 64, 112, 112)

@@ -556,6 +556,30 @@ def test_pool_against_the_library_routine():
     np.testing.assert_array_equal(ob.pool(X1, "max", [3], None, [2]), F.max_pool1d(torch.from_numpy(X1), 3, 2).numpy())
 
 
+def test_pool3d_against_the_library_routine_and_the_2d_operator():
+    """Three spatial axes: torch's pooling as the independent implementation (floor mode), every axis with its own extent, window,
+    stride and padding; a volume of depth one must give the 2-D operator's bits; the reference's MaxPool3d shape."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(13)
+    X = rng.standard_normal((2, 3, 7, 9, 8)).astype(np.float32)
+    t = torch.from_numpy(X)
+    np.testing.assert_array_equal(ob.pool(X, "max", [3, 2, 4], [1, 0, 2, 1, 0, 2], [2, 1, 3]), F.max_pool3d(t, (3, 2, 4), (2, 1, 3), (1, 0, 2)).numpy())
+    for include in (0, 1):
+        want = F.avg_pool3d(t, (3, 2, 2), (2, 1, 2), (1, 1, 0), count_include_pad=bool(include)).numpy()
+        np.testing.assert_allclose(ob.pool(X, "average", [3, 2, 2], [1, 1, 0, 1, 1, 0], [2, 1, 2], count_include_pad=include), want, rtol=2e-6, atol=2e-6)
+    want = F.max_pool3d(t, (2, 3, 2), (2, 2, 3), (0, 1, 0), ceil_mode=True).numpy()
+    np.testing.assert_array_equal(ob.pool(X, "max", [2, 3, 2], [0, 1, 0, 0, 1, 0], [2, 2, 3], ceil_mode=1), want)
+    X2 = rng.standard_normal((2, 3, 6, 10)).astype(np.float32)
+    for mode in ("max", "average"):
+        flat = ob.pool(X2, mode, [3, 2], [1, 0, 0, 1], [2, 3], count_include_pad=1)
+        deep = ob.pool(X2[:, :, None], mode, [1, 3, 2], [0, 1, 0, 0, 0, 1], [1, 2, 3], count_include_pad=1)
+        assert np.array_equal(deep[:, :, 0].view(np.uint32), flat.view(np.uint32))
+    X3 = np.arange(27, dtype=np.float32).reshape(1, 1, 3, 3, 3)
+    assert ob.pool(X3, "max", [2, 2, 2], None, [1, 1, 1]).shape == (1, 1, 2, 2, 2)
+    np.testing.assert_array_equal(ob.pool(X3, "average", [3, 3, 3]).ravel(), [13.0])
+
+
 def test_pool_special_cases():
     X = np.arange(2 * 3 * 4 * 5, dtype=np.float32).reshape(2, 3, 4, 5)
     # a window that is the image is GlobalAveragePool; a 1x1 window with stride 1 is the identity
