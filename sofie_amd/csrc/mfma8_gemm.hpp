@@ -44,8 +44,9 @@ constexpr size_t mfma8_general_lds_bytes()
    return ring > store ? ring : store;
 }
 
-template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool ALIGNED, class EPI, class ASRC = RowMajorRows>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mfma8_gemm_kernel(ASRC A, RowMajorRows Bt, int M, int N,
+// OCC: waves per SIMD the register allocation leaves room for.
+template <class MMA, int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool ALIGNED, class EPI, class ASRC = RowMajorRows, int OCC = 1>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64, OCC) void mfma8_gemm_kernel(ASRC A, RowMajorRows Bt, int M, int N,
                                                                             int K, EPI ep, int tiles_m, int tiles_n, int sw)
 {
    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
@@ -262,7 +263,10 @@ static int launch_mfma8_gather_kp(const LaunchCfg &lc, const GatherConvRows &a, 
    if (nwg > 0x7fffffffLL)
       return fail(SOFIE_HIP_ERR_INVALID, "conv: too many tiles");
    constexpr size_t smem = mfma8_general_lds_bytes<BM, BN, BK, 4, 1>();
-   auto kern = mfma8_gemm_kernel<MfmaI8, BM, BN, BK, 4, 1, true, EPI, GatherConvRowsT<KP>>;
+   // three waves per SIMD (at most 170 registers; the kernel needs 168): each workgroup is one chain of memory round trips
+   // (gather, weights, store), so the time goes down with the number of workgroups a CU holds (first layer of the benchmark CNN:
+   // 74 us with two, 59 us with three; four would spill)
+   auto kern = mfma8_gemm_kernel<MfmaI8, BM, BN, BK, 4, 1, true, EPI, GatherConvRowsT<KP>, 3>;
    static bool configured[64] = {};
    if (int st = configure_lds_once(kern, smem, configured))
       return st;
