@@ -103,6 +103,12 @@ struct F8Epilogue {
       default: f(std::integral_constant<int, 7>{}); break;
       }
    }
+   // the name the pipelined kernel calls (the int8 store has one more mode there)
+   template <class F>
+   __device__ __forceinline__ void dispatch_with_reciprocal(F f) const
+   {
+      dispatch(f);
+   }
    template <int MODE>
    static constexpr int out_bytes()
    {

@@ -26,7 +26,9 @@ __global__ __launch_bounds__(256) void transpose_i8_kernel(int8_t *__restrict__ 
 }
 
 
-int gemm_i8_nt(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep)
+// The fields of the epilogue that follow from the others: what the stores may assume about alignment, and whether the
+// quotient of SOFIE_I8OUT_I8_DQQ may be formed from the reciprocal (a per-tensor scale known here, in a safe range).
+static void derive_epilogue_fields(I8Epilogue &ep, int N)
 {
    const size_t esz = ep.out == SOFIE_I8OUT_I32 || ep.out == SOFIE_I8OUT_F32 ? 4 : 1;
    ep.N = N;
@@ -34,28 +36,25 @@ int gemm_i8_nt(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, in
                  (((uintptr_t)ep.Y & 15) == 0);
    ep.vec_param = (ep.n_offset % 4 == 0) && (!ep.bias || ((uintptr_t)ep.bias & 15) == 0) &&
                   (!ep.scale || ((uintptr_t)ep.scale & 15) == 0);
+   ep.q_rcp = 0.0f;
+   ep.q_by_rcp = ep.out == SOFIE_I8OUT_I8_DQQ && !ep.scale && quotient_plan(ep.scale_scalar, ep.q_scale, ep.q_rcp);
+}
+
+int gemm_i8_nt(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep)
+{
+   derive_epilogue_fields(ep, N);
    return launch_mfma8_best<MfmaI8, I8Epilogue>(lc, A, Bt, M, N, K, lda, ldb, ep);
 }
 
 int conv_i8_implicit(const LaunchCfg &lc, const ConvRows &src, int Cg, const int8_t *Wp, int M, int N, int K, I8Epilogue ep)
 {
-   const size_t esz = ep.out == SOFIE_I8OUT_I32 || ep.out == SOFIE_I8OUT_F32 ? 4 : 1;
-   ep.N = N;
-   ep.stage_ok = (ep.nchw_ohw == 0) && (((size_t)ep.ldy * esz) % 16 == 0) && (((size_t)ep.n_offset * esz) % 16 == 0) &&
-                 (((uintptr_t)ep.Y & 15) == 0);
-   ep.vec_param = (ep.n_offset % 4 == 0) && (!ep.bias || ((uintptr_t)ep.bias & 15) == 0) &&
-                  (!ep.scale || ((uintptr_t)ep.scale & 15) == 0);
+   derive_epilogue_fields(ep, N);
    return launch_mfma8_conv<I8Epilogue>(lc, src, Cg, Wp, M, N, K, ep);
 }
 
 int conv_i8_gather(const LaunchCfg &lc, const GatherConvRows &src, const int8_t *Wp, int M, int N, int Kp, I8Epilogue ep)
 {
-   const size_t esz = ep.out == SOFIE_I8OUT_I32 || ep.out == SOFIE_I8OUT_F32 ? 4 : 1;
-   ep.N = N;
-   ep.stage_ok = (ep.nchw_ohw == 0) && (((size_t)ep.ldy * esz) % 16 == 0) && (((size_t)ep.n_offset * esz) % 16 == 0) &&
-                 (((uintptr_t)ep.Y & 15) == 0);
-   ep.vec_param = (ep.n_offset % 4 == 0) && (!ep.bias || ((uintptr_t)ep.bias & 15) == 0) &&
-                  (!ep.scale || ((uintptr_t)ep.scale & 15) == 0);
+   derive_epilogue_fields(ep, N);
    return launch_mfma8_gather<I8Epilogue>(lc, src, Wp, M, N, Kp, ep);
 }
 

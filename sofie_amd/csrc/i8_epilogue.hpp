@@ -2,6 +2,7 @@
 // optional relu, and the output addressing (row-major [M,N], or NCHW when the GEMM rows are the
 // output pixels of a convolution).  Plugs into tile_store_via_lds (mfma8_common.hpp).
 #pragma once
+#include "exact_quotient.hpp"
 #include "mfma8_dispatch.hpp"
 
 namespace sofie_hip {
@@ -22,6 +23,8 @@ struct I8Epilogue {
    int n_offset;  // added to n for bias/scale/Y addressing (grouped convolution)
    int rows_per_plane = 0; // non-zero (with out = SOFIE_I8OUT_I8): the int8 values of the rows of a plane are added up instead of stored;
                        // Y is int32 [M / rows_per_plane][ldy]
+   float q_rcp = 0.0f;     // RN(1 / q_scale) when q_by_rcp is set
+   int q_by_rcp = 0;       // SOFIE_I8OUT_I8_DQQ: the quotient is formed with quotient_by_reciprocal (same bits as the division)
 
    template <class F>
    __device__ __forceinline__ void dispatch(F f) const
@@ -32,6 +35,31 @@ struct I8Epilogue {
       case SOFIE_I8OUT_I8: f(std::integral_constant<int, SOFIE_I8OUT_I8>{}); break;
       default: f(std::integral_constant<int, SOFIE_I8OUT_I8_DQQ>{}); break;
       }
+   }
+   // The same with a fifth store for SOFIE_I8OUT_I8_DQQ whose quotient may come from the reciprocal.  Only the kernels with
+   // registers to spare for one more instance of the store take it (the 256 x 256 tiles have none).
+   template <class F>
+   __device__ __forceinline__ void dispatch_with_reciprocal(F f) const
+   {
+      if (out == SOFIE_I8OUT_I8_DQQ && q_by_rcp)
+         f(std::integral_constant<int, kOutDqqByRcp>{});
+      else
+         dispatch(f);
+   }
+   // SOFIE_I8OUT_I8_DQQ with the quotient taken through the reciprocal: a store mode of the kernels only
+   static constexpr int kOutDqqByRcp = 5;
+   template <int OUT>
+   static constexpr bool divides()
+   {
+      return OUT == SOFIE_I8OUT_I8_DQQ || OUT == kOutDqqByRcp;
+   }
+   // (float(acc) * s) / q_scale, correctly rounded
+   template <int OUT>
+   __device__ __forceinline__ float quotient(float v) const
+   {
+      if (OUT == kOutDqqByRcp)
+         return quotient_by_reciprocal(v, q_scale, q_rcp);
+      return __fdiv_rn(v, q_scale);
    }
    template <int OUT>
    static constexpr int out_bytes()
@@ -82,7 +110,7 @@ struct I8Epilogue {
    {
       if (OUT == SOFIE_I8OUT_I8)
          return quantize_rne_clamp(mul_nofma((float)acc, s), relu_out ? 0 : -128);
-      return quantize_rne_clamp(__fdiv_rn(mul_nofma((float)acc, s), q_scale), -128);
+      return quantize_rne_clamp(quotient<OUT>(mul_nofma((float)acc, s)), -128);
    }
 
    // bias and scale of C consecutive columns
@@ -141,8 +169,8 @@ struct I8Epilogue {
          acc[i] += p.b[4 * q + i];
          acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
          float v = mul_nofma((float)acc[i], p.s[4 * q + i]);
-         if (OUT == SOFIE_I8OUT_I8_DQQ)
-            v = __fdiv_rn(v, q_scale);
+         if (divides<OUT>())
+            v = quotient<OUT>(v);
          r[i] = (int)i8_bits(v, (OUT == SOFIE_I8OUT_I8 && relu_out) ? 0.0f : -128.0f) - 0x4B400000; // needs the tamed scale, like pack4_short
       }
    }
@@ -163,7 +191,7 @@ struct I8Epilogue {
    template <int OUT, int C>
    __device__ __forceinline__ void pack4_short(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, uint32_t *w) const
    {
-      static_assert(OUT == SOFIE_I8OUT_I8 || OUT == SOFIE_I8OUT_I8_DQQ, "1-byte outputs");
+      static_assert(OUT == SOFIE_I8OUT_I8 || divides<OUT>(), "1-byte outputs");
       int acc[4] = {a0, a1, a2, a3};
       uint32_t b[4];
       const int acc_floor = relu_acc ? 0 : (int)0x80000000;
@@ -173,8 +201,8 @@ struct I8Epilogue {
          acc[i] += p.b[4 * q + i];
          acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
          float v = mul_nofma((float)acc[i], p.s[4 * q + i]);
-         if (OUT == SOFIE_I8OUT_I8_DQQ)
-            v = __fdiv_rn(v, q_scale);
+         if (divides<OUT>())
+            v = quotient<OUT>(v);
          b[i] = i8_bits(v, lo);
       }
       const uint32_t lo2 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);

@@ -186,7 +186,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, OCC) void mfma8_gemm_dma_ker
    wait_vmcnt<0>();
    __syncthreads();
    char *wsm = (char *)smem + wave * tile_store_lds_bytes(TN);
-   ep.dispatch([&](auto mode) {
+   ep.dispatch_with_reciprocal([&](auto mode) {
       tile_store_via_lds<decltype(mode)::value, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, M, N, lane, wsm);
    });
 }

@@ -89,6 +89,30 @@ def test_fused_epilogues_bit_exact(rt, out, relu_acc, relu_out, M, N, K):
         assert got.min() <= (0 if relu_out else -100) and got.max() >= 100  # the data really spans the int8 range
 
 
+def _f32_from_bits(b):
+    return np.array([b], dtype=np.uint32).view(np.float32)[0]
+
+
+@pytest.mark.parametrize("q", [3.0, 0.037, 0.601829112, 16.3691254, -7.25, float(_f32_from_bits(0x3fffffff)), 2.0 ** -31])
+@pytest.mark.parametrize("M,N,K", [(256, 384, 512), (200, 136, 512), (64, 50, 1000)])
+def test_dequantize_quantize_with_a_per_tensor_scale(rt, q, M, N, K):
+    """With a per-tensor scale the runtime may form the quotient of SOFIE_I8OUT_I8_DQQ from the reciprocal of q_scale; the
+    last two divisors (significand all ones, out of range) keep the division.  Either way the bytes are those of
+    sat8(rne(fl(fl(acc * s) / q))) in IEEE fp32, here from numpy's division.  s = q / 2 puts every odd accumulator on a tie."""
+    A = util.int8_sym(51, M * K).reshape(M, K)
+    Bt = util.int8_sym(52, N * K).reshape(N, K)
+    acc = ob.matmul_integer(A, Bt, M=M, N=N, K=K, transB=1)
+    q = np.float32(q)
+    spread = np.float32(np.abs(acc).max())
+    for s in (np.float32(abs(q) * 127.0 / spread), np.float32(abs(q) * 300.0 / spread), np.float32(abs(q) / 2)):
+        got = run_gemm(rt, A, Bt, M, N, K, transB=1, scale_scalar=s, q_scale=q, out=R.I8OUT_I8_DQQ)
+        v = (acc.astype(np.float32) * s).astype(np.float32)
+        want = np.clip(np.rint((v / q).astype(np.float32)), -128, 127).astype(np.int8)
+        assert np.array_equal(got, want), (float(q), float(s))
+        assert np.array_equal(got, ob.gemm_i8(A, Bt, M=M, N=N, K=K, transB=1, scale_scalar=s, q_scale=q, out=R.I8OUT_I8_DQQ))
+    assert got.min() == -128 and got.max() == 127
+
+
 def test_per_tensor_scale_and_odd_leading_dimensions(rt):
     M, N, K = 70, 90, 160
     lda, ldb, ldy = 176, 192, 101
