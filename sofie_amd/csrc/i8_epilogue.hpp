@@ -110,6 +110,8 @@ struct I8Epilogue {
    {
       if (OUT == SOFIE_I8OUT_I8)
          return quantize_rne_clamp(mul_nofma((float)acc, s), relu_out ? 0 : -128);
+      if (OUT == kOutDqqByRcp) // a finite per-tensor scale (the condition of this mode): no NaN to keep out of the short conversion
+         return (int)i8_bits(quotient<OUT>(mul_nofma((float)acc, s)), -128.0f);
       return quantize_rne_clamp(quotient<OUT>(mul_nofma((float)acc, s)), -128);
    }
 
@@ -226,7 +228,8 @@ struct I8Epilogue {
    {
       int acc[4] = {a0, a1, a2, a3};
       float s[4];
-      const int acc_floor = relu_acc ? 0 : (int)0x80000000; // relu on the accumulator as one max
+      int acc_floor = relu_acc ? 0 : (int)0x80000000; // relu on the accumulator as one max
+      asm volatile("" : "+s"(acc_floor));              // kept a number: as a known pair of cases it becomes a max AND a select per element
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
          acc[i] += p.b[4 * q + i];
