@@ -165,7 +165,8 @@ struct I8Epilogue {
    __device__ __forceinline__ void quantize4(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, int (&r)[4]) const
    {
       int acc[4] = {a0, a1, a2, a3};
-      const int acc_floor = relu_acc ? 0 : (int)0x80000000;
+      int acc_floor = relu_acc ? 0 : (int)0x80000000;
+      asm volatile("" : "+s"(acc_floor)); // kept a number (see pack4)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
          acc[i] += p.b[4 * q + i];
@@ -196,7 +197,8 @@ struct I8Epilogue {
       static_assert(OUT == SOFIE_I8OUT_I8 || divides<OUT>(), "1-byte outputs");
       int acc[4] = {a0, a1, a2, a3};
       uint32_t b[4];
-      const int acc_floor = relu_acc ? 0 : (int)0x80000000;
+      int acc_floor = relu_acc ? 0 : (int)0x80000000;
+      asm volatile("" : "+s"(acc_floor)); // kept a number (see pack4)
       const float lo = (OUT == SOFIE_I8OUT_I8 && relu_out) ? 0.0f : -128.0f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
