@@ -234,16 +234,12 @@ struct ConvRows {
          const int ow = r - oh * OW;
          const int ih0 = oh * stride_h - pad_h0, iw0 = ow * stride_w - pad_w0;
          off = ((n * H + ih0) * W + iw0) * C + cbyte;
-         int khi = 0, kwi = 0; // tap t = khi * kw + kwi, stepped without dividing
-         for (int t = 0; t < ntaps; ++t) {
-            const int ih = ih0 + khi * dil_h, iw = iw0 + kwi * dil_w;
-            if ((unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W)
-               mask |= 1u << t;
-            if (++kwi == kw) {
-               kwi = 0;
-               ++khi;
-            }
-         }
+         // tap t = khi * kw + kwi lies inside when its row and its column do: one pass over the columns, one over the rows
+         uint32_t cols = 0;
+         for (int kwi = 0, iw = iw0; kwi < kw; ++kwi, iw += dil_w)
+            cols |= ((unsigned)iw < (unsigned)W ? 1u : 0u) << kwi;
+         for (int t0 = 0, ih = ih0; t0 < ntaps; t0 += kw, ih += dil_h)
+            mask |= ((unsigned)ih < (unsigned)H ? cols : 0u) << t0;
       }
       st.off[i] = off;
       st.mask[i] = mask;

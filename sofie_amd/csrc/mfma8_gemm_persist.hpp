@@ -324,9 +324,7 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const i
       m0 = tm * BM;
       n0 = tn * BN;
    };
-   auto load_origin = [&](int it, typename ASRC::tile_state &ta, const int8_t *&pb) {
-      int m0, n0;
-      tile_origin(it, m0, n0);
+   auto load_origin = [&](int m0, int n0, typename ASRC::tile_state &ta, const int8_t *&pb) {
       if constexpr (ASRC::kConv) {
          // what the source keeps per lane is only needed here, once per tile: worked out again from the lane number (made
          // opaque, so that it is not kept in registers across the K loop instead)
@@ -343,8 +341,12 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const i
    int l_kp = 0; // pair (of the tile being loaded) the next loads fetch
    typename ASRC::tile_state l_a, n_a;
    const int8_t *l_b, *n_b;
-   load_origin(0, l_a, l_b);
-   load_origin(1, n_a, n_b);
+   // origins of the tile in work and of the one after it (the tile order costs a few integer divisions: once per tile)
+   int m_cur, n_cur, m_nxt, n_nxt;
+   tile_origin(0, m_cur, n_cur);
+   tile_origin(1, m_nxt, n_nxt);
+   load_origin(m_cur, n_cur, l_a, l_b);
+   load_origin(m_nxt, n_nxt, n_a, n_b);
    // load q (0..7) of the pair: operand q/4, wave instruction (q/2)%2, half q%2 of the 128-byte line
    auto issue_load = [&](int slot0, int slot1, auto q_c) {
       constexpr int q = decltype(q_c)::value;
@@ -382,11 +384,7 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const i
    };
 
    uint32_t col_words[EPI::kColWords]; // the epilogue's constants of column n0 + wn*TN + lane of the tile in work
-   {
-      int m0, n0;
-      tile_origin(0, m0, n0);
-      ep.load_column_tamed(n0 + wn * TN + lane, col_words);
-   }
+   ep.load_column_tamed(n_cur + wn * TN + lane, col_words);
    acc_t acc[MT][NT];
    auto zero_acc = [&]() {
 #pragma unroll
@@ -465,17 +463,19 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const i
          rslot = (rslot + 1 == STAGES) ? 0 : rslot + 1;
          lslot = (lslot + 2 >= STAGES) ? lslot + 2 - STAGES : lslot + 2;
       }
-      // the loads have moved on to tile it + 1 (K spans at least three pairs): the tile after that is it + 2
-      load_origin(it + 2, n_a, n_b);
-      int m0, n0;
-      tile_origin(it, m0, n0);
       ep.dispatch([&](auto mode) {
-         tile_store_or_sum_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, m0 + wm * TM, n0 + wn * TN, lane, col_words);
+         tile_store_or_sum_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, m_cur + wm * TM, n_cur + wn * TN, lane, col_words);
       });
       zero_acc();
+      // The loads have moved on to tile it + 1 (K spans at least three pairs): the tile after that is it + 2.  Its lane
+      // state is worked out here, behind the stores, whose acknowledgements are still on their way.
+      int m2, n2;
+      tile_origin(it + 2, m2, n2);
+      load_origin(m2, n2, n_a, n_b);
       // the column constants of the next tile: fetched now, used after its K loop
-      tile_origin(it + 1, m0, n0);
-      ep.load_column_tamed(n0 + wn * TN + lane, col_words);
+      ep.load_column_tamed(n_nxt + wn * TN + lane, col_words);
+      m_cur = m_nxt, n_cur = n_nxt;
+      m_nxt = m2, n_nxt = n2;
    }
    wait_vmcnt<0>();
 }
