@@ -103,7 +103,12 @@ struct F8Epilogue {
       default: f(std::integral_constant<int, 7>{}); break;
       }
    }
-   // the name the pipelined kernel calls (the int8 store has one more mode there)
+   // the names the pipelined and the persistent kernel call (the int8 store has one more mode in each)
+   template <class F>
+   __device__ __forceinline__ void dispatch_for_registers(F f) const
+   {
+      dispatch(f);
+   }
    template <class F>
    __device__ __forceinline__ void dispatch_with_reciprocal(F f) const
    {

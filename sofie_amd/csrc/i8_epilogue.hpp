@@ -46,8 +46,24 @@ struct I8Epilogue {
       else
          dispatch(f);
    }
-   // SOFIE_I8OUT_I8_DQQ with the quotient taken through the reciprocal: a store mode of the kernels only
-   static constexpr int kOutDqqByRcp = 5;
+   // The store from registers (the 256 x 256 tile of the persistent kernel, where every instruction per element counts) has
+   // SOFIE_I8OUT_I8 twice: with the relu on the accumulator and, kOutI8NoFloor, without that instruction.
+   template <class F>
+   __device__ __forceinline__ void dispatch_for_registers(F f) const
+   {
+      if (out == SOFIE_I8OUT_I8 && !relu_acc)
+         f(std::integral_constant<int, kOutI8NoFloor>{});
+      else
+         dispatch(f);
+   }
+   // store modes of the kernels only: SOFIE_I8OUT_I8_DQQ with the quotient taken through the reciprocal, SOFIE_I8OUT_I8
+   // without a relu on the accumulator
+   static constexpr int kOutDqqByRcp = 5, kOutI8NoFloor = 6;
+   template <int OUT>
+   static constexpr bool requantizes()
+   {
+      return OUT == SOFIE_I8OUT_I8 || OUT == kOutI8NoFloor;
+   }
    template <int OUT>
    static constexpr bool divides()
    {
@@ -170,11 +186,12 @@ struct I8Epilogue {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
          acc[i] += p.b[4 * q + i];
-         acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
+         if (OUT != kOutI8NoFloor)
+            acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
          float v = mul_nofma((float)acc[i], p.s[4 * q + i]);
          if (divides<OUT>())
             v = quotient<OUT>(v);
-         r[i] = (int)i8_bits(v, (OUT == SOFIE_I8OUT_I8 && relu_out) ? 0.0f : -128.0f) - 0x4B400000; // needs the tamed scale, like pack4_short
+         r[i] = (int)i8_bits(v, (requantizes<OUT>() && relu_out) ? 0.0f : -128.0f) - 0x4B400000; // needs the tamed scale, like pack4_short
       }
    }
 
@@ -194,16 +211,17 @@ struct I8Epilogue {
    template <int OUT, int C>
    __device__ __forceinline__ void pack4_short(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, uint32_t *w) const
    {
-      static_assert(OUT == SOFIE_I8OUT_I8 || divides<OUT>(), "1-byte outputs");
+      static_assert(requantizes<OUT>() || divides<OUT>(), "1-byte outputs");
       int acc[4] = {a0, a1, a2, a3};
       uint32_t b[4];
       int acc_floor = relu_acc ? 0 : (int)0x80000000;
       asm volatile("" : "+s"(acc_floor)); // kept a number (see pack4)
-      const float lo = (OUT == SOFIE_I8OUT_I8 && relu_out) ? 0.0f : -128.0f;
+      const float lo = (requantizes<OUT>() && relu_out) ? 0.0f : -128.0f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
          acc[i] += p.b[4 * q + i];
-         acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
+         if (OUT != kOutI8NoFloor)
+            acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
          float v = mul_nofma((float)acc[i], p.s[4 * q + i]);
          if (divides<OUT>())
             v = quotient<OUT>(v);

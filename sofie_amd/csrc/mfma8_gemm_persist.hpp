@@ -463,7 +463,7 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const i
          rslot = (rslot + 1 == STAGES) ? 0 : rslot + 1;
          lslot = (lslot + 2 >= STAGES) ? lslot + 2 - STAGES : lslot + 2;
       }
-      ep.dispatch([&](auto mode) {
+      ep.dispatch_for_registers([&](auto mode) {
          tile_store_or_sum_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, m_cur + wm * TM, n_cur + wn * TN, lane, col_words);
       });
       zero_acc();
