@@ -53,26 +53,26 @@ __global__ __launch_bounds__(256) void quantize_fp8_kernel(uint8_t *__restrict__
       dst[i] = f32_to_e4m3_rne_sat(__fdiv_rn(src[i], scale));
 }
 
-// GELU (erf form) for the FP8 store: erf by the rational approximation 7.1.26 of Abramowitz & Stegun,
-//   erf(z) = 1 - (a1 t + ... + a5 t^5) exp(-z^2),  t = 1/(1 + p z),  z >= 0,   |error| <= 1.5e-7,
-// one exponential and one reciprocal per element instead of the library erff (the tile store of a
-// 256 x 256 tile evaluates it 256 times per lane, which with erff costs half as much as the whole K loop).
-// The reciprocal is the hardware's (v_rcp_f32, one ulp): the correctly rounded one is a division sequence of ten
-// instructions, a third of this function.  The absolute error of the result, <= 3e-7 |v|, is far inside the FP8 GEMM's
-// stated bound.
+// GELU (erf form) for the FP8 store, v Phi(v) with Phi from the rational approximation 7.1.26 of Abramowitz & Stegun,
+//   erfc(z) = (a1 t + ... + a5 t^5) exp(-z^2),  t = 1/(1 + p z),  z = |v| / sqrt 2 >= 0,   |error| <= 1.5e-7,
+// one exponential and one reciprocal per element instead of the library erff (the tile store of a 256 x 256 tile evaluates
+// it 256 times per lane, which with erff costs half as much as the whole K loop).  Written in v directly: the factor 1/2 of
+// Phi(-|v|) = erfc(z) / 2 sits in the coefficients, p / sqrt 2 in the reciprocal's argument, and exp(-z^2) is
+// 2^-(v sqrt(log2(e) / 2))^2, the hardware's own exponential.  The reciprocal is the hardware's too (v_rcp_f32, one ulp): the
+// correctly rounded one is a division sequence of ten instructions.  Sixteen plain instructions and the two transcendental
+// ones; the absolute error of the result, <= 5e-7 |v|, is far inside the FP8 GEMM's stated bound.
 __device__ __forceinline__ float gelu_erf_fast(float v)
 {
-   const float z = __fmul_rn(v, 0.7071067811865475f);
-   const float az = fabsf(z);
-   const float t = __builtin_amdgcn_rcpf(__fmaf_rn(0.3275911f, az, 1.0f));
-   float poly = __fmaf_rn(t, 1.061405429f, -1.453152027f);
-   poly = __fmaf_rn(t, poly, 1.421413741f);
-   poly = __fmaf_rn(t, poly, -0.284496736f);
-   poly = __fmaf_rn(t, poly, 0.254829592f);
+   const float t = __builtin_amdgcn_rcpf(__fmaf_rn(0.23164189f, fabsf(v), 1.0f));
+   float poly = __fmaf_rn(t, 0.5306527145f, -0.7265760135f);
+   poly = __fmaf_rn(t, poly, 0.7107068705f);
+   poly = __fmaf_rn(t, poly, -0.142248368f);
+   poly = __fmaf_rn(t, poly, 0.127414796f);
    poly = __fmul_rn(poly, t);
-   const float q = __fmul_rn(poly, __expf(-__fmul_rn(az, az))); // erfc(|z|)
-   const float one_plus_erf = (z < 0.0f) ? q : (2.0f - q);
-   return __fmul_rn(__fmul_rn(0.5f, v), one_plus_erf);
+   const float u = __fmul_rn(v, 0.8493218003f);
+   const float h = __fmul_rn(poly, __builtin_amdgcn_exp2f(-__fmul_rn(u, u))); // Phi(-|v|)
+   const float phi = (v < 0.0f) ? h : (1.0f - h);
+   return __fmul_rn(v, phi);
 }
 
 struct F8Epilogue {
@@ -133,11 +133,11 @@ struct F8Epilogue {
    {
 #pragma unroll
       for (int i = 0; i < C; ++i)
-         p.b[i] = bias ? bias[n + i < N ? n + i : N - 1] : 0.0f;
+         p.b[i] = bias ? bias[n + i < N ? n + i : N - 1] : -0.0f; // -0: the neutral element of the addition
    }
    // the constants of one column as 32-bit words (what the register tile store hands from lane to lane): the bias
    static constexpr int kColWords = 1;
-   __device__ __forceinline__ void load_column(int n, uint32_t (&w)[kColWords]) const { w[0] = __float_as_uint(bias ? bias[n] : 0.0f); }
+   __device__ __forceinline__ void load_column(int n, uint32_t (&w)[kColWords]) const { w[0] = __float_as_uint(bias ? bias[n] : -0.0f); }
    __device__ __forceinline__ void load_column_tamed(int n, uint32_t (&w)[kColWords]) const { load_column(n, w); }
    template <int C>
    static __device__ __forceinline__ void set_column(col_params<C> &p, int i, const uint32_t (&w)[kColWords])
@@ -155,9 +155,7 @@ struct F8Epilogue {
       float v[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-         v[i] = mul_nofma(a[i], scale);
-         if (bias)
-            v[i] = v[i] + p.b[4 * q + i];
+         v[i] = mul_nofma(a[i], scale) + p.b[4 * q + i]; // without a bias the constant is -0, which leaves every v as it is
          if constexpr (cls == kClassRelu)
             v[i] = apply_activation(v[i], SOFIE_ACT_RELU, 0.0f);
          else if constexpr (cls == kClassGelu)
