@@ -29,6 +29,8 @@ HBM_PEAK = 8.0e12
 # WRITE_SIZE counters of this same workload, each scaled by what the counter reads for a 256 MiB copy
 # (profiles/mfma8_gemm_dma_128x128_int8_mlp_batch1024.md): (15542 KiB * 2.000 + 4096 KiB * 1.000) * 1024
 DOMINANT_KERNEL_TRAFFIC_BYTES = 36024320
+# shader clock the board holds in the 8192^3 GEMMs (rocprofv3: SQ_BUSY_CYCLES / 32 / kernel duration); the 5.0 POP/s peak assumes 2.4 GHz
+SUSTAINED_CLOCK_GHZ = 1.67
 
 
 def build_mlp():
@@ -404,7 +406,16 @@ def main():
                    "mlp_tops": round(ops_per_inference_batch / (ms_per_step * 1e-3) / 1e12, 2),
                    "mlp_algorithmic_bytes": algo_bytes,
                    "gemm_sweep_int8_requant_bias_relu": sweep,
-                   "gemm_sweep_fp8_bias_gelu_bf16": f8, **extra},
+                   "gemm_sweep_fp8_bias_gelu_bf16": f8,
+                   # the peak at the clock the board holds under this load, beside the nominal one the fractions above use
+                   "peak_at_sustained_clock": {
+                       "nominal_clock_ghz": 2.4, "sustained_clock_ghz": SUSTAINED_CLOCK_GHZ,
+                       "source": "SQ_BUSY_CYCLES / kernel duration of the 8192^3 GEMMs in profiles/bench_all_legs_kernels_and_counters.md "
+                                 "(counters of an earlier run, not of this one)",
+                       "int8_and_fp8_peak_tops": round(INT8_PEAK / 1e12 * SUSTAINED_CLOCK_GHZ / 2.4, 1),
+                       "int8_8192_frac_of_it": (round(sweep[2]["frac_of_int8_peak"] * 2.4 / SUSTAINED_CLOCK_GHZ, 4) if sweep else None),
+                       "fp8_8192_frac_of_it": (round(f8[2]["frac_of_fp8_peak"] * 2.4 / SUSTAINED_CLOCK_GHZ, 4) if f8 else None)},
+                   **extra},
         "roofline": {"bound": "mfma", "achieved": round(achieved / 1e12, 2), "peak": INT8_PEAK / 1e12, "unit": "TFLOP/s",
                      "frac": round(achieved / INT8_PEAK, 4), "traffic": DOMINANT_KERNEL_TRAFFIC_BYTES,
                      "kernel": "mfma8_gemm_dma_kernel<MfmaI8, 128, 128, 128, 2, 2, 3, ...> (layers 1 and 2 of the MLP: 2 launches per inference, "
