@@ -221,6 +221,37 @@ def test_persistent_kernel_forced_on_small_shapes(rt, opt, out, relu_acc, relu_o
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
 
 
+@pytest.mark.parametrize("tile", [0, 64, 512])
+@pytest.mark.parametrize("out,relu_acc,relu_out", [(R.I8OUT_I8, 0, 0), (R.I8OUT_I8, 0, 1), (R.I8OUT_I8, 1, 0), (R.I8OUT_I8_DQQ, 0, 0),
+                                                   (R.I8OUT_I8_DQQ, 1, 0), (R.I8OUT_F32, 0, 1)])
+def test_scales_that_are_negative_zero_huge_or_not_numbers(rt, opt, tile, out, relu_acc, relu_out):
+    """Per-channel scales the conversions have short cuts around: negative, +-0, subnormal, the largest float, +-infinity and
+    NaN, next to ordinary ones.  The 1-byte stores must give the oracle's bytes (a NaN product is stored as 0, an infinite one
+    saturates), the fp32 store its values (NaN where the oracle has NaN).  Tile 0: the heuristic's kernel (store through LDS),
+    64: the small tile, 512: the persistent kernel (store from registers)."""
+    M, N, K = 256, 512, 384
+    A = util.int8_sym(71, M * K).reshape(M, K)
+    A[5, :] = 0                                   # a row of zero accumulators: 0 * inf is NaN
+    Bt = util.int8_sym(72, N * K).reshape(N, K)
+    scale = ((0.5 + util.uniform01(73, N)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    special = [-1e-3, -0.0, 0.0, 1e-42, -1e-42, 3.4028235e38, -3.4028235e38, np.inf, -np.inf, np.nan, 1e30, -7.0]
+    for k, v in enumerate(special):
+        scale[3 + 17 * k] = np.float32(v)
+        scale[260 + 11 * k] = np.float32(v)
+    bias = util.int32_range(74, N, -(1 << 12), 1 << 12)
+    kw = dict(bias=bias, scale=scale, q_scale=np.float32(0.37), relu_acc=relu_acc, relu_out=relu_out, out=out)
+    opt("i8_tile", tile)
+    got = run_gemm(rt, A, Bt, M, N, K, transB=1, **kw)
+    with np.errstate(all="ignore"):
+        want = ob.gemm_i8(A, Bt, M=M, N=N, K=K, transB=1, **kw)
+    if out == R.I8OUT_F32:
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        ok = ~np.isnan(want)
+        assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))
+    else:
+        assert np.array_equal(got, want), np.argwhere(got != want)[:8]
+
+
 def test_persistent_kernel_more_tiles_than_cus(rt):
     """2304 x 8192: 9 x 32 = 288 tiles on 256 CUs, so 32 workgroups take a second tile and the loads of the others run past
     the end of their lists; per-tensor scale (no bias, no scale vector)."""
