@@ -67,7 +67,9 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
                constexpr int i = decltype(ci)::value;
                uint32_t w[4];
                ep.template pack4<MODE, 4>(prm, 0, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3], w);
-               *(uint4 *)(out + ep.out_index(m_base + i * R + lr, n_base + c0) * 4) = make_uint4(w[0], w[1], w[2], w[3]);
+               typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+               const u4 v = {w[0], w[1], w[2], w[3]};
+               __builtin_nontemporal_store(v, (u4 *)(out + ep.out_index(m_base + i * R + lr, n_base + c0) * 4));
             });
          });
       });
@@ -107,8 +109,11 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
                bot[d] = t[1];
             }
             const int n = n_base + j * R + chunk * 8;
-            *(uint4 *)(out + ep.out_index(m_base + i * R + (lane & 15), n) * 2) = make_uint4(top[0], top[1], top[2], top[3]);
-            *(uint4 *)(out + ep.out_index(m_base + i * R + 16 + (lane & 15), n) * 2) = make_uint4(bot[0], bot[1], bot[2], bot[3]);
+            // (streamed like the 1-byte tiles below: FP8 4096^3 -3.8 %, 8192^3 -1 %)
+            typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+            const u4 vt = {top[0], top[1], top[2], top[3]}, vb = {bot[0], bot[1], bot[2], bot[3]};
+            __builtin_nontemporal_store(vt, (u4 *)(out + ep.out_index(m_base + i * R + (lane & 15), n) * 2));
+            __builtin_nontemporal_store(vb, (u4 *)(out + ep.out_index(m_base + i * R + 16 + (lane & 15), n) * 2));
          });
       });
    } else {
