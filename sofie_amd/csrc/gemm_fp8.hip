@@ -137,8 +137,10 @@ struct F8Epilogue {
    }
    // the constants of one column as 32-bit words (what the register tile store hands from lane to lane): the bias
    static constexpr int kColWords = 1;
+   static constexpr bool kBiasInAccumulator = false; // floating-point sums: the bias is added to the finished sum, as the definition has it
+   static constexpr int kBiasWord = 0;
    __device__ __forceinline__ void load_column(int n, uint32_t (&w)[kColWords]) const { w[0] = __float_as_uint(bias ? bias[n] : -0.0f); }
-   __device__ __forceinline__ void load_column_tamed(int n, uint32_t (&w)[kColWords]) const { load_column(n, w); }
+   __device__ __forceinline__ void load_column_for_registers(int n, uint32_t (&w)[kColWords]) const { load_column(n, w); }
    template <int C>
    static __device__ __forceinline__ void set_column(col_params<C> &p, int i, const uint32_t (&w)[kColWords])
    {

@@ -96,11 +96,18 @@ struct I8Epilogue {
    }
    __device__ __forceinline__ bool rows_vectorizable() const { return stage_ok != 0; }
    // row-major output with 16-byte aligned rows, every element stored (what the register tile store handles)
-   bool stores_plain_rows() const { return stage_ok != 0 && nchw_ohw == 0 && rows_per_plane == 0; }
+   // (and, for SOFIE_I8OUT_I8_DQQ, a q_scale against which the largest finite float still saturates: see
+   // load_column_for_registers)
+   bool stores_plain_rows() const
+   {
+      return stage_ok != 0 && nchw_ohw == 0 && rows_per_plane == 0 && q_scale_saturates();
+   }
+   bool q_scale_saturates() const { return out != SOFIE_I8OUT_I8_DQQ || (q_scale > -1e30f && q_scale < 1e30f); }
    // plane sums (of int8 results) whose planes are made of whole groups of `rows` GEMM rows
    bool sums_rows_of_whole_wave_tiles(int rows) const
    {
-      return rows_per_plane != 0 && rows_per_plane % rows == 0 && (out == SOFIE_I8OUT_I8 || out == SOFIE_I8OUT_I8_DQQ) && nchw_ohw == 0;
+      return rows_per_plane != 0 && rows_per_plane % rows == 0 && (out == SOFIE_I8OUT_I8 || out == SOFIE_I8OUT_I8_DQQ) && nchw_ohw == 0 &&
+             q_scale_saturates();
    }
    __device__ __forceinline__ char *out_base() const { return (char *)Y; }
    __device__ __forceinline__ size_t out_index(int m, int n) const
@@ -124,7 +131,7 @@ struct I8Epilogue {
    template <int OUT>
    __device__ __forceinline__ int to_i8(int acc, float s) const
    {
-      if (OUT == SOFIE_I8OUT_I8)
+      if (requantizes<OUT>())
          return quantize_rne_clamp(mul_nofma((float)acc, s), relu_out ? 0 : -128);
       if (OUT == kOutDqqByRcp) // a finite per-tensor scale (the condition of this mode): no NaN to keep out of the short conversion
          return (int)i8_bits(quotient<OUT>(mul_nofma((float)acc, s)), -128.0f);
@@ -164,6 +171,11 @@ struct I8Epilogue {
 
    // The constants of ONE column as 32-bit words (what the register tile store hands from lane to lane): bias, scale.
    static constexpr int kColWords = 2;
+   // The persistent kernel starts a tile's accumulators at the bias of their columns (word kBiasWord) instead of zero: the
+   // sums are exact integers, so the result is that of adding the bias afterwards, and its store (the template argument
+   // BIAS_DONE of the conversions below) saves that addition per element.
+   static constexpr bool kBiasInAccumulator = true;
+   static constexpr int kBiasWord = 0;
    __device__ __forceinline__ void load_column(int n, uint32_t (&w)[kColWords]) const
    {
       w[0] = (uint32_t)(bias ? bias[n + n_offset] : 0);
@@ -177,7 +189,7 @@ struct I8Epilogue {
    }
 
    // the int8 results of columns 4q..4q+3 as integers (what the plane sums of a convolution add up)
-   template <int OUT, int C>
+   template <int OUT, int C, bool BIAS_DONE = false>
    __device__ __forceinline__ void quantize4(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, int (&r)[4]) const
    {
       int acc[4] = {a0, a1, a2, a3};
@@ -185,7 +197,8 @@ struct I8Epilogue {
       asm volatile("" : "+s"(acc_floor)); // kept a number (see pack4)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-         acc[i] += p.b[4 * q + i];
+         if (!BIAS_DONE)
+            acc[i] += p.b[4 * q + i];
          if (OUT != kOutI8NoFloor)
             acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
          float v = mul_nofma((float)acc[i], p.s[4 * q + i]);
@@ -206,53 +219,65 @@ struct I8Epilogue {
       return __float_as_uint(c + 12582912.0f);
    }
    // pack4 for the 1-byte outputs with the short conversion.  float(acc) * s is NaN only for a scale that is NaN, or
-   // infinite against an accumulator of 0; load_column_tamed() below replaces such scales by ones that give the same results
+   // infinite against an accumulator of 0; load_column_for_registers() below replaces such scales by ones that give the same results
    // without NaN.
-   template <int OUT, int C>
+   template <int OUT, int C, bool BIAS_DONE = false>
    __device__ __forceinline__ void pack4_short(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, uint32_t *w) const
    {
       static_assert(requantizes<OUT>() || divides<OUT>(), "1-byte outputs");
       int acc[4] = {a0, a1, a2, a3};
-      uint32_t b[4];
+      float c[4];
       int acc_floor = relu_acc ? 0 : (int)0x80000000;
       asm volatile("" : "+s"(acc_floor)); // kept a number (see pack4)
       const float lo = (requantizes<OUT>() && relu_out) ? 0.0f : -128.0f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-         acc[i] += p.b[4 * q + i];
+         if (!BIAS_DONE)
+            acc[i] += p.b[4 * q + i];
          if (OUT != kOutI8NoFloor)
             acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
          float v = mul_nofma((float)acc[i], p.s[4 * q + i]);
          if (divides<OUT>())
             v = quotient<OUT>(v);
-         b[i] = i8_bits(v, lo);
+         c[i] = __builtin_amdgcn_fmed3f(v, lo, 127.0f);
       }
-      const uint32_t lo2 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
-      const uint32_t hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u);
-      w[0] = __builtin_amdgcn_perm(hi2, lo2, 0x05040100u);
+      // i8_bits() of the four, each addition writing its low byte straight into its place of the dword (sub-dword
+      // destination select): no byte permutes
+      const float magic = 12582912.0f;
+      uint32_t r;
+      asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(r) : "v"(c[0]), "v"(magic));
+      asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(r) : "v"(c[1]), "v"(magic));
+      asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(r) : "v"(c[2]), "v"(magic));
+      asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(r) : "v"(c[3]), "v"(magic));
+      w[0] = r;
    }
-   // load_column with the scale made safe for pack4_short: NaN becomes 0 and +-inf the largest finite number.  The results
-   // are those of the plain scale: a NaN product is stored as 0, and so is 0 * s; a non-zero accumulator times +-inf
-   // saturates like one times +-FLT_MAX.
-   __device__ __forceinline__ void load_column_tamed(int n, uint32_t (&w)[kColWords]) const
+   // load_column for the store from registers.  Its 1-byte conversions (pack4_short, quantize4) need the scale made safe:
+   // NaN becomes 0 and +-inf the largest finite number.  The results are those of the plain scale: a NaN product is stored
+   // as 0, and so is 0 * s; a non-zero accumulator times +-inf saturates like one times +-FLT_MAX (for SOFIE_I8OUT_I8_DQQ
+   // as long as FLT_MAX / q_scale still saturates: stores_plain_rows() keeps larger q_scale away from this store).  The
+   // 4-byte outputs keep the scale as it is: they hand NaN and infinities on.
+   __device__ __forceinline__ void load_column_for_registers(int n, uint32_t (&w)[kColWords]) const
    {
       load_column(n, w);
       float s = __uint_as_float(w[1]);
-      s = (s == s) ? s : 0.0f;
-      w[1] = __float_as_uint(__builtin_amdgcn_fmed3f(s, -3.402823466e38f, 3.402823466e38f));
+      float t = (s == s) ? s : 0.0f;
+      t = __builtin_amdgcn_fmed3f(t, -3.402823466e38f, 3.402823466e38f);
+      w[1] = __float_as_uint((out == SOFIE_I8OUT_I32 || out == SOFIE_I8OUT_F32) ? s : t);
    }
 
    // converts columns 4q..4q+3 of the lane's columns (exact int32 dot products) into 4*out_bytes() bytes
-   template <int OUT, int C>
+   template <int OUT, int C, bool BIAS_DONE = false>
    __device__ __forceinline__ void pack4(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, uint32_t *w) const
    {
+      static_assert(OUT != kOutI8NoFloor, "the store without a floor on the accumulator exists for the short conversion only");
       int acc[4] = {a0, a1, a2, a3};
       float s[4];
       int acc_floor = relu_acc ? 0 : (int)0x80000000; // relu on the accumulator as one max
       asm volatile("" : "+s"(acc_floor));              // kept a number: as a known pair of cases it becomes a max AND a select per element
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-         acc[i] += p.b[4 * q + i];
+         if (!BIAS_DONE)
+            acc[i] += p.b[4 * q + i];
          s[i] = p.s[4 * q + i];
          acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
       }

@@ -58,6 +58,7 @@ struct MfmaI8x16 {
    // XOR applied to the chunk index of row r in a slab of 64-byte rows so that this instruction's fragment read (lane = lk*16 + row,
    // chunk lk) is free of bank conflicts: measured 240 B/clk per CU against 126 B/clk with the (r/4)%4 of the 32-row fragments
    static __device__ __forceinline__ int lds_swizzle(int r) { return (r >> 1) & 3; }
+   static constexpr bool kColumnsOutside = true; // order of a step's MFMAs in the persistent kernel
    struct frag_t {
       v4i c[1];
    };
@@ -79,6 +80,7 @@ struct MfmaF8 {
    static constexpr int ACC = 16;
    // chunk XOR of row r in 64-byte LDS rows: conflict-free for this fragment (lane = lk*32 + row, chunks 2*lk and 2*lk + 1)
    static __device__ __forceinline__ int lds_swizzle(int r) { return (r >> 2) & 3; }
+   static constexpr bool kColumnsOutside = false;
    struct frag_t {
       v4i c[2];
    };

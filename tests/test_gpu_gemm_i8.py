@@ -223,7 +223,7 @@ def test_persistent_kernel_forced_on_small_shapes(rt, opt, out, relu_acc, relu_o
 
 @pytest.mark.parametrize("tile", [0, 64, 512])
 @pytest.mark.parametrize("out,relu_acc,relu_out", [(R.I8OUT_I8, 0, 0), (R.I8OUT_I8, 0, 1), (R.I8OUT_I8, 1, 0), (R.I8OUT_I8_DQQ, 0, 0),
-                                                   (R.I8OUT_I8_DQQ, 1, 0), (R.I8OUT_F32, 0, 1)])
+                                                   (R.I8OUT_I8_DQQ, 1, 0), (R.I8OUT_F32, 0, 1), (R.I8OUT_F32, 0, 0)])
 def test_scales_that_are_negative_zero_huge_or_not_numbers(rt, opt, tile, out, relu_acc, relu_out):
     """Per-channel scales the conversions have short cuts around: negative, +-0, subnormal, the largest float, +-infinity and
     NaN, next to ordinary ones.  The 1-byte stores must give the oracle's bytes (a NaN product is stored as 0, an infinite one
@@ -250,6 +250,63 @@ def test_scales_that_are_negative_zero_huge_or_not_numbers(rt, opt, tile, out, r
         assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))
     else:
         assert np.array_equal(got, want), np.argwhere(got != want)[:8]
+
+
+@pytest.mark.parametrize("tile", [0, 512])
+def test_dequantize_quantize_with_a_huge_output_scale_and_infinite_channel_scales(rt, opt, tile):
+    """SOFIE_I8OUT_I8_DQQ with q_scale near the top of the float range: (acc * inf) / q_scale saturates, (acc * FLT_MAX) /
+    q_scale does not.  The store from registers, which replaces an infinite scale by FLT_MAX, must not be given this product
+    (tile 512 asks for it; the library has to decline and take a kernel with the exact conversion)."""
+    M, N, K = 256, 256, 384
+    A = util.int8_sym(81, M * K).reshape(M, K)
+    A[7, :] = 0
+    A[9, :] = 0
+    A[9, 0] = 1                                   # accumulators of +-1 .. +-127: the smallest non-zero products
+    Bt = util.int8_sym(82, N * K).reshape(N, K)
+    scale = np.full(N, np.float32(1e-3), np.float32)
+    scale[::3] = np.inf
+    scale[1::7] = -np.inf
+    scale[2::11] = np.float32(3.4028235e38)
+    kw = dict(scale=scale, q_scale=np.float32(3e37), relu_acc=0, relu_out=0, out=R.I8OUT_I8_DQQ)
+    opt("i8_tile", tile)
+    got = run_gemm(rt, A, Bt, M, N, K, transB=1, **kw)
+    with np.errstate(all="ignore"):
+        want = ob.gemm_i8(A, Bt, M=M, N=N, K=K, transB=1, **kw)
+    assert np.array_equal(got, want), np.argwhere(got != want)[:8]
+
+
+def test_config3_at_1024_int8_output_in_full(rt):
+    """benchmark configuration 3 at M=N=K=1024 with its own epilogue (per-channel scale, bias, relu, int8 out): every element."""
+    M = N = K = 1024
+    A = util.int8_sym(3001, M * K).reshape(M, K)
+    Bt = util.int8_sym(3002, N * K).reshape(N, K)
+    bias = util.int32_range(3003, N, -(1 << 15), 1 << 15)
+    scale = ((0.5 + util.uniform01(3004, N)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    kw = dict(bias=bias, scale=scale, relu_out=1, out=R.I8OUT_I8)
+    got = run_gemm(rt, A, Bt, M, N, K, transB=1, **kw)
+    want = ob.gemm_i8(A, Bt, M=M, N=N, K=K, transB=1, omp=True, **kw)
+    assert np.array_equal(got, want)
+    assert got.max() == 127 and (got == 0).mean() > 0.3
+
+
+def test_config3_at_4096_sampled_rows_and_columns(rt):
+    """benchmark configuration 3 at M=N=K=4096 (one 256 x 256 tile per compute unit: no workgroup takes a second tile, and
+    the loads that run past the end of each one-tile list are the filler path): sampled full rows and columns, bit-exact."""
+    M = N = K = 4096
+    A = util.int8_sym(3001, M * K).reshape(M, K)
+    Bt = util.int8_sym(3002, N * K).reshape(N, K)
+    bias = util.int32_range(3003, N, -(1 << 15), 1 << 15)
+    scale = ((0.5 + util.uniform01(3004, N)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    got = run_gemm(rt, A, Bt, M, N, K, transB=1, bias=bias, scale=scale, relu_out=1, out=R.I8OUT_I8)
+    rows = np.array([0, 1, 15, 16, 127, 128, 255, 256, 2047, 2048, 3000, 4094, 4095])
+    want = ob.gemm_i8(np.ascontiguousarray(A[rows]), Bt, M=len(rows), N=N, K=K, transB=1, omp=True, bias=bias, scale=scale,
+                      relu_out=1, out=R.I8OUT_I8)
+    assert np.array_equal(got[rows], want)
+    cols = np.array([0, 3, 4, 63, 64, 255, 256, 2049, 4095])
+    want_c = ob.gemm_i8(A, np.ascontiguousarray(Bt[cols]), M=M, N=len(cols), K=K, transB=1, omp=True, bias=bias[cols],
+                        scale=scale[cols], relu_out=1, out=R.I8OUT_I8)
+    assert np.array_equal(got[:, cols], want_c)
+    assert got.max() == 127 and (got == 0).mean() > 0.3
 
 
 def test_persistent_kernel_more_tiles_than_cus(rt):
