@@ -4,11 +4,16 @@
 Workload (benchmark configuration 2): int8 quantised MLP 1024 -> 4096 -> 4096 -> 1024 at batch 1024,
 QuantizeLinear -> [int8 Gemm (int32 accumulate) -> Relu -> DequantizeLinear]x3, per-tensor scales,
 synthetic seeded data, fp32 input already resident in HBM.  One step = one inference over the batch.
-What is timed for `value` is the Session the generator EMITS for this model (tests/emitted/Config2_int8_MLP_GPU_HIP.hxx, weights
-from a safetensors file), the way the reference's benchmark times its generated code (benchmark/src/BenchmarkEmitter.cxx.in:486-504):
+What is timed for `value` is the Session the generator EMITS for this model (sofie_amd/benchsupport/emitted/Config2_int8_MLP_GPU_HIP.hxx,
+weights from a safetensors file), the way the reference's benchmark times its generated code (benchmark/src/BenchmarkEmitter.cxx.in:486-504):
 K x infer_nosync, one wait, wall clock; `value` is the MEDIAN of five such regions.
 Prints ONE JSON line; `value` = inferences/s.  Also times the stand-alone int8 and FP8 GEMM sweeps (M=N=K in 1024/4096/8192), the
-fp32 MLP and the int8 CNN, and the CPU oracle on bounded samples.
+emitted one-operator Session of the 8192^3 int8 GEMM, the fp32 MLP, the emitted Session of the int8 CNN, and the CPU oracle on
+bounded samples.
+
+Every timed region starts on a chip that has been running the same launches for at least CLOCK_WARM_MS: after an idle spell the
+board needs some 20 - 40 ms of load to settle on the clock it then holds (regions timed earlier read up to 20 % slow, and the
+first ones after them still 3 %), so a region measures the steady state the path runs at in service, whatever --warmup says.
 """
 import argparse
 import ctypes as C
@@ -25,17 +30,26 @@ import numpy as np
 
 INT8_PEAK = 5.0e15  # MI355X dense int8 MFMA peak, op/s
 HBM_PEAK = 8.0e12
-# HBM bytes per launch of the dominant kernel (average of the layer-1 and layer-2 launches), from the FETCH_SIZE and
-# WRITE_SIZE counters of this same workload, each scaled by what the counter reads for a 256 MiB copy
-# (profiles/mfma8_gemm_dma_128x128_int8_mlp_batch1024.md): (15542 KiB * 2.000 + 4096 KiB * 1.000) * 1024
-DOMINANT_KERNEL_TRAFFIC_BYTES = 36024320
-# shader clock the board holds in the 8192^3 GEMMs (rocprofv3: SQ_BUSY_CYCLES / 32 / kernel duration); the 5.0 POP/s peak assumes 2.4 GHz
-SUSTAINED_CLOCK_GHZ = 1.67
+CLOCK_WARM_MS = 60.0   # untimed load in front of every timed region
+PROFILE_OF_DOMINANT_KERNEL = os.path.join(ROOT, "profiles", "mfma8_gemm_dma_128x128_int8_mlp_batch1024.md")
+
+
+def dominant_kernel_traffic_bytes():
+    """HBM bytes per launch of the dominant kernel (average of the layer-1 and layer-2 launches), from the FETCH_SIZE and WRITE_SIZE
+    counters of this same workload, each scaled by what the counter reads for a 256 MiB copy: read from the committed profile
+    summary (its line `traffic_bytes_per_launch: N`), so that the figure and its evidence cannot drift apart; None without it."""
+    try:
+        for line in open(PROFILE_OF_DOMINANT_KERNEL):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":", 1)[1].split()[0])
+    except (OSError, ValueError):
+        pass
+    return None
 
 
 def build_mlp():
-    """The constants of the emitted benchmark model (tests/emitted_models.bench_mlp_spec): weights, frozen scales, the input batch."""
-    from tests import emitted_models as em
+    """The constants of the emitted benchmark model (benchsupport.emitted.bench_mlp_spec): weights, frozen scales, the input batch."""
+    from sofie_amd.benchsupport import emitted as em
     spec = em.bench_mlp_spec()
     c = spec["consts"]
     return [1024, 4096, 4096, 1024], 1024, spec["feeds"][0], c["weights"], c["w_scales"], c["in_scales"]
@@ -53,24 +67,42 @@ def time_region(rt, fn, reps):
 
 
 def region_launches(rt, fn, least):
-    """Launches per timed region: at least `least`, and enough for a region of about 20 ms (the chip takes a few milliseconds of
-    load to settle on the clock it then holds: regions of 2 ms read 15 % slower than regions of 40 ms)."""
+    """Launches per timed region: at least `least`, and enough for a region of about 20 ms."""
     ms, _ = time_region(rt, fn, least)
     return max(least, min(5000, int(20.0 / max(ms / least, 1e-4)) + 1))
 
 
+def warm_clock(rt, fn, per_call_ms):
+    """CLOCK_WARM_MS of the same launches, untimed, straight in front of a timed region."""
+    n = max(1, min(20000, int(CLOCK_WARM_MS / max(per_call_ms, 1e-4)) + 1))
+    for _ in range(n):
+        fn()
+    rt.sync()
+
+
+def steady_regions(rt, fn, least, count=5):
+    """`count` timed regions of fn on a warmed chip: (sorted region times in ms, launches per region)."""
+    n_launch = region_launches(rt, fn, least)
+    ms, _ = time_region(rt, fn, n_launch)
+    warm_clock(rt, fn, ms / n_launch)
+    return sorted(time_region(rt, fn, n_launch)[0] for _ in range(count)), n_launch
+
+
 def gemm_sweep(rt, sizes, reps=20, warmup=10):
-    """Stand-alone int8 GEMM with per-channel requant + bias + relu (benchmark configuration 3)."""
+    """Stand-alone int8 GEMM with per-channel requant + bias + relu (benchmark configuration 3) through the C-ABI; each size is
+    checked on sampled rows against the CPU oracle outside the timed regions."""
+    from oracle import binding as ob
     from sofie_amd import runtime as R
-    from tests import util
+    from sofie_amd.benchsupport import synthetic as util
     import torch
     out = []
     for n in sizes:
         M = N = K = n
-        A = util.to_dev(util.int8_sym(3001, M * K).reshape(M, K))
-        Bt = util.to_dev(util.int8_sym(3002, N * K).reshape(N, K))
-        bias = util.to_dev(util.int32_range(3003, N, -(1 << 15), 1 << 15))
-        scale = util.to_dev(((0.5 + util.uniform01(3004, N)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32))
+        hA = util.int8_sym(3001, M * K).reshape(M, K)
+        hBt = util.int8_sym(3002, N * K).reshape(N, K)
+        hbias = util.int32_range(3003, N, -(1 << 15), 1 << 15)
+        hscale = ((0.5 + util.uniform01(3004, N)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+        A, Bt, bias, scale = util.to_dev(hA), util.to_dev(hBt), util.to_dev(hbias), util.to_dev(hscale)
         Y = util.dev_empty((M, N), np.int8)
         torch.cuda.synchronize()
         d = R.GemmI8Desc()
@@ -80,54 +112,94 @@ def gemm_sweep(rt, sizes, reps=20, warmup=10):
         fn = lambda: rt.call("sofie_hip_gemm_i8", C.byref(d))
         for _ in range(warmup):
             fn()
-        n_launch = region_launches(rt, fn, reps)
-        regions = sorted(time_region(rt, fn, n_launch)[0] for _ in range(5))
+        regions, n_launch = steady_regions(rt, fn, reps)
         t = regions[2] / n_launch * 1e-3  # the median region
+        rows = np.array(sorted({0, 1, 255 % M, 256 % M, M // 2, M - 1}))
+        want = ob.gemm_i8(np.ascontiguousarray(hA[rows]), hBt, M=len(rows), N=N, K=K, transB=1, omp=True, bias=hbias, scale=hscale,
+                          relu_out=1, out=R.I8OUT_I8)
+        parity = bool(np.array_equal(util.to_host(Y)[rows], want))
         ops = 2.0 * M * N * K
         out.append({"M": M, "N": N, "K": K, "ms": round(t * 1e3, 5), "ms_fastest_region": round(regions[0] / n_launch, 5), "launches_per_region": n_launch,
                     "tops": round(ops / t / 1e12, 2),
                     "frac_of_int8_peak": round(ops / t / INT8_PEAK, 4),
-                    "hbm_gbps_algorithmic": round((M * K + K * N + M * N + 8 * N) / t / 1e9, 1)})
+                    "hbm_gbps_algorithmic": round((M * K + K * N + M * N + 8 * N) / t / 1e9, 1),
+                    "parity": {"rows_vs_oracle": [int(r) for r in rows], "bit_exact": parity}})
         del A, Bt, Y
         torch.cuda.empty_cache()
     return out
 
 
+def emitted_gemm_leg(steps=20):
+    """benchmark configuration 3 at 8192^3 as the generator emits it: a one-operator model (QGemm + Relu), B re-laid out once in the
+    Session's constructor, steps x infer_nosync + one wait (benchmark/src/BenchmarkEmitter.cxx.in:486-504)."""
+    from oracle import binding as ob
+    from sofie_amd.benchsupport import emitted as em
+    spec = em.bench_gemm_spec()
+    c, A = spec["consts"], spec["feeds"][0]
+    n = A.shape[0]
+    s = em.BenchSession(em.GEMM_MODEL)
+    try:
+        s.upload(A)
+        _, ev = s.run(steps)
+        s.run(max(steps, int(CLOCK_WARM_MS / max(ev / steps, 1e-3)) + 1))   # the clock warm-up
+        regions = sorted(s.run(steps)[1] for _ in range(5))
+        rows = np.array([0, 1, 255, 256, n // 2, n - 1])
+        got = s.download((n, n), np.int8)[rows]
+    finally:
+        s.close()
+    want = ob.gemm_i8(np.ascontiguousarray(A[rows]), c["Bt"], M=len(rows), N=n, K=n, transB=1, omp=True, bias=c["bias"], scale=c["scale"],
+                      relu_out=1, out=2)
+    t = regions[2] / steps * 1e-3
+    ops = 2.0 * n * n * n
+    return {"model": em.GEMM_MODEL, "M": n, "N": n, "K": n, "ms": round(t * 1e3, 5), "ms_fastest_region": round(regions[0] / steps, 5),
+            "launches_per_region": steps, "tops": round(ops / t / 1e12, 2), "frac_of_int8_peak": round(ops / t / INT8_PEAK, 4),
+            "parity": {"rows_vs_oracle": [int(r) for r in rows], "bit_exact": bool(np.array_equal(got, want))}}
+
+
 def fp8_sweep(rt, sizes, reps=20, warmup=10):
-    """Stand-alone FP8 e4m3 GEMM, fp32 accumulate, per-tensor scale, bias + GELU, bf16 output (benchmark configuration 4)."""
+    """Stand-alone FP8 e4m3 GEMM, fp32 accumulate, per-tensor scale, bias + GELU, bf16 output (benchmark configuration 4): A, B ~ N(0,1)
+    from the counter generator (seeds 4001 / 4002), each scaled by s = max|x| / 448 and rounded to e4m3fn; bias ~ N(0,1) (seed 4003):
+    the data the full-size parity test checks.  Each size is checked on sampled rows against the CPU oracle (the stated bound of
+    sofie_hip_gemm_fp8) outside the timed regions."""
+    from oracle import binding as ob
     from sofie_amd import runtime as R
-    from tests import util
+    from sofie_amd.benchsupport import synthetic as util
+    from sofie_amd.benchsupport.models import fp8_operand
     import torch
+
+    def quantize(x, s_):
+        dx, dq = util.to_dev(x), util.dev_empty(x.shape, np.uint8)
+        rt.call("sofie_hip_quantize_fp8", util.ptr(dq), util.ptr(dx), C.c_size_t(x.size), C.c_float(s_))
+        rt.sync()
+        return dq
     out = []
     for n in sizes:
         M = N = K = n
-        g = torch.Generator(device="cuda")
-        g.manual_seed(4000 + n)
-        Af = torch.randn((M, K), generator=g, device="cuda", dtype=torch.float32)
-        Bf = torch.randn((N, K), generator=g, device="cuda", dtype=torch.float32)
-        A, Bt = util.dev_empty((M, K), np.uint8), util.dev_empty((N, K), np.uint8)
-        bias = util.to_dev(util.normal(4003, N))
+        A, sa = fp8_operand(4001, M, K, quantize)
+        Bt, sb = fp8_operand(4002, N, K, quantize)
+        hbias = util.normal(4003, N)
+        bias = util.to_dev(hbias)
         Y = util.dev_empty((M, N), np.uint16)
         torch.cuda.synchronize()
-        s = 4.0 / 448.0  # N(0,1) scaled into the e4m3 range: 4 sigma -> 448
-        rt.call("sofie_hip_quantize_fp8", util.ptr(A), util.ptr(Af), C.c_size_t(M * K), C.c_float(s))
-        rt.call("sofie_hip_quantize_fp8", util.ptr(Bt), util.ptr(Bf), C.c_size_t(N * K), C.c_float(s))
-        rt.sync()
-        del Af, Bf
         d = R.GemmFp8Desc()
         d.M, d.N, d.K, d.transB = M, N, K, 1
         d.A, d.B, d.bias, d.Y = util.ptr(A), util.ptr(Bt), util.ptr(bias), util.ptr(Y)
-        d.scale, d.act, d.out = s * s, R.ACT_GELU, 0
+        scale = np.float32(sa * sb)
+        d.scale, d.act, d.out = float(scale), R.ACT_GELU, 0
         fn = lambda: rt.call("sofie_hip_gemm_fp8", C.byref(d))
         for _ in range(warmup):
             fn()
-        n_launch = region_launches(rt, fn, reps)
-        regions = sorted(time_region(rt, fn, n_launch)[0] for _ in range(5))
+        regions, n_launch = steady_regions(rt, fn, reps)
         t = regions[2] / n_launch * 1e-3  # the median region
+        rows = np.array(sorted({0, 255 % M, M // 2, M - 1}))
+        hA, hBt = util.to_host(A)[rows], util.to_host(Bt)
+        got = ob.bf16_bits_to_f32(util.to_host(Y).view(np.uint16)[rows])
+        excess = ob.fp8_gemm_bound_excess(got, np.ascontiguousarray(hA), hBt, hbias, scale, R.ACT_GELU, bf16=True)
         ops = 2.0 * M * N * K
         out.append({"M": M, "N": N, "K": K, "ms": round(t * 1e3, 5), "ms_fastest_region": round(regions[0] / n_launch, 5), "launches_per_region": n_launch,
                     "tflops": round(ops / t / 1e12, 2),
-                    "frac_of_fp8_peak": round(ops / t / INT8_PEAK, 4)})
+                    "frac_of_fp8_peak": round(ops / t / INT8_PEAK, 4),
+                    "parity": {"rows_vs_oracle": [int(r) for r in rows], "within_stated_bound": bool(excess <= 0.0)}})
         del A, Bt, Y
         torch.cuda.empty_cache()
     return out
@@ -139,7 +211,7 @@ def fp32_mlp_leg(steps=200):
     generated code on the same batch."""
     from sofie_amd import Runtime, runtime as R
     from oracle import binding as ob
-    from tests import util
+    from sofie_amd.benchsupport import synthetic as util
     dims, batch = [784, 128, 64, 10], 64
     rt = Runtime(0)
     x = util.uniform01(2001, batch * 784).reshape(batch, 784)
@@ -166,10 +238,12 @@ def fp32_mlp_leg(steps=200):
             rt.call("sofie_hip_gemm_f32", C.byref(descs[l]))
     for _ in range(10):
         step_by_layer()
-    ms_layers, _ = time_region(rt, step_by_layer, steps)
+    r, n_l = steady_regions(rt, step_by_layer, steps, count=3)
+    ms_layers = r[1] * steps / n_l
     for _ in range(10):
         step()
-    ms, _ = time_region(rt, step, steps)
+    r, n_l = steady_regions(rt, step, steps, count=3)
+    ms = r[1] * steps / n_l
     got = util.to_host(H[2])
     rt.close()
     t0 = time.perf_counter()
@@ -186,31 +260,33 @@ def fp32_mlp_leg(steps=200):
             "max_rel_err_vs_oracle": err, "cpu_oracle_us_per_batch_1_core": round(cpu_s * 1e6, 1)}
 
 
-def int8_cnn_leg(steps=10, parity=True):
+def int8_cnn_leg(steps=20, parity=True):
     """benchmark configuration 5: 4 x [Conv3x3 s1 p1 + folded BatchNorm + Relu] 3->64->128->256->256 on 64x64 images, batch 256,
-    global average pool, Gemm 256->10; int8 weights, per-channel scales.  Parity: the CPU chain on four of the 256 images."""
-    from sofie_amd import Runtime
-    from sofie_amd.session import Int8CNNSession
-    from tests.refmodels import make_int8_cnn, int8_cnn_oracle
-    batch = 256
-    m = make_int8_cnn(batch, 64)
-    rt = Runtime(0)
-    s = Int8CNNSession(rt, m["batch"], m["in_shape"], m["in_scale"], m["convs"], m["last_scale"], m["fc_w"], m["fc_b"])
-    got = s.infer(m["x"])
-    rt.sync()
-    for _ in range(3):
-        s.infer_nosync()
-    steps = max(steps, 20)
-    regions = sorted(time_region(rt, s.infer_nosync, steps)[0] for _ in range(3))
-    ms = regions[1]  # the median of three regions of about 25 ms
-    rt.close()
+    global average pool, Gemm 256->10; int8 weights, per-channel scales.  Timed: the Session the generator emits for the model
+    (parsed from ONNX, weights from a safetensors file), steps x infer_nosync + one wait.  Parity: the CPU chain on four of the
+    256 images."""
+    from oracle.chains import int8_cnn_oracle
+    from sofie_amd.benchsupport import emitted as em
+    spec = em.bench_cnn_spec()
+    m, x = spec["consts"], spec["feeds"][0]
+    batch = x.shape[0]
+    s = em.BenchSession(em.CNN_MODEL)
+    try:
+        s.upload(x)
+        _, ev = s.run(steps)
+        s.run(max(steps, int(CLOCK_WARM_MS / max(ev / steps, 1e-3)) + 1))   # the clock warm-up
+        regions = sorted(s.run(steps)[1] for _ in range(5))
+        got = s.download((batch, 10))
+    finally:
+        s.close()
+    ms = regions[2]  # the median of five regions of about 20 ms
     ops = 2.0 * batch * 64 * 64 * sum(cv["W"].size for cv in m["convs"])
     t = ms / steps * 1e-3
-    out = {"ms_per_batch": round(t * 1e3, 4), "images_per_s": round(batch / t, 0), "tops": round(ops / t / 1e12, 1),
-           "frac_of_int8_peak": round(ops / t / INT8_PEAK, 4)}
+    out = {"model": em.CNN_MODEL, "ms_per_batch": round(t * 1e3, 4), "ms_per_batch_fastest_region": round(regions[0] / steps, 4),
+           "images_per_s": round(batch / t, 0), "tops": round(ops / t / 1e12, 1), "frac_of_int8_peak": round(ops / t / INT8_PEAK, 4)}
     if parity:
         sample = [0, 85, 170, 255]
-        want = int8_cnn_oracle(m, np.ascontiguousarray(m["x"][sample]))
+        want = int8_cnn_oracle(m, np.ascontiguousarray(x[sample]))
         err = float(np.abs(got[sample] - want).max() / max(1.0, float(np.abs(want).max())))
         out["parity_images_vs_oracle"] = sample
         out["max_rel_err_vs_oracle"] = err
@@ -257,8 +333,8 @@ def cpu_baseline(x, weights, w_scales, in_scales, rows):
     """The oracle's unfused CPU chain (oracle/sofie_oracle.c) on the host cores: all threads on the whole batch, one thread on a
     sample of rows; and the 8192^3 int8 product with its requantising store on a slice of 1024 of its 8192 rows."""
     from oracle import binding as ob
-    from tests import util
-    from tests.refmodels import int8_mlp_oracle
+    from oracle.chains import int8_mlp_oracle
+    from sofie_amd.benchsupport import synthetic as util
     threads = int(ob.load(True).oracle_num_threads())
     int8_mlp_oracle(x[:2], weights, w_scales, in_scales, omp=True)  # warm the caches / thread pool
     passes, t0 = 0, time.perf_counter()
@@ -313,10 +389,12 @@ def main():
     from sofie_amd.session import Int8MLPSession
 
     dims, batch, x, weights, w_scales, in_scales = build_mlp()
-    from tests import emitted_models as em
+    from sofie_amd.benchsupport import emitted as em
     emitted = em.BenchSession()   # raises if the emitted Session has not been built (__graft_entry__.build())
     emitted.upload(x)
-    emitted.run(args.warmup)
+    w_wall, _ = emitted.run(max(args.warmup, 1))
+    # the clock warm-up: at least CLOCK_WARM_MS of the same inferences straight in front of the timed regions
+    emitted.run(int(CLOCK_WARM_MS / max(w_wall / max(args.warmup, 1), 1e-3)) + 1)
     regions = [emitted.run(args.steps) for _ in range(5)]   # (wall ms, event ms) of K x infer_nosync + one wait
     walls = sorted(w for w, _ in regions)
     wall = walls[2]                                         # the median region is the one reported
@@ -345,7 +423,8 @@ def main():
         for d in dom:
             rt.call("sofie_hip_gemm_i8", C.byref(d))
     dominant_only()
-    gms, _ = time_region(rt, dominant_only, args.steps)
+    g_regions, g_n = steady_regions(rt, dominant_only, args.steps, count=3)
+    gms = g_regions[1] * args.steps / g_n      # the median region, scaled to args.steps calls
     launches = len(dom) * args.steps
     ops_per_inference_batch = 2.0 * batch * sum(dims[l] * dims[l + 1] for l in range(3))
     ops_per_launch = sum(2.0 * d.M * d.N * d.K for d in dom) / len(dom)
@@ -372,6 +451,7 @@ def main():
 
     sweep = [] if args.no_sweep else gemm_sweep(rt, [1024, 4096, 8192])
     f8 = [] if args.no_sweep else fp8_sweep(rt, [1024, 4096, 8192])
+    emitted_gemm = None if args.no_sweep else emitted_gemm_leg()
     if args.calibrate_copy:
         nbytes = 256 << 20
         src = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
@@ -397,7 +477,7 @@ def main():
         "config": {"workload": "int8 MLP 1024->4096->4096->1024, batch 1024, Q -> [i8 Gemm(i32) -> Relu -> DQ]x3, "
                                "per-tensor symmetric scales, input resident in HBM (benchmark configuration 2)",
                    "timed": "the emitted Session (Config2_int8_MLP_GPU_HIP.hxx, safetensors weights): K x infer_nosync + one wait, wall clock, "
-                            "median of 5 regions",
+                            "median of 5 regions, on a chip warmed by %g ms of the same inferences" % CLOCK_WARM_MS,
                    "global_batch": batch, "launches_per_step": 4, "event_ms_per_step": round(event_ms_per_step, 5),
                    "ms_per_step_of_5_regions": repeats,
                    "h2d_ms_per_batch": h2d_ms, "d2h_ms_per_batch": d2h_ms,
@@ -405,19 +485,13 @@ def main():
                    "parity_vs_oracle_rows": args.cpu_rows, "parity_bit_exact": parity,
                    "mlp_tops": round(ops_per_inference_batch / (ms_per_step * 1e-3) / 1e12, 2),
                    "mlp_algorithmic_bytes": algo_bytes,
+                   "clock_warm_ms_before_each_timed_region": CLOCK_WARM_MS,
                    "gemm_sweep_int8_requant_bias_relu": sweep,
+                   "gemm_int8_8192_emitted_session": emitted_gemm,
                    "gemm_sweep_fp8_bias_gelu_bf16": f8,
-                   # the peak at the clock the board holds under this load, beside the nominal one the fractions above use
-                   "peak_at_sustained_clock": {
-                       "nominal_clock_ghz": 2.4, "sustained_clock_ghz": SUSTAINED_CLOCK_GHZ,
-                       "source": "SQ_BUSY_CYCLES / kernel duration of the 8192^3 GEMMs in profiles/bench_all_legs_kernels_and_counters.md "
-                                 "(counters of an earlier run, not of this one)",
-                       "int8_and_fp8_peak_tops": round(INT8_PEAK / 1e12 * SUSTAINED_CLOCK_GHZ / 2.4, 1),
-                       "int8_8192_frac_of_it": (round(sweep[2]["frac_of_int8_peak"] * 2.4 / SUSTAINED_CLOCK_GHZ, 4) if sweep else None),
-                       "fp8_8192_frac_of_it": (round(f8[2]["frac_of_fp8_peak"] * 2.4 / SUSTAINED_CLOCK_GHZ, 4) if f8 else None)},
                    **extra},
-        "roofline": {"bound": "mfma", "achieved": round(achieved / 1e12, 2), "peak": INT8_PEAK / 1e12, "unit": "TFLOP/s",
-                     "frac": round(achieved / INT8_PEAK, 4), "traffic": DOMINANT_KERNEL_TRAFFIC_BYTES,
+        "roofline": {"bound": "mfma", "achieved": round(achieved / 1e12, 2), "peak": INT8_PEAK / 1e12, "unit": "TOP/s",
+                     "frac": round(achieved / INT8_PEAK, 4), "traffic": dominant_kernel_traffic_bytes(),
                      "kernel": "mfma8_gemm_dma_kernel<MfmaI8, 128, 128, 128, 2, 2, 3, ...> (layers 1 and 2 of the MLP: 2 launches per inference, "
                                "avg %.2f us, %.3e int8 op per launch on average)" % (avg_launch_s * 1e6, ops_per_launch)},
         "cpu_baseline": cpu,

@@ -417,3 +417,32 @@ def gemm_fp8(A, B, *, M, N, K, transB=0, bias=None, scale=1.0, act=0, out=1, wan
     sa = np.empty((M, N), dtype=np.float32) if want_abs_sum else None
     load(omp).oracle_gemm_fp8(M, N, K, transB, _ptr(A), _ptr(B), _ptr(b), C.c_float(scale), act, out, _ptr(Y), _ptr(sa))
     return (Y, sa) if want_abs_sum else Y
+
+
+def fp8_gemm_bound(A, Bt, bias, scale, act, bf16, omp=True):
+    """The per-element bound that include/sofie_hip.h states for sofie_hip_gemm_fp8, evaluated for A [M,K] x Bt [N,K]^T:
+    returns (y0, bound) with y0 the fp32 result of exact accumulation."""
+    M, K = A.shape
+    N = Bt.shape[0]
+    scale = np.float32(scale)
+    y0, S = gemm_fp8(A, Bt, M=M, N=N, K=K, transB=1, bias=bias, scale=scale, act=act, out=1, want_abs_sum=True, omp=omp)
+    v0 = y0 if act == 0 else gemm_fp8(A, Bt, M=M, N=N, K=K, transB=1, bias=bias, scale=scale, act=0, out=1, omp=omp)
+    y0 = y0.astype(np.float64)
+    v0 = np.abs(v0.astype(np.float64))
+    b = np.zeros(N) if bias is None else np.abs(np.asarray(bias, dtype=np.float64))
+    lip = 1.13 if act in (4, 5) else 1.0     # SOFIE_ACT_GELU, SOFIE_ACT_GELU_TANH
+    bound = lip * (2.0 ** -14 * S.astype(np.float64) * float(scale) + 2.0 ** -22 * (v0 + b[None, :]))
+    if act == 4:
+        bound = bound + 1e-6 * v0
+    bound = bound + 2.0 ** -21 * np.abs(y0)
+    if bf16:
+        # half an ulp of bf16 (8 significant bits) at the largest magnitude the result may have
+        top = np.maximum(np.abs(y0) + bound, 2.0 ** -126)
+        bound = bound + np.ldexp(1.0, np.floor(np.log2(top)).astype(np.int64) - 8)
+    return y0, bound
+
+
+def fp8_gemm_bound_excess(got, A, Bt, bias, scale, act, bf16, omp=True):
+    """max over the elements of |got - y0| - bound: positive where a result leaves the stated bound."""
+    y0, bound = fp8_gemm_bound(A, Bt, bias, scale, act, bf16, omp=omp)
+    return float((np.abs(np.asarray(got, dtype=np.float64) - y0) - bound).max())

@@ -498,7 +498,7 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
       }
       // element type and rank of what this node produces
       int outType = inType;
-      if (n.op == "QuantizeLinear" || n.op == "QLinearConv" || n.op == "QLinearMatMul")
+      if (n.op == "QuantizeLinear" || n.op == "QLinearConv" || n.op == "QLinearMatMul" || n.op == "QGemm")
          outType = 3;
       else if (n.op == "MatMulInteger" || n.op == "ConvInteger")
          outType = 6;
@@ -526,7 +526,7 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          // a node must name the inputs its operator reads below and one output, whatever the file claims
          static const std::map<std::string, size_t> minInputs = {
             {"Gemm", 2}, {"MatMul", 2}, {"Add", 2}, {"Sub", 2}, {"Mul", 2}, {"Div", 2}, {"Pow", 2}, {"Conv", 2}, {"QuantizeLinear", 2}, {"DequantizeLinear", 2}, {"BatchNormalization", 5},
-            {"MatMulInteger", 2}, {"ConvInteger", 2}, {"QLinearConv", 8}, {"QLinearMatMul", 8}};
+            {"MatMulInteger", 2}, {"ConvInteger", 2}, {"QLinearConv", 8}, {"QLinearMatMul", 8}, {"QGemm", 9}};
          auto f = minInputs.find(n.op);
          const size_t need = f == minInputs.end() ? 1 : f->second;
          if (n.in.size() < need || n.out.empty())
@@ -755,6 +755,44 @@ std::unique_ptr<RModel> RModelParser_ONNX::Parse(std::string filename, bool verb
          const std::string mname = n.out[0] + "_requant_scale";
          model->AddInitializedTensor(mname, ETensorType::FLOAT, {ncols}, mult.data());
          auto op = std::make_unique<ROperator_QGemm>(n.in[0], n.in[3], n.out[0]);
+         op->SetRequantize(mname, false);
+         model->AddOperator(std::move(op));
+      } else if (n.op == "QGemm") {
+         // The contrib operator (domain com.microsoft): Y = sat8(rne((A x B + C) * ((a_scale * b_scale[n]) / y_scale))) with an
+         // int32 bias C [N] that counts in units of a_scale * b_scale, i.e. is added to the accumulator.  Inputs: A, a_scale,
+         // a_zero_point, B, b_scale, b_zero_point, C, y_scale, y_zero_point.  Symmetric quantisation, alpha = 1, a constant B
+         // stored [K,N].
+         if (n.in.size() != 9)
+            throw std::runtime_error("SOFIE ONNX parser: QGemm " + n.name + " needs 9 inputs (the quantised output form)");
+         if (attrF(n, "alpha", 1.f) != 1.f || attrI(n, "transA", 0) != 0 || attrI(n, "transB", 0) != 0)
+            throw std::runtime_error("SOFIE ONNX parser: QGemm " + n.name + ": alpha = 1, transA = 0 and transB = 0 only");
+         for (int z : {2, 5, 8}) {
+            const std::string zn = UTILITY::Clean_name(n.in[z]);
+            if (!model->IsInitializedTensor(zn) || model->GetTensorType(zn) != ETensorType::INT8)
+               throw std::runtime_error("SOFIE ONNX parser: QGemm zero point " + n.in[z] + " must be an int8 initializer");
+            const auto *p = static_cast<const int8_t *>(model->GetInitializedTensorData(zn).get());
+            for (size_t k = 0; k < ConvertShapeToLength(model->GetTensorShape(zn)); ++k)
+               if (p[k] != 0)
+                  throw std::runtime_error("SOFIE ONNX parser: QGemm zero point " + n.in[z] + " is not 0; symmetric quantisation only");
+         }
+         const float as = model->GetScalarInitializer(n.in[1]), ys = model->GetScalarInitializer(n.in[7]);
+         const std::string bsn = UTILITY::Clean_name(n.in[4]), bn = UTILITY::Clean_name(n.in[3]);
+         if (!model->IsInitializedTensor(bsn) || model->GetTensorType(bsn) != ETensorType::FLOAT || !model->IsInitializedTensor(bn))
+            throw std::runtime_error("SOFIE ONNX parser: QGemm needs an initializer B with a float scale initializer");
+         const size_t ncols = model->GetTensorShape(bn).back(), nbs = ConvertShapeToLength(model->GetTensorShape(bsn));
+         if (nbs != 1 && nbs != ncols)
+            throw std::runtime_error("SOFIE ONNX parser: QGemm scale of B must have 1 or N elements");
+         const float *bs = static_cast<const float *>(model->GetInitializedTensorData(bsn).get());
+         std::vector<float> mult(ncols);
+         for (size_t c = 0; c < ncols; ++c) {
+            volatile float prod = as * bs[nbs == 1 ? 0 : c];
+            mult[c] = prod / ys;
+         }
+         const std::string mname = n.out[0] + "_requant_scale";
+         model->AddInitializedTensor(mname, ETensorType::FLOAT, {ncols}, mult.data());
+         auto op = std::make_unique<ROperator_QGemm>(n.in[0], n.in[3], n.out[0]);
+         if (!n.in[6].empty())
+            op->SetBias(n.in[6]);
          op->SetRequantize(mname, false);
          model->AddOperator(std::move(op));
       } else if (n.op == "Flatten") {

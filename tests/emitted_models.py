@@ -8,8 +8,9 @@ import subprocess
 
 import numpy as np
 
-from tests import onnx_write as ow
-from tests import util
+from sofie_amd.benchsupport import onnx_write as ow
+from sofie_amd.benchsupport import synthetic as util
+from sofie_amd.benchsupport.models import int8_mlp, int8_cnn  # noqa: F401  (models shared with the benchmark)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 OUT = os.path.join(ROOT, "tests", "emitted")
@@ -36,33 +37,6 @@ def fp32_mlp(batch=64):
     return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 784])], outputs=[(x, np.float32, [batch, 10])], init=init, feeds=[X])
 
 
-def int8_mlp(dims, batch, seed=1100):
-    """benchmark configuration 2 as ONNX operators: per layer QuantizeLinear -> MatMulInteger -> Relu -> DequantizeLinear,
-    per-tensor symmetric scales (zero points 0).  Returns the model and the constants the CPU chain needs."""
-    weights = [util.int8_sym(seed + 1 + l, dims[l] * dims[l + 1]).reshape(dims[l], dims[l + 1]) for l in range(len(dims) - 1)]
-    X = util.normal(seed + 1001, batch * dims[0]).reshape(batch, dims[0])
-    w_scales = [np.float32(1.0 / 127.0)] * len(weights)
-    in_scales = [np.float32(np.abs(X).max() / 127.0)]
-    h = X[:8]
-    for l, w in enumerate(weights[:-1]):
-        q = np.clip(np.rint(h / in_scales[l]), -128, 127).astype(np.int32)   # calibration only: plain numpy
-        acc = np.maximum(q @ w.astype(np.int32), 0)
-        h = acc.astype(np.float32) * np.float32(in_scales[l] * w_scales[l])
-        in_scales.append(np.float32(max(h.max(), 1e-6) / 127.0))
-    init, nodes, x = {}, [], "X"
-    for l, w in enumerate(weights):
-        init["W%d" % l] = w
-        init["sx%d" % l] = np.array(in_scales[l], dtype=np.float32)
-        init["sy%d" % l] = np.array(np.float32(in_scales[l] * w_scales[l]), dtype=np.float32)
-        nodes.append(ow.node("QuantizeLinear", [x, "sx%d" % l], ["Q%d" % l]))
-        nodes.append(ow.node("MatMulInteger", ["Q%d" % l, "W%d" % l], ["A%d" % l]))
-        nodes.append(ow.node("Relu", ["A%d" % l], ["R%d" % l]))
-        nodes.append(ow.node("DequantizeLinear", ["R%d" % l, "sy%d" % l], ["D%d" % l]))
-        x = "D%d" % l
-    return dict(nodes=nodes, inputs=[("X", np.float32, [batch, dims[0]])], outputs=[(x, np.float32, [batch, dims[-1]])], init=init,
-                feeds=[X], consts=dict(weights=weights, w_scales=w_scales, in_scales=in_scales))
-
-
 def fp32_cnn(batch=2):
     """A small fp32 form of benchmark configuration 5: 2 x [Conv3x3 s1 p1 + Relu], GlobalAveragePool, Gemm."""
     init = {"W0": util.normal(5101, 8 * 3 * 9, 0.2).reshape(8, 3, 3, 3), "B0": util.normal(5102, 8, 0.1),
@@ -78,40 +52,6 @@ def fp32_cnn(batch=2):
     nodes[-1] = ow.node("Gemm", ["P", "WF", "BF"], ["Y"], alpha=1.0, beta=1.0)
     X = util.uniform01(5001, batch * 3 * 12 * 12).reshape(batch, 3, 12, 12)
     return dict(nodes=nodes, inputs=[("X", np.float32, [batch, 3, 12, 12])], outputs=[("Y", np.float32, [batch, 10])], init=init, feeds=[X])
-
-
-def int8_cnn(batch=2, hw=12, channels=(3, 64, 128, 256, 256), n_out=10):
-    """benchmark configuration 5 as ONNX operators: QuantizeLinear, then per stage QLinearConv 3x3 s1 p1 (per-channel weight scales,
-    int32 bias: the folded BatchNorm) + Relu, then DequantizeLinear, GlobalAveragePool, Flatten, Gemm.  Returns the model and
-    the constants of the CPU chain (tests.refmodels.int8_cnn_oracle)."""
-    from tests.refmodels import make_int8_cnn
-    m = make_int8_cnn(batch, hw, channels, n_out)
-    init, nodes = {}, []
-    init["zp"] = np.zeros((), dtype=np.int8)
-    xs = np.float32(m["in_scale"])
-    init["sx"] = np.array(xs, dtype=np.float32)
-    nodes.append(ow.node("QuantizeLinear", ["X", "sx", "zp"], ["Q"]))
-    x = "Q"
-    for l, cv in enumerate(m["convs"]):
-        ys = np.float32(0.05 + 0.01 * l)                      # activation scale of this stage's output
-        wsc = (cv["scale"] * ys / xs).astype(np.float32)     # per-channel weight scales
-        cv["scale"] = ((xs * wsc).astype(np.float32) / ys).astype(np.float32)   # what the generator forms: two fp32 roundings
-        init["W%d" % l], init["B%d" % l] = cv["W"], cv["bias"]
-        init["xs%d" % l] = np.array(xs, dtype=np.float32)
-        init["ws%d" % l] = wsc
-        init["ys%d" % l] = np.array(ys, dtype=np.float32)
-        nodes.append(ow.node("QLinearConv", [x, "xs%d" % l, "zp", "W%d" % l, "ws%d" % l, "zp", "ys%d" % l, "zp", "B%d" % l], ["C%d" % l],
-                             kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1]))
-        nodes.append(ow.node("Relu", ["C%d" % l], ["R%d" % l]))
-        x, xs = "R%d" % l, ys
-    m["last_scale"] = xs
-    nodes.append(ow.node("DequantizeLinear", [x, "ys%d" % (len(m["convs"]) - 1), "zp"], ["D"]))
-    nodes.append(ow.node("GlobalAveragePool", ["D"], ["P"]))
-    nodes.append(ow.node("Flatten", ["P"], ["F"], axis=1))
-    init["WF"], init["BF"] = m["fc_w"], m["fc_b"]
-    nodes.append(ow.node("Gemm", ["F", "WF", "BF"], ["Y"], alpha=1.0, beta=1.0))
-    return dict(nodes=nodes, inputs=[("X", np.float32, [batch] + list(m["in_shape"]))], outputs=[("Y", np.float32, [batch, n_out])],
-                init=init, feeds=[m["x"]], consts=m)
 
 
 def conv_batchnorm_relu(batch=2):
@@ -624,78 +564,6 @@ extern "C" int run_model(const char *weights, const float *const *inputs, float 
 # Benchmark harness around the emitted Session of the int8 MLP at its full size: the Session lives across calls, the input
 # stays resident on the device, and the timed region is the reference benchmark's (benchmark/src/BenchmarkEmitter.cxx.in:486-504):
 # N x infer_nosync, one wait, wall clock.
-BENCH_HARNESS = r'''
-#include "%(model)s_GPU_HIP.hxx"
-#include <chrono>
-#include <cstring>
-using Session = SOFIE_%(model)s::Session;
-static void set_error(char *err, int errlen, const char *what)
-{
-   std::strncpy(err, what, errlen - 1);
-   err[errlen - 1] = 0;
-}
-extern "C" void *bench_open(const char *weights, char *err, int errlen)
-{
-   try {
-      return new Session(weights);
-   } catch (const std::exception &e) {
-      set_error(err, errlen, e.what());
-      return nullptr;
-   }
-}
-extern "C" void bench_close(void *h) { delete static_cast<Session *>(h); }
-// uploads one batch into the Session's input region; returns 0, or 1 with the exception text in err
-extern "C" int bench_upload(void *h, const float *x, unsigned long n, char *err, int errlen)
-{
-   try {
-      Session &s = *static_cast<Session *>(h);
-      if (sofie_hip_upload(s.context(), s.device_input_%(input)s(), x, n * sizeof(float)) || sofie_hip_sync(s.context()))
-         throw std::runtime_error(sofie_hip_last_error());
-      return 0;
-   } catch (const std::exception &e) {
-      set_error(err, errlen, e.what());
-      return 1;
-   }
-}
-extern "C" int bench_download(void *h, float *y, unsigned long n, char *err, int errlen)
-{
-   try {
-      Session &s = *static_cast<Session *>(h);
-      if (sofie_hip_download(s.context(), y, s.device_output_%(output)s(), n * sizeof(float)) || sofie_hip_sync(s.context()))
-         throw std::runtime_error(sofie_hip_last_error());
-      return 0;
-   } catch (const std::exception &e) {
-      set_error(err, errlen, e.what());
-      return 1;
-   }
-}
-// `steps` inferences enqueued back to back, one wait: wall-clock milliseconds of the region (and, through *event_ms, what a pair
-// of events on the Session's stream measured); negative on failure
-extern "C" double bench_run(void *h, int steps, float *event_ms, char *err, int errlen)
-{
-   try {
-      Session &s = *static_cast<Session *>(h);
-      s.sync();
-      const auto t0 = std::chrono::steady_clock::now();
-      if (sofie_hip_timer_start(s.context()))
-         throw std::runtime_error(sofie_hip_last_error());
-      for (int i = 0; i < steps; ++i)
-         s.infer_nosync();
-      float ms = 0;
-      if (sofie_hip_timer_stop(s.context(), &ms)) // records the second event and waits for it
-         throw std::runtime_error(sofie_hip_last_error());
-      const auto t1 = std::chrono::steady_clock::now();
-      if (event_ms)
-         *event_ms = ms;
-      return std::chrono::duration<double, std::milli>(t1 - t0).count();
-   } catch (const std::exception &e) {
-      set_error(err, errlen, e.what());
-      return -1.0;
-   }
-}
-'''
-
-
 def _run(cmd):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
@@ -733,72 +601,7 @@ def compile_shared(src, lib):
     return lib
 
 
-BENCH_MODEL = "Config2_int8_MLP"
-
-
-def bench_mlp_spec():
-    """benchmark configuration 2 at its full size: 1024 -> 4096 -> 4096 -> 1024, batch 1024 (same seeds as bench.py's model)."""
-    return int8_mlp([1024, 4096, 4096, 1024], 1024, seed=1100)
-
-
-def build_bench_model():
-    """Emits benchmark configuration 2 at full size with its weights in a safetensors file and compiles the benchmark harness
-    around the emitted Session: what bench.py times and what the full-size parity test runs."""
-    spec = bench_mlp_spec()
-    p = os.path.join(OUT, BENCH_MODEL + ".onnx")
-    ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name=BENCH_MODEL)
-    _run([EMIT, p, OUT, "--safetensors"])
-    src = os.path.join(OUT, BENCH_MODEL + "_bench.cxx")
-    with open(src, "w") as f:
-        f.write(BENCH_HARNESS % dict(model=BENCH_MODEL, input=spec["inputs"][0][0], output=spec["outputs"][0][0]))
-    return compile_shared(src, os.path.join(OUT, "lib%s_bench.so" % BENCH_MODEL))
-
-
-class BenchSession:
-    """The emitted Session of the full-size int8 MLP behind its benchmark harness (ctypes)."""
-
-    def __init__(self):
-        import ctypes as C
-        lib_path = os.path.join(OUT, "lib%s_bench.so" % BENCH_MODEL)
-        if not os.path.exists(lib_path):
-            raise RuntimeError("%s is missing: __graft_entry__.build() emits and compiles it" % lib_path)
-        self.C = C
-        self.lib = C.CDLL(lib_path)
-        self.lib.bench_open.restype = C.c_void_p
-        self.lib.bench_open.argtypes = [C.c_char_p, C.c_char_p, C.c_int]
-        self.lib.bench_close.argtypes = [C.c_void_p]
-        self.lib.bench_upload.argtypes = [C.c_void_p, C.c_void_p, C.c_ulong, C.c_char_p, C.c_int]
-        self.lib.bench_download.argtypes = [C.c_void_p, C.c_void_p, C.c_ulong, C.c_char_p, C.c_int]
-        self.lib.bench_run.restype = C.c_double
-        self.lib.bench_run.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_float), C.c_char_p, C.c_int]
-        self.err = C.create_string_buffer(1024)
-        self.h = self.lib.bench_open(os.path.join(OUT, BENCH_MODEL + "_GPU_HIP.safetensors").encode(), self.err, 1024)
-        if not self.h:
-            raise RuntimeError("emitted Session: " + self.err.value.decode())
-
-    def close(self):
-        if self.h:
-            self.lib.bench_close(self.h)
-            self.h = None
-
-    def upload(self, x):
-        x = np.ascontiguousarray(x, dtype=np.float32)
-        if self.lib.bench_upload(self.h, x.ctypes.data, x.size, self.err, 1024):
-            raise RuntimeError(self.err.value.decode())
-
-    def download(self, shape):
-        y = np.empty(shape, dtype=np.float32)
-        if self.lib.bench_download(self.h, y.ctypes.data, y.size, self.err, 1024):
-            raise RuntimeError(self.err.value.decode())
-        return y
-
-    def run(self, steps):
-        """steps x infer_nosync + one wait: (wall ms, event ms) of the region."""
-        ev = self.C.c_float()
-        wall = self.lib.bench_run(self.h, steps, self.C.byref(ev), self.err, 1024)
-        if wall < 0:
-            raise RuntimeError(self.err.value.decode())
-        return wall, ev.value
+from sofie_amd.benchsupport.emitted import BenchSession, BENCH_MODEL, bench_mlp_spec  # noqa: F401,E402
 
 
 def build_all(jobs=8):
@@ -852,7 +655,6 @@ def build_all(jobs=8):
         f.write(DYNAMIC_HARNESS % dict(model="ApiDynamicFp8Gemm", args="inputs[0]"))
     compile_shared(src, os.path.join(OUT, "libApiDynamicFp8Gemm.so"))
     compile_shared(os.path.join(ROOT, "tests", "harness_custom_memory.cxx"), os.path.join(OUT, "libCustomMemory.so"))
-    build_bench_model()
     return [w[0] for w in work] + list(API_MODELS) + ["ElementwiseChains", "ParseRewrites", "ClassifierHead", "LayerNormBlock", "ReduceBlock", "HardActivations", "IndexingBlock"]
 
 

@@ -227,6 +227,28 @@ def test_qlinear_matmul_and_conv_integer_become_one_launch_each(emitted):
     assert "sofie_hip_dequantize_linear_i32(" in body and "sofie_hip_unary_f32" not in body
 
 
+def test_qgemm_with_bias_and_relu_is_one_launch_on_an_int8_input(tmp_path):
+    """The contrib operator QGemm (int8 graph input, int32 bias, per-column scales) followed by Relu: one sofie_hip_gemm_i8 with the
+    bias on the accumulator and the Relu on the requantised output; the Session takes and returns int8."""
+    from sofie_amd.benchsupport import models
+    spec = models.int8_gemm_requant(64)
+    p = str(tmp_path / "QGemmSmall.onnx")
+    ow.write(p, spec["nodes"], spec["inputs"], spec["outputs"], spec["init"], name="QGemmSmall")
+    em._run([em.EMIT, p, str(tmp_path)])
+    txt = open(str(tmp_path / "QGemmSmall_GPU_HIP.hxx")).read()
+    body = ops_body(txt)
+    assert body.count("sofie_hip_gemm_i8(") == 1 and "sofie_hip_unary" not in body
+    assert "d.bias = tensor_bias; d.scale = tensor_P_requant_scale;" in body
+    assert "d.relu_acc = 0; d.relu_out = 1; d.out = SOFIE_I8OUT_I8; d.Y = tensor_Y;" in body
+    assert re.search(r"std::vector<int8_t> infer\(int8_t const ?\* ?host_A\)", txt)
+    assert "sofie_hip_transpose_i8(fCtx, packed_B, tensor_B, 64, 64, 0, 0)" in txt
+    # forms the reference's parser would refuse by name are refused here too
+    bad = dict(spec, nodes=[ow.node("QGemm", ["A", "sa", "zp", "B", "sb", "zp", "bias", "sy", "zp"], ["P"], alpha=0.5), spec["nodes"][1]])
+    ow.write(p, bad["nodes"], bad["inputs"], bad["outputs"], bad["init"], name="QGemmSmall")
+    with pytest.raises(RuntimeError, match="alpha = 1"):
+        em._run([em.EMIT, p, str(tmp_path)])
+
+
 def test_run_time_batch_signatures_follow_the_reference_convention(emitted):
     txt = read(emitted, "DynamicLinear")
     # the constructor takes the maximum after the weight file, infer takes the value first (core/src/RModel.cxx:1537-1547, 1375-1395)

@@ -91,8 +91,62 @@ def test_emitted_int8_mlp_at_full_size_on_sampled_rows(rt):
     assert np.array_equal(got[rows].view(np.uint32), h.view(np.uint32))
     assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
     assert np.abs(h).max() > 0 and (got > 0).mean() > 0.1
-    txt = open(os.path.join(em.OUT, em.BENCH_MODEL + "_GPU_HIP.hxx")).read()
+    from sofie_amd.benchsupport import emitted as be
+    txt = open(os.path.join(be.OUT, be.BENCH_MODEL + "_GPU_HIP.hxx")).read()
     assert txt.count("sofie_hip_gemm_i8(") == 3 and "SOFIE_I8OUT_I8_DQQ" in txt and "safetensors" in txt
+
+
+def test_emitted_full_size_int8_cnn_sampled_images(rt):
+    """benchmark configuration 5 at its full size (batch 256, 64 x 64 images) through the Session the generator emits, the one the
+    benchmark times.  The images of a batch are independent, so the unfused CPU chain runs on a sample of them: the int8
+    stages are bit-exact, the fp32 tail (average, Gemm) is held to 1e-5."""
+    from oracle.chains import int8_cnn_oracle
+    from sofie_amd.benchsupport import emitted as be
+    spec = be.bench_cnn_spec()
+    m, X = spec["consts"], spec["feeds"][0]
+    sample = [0, 1, 85, 170, 254, 255]
+    want = int8_cnn_oracle(m, np.ascontiguousarray(X[sample]))
+    print("emitted Config5_int8_CNN (full size)", flush=True)
+    s = be.BenchSession(be.CNN_MODEL)
+    try:
+        s.upload(X)
+        s.run(1)
+        got = s.download((256, 10))
+        s.run(2)
+        again = s.download((256, 10))
+    finally:
+        s.close()
+    assert np.abs(got[sample] - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+    txt = open(os.path.join(be.OUT, be.CNN_MODEL + "_GPU_HIP.hxx")).read()
+    assert txt.count("sofie_hip_conv_i8(") == 4 and "planes summed for the GlobalAveragePool" in txt
+
+
+def test_emitted_int8_gemm_8192_sampled_rows_and_columns(rt):
+    """benchmark configuration 3 at M = N = K = 8192 as a one-operator model (QGemm + Relu parsed from ONNX, B re-laid out once
+    in the constructor): the emitted Session's output on sampled full rows and columns, bit-exact against the oracle."""
+    from oracle import binding as ob
+    from sofie_amd.benchsupport import emitted as be
+    spec = be.bench_gemm_spec()
+    c, A = spec["consts"], spec["feeds"][0]
+    n = 8192
+    print("emitted Config3_int8_GEMM_8192", flush=True)
+    s = be.BenchSession(be.GEMM_MODEL)
+    try:
+        s.upload(A)
+        s.run(1)
+        got = s.download((n, n), np.int8)
+    finally:
+        s.close()
+    rows = np.array([0, 1, 255, 256, 4095, 4096, 8191, 777])
+    want = ob.gemm_i8(np.ascontiguousarray(A[rows]), c["Bt"], M=len(rows), N=n, K=n, transB=1, omp=True, bias=c["bias"], scale=c["scale"],
+                      relu_out=1, out=2)
+    assert np.array_equal(got[rows], want)
+    cols = np.array([0, 63, 64, 4097, 8191])
+    want_c = ob.gemm_i8(A, np.ascontiguousarray(c["Bt"][cols]), M=n, N=len(cols), K=n, transB=1, omp=True, bias=c["bias"][cols],
+                        scale=c["scale"][cols], relu_out=1, out=2)
+    assert np.array_equal(got[:, cols], want_c)
+    assert got.max() == 127 and (got == 0).mean() > 0.3
 
 
 def test_emitted_int8_cnn_matches_cpu_chain(rt):

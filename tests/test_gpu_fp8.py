@@ -1,11 +1,11 @@
 """FP8 (e4m3fn) GEMM and quantiser through the C-ABI.
 
-Stated per-element bound of the GEMM.  The matrix core adds the 64 products of one K-step in a
-fixed-point tree aligned to the largest term, not in IEEE fp32: measured on MI355X the error of a single
-step reaches 2^-16 of sum_k |a_k b_k| and grows more slowly than K after that.  The tests hold the kernel to
-   |acc - exact| <= 2^-14 * sum_k |a_k b_k|         (exact = float64 sum of the exact products)
-which is four times the worst case seen, and then allow the fp32 rounding of scale, bias and activation
-and one bf16 rounding (relative 2^-9) for bf16 output."""
+Stated per-element bound of the GEMM (include/sofie_hip.h, at sofie_hip_gemm_fp8; evaluated by oracle.binding.fp8_gemm_bound).
+The matrix core adds the 64 products of one K-step in a fixed-point tree aligned to the largest term, not in IEEE fp32:
+measured on MI355X the error of a single step reaches 2^-16 of S = sum_k |a_k b_k| and grows more slowly than K after that.
+The tests hold every checked element to
+   |Y - y0| <= L (2^-14 S scale + 2^-22 (|v0| + |bias|)) + [GELU: 1e-6 |v0|] + 2^-21 |y0| + [bf16: half an ulp of bf16]
+with y0 (v0) the result (the value before the activation) of exact accumulation and L the activation's largest slope."""
 import ctypes as C
 
 import numpy as np
@@ -79,9 +79,7 @@ def test_fp32_output_within_accumulation_bound(rt, M, N, K, transB):
     B = Bt if transB else np.ascontiguousarray(Bt.T)
     scale = np.float32(sa * sb)
     got = run_fp8(rt, A, B, M, N, K, transB=transB, scale=scale, out=1)
-    want, abs_sum = ob.gemm_fp8(A, B, M=M, N=N, K=K, transB=transB, scale=scale, out=1, want_abs_sum=True, omp=True)
-    bound = 2.0 ** -14 * abs_sum.astype(np.float64) * float(scale) + 2.0 ** -22 * np.abs(want) + 1e-30
-    assert np.all(np.abs(got.astype(np.float64) - want) <= bound)
+    assert ob.fp8_gemm_bound_excess(got, A, Bt, None, scale, R.ACT_NONE, bf16=False) <= 0.0
 
 
 def test_exact_cases(rt):
@@ -105,22 +103,12 @@ def test_bf16_output_with_bias_and_activation(rt, act):
     bias = util.normal(4003, N)
     scale = np.float32(sa * sb)
     got = ob.bf16_bits_to_f32(run_fp8(rt, A, Bt, M, N, K, bias=bias, scale=scale, act=act, out=0))
-    want, abs_sum = ob.gemm_fp8(A, Bt, M=M, N=N, K=K, transB=1, bias=bias, scale=scale, act=act, out=1, want_abs_sum=True)
-    # accumulation bound propagated through bias (one fp32 rounding) and an activation with slope <= 1.13,
-    # plus half an ulp of bf16 (2^-9 relative) for the final rounding
-    acc_err = 2.0 ** -14 * abs_sum.astype(np.float64) * float(scale)
-    bound = 1.2 * acc_err + 2.0 ** -8 * np.abs(want) + 1e-6
-    assert np.all(np.abs(got.astype(np.float64) - want) <= bound)
+    assert ob.fp8_gemm_bound_excess(got, A, Bt, bias, scale, act, bf16=True) <= 0.0
 
 
 def check_fp8_against_oracle(got_f32, A, Bt, bias, scale, act, bf16):
-    """|got - oracle| within the accumulation bound (propagated through bias and an activation of slope <= 1.13) plus the
-    rounding of the output type."""
-    M, K = A.shape
-    N = Bt.shape[0]
-    want, abs_sum = ob.gemm_fp8(A, Bt, M=M, N=N, K=K, transB=1, bias=bias, scale=scale, act=act, out=1, want_abs_sum=True, omp=True)
-    acc_err = 2.0 ** -14 * abs_sum.astype(np.float64) * float(scale)
-    bound = 1.2 * acc_err + (2.0 ** -8 if bf16 else 2.0 ** -21) * np.abs(want) + 1e-6
+    """|got - oracle| within the bound stated for sofie_hip_gemm_fp8; returns the oracle's values."""
+    want, bound = ob.fp8_gemm_bound(A, Bt, bias, scale, act, bf16)
     err = np.abs(got_f32.astype(np.float64) - want)
     assert np.all(err <= bound), "worst excess %g at %s" % ((err - bound).max(), np.unravel_index(np.argmax(err - bound), err.shape))
     return want
