@@ -22,7 +22,11 @@
 extern "C" {
 #endif
 
-#define SOFIE_HIP_ABI_VERSION 2
+/* Version of this interface: raised whenever an entry point is added, removed or changes its meaning (3: the kernel-choice
+ * options are read from the environment once, when a context is created, and changed through sofie_hip_ctx_set_option; entry
+ * points added for 3-D operators and for callers that cannot allocate).  An emitted Session compares the value it was compiled
+ * with against sofie_hip_abi_version() of the library it finds at run time, and refuses to run on a different one. */
+#define SOFIE_HIP_ABI_VERSION 3
 
 typedef struct sofie_hip_ctx sofie_hip_ctx;
 

@@ -148,6 +148,7 @@ struct F8Epilogue {
    }
    // row-major output with 16-byte aligned rows (what the register tile store handles)
    bool stores_plain_rows() const { return stage_ok != 0; }
+   int elements_per_16_bytes() const { return out == SOFIE_F8OUT_F32 ? 4 : 8; }
    // v = acc*scale + bias[n]; activation in fp32; then fp32 or bf16 (round to nearest even)
    template <int MODE, int C>
    __device__ __forceinline__ void pack4(const col_params<C> &p, int q, float a0, float a1, float a2, float a3, uint32_t *w) const

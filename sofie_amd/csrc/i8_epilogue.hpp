@@ -102,6 +102,8 @@ struct I8Epilogue {
    {
       return stage_ok != 0 && nchw_ohw == 0 && rows_per_plane == 0 && q_scale_saturates();
    }
+   // output elements per 16 bytes (the unit of the vector stores)
+   int elements_per_16_bytes() const { return (out == SOFIE_I8OUT_I32 || out == SOFIE_I8OUT_F32) ? 4 : 16; }
    bool q_scale_saturates() const { return out != SOFIE_I8OUT_I8_DQQ || (q_scale > -1e30f && q_scale < 1e30f); }
    // plane sums (of int8 results) whose planes are made of whole groups of `rows` GEMM rows
    bool sums_rows_of_whole_wave_tiles(int rows) const

@@ -18,7 +18,7 @@ static int launch_mfma8_best(const LaunchCfg &lc, const int8_t *A, const int8_t 
    const bool k128 = (K % 128 == 0);
    if constexpr (MMA::KSTEP * 2 <= 64) {
       // Large products that divide into whole 256 x 256 tiles: the persistent kernel (512 asks for it by force)
-      if ((force_tile == 512 || (!force_tile && variant == 0 && tile == 256)) && mfma8_persist_applies(A, Bt, M, N, K, lda, ldb) &&
+      if ((force_tile == 512 || (!force_tile && variant == 0 && tile == 256)) && mfma8_persist_applies(A, Bt, M, N, K, lda, ldb, ep.elements_per_16_bytes()) &&
           ep.stores_plain_rows())
          return launch_mfma8_persist<MfmaI8x16, EPI>(lc, A, Bt, M, N, K, lda, ldb, ep);
       // Short reductions over many tiles: the 256 x 128 tile with a ring of three slabs fits twice on a CU, and one
@@ -32,7 +32,7 @@ static int launch_mfma8_best(const LaunchCfg &lc, const int8_t *A, const int8_t 
       // two K-steps per slab are the minimum: a 64-byte K-step needs 128-byte slabs
       if (!k128)
          return launch_mfma8_auto<MMA, EPI>(lc, A, Bt, M, N, K, lda, ldb, ep);
-      if ((force_tile == 512 || (!force_tile && variant == 0 && tile == 256)) && mfma8_persist_applies(A, Bt, M, N, K, lda, ldb) &&
+      if ((force_tile == 512 || (!force_tile && variant == 0 && tile == 256)) && mfma8_persist_applies(A, Bt, M, N, K, lda, ldb, ep.elements_per_16_bytes()) &&
           ep.stores_plain_rows())
          return launch_mfma8_persist<MMA, EPI>(lc, A, Bt, M, N, K, lda, ldb, ep);
       switch (tile) {
@@ -88,7 +88,8 @@ static int launch_mfma8_conv(const LaunchCfg &lc, const ConvRows &a, int Cg, con
                                                              : 64;
    // Whole 256 x 256 tiles, at least one per CU, and a store the register path handles (NHWC rows, or the plane sums of
    // planes that hold whole wave tiles): the persistent kernel.  512 asks for it by force.
-   if ((force_tile == 512 || (!force_tile && lc.variant == 0 && tiles(256, 256) >= 256)) && mfma8_persist_conv_applies(a, Wp, M, N, K) &&
+   if ((force_tile == 512 || (!force_tile && lc.variant == 0 && tiles(256, 256) >= 256)) &&
+       mfma8_persist_conv_applies(a, Wp, M, N, K, ep.elements_per_16_bytes(), !ep.stores_plain_rows()) &&
        (ep.stores_plain_rows() || ep.sums_rows_of_whole_wave_tiles(128)))
       return launch_mfma8_persist_src<MfmaI8x16, EPI, PersistConvRows>(lc, PersistConvRows{a}, Wp, M, N, K, K, ep);
    if (tile == 512)

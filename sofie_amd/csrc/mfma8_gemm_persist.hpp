@@ -1,4 +1,4 @@
-// Persistent tile loop of the int8 / FP8 GEMM for large shapes that divide evenly into 256 x 256 tiles.
+// Persistent tile loop of the int8 / FP8 GEMM for large shapes, walked in 256 x 256 tiles.
 //
 // One workgroup of EIGHT waves per CU (two per SIMD, 256 registers each) walks a list of output tiles; the K loop runs
 // straight through the tile boundaries:
@@ -291,8 +291,8 @@ struct PersistConvRows {
 };
 
 template <class MMA, class EPI, class ASRC>
-__global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const int8_t *__restrict__ Bt, int ldb, int K, EPI ep, int tiles_m,
-                                                                  int tiles_n, int sw)
+__global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const int8_t *__restrict__ Bt, int ldb, int M, int N, int K, EPI ep,
+                                                                  int tiles_m, int tiles_n, int sw)
 {
    constexpr int BM = 256, BN = 256, BK = 64, STAGES = 5, NW = 8, WAVES_N = 4;
    constexpr int R = MMA::ROWS;
@@ -342,8 +342,11 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const i
    auto tile_origin = [&](int it, int &m0, int &n0) {
       int tm, tn;
       tile_of_block((it < my_tiles ? it : my_tiles - 1) * nwg + bid, ntiles, tiles_m, tiles_n, sw, tm, tn);
-      m0 = tm * BM;
-      n0 = tn * BN;
+      // Sizes that are not multiples of the tile: the last tile of a row or column of tiles is moved back until it ends at
+      // the edge.  It then overlaps its neighbour, and both compute (and store) the rows or columns they share: the same
+      // values twice, instead of loads and stores that would have to be predicated lane by lane.
+      m0 = min(tm * BM, M - BM);
+      n0 = min(tn * BN, N - BN);
    };
    auto load_origin = [&](int m0, int n0, typename ASRC::tile_state &ta, const int8_t *&pb) {
       if constexpr (ASRC::kConv) {
@@ -536,20 +539,23 @@ __global__ __launch_bounds__(512) void mfma8_gemm_persist_kernel(ASRC A, const i
    wait_vmcnt<0>();
 }
 
-// Whether the persistent kernel takes this product: whole 256 x 256 tiles, K a multiple of 128, 16-byte aligned rows, at
-// least as many tiles as CUs would otherwise idle.
-inline bool mfma8_persist_applies(const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb)
+// Whether the persistent kernel takes this product: at least one whole 256 x 256 tile in each direction (a last tile that
+// does not fit is moved back to end at the edge, see tile_origin in the kernel), K a multiple of 128, 16-byte aligned rows.
+// `n_align` = elements per 16 bytes of output: the moved tile must start on a 16-byte boundary of the output rows.
+inline bool mfma8_persist_applies(const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, int n_align)
 {
-   return M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0 && K >= 384 && K % 128 == 0 && lda % 16 == 0 && ldb % 16 == 0 &&
-          (((uintptr_t)A | (uintptr_t)Bt) & 15) == 0 && (long long)(M / 256) * (N / 256) <= 0x7fffffLL &&
+   return M >= 256 && N >= 256 && N % n_align == 0 && K >= 384 && K % 128 == 0 && lda % 16 == 0 && ldb % 16 == 0 &&
+          (((uintptr_t)A | (uintptr_t)Bt) & 15) == 0 && (long long)((M + 255) / 256) * ((N + 255) / 256) <= 0x7fffffLL &&
           (size_t)256 * (size_t)(lda > ldb ? lda : ldb) < 0xffffffffULL;
 }
 // The same for a convolution read through ConvRows (whose own conditions the caller has checked: channels per group a power
-// of two >= 64, 32-bit offsets): one bit per tap and pixel must fit the lane's mask.
-inline bool mfma8_persist_conv_applies(const ConvRows &a, const int8_t *Wp, int M, int N, int K)
+// of two >= 64, 32-bit offsets): one bit per tap and pixel must fit the lane's mask.  `whole_tiles`: the store adds results up
+// (plane sums), so no output may be computed twice.
+inline bool mfma8_persist_conv_applies(const ConvRows &a, const int8_t *Wp, int M, int N, int K, int n_align, bool whole_tiles)
 {
-   return M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0 && K >= 384 && K % 128 == 0 && a.ntaps <= 16 && (((uintptr_t)a.X | (uintptr_t)Wp) & 15) == 0 &&
-          (long long)(M / 256) * (N / 256) <= 0x7fffffLL && (size_t)256 * (size_t)K < 0xffffffffULL;
+   return M >= 256 && N >= 256 && N % n_align == 0 && (!whole_tiles || (M % 256 == 0 && N % 256 == 0)) && K >= 384 && K % 128 == 0 && a.ntaps <= 16 &&
+          (((uintptr_t)a.X | (uintptr_t)Wp) & 15) == 0 && (long long)((M + 255) / 256) * ((N + 255) / 256) <= 0x7fffffLL &&
+          (size_t)256 * (size_t)K < 0xffffffffULL;
 }
 
 inline int cu_count_of_current_device(int &ncu)
@@ -569,7 +575,7 @@ inline int cu_count_of_current_device(int &ncu)
 template <class MMA, class EPI, class ASRC>
 static int launch_mfma8_persist_src(const LaunchCfg &lc, const ASRC &a, const int8_t *Bt, int M, int N, int K, int ldb, const EPI &ep)
 {
-   const int tiles_m = M / 256, tiles_n = N / 256;
+   const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
    const int ntiles = tiles_m * tiles_n;
    constexpr size_t smem = (size_t)5 * 512 * 64;
    static_assert(smem <= 160 * 1024, "LDS ring larger than the CU's LDS");
@@ -581,7 +587,7 @@ static int launch_mfma8_persist_src(const LaunchCfg &lc, const ASRC &a, const in
    if (int st = cu_count_of_current_device(ncu))
       return st;
    const int grid = ntiles < ncu ? ntiles : ncu;
-   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, lc.stream, a, Bt, ldb, K, ep, tiles_m, tiles_n, lc.swizzle);
+   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, lc.stream, a, Bt, ldb, M, N, K, ep, tiles_m, tiles_n, lc.swizzle);
    return launch_status("mfma8_gemm_persist_kernel");
 }
 

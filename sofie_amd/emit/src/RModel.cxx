@@ -997,6 +997,9 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    }
    if (customMemory)
       gc << "      if (!fProvider.alloc)\n         throw std::runtime_error(\"SOFIE HIP Session: the memory provider has no alloc function\");\n";
+   gc << "      if (sofie_hip_abi_version() != SOFIE_HIP_ABI_VERSION)\n"
+      << "         throw std::runtime_error(\"SOFIE HIP: this Session was generated for version \" + std::to_string(SOFIE_HIP_ABI_VERSION) +\n"
+      << "                                  \" of the runtime library's interface, the library loaded has version \" + std::to_string(sofie_hip_abi_version()));\n";
    gc << "      detail::Check(sofie_hip_ctx_create(&fCtx, device, " << (externalStream ? "stream" : "nullptr") << "), \"Session\");\n";
    gc << "      try {\n";
    if (customMemory) {

@@ -221,6 +221,26 @@ def test_persistent_kernel_forced_on_small_shapes(rt, opt, out, relu_acc, relu_o
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
 
 
+@pytest.mark.parametrize("out,relu_acc,relu_out,M,N,K", [(R.I8OUT_I8, 0, 1, 300, 528, 384), (R.I8OUT_I8, 0, 0, 1000, 272, 512), (R.I8OUT_I8_DQQ, 1, 0, 257, 256, 640),
+                                                         (R.I8OUT_I32, 0, 0, 260, 516, 384), (R.I8OUT_F32, 1, 0, 511, 260, 384),
+                                                         (R.I8OUT_I8, 0, 1, 2000, 8208, 512)])
+def test_persistent_kernel_on_sizes_that_are_not_multiples_of_its_tile(rt, opt, out, relu_acc, relu_out, M, N, K):
+    """M and N that do not divide into 256 x 256 tiles: the last tile of a row / column of tiles is moved back to end at the edge
+    and overlaps its neighbour (both store the shared outputs, with the same values).  N must keep the moved tile on a 16-byte
+    boundary of the output rows (16 elements for 1-byte outputs, 4 for 4-byte ones).  2000 x 8208: 8 x 33 = 264 tiles, more
+    than compute units, by the heuristic's own choice; the others are forced."""
+    A = util.int8_sym(91 + M, M * K).reshape(M, K)
+    Bt = util.int8_sym(92 + N, N * K).reshape(N, K)
+    bias = util.int32_range(93, N, -(1 << 15), 1 << 15)
+    scale = ((0.5 + util.uniform01(94, N)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    kw = dict(bias=bias, scale=scale, q_scale=np.float32(0.041), relu_acc=relu_acc, relu_out=relu_out, out=out)
+    if M < 2000:
+        opt("i8_tile", 512)
+    got = run_gemm(rt, A, Bt, M, N, K, transB=1, **kw)
+    want = ob.gemm_i8(A, Bt, M=M, N=N, K=K, transB=1, omp=True, **kw)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
 @pytest.mark.parametrize("tile", [0, 64, 512])
 @pytest.mark.parametrize("out,relu_acc,relu_out", [(R.I8OUT_I8, 0, 0), (R.I8OUT_I8, 0, 1), (R.I8OUT_I8, 1, 0), (R.I8OUT_I8_DQQ, 0, 0),
                                                    (R.I8OUT_I8_DQQ, 1, 0), (R.I8OUT_F32, 0, 1), (R.I8OUT_F32, 0, 0)])
