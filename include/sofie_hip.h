@@ -255,12 +255,15 @@ int sofie_hip_transpose_i8(sofie_hip_ctx *ctx, int8_t *dst, const int8_t *src, i
  * bit-defined; it is held to the exactly accumulated one.  With S = sum_k |a_k b_k| (exact products), v0 the value before
  * the activation and y0 the result when the sum is exact and every later step is one correctly rounded fp32 operation:
  *   |Y - y0| <= L * (2^-14 * S * scale  +  2^-22 * (|v0| + |bias[n]|))    accumulation; roundings of the scaling and the bias
- *             + 1e-6 * |v0|                                               SOFIE_ACT_GELU only, see below
+ *             + g * |v0|                                                  SOFIE_ACT_GELU only: g = 1e-6 (fp32 output), 8e-5 (bf16 output)
  *             + 2^-21 * |y0|                                              the activation's own fp32 evaluation
  *             + half an ulp of bf16 at the result (at most 2^-8 * |Y|)    SOFIE_F8OUT_BF16 only
  * L = 1.13 for the two GELU forms (the largest slope of GELU), 1 otherwise.  SOFIE_ACT_GELU is evaluated in the store as
- * v * Phi(v) with Phi from the rational approximation 7.1.26 of Abramowitz and Stegun (|error of erfc| <= 1.5e-7), the
- * hardware's reciprocal and 2^x (one ulp each) and seven more fp32 operations: |error of Phi| <= 1e-6, hence the term above.
+ * v * Phi(v).  For fp32 output Phi comes from the rational approximation 7.1.26 of Abramowitz and Stegun (|error of erfc| <=
+ * 1.5e-7), the hardware's reciprocal and 2^x (one ulp each) and seven more fp32 operations: |error of Phi| <= 1e-6.  For bf16
+ * output, whose half ulp is 2^-9 .. 2^-8 of the result, Phi - 1/2 is an odd polynomial of degree 15 in v clamped to [-4, 4]:
+ * |error of Phi| <= 8e-5, a fiftieth of that half ulp, at half the instructions (the store of a tile is time the matrix cores
+ * stand idle).
  * 2^-14 is four times the largest accumulation error measured (about 2^-16 * S per 64-element K step, not growing with K). */
 enum { SOFIE_F8OUT_BF16 = 0, SOFIE_F8OUT_F32 = 1 };
 typedef struct sofie_gemm_fp8_desc {

@@ -433,7 +433,7 @@ def fp8_gemm_bound(A, Bt, bias, scale, act, bf16, omp=True):
     lip = 1.13 if act in (4, 5) else 1.0     # SOFIE_ACT_GELU, SOFIE_ACT_GELU_TANH
     bound = lip * (2.0 ** -14 * S.astype(np.float64) * float(scale) + 2.0 ** -22 * (v0 + b[None, :]))
     if act == 4:
-        bound = bound + 1e-6 * v0
+        bound = bound + (8e-5 if bf16 else 1e-6) * v0
     bound = bound + 2.0 ** -21 * np.abs(y0)
     if bf16:
         # half an ulp of bf16 (8 significant bits) at the largest magnitude the result may have
