@@ -30,7 +30,8 @@ import numpy as np
 
 INT8_PEAK = 5.0e15  # MI355X dense int8 MFMA peak, op/s
 HBM_PEAK = 8.0e12
-CLOCK_WARM_MS = 60.0   # untimed load in front of every timed region
+CLOCK_WARM_MS = 60.0   # untimed load in front of every timed region (--clock-warm-ms)
+REGION_MS = 20.0       # length a timed region of the sweeps is sized to (--region-ms)
 PROFILE_OF_DOMINANT_KERNEL = os.path.join(ROOT, "profiles", "mfma8_gemm_dma_128x128_int8_mlp_batch1024.md")
 
 
@@ -69,12 +70,12 @@ def time_region(rt, fn, reps):
 def region_launches(rt, fn, least):
     """Launches per timed region: at least `least`, and enough for a region of about 20 ms."""
     ms, _ = time_region(rt, fn, least)
-    return max(least, min(5000, int(20.0 / max(ms / least, 1e-4)) + 1))
+    return max(least, min(5000, int(REGION_MS / max(ms / least, 1e-4)) + 1))
 
 
 def warm_clock(rt, fn, per_call_ms):
     """CLOCK_WARM_MS of the same launches, untimed, straight in front of a timed region."""
-    n = max(1, min(20000, int(CLOCK_WARM_MS / max(per_call_ms, 1e-4)) + 1))
+    n = min(20000, int(CLOCK_WARM_MS / max(per_call_ms, 1e-4)) + 1) if CLOCK_WARM_MS > 0 else 0
     for _ in range(n):
         fn()
     rt.sync()
@@ -141,7 +142,8 @@ def emitted_gemm_leg(steps=20):
     try:
         s.upload(A)
         _, ev = s.run(steps)
-        s.run(max(steps, int(CLOCK_WARM_MS / max(ev / steps, 1e-3)) + 1))   # the clock warm-up
+        if CLOCK_WARM_MS > 0:
+            s.run(max(steps, int(CLOCK_WARM_MS / max(ev / steps, 1e-3)) + 1))   # the clock warm-up
         regions = sorted(s.run(steps)[1] for _ in range(5))
         rows = np.array([0, 1, 255, 256, n // 2, n - 1])
         got = s.download((n, n), np.int8)[rows]
@@ -274,7 +276,8 @@ def int8_cnn_leg(steps=20, parity=True):
     try:
         s.upload(x)
         _, ev = s.run(steps)
-        s.run(max(steps, int(CLOCK_WARM_MS / max(ev / steps, 1e-3)) + 1))   # the clock warm-up
+        if CLOCK_WARM_MS > 0:
+            s.run(max(steps, int(CLOCK_WARM_MS / max(ev / steps, 1e-3)) + 1))   # the clock warm-up
         regions = sorted(s.run(steps)[1] for _ in range(5))
         got = s.download((batch, 10))
     finally:
@@ -372,12 +375,17 @@ def main():
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--cpu-rows", type=int, default=1024, help="batch rows the CPU baseline runs (1024 = the whole batch)")
+    ap.add_argument("--clock-warm-ms", type=float, default=CLOCK_WARM_MS,
+                    help="untimed load in front of every timed region; 0 for profiling runs, which count dispatches and not time")
+    ap.add_argument("--region-ms", type=float, default=REGION_MS, help="length the timed regions of the sweeps are sized to")
     ap.add_argument("--no-sweep", action="store_true", help="skip the stand-alone GEMM sweep (profiling runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device-to-device copies: a kernel of known traffic that scales the FETCH_SIZE / "
                          "WRITE_SIZE counters of a profiling run")
     args = ap.parse_args()
+    global CLOCK_WARM_MS, REGION_MS
+    CLOCK_WARM_MS, REGION_MS = max(0.0, args.clock_warm_ms), max(0.1, args.region_ms)
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (the path is data-parallel over the batch; "
               "no multi-GPU figure is produced). Use --gpus 1.", file=sys.stderr)
@@ -394,7 +402,8 @@ def main():
     emitted.upload(x)
     w_wall, _ = emitted.run(max(args.warmup, 1))
     # the clock warm-up: at least CLOCK_WARM_MS of the same inferences straight in front of the timed regions
-    emitted.run(int(CLOCK_WARM_MS / max(w_wall / max(args.warmup, 1), 1e-3)) + 1)
+    if CLOCK_WARM_MS > 0:
+        emitted.run(int(CLOCK_WARM_MS / max(w_wall / max(args.warmup, 1), 1e-3)) + 1)
     regions = [emitted.run(args.steps) for _ in range(5)]   # (wall ms, event ms) of K x infer_nosync + one wait
     walls = sorted(w for w, _ in regions)
     wall = walls[2]                                         # the median region is the one reported

@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 def run_chain(rt, X, layers, alias=None):
     """layers: dicts with W (stored as given), transB, bias (or None), bias_mode, act, act_alpha, alpha, post (list or None),
     residual (array of the output's shape or None).  alias = {l: m}: layer l writes into the buffer of layer m < l (same
-    size).  Returns the device results of every layer."""
+    size, or the first floats of it when the shapes differ).  Returns the device results of every layer."""
     n = len(layers)
     descs = (R.GemmF32Desc * n)()
     keep, outs = [], []
@@ -27,7 +27,12 @@ def run_chain(rt, X, layers, alias=None):
         dW = util.to_dev(L["W"])
         dC = None if L.get("bias") is None else util.to_dev(L["bias"])
         dR = None if L.get("residual") is None else util.to_dev(L["residual"])
-        dY = outs[alias[l]] if alias and l in alias else util.dev_empty((M, N), np.float32)
+        if alias and l in alias:
+            dY = outs[alias[l]]
+            if tuple(dY.shape) != (M, N):      # another shape: the first M * N floats of that buffer
+                dY = dY.view(-1)[:M * N].view(M, N)
+        else:
+            dY = util.dev_empty((M, N), np.float32)
         d = descs[l]
         d.M, d.N, d.K, d.transA, d.transB = M, N, K, 0, int(L["transB"])
         d.alpha, d.beta, d.batch = L.get("alpha", 1.0), L.get("beta", 1.0), 1
@@ -134,6 +139,20 @@ def test_layers_that_share_memory_run_layer_by_layer(rt):
     want, mags = oracle_chain(X, layers)
     check(got[1:], want[1:], mags[1:])
     assert np.array_equal(got[0], got[2])  # the shared buffer holds layer 2's result
+
+
+@pytest.mark.parametrize("fused", [-1, 1])
+def test_layers_that_share_memory_in_another_shape_run_layer_by_layer(rt, opt, fused):
+    """Layer 2 (64 columns) written into the first half of the buffer of layer 0 (128 columns): the rows of the two tensors do not
+    coincide, so one launch would let a workgroup's layer-2 rows overwrite layer-0 rows that another workgroup still has to
+    read.  The entry point must launch layer by layer, by its own choice (-1) and when the one-launch form is asked for (1)."""
+    opt("f32_chain", fused)
+    M = 64
+    X = util.normal(970, M * 32).reshape(M, 32)
+    layers = mlp_layers([32, 128, 64, 64], 971, act=R.ACT_TANH)
+    got = run_chain(rt, X, layers, alias={2: 0})
+    want, mags = oracle_chain(X, layers)
+    check(got[1:], want[1:], mags[1:])
 
 
 def test_chain_of_one_wide_rows_and_refusals(rt):
