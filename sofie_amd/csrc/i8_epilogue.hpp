@@ -102,6 +102,8 @@ struct I8Epilogue {
    {
       return stage_ok != 0 && nchw_ohw == 0 && rows_per_plane == 0 && q_scale_saturates();
    }
+   // 1-byte elements stored as rows: the store from registers then issues one 16-byte store per lane and 16-row block
+   __device__ __forceinline__ bool stores_one_byte_rows() const { return out != SOFIE_I8OUT_I32 && out != SOFIE_I8OUT_F32 && rows_per_plane == 0; }
    // output elements per 16 bytes (the unit of the vector stores)
    int elements_per_16_bytes() const { return (out == SOFIE_I8OUT_I32 || out == SOFIE_I8OUT_F32) ? 4 : 16; }
    bool q_scale_saturates() const { return out != SOFIE_I8OUT_I8_DQQ || (q_scale > -1e30f && q_scale < 1e30f); }

@@ -1,6 +1,6 @@
 // Kernel choice for the int8 / FP8 GEMM and the int8 convolution: which tile, which pipelined kernel, or the general one.
 #pragma once
-#include "mfma8_gemm_persist.hpp"
+#include "conv_i8_resident.hpp"
 
 namespace sofie_hip {
 
@@ -86,13 +86,18 @@ static int launch_mfma8_conv(const LaunchCfg &lc, const ConvRows &a, int Cg, con
              : (N >= 128 && tiles(256, 128) >= 512)          ? 258
              : (N > 64 && tiles(128, 128) >= 192)            ? 128
                                                              : 64;
+   // A small 3 x 3 layer (64 channels in, 128 out): weights resident in LDS, each tile's pixels fetched once with their halo.
+   // 576 asks for it by force (and any other forced tile keeps it away).
+   if ((force_tile == 576 || (!force_tile && lc.variant == 0 && tiles(256, 128) >= 256)) && conv_i8_resident_applies(a, Cg, Wp, M, N, K) &&
+       ep.stores_plain_rows())
+      return launch_conv_i8_resident<EPI>(lc, a, Wp, M, ep);
    // Whole 256 x 256 tiles, at least one per CU, and a store the register path handles (NHWC rows, or the plane sums of
    // planes that hold whole wave tiles): the persistent kernel.  512 asks for it by force.
    if ((force_tile == 512 || (!force_tile && lc.variant == 0 && tiles(256, 256) >= 256)) &&
        mfma8_persist_conv_applies(a, Wp, M, N, K, ep.elements_per_16_bytes(), !ep.stores_plain_rows()) &&
        (ep.stores_plain_rows() || ep.sums_rows_of_whole_wave_tiles(128)))
       return launch_mfma8_persist_src<MfmaI8x16, EPI, PersistConvRows>(lc, PersistConvRows{a}, Wp, M, N, K, K, ep);
-   if (tile == 512)
+   if (tile == 512 || tile == 576)
       tile = 256;
    switch (tile) {
    case 256:

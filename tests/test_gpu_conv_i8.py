@@ -156,6 +156,36 @@ def test_conv_i8_persistent_kernel(rt, case, forced, opt):
     assert (want != 0).mean() > 0.2 and np.abs(want).max() > 60  # neither all zero nor saturated
 
 
+@pytest.mark.parametrize("case", [
+    (3, 64, 16, 16, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),        # 16 x 16: 18 x 18 patches, one tile per image
+    (2, 64, 32, 32, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),        # 32 x 32: tiles of 8 rows, 4 per image
+    (5, 64, 64, 64, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),        # the benchmark's second layer: 80 tiles
+    (2, 64, 34, 66, 128, 3, 3, (0, 0, 0, 0), (1, 1), (1, 1), 1),        # no padding: 32 x 64 outputs from 34 x 66 inputs
+    (2, 64, 17, 31, 128, 3, 3, (0, 2, 1, 1), (1, 1), (1, 1), 1),        # unequal pads: 16 x 32 outputs
+    (2, 128, 16, 32, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 2),       # two groups of 64 -> 128 channels
+    (70, 64, 32, 32, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),       # 280 tiles: more than one per workgroup
+])
+@pytest.mark.parametrize("out,relu", [(R.I8OUT_I8, 1), (R.I8OUT_I8, 0), (R.I8OUT_I32, 1), (R.I8OUT_F32, 0)])
+def test_conv_i8_small_layer_with_resident_weights(rt, case, out, relu, opt):
+    """3 x 3, stride 1, 64 input and 128 output channels per group: the kernel that keeps the weights in LDS and loads each
+    tile's pixels once with their halo (asked for by force: tile 576; by the heuristic's own choice when there are at least 256
+    tiles).  Bit-exact against the oracle, edges (zeros outside the image) and image boundaries between tiles included."""
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    if N * 0 == 0 and (out != R.I8OUT_I8 or relu == 0) and N > 5:
+        pytest.skip("the long case runs with the benchmark's store only")
+    opt("i8_tile", 576)
+    X = util.int8_sym(184, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.int8_sym(185, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
+    bias = util.int32_range(186, Cout, -2000, 2000)
+    K = (Cc // group) * kh * kw
+    scale = ((0.5 + util.uniform01(187, Cout)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    want = ob.conv_i8(X, Wt, bias, scale, pads=pads, strides=strides, dils=dils, group=group, relu=relu, out=out, omp=True)
+    got = run_conv(rt, X, Wt, bias, scale, case, relu, out, R.LAYOUT_NHWC, R.LAYOUT_NHWC, 1)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    if out == R.I8OUT_I8:
+        assert (want != 0).mean() > 0.2 and np.abs(want).max() > 60
+
+
 def test_first_layer_of_an_image_network_needs_no_workspace(rt):
     """3 input channels, 3x3: K = 27 fits one slab, the rows are gathered in the kernel (NCHW in, NHWC out, a ragged last tile)."""
     case = (3, 3, 21, 19, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1)
