@@ -141,6 +141,7 @@ struct F8Epilogue {
    __device__ __forceinline__ bool rows_vectorizable() const { return stage_ok != 0; }
    __device__ __forceinline__ char *out_base() const { return (char *)Y; }
    __device__ __forceinline__ size_t out_index(int m, int n) const { return (size_t)m * (size_t)ldy + n; }
+   __device__ __forceinline__ size_t out_index_of_plain_rows(int m, int n) const { return out_index(m, n); }
    template <int C>
    struct col_params {
       float b[C];

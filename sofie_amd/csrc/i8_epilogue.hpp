@@ -123,6 +123,9 @@ struct I8Epilogue {
       return (size_t)m * (size_t)ldy + n + n_offset;
    }
 
+   // the same for a store that only exists for row-major outputs (stores_plain_rows()): no case to tell apart per element
+   __device__ __forceinline__ size_t out_index_of_plain_rows(int m, int n) const { return (size_t)m * (size_t)ldy + n + n_offset; }
+
    // DequantizeLinear of one accumulator: one fp32 multiply, then max(.,0) if relu_out
    __device__ __forceinline__ float to_f32(int acc, float s) const
    {
@@ -192,9 +195,12 @@ struct I8Epilogue {
       p.s[i] = __uint_as_float(w[1]);
    }
 
-   // the int8 results of columns 4q..4q+3 as integers (what the plane sums of a convolution add up)
+   // the int8 results of columns 4q..4q+3 as integers (what the plane sums of a convolution add up), each with kI8BitsBias
+   // added (the word i8_bits() returns): sums of such words are taken as they are, modulo 2^32, and the bias is subtracted
+   // once per sum instead of once per element
+   static constexpr uint32_t kI8BitsBias = 0x4B400000u;
    template <int OUT, int C, bool BIAS_DONE = false>
-   __device__ __forceinline__ void quantize4(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, int (&r)[4]) const
+   __device__ __forceinline__ void quantize4_biased(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, uint32_t (&r)[4]) const
    {
       int acc[4] = {a0, a1, a2, a3};
       int acc_floor = relu_acc ? 0 : (int)0x80000000;
@@ -208,7 +214,7 @@ struct I8Epilogue {
          float v = mul_nofma((float)acc[i], p.s[4 * q + i]);
          if (divides<OUT>())
             v = quotient<OUT>(v);
-         r[i] = (int)i8_bits(v, (requantizes<OUT>() && relu_out) ? 0.0f : -128.0f) - 0x4B400000; // needs the tamed scale, like pack4_short
+         r[i] = i8_bits(v, (requantizes<OUT>() && relu_out) ? 0.0f : -128.0f); // needs the tamed scale, like pack4_short
       }
    }
 

@@ -96,7 +96,7 @@ static int launch_mfma8_conv(const LaunchCfg &lc, const ConvRows &a, int Cg, con
    if ((force_tile == 512 || (!force_tile && lc.variant == 0 && tiles(256, 256) >= 256)) &&
        mfma8_persist_conv_applies(a, Wp, M, N, K, ep.elements_per_16_bytes(), !ep.stores_plain_rows()) &&
        (ep.stores_plain_rows() || ep.sums_rows_of_whole_wave_tiles(128)))
-      return launch_mfma8_persist_src<MfmaI8x16, EPI, PersistConvRows>(lc, PersistConvRows{a}, Wp, M, N, K, K, ep);
+      return launch_mfma8_persist_src<MfmaI8x16, EPI, PersistConvRows>(lc, persist_conv_rows(a), Wp, M, N, K, K, ep);
    if (tile == 512 || tile == 576)
       tile = 256;
    switch (tile) {

@@ -78,7 +78,7 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
                convert4(mode_c, prm, acc[i][j], g, w);
                typedef unsigned int u4 __attribute__((ext_vector_type(4)));
                const u4 v = {w[0], w[1], w[2], w[3]};
-               __builtin_nontemporal_store(v, (u4 *)(out + ep.out_index(m_base + i * R + lr, n_base + c0) * 4));
+               __builtin_nontemporal_store(v, (u4 *)(out + ep.out_index_of_plain_rows(m_base + i * R + lr, n_base + c0) * 4));
             });
          });
       });
@@ -121,8 +121,8 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
             // (streamed like the 1-byte tiles below: FP8 4096^3 -3.8 %, 8192^3 -1 %)
             typedef unsigned int u4 __attribute__((ext_vector_type(4)));
             const u4 vt = {top[0], top[1], top[2], top[3]}, vb = {bot[0], bot[1], bot[2], bot[3]};
-            __builtin_nontemporal_store(vt, (u4 *)(out + ep.out_index(m_base + i * R + (lane & 15), n) * 2));
-            __builtin_nontemporal_store(vb, (u4 *)(out + ep.out_index(m_base + i * R + 16 + (lane & 15), n) * 2));
+            __builtin_nontemporal_store(vt, (u4 *)(out + ep.out_index_of_plain_rows(m_base + i * R + (lane & 15), n) * 2));
+            __builtin_nontemporal_store(vb, (u4 *)(out + ep.out_index_of_plain_rows(m_base + i * R + 16 + (lane & 15), n) * 2));
          });
       });
    } else {
@@ -155,7 +155,7 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
                // neighbouring pixels, which are, keep their lines): -0.8 % on the int8 CNN
                typedef unsigned int u4 __attribute__((ext_vector_type(4)));
                const u4 v = {t01[0], t01[1], t23[0], t23[1]};
-               __builtin_nontemporal_store(v, (u4 *)(out + ep.out_index(m_base + (i0 + i) * R + lr, n_base + lk * 16)));
+               __builtin_nontemporal_store(v, (u4 *)(out + ep.out_index_of_plain_rows(m_base + (i0 + i) * R + lr, n_base + lk * 16)));
             }
          });
       });
@@ -163,14 +163,17 @@ __device__ __forceinline__ void tile_store_from_registers(const EPI &ep, ACC (&a
 }
 
 // The plane sums of a convolution that feeds a global average pool, from the accumulator registers: the int8 results of the
-// wave tile's rows (all in one plane) are added up per column instead of stored.  A lane adds its row blocks in registers,
-// the R lanes that share columns combine by xor-shuffles, and one lane per group of 4 columns adds the sums to memory.
+// wave tile's rows (all in one plane) are added up per column instead of stored.  A lane adds its row blocks in registers
+// (the converted words as they are, two per addition; their common offset leaves once per sum), the R = 16 lanes that share
+// columns, one row of the data-parallel-primitive network, combine in four additions that read a neighbour's register
+// (pairs, quads, the mirrored half row, the mirrored row), and one lane per group of 4 columns adds the sums to memory.
 template <int MODE, class MMA, int MT, int NT, class EPI, class ACC>
 __device__ __forceinline__ void tile_sum_from_registers(const EPI &ep, ACC (&acc)[MT][NT], int m_base, int n_base, int lane,
                                                         const uint32_t (&col_words)[EPI::kColWords])
 {
    constexpr int R = MMA::ROWS, LK = MMA::LK, G = MMA::ACC / 4;
    static_assert(NT * R == 64, "one column constant per lane");
+   static_assert(R == 16 && MT % 2 == 0, "the lanes of a 16-lane row share columns; row blocks are added in pairs");
    const int lr = lane % R, lk = lane / R;
    int first_col_addr = lk * 16;
    asm volatile("" : "+v"(first_col_addr));
@@ -188,22 +191,29 @@ __device__ __forceinline__ void tile_sum_from_registers(const EPI &ep, ACC (&acc
                w[k] = (EPI::kBiasInAccumulator && k == EPI::kBiasWord) ? 0u : (uint32_t)__builtin_amdgcn_ds_bpermute(first_col_addr + (cb + v) * 4, (int)col_words[k]);
             EPI::template set_column<4>(prm, v, w);
          }
-         int sum[4] = {0, 0, 0, 0};
-         static_for<MT>([&](auto ci) {
-            constexpr int i = decltype(ci)::value;
-            int q[4];
-            ep.template quantize4<MODE, 4, EPI::kBiasInAccumulator>(prm, 0, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3], q);
+         uint32_t sum[4] = {0, 0, 0, 0};
+         static_for<MT / 2>([&](auto ci) {
+            constexpr int i = 2 * decltype(ci)::value;
+            uint32_t q0[4], q1[4];
+            ep.template quantize4_biased<MODE, 4, EPI::kBiasInAccumulator>(prm, 0, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3], q0);
+            ep.template quantize4_biased<MODE, 4, EPI::kBiasInAccumulator>(prm, 0, acc[i + 1][j][4 * g + 0], acc[i + 1][j][4 * g + 1], acc[i + 1][j][4 * g + 2],
+                                                                           acc[i + 1][j][4 * g + 3], q1);
 #pragma unroll
             for (int v = 0; v < 4; ++v)
-               sum[v] += q[v];
+               sum[v] = sum[v] + q0[v] + q1[v];
          });
+         int total[4];
 #pragma unroll
-         for (int d = 1; d < R; d <<= 1)
-#pragma unroll
-            for (int v = 0; v < 4; ++v)
-               sum[v] += __shfl_xor(sum[v], d, 64);
+         for (int v = 0; v < 4; ++v) {
+            int t = (int)(sum[v] - (uint32_t)MT * EPI::kI8BitsBias);
+            t += __builtin_amdgcn_update_dpp(0, t, 0xB1, 0xf, 0xf, false);  // quad_perm [1,0,3,2]: lane ^ 1
+            t += __builtin_amdgcn_update_dpp(0, t, 0x4E, 0xf, 0xf, false);  // quad_perm [2,3,0,1]: lane ^ 2
+            t += __builtin_amdgcn_update_dpp(0, t, 0x141, 0xf, 0xf, false); // row_half_mirror: the other quad of the half row
+            t += __builtin_amdgcn_update_dpp(0, t, 0x140, 0xf, 0xf, false); // row_mirror: the other half row
+            total[v] = t;
+         }
          if (lr == 0)
-            ep.add_row_sums(m_base, n_base + cb + lk * 4, ep.N, sum);
+            ep.add_row_sums(m_base, n_base + cb + lk * 4, ep.N, total);
       });
    });
 }
@@ -252,6 +262,10 @@ struct PersistPlainRows {
 struct PersistConvRows {
    static constexpr bool kConv = true;
    ConvRows g;
+   // log2(OW) when a tile is whole output rows of one image (OW a power of two that divides 256, planes of whole tiles), else
+   // -1.  A tile's image and first output row are then the same for all lanes (scalar arithmetic, once), and a lane's pixel is
+   // a fixed number of rows and columns from there: no division per lane and tile.
+   int ow_shift;
    struct lane_state {
       int row[2], swz[2]; // swz: the chunk of the 64-byte slab row this lane supplies
    };
@@ -266,6 +280,27 @@ struct PersistConvRows {
    }
    __device__ __forceinline__ void tile(tile_state &ts, const lane_state &ls, int m0) const
    {
+      if (ow_shift >= 0) {
+         const int ohw = g.OH * g.OW;
+         const int m0u = __builtin_amdgcn_readfirstlane(m0);
+         const int n = g.ohw_mul ? (int)__umul64hi((unsigned long long)(unsigned)m0u, g.ohw_mul) : m0u;
+         const int oh0 = (m0u - n * ohw) >> ow_shift;
+         uint32_t mask = 0;
+#pragma unroll
+         for (int i = 0; i < 2; ++i) {
+            const int oh = oh0 + (ls.row[i] >> ow_shift), ow = ls.row[i] & (g.OW - 1);
+            const int ih0 = oh * g.stride_h - g.pad_h0, iw0 = ow * g.stride_w - g.pad_w0;
+            ts.off[i] = ((n * g.H + ih0) * g.W + iw0) * g.C + ls.swz[i];
+            uint32_t cols = 0, mk = 0;
+            for (int kwi = 0, iw = iw0; kwi < g.kw; ++kwi, iw += g.dil_w)
+               cols |= ((unsigned)iw < (unsigned)g.W ? 1u : 0u) << kwi;
+            for (int t0 = 0, ih = ih0; t0 < g.ntaps; t0 += g.kw, ih += g.dil_h)
+               mk |= ((unsigned)ih < (unsigned)g.H ? cols : 0u) << t0;
+            mask |= mk << (16 * i);
+         }
+         ts.mask = mask;
+         return;
+      }
       ConvRows::lane_state<2> st;
       g.template init<2>(st, 0, m0, ls.row[0], ls.swz[0], 0x7fffffff);
       g.template init<2>(st, 1, m0, ls.row[1], ls.swz[1], 0x7fffffff);
@@ -589,6 +624,18 @@ static int launch_mfma8_persist_src(const LaunchCfg &lc, const ASRC &a, const in
    const int grid = ntiles < ncu ? ntiles : ncu;
    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, lc.stream, a, Bt, ldb, M, N, K, ep, tiles_m, tiles_n, lc.swizzle);
    return launch_status("mfma8_gemm_persist_kernel");
+}
+
+inline PersistConvRows persist_conv_rows(const ConvRows &a)
+{
+   PersistConvRows p;
+   p.g = a;
+   p.ow_shift = -1;
+   if (a.OW >= 1 && a.OW <= 256 && (a.OW & (a.OW - 1)) == 0 && (a.OH * a.OW) % 256 == 0)
+      for (int sh = 0; sh <= 8; ++sh)
+         if ((1 << sh) == a.OW)
+            p.ow_shift = sh;
+   return p;
 }
 
 template <class MMA, class EPI>
