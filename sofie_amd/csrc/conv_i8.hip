@@ -315,6 +315,21 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
          ep.nchw_ohw = (a->y_layout == SOFIE_LAYOUT_NHWC || plane_sums) ? 0 : OHW;
          ep.rows_per_plane = plane_sums ? OHW : 0;
          ep.Y = a->Y;
+         if (!nhwc && d->stride_w == 1 && d->dil_w == 1) {
+            FewChannelConv fc;
+            fc.X = src.X;
+            fc.H = d->H; fc.W = d->W; fc.OH = g.OH; fc.OW = g.OW;
+            fc.stride_h = d->stride_h; fc.pad_h0 = d->pad_h0; fc.pad_w0 = d->pad_w0; fc.dil_h = d->dil_h;
+            fc.kh = d->kh; fc.kw = d->kw; fc.Cg = g.Cg;
+            fc.img_stride = src.img_stride;
+            fc.ow_mul = fc.oh_mul = 0;
+            bool taken = false;
+            st = conv_i8_few_channels(launch_cfg_i8(ctx), fc, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.Kp, ep, &taken);
+            if (st)
+               return st;
+            if (taken)
+               continue;
+         }
          st = conv_i8_gather(launch_cfg_i8(ctx), src, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.Kp, ep);
          if (st)
             return st;

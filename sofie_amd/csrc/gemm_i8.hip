@@ -1,6 +1,7 @@
 // int8 x int8 -> int32 GEMM on the gfx950 matrix cores (v_mfma_i32_32x32x32_i8) with the
 // requantisation / dequantisation epilogue fused into the store, and the int8 re-layout kernel.
 #include "i8_epilogue.hpp"
+#include "conv_i8_few_channels.hpp"
 #include <cmath>
 #include <mutex>
 
@@ -56,6 +57,19 @@ int conv_i8_gather(const LaunchCfg &lc, const GatherConvRows &src, const int8_t 
 {
    derive_epilogue_fields(ep, N);
    return launch_mfma8_gather<I8Epilogue>(lc, src, Wp, M, N, Kp, ep);
+}
+
+int conv_i8_few_channels(const LaunchCfg &lc, const FewChannelConv &src, const int8_t *Wp, int M, int N, int Kp, I8Epilogue ep, bool *taken)
+{
+   derive_epilogue_fields(ep, N);
+   *taken = false;
+   // 27 asks for it by force; any other forced tile or variant keeps it away
+   if (!((lc.tile == 0 && lc.variant == 0) || lc.tile == 27))
+      return SOFIE_HIP_OK;
+   if (N != 64 || M % 64 != 0 || !ep.stores_plain_rows() || !conv_i8_few_channels_applies(src, Wp))
+      return SOFIE_HIP_OK;
+   *taken = true;
+   return launch_conv_i8_few_channels<I8Epilogue>(lc, src, Wp, M, Kp, ep);
 }
 
 int transpose_i8(hipStream_t stream, int8_t *dst, const int8_t *src, int rows, int cols, int ld_src, int ld_dst)

@@ -314,6 +314,9 @@ struct I8Epilogue {
 int gemm_i8_nt(const LaunchCfg &lc, const int8_t *A, const int8_t *Bt, int M, int N, int K, int lda, int ldb, I8Epilogue ep);
 // Convolution whose whole reduction fits one 64-byte slab (few input channels): rows gathered byte by byte, one launch.
 int conv_i8_gather(const LaunchCfg &lc, const GatherConvRows &src, const int8_t *Wp, int M, int N, int Kp, I8Epilogue ep);
+// The same for NCHW input with stride and dilation 1 in x, 64 output channels and rows stored as they are: windows of four
+// bytes instead of single bytes.  *taken tells whether the shape was this kernel's (else nothing was launched).
+int conv_i8_few_channels(const LaunchCfg &lc, const FewChannelConv &src, const int8_t *Wp, int M, int N, int Kp, I8Epilogue ep, bool *taken);
 // Convolution as an implicit GEMM: rows of A come from `src`, Wp is [N][K] with K = taps * Cg.
 int conv_i8_implicit(const LaunchCfg &lc, const ConvRows &src, int Cg, const int8_t *Wp, int M, int N, int K, I8Epilogue ep);
 

@@ -198,6 +198,16 @@ struct GatherConvRowsT : GatherConvRows {
    static constexpr int kKP = KP;
 };
 
+// The geometry of a convolution over few input channels whose NCHW input is read window by window (conv_i8_few_channels.hpp).
+struct FewChannelConv {
+   const int8_t *X;      // NCHW, first channel of the group
+   int H, W, OH, OW;
+   int stride_h, pad_h0, pad_w0, dil_h;
+   int kh, kw, Cg;
+   long long img_stride; // bytes per image: all channels
+   uint32_t ow_mul, oh_mul; // ceil(2^24 / OW), ceil(2^24 / OH): t / OW == (t * ow_mul) >> 24 while t * OW < 2^24
+};
+
 // 256 zero bytes: what a load of a padded (out-of-image) position reads.
 static __device__ __attribute__((aligned(256))) int8_t conv_zero_page[256] = {};
 

@@ -186,6 +186,38 @@ def test_conv_i8_small_layer_with_resident_weights(rt, case, out, relu, opt):
         assert (want != 0).mean() > 0.2 and np.abs(want).max() > 60
 
 
+@pytest.mark.parametrize("case", [
+    (4, 3, 16, 16, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),      # RGB 3 x 3: the benchmark's first layer in small
+    (2, 3, 64, 64, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),      # the benchmark's image size: a group of 64 pixels is one row
+    (16, 1, 8, 8, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),       # one channel, the narrowest row the loads allow (8 bytes)
+    (64, 4, 9, 8, 64, 4, 4, (0, 0, 0, 0), (1, 1), (1, 1), 1),       # 4 x 4 over 4 channels: all 16 pairs, no padding, 6 x 5 outputs
+    (16, 3, 20, 12, 64, 5, 3, (2, 3, 2, 0), (1, 1), (1, 1), 1),     # 5 rows of taps, three columns of padding on the left, none on the right
+    (8, 2, 17, 16, 64, 3, 2, (1, 0, 1, 1), (2, 1), (2, 1), 1),      # stride 2 and dilation 2 in y, two columns of taps
+    (4, 6, 16, 16, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 2),     # two groups of 3 -> 64 channels
+    (70, 3, 32, 32, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),     # 1120 groups of pixels: more than one per wave
+])
+@pytest.mark.parametrize("out,relu", [(R.I8OUT_I8, 1), (R.I8OUT_I8, 0), (R.I8OUT_I32, 1), (R.I8OUT_F32, 0)])
+def test_conv_i8_few_input_channels_read_as_windows(rt, case, out, relu, opt):
+    """NCHW input with few channels, 64 output channels, stride and dilation 1 in x: the kernel that reads each (channel, row of
+    taps) as one four-byte window cut from an aligned load (asked for by force: tile 27; it is also the heuristic's choice).
+    Bit-exact against the oracle: zeros left, right, above and below the image, images and rows that change inside a group of
+    64 pixels."""
+    N, Cc, H, W, Cout, kh, kw, pads, strides, dils, group = case
+    if N > 16 and (out != R.I8OUT_I8 or relu == 0):
+        pytest.skip("the long cases run with the benchmark's store only")
+    opt("i8_tile", 27)
+    X = util.int8_sym(194, N * Cc * H * W).reshape(N, Cc, H, W)
+    Wt = util.int8_sym(195, Cout * (Cc // group) * kh * kw).reshape(Cout, Cc // group, kh, kw)
+    bias = util.int32_range(196, Cout, -500, 500)
+    K = (Cc // group) * kh * kw
+    scale = ((0.5 + util.uniform01(197, Cout)) / np.float32(127.0 * np.sqrt(K))).astype(np.float32)
+    want = ob.conv_i8(X, Wt, bias, scale, pads=pads, strides=strides, dils=dils, group=group, relu=relu, out=out, omp=True)
+    got = run_conv(rt, X, Wt, bias, scale, case, relu, out, R.LAYOUT_NCHW, R.LAYOUT_NHWC, 1)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    if out == R.I8OUT_I8:
+        assert (want != 0).mean() > 0.2 and np.abs(want).max() > 60
+
+
 def test_first_layer_of_an_image_network_needs_no_workspace(rt):
     """3 input channels, 3x3: K = 27 fits one slab, the rows are gathered in the kernel (NCHW in, NHWC out, a ragged last tile)."""
     case = (3, 3, 21, 19, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1)
