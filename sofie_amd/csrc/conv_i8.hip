@@ -322,7 +322,6 @@ int sofie_hip_conv_i8(sofie_hip_ctx *ctx, const sofie_conv_desc *d, const sofie_
             fc.stride_h = d->stride_h; fc.pad_h0 = d->pad_h0; fc.pad_w0 = d->pad_w0; fc.dil_h = d->dil_h;
             fc.kh = d->kh; fc.kw = d->kw; fc.Cg = g.Cg;
             fc.img_stride = src.img_stride;
-            fc.ow_mul = fc.oh_mul = 0;
             bool taken = false;
             st = conv_i8_few_channels(launch_cfg_i8(ctx), fc, Wp + (size_t)grp * Cout_g * g.Kp, (int)rows, Cout_g, g.Kp, ep, &taken);
             if (st)

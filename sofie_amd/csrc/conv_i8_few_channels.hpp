@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void conv_i8_few_channels_kernel(FewChannelCon
       uint32_t w[4] = {0, 0, 0, 0};
       for (int b = 0; b < 16; ++b) {
          const int pair = q * 4 + (b >> 2), kx = b & 3;
-         const int c = pair / g.kh, ky = pair - c * g.kh;
+         const int c = g.pair_c[pair], ky = g.pair_ky[pair];
          int8_t v = 0;
          if (pair < npairs && kx < g.kw)
             v = Wp[(size_t)col * Kp + (ky * g.kw + kx) * g.Cg + c];
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void conv_i8_few_channels_kernel(FewChannelCon
 #pragma unroll
    for (int q = 0; q < 4; ++q) {
       const int pair = lk * 4 + q;
-      const int c = pair / g.kh, ky = pair - c * g.kh;
+      const int c = g.pair_c[pair], ky = g.pair_ky[pair];
       pair_off[q] = (c * g.H + ky * g.dil_h) * g.W;
       pair_dy[q] = pair < npairs ? ky * g.dil_h : (1 << 24);
    }
@@ -77,25 +77,32 @@ __global__ __launch_bounds__(256) void conv_i8_few_channels_kernel(FewChannelCon
             acc0[j][v] = EPI::kBiasInAccumulator ? __builtin_amdgcn_ds_bpermute(first_col_addr + (j * R + v) * 4, (int)col_words[EPI::kBiasWord]) : 0;
    }
 
+   // The windows of a group are requested one group ahead: while they are on their way, the group before is multiplied,
+   // converted and stored.
    const int ohw = g.OH * g.OW;
-   for (int grp = blockIdx.x * 4 + wave; grp < ngroups; grp += gridDim.x * 4) {
+   uint64_t chunk[MT][4];
+   bool ok[MT][4];
+   int rsh[MT], lsh[MT];
+   auto request = [&](int grp) {
       // first pixel of the group (uniform): image, row, column
       const int p0 = grp * 64;
       const int n0 = p0 / ohw, r0 = p0 - n0 * ohw;
       const int oh0 = r0 / g.OW, ow0 = r0 - oh0 * g.OW;
-      uint64_t chunk[MT][4];
-      bool ok[MT][4];
-      int rsh[MT], lsh[MT];
+      const int8_t *img0 = g.X + (long long)n0 * g.img_stride; // uniform: the loads take it as their scalar base
+      // pixel p0 + lr, and the lane's other pixels 16, 32, 48 further on: at most one row further each time (OW >= 16),
+      // which may be the first row of the next image
+      int ow = ow0 + lr, oh = oh0, dn = 0;
+      auto wrap = [&]() {
+         if (ow >= g.OW) {
+            ow -= g.OW;
+            oh += 1;
+            if (oh >= g.OH)
+               oh = 0, dn += 1;
+         }
+      };
+      wrap();
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
-         // pixel p0 + 16 i + lr: at most 63 pixels on from the first one
-         const uint32_t tc = (uint32_t)(ow0 + i * R + lr);
-         const int qc = (int)(__umul24(tc, g.ow_mul) >> 24);
-         const int ow = (int)tc - qc * g.OW;
-         const uint32_t tr = (uint32_t)(oh0 + qc);
-         const int qr = (int)(__umul24(tr, g.oh_mul) >> 24);
-         const int oh = (int)tr - qr * g.OH;
-         const int n = n0 + qr;
          const int ih0 = oh * g.stride_h - g.pad_h0, iw0 = ow - g.pad_w0;
          int cs = iw0 & ~3;
          cs = cs < 0 ? 0 : cs;
@@ -103,15 +110,22 @@ __global__ __launch_bounds__(256) void conv_i8_few_channels_kernel(FewChannelCon
          const int s = iw0 - cs; // -3 .. 7
          rsh[i] = s > 0 ? 8 * s : 0;
          lsh[i] = s < 0 ? -8 * s : 0;
-         const int8_t *img = g.X + (long long)n * g.img_stride;
-         const int row_off = ih0 * g.W + cs;
+         const uint32_t row_off = (uint32_t)(dn * (int)g.img_stride + ih0 * g.W + cs);
 #pragma unroll
          for (int q = 0; q < 4; ++q) {
             ok[i][q] = (unsigned)(ih0 + pair_dy[q]) < (unsigned)g.H;
-            const int off = ok[i][q] ? row_off + pair_off[q] : 0;
-            chunk[i][q] = *(const u64_dword_aligned *)(img + off);
+            const uint32_t off = ok[i][q] ? row_off + (uint32_t)pair_off[q] : 0u;
+            chunk[i][q] = *(const u64_dword_aligned *)(img0 + off);
          }
+         ow += R;
+         wrap();
       }
+   };
+   const int stride = gridDim.x * 4;
+   int grp = blockIdx.x * 4 + wave;
+   if (grp < ngroups)
+      request(grp);
+   for (; grp < ngroups; grp += stride) {
       frag_t fa[MT];
 #pragma unroll
       for (int i = 0; i < MT; ++i)
@@ -120,6 +134,8 @@ __global__ __launch_bounds__(256) void conv_i8_few_channels_kernel(FewChannelCon
             const uint32_t win = (uint32_t)((chunk[i][q] >> rsh[i]) << lsh[i]);
             fa[i].c[0][q] = ok[i][q] ? (int)win : 0;
          }
+      if (grp + stride < ngroups)
+         request(grp + stride);
       acc_t acc[MT][NT];
 #pragma unroll
       for (int j = 0; j < NT; ++j)
@@ -127,7 +143,7 @@ __global__ __launch_bounds__(256) void conv_i8_few_channels_kernel(FewChannelCon
          for (int i = 0; i < MT; ++i)
             acc[i][j] = MMA::mma(fb[j], fa[i], acc0[j]);
       ep.dispatch_for_registers([&](auto mode) {
-         tile_store_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, p0, 0, lane, col_words);
+         tile_store_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, grp * 64, 0, lane, col_words);
       });
    }
 }
@@ -135,23 +151,26 @@ __global__ __launch_bounds__(256) void conv_i8_few_channels_kernel(FewChannelCon
 // Shapes the kernel takes (the caller has checked the output: 64 channels, whole groups of 64 pixels, rows stored as they are).
 inline bool conv_i8_few_channels_applies(const FewChannelConv &g, const int8_t *Wp)
 {
-   return g.kw <= 4 && g.Cg * g.kh <= 16 && g.pad_w0 <= 3 && g.W % 4 == 0 && g.W >= 8 && g.OW >= 2 && g.OW <= 4000 && g.OH >= 2 && g.OH <= 4000 &&
+   return g.kw <= 4 && g.Cg * g.kh <= 16 && g.pad_w0 <= 3 && g.W % 4 == 0 && g.W >= 8 && g.OW >= 16 && g.img_stride < (1LL << 28) &&
           (((uintptr_t)g.X | (uintptr_t)g.img_stride) & 3) == 0 && Wp != nullptr;
 }
 
 template <class EPI>
 static int launch_conv_i8_few_channels(const LaunchCfg &lc, FewChannelConv g, const int8_t *Wp, int M, int Kp, const EPI &ep)
 {
-   g.ow_mul = (uint32_t)(((1u << 24) + g.OW - 1) / g.OW);
-   g.oh_mul = (uint32_t)(((1u << 24) + g.OH - 1) / g.OH);
    const int ngroups = M / 64;
    int ncu = 0;
    if (int st = cu_count_of_current_device(ncu))
       return st;
-   // four waves per workgroup, up to four workgroups per CU (the registers allow it): every wave gets about the same share
+   for (int pair = 0; pair < 16; ++pair) {
+      g.pair_c[pair] = (unsigned char)(pair / g.kh);
+      g.pair_ky[pair] = (unsigned char)(pair % g.kh);
+   }
+   // four waves per workgroup, two workgroups per CU (what the registers allow): all of them resident at once, the weights
+   // re-ordered once per workgroup
    int grid = (ngroups + 3) / 4;
-   if (grid > 4 * ncu)
-      grid = 4 * ncu;
+   if (grid > 2 * ncu)
+      grid = 2 * ncu;
    hipLaunchKernelGGL(conv_i8_few_channels_kernel<EPI>, dim3((unsigned)grid), dim3(256), 0, lc.stream, g, Wp, Kp, ep, ngroups);
    return launch_status("conv_i8_few_channels_kernel");
 }

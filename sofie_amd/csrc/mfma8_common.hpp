@@ -205,7 +205,7 @@ struct FewChannelConv {
    int stride_h, pad_h0, pad_w0, dil_h;
    int kh, kw, Cg;
    long long img_stride; // bytes per image: all channels
-   uint32_t ow_mul, oh_mul; // ceil(2^24 / OW), ceil(2^24 / OH): t / OW == (t * ow_mul) >> 24 while t * OW < 2^24
+   unsigned char pair_c[16], pair_ky[16]; // channel and row of taps of (channel, ky) pair p = channel * kh + ky (filled in by the launcher)
 };
 
 // 256 zero bytes: what a load of a padded (out-of-image) position reads.

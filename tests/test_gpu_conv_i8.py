@@ -189,9 +189,9 @@ def test_conv_i8_small_layer_with_resident_weights(rt, case, out, relu, opt):
 @pytest.mark.parametrize("case", [
     (4, 3, 16, 16, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),      # RGB 3 x 3: the benchmark's first layer in small
     (2, 3, 64, 64, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),      # the benchmark's image size: a group of 64 pixels is one row
-    (16, 1, 8, 8, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),       # one channel, the narrowest row the loads allow (8 bytes)
-    (64, 4, 9, 8, 64, 4, 4, (0, 0, 0, 0), (1, 1), (1, 1), 1),       # 4 x 4 over 4 channels: all 16 pairs, no padding, 6 x 5 outputs
-    (16, 3, 20, 12, 64, 5, 3, (2, 3, 2, 0), (1, 1), (1, 1), 1),     # 5 rows of taps, three columns of padding on the left, none on the right
+    (4, 1, 16, 16, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),      # one channel; rows of 16: the last load of a row starts at byte 8 for five pixels
+    (8, 4, 11, 20, 64, 4, 4, (0, 0, 0, 0), (1, 1), (1, 1), 1),      # 4 x 4 over 4 channels: all 16 pairs, no padding, 8 x 17 outputs
+    (16, 3, 20, 16, 64, 5, 3, (2, 3, 2, 0), (1, 1), (1, 1), 1),     # 5 rows of taps, three columns of padding on the left, none on the right: 20 x 17 outputs
     (8, 2, 17, 16, 64, 3, 2, (1, 0, 1, 1), (2, 1), (2, 1), 1),      # stride 2 and dilation 2 in y, two columns of taps
     (4, 6, 16, 16, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 2),     # two groups of 3 -> 64 channels
     (70, 3, 32, 32, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1),     # 1120 groups of pixels: more than one per wave
