@@ -370,6 +370,7 @@ def cpu_baseline(x, weights, w_scales, in_scales, rows):
 
 
 def main():
+    global CLOCK_WARM_MS, REGION_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
@@ -384,7 +385,6 @@ def main():
                     help="also run three 256 MiB device-to-device copies: a kernel of known traffic that scales the FETCH_SIZE / "
                          "WRITE_SIZE counters of a profiling run")
     args = ap.parse_args()
-    global CLOCK_WARM_MS, REGION_MS
     CLOCK_WARM_MS, REGION_MS = max(0.0, args.clock_warm_ms), max(0.1, args.region_ms)
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (the path is data-parallel over the batch; "
