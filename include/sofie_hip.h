@@ -24,9 +24,10 @@ extern "C" {
 
 /* Version of this interface: raised whenever an entry point is added, removed or changes its meaning (3: the kernel-choice
  * options are read from the environment once, when a context is created, and changed through sofie_hip_ctx_set_option; entry
- * points added for 3-D operators and for callers that cannot allocate).  An emitted Session compares the value it was compiled
- * with against sofie_hip_abi_version() of the library it finds at run time, and refuses to run on a different one. */
-#define SOFIE_HIP_ABI_VERSION 3
+ * points added for 3-D operators and for callers that cannot allocate; 4: sofie_hip_plane_sums_take_average added).  An
+ * emitted Session compares the value it was compiled with against sofie_hip_abi_version() of the library it finds at run
+ * time, and refuses to run on a different one. */
+#define SOFIE_HIP_ABI_VERSION 4
 
 typedef struct sofie_hip_ctx sofie_hip_ctx;
 
@@ -445,6 +446,11 @@ int sofie_hip_global_avg_pool_i8(sofie_hip_ctx *ctx, float *Y /* [N,C] */, const
  * on the feature map that was never stored. */
 int sofie_hip_plane_sums_to_average(sofie_hip_ctx *ctx, float *Y /* [NC] */, const int32_t *sums /* [NC] */, int32_t NC, int32_t HW,
                                     float scale);
+/* The same average, and the sums are set back to zero behind the read.  For a caller that keeps one sums buffer per
+ * convolution and clears it once (an emitted Session does, at construction): every inference leaves the buffer as the next
+ * one needs it, and the clearing launch per inference goes away. */
+int sofie_hip_plane_sums_take_average(sofie_hip_ctx *ctx, float *Y /* [NC] */, int32_t *sums /* [NC], zero afterwards */, int32_t NC,
+                                      int32_t HW, float scale);
 
 /* Softmax / LogSoftmax along one axis of a tensor seen as [outer, axis_len, inner] (ROperator_Softmax::Generate,
  * core/inc/SOFIE/operators/ROperator_Softmax.hxx:82-198): vmax = max over the axis, e = exp(x - vmax), sum = sum of e;

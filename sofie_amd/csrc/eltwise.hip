@@ -407,6 +407,16 @@ __global__ __launch_bounds__(256) void plane_sums_to_average_kernel(float *__res
       Y[i] = __fdiv_rn(mul_nofma((float)sums[i], scale), (float)HW);
 }
 
+// The same, and the sums are cleared behind the read: a buffer that starts out zero is zero again for the next convolution.
+__global__ __launch_bounds__(256) void plane_sums_take_average_kernel(float *__restrict__ Y, int32_t *__restrict__ sums, int NC, int HW, float scale)
+{
+   const int i = blockIdx.x * blockDim.x + threadIdx.x;
+   if (i < NC) {
+      Y[i] = __fdiv_rn(mul_nofma((float)sums[i], scale), (float)HW);
+      sums[i] = 0;
+   }
+}
+
 // NHWC int8 input with C a multiple of 16 (and 16-byte aligned): one workgroup per (image, block of 256 channels).
 // A thread owns 16 consecutive channels and every (256 / chunks)-th pixel, reads 16 bytes per pixel, and the
 // per-thread int32 sums are added up through LDS (integer sums: exact in any order).
@@ -811,6 +821,17 @@ int sofie_hip_plane_sums_to_average(sofie_hip_ctx *ctx, float *Y, const int32_t 
    SOFIE_HIP_REQUIRE(Y && sums, "sofie_hip_plane_sums_to_average: NULL pointer");
    hipLaunchKernelGGL(plane_sums_to_average_kernel, dim3((NC + 255) / 256), dim3(256), 0, ctx->stream, Y, sums, NC, HW, scale);
    return launch_status("plane_sums_to_average_kernel");
+}
+
+int sofie_hip_plane_sums_take_average(sofie_hip_ctx *ctx, float *Y, int32_t *sums, int32_t NC, int32_t HW, float scale)
+{
+   SOFIE_HIP_REQUIRE(ctx != nullptr, "sofie_hip_plane_sums_take_average: ctx is NULL");
+   SOFIE_HIP_REQUIRE(NC >= 0 && HW > 0, "sofie_hip_plane_sums_take_average: bad shape");
+   if (NC == 0)
+      return SOFIE_HIP_OK;
+   SOFIE_HIP_REQUIRE(Y && sums, "sofie_hip_plane_sums_take_average: NULL pointer");
+   hipLaunchKernelGGL(plane_sums_take_average_kernel, dim3((NC + 255) / 256), dim3(256), 0, ctx->stream, Y, sums, NC, HW, scale);
+   return launch_status("plane_sums_take_average_kernel");
 }
 
 } // extern "C"

@@ -96,6 +96,7 @@ public:
       int begin, end; // lifetime in operator indices, [begin, end); statics have begin = -1
       bool pooled;
       bool perBatch = false; // offset and bytes are per batch entry, counted from the end of the static region
+      bool view = false;     // placed on the tensor it is a view of (an operator that hands its input's bytes on unchanged)
    };
    const std::vector<PlannedTensor> &GetMemoryPlan() const { return fPlan; }
    std::size_t GetArenaBytes() const { return fArenaBytes; }

@@ -30,6 +30,11 @@ public:
    virtual std::size_t GetWorkspaceBytes() { return 0; }
    // in a model with a run-time batch: true if GetWorkspaceBytes() is the need of ONE batch entry
    virtual bool WorkspacePerBatchEntry() const { return false; }
+   // An operator whose output holds the bytes of its input unchanged (Reshape, Flatten, Squeeze, Unsqueeze) can give its
+   // output as a VIEW: the memory plan then places the output on the input and the operator generates no copy.  The plan
+   // asks CanBeView() and tells the operator its decision with SetView().
+   virtual bool CanBeView() const { return false; }
+   virtual void SetView(bool) {}
    // true for an operator that reads a tensor with a run-time batch and folds the batch away (a reduction over it): its outputs carry none
    virtual bool ConsumesBatch() const { return false; }
    virtual OperatorKind GetKind() const { return fKind; }

@@ -151,9 +151,18 @@ public:
       model.SetTensorLayout(fNY, fYLayout);
    }
    std::size_t PackedK() const { return ((fGeo.C / fGeo.group) * fGeo.kh * fGeo.kw + 15) / 16 * 16; }
+   // The int32 plane sums [N][Cout] of a convolution that feeds a GlobalAveragePool.  With a fixed batch they have a buffer of
+   // their own, cleared once at construction: the averaging call clears them again behind its read, so no inference starts
+   // with a clearing launch.  With a run-time batch (N is 1 here and the bytes are per batch entry) they are a workspace,
+   // cleared by every inference.
+   bool KeepsPlaneSums() const { return fSumPlanes && !fDynamic; }
+   std::size_t PlaneSumBytes() const { return (fGeo.N * fGeo.Cout * 4 + 255) / 256 * 256; }
    std::vector<std::pair<std::string, std::size_t>> GetPersistentBuffers() override
    {
-      return {{"packed_" + fNW, (fGeo.Cout * PackedK() + 255) / 256 * 256}};
+      std::vector<std::pair<std::string, std::size_t>> b = {{"packed_" + fNW, (fGeo.Cout * PackedK() + 255) / 256 * 256}};
+      if (KeepsPlaneSums())
+         b.emplace_back("planesums_" + fNY, PlaneSumBytes());
+      return b;
    }
    std::string GenerateInitCode_GPU_HIP() override
    {
@@ -162,6 +171,9 @@ public:
       out << SP << "      " << "sofie_conv_desc d" << fGeo.DescInitializer() << ";\n";
       out << SP << "      " << "detail::Check(sofie_hip_pack_conv_weight_i8(fCtx, &d, packed_" << fNW << ", tensor_" << fNW << "), \"re-layout of "
           << fNW << "\");\n";
+      if (KeepsPlaneSums())
+         out << SP << "      " << "detail::Check(sofie_hip_fill_zero(fCtx, planesums_" << fNY << ", " << PlaneSumBytes() << "), \"clearing of the plane sums of "
+             << fNY << "\");\n";
       out << SP << "   " << "}\n";
       return out.str();
    }
@@ -182,8 +194,8 @@ public:
    }
    std::size_t GetWorkspaceBytes() override
    {
-      if (fSumPlanes) // the int32 plane sums [N][Cout]; with a run-time batch N is 1 here and the bytes are per batch entry
-         return (fGeo.N * fGeo.Cout * 4 + 255) / 256 * 256;
+      if (fSumPlanes)
+         return KeepsPlaneSums() ? 0 : PlaneSumBytes();
       if (ImplicitGemm() || GatheredGemm())
          return 0;
       const std::size_t per_image = (fGeo.OH * fGeo.OW * PackedK() + 255) / 256 * 256;
@@ -193,7 +205,7 @@ public:
    bool WorkspacePerBatchEntry() const override { return fDynamic; }
    std::string Generate_GPU_HIP(std::string opName) override
    {
-      const std::string ws = "workspace_op_" + opName;
+      const std::string ws = KeepsPlaneSums() ? "planesums_" + fNY : "workspace_op_" + opName;
       opName = "op_" + opName;
       std::stringstream out;
       out << "\n" << SP << "//----  operator " << (fInt32Out ? "ConvInteger " : "QLinearConv ") << opName << " --> " << ConvertShapeToString(fGeo.OutputShape())
@@ -208,13 +220,18 @@ public:
           << "; a.x_layout = " << (fXLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.y_layout = "
           << (fYLayout == kLayoutNHWC ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << "; a.Y = " << (fSumPlanes ? ws : "tensor_" + fNY) << ";\n";
       if (fSumPlanes) {
-         // rows of Cout int32 sums, one per image; cleared, filled by the convolution's store, then averaged
+         // rows of Cout int32 sums, one per image; zero before, filled by the convolution's store, then averaged
          const std::string count = BatchScaledInt(fDynamic, fGeo.N * fGeo.Cout);
-         out << SP << "   " << "detail::Check(sofie_hip_fill_zero(fCtx, " << ws << ", static_cast<std::size_t>(" << count << ") * 4), \"" << opName
-             << " clear plane sums\");\n";
+         if (!KeepsPlaneSums())
+            out << SP << "   " << "detail::Check(sofie_hip_fill_zero(fCtx, " << ws << ", static_cast<std::size_t>(" << count << ") * 4), \"" << opName
+                << " clear plane sums\");\n";
          out << SP << "   " << "detail::Check(sofie_hip_conv_i8(fCtx, &d, &a), \"" << opName << " QLinearConv\");\n";
-         out << SP << "   " << "detail::Check(sofie_hip_plane_sums_to_average(fCtx, tensor_" << fNPooled << ", static_cast<const int32_t *>(static_cast<const void *>(" << ws
-             << ")), " << count << ", " << fGeo.OH * fGeo.OW << ", " << FloatLiteral(fPoolScale) << "), \"" << opName << " GlobalAveragePool\");\n";
+         if (KeepsPlaneSums())
+            out << SP << "   " << "detail::Check(sofie_hip_plane_sums_take_average(fCtx, tensor_" << fNPooled << ", static_cast<int32_t *>(static_cast<void *>(" << ws
+                << ")), " << count << ", " << fGeo.OH * fGeo.OW << ", " << FloatLiteral(fPoolScale) << "), \"" << opName << " GlobalAveragePool\");\n";
+         else
+            out << SP << "   " << "detail::Check(sofie_hip_plane_sums_to_average(fCtx, tensor_" << fNPooled << ", static_cast<const int32_t *>(static_cast<const void *>(" << ws
+                << ")), " << count << ", " << fGeo.OH * fGeo.OW << ", " << FloatLiteral(fPoolScale) << "), \"" << opName << " GlobalAveragePool\");\n";
          out << SP << "}\n";
          return out.str();
       }

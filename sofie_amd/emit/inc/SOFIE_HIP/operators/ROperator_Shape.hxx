@@ -149,11 +149,17 @@ public:
       fShapeOut = out;
       model.AddIntermediateTensor(fNOutput, fType, out, fDynamic);
    }
+   bool CanBeView() const override { return true; }
+   void SetView(bool v) override { fIsView = v; }
    std::string Generate_GPU_HIP(std::string opName) override
    {
       opName = "op_" + opName;
       std::stringstream out;
       out << "\n" << SP << "//----  " << Name() << " " << opName << " --> " << ConvertShapeToString(fShapeOut) << "\n";
+      if (fIsView) {
+         out << SP << "// tensor_" << fNOutput << " is a view of tensor_" << fNData << " (same arena offset): nothing to copy\n";
+         return out.str();
+      }
       out << SP << "detail::Check(sofie_hip_copy(fCtx, tensor_" << fNOutput << ", tensor_" << fNData << ", " << BatchScaled(fDynamic, fBytes) << "), \"" << opName << " "
           << Name() << "\");\n";
       return out.str();
@@ -168,6 +174,7 @@ private:
    ETensorType fType = ETensorType::FLOAT;
    std::size_t fBytes = 0;
    bool fDynamic = false;
+   bool fIsView = false;
 };
 
 template <typename T>

@@ -547,12 +547,36 @@ void RModel::PlanMemoryPass(const std::set<std::size_t> &wholeChain)
             opFirst[i] = (int)ch.first;
             opLast[i] = (int)(ch.first + ch.second - 1);
          }
+   // Views: the output of an operator that only hands its input's bytes on is placed ON its input when both live in the pool
+   // (not a graph input or output, which have regions of their own).  The tensor at the root of a chain of views then lives
+   // until the last reader of any of them.
+   std::map<std::string, std::string> viewRoot; // view -> the pool tensor whose bytes it is
+   std::vector<std::pair<std::string, std::size_t>> views; // (view, its operator) in operator order
+   for (std::size_t i = 0; i < fOperators.size(); ++i) {
+      auto &op = fOperators[i];
+      if (!op->CanBeView())
+         continue;
+      op->SetView(false);
+      if (op->GetInputTensorNames().empty() || op->GetOutputTensorNames().size() != 1)
+         continue;
+      const std::string x(op->GetInputTensorNames()[0]), y(op->GetOutputTensorNames()[0]);
+      auto pooledTensor = [&](const std::string &t) {
+         return fIntermediateTensorInfos.count(t) && !fOffsets.count("tensor_" + t) && (!dyn || IsDynamicTensor(t));
+      };
+      if (!pooledTensor(x) || !pooledTensor(y) || opFirst[i] != (int)i || opLast[i] != (int)i)
+         continue;
+      viewRoot[y] = viewRoot.count(x) ? viewRoot[x] : x;
+      views.emplace_back(y, i);
+      op->SetView(true);
+   }
    std::vector<TensorLifeInfo> life;
    std::vector<std::string> names;
    for (std::size_t i = 0; i < fOperators.size(); ++i) {
       for (auto &y : fOperators[i]->GetOutputTensorNames()) {
          if (!fIntermediateTensorInfos.count(y) || fOffsets.count("tensor_" + y))
             continue; // graph outputs are placed above
+         if (viewRoot.count(y))
+            continue; // placed on its root below
          const auto &ti = fIntermediateTensorInfos[y];
          if (dyn && !IsDynamicTensor(y)) { // rare: an intermediate that does not depend on the batch keeps a region of its own
             addStatic("tensor_" + y, tensorBytes(ti));
@@ -560,9 +584,11 @@ void RModel::PlanMemoryPass(const std::set<std::size_t> &wholeChain)
          }
          int last = opLast[i];
          for (std::size_t j = i + 1; j < fOperators.size(); ++j)
-            for (auto &in : fOperators[j]->GetInputTensorNames())
-               if (in == y)
+            for (auto &in : fOperators[j]->GetInputTensorNames()) {
+               auto v = viewRoot.find(std::string(in));
+               if (in == y || (v != viewRoot.end() && v->second == y))
                   last = std::max(last, opLast[j]);
+            }
          life.push_back({opFirst[i], last + 1, dyn ? alignEntry(tensorBytes(ti)) : AlignUp(tensorBytes(ti))});
          names.push_back("tensor_" + y);
       }
@@ -581,6 +607,16 @@ void RModel::PlanMemoryPass(const std::set<std::size_t> &wholeChain)
    for (std::size_t t = 0; t < life.size(); ++t) {
       fPlan.push_back({names[t], poolBase + r.offsets[t], life[t].size, life[t].begin, life[t].end, true, dyn});
       fOffsets[names[t]] = poolBase + r.offsets[t];
+   }
+   for (auto &v : views) {
+      const std::string root = "tensor_" + viewRoot[v.first];
+      for (std::size_t t = 0; t < life.size(); ++t)
+         if (names[t] == root) {
+            const auto &ti = fIntermediateTensorInfos[v.first];
+            fPlan.push_back({"tensor_" + v.first, poolBase + r.offsets[t], dyn ? alignEntry(tensorBytes(ti)) : AlignUp(tensorBytes(ti)), (int)v.second,
+                             life[t].end, true, dyn, true});
+            fOffsets["tensor_" + v.first] = poolBase + r.offsets[t];
+         }
    }
    fPoolBytes = r.total_bytes; // per batch entry when the batch is a run-time parameter
    fPoolBase = poolBase;
@@ -966,7 +1002,7 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    };
    for (auto &p : fPlan)
       gc << "   " << typeOf(p.name) << " *" << p.name << " = nullptr; // " << (p.perBatch ? "per batch entry: offset " : "arena offset ") << p.offset
-         << ", " << p.bytes << " bytes" << (p.pooled ? ", live [" + std::to_string(p.begin) + "," + std::to_string(p.end) + ")" : "") << "\n";
+         << ", " << p.bytes << " bytes" << (p.pooled ? ", live [" + std::to_string(p.begin) + "," + std::to_string(p.end) + ")" : "") << (p.view ? ", a view" : "") << "\n";
    gc << "\n";
    // constructor
    if (safetensors) {

@@ -37,7 +37,7 @@ int main(int argc, char **argv)
             std::cout << "static " << model->GetStaticBytes() << " per_batch_entry " << model->GetBytesPerBatchEntry() << " parameter "
                       << model->GetBatchParamName() << "\n";
          for (auto &p : model->GetMemoryPlan())
-            std::cout << p.name << " " << p.offset << " " << p.bytes << " " << p.begin << " " << p.end << " " << (p.pooled ? 1 : 0)
+            std::cout << p.name << " " << p.offset << " " << p.bytes << " " << p.begin << " " << p.end << " " << (p.view ? 2 : p.pooled ? 1 : 0)
                       << (model->HasDynamicBatch() ? (p.perBatch ? " per_batch_entry" : " static") : "") << "\n";
       }
    } catch (const std::exception &e) {

@@ -153,6 +153,7 @@ SYMBOLS = {
     "sofie_hip_softmax_f32": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, C.c_int64, C.c_int32]),
     "sofie_hip_gemm_chain_f32": (C.c_int, [_P, _P, C.c_int32]),
     "sofie_hip_plane_sums_to_average": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_float]),
+    "sofie_hip_plane_sums_take_average": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_float]),
     "sofie_hip_batchnorm_f32": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "sofie_hip_global_avg_pool_i8": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float]),
     "sofie_hip_conv_weight_i8_packed_bytes": (C.c_size_t, [C.POINTER(ConvDesc)]),

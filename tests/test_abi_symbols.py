@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     assert not missing, missing
     assert set(runtime.SYMBOLS) == set(declared_symbols())
     lib.sofie_hip_abi_version.restype = C.c_int
-    assert lib.sofie_hip_abi_version() == 3
+    assert lib.sofie_hip_abi_version() == 4
 
 
 def test_error_path_without_a_gpu_call():

@@ -59,6 +59,8 @@ def test_plan_alignment_and_liveness(emitted, tmp_path, model):
             overlap_mem = a["offset"] < b["offset"] + b["bytes"] and b["offset"] < a["offset"] + a["bytes"]
             if not overlap_mem:
                 continue
+            if 2 in (a["pooled"], b["pooled"]) and a["offset"] == b["offset"] and a["bytes"] == b["bytes"]:
+                continue    # a view (Reshape, Flatten ...) lies on the tensor it is a view of
             # sharing bytes is allowed only between pooled tensors whose lifetimes are disjoint
             assert a["pooled"] and b["pooled"], (a, b)
             assert a["last"] <= b["first"] or b["last"] <= a["first"], (a, b)
@@ -136,6 +138,36 @@ def _emit(tmp_path, nodes, inputs, outputs, init, name="m"):
     return subprocess.run([em.EMIT, p, str(tmp_path)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
 
 
+def test_reshapes_of_pool_tensors_are_views(tmp_path):
+    """Operators that hand their input's bytes on unchanged generate no copy when input and output both live in the pool: the
+    output is placed on the input, and the tensor at the root of a chain of views lives until the last reader of any of them.
+    A graph input or output has a region of its own, so a Reshape that reads or writes one still copies."""
+    init = {"shape": np.array([4, 6], dtype=np.int64), "shape2": np.array([6, 4], dtype=np.int64)}
+    nodes = [ow.node("Reshape", ["X", "shape2"], ["X2"]),    # 0: reads a graph input: a copy
+             ow.node("Relu", ["X2"], ["A"]),                 # 1
+             ow.node("Flatten", ["A"], ["F"], axis=0),       # 2: a view of A ([1, 24])
+             ow.node("Reshape", ["F", "shape"], ["G"]),      # 3: a view of a view
+             ow.node("Exp", ["G"], ["Y"]),                   # 4
+             ow.node("Neg", ["A"], ["N"]),                   # 5: A is read again behind the views
+             ow.node("Reshape", ["N", "shape"], ["Z"])]      # 6: writes a graph output: a copy
+    p = os.path.join(str(tmp_path), "views.onnx")
+    ow.write(p, nodes, [("X", np.float32, [2, 3, 4])], [("Y", np.float32, [4, 6]), ("Z", np.float32, [4, 6])], init, name="views")
+    out = subprocess.run([em.EMIT, p, str(tmp_path), "--plan"], check=True, stdout=subprocess.PIPE, text=True).stdout.split("\n")
+    rows = {f[0]: dict(offset=int(f[1]), bytes=int(f[2]), first=int(f[3]), last=int(f[4]), kind=int(f[5])) for f in (l.split() for l in out[1:]) if len(f) == 6}
+    assert rows["tensor_F"]["kind"] == 2 and rows["tensor_G"]["kind"] == 2 and rows["tensor_A"]["kind"] == 1 and rows["tensor_X2"]["kind"] == 1
+    assert rows["tensor_F"]["offset"] == rows["tensor_G"]["offset"] == rows["tensor_A"]["offset"]
+    assert rows["tensor_A"]["first"] == 1 and rows["tensor_A"]["last"] == 6      # through Neg (operator 5), past Exp (4), the views' reader
+    # nothing else may take A's bytes while its views are read
+    for n, r in rows.items():
+        if r["kind"] == 1 and n != "tensor_A" and r["offset"] < rows["tensor_A"]["offset"] + rows["tensor_A"]["bytes"] and \
+           rows["tensor_A"]["offset"] < r["offset"] + r["bytes"]:
+            assert r["last"] <= 1 or r["first"] >= 6, (n, r)
+    body = ops_body(open(os.path.join(str(tmp_path), "views_GPU_HIP.hxx")).read())
+    assert "tensor_F is a view of tensor_A" in body and "tensor_G is a view of tensor_F" in body
+    assert body.count("sofie_hip_copy(") == 2 and "sofie_hip_copy(fCtx, tensor_X2, tensor_X" in body and "sofie_hip_copy(fCtx, tensor_Z, tensor_N" in body
+    assert "SOFIE_ACT_EXP" in body and "tensor_G" in body[body.index("SOFIE_ACT_EXP") - 200:body.index("SOFIE_ACT_EXP") + 200]
+
+
 def test_unsupported_operator_is_refused_by_name(tmp_path):
     r = _emit(tmp_path, [ow.node("LSTM", ["X"], ["Y"])], [("X", np.float32, [1, 4])], [("Y", np.float32, [1, 4])], {})
     assert r.returncode != 0 and "LSTM" in r.stdout
@@ -202,17 +234,21 @@ def test_global_average_pool_joins_a_convolution_whose_planes_the_runtime_can_su
     txt = read(emitted, "Int8_CNN_plane_sums")
     body = ops_body(txt)
     assert body.count("sofie_hip_conv_i8(") == 2 and body.count("a.out = SOFIE_I8OUT_I8_PLANE_SUMS") == 1
-    assert "sofie_hip_global_avg_pool_i8(" not in body and body.count("sofie_hip_plane_sums_to_average(") == 1
-    # cleared, summed into, averaged: in that order, on the operator's own workspace (2 images x 128 channels of int32)
-    order = [body.index(k) for k in ("sofie_hip_fill_zero(fCtx, workspace_op_2, static_cast<std::size_t>(256) * 4)", "a.Y = workspace_op_2",
-                                     "sofie_hip_conv_i8(fCtx, &d, &a), \"op_2", "sofie_hip_plane_sums_to_average(fCtx, tensor_")]
-    assert order[1] < order[0] < order[2] < order[3]
-    assert ", 256, 256, " in body[order[3]:order[3] + 300]        # 256 sums, planes of 256 pixels
+    assert "sofie_hip_global_avg_pool_i8(" not in body and body.count("sofie_hip_plane_sums_take_average(") == 1
+    # a buffer of the operator's own (2 images x 128 channels of int32), cleared once in the constructor; every inference sums
+    # into it and the averaging call clears it again behind its read: no clearing launch per inference
+    assert "sofie_hip_fill_zero(" not in body and "workspace_op_2" not in body
+    ctor = txt[txt.index("Session(std::string filename"):txt.index("void doInfer(")]
+    assert ctor.count("sofie_hip_fill_zero(fCtx, planesums_") == 1 and ", 1024), " in ctor[ctor.index("sofie_hip_fill_zero(fCtx, planesums_"):][:200]
+    order = [body.index(k) for k in ("a.Y = planesums_", "sofie_hip_conv_i8(fCtx, &d, &a), \"op_2", "sofie_hip_plane_sums_take_average(fCtx, tensor_")]
+    assert order[0] < order[1] < order[2]
+    assert ", 256, 256, " in body[order[2]:order[2] + 300]        # 256 sums, planes of 256 pixels
     # planes of 144 pixels (12 x 12) stay with the stand-alone kernel
     assert "PLANE_SUMS" not in read(emitted, "Config5_int8_CNN_small")
     # with a run-time batch the sums are a per-batch-entry workspace and the counts scale with the batch
     dyn = ops_body(read(emitted, "Dynamic_int8_CNN_plane_sums"))
     assert "a.out = SOFIE_I8OUT_I8_PLANE_SUMS" in dyn and "sofie_batch * 128" in dyn
+    assert "sofie_hip_fill_zero(fCtx, workspace_op_" in dyn and "sofie_hip_plane_sums_to_average(" in dyn
 
 
 def test_qlinear_matmul_and_conv_integer_become_one_launch_each(emitted):
@@ -291,9 +327,13 @@ def test_per_batch_entry_plan_scales_without_overlap(emitted, tmp_path):
     assert {"tensor_X", "tensor_Y", "tensor_Q", "tensor_R0", "tensor_R3"} <= names and not any(n.startswith("packed_") for n in names)
     # per-entry offsets are multiples of 16, so that capacity (a multiple of 16) times the offset is a multiple of 256
     assert all(r["offset"] % 16 == 0 and r["offset"] + r["bytes"] <= entry_bytes for r in per)
+    views = [r for r in per if r["pooled"] == 2]
+    assert [r["name"] for r in views] == ["tensor_F"]           # the Flatten behind the average pool: placed on its input
     for i, a in enumerate(per):
         for b in per[i + 1:]:
             if a["offset"] < b["offset"] + b["bytes"] and b["offset"] < a["offset"] + a["bytes"]:
+                if 2 in (a["pooled"], b["pooled"]) and a["offset"] == b["offset"] and a["bytes"] == b["bytes"]:
+                    continue    # a view and the tensor it is a view of (or another view of it)
                 assert a["pooled"] and b["pooled"] and (a["last"] <= b["first"] or b["last"] <= a["first"]), (a, b)
 
 
@@ -349,8 +389,9 @@ def test_one_to_one_operators_join_their_producer(emitted, tmp_path):
 
 def test_equal_shaped_adds_join_the_store_of_their_producer(emitted, tmp_path):
     body = ops_body(read(emitted, "ResidualBlock"))
-    # 8 operators in the graph, 4 launches: Conv(+Add+Relu), GlobalAveragePool, Flatten, Gemm(+Add+Sigmoid)
-    assert body.count("detail::Check(") == 4 and "sofie_hip_add_f32" not in body and "sofie_hip_unary_f32" not in body
+    # 8 operators in the graph, 3 launches: Conv(+Add+Relu), GlobalAveragePool, Gemm(+Add+Sigmoid); the Flatten is a view
+    assert body.count("detail::Check(") == 3 and "sofie_hip_add_f32" not in body and "sofie_hip_unary_f32" not in body
+    assert "is a view of tensor_" in body and "sofie_hip_copy(" not in body
     assert "SOFIE_ACT_RELU, 0.0f, tensor_r0, nullptr, tensor_X)" in body
     assert "d.residual = tensor_Z;" in body and "d.act = SOFIE_ACT_SIGMOID" in body
     # a broadcasting Add (bias-like operand of another shape) and an Add behind an activation stay operators of their own

@@ -172,7 +172,7 @@ def test_emitted_int8_cnn_whose_last_convolution_sums_its_planes(rt):
     assert np.abs(got - want).max() <= 1e-5 * max(1.0, float(np.abs(want).max()))
     assert np.abs(want).max() > 1e-3
     txt = open(os.path.join(em.OUT, "Int8_CNN_plane_sums_GPU_HIP.hxx")).read()
-    assert txt.count("SOFIE_I8OUT_I8_PLANE_SUMS") == 1 and "sofie_hip_plane_sums_to_average" in txt and "sofie_hip_global_avg_pool_i8" not in txt
+    assert txt.count("SOFIE_I8OUT_I8_PLANE_SUMS") == 1 and "sofie_hip_plane_sums_take_average" in txt and "sofie_hip_global_avg_pool_i8" not in txt
 
 
 def test_model_built_through_the_api_external_stream_option(rt):
