@@ -8,16 +8,24 @@
 //     of OW + 2 pixels of 64 channels (zeros outside the image), is loaded with global_load_lds into one of two buffers while
 //     the tile before it is multiplied: the only loads of the loop, 9 times fewer bytes than tap-by-tap gathering;
 //   * the A fragment of tap (ky, kx) is read from the patch at a tap offset, the B fragment from the resident weights: no
-//     barrier inside a tile.  The eight waves meet once per tile, and one of the two waves of every SIMD stores its tile after
-//     the next tile's barrier: one wave's conversion and store run under the other's MFMAs;
+//     barrier inside a tile.  The eight waves meet once per tile;
 //   * pixels and weight rows are 64 + 32 (576 + 32) bytes apart in LDS: records 96 bytes (mod 256) apart are read by
 //     ds_read_b128 at the full rate from any starting record (measured: 237 B/clk; 80, 112, 144 or 592 bytes apart: 123), so no
-//     swizzle is needed and every fragment address is a lane constant plus a uniform offset.
-// Workgroup = 8 waves (4 x 2), wave tile 64 x 64 (v_mfma_i32_16x16x64_i8, 64 accumulators), store from registers.
+//     swizzle is needed and every fragment address is a lane constant plus a uniform offset;
+//   * a wave's 64 x 64 tile is worked in two halves of 64 x 32, each over all nine taps: 32 accumulators per half, so TWO
+//     halves fit the registers, and the half finished last is converted and stored between the MFMAs of the half in work,
+//     one output element (four vector instructions) per pair of MFMAs.  The MFMAs run through the halves and through the
+//     tile boundaries: during the last tap of a half the first fragments of the next one are read.
+// Workgroup = 8 waves (4 x 2), v_mfma_i32_16x16x64_i8, store from registers.
 //
-// What bounds it (batch 256 of 64 x 64 images, 70 us): not the matrix cores (33 us of MFMA at the clock it runs at) and not
-// the LDS reads (the same time with the fragments of taps 2..8 not read at all), but the memory side: 134 MB of output and
-// 67 MB of input (100 MB with the halo rows) per launch.  With one MFMA in sixteen the launch still takes 52 us.
+// What bounds it (batch 256 of 64 x 64 images, 67 us against 33 us of MFMA at the clock it runs at): the matrix cores, the LDS
+// reads of the fragments and the vector instructions of the conversion each need about half of the launch and do not overlap
+// freely.  Measured: the loop without store and conversion 57 us; with one MFMA in eight 48 us; neither 31 us (864 KB of
+// fragment reads per tile and CU, 208 B/clk: near the LDS's rate); a wave of vector instructions beside a wave of MFMAs on one
+// SIMD runs at 61 % of its own rate and does not slow the MFMAs.  The HBM traffic (134 MB written, 100 MB read) is not the
+// bound: the same time with every tile stored to one place.  Wave tiles of 64 x 64 as ONE piece (one set of accumulators, the
+// store of one wave of each SIMD delayed behind the next barrier so that it runs under the other's MFMAs) read a third fewer
+// fragments and take 69 - 70 us; sixteen waves of 32 x 64 take 72 us.
 #pragma once
 #include "mfma8_gemm_persist.hpp"
 
@@ -65,19 +73,8 @@ __global__ __launch_bounds__(512) void conv_i8_resident_kernel(ResidentConv g, c
       __builtin_amdgcn_global_load_lds((global_void_t *)src, (lds_void_t *)(wl + (j * NW + wave) * 1024), 16, 0, 0);
    }
 
-   // ---- the patch loader: LDS chunk q of a buffer holds chunk q % 6 of patch pixel q / 6 (chunks 4 and 5 are padding)
-   int p_off[PLD];      // byte offset of the lane's chunk from the patch's first pixel (row -pad_h0 of the tile, column -pad_w0)
-   int p_row[PLD];      // its patch row, or a large number when the chunk is padding or its column lies outside the image
-#pragma unroll
-   for (int j = 0; j < PLD; ++j) {
-      const int q = (j * NW + wave) * 64 + lane;
-      const int p = q / PCH, c = q - p * PCH;
-      const int pr = p / PW, pc = p - pr * PW;
-      const int iw = pc - g.pad_w0;
-      const bool ok = p < PP && c < 4 && (unsigned)iw < (unsigned)g.W;
-      p_off[j] = (pr * g.W + iw) * g.C + c * 16;
-      p_row[j] = ok ? pr : (1 << 20);
-   }
+   // ---- the patch loader: LDS chunk q of a buffer holds chunk q % 6 of patch pixel q / 6 (chunks 4 and 5 are padding).  What a
+   // lane loads is worked out again for every patch (from the lane number, made opaque): ten registers less across the tile loop.
    auto tile_of = [&](int it, int &m0, int &img, int &oh0) {
       const int T = (it < my_tiles ? it : my_tiles - 1) * nwg + bid;
       m0 = T * 256;
@@ -87,10 +84,16 @@ __global__ __launch_bounds__(512) void conv_i8_resident_kernel(ResidentConv g, c
    auto load_patch = [&](int buf, int img, int oh0) {
       const int ih0 = oh0 - g.pad_h0;
       const int8_t *origin = g.X + ((ptrdiff_t)img * g.H + ih0) * (ptrdiff_t)g.W * g.C; // may lie before X: only added to offsets of valid rows
+      int ln = lane;
+      asm volatile("" : "+v"(ln));
 #pragma unroll
       for (int j = 0; j < PLD; ++j) {
-         const bool ok = (unsigned)(ih0 + p_row[j]) < (unsigned)g.H;
-         const int8_t *src = ok ? origin + p_off[j] : (const int8_t *)conv_zero_page;
+         const int q = (j * NW + wave) * 64 + ln;
+         const int p = q / PCH, c = q - p * PCH;
+         const int pr = p / PW, pc = p - pr * PW;
+         const int iw = pc - g.pad_w0;
+         const bool ok = p < PP && c < 4 && (unsigned)iw < (unsigned)g.W && (unsigned)(ih0 + pr) < (unsigned)g.H;
+         const int8_t *src = ok ? origin + ((pr * g.W + iw) * g.C + c * 16) : (const int8_t *)conv_zero_page;
          __builtin_amdgcn_global_load_lds((global_void_t *)src, (lds_void_t *)(patch + buf * PBYTES + (j * NW + wave) * 1024), 16, 0, 0);
       }
    };
@@ -104,103 +107,175 @@ __global__ __launch_bounds__(512) void conv_i8_resident_kernel(ResidentConv g, c
       const int p = wm * TM + i * R;
       a_blk[i] = ((p >> g.ow_shift) * PW + (p & (g.OW - 1))) * PIX;
    }
-   auto read_tap = [&](const int8_t *pbuf, int tap_off_a, int tap, frag_t(&fa)[MT], frag_t(&fb)[NT]) {
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-         fb[j].c[0] = *(const v4i *)(wl + b_lane + j * R * WROW + tap * 64);
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-         fa[i].c[0] = *(const v4i *)(pbuf + a_lane + a_blk[i] + tap_off_a);
-   };
 
    int m_cur, img, oh0;
    tile_of(0, m_cur, img, oh0);
    load_patch(0, img, oh0);
    uint32_t col_words[EPI::kColWords];
    ep.load_column_for_registers(wn * TN + lane, col_words); // one column tile: the constants are the same for every tile
-   constexpr bool kBias = EPI::kBiasInAccumulator;
-   acc_t acc[MT][NT];
-   // Half of the waves, one of the two on every SIMD (waves w and w + 4 share one), store a tile only after the NEXT tile's
-   // barrier: their conversion and store then run while the other wave of the SIMD multiplies, and the other way round
-   // later in the tile.  Every wave passes the same number of barriers (one per tile and one more).
-   const bool late_store = wave >= NW / 2;
-   auto store_tile = [&](int m_tile) {
-      ep.dispatch_for_registers([&](auto mode) {
-         tile_store_or_sum_from_registers<decltype(mode)::value, MMA, MT, NT>(ep, acc, m_tile + wm * TM, wn * TN, lane, col_words);
-      });
-   };
-   int m_prev = m_cur;
-   for (int it = 0; it <= my_tiles; ++it) {
-      // the patch of this tile has landed for every wave, and every wave is done multiplying the tile before (whose buffer the
-      // next patch goes to).  A wave's loads of the patch are older than the stores it has issued since, which may stay in
-      // flight: loads return in order, so "at most as many operations outstanding as one tile's stores" means the loads are done.
-      if (it == 0 || !ep.stores_one_byte_rows())
-         wait_vmcnt<0>();
-      else
-         wait_vmcnt<MT>();
-      __builtin_amdgcn_s_barrier();
-      int m_nxt, img_n, oh_n;
-      tile_of(it + 1, m_nxt, img_n, oh_n);
-      if (it < my_tiles)
-         load_patch((it + 1) & 1, img_n, oh_n);
-      if (late_store && it > 0)
-         store_tile(m_prev);
-      if (it == my_tiles)
-         break;
-      // accumulators: the bias of the lane's columns (or zero)
+   static_assert(EPI::kBiasInAccumulator && MMA::ACC == 4, "integer epilogue: the accumulators start at the bias");
+   char *const out = ep.out_base();
+   // The store mode is fixed for the launch: the whole tile loop exists once per mode, so that a tap's MFMAs and the part of the
+   // store that goes with them are one straight piece of code.
+   ep.dispatch_for_registers([&](auto mode_c) {
+      constexpr int MODE = decltype(mode_c)::value;
+      constexpr int ESZ = EPI::template out_bytes<MODE>();
+      constexpr int HN = NT / 2; // column blocks of a half
+      // scale and bias of the lane's columns (4 per column block), once for the launch
+      typename EPI::template col_params<4> prm[NT];
+      acc_t acc0[NT];
       {
          int first_col_addr = lk * 16;
-         asm volatile("" : "+v"(first_col_addr));
-         static_for<NT>([&](auto cj) {
-            constexpr int j = decltype(cj)::value;
-            acc_t b = {0, 0, 0, 0};
-            if constexpr (kBias) {
 #pragma unroll
-               for (int v = 0; v < 4; ++v)
-                  b[v] = __builtin_amdgcn_ds_bpermute(first_col_addr + (j * R + v) * 4, (int)col_words[EPI::kBiasWord]);
+         for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+               uint32_t w[EPI::kColWords];
+#pragma unroll
+               for (int k = 0; k < EPI::kColWords; ++k)
+                  w[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(first_col_addr + (j * R + v) * 4, (int)col_words[k]);
+               acc0[j][v] = (int)w[EPI::kBiasWord];
+               w[EPI::kBiasWord] = 0;
+               EPI::template set_column<4>(prm[j], v, w);
             }
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-               acc[i][j] = b;
-         });
       }
-      const int8_t *pbuf = patch + (it & 1) * PBYTES;
-      // fragments of three taps in registers: tap t is multiplied while those of tap t + 2 are on their way (the reads of one
-      // tap ahead would have the 16 MFMAs of a tap to arrive in: too short with eight waves reading)
-      frag_t fa[3][MT], fb[3][NT];
-      __builtin_amdgcn_sched_barrier(0);
-      read_tap(pbuf, 0, 0, fa[0], fb[0]);
-      read_tap(pbuf, (1 / KW * PW + 1 % KW) * PIX, 1, fa[1], fb[1]);
-      static_for<NTAPS>([&](auto tc) {
-         constexpr int tap = decltype(tc)::value;
-         constexpr int cur = tap % 3;
-         // (the scheduling fences keep the reads where they are written: left alone, the compiler sinks each one to just in
-         // front of its first use and waits for it there, every four MFMAs)
-         __builtin_amdgcn_sched_barrier(0);
-         if constexpr (tap + 2 < NTAPS) {
-            constexpr int ky = (tap + 2) / KW, kx = (tap + 2) % KW;
-            read_tap(pbuf, (ky * PW + kx) * PIX, tap + 2, fa[(tap + 2) % 3], fb[(tap + 2) % 3]);
+      // A wave's 64 x 64 tile is worked in two HALVES of 64 x 32 (column blocks 2 h, 2 h + 1), each over all nine taps, into
+      // acc[h]: 32 accumulators per half, so that two halves fit the registers and the one finished last is converted and
+      // stored, slice by slice, between the MFMAs of the one in work.  (The A fragments are read once per half: half as many
+      // LDS reads again.)
+      acc_t acc[2][MT][HN];
+      uint32_t packed[MT][NT]; // 1-byte modes: the converted dwords of a tile until its second half completes the rows
+      // Slice sl (0 .. 8 MT - 1) of the store of half h: one output element of a 1-byte store (convert, scale, clamp,
+      // round-and-place: four vector instructions); the second half's last slice of a row block exchanges the dwords between the
+      // four lanes of a row (see tile_store_from_registers) and stores 16 bytes per lane.  4-byte outputs convert and store a
+      // column block (16 bytes per lane) in every fourth slice.
+      auto store_slice = [&](auto h_c, auto slice_c, int m_tile) {
+         constexpr int h = decltype(h_c)::value, sl = decltype(slice_c)::value;
+         constexpr int i = sl / (4 * HN), jj = (sl / 4) % HN, j = HN * h + jj, v = sl % 4;
+         typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+         if constexpr (ESZ == 4) {
+            if constexpr (v == 3) {
+               const int m = m_tile + wm * TM + i * R + lr;
+               uint32_t w[4];
+               ep.template pack4<MODE, 4, true>(prm[j], 0, acc[h][i][jj][0], acc[h][i][jj][1], acc[h][i][jj][2], acc[h][i][jj][3], w);
+               const u4 x = {w[0], w[1], w[2], w[3]};
+               __builtin_nontemporal_store(x, (u4 *)(out + ep.out_index_of_plain_rows(m, wn * TN + j * R + lk * 4) * 4));
+            }
+         } else {
+            const float c = ep.template clamp1_short<MODE, true>(acc[h][i][jj][v], 0, prm[j].s[v]);
+            EPI::template place_i8_byte<v>(packed[i][j], c);
+            if constexpr (h == 1 && jj == HN - 1 && v == 3) {
+               const int m = m_tile + wm * TM + i * R + lr;
+               auto s02 = __builtin_amdgcn_permlane32_swap(packed[i][0], packed[i][2], false, false);
+               auto s13 = __builtin_amdgcn_permlane32_swap(packed[i][1], packed[i][3], false, false);
+               auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+               auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+               const u4 x = {t01[0], t01[1], t23[0], t23[1]};
+               __builtin_nontemporal_store(x, (u4 *)(out + ep.out_index_of_plain_rows(m, wn * TN + lk * 16)));
+            }
          }
-         static_for<NT>([&](auto cj) {
-            constexpr int j = decltype(cj)::value;
-            static_for<MT>([&](auto ci) {
-               constexpr int i = (j & 1) ? MT - 1 - decltype(ci)::value : decltype(ci)::value;
-               acc[i][j] = MMA::mma(fb[cur][j], fa[cur][i], acc[i][j]);
+      };
+      constexpr int STORES = ESZ == 4 ? MT * NT : MT; // memory stores of one tile per wave
+      constexpr int SLICES = 4 * MT * HN;             // of one half
+      constexpr int GROUPS = MT * HN / 2;             // of a tap: two MFMAs each
+      constexpr int PER_GROUP = (SLICES + (NTAPS - 1) * GROUPS - 1) / ((NTAPS - 1) * GROUPS); // slices per group, the last tap left free
+      // The MFMAs run through the halves and the tile boundaries.  During the last tap of a half the first fragments of the
+      // next one are read (of the next tile's patch after the second half).  The workgroup meets once per tile, in front of
+      // that last tap of the second half: by then a wave holds the last fragments of this tile's patch in registers and has
+      // its own loads of the next patch back, so past the barrier the next patch is complete for everybody and this tile's
+      // buffer is free for the patch after the next.
+      frag_t fa[2][MT], fb[2][HN]; // fragments of the tap in work and of the one after it; nine taps: the roles swap per half
+      auto half_body = [&](auto h_c, auto prev_c, int it) {
+         constexpr int h = decltype(h_c)::value;
+         constexpr bool prev = decltype(prev_c)::value; // a half before this one is waiting to be stored
+         // the half before: the other half of this tile, or the second half of the tile before
+         const int m_prev = ((h ? it : it - 1) * nwg + bid) * 256;
+         const int8_t *pbuf = patch + (it & 1) * PBYTES, *pnext = patch + ((it + 1) & 1) * PBYTES;
+         static_for<NTAPS>([&](auto tc) {
+            constexpr int tap = decltype(tc)::value;
+            constexpr int cur = (tap + h) % 2;
+            constexpr bool last = tap + 1 == NTAPS;
+            constexpr int ntap = last ? 0 : tap + 1;     // the tap whose fragments are read meanwhile (of the next half after the last one)
+            constexpr int nh = last ? 1 - h : h;         // and its half
+            constexpr int ky = ntap / KW, kx = ntap % KW;
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (last && h == 1) {
+               if (it + 1 < my_tiles) { // (uniform)
+                  // a wave's loads of the next patch are older than the stores it has issued since, which may stay in flight
+                  wait_vmcnt<STORES>();
+                  __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this tap's fragments
+                  __builtin_amdgcn_s_barrier();
+                  if (it + 2 < my_tiles) {
+                     int m2, img2, oh2;
+                     tile_of(it + 2, m2, img2, oh2);
+                     load_patch(it & 1, img2, oh2);
+                  }
+               }
+               __builtin_amdgcn_sched_barrier(0);
+            }
+            const int8_t *rbuf = (last && h == 1) ? pnext : pbuf;
+            // A tap in groups, each fenced so that it is issued as written: two MFMAs and slices of the store of the half
+            // before, then two LDS reads of the next tap's fragments (all of them in the first groups, so that the wait in
+            // front of the next tap's first MFMA finds them done).  (Left to the scheduler, the store's instructions end up
+            // in runs of thirty to fifty between runs of MFMAs.)
+            static_for<GROUPS>([&](auto gc) {
+               constexpr int grp = decltype(gc)::value;
+               static_for<2>([&](auto qc) {
+                  constexpr int n = grp * 2 + decltype(qc)::value;
+                  constexpr int jj = n / MT, i = (jj & 1) ? MT - 1 - n % MT : n % MT;
+                  if constexpr (tap == 0)
+                     acc[h][i][jj] = MMA::mma(fb[cur][jj], fa[cur][i], acc0[HN * h + jj]);
+                  else
+                     acc[h][i][jj] = MMA::mma(fb[cur][jj], fa[cur][i], acc[h][i][jj]);
+               });
+               if constexpr (prev && !last) {
+                  static_for<PER_GROUP>([&](auto sc) {
+                     constexpr int sl = (tap * GROUPS + grp) * PER_GROUP + decltype(sc)::value;
+                     if constexpr (sl < SLICES)
+                        store_slice(std::integral_constant<int, 1 - h>{}, std::integral_constant<int, sl>{}, m_prev);
+                  });
+               }
+               __builtin_amdgcn_sched_barrier(0);
+               if constexpr (2 * grp < MT + HN) {
+                  static_for<2>([&](auto rc) {
+                     constexpr int f = 2 * grp + decltype(rc)::value;
+                     if constexpr (f < HN)
+                        fb[1 - cur][f].c[0] = *(const v4i *)(wl + b_lane + (HN * nh + f) * R * WROW + ntap * 64);
+                     else if constexpr (f < HN + MT)
+                        fa[1 - cur][f - HN].c[0] = *(const v4i *)(rbuf + a_lane + a_blk[f - HN] + (ky * PW + kx) * PIX);
+                  });
+                  __builtin_amdgcn_sched_barrier(0);
+               }
             });
          });
-         if constexpr (tap + 2 < NTAPS) {
-            static_for<MT + NT>([&](auto gc) {
-               __builtin_amdgcn_sched_group_barrier(0x008, (MT * NT) / (MT + NT), 0);
-               __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            });
-         }
-         __builtin_amdgcn_sched_barrier(0);
-      });
-      if (!late_store)
-         store_tile(m_cur);
-      m_prev = m_cur;
-      m_cur = m_nxt;
-   }
+      };
+      constexpr std::integral_constant<int, 0> h0{};
+      constexpr std::integral_constant<int, 1> h1{};
+      // the patches of the first two tiles, the first tap of the first half
+      {
+         int m1, img1, oh1;
+         tile_of(1, m1, img1, oh1);
+         if (1 < my_tiles)
+            load_patch(1, img1, oh1);
+         wait_vmcnt<0>();
+         __builtin_amdgcn_s_barrier();
+#pragma unroll
+         for (int f = 0; f < HN; ++f)
+            fb[0][f].c[0] = *(const v4i *)(wl + b_lane + f * R * WROW);
+#pragma unroll
+         for (int i = 0; i < MT; ++i)
+            fa[0][i].c[0] = *(const v4i *)(patch + a_lane + a_blk[i]);
+      }
+      half_body(h0, std::false_type{}, 0);
+      half_body(h1, std::true_type{}, 0);
+      for (int it = 1; it < my_tiles; ++it) {
+         half_body(h0, std::true_type{}, it);
+         half_body(h1, std::true_type{}, it);
+      }
+      // the last half: nothing left to multiply
+      const int m_last = ((my_tiles - 1) * nwg + bid) * 256;
+      static_for<SLICES>([&](auto sc) { store_slice(h1, sc, m_last); });
+   });
    wait_vmcnt<0>();
 }
 

@@ -228,37 +228,53 @@ struct I8Epilogue {
       const float c = __builtin_amdgcn_fmed3f(v, lo, 127.0f);
       return __float_as_uint(c + 12582912.0f);
    }
+   // One element of pack4_short: bias (unless it sits in the accumulator), floor, scale, quotient, clamp to [lo, 127].
+   template <int OUT, bool BIAS_DONE>
+   __device__ __forceinline__ float clamp1_short(int acc, int b, float s) const
+   {
+      static_assert(requantizes<OUT>() || divides<OUT>(), "1-byte outputs");
+      int acc_floor = relu_acc ? 0 : (int)0x80000000;
+      asm volatile("" : "+s"(acc_floor)); // kept a number (see pack4)
+      const float lo = (requantizes<OUT>() && relu_out) ? 0.0f : -128.0f;
+      if (!BIAS_DONE)
+         acc += b;
+      if (OUT != kOutI8NoFloor)
+         acc = acc > acc_floor ? acc : acc_floor;
+      float v = mul_nofma((float)acc, s);
+      if (divides<OUT>())
+         v = quotient<OUT>(v);
+      return __builtin_amdgcn_fmed3f(v, lo, 127.0f);
+   }
+   // i8_bits() of a clamped element, the addition writing its low byte straight into byte K of the dword (sub-dword
+   // destination select): no byte permutes.  K = 0 starts the dword.
+   template <int K>
+   static __device__ __forceinline__ void place_i8_byte(uint32_t &r, float c)
+   {
+      const float magic = 12582912.0f;
+      if constexpr (K == 0)
+         asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(r) : "v"(c), "v"(magic));
+      else if constexpr (K == 1)
+         asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(r) : "v"(c), "v"(magic));
+      else if constexpr (K == 2)
+         asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(r) : "v"(c), "v"(magic));
+      else
+         asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(r) : "v"(c), "v"(magic));
+   }
    // pack4 for the 1-byte outputs with the short conversion.  float(acc) * s is NaN only for a scale that is NaN, or
    // infinite against an accumulator of 0; load_column_for_registers() below replaces such scales by ones that give the same results
    // without NaN.
    template <int OUT, int C, bool BIAS_DONE = false>
    __device__ __forceinline__ void pack4_short(const col_params<C> &p, int q, int a0, int a1, int a2, int a3, uint32_t *w) const
    {
-      static_assert(requantizes<OUT>() || divides<OUT>(), "1-byte outputs");
-      int acc[4] = {a0, a1, a2, a3};
-      float c[4];
-      int acc_floor = relu_acc ? 0 : (int)0x80000000;
-      asm volatile("" : "+s"(acc_floor)); // kept a number (see pack4)
-      const float lo = (requantizes<OUT>() && relu_out) ? 0.0f : -128.0f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-         if (!BIAS_DONE)
-            acc[i] += p.b[4 * q + i];
-         if (OUT != kOutI8NoFloor)
-            acc[i] = acc[i] > acc_floor ? acc[i] : acc_floor;
-         float v = mul_nofma((float)acc[i], p.s[4 * q + i]);
-         if (divides<OUT>())
-            v = quotient<OUT>(v);
-         c[i] = __builtin_amdgcn_fmed3f(v, lo, 127.0f);
-      }
-      // i8_bits() of the four, each addition writing its low byte straight into its place of the dword (sub-dword
-      // destination select): no byte permutes
-      const float magic = 12582912.0f;
+      const float c0 = clamp1_short<OUT, BIAS_DONE>(a0, p.b[4 * q + 0], p.s[4 * q + 0]);
+      const float c1 = clamp1_short<OUT, BIAS_DONE>(a1, p.b[4 * q + 1], p.s[4 * q + 1]);
+      const float c2 = clamp1_short<OUT, BIAS_DONE>(a2, p.b[4 * q + 2], p.s[4 * q + 2]);
+      const float c3 = clamp1_short<OUT, BIAS_DONE>(a3, p.b[4 * q + 3], p.s[4 * q + 3]);
       uint32_t r;
-      asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(r) : "v"(c[0]), "v"(magic));
-      asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(r) : "v"(c[1]), "v"(magic));
-      asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(r) : "v"(c[2]), "v"(magic));
-      asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(r) : "v"(c[3]), "v"(magic));
+      place_i8_byte<0>(r, c0);
+      place_i8_byte<1>(r, c1);
+      place_i8_byte<2>(r, c2);
+      place_i8_byte<3>(r, c3);
       w[0] = r;
    }
    // load_column for the store from registers.  Its 1-byte conversions (pack4_short, quantize4) need the scale made safe:
