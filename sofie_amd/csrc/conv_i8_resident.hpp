@@ -73,8 +73,19 @@ __global__ __launch_bounds__(512) void conv_i8_resident_kernel(ResidentConv g, c
       __builtin_amdgcn_global_load_lds((global_void_t *)src, (lds_void_t *)(wl + (j * NW + wave) * 1024), 16, 0, 0);
    }
 
-   // ---- the patch loader: LDS chunk q of a buffer holds chunk q % 6 of patch pixel q / 6 (chunks 4 and 5 are padding).  What a
-   // lane loads is worked out again for every patch (from the lane number, made opaque): ten registers less across the tile loop.
+   // ---- the patch loader: LDS chunk q of a buffer holds chunk q % 6 of patch pixel q / 6 (chunks 4 and 5 are padding)
+   int p_off[PLD];      // byte offset of the lane's chunk from the patch's first pixel (row -pad_h0 of the tile, column -pad_w0)
+   int p_row[PLD];      // its patch row, or a large number when the chunk is padding or its column lies outside the image
+#pragma unroll
+   for (int j = 0; j < PLD; ++j) {
+      const int q = (j * NW + wave) * 64 + lane;
+      const int p = q / PCH, c = q - p * PCH;
+      const int pr = p / PW, pc = p - pr * PW;
+      const int iw = pc - g.pad_w0;
+      const bool ok = p < PP && c < 4 && (unsigned)iw < (unsigned)g.W;
+      p_off[j] = (pr * g.W + iw) * g.C + c * 16;
+      p_row[j] = ok ? pr : (1 << 20);
+   }
    auto tile_of = [&](int it, int &m0, int &img, int &oh0) {
       const int T = (it < my_tiles ? it : my_tiles - 1) * nwg + bid;
       m0 = T * 256;
@@ -84,28 +95,26 @@ __global__ __launch_bounds__(512) void conv_i8_resident_kernel(ResidentConv g, c
    auto load_patch = [&](int buf, int img, int oh0) {
       const int ih0 = oh0 - g.pad_h0;
       const int8_t *origin = g.X + ((ptrdiff_t)img * g.H + ih0) * (ptrdiff_t)g.W * g.C; // may lie before X: only added to offsets of valid rows
-      int ln = lane;
-      asm volatile("" : "+v"(ln));
 #pragma unroll
       for (int j = 0; j < PLD; ++j) {
-         const int q = (j * NW + wave) * 64 + ln;
-         const int p = q / PCH, c = q - p * PCH;
-         const int pr = p / PW, pc = p - pr * PW;
-         const int iw = pc - g.pad_w0;
-         const bool ok = p < PP && c < 4 && (unsigned)iw < (unsigned)g.W && (unsigned)(ih0 + pr) < (unsigned)g.H;
-         const int8_t *src = ok ? origin + ((pr * g.W + iw) * g.C + c * 16) : (const int8_t *)conv_zero_page;
+         const bool ok = (unsigned)(ih0 + p_row[j]) < (unsigned)g.H;
+         const int8_t *src = ok ? origin + p_off[j] : (const int8_t *)conv_zero_page;
          __builtin_amdgcn_global_load_lds((global_void_t *)src, (lds_void_t *)(patch + buf * PBYTES + (j * NW + wave) * 1024), 16, 0, 0);
       }
    };
 
-   // ---- fragment addresses: a lane constant plus uniform offsets
-   const int a_lane = lr * PIX + lk * 16;
+   // ---- fragment addresses.  B: a lane constant plus compile-time offsets.  A: one register per (row of taps, row block) holding
+   // the LDS byte offset of the lane's chunk at tap (ky, 0) in the patch buffer of the tile in work, so that a fragment read is
+   // that register plus a compile-time kx * PIX; the registers move to the other buffer once per tile (one addition each).
    const int b_lane = (wn * TN + lr) * WROW + lk * 16;
-   int a_blk[MT]; // patch byte offset of the first pixel of the wave's i-th block of 16 output pixels, tap (0, 0)
+   int a_row[KH][MT];
 #pragma unroll
    for (int i = 0; i < MT; ++i) {
       const int p = wm * TM + i * R;
-      a_blk[i] = ((p >> g.ow_shift) * PW + (p & (g.OW - 1))) * PIX;
+      const int blk = ((p >> g.ow_shift) * PW + (p & (g.OW - 1))) * PIX; // first pixel of the wave's i-th block of 16 output pixels, tap (0, 0)
+#pragma unroll
+      for (int ky = 0; ky < KH; ++ky)
+         a_row[ky][i] = WBYTES + blk + ky * PW * PIX + lr * PIX + lk * 16;
    }
 
    int m_cur, img, oh0;
@@ -190,7 +199,6 @@ __global__ __launch_bounds__(512) void conv_i8_resident_kernel(ResidentConv g, c
          constexpr bool prev = decltype(prev_c)::value; // a half before this one is waiting to be stored
          // the half before: the other half of this tile, or the second half of the tile before
          const int m_prev = ((h ? it : it - 1) * nwg + bid) * 256;
-         const int8_t *pbuf = patch + (it & 1) * PBYTES, *pnext = patch + ((it + 1) & 1) * PBYTES;
          static_for<NTAPS>([&](auto tc) {
             constexpr int tap = decltype(tc)::value;
             constexpr int cur = (tap + h) % 2;
@@ -211,9 +219,15 @@ __global__ __launch_bounds__(512) void conv_i8_resident_kernel(ResidentConv g, c
                      load_patch(it & 1, img2, oh2);
                   }
                }
+               // from here on the fragments come from the next tile's patch: the other buffer
+               const int to_other = (it & 1) ? -PBYTES : PBYTES;
+#pragma unroll
+               for (int ky2 = 0; ky2 < KH; ++ky2)
+#pragma unroll
+                  for (int i2 = 0; i2 < MT; ++i2)
+                     a_row[ky2][i2] += to_other;
                __builtin_amdgcn_sched_barrier(0);
             }
-            const int8_t *rbuf = (last && h == 1) ? pnext : pbuf;
             // A tap in groups, each fenced so that it is issued as written: two MFMAs and slices of the store of the half
             // before, then two LDS reads of the next tap's fragments (all of them in the first groups, so that the wait in
             // front of the next tap's first MFMA finds them done).  (Left to the scheduler, the store's instructions end up
@@ -242,7 +256,7 @@ __global__ __launch_bounds__(512) void conv_i8_resident_kernel(ResidentConv g, c
                      if constexpr (f < HN)
                         fb[1 - cur][f].c[0] = *(const v4i *)(wl + b_lane + (HN * nh + f) * R * WROW + ntap * 64);
                      else if constexpr (f < HN + MT)
-                        fa[1 - cur][f - HN].c[0] = *(const v4i *)(rbuf + a_lane + a_blk[f - HN] + (ky * PW + kx) * PIX);
+                        fa[1 - cur][f - HN].c[0] = *(const v4i *)(smem + (a_row[ky][f - HN] + kx * PIX));
                   });
                   __builtin_amdgcn_sched_barrier(0);
                }
@@ -264,7 +278,7 @@ __global__ __launch_bounds__(512) void conv_i8_resident_kernel(ResidentConv g, c
             fb[0][f].c[0] = *(const v4i *)(wl + b_lane + f * R * WROW);
 #pragma unroll
          for (int i = 0; i < MT; ++i)
-            fa[0][i].c[0] = *(const v4i *)(patch + a_lane + a_blk[i]);
+            fa[0][i].c[0] = *(const v4i *)(smem + a_row[0][i]);
       }
       half_body(h0, std::false_type{}, 0);
       half_body(h1, std::true_type{}, 0);
