@@ -301,6 +301,25 @@ def test_conv_i8_plane_sums_equal_the_sums_of_the_stored_map(rt, case, x_layout,
     assert np.array_equal(avg.view(np.uint32), want_avg.view(np.uint32))
 
 
+def test_plane_sums_take_average_gives_the_same_average_and_clears_the_sums(rt):
+    """sofie_hip_plane_sums_take_average: the bits of sofie_hip_plane_sums_to_average, and the sums are zero afterwards, so that a
+    convolution can add the next inference's planes up in the same buffer without a clearing launch (twice in a row here)."""
+    nc, hw = 5 * 77, 1024
+    sums = util.int32_range(311, nc, -120000, 130000)
+    d1, d2 = util.to_dev(sums), util.to_dev(sums)
+    y1, y2 = util.dev_empty((nc,), np.float32), util.dev_empty((nc,), np.float32)
+    rt.call("sofie_hip_plane_sums_to_average", util.ptr(y1), util.ptr(d1), nc, hw, C.c_float(0.037))
+    for again in range(2):
+        if again:
+            d2.copy_(util.to_dev(sums))
+        rt.call("sofie_hip_plane_sums_take_average", util.ptr(y2), util.ptr(d2), nc, hw, C.c_float(0.037))
+        rt.sync()
+        assert np.array_equal(util.to_host(y1).view(np.uint32), util.to_host(y2).view(np.uint32))
+        assert not util.to_host(d2).any() and np.array_equal(util.to_host(d1), sums)
+    want = (sums.astype(np.float32) * np.float32(0.037)) / np.float32(hw)
+    assert np.array_equal(util.to_host(y2).view(np.uint32), want.view(np.uint32))
+
+
 def test_conv_i8_plane_sums_refuse_a_column_matrix_shape(rt):
     case = (2, 16, 16, 16, 32, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1), 1)     # 144-byte reduction over NCHW input: needs a column matrix
     N, Cc, H, W, Cout, kh, kw, *_ = case
