@@ -72,6 +72,12 @@ public:
    bool IsOutputTensor(const std::string &name) const;
    // true if the tensor's leading dimension is the run-time batch; its stored shape then has 1 there
    bool IsDynamicTensor(const std::string &name) const { return fBatched.count(UTILITY::Clean_name(name)) != 0; }
+   // Options::kStridedInput: a graph input is read through strides handed to the Session's constructor
+   // (core/src/RModel.cxx:376-385 of the reference)
+   bool IsStridedInputTensor(const std::string &name) const
+   {
+      return fStridedInput && std::find(fInputTensorNames.begin(), fInputTensorNames.end(), UTILITY::Clean_name(name)) != fInputTensorNames.end();
+   }
    bool HasDynamicBatch() const { return !fBatchParam.empty(); }
    const std::string &GetBatchParamName() const { return fBatchParam; }
    // kinds of the operators that read `name` (after fusion)
@@ -138,6 +144,7 @@ private:
    std::size_t fBatchDefault = 1;
    bool fInitialized = false;
    bool fSafetensors = false;
+   bool fStridedInput = false;
    std::string fGC;
    std::string fWeightFileName;
 

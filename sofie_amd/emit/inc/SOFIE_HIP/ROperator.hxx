@@ -35,6 +35,9 @@ public:
    // asks CanBeView() and tells the operator its decision with SetView().
    virtual bool CanBeView() const { return false; }
    virtual void SetView(bool) {}
+   // Options::kStridedInput: true for an operator that reads a graph input through the strides given to the Session
+   // (the reference's default is false too, core/inc/SOFIE/operators/ROperator.hxx:121)
+   virtual bool SupportsStridedInput() const { return false; }
    // true for an operator that reads a tensor with a run-time batch and folds the batch away (a reduction over it): its outputs carry none
    virtual bool ConsumesBatch() const { return false; }
    virtual OperatorKind GetKind() const { return fKind; }

@@ -43,6 +43,7 @@ enum class Options {
    kDefault = 0x0,
    kNoWeightFile = 0x2,
    kSafetensorsWeightFile = 0x100,
+   kStridedInput = 0x200, // the Session's constructor takes the strides of the graph inputs (operands of Gemm)
    kExternalStream = 0x400,
    kCustomMemory = 0x800,
 };
@@ -50,6 +51,9 @@ inline std::underlying_type_t<Options> operator|(Options a, Options b)
 {
    return static_cast<std::underlying_type_t<Options>>(a) | static_cast<std::underlying_type_t<Options>>(b);
 }
+
+// Session member that holds the strides given for a graph input (the reference's name, core/inc/SOFIE/operators/ROperator.hxx:109)
+inline std::string InputStrideMemberName(const std::string &inputName) { return "fInputStride_" + inputName; }
 
 inline std::size_t GetTypeSize(ETensorType t)
 {

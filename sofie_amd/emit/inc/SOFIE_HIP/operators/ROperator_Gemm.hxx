@@ -132,9 +132,23 @@ public:
    const std::vector<std::size_t> &OutputShape() const { return fShapeY; }
    bool IsBatched() const { return fDynamic; }
 
+   bool SupportsStridedInput() const override { return true; }
+
    void Initialize(RModel &model) override
    {
       ResolveShapes(model);
+      // The operands A and B can be graph inputs read through the strides given to the Session (Options::kStridedInput).  A
+      // matrix is described to the kernels by a row stride and a transpose flag, so one of an operand's two strides must be
+      // 1; the plain 2-D product only (core/inc/SOFIE/operators/ROperator_Gemm.hxx:388-399 of the reference).
+      fStridedA = model.IsStridedInputTensor(fNA);
+      fStridedB = model.IsStridedInputTensor(fNB);
+      if ((!fNC.empty() && model.IsStridedInputTensor(fNC)) || (!fNR.empty() && model.IsStridedInputTensor(fNR)))
+         throw std::runtime_error("SOFIE Gemm Op - strided input is not supported for the bias (C)");
+      if ((fStridedA || fStridedB) && (model.GetTensorShape(fNA).size() != 2 || model.GetTensorShape(fNB).size() != 2))
+         throw std::runtime_error("SOFIE Gemm Op - strided input is only supported for a plain 2D Gemm "
+                                  "(no MatMul batching, no low rank factorization)");
+      fStoredA = model.GetTensorShape(fNA);
+      fStoredB = model.GetTensorShape(fNB);
       if (!fNR.empty() && (!model.CheckIfTensorAlreadyExist(fNR) || model.GetTensorType(fNR) != ETensorType::FLOAT ||
                            model.GetTensorShape(fNR) != fShapeY || model.IsDynamicTensor(fNR) != fDynamic))
          throw std::runtime_error("SOFIE Gemm Op: residual tensor " + fNR + " does not have the shape of the product");
@@ -332,10 +346,34 @@ public:
          out << SP << "   " << PostOpsDeclaration(post, fPost) << " " << d << ".post = &" << post << ";\n";
       if (!fNR.empty())
          out << SP << "   " << d << ".residual = tensor_" << fNR << ";\n";
+      // An operand read through strides {s0, s1}: element (i, j) of the stored matrix is at i * s0 + j * s1.  Row-major with
+      // s1 == 1: row stride s0.  Column-major with s0 == 1: row stride s1 and the transpose flag flipped.  Without a unit
+      // stride the matrix cannot be described (ROperator_Gemm.hxx:644-668 and 898-927 of the reference).
+      auto resolve = [&](const char *tag, const std::string &name, const std::vector<std::size_t> &stored, bool batchedRows) {
+         const std::string member = "this->" + InputStrideMemberName(name);
+         const std::string rows = batchedRows ? "static_cast<std::size_t>(sofie_batch)" : "static_cast<std::size_t>(" + std::to_string(stored[0]) + ")";
+         const std::string cols = "static_cast<std::size_t>(" + std::to_string(stored[1]) + ")";
+         out << SP << "   " << "if (!" << member << ".empty()) {\n";
+         out << SP << "      " << "if (" << member << "[1] == 1) {\n";
+         out << SP << "         " << d << ".ld" << (tag[0] == 'A' ? "a" : "b") << " = static_cast<std::int32_t>(std::max<std::size_t>(" << member << "[0], " << cols << "));\n";
+         out << SP << "      " << "} else if (" << member << "[0] == 1) {\n";
+         out << SP << "         " << d << ".trans" << tag << " = !" << d << ".trans" << tag << ";\n";
+         out << SP << "         " << d << ".ld" << (tag[0] == 'A' ? "a" : "b") << " = static_cast<std::int32_t>(std::max<std::size_t>(" << member << "[1], " << rows << "));\n";
+         out << SP << "      " << "} else {\n";
+         out << SP << "         " << "throw std::runtime_error(\"SOFIE Gemm Op - input tensor " << name << " has strides {\" + std::to_string(" << member
+             << "[0]) + \", \" + std::to_string(" << member << "[1]) + \"} without a unit stride, which BLAS cannot handle\");\n";
+         out << SP << "      " << "}\n";
+         out << SP << "   " << "}\n";
+      };
+      if (fStridedA)
+         resolve("A", fNA, fStoredA, fDynamicRows);
+      if (fStridedB)
+         resolve("B", fNB, fStoredB, false);
       return out.str();
    }
    // Can this product stand in a chain handed to sofie_hip_gemm_chain_f32 (it exists at run time and is a plain 2-D product)?
-   bool IsChainLink() const { return fM != 0 && !fIsOutputConstant && fBatch == 1 && !fDynamicStack && !fAttrTransA; }
+   // (an operand read through strides may turn out transposed at run time: such a product stays on its own)
+   bool IsChainLink() const { return fM != 0 && !fIsOutputConstant && fBatch == 1 && !fDynamicStack && !fAttrTransA && !fStridedA && !fStridedB; }
    const std::string &NameA() const { return fNA; }
    const std::string &NameY() const { return fNY; }
 
@@ -351,6 +389,8 @@ private:
    std::size_t fM = 0, fN = 0, fK = 0, fBatch = 1, fStrideA = 0, fStrideB = 0, fStrideC = 0;
    std::string fBiasMode;
    bool fDynamic = false, fDynamicRows = false, fDynamicStack = false, fIsOutputConstant = false;
+   bool fStridedA = false, fStridedB = false; // graph inputs read through the strides given to the Session
+   std::vector<std::size_t> fStoredA, fStoredB; // the operands' shapes as stored
 };
 
 } // namespace SOFIE_HIP

@@ -412,6 +412,14 @@ void RModel::Initialize(int batchSize)
          batchedIn = batchedIn || IsDynamicTensor(in);
       for (auto &y : fOperators[i]->GetOutputTensorNames())
          batchedOut = batchedOut || IsDynamicTensor(y);
+      // every operator that reads a strided graph input must be able to read it through its strides
+      // (core/src/RModel.cxx:764-772 of the reference)
+      if (fStridedInput)
+         for (auto &in : fOperators[i]->GetInputTensorNames())
+            if (IsStridedInputTensor(in) && !fOperators[i]->SupportsStridedInput())
+               throw std::runtime_error("sofie: Options::kStridedInput - operator " + std::to_string(i) + " (output " +
+                                        fOperators[i]->GetOutputTensorNames().at(0) + ") reads the input tensor " + in +
+                                        " but does not support strided input access");
       if (batchedIn && !batchedOut && !fOperators[i]->ConsumesBatch())
          throw std::runtime_error("SOFIE: operator " + std::to_string(i) + " (output " + fOperators[i]->GetOutputTensorNames().at(0) +
                                   ") does not support a run-time batch; generate with a fixed batch size");
@@ -941,13 +949,14 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    const bool noWeightFile = options & static_cast<std::underlying_type_t<Options>>(Options::kNoWeightFile);
    const bool customMemory = options & static_cast<std::underlying_type_t<Options>>(Options::kCustomMemory);
    const bool safetensors = !noWeightFile && (options & static_cast<std::underlying_type_t<Options>>(Options::kSafetensorsWeightFile));
+   const bool strided = fStridedInput;
    fSafetensors = safetensors;
    std::stringstream gc;
    std::string guard = "SOFIE_" + fName;
    std::transform(guard.begin(), guard.end(), guard.begin(), [](unsigned char c) { return std::toupper(c); });
    gc << "//Code generated automatically by SOFIE (gfx950 HIP backend)\n";
    gc << "#ifndef " << guard << "_GPU_HIP\n#define " << guard << "_GPU_HIP\n\n";
-   gc << "#include <array>\n#include <cstddef>\n#include <cstdint>\n#include <cstdlib>\n#include <fstream>\n#include <stdexcept>\n#include <string>\n#include <string_view>\n"
+   gc << "#include <algorithm>\n#include <array>\n#include <cstddef>\n#include <cstdint>\n#include <cstdlib>\n#include <fstream>\n#include <stdexcept>\n#include <string>\n#include <string_view>\n"
          "#include <tuple>\n#include <type_traits>\n#include <vector>\n#if __cplusplus >= 202002L\n#include <span>\n#endif\n#include \"sofie_hip.h\"\n";
    if (customMemory)
       gc << "#include <functional>\n";
@@ -976,6 +985,7 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
       if (bp == reserved)
          bp += "_batch";
    const std::string arenaBytes = dyn ? "ArenaBytes(fMaxBatch)" : "kArenaBytes";
+   const std::string arenaTotal = strided ? arenaBytes + " + sofie_strided_bytes" : arenaBytes;
    if (dyn) {
       gc << "   // the batch is a run-time parameter: what carries it is planned per batch entry and scaled by the capacity,\n";
       gc << "   // the constructor's maximum rounded up to a multiple of 16 (every region stays 256-byte aligned)\n";
@@ -990,6 +1000,32 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
       gc << "   static constexpr std::size_t kIntermediatePoolBytes = " << fPoolBytes << ";\n";
    }
    gc << "   sofie_hip_ctx *fCtx = nullptr;\n";
+   // Options::kStridedInput: the strides (in elements) of the graph inputs as the constructor received them, one member per
+   // input (empty = contiguous), as in the reference's Sessions (core/src/RModel.cxx:1272-1300, 1517-1520)
+   auto extentOf = [&](const std::string &n, const std::string &batch) {
+      return strided ? "InputExtent_" + n + "(" + (IsDynamicTensor(n) ? batch : std::string()) + ")"
+                     : (IsDynamicTensor(n) ? batch + " * " : std::string()) + std::to_string(ConvertShapeToLength(GetTensorShape(n)));
+   };
+   if (strided) {
+      for (auto &n : fInputTensorNames)
+         gc << "   std::vector<std::size_t> " << InputStrideMemberName(n) << ";\n";
+      gc << "   // elements a graph input spans in memory: from its first to its last element through the strides, or its length\n";
+      for (auto &n : fInputTensorNames) {
+         const auto &shape = GetTensorShape(n);
+         const bool dynIn = IsDynamicTensor(n);
+         gc << "   std::size_t InputExtent_" << n << "(" << (dynIn ? "std::size_t sofie_rows" : "") << ") const\n   {\n";
+         gc << "      const std::size_t shape[" << std::max<std::size_t>(shape.size(), 1) << "] = {";
+         for (std::size_t d = 0; d < shape.size(); ++d)
+            gc << (d ? ", " : "") << (d == 0 && dynIn ? std::string("sofie_rows") : std::to_string(shape[d]));
+         if (shape.empty())
+            gc << "1";
+         gc << "};\n";
+         gc << "      std::size_t length = 1, last = 0;\n";
+         gc << "      for (std::size_t d = 0; d < " << shape.size() << "; ++d) {\n         length *= shape[d];\n";
+         gc << "         if (!" << InputStrideMemberName(n) << ".empty() && shape[d])\n            last += (shape[d] - 1) * " << InputStrideMemberName(n) << "[d];\n      }\n";
+         gc << "      return " << InputStrideMemberName(n) << ".empty() || length == 0 ? length : last + 1;\n   }\n";
+      }
+   }
    if (customMemory)
       gc << "   MemoryProvider fProvider;\n   void *fBlock = nullptr;\n";
    auto typeOf = [&](const std::string &planName) -> std::string {
@@ -1005,24 +1041,50 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
          << ", " << p.bytes << " bytes" << (p.pooled ? ", live [" + std::to_string(p.begin) + "," + std::to_string(p.end) + ")" : "") << (p.view ? ", a view" : "") << "\n";
    gc << "\n";
    // constructor
+   // (Options::kStridedInput adds the strides of the inputs behind the shape parameter, as the reference does:
+   // core/src/RModel.cxx:1546-1549)
+   const std::string stridesDecl = strided ? ", std::vector<std::vector<std::size_t>> inputStrides = {}" : "";
+   const std::string stridesArg = strided ? ", inputStrides" : "";
    if (safetensors) {
       // the file is read whole and handed to the constructor that takes the payload
       gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "std::string filename = \"" << fName << "_GPU_HIP.safetensors\""
-         << (dyn ? ", std::size_t " + bp + " = " + std::to_string(fBatchDefault) : std::string()) << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
+         << (dyn ? ", std::size_t " + bp + " = " + std::to_string(fBatchDefault) : std::string()) << stridesDecl << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
       gc << "      : Session(" << (customMemory ? "std::move(provider), " : "") << "SafetensorsBlob(detail::LoadWeightsFromFile(filename))"
-         << (dyn ? ", " + bp : std::string()) << (externalStream ? ", stream" : "") << ", device)\n   {\n   }\n";
+         << (dyn ? ", " + bp : std::string()) << stridesArg << (externalStream ? ", stream" : "") << ", device)\n   {\n   }\n";
       gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "SafetensorsBlob weights_blob"
-         << (dyn ? ", std::size_t " + bp + " = " + std::to_string(fBatchDefault) : std::string()) << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
+         << (dyn ? ", std::size_t " + bp + " = " + std::to_string(fBatchDefault) : std::string()) << stridesDecl << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
    } else {
       gc << "   Session(" << (customMemory ? "MemoryProvider provider, " : "") << "std::string filename = \""
-         << (noWeightFile ? "" : fName + "_GPU_HIP.dat") << "\"" << (dyn ? ", std::size_t " + bp + " = " + std::to_string(fBatchDefault) : std::string()) << (externalStream ? ", void *stream = nullptr" : "")
-         << ", int device = 0)\n";
+         << (noWeightFile ? "" : fName + "_GPU_HIP.dat") << "\"" << (dyn ? ", std::size_t " + bp + " = " + std::to_string(fBatchDefault) : std::string()) << stridesDecl
+         << (externalStream ? ", void *stream = nullptr" : "") << ", int device = 0)\n";
    }
    if (customMemory)
       gc << "      : fProvider(std::move(provider))\n";
    gc << "   {\n";
    if (dyn)
       gc << "      fMaxBatch = " << bp << ";\n      fCapacity = Capacity(" << bp << ");\n";
+   if (strided) {
+      // the checks and messages of the reference (core/src/RModel.cxx:1272-1300)
+      gc << "      if (!inputStrides.empty()) {\n";
+      gc << "         if (inputStrides.size() != " << fInputTensorNames.size() << ")\n";
+      gc << "            throw std::runtime_error(\"sofie: expected " << fInputTensorNames.size() << " input stride array(s), one per input tensor\");\n";
+      for (std::size_t i = 0; i < fInputTensorNames.size(); ++i) {
+         const auto &n = fInputTensorNames[i];
+         const std::string member = InputStrideMemberName(n);
+         gc << "         " << member << " = inputStrides[" << i << "];\n";
+         gc << "         if (!" << member << ".empty() && " << member << ".size() != " << GetTensorShape(n).size() << ")\n";
+         gc << "            throw std::runtime_error(\"sofie: the stride array of input tensor " << n << " must have " << GetTensorShape(n).size()
+            << " element(s)\");\n";
+      }
+      gc << "      }\n";
+      gc << "      // an input given with strides does not fit its planned region: it gets one behind the planned arena, sized by its extent\n";
+      gc << "      std::size_t sofie_strided_bytes = 0;\n";
+      for (auto &n : fInputTensorNames) {
+         gc << "      const std::size_t sofie_strided_offset_" << n << " = sofie_strided_bytes;\n";
+         gc << "      if (!" << InputStrideMemberName(n) << ".empty())\n         sofie_strided_bytes += (" << extentOf(n, "fMaxBatch") << " * sizeof("
+            << ConvertTypeToString(fInputTensorInfos[n].type) << ") + 255) / 256 * 256;\n";
+      }
+   }
    if (safetensors) {
       // the payload is checked against the model before any device work
       gc << "      detail::SafetensorsReader sofie_weights_reader(weights_blob);\n";
@@ -1039,21 +1101,29 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
    gc << "      detail::Check(sofie_hip_ctx_create(&fCtx, device, " << (externalStream ? "stream" : "nullptr") << "), \"Session\");\n";
    gc << "      try {\n";
    if (customMemory) {
-      gc << "         fBlock = fProvider.alloc(" << arenaBytes << ");\n";
+      gc << "         fBlock = fProvider.alloc(" << arenaTotal << ");\n";
       gc << "         if (!fBlock)\n            throw std::runtime_error(\"SOFIE HIP Session: the memory provider returned no block\");\n";
-      gc << "         detail::Check(sofie_hip_arena_adopt(fCtx, fBlock, " << arenaBytes << "), \"adoption of the caller's block\");\n";
+      gc << "         detail::Check(sofie_hip_arena_adopt(fCtx, fBlock, " << arenaTotal << "), \"adoption of the caller's block\");\n";
       gc << "         auto place = [&](std::size_t offset) -> char * {\n"
             "            void *p = fProvider.assign ? fProvider.assign(offset) : static_cast<char *>(fBlock) + offset;\n"
             "            if (!p)\n               throw std::runtime_error(\"SOFIE HIP Session: the memory provider assigned no address\");\n"
             "            return static_cast<char *>(p);\n         };\n";
       for (auto &p : fPlan)
          gc << "         " << p.name << " = reinterpret_cast<" << typeOf(p.name) << " *>(place(" << offsetText(p) << "));\n";
+      if (strided)
+         for (auto &n : fInputTensorNames)
+            gc << "         if (!" << InputStrideMemberName(n) << ".empty())\n            tensor_" << n << " = reinterpret_cast<" << ConvertTypeToString(fInputTensorInfos[n].type)
+               << " *>(place(" << arenaBytes << " + sofie_strided_offset_" << n << "));\n";
    } else {
-      gc << "         detail::Check(sofie_hip_arena_create(fCtx, " << arenaBytes << ", " << kPoolAlignBytes << "), \"arena allocation\");\n";
+      gc << "         detail::Check(sofie_hip_arena_create(fCtx, " << arenaTotal << ", " << kPoolAlignBytes << "), \"arena allocation\");\n";
       gc << "         char *base = static_cast<char *>(sofie_hip_arena_ptr(fCtx, 0));\n";
       gc << "         if (!base)\n            throw std::runtime_error(\"SOFIE HIP runtime error: arena is null\");\n";
       for (auto &p : fPlan)
          gc << "         " << p.name << " = reinterpret_cast<" << typeOf(p.name) << " *>(base + " << offsetText(p) << ");\n";
+      if (strided)
+         for (auto &n : fInputTensorNames)
+            gc << "         if (!" << InputStrideMemberName(n) << ".empty())\n            tensor_" << n << " = reinterpret_cast<" << ConvertTypeToString(fInputTensorInfos[n].type)
+               << " *>(base + " << arenaBytes << " + sofie_strided_offset_" << n << ");\n";
    }
    bool anyWeights = false, anyConstants = false;
    for (auto &kv : fInitializedTensors)
@@ -1259,7 +1329,7 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
          return (IsDynamicTensor(n) ? bp + " * " : std::string()) + std::to_string(ConvertShapeToLength(GetTensorShape(n)));
       };
       for (std::size_t i = 0; i < fInputTensorNames.size(); ++i)
-         gc << "      if (inputs[" << i << "].size < " << lenOf(fInputTensorNames[i]) << " || !inputs[" << i << "].data)\n"
+         gc << "      if (inputs[" << i << "].size < " << extentOf(fInputTensorNames[i], bp) << " || !inputs[" << i << "].data)\n"
             << "         throw std::runtime_error(\"SOFIE HIP Session: the view of input " << fInputTensorNames[i] << " is too small\");\n";
       for (std::size_t i = 0; i < fOutputTensorNames.size(); ++i)
          gc << "      if (outputs[" << i << "].size < " << lenOf(fOutputTensorNames[i]) << " || !outputs[" << i << "].data)\n"
@@ -1270,7 +1340,7 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
       for (std::size_t i = 0; i < fInputTensorNames.size(); ++i) {
          const auto &n = fInputTensorNames[i];
          gc << "      float const *in_" << n << " = inputs[" << i << "].data;\n";
-         gc << "      if (!inPlace(in_" << n << ")) {\n         detail::Check(sofie_hip_copy(fCtx, tensor_" << n << ", in_" << n << ", (" << lenOf(n)
+         gc << "      if (!inPlace(in_" << n << ")) {\n         detail::Check(sofie_hip_copy(fCtx, tensor_" << n << ", in_" << n << ", (" << extentOf(n, bp)
             << ") * sizeof(float)), \"copy of input " << n << "\");\n         in_" << n << " = tensor_" << n << ";\n      }\n";
       }
       for (std::size_t i = 0; i < fOutputTensorNames.size(); ++i) {
@@ -1321,8 +1391,12 @@ void RModel::GenerateSessionCode(std::underlying_type_t<Options> options)
          << " exceeds the initialized maximum allowed shape.\");\n      }\n";
    for (auto &n : fInputTensorNames) {
       const auto &ti = fInputTensorInfos[n];
-      gc << "      detail::Check(sofie_hip_upload(fCtx, tensor_" << n << ", host_" << n << ", " << (IsDynamicTensor(n) ? bp + " * " : "")
-         << ConvertShapeToLength(ti.shape) * GetTypeSize(ti.type) << "), \"upload of input " << n << "\");\n";
+      if (strided)
+         gc << "      detail::Check(sofie_hip_upload(fCtx, tensor_" << n << ", host_" << n << ", " << extentOf(n, bp) << " * " << GetTypeSize(ti.type)
+            << "), \"upload of input " << n << "\");\n";
+      else
+         gc << "      detail::Check(sofie_hip_upload(fCtx, tensor_" << n << ", host_" << n << ", " << (IsDynamicTensor(n) ? bp + " * " : "")
+            << ConvertShapeToLength(ti.shape) * GetTypeSize(ti.type) << "), \"upload of input " << n << "\");\n";
    }
    gc << "      infer_nosync(" << (dyn ? bp : "") << ");\n";
    for (std::size_t i = 0; i < fOutputTensorNames.size(); ++i) {
@@ -1387,6 +1461,7 @@ void RModel::GenerateGPU_HIP(std::underlying_type_t<Options> options, int batchS
 {
    if (fOutputTensorNames.empty())
       throw std::runtime_error("SOFIE: the model has no output tensor");
+   fStridedInput = options & static_cast<std::underlying_type_t<Options>>(Options::kStridedInput);
    Initialize(batchSize);
    PlanMemory();
    GenerateSessionCode(options);

@@ -93,6 +93,63 @@ int main(int argc, char **argv)
       f8d.AddOutputTensorNameList({"Y"});
       f8d.GenerateGPU_HIP();
       f8d.OutputGenerated(std::string(argv[1]) + "/ApiDynamicFp8Gemm_GPU_HIP.hxx");
+      // Gemm operands that are graph inputs read through strides given to the Session (Options::kStridedInput): the four
+      // models of the reference's tests/models/StridedInputModelGenerator.cxx:104-129, 738-745, with its weights
+      // (tests/common/strided_input_test_utils.h:43-49: v[i] = scale * ((7 i) mod 11) - 0.5)
+      auto gemmValues = [](std::size_t n, float scale) {
+         std::vector<float> v(n);
+         for (std::size_t i = 0; i < n; i++)
+            v[i] = scale * float((i * 7) % 11) - 0.5f;
+         return v;
+      };
+      {
+         RModel m("StridedGemmBiasRelu"); // Y = Relu(X[3,5] * W[5,4] + B)
+         m.AddInputTensorInfo("X", ETensorType::FLOAT, std::vector<std::size_t>{3, 5});
+         m.AddInputTensorName("X");
+         auto W = gemmValues(5 * 4, 0.1f), B = gemmValues(4, 0.3f);
+         m.AddInitializedTensor("W", ETensorType::FLOAT, {5, 4}, W.data());
+         m.AddInitializedTensor("B", ETensorType::FLOAT, {4}, B.data());
+         m.AddOperator(std::make_unique<ROperator_Gemm<float>>(1.0f, 1.0f, 0, 0, "X", "W", "B", "H"));
+         m.AddOperator(std::make_unique<ROperator_Relu<float>>("H", "Y"));
+         m.AddOutputTensorNameList({"Y"});
+         m.GenerateGPU_HIP(Options::kStridedInput);
+         m.OutputGenerated(std::string(argv[1]) + "/" + m.GetName() + "_GPU_HIP.hxx");
+      }
+      {
+         RModel m("StridedGemmTransAB"); // Y = X^T * W^T, X stored [5,3], W stored [4,5]
+         m.AddInputTensorInfo("X", ETensorType::FLOAT, std::vector<std::size_t>{5, 3});
+         m.AddInputTensorName("X");
+         auto W = gemmValues(4 * 5, 0.1f);
+         m.AddInitializedTensor("W", ETensorType::FLOAT, {4, 5}, W.data());
+         m.AddOperator(std::make_unique<ROperator_Gemm<float>>(1.0f, 0.0f, 1, 1, "X", "W", "Y"));
+         m.AddOutputTensorNameList({"Y"});
+         m.GenerateGPU_HIP(Options::kStridedInput);
+         m.OutputGenerated(std::string(argv[1]) + "/" + m.GetName() + "_GPU_HIP.hxx");
+      }
+      for (int t = 0; t < 2; ++t) {
+         RModel m(t ? "StridedGemmABt" : "StridedGemmAB"); // both operands graph inputs; t: Y = A^T * B^T
+         m.AddInputTensorInfo("A", ETensorType::FLOAT, t ? std::vector<std::size_t>{5, 3} : std::vector<std::size_t>{3, 5});
+         m.AddInputTensorInfo("B", ETensorType::FLOAT, t ? std::vector<std::size_t>{4, 5} : std::vector<std::size_t>{5, 4});
+         m.AddInputTensorName("A");
+         m.AddInputTensorName("B");
+         m.AddOperator(std::make_unique<ROperator_Gemm<float>>(1.0f, 0.0f, t, t, "A", "B", "Y"));
+         m.AddOutputTensorNameList({"Y"});
+         m.GenerateGPU_HIP(Options::kStridedInput | Options::kNoWeightFile);
+         m.OutputGenerated(std::string(argv[1]) + "/" + m.GetName() + "_GPU_HIP.hxx");
+      }
+      {
+         // the batch a run-time parameter (maximum given to the constructor, default 8): rows of a larger matrix
+         RModel m("StridedGemmDynamic"); // Y[N,4] = X[N,5] * W[5,4] + B
+         m.AddInputTensorInfo("X", ETensorType::FLOAT, std::vector<Dim>{Dim(std::string("N"), 8), Dim(5)});
+         m.AddInputTensorName("X");
+         auto W = gemmValues(5 * 4, 0.1f), B = gemmValues(4, 0.3f);
+         m.AddInitializedTensor("W", ETensorType::FLOAT, {5, 4}, W.data());
+         m.AddInitializedTensor("B", ETensorType::FLOAT, {4}, B.data());
+         m.AddOperator(std::make_unique<ROperator_Gemm<float>>(1.0f, 1.0f, 0, 0, "X", "W", "B", "Y"));
+         m.AddOutputTensorNameList({"Y"});
+         m.GenerateGPU_HIP(Options::kStridedInput);
+         m.OutputGenerated(std::string(argv[1]) + "/" + m.GetName() + "_GPU_HIP.hxx");
+      }
    } catch (const std::exception &e) {
       std::cerr << "error: " << e.what() << "\n";
       return 1;

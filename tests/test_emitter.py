@@ -168,6 +168,54 @@ def test_reshapes_of_pool_tensors_are_views(tmp_path):
     assert "SOFIE_ACT_EXP" in body and "tensor_G" in body[body.index("SOFIE_ACT_EXP") - 200:body.index("SOFIE_ACT_EXP") + 200]
 
 
+def test_strided_input_option_adds_the_strides_to_the_session(emitted):
+    """Options::kStridedInput (core/src/RModel.cxx:1272-1300, 1546-1549 of the reference): the constructor takes one stride array
+    per input behind the shape parameter, checks count and rank with the reference's messages, and the Gemm resolves the row
+    stride and the transpose flag of a strided operand when it runs."""
+    txt = read(emitted, "StridedGemmAB")
+    assert 'Session(std::string filename = "", std::vector<std::vector<std::size_t>> inputStrides = {}, int device = 0)' in txt
+    assert "std::vector<std::size_t> fInputStride_A;" in txt and "std::vector<std::size_t> fInputStride_B;" in txt
+    assert "sofie: expected 2 input stride array(s), one per input tensor" in txt
+    assert "sofie: the stride array of input tensor B must have 2 element(s)" in txt
+    body = ops_body(txt)
+    assert "d.transA = !d.transA;" in body and "d.ldb = static_cast<std::int32_t>(std::max<std::size_t>(this->fInputStride_B[0]" in body
+    assert "without a unit stride, which BLAS cannot handle" in body
+    # the arena grows by the extents of the inputs that came with strides, and those inputs live there
+    assert "sofie_hip_arena_create(fCtx, kArenaBytes + sofie_strided_bytes, 256)" in txt
+    assert "tensor_A = reinterpret_cast<float *>(base + kArenaBytes + sofie_strided_offset_A);" in txt
+    # the shape parameter comes first, as in the reference's signature
+    dyn = read(emitted, "StridedGemmDynamic")
+    assert 'std::size_t N = 8, std::vector<std::vector<std::size_t>> inputStrides = {}, int device = 0)' in dyn
+    assert "InputExtent_X(fMaxBatch)" in dyn and "InputExtent_X(N) * 4" in dyn
+    # without the option nothing of it is emitted
+    assert "inputStrides" not in read(emitted, "ApiGemmRelu")
+
+
+def _emit_strided(tmp_path, nodes, inputs, outputs, init, name="m"):
+    p = os.path.join(str(tmp_path), name + ".onnx")
+    ow.write(p, nodes, inputs, outputs, init, name=name)
+    return subprocess.run([em.EMIT, p, str(tmp_path), "--strided-input"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+
+
+def test_strided_input_is_refused_where_no_operator_can_read_it(tmp_path):
+    """The refusals of the reference at generation (tests/cpu/TestStridedInput.cxx:198-208, 261-274; ROperator_Gemm.hxx:394-399):
+    an operator that cannot read through strides, a strided bias, a strided operand that is not a plain 2-D matrix."""
+    W = {"W": np.zeros((4, 3), dtype=np.float32)}
+    r = _emit_strided(tmp_path, [ow.node("Relu", ["X"], ["Y"])], [("X", np.float32, [2, 4])], [("Y", np.float32, [2, 4])], {})
+    assert r.returncode != 0 and "Options::kStridedInput" in r.stdout and "reads the input tensor X but does not support strided input access" in r.stdout
+    r = _emit_strided(tmp_path, [ow.node("Gemm", ["X", "W", "C"], ["Y"])], [("X", np.float32, [2, 4]), ("C", np.float32, [2, 3])],
+                      [("Y", np.float32, [2, 3])], W)
+    assert r.returncode != 0 and "strided input is not supported for the bias (C)" in r.stdout
+    r = _emit_strided(tmp_path, [ow.node("MatMul", ["X", "W"], ["Y"])], [("X", np.float32, [5, 2, 4])], [("Y", np.float32, [5, 2, 3])], W)
+    assert r.returncode != 0 and "strided input is only supported for a plain 2D Gemm" in r.stdout
+    # the same Gemm with only its A operand a graph input is taken, and an activation behind it still joins its store
+    r = _emit_strided(tmp_path, [ow.node("Gemm", ["X", "W"], ["H"]), ow.node("Relu", ["H"], ["Y"])], [("X", np.float32, [2, 4])],
+                      [("Y", np.float32, [2, 3])], W, name="ok")
+    assert r.returncode == 0, r.stdout
+    txt = open(os.path.join(str(tmp_path), "ok_GPU_HIP.hxx")).read()
+    assert "fInputStride_X" in ops_body(txt) and "SOFIE_ACT_RELU" in ops_body(txt)
+
+
 def test_unsupported_operator_is_refused_by_name(tmp_path):
     r = _emit(tmp_path, [ow.node("LSTM", ["X"], ["Y"])], [("X", np.float32, [1, 4])], [("Y", np.float32, [1, 4])], {})
     assert r.returncode != 0 and "LSTM" in r.stdout

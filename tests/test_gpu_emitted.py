@@ -216,6 +216,18 @@ def test_custom_memory_sessions(rt):
     assert failures == 0 and "FAIL" not in text and text.count("ok ") >= 14
 
 
+def test_strided_input_sessions(rt):
+    """Options::kStridedInput: the Session's constructor takes the strides of the graph inputs and the Gemm reads its operands
+    through them: row padding as a row stride, column-major storage as the transposed operand (tests/harness_strided_input.cxx
+    runs the Gemm scenarios of the reference's TestAlpakaStridedInput.cxx and reports them line by line)."""
+    lib = ctypes.CDLL(os.path.join(em.OUT, "libStridedInput.so"))
+    report = ctypes.create_string_buffer(8192)
+    print("strided input sessions", flush=True)
+    failures = lib.run_strided_input(em.OUT.encode(), report, 8192)
+    text = report.value.decode()
+    assert failures == 0 and "FAIL" not in text and text.count("ok ") >= 22, text
+
+
 def test_emitted_conv_batchnorm_relu(rt):
     spec = em.conv_batchnorm_relu(2)
     g = onnx_lite.load(os.path.join(em.OUT, "ConvBatchNormRelu.onnx"))
