@@ -150,6 +150,21 @@ int main(int argc, char **argv)
          m.GenerateGPU_HIP(Options::kStridedInput);
          m.OutputGenerated(std::string(argv[1]) + "/" + m.GetName() + "_GPU_HIP.hxx");
       }
+      {
+         // strided input together with every other Session option: run-time batch, caller-owned memory and stream,
+         // weights in a safetensors file (the constructor that reads the file hands the strides on to the one that takes the payload)
+         RModel m("StridedGemmAllOptions"); // Y[N,4] = X[N,5] * W[5,4] + B
+         m.AddInputTensorInfo("X", ETensorType::FLOAT, std::vector<Dim>{Dim(std::string("N"), 8), Dim(5)});
+         m.AddInputTensorName("X");
+         auto W = gemmValues(5 * 4, 0.1f), B = gemmValues(4, 0.3f);
+         m.AddInitializedTensor("W", ETensorType::FLOAT, {5, 4}, W.data());
+         m.AddInitializedTensor("B", ETensorType::FLOAT, {4}, B.data());
+         m.AddOperator(std::make_unique<ROperator_Gemm<float>>(1.0f, 1.0f, 0, 0, "X", "W", "B", "Y"));
+         m.AddOutputTensorNameList({"Y"});
+         m.GenerateGPU_HIP((Options::kCustomMemory | Options::kExternalStream) | static_cast<std::underlying_type_t<Options>>(Options::kSafetensorsWeightFile) |
+                           static_cast<std::underlying_type_t<Options>>(Options::kStridedInput));
+         m.OutputGenerated(std::string(argv[1]) + "/" + m.GetName() + "_GPU_HIP.hxx");
+      }
    } catch (const std::exception &e) {
       std::cerr << "error: " << e.what() << "\n";
       return 1;

@@ -7,6 +7,7 @@
 // The device memory of the views is the arena of a second runtime context, so this file needs no HIP header.
 #include "StridedGemmAB_GPU_HIP.hxx"
 #include "StridedGemmABt_GPU_HIP.hxx"
+#include "StridedGemmAllOptions_GPU_HIP.hxx"
 #include "StridedGemmBiasRelu_GPU_HIP.hxx"
 #include "StridedGemmDynamic_GPU_HIP.hxx"
 #include "StridedGemmTransAB_GPU_HIP.hxx"
@@ -297,6 +298,39 @@ extern "C" int run_strided_input(const char *dir, char *report, int len)
          Laid x({8, 5}, {5, 1}, ramp);
          Session s(wDyn, 8);
          expect(Close(s.infer(8, x.storage.data()), BiasProduct(x.logical, 8, false)), "run-time batch without strides: the current shape, contiguous");
+      }
+      {
+         // every Session option at once: the caller's block holds the planned arena AND the region of the strided input
+         using namespace SOFIE_StridedGemmAllOptions;
+         const std::string wAll = std::string(dir) + "/StridedGemmAllOptions_GPU_HIP.safetensors";
+         char *memory = static_cast<char *>(sofie_hip_arena_ptr(helper, 512 * 1024));
+         std::size_t asked = 0, assignedPastPlan = 0;
+         int freed = 0;
+         MemoryProvider provider;
+         provider.alloc = [&](std::size_t bytes) -> void * {
+            asked = bytes;
+            return memory;
+         };
+         provider.assign = [&](std::size_t off) -> void * {
+            assignedPastPlan += off >= Session::ArenaBytes(8) ? 1 : 0;
+            return memory + off;
+         };
+         provider.dealloc = [&](void *) { ++freed; };
+         {
+            Laid x({6, 5}, {7, 1}, ramp);
+            Session s(provider, wAll, 8, {{7, 1}}, sofie_hip_stream(helper));
+            // the input's extent at the maximum batch: 7 rows of 7 + 5 elements = 54 floats, rounded up to 256 bytes
+            expect(asked == Session::ArenaBytes(8) + 256 && assignedPastPlan == 1, "caller's memory: the block is the planned arena plus the strided input's region");
+            expect(s.stream() == sofie_hip_stream(helper) && Close(s.infer(6, x.storage.data()), BiasProduct(x.logical, 6, false)),
+                   "caller's memory and stream, safetensors weights, run-time batch, input strides {7, 1}");
+         }
+         expect(freed == 1, "caller's memory: block returned once");
+         {
+            Laid x({8, 5}, {5, 1}, ramp);
+            asked = 0;
+            Session s(provider, wAll, 8);
+            expect(asked == Session::ArenaBytes(8) && Close(s.infer(8, x.storage.data()), BiasProduct(x.logical, 8, false)), "the same Session without strides asks for the planned arena only");
+         }
       }
    } catch (const std::exception &e) {
       out << "FAIL exception: " << e.what() << "\n";

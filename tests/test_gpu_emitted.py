@@ -225,7 +225,7 @@ def test_strided_input_sessions(rt):
     print("strided input sessions", flush=True)
     failures = lib.run_strided_input(em.OUT.encode(), report, 8192)
     text = report.value.decode()
-    assert failures == 0 and "FAIL" not in text and text.count("ok ") >= 22, text
+    assert failures == 0 and "FAIL" not in text and text.count("ok ") >= 26, text
 
 
 def test_emitted_conv_batchnorm_relu(rt):
